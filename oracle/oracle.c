@@ -1,0 +1,296 @@
+/*
+ * CPU oracle for the weight-compressed FullyConnected path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file restates, in plain C, the arithmetic the
+ * OpenVINO reference performs for FullyConnectedCompressed.  It is linked only by
+ * the tests, by the smoke check and by the benchmark's cpu_baseline leg; the
+ * product library never calls it.
+ *
+ * Reference files restated (paths relative to the OpenVINO source tree):
+ *   - nibble order of u4/i4 buffers, sign extension of i4:
+ *       src/core/dev_api/openvino/core/type/element_iterator.hpp:76,161-176,248-259
+ *   - IEEE binary16 <-> binary32, round-to-nearest-even:
+ *       src/core/src/type/float16.cpp:32-110 (to half), :112-140 (to float)
+ *   - per-element FullyConnected-with-decompression formula
+ *       y[m,n] = sum_k x[m,k] * ((q[n,k] - zp[n,k/G]) * s[n,k/G]) (+ bias[n]):
+ *       src/plugins/intel_gpu/src/kernel_selector/cl_kernels/fully_connected_gpu_bfyx_ref.cl:88-160
+ *   - weights are [N,K] (MatMul with transpose_b = true):
+ *       src/common/transformations/src/ov_ops/fully_connected.cpp:40-57
+ *   - the dot product itself is the textbook triple loop of
+ *       src/core/reference/include/openvino/reference/matmul.hpp:19-46
+ *
+ * How each function is pinned (see tests/test_oracle_*.py):
+ *   unpack/pack      known-answer bytes of src/core/tests/element_iterator_test.cpp,
+ *                    uint4.cpp, int4.cpp; the reference's own element_iterator.hpp
+ *                    compiled into oracle/_ref where the reference tree is present
+ *   f16 conversion   exhaustive 65536-pattern round trip + numpy.float16 on random and
+ *                    edge values; the reference's float16.cpp compiled into oracle/_ref
+ *   fc_reference     exact golden vectors of fully_connected_gpu_test.cpp
+ *                    (:1425-1481, :2842-2909, :3014-3066, :3068-3119, :3121-3180,
+ *                    :1819-1877), an independent numpy float64 restatement, and
+ *                    algebraic invariants (zp == q gives 0, scale linearity, unit-vector
+ *                    probes, i4 == u4 xor 8 with zp 8, row permutation)
+ */
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* element type tags shared with oracle.py */
+enum {
+    OVO_NONE = 0,
+    OVO_U4 = 1,
+    OVO_I4 = 2,
+    OVO_U8 = 3,
+    OVO_I8 = 4,
+    OVO_F16 = 5,
+    OVO_F32 = 6
+};
+
+/* ---- 4-bit packing: element i lives in byte i/2, low nibble when i is even ---- */
+
+static inline uint8_t nibble_at(const uint8_t* bytes, size_t i) {
+    uint8_t b = bytes[i >> 1];
+    return (i & 1) ? (uint8_t)(b >> 4) : (uint8_t)(b & 0x0F);
+}
+
+static inline int8_t sext4(uint8_t v) {
+    return (int8_t)((v & 0x8) ? (int)v - 16 : (int)v);
+}
+
+void ovo_unpack_u4(const uint8_t* src, size_t n, uint8_t* dst) {
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = nibble_at(src, i);
+}
+
+void ovo_unpack_i4(const uint8_t* src, size_t n, int8_t* dst) {
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = sext4(nibble_at(src, i));
+}
+
+/* dst has (n+1)/2 bytes; a trailing unused high nibble is left zero */
+void ovo_pack_u4(const uint8_t* src, size_t n, uint8_t* dst) {
+    memset(dst, 0, (n + 1) / 2);
+    for (size_t i = 0; i < n; ++i) {
+        uint8_t v = (uint8_t)(src[i] & 0x0F);
+        dst[i >> 1] |= (i & 1) ? (uint8_t)(v << 4) : v;
+    }
+}
+
+void ovo_pack_i4(const int8_t* src, size_t n, uint8_t* dst) {
+    memset(dst, 0, (n + 1) / 2);
+    for (size_t i = 0; i < n; ++i) {
+        uint8_t v = (uint8_t)((uint8_t)src[i] & 0x0F);
+        dst[i >> 1] |= (i & 1) ? (uint8_t)(v << 4) : v;
+    }
+}
+
+/* ---- binary16 <-> binary32 ---- */
+
+uint16_t ovo_f32_to_f16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t e32 = (u >> 23) & 0xFFu;
+    const uint32_t m32 = u & 0x7FFFFFu;
+
+    if (e32 == 0xFFu) { /* inf / nan: keep the top payload bits, never turn a nan into inf */
+        if (m32 == 0)
+            return (uint16_t)(sign | 0x7C00u);
+        uint16_t payload = (uint16_t)(m32 >> 13);
+        if (payload == 0)
+            payload = 1;
+        return (uint16_t)(sign | 0x7C00u | payload);
+    }
+    if (e32 == 0) /* float zero or float subnormal: far below half's smallest subnormal */
+        return sign;
+
+    const int e = (int)e32 - 127; /* unbiased */
+    if (e > 15)
+        return (uint16_t)(sign | 0x7C00u);
+
+    if (e >= -14) { /* normal half unless rounding carries out */
+        uint32_t mant = m32 >> 13; /* 10 kept bits */
+        const uint32_t rest = m32 & 0x1FFFu;
+        uint32_t h = ((uint32_t)(e + 15) << 10) | mant;
+        if (rest > 0x1000u || (rest == 0x1000u && (mant & 1u)))
+            h += 1; /* a carry walks into the exponent, up to inf, which is what RNE wants */
+        return (uint16_t)(sign | h);
+    }
+
+    /* subnormal half: value = full * 2^(e-23), target unit 2^-24 */
+    if (e < -25)
+        return sign; /* below half of the smallest subnormal */
+    const uint32_t full = m32 | 0x800000u;
+    const int shift = -e - 1; /* 14..24 */
+    uint32_t mant = full >> shift;
+    const uint32_t rest = full & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1);
+    if (rest > half || (rest == half && (mant & 1u)))
+        mant += 1; /* may become 0x400 = smallest normal, encoded correctly */
+    return (uint16_t)(sign | mant);
+}
+
+float ovo_f16_to_f32(uint16_t h) {
+    const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1Fu;
+    uint32_t m = h & 0x3FFu;
+    uint32_t u;
+    if (e == 0x1Fu) {
+        u = sign | 0x7F800000u | (m << 13);
+    } else if (e != 0) {
+        u = sign | ((e + 112u) << 23) | (m << 13);
+    } else if (m == 0) {
+        u = sign;
+    } else { /* subnormal: renormalise */
+        int k = 0;
+        while (!(m & 0x400u)) {
+            m <<= 1;
+            ++k;
+        }
+        u = sign | ((uint32_t)(113 - k) << 23) | ((m & 0x3FFu) << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+void ovo_f32_to_f16_n(const float* src, size_t n, uint16_t* dst) {
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = ovo_f32_to_f16(src[i]);
+}
+
+void ovo_f16_to_f32_n(const uint16_t* src, size_t n, float* dst) {
+    for (size_t i = 0; i < n; ++i)
+        dst[i] = ovo_f16_to_f32(src[i]);
+}
+
+/* ---- FullyConnected with weight decompression ---- */
+
+typedef struct {
+    int64_t M, N, K;
+    int64_t group_size;  /* along K; == K for per-output-channel parameters */
+    int32_t w_type;      /* OVO_U4 / OVO_I4 / OVO_U8 / OVO_I8, row-major [N,K] */
+    int32_t scale_type;  /* OVO_F16 / OVO_F32, [N, K/group_size] */
+    int32_t zp_type;     /* OVO_NONE / OVO_U4 / OVO_U8 / OVO_F32, [N, K/group_size] or one element */
+    int32_t zp_scalar;   /* non-zero: zp holds exactly one element used everywhere */
+    int32_t bias_type;   /* OVO_NONE / OVO_F16 / OVO_F32, [N] */
+    int32_t x_type;      /* OVO_F16 / OVO_F32, [M,K] */
+    int32_t acc_f64;     /* 0: float accumulator, k ascending (the reference kernel's order); 1: double */
+    int32_t reserved;
+    const void* w;
+    const void* scale;
+    const void* zp;
+    const void* bias;
+    const void* x;
+    const int64_t* n_index; /* optional subset of output channels (NULL = all) */
+    int64_t n_count;        /* length of n_index; y is then [M, n_count] */
+} ovo_fc_args;
+
+static inline float load_real(const void* p, int32_t type, size_t i) {
+    if (type == OVO_F32)
+        return ((const float*)p)[i];
+    return ovo_f16_to_f32(((const uint16_t*)p)[i]);
+}
+
+static inline float load_weight(const void* w, int32_t type, size_t i) {
+    switch (type) {
+    case OVO_U4: return (float)nibble_at((const uint8_t*)w, i);
+    case OVO_I4: return (float)sext4(nibble_at((const uint8_t*)w, i));
+    case OVO_U8: return (float)((const uint8_t*)w)[i];
+    default:     return (float)((const int8_t*)w)[i];
+    }
+}
+
+static inline float load_zp(const void* zp, int32_t type, size_t i) {
+    switch (type) {
+    case OVO_NONE: return 0.0f;
+    case OVO_U4:   return (float)nibble_at((const uint8_t*)zp, i);
+    case OVO_U8:   return (float)((const uint8_t*)zp)[i];
+    default:       return ((const float*)zp)[i];
+    }
+}
+
+/* Returns 0 on success, a negative number naming the bad argument otherwise.
+ * y is float [M, n_count or N]; bias is added after the accumulation, before any output cast
+ * (fully_connected_gpu_bfyx_ref.cl:139-156); the cast to the output type is the caller's. */
+int ovo_fc_reference(const ovo_fc_args* a, float* y) {
+    if (!a || !y || !a->w || !a->scale || !a->x) return -1;
+    if (a->M < 0 || a->N <= 0 || a->K <= 0) return -2;
+    if (a->group_size <= 0 || a->K % a->group_size) return -3;
+    if (a->w_type < OVO_U4 || a->w_type > OVO_I8) return -4;
+    if (a->scale_type != OVO_F16 && a->scale_type != OVO_F32) return -5;
+    if (a->zp_type != OVO_NONE && a->zp_type != OVO_U4 && a->zp_type != OVO_U8 && a->zp_type != OVO_F32) return -6;
+    if (a->zp_type != OVO_NONE && !a->zp) return -6;
+    if (a->bias_type != OVO_NONE && a->bias_type != OVO_F16 && a->bias_type != OVO_F32) return -7;
+    if (a->bias_type != OVO_NONE && !a->bias) return -7;
+    if (a->x_type != OVO_F16 && a->x_type != OVO_F32) return -8;
+
+    const int64_t M = a->M, N = a->N, K = a->K, G = a->group_size, ng = K / G;
+    const int64_t ncols = a->n_index ? a->n_count : N;
+    int status = 0;
+
+    /* activations as float, converted once */
+    float* xf = (float*)__builtin_malloc((size_t)(M > 0 ? M : 1) * (size_t)K * sizeof(float));
+    if (!xf) return -10;
+    for (int64_t i = 0; i < M * K; ++i)
+        xf[i] = load_real(a->x, a->x_type, (size_t)i);
+
+#pragma omp parallel
+    {
+        float* wrow = (float*)__builtin_malloc((size_t)K * sizeof(float));
+#pragma omp for schedule(dynamic, 4)
+        for (int64_t c = 0; c < ncols; ++c) {
+            const int64_t n = a->n_index ? a->n_index[c] : c;
+            if (n < 0 || n >= N || !wrow) {
+                status = -9;
+                continue;
+            }
+            /* dequantise one weight row: (q - zp) * s, all in float */
+            for (int64_t k = 0; k < K; ++k) {
+                const int64_t g = k / G;
+                const float q = load_weight(a->w, a->w_type, (size_t)(n * K + k));
+                const float z = load_zp(a->zp, a->zp_type, a->zp_scalar ? 0 : (size_t)(n * ng + g));
+                const float s = load_real(a->scale, a->scale_type, (size_t)(n * ng + g));
+                wrow[k] = (q - z) * s;
+            }
+            const float b = a->bias_type == OVO_NONE ? 0.0f : load_real(a->bias, a->bias_type, (size_t)n);
+            for (int64_t m = 0; m < M; ++m) {
+                const float* xrow = xf + m * K;
+                if (a->acc_f64) {
+                    double acc = 0.0;
+                    for (int64_t k = 0; k < K; ++k)
+                        acc += (double)xrow[k] * (double)wrow[k];
+                    y[m * ncols + c] = (float)(acc + (double)b);
+                } else {
+                    float acc = 0.0f;
+                    for (int64_t k = 0; k < K; ++k)
+                        acc += xrow[k] * wrow[k];
+                    y[m * ncols + c] = acc + b;
+                }
+            }
+        }
+        __builtin_free(wrow);
+    }
+    __builtin_free(xf);
+    return status;
+}
+
+int ovo_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+void ovo_set_num_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}

@@ -1,0 +1,254 @@
+"""CPU oracle for FullyConnectedCompressed -- TEST INFRASTRUCTURE ONLY.
+
+Loads ``oracle/liboracle.so`` (built from ``oracle/oracle.c`` by ``oracle/Makefile``) and
+offers an independent numpy float64 restatement of the same formula for small cases.
+Only tests, the smoke check and the benchmark's ``cpu_baseline`` leg may import this
+module; the product package never does.
+
+Formula (OpenVINO: fully_connected_gpu_bfyx_ref.cl:88-160, ov_ops/fully_connected.cpp:40-57)::
+
+    y[m, n] = sum_k x[m, k] * ((q[n, k] - zp[n, k // G]) * s[n, k // G]) + bias[n]
+
+with ``q`` stored row-major ``[N, K]``; u4/i4 buffers hold element ``i`` in byte ``i // 2``,
+low nibble first (element_iterator.hpp:76,161-176), i4 sign-extended (:248-259).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+NONE, U4, I4, U8, I8, F16, F32 = range(7)
+TYPE_NAMES = {"none": NONE, "u4": U4, "i4": I4, "u8": U8, "i8": I8, "f16": F16, "f32": F32}
+
+
+class _FcArgs(ctypes.Structure):
+    _fields_ = [
+        ("M", ctypes.c_int64), ("N", ctypes.c_int64), ("K", ctypes.c_int64),
+        ("group_size", ctypes.c_int64),
+        ("w_type", ctypes.c_int32), ("scale_type", ctypes.c_int32),
+        ("zp_type", ctypes.c_int32), ("zp_scalar", ctypes.c_int32),
+        ("bias_type", ctypes.c_int32), ("x_type", ctypes.c_int32),
+        ("acc_f64", ctypes.c_int32), ("reserved", ctypes.c_int32),
+        ("w", ctypes.c_void_p), ("scale", ctypes.c_void_p), ("zp", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p), ("x", ctypes.c_void_p),
+        ("n_index", ctypes.c_void_p), ("n_count", ctypes.c_int64),
+    ]
+
+
+_lib = None
+_ref = None
+
+
+def build(force: bool = False) -> None:
+    """Compile liboracle.so (and oracle/_ref when the reference tree is present)."""
+    args = ["make", "-C", HERE]
+    if force:
+        args.append("-B")
+    subprocess.run(args, check=True, stdout=subprocess.DEVNULL)
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        path = os.path.join(HERE, "liboracle.so")
+        if not os.path.exists(path):
+            build()
+        L = ctypes.CDLL(path)
+        L.ovo_f32_to_f16.argtypes = [ctypes.c_float]
+        L.ovo_f32_to_f16.restype = ctypes.c_uint16
+        L.ovo_f16_to_f32.argtypes = [ctypes.c_uint16]
+        L.ovo_f16_to_f32.restype = ctypes.c_float
+        for name in ("ovo_unpack_u4", "ovo_unpack_i4", "ovo_pack_u4", "ovo_pack_i4",
+                     "ovo_f32_to_f16_n", "ovo_f16_to_f32_n"):
+            getattr(L, name).argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+            getattr(L, name).restype = None
+        L.ovo_fc_reference.argtypes = [ctypes.POINTER(_FcArgs), ctypes.c_void_p]
+        L.ovo_fc_reference.restype = ctypes.c_int
+        L.ovo_num_threads.restype = ctypes.c_int
+        L.ovo_set_num_threads.argtypes = [ctypes.c_int]
+        _lib = L
+    return _lib
+
+
+def ref_lib():
+    """The reference's own element iterator / float16, or None where it was not built."""
+    global _ref
+    if _ref is None:
+        path = os.path.join(HERE, "_ref", "libovref.so")
+        if not os.path.exists(path):
+            return None
+        R = ctypes.CDLL(path)
+        R.ref_f32_to_f16.argtypes = [ctypes.c_float]
+        R.ref_f32_to_f16.restype = ctypes.c_uint16
+        R.ref_f16_to_f32.argtypes = [ctypes.c_uint16]
+        R.ref_f16_to_f32.restype = ctypes.c_float
+        for name in ("ref_unpack_u4", "ref_unpack_i4", "ref_pack_u4", "ref_pack_i4"):
+            getattr(R, name).argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+            getattr(R, name).restype = None
+        _ref = R
+    return _ref
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+# ---------------------------------------------------------------- packing ----
+
+def unpack_u4(packed: np.ndarray, n: int) -> np.ndarray:
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    assert packed.size >= (n + 1) // 2
+    out = np.empty(n, dtype=np.uint8)
+    lib().ovo_unpack_u4(_ptr(packed), n, _ptr(out))
+    return out
+
+
+def unpack_i4(packed: np.ndarray, n: int) -> np.ndarray:
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    assert packed.size >= (n + 1) // 2
+    out = np.empty(n, dtype=np.int8)
+    lib().ovo_unpack_i4(_ptr(packed), n, _ptr(out))
+    return out
+
+
+def pack_u4(values: np.ndarray) -> np.ndarray:
+    values = np.ascontiguousarray(values, dtype=np.uint8).ravel()
+    out = np.empty((values.size + 1) // 2, dtype=np.uint8)
+    lib().ovo_pack_u4(_ptr(values), values.size, _ptr(out))
+    return out
+
+
+def pack_i4(values: np.ndarray) -> np.ndarray:
+    values = np.ascontiguousarray(values, dtype=np.int8).ravel()
+    out = np.empty((values.size + 1) // 2, dtype=np.uint8)
+    lib().ovo_pack_i4(_ptr(values), values.size, _ptr(out))
+    return out
+
+
+def f32_to_f16_bits(x: np.ndarray) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    out = np.empty(x.size, dtype=np.uint16)
+    lib().ovo_f32_to_f16_n(_ptr(x), x.size, _ptr(out))
+    return out
+
+
+def f16_bits_to_f32(h: np.ndarray) -> np.ndarray:
+    h = np.ascontiguousarray(h, dtype=np.uint16).ravel()
+    out = np.empty(h.size, dtype=np.float32)
+    lib().ovo_f16_to_f32_n(_ptr(h), h.size, _ptr(out))
+    return out
+
+
+# ------------------------------------------------------------ FC reference ----
+
+def _as_real(a, name):
+    """float16 / float32 array -> (contiguous array, type tag)."""
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float16:
+        return a, F16
+    if a.dtype == np.float32:
+        return a, F32
+    raise TypeError(f"{name}: expected float16 or float32, got {a.dtype}")
+
+
+def fc_reference(x, w, w_type, scale, zp=None, zp_type=NONE, bias=None, *, N, K, group_size,
+                 zp_scalar=False, acc_f64=False, n_index=None) -> np.ndarray:
+    """C oracle.  ``w`` and u4 ``zp`` are the raw packed bytes in OpenVINO order.
+
+    x: [M, K] float16/float32; scale: [N, K/G] float16/float32; zp: packed u4 bytes, u8 or
+    float32 [N, K/G] (or one element with ``zp_scalar``); bias: [N].  Returns float32 [M, N]
+    (or [M, len(n_index)]), not rounded to the output type.
+    """
+    x, x_type = _as_real(x, "x")
+    x = x.reshape(-1, K)
+    M = x.shape[0]
+    w = np.ascontiguousarray(w, dtype=np.int8 if w_type == I8 else np.uint8)
+    scale, scale_type = _as_real(scale, "scale")
+    a = _FcArgs()
+    a.M, a.N, a.K, a.group_size = M, N, K, group_size
+    a.w_type, a.scale_type, a.x_type = w_type, scale_type, x_type
+    a.zp_type, a.zp_scalar = zp_type, int(bool(zp_scalar))
+    if zp_type != NONE:
+        zp = np.ascontiguousarray(zp, dtype=np.float32 if zp_type == F32 else np.uint8)
+    else:
+        zp = None
+    if bias is not None:
+        bias, a.bias_type = _as_real(bias, "bias")
+    else:
+        a.bias_type = NONE
+    a.acc_f64 = int(bool(acc_f64))
+    a.w, a.scale, a.zp, a.bias, a.x = _ptr(w), _ptr(scale), _ptr(zp), _ptr(bias), _ptr(x)
+    ncols = N
+    idx = None
+    if n_index is not None:
+        idx = np.ascontiguousarray(n_index, dtype=np.int64)
+        a.n_index, a.n_count = _ptr(idx), idx.size
+        ncols = idx.size
+    y = np.empty((M, ncols), dtype=np.float32)
+    rc = lib().ovo_fc_reference(ctypes.byref(a), _ptr(y))
+    if rc != 0:
+        raise ValueError(f"ovo_fc_reference rejected its arguments (code {rc})")
+    return y
+
+
+# ---- independent numpy restatement (bit operations and float64 matmul) ----
+
+def np_unpack_nibbles(packed: np.ndarray, n: int, signed: bool) -> np.ndarray:
+    packed = np.asarray(packed, dtype=np.uint8).ravel()
+    both = np.stack([packed & 0x0F, packed >> 4], axis=1).ravel()[:n].astype(np.int16)
+    if signed:
+        both = np.where(both >= 8, both - 16, both)
+    return both
+
+
+def np_dequantise(w, w_type, scale, zp=None, zp_type=NONE, *, N, K, group_size,
+                  zp_scalar=False) -> np.ndarray:
+    """Dequantised weights as float64 [N, K]: (q - zp) * s evaluated in float32 like the oracle."""
+    ng = K // group_size
+    if w_type in (U4, I4):
+        q = np_unpack_nibbles(w, N * K, w_type == I4).reshape(N, K)
+    else:
+        q = np.asarray(w, dtype=np.int8 if w_type == I8 else np.uint8).reshape(N, K).astype(np.int16)
+    s = np.asarray(scale).astype(np.float32).reshape(N, ng)
+    if zp_type == NONE:
+        z = np.zeros((N, ng), dtype=np.float32)
+    else:
+        if zp_type == U4:
+            cnt = 1 if zp_scalar else N * ng
+            zz = np_unpack_nibbles(zp, cnt, False).astype(np.float32)
+        else:
+            zz = np.asarray(zp).astype(np.float32).ravel()
+        z = np.full((N, ng), zz[0], dtype=np.float32) if zp_scalar else zz.reshape(N, ng)
+    qf = q.astype(np.float32).reshape(N, ng, group_size)
+    deq = (qf - z[:, :, None]) * s[:, :, None]          # float32, as the reference kernel does
+    return deq.reshape(N, K).astype(np.float64)
+
+
+def fc_reference_numpy(x, w, w_type, scale, zp=None, zp_type=NONE, bias=None, *, N, K, group_size,
+                       zp_scalar=False) -> np.ndarray:
+    """float64 result [M, N] of the same formula, written with numpy only."""
+    deq = np_dequantise(w, w_type, scale, zp, zp_type, N=N, K=K, group_size=group_size,
+                        zp_scalar=zp_scalar)
+    y = np.asarray(x).astype(np.float64).reshape(-1, K) @ deq.T
+    if bias is not None:
+        y = y + np.asarray(bias).astype(np.float64).reshape(1, N)
+    return y
+
+
+# ---- error measures used by every parity test ----
+
+def rel_l2(y, y_ref) -> float:
+    y = np.asarray(y, dtype=np.float64)
+    y_ref = np.asarray(y_ref, dtype=np.float64)
+    den = np.linalg.norm(y_ref.ravel())
+    return float(np.linalg.norm((y - y_ref).ravel()) / (den if den > 0 else 1.0))
+
+
+def max_abs(y, y_ref) -> float:
+    return float(np.max(np.abs(np.asarray(y, dtype=np.float64) - np.asarray(y_ref, dtype=np.float64)))) \
+        if np.size(y) else 0.0
