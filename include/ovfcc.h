@@ -1,0 +1,196 @@
+/*
+ * ovfcc -- MI355X (gfx950) implementation of OpenVINO's weight-compressed FullyConnected,
+ * ov::op::internal::FullyConnectedCompressed, behind a plain C ABI.
+ *
+ *   Y[m,n] = sum_k X[m,k] * ((W[n,k] - ZP[n,k/G]) * S[n,k/G]) (+ bias[n])
+ *
+ * All entry points return OVFCC_OK (0) or a negative OVFCC_E* code; the reason is kept in a
+ * thread-local string readable with ovfcc_last_error().  No exceptions, no C++ or HIP types.
+ * Host pointers hold OpenVINO's constant layout: weights row-major [N,K] (MatMul with
+ * transpose_b = true), 4-bit types two per byte with the even element in the low nibble.
+ *
+ * Each declaration names the piece of the OpenVINO source tree it stands in for
+ * (paths relative to the OpenVINO repository root).
+ */
+#ifndef OVFCC_H
+#define OVFCC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OVFCC_OK 0
+#define OVFCC_EINVAL (-1)       /* bad argument (null pointer, shape, type tag) */
+#define OVFCC_EUNSUPPORTED (-2) /* valid OpenVINO configuration this library does not run */
+#define OVFCC_EDEVICE (-3)      /* HIP runtime error (no device, launch failure, ...) */
+#define OVFCC_ENOMEM (-4)       /* host or device allocation failed */
+
+/* element type tags; the subset of ov::element::Type_t this path uses
+ * (src/core/include/openvino/core/type/element_type.hpp) */
+enum ovfcc_type {
+    OVFCC_NONE = 0,
+    OVFCC_U4 = 1,
+    OVFCC_I4 = 2,
+    OVFCC_U8 = 3,
+    OVFCC_I8 = 4,
+    OVFCC_F16 = 5,
+    OVFCC_F32 = 6
+};
+
+/* One FullyConnectedCompressed node: the five inputs X, W, bias, weight_scales,
+ * weight_zero_points of src/common/transformations/include/ov_ops/fully_connected_compressed.hpp:15-37
+ * after ConvertFullyConnectedToFullyConnectedCompressed has re-viewed the constants as
+ * W [N,K], S/ZP [N,K/G] (src/common/transformations/src/transformations/op_conversions/
+ * convert_fc_to_compressed.cpp:42-78).  An absent input (the reference's
+ * Constant(dynamic, Shape{0})) is type OVFCC_NONE with a null pointer. */
+typedef struct ovfcc_fc_desc {
+    int64_t N;          /* output channels (OC) */
+    int64_t K;          /* input channels (IC) */
+    int64_t group_size; /* G along K; K for per-output-channel scale/zp */
+    int32_t w_type;     /* OVFCC_U4 | OVFCC_I4 | OVFCC_U8 | OVFCC_I8 */
+    int32_t scale_type; /* OVFCC_F16 */
+    int32_t zp_type;    /* OVFCC_NONE | OVFCC_U4 | OVFCC_U8 */
+    int32_t zp_scalar;  /* non-zero: zp holds one element (Shape{} / Shape{1}) used for every (n, group) */
+    int32_t bias_type;  /* OVFCC_NONE | OVFCC_F16, [N] */
+    int32_t act_type;   /* OVFCC_F16 */
+    int32_t out_type;   /* OVFCC_F16 (FullyConnected's output_type; default = activation type) */
+    int32_t flags;      /* 0 */
+} ovfcc_fc_desc;
+
+typedef struct ovfcc_ctx ovfcc_ctx;         /* one device + its kernels */
+typedef struct ovfcc_weights ovfcc_weights; /* repacked, device-resident W/S/ZP/bias of one node */
+typedef struct ovfcc_request ovfcc_request; /* one HIP stream + staging + split-K workspace */
+
+/* kernel families, as reported by ovfcc_last_kernel_info and accepted by ovfcc_request_force_kernel */
+enum ovfcc_kernel {
+    OVFCC_KERNEL_AUTO = 0,
+    OVFCC_KERNEL_PLAIN = 1,  /* any shape, OpenVINO layout, one wave per output channel */
+    OVFCC_KERNEL_DECODE = 2, /* M <= 32: split-K streaming kernel over the tiled layout */
+    OVFCC_KERNEL_PREFILL = 3 /* M > 32: LDS-dequantise + MFMA tiles over the tiled layout */
+};
+
+typedef struct ovfcc_kernel_info {
+    int32_t kernel;     /* enum ovfcc_kernel actually launched */
+    int32_t grid[3];
+    int32_t block;
+    int32_t split_k;
+    int32_t tile_m, tile_n;
+    char name[64];
+} ovfcc_kernel_info;
+
+/* ---- life cycle ---------------------------------------------------------------------------- */
+
+/* Plugin creation for one device: stands in for the device-side part of
+ * ov::IPlugin construction (src/inference/dev_api/openvino/runtime/iplugin.hpp:74-255;
+ * template: src/plugins/template/src/plugin.cpp:36-60).  Fails with OVFCC_EDEVICE when no
+ * gfx950 device is visible. */
+int ovfcc_init(int device, ovfcc_ctx** out);
+void ovfcc_destroy(ovfcc_ctx* ctx);
+
+/* Number of visible HIP devices (0 on a host without a GPU); never fails. */
+int ovfcc_device_count(void);
+
+/* Compile-time weight preparation: what DnnlFCPrimitive::createShapeAgnosticData +
+ * utils::prepareWeightsMemory do once per node on the CPU plugin
+ * (src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_fullyconnected_primitive.cpp:421-484,
+ * src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_utils.cpp:49-122) and
+ * reorder_weights_int4.cl does on the Intel GPU plugin.  Validates the descriptor with this
+ * library's analogue of FullyConnected::isSupportedCompressedOperation
+ * (src/plugins/intel_cpu/src/nodes/fullyconnected.cpp:143-218), repacks on the host into
+ * wave64 tiles and uploads.  Host buffers may be released on return. */
+int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* w, const void* scales,
+                         const void* zp, const void* bias, ovfcc_weights** out);
+void ovfcc_weights_destroy(ovfcc_weights* w);
+/* A second device copy of an existing node (same bytes at distinct addresses, no host work):
+ * what sharing one compressed constant between several FullyConnected nodes needs when each node
+ * must own its buffer (shared weights: src/tests/functional/plugin/shared/src/subgraph/
+ * shared_matmul_weights_decompression.cpp); the benchmark uses it to build a rotating weight set. */
+int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out);
+/* device bytes held by the repacked node */
+int64_t ovfcc_weights_device_bytes(const ovfcc_weights* w);
+/* 1 when the node uses the tiled layout (fast kernels), 0 for the OpenVINO-layout fallback */
+int ovfcc_weights_is_tiled(const ovfcc_weights* w);
+
+/* One infer request: ov::ISyncInferRequest
+ * (src/inference/dev_api/openvino/runtime/isync_infer_request.hpp:30-175).  Different requests
+ * may run concurrently from different threads; one request is used by one thread at a time. */
+int ovfcc_request_create(ovfcc_ctx* ctx, ovfcc_request** out);
+void ovfcc_request_destroy(ovfcc_request* req);
+
+/* ---- execution ----------------------------------------------------------------------------- */
+
+/* ISyncInferRequest::infer for one node with host tensors: copies X [M,K] f16 to the device,
+ * runs the kernel, copies Y [M,N] f16 back and waits.  The CPU plugin's equivalent is
+ * FullyConnected::execute -> DnnlFCPrimitive::execute
+ * (src/plugins/intel_cpu/src/nodes/fullyconnected.cpp:427-433,
+ * .../dnnl_fullyconnected_primitive.cpp:518-520).  M may be 0. */
+int ovfcc_fc_run(ovfcc_request* req, const ovfcc_weights* w, const void* x_host, void* y_host, int64_t M);
+
+/* Same with device-resident X and Y (a remote tensor in OpenVINO terms,
+ * src/inference/dev_api/openvino/runtime/iremote_tensor.hpp): enqueues on the request's
+ * stream and returns without waiting. */
+int ovfcc_fc_run_device(ovfcc_request* req, const ovfcc_weights* w, const void* x_dev, void* y_dev, int64_t M);
+
+/* Wait for everything enqueued on the request (IAsyncInferRequest::wait). */
+int ovfcc_request_sync(ovfcc_request* req);
+
+/* Kernel choice override for tests and profiling (enum ovfcc_kernel; AUTO restores the policy),
+ * and split-K override (0 = heuristic). */
+int ovfcc_request_force_kernel(ovfcc_request* req, int kernel, int split_k);
+
+/* What the last ovfcc_fc_run* on this request launched: the data behind
+ * ICompiledModel::get_runtime_model's primitiveType / IInferRequest::get_profiling_info
+ * (src/inference/dev_api/openvino/runtime/exec_model_info.hpp:31-73). */
+int ovfcc_last_kernel_info(const ovfcc_request* req, ovfcc_kernel_info* info);
+
+/* Timed back-to-back launches for the benchmark: runs `iters` passes over the `n_layers` nodes
+ * in order (layer i reads x_dev, writes y_dev; buffers must fit the largest layer), all on the
+ * request's stream, bracketed by HIP events on that stream.  Returns elapsed milliseconds of the
+ * whole timed region.  use_graph != 0 captures one pass into a HIP graph and replays it. */
+int ovfcc_bench_layers(ovfcc_request* req, const ovfcc_weights* const* layers, int n_layers, const void* x_dev,
+                       void* y_dev, int64_t M, int warmup, int iters, int use_graph, float* elapsed_ms);
+
+/* ---- device memory helpers (plain pointers; for hosts that do not link HIP themselves) ------ */
+int ovfcc_device_malloc(ovfcc_ctx* ctx, size_t bytes, void** out);
+int ovfcc_device_free(ovfcc_ctx* ctx, void* ptr);
+int ovfcc_memcpy_h2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
+int ovfcc_memcpy_d2h(ovfcc_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
+/* Plain device-to-device copy kernel of `bytes` (multiple of 16) repeated `iters` times, timed with
+ * HIP events: the yardstick the HBM counters and the achieved-bandwidth figures are scaled by. */
+int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, int iters, float* elapsed_ms);
+
+/* ---- host-only pieces (no device needed) ----------------------------------------------------- */
+
+/* Validation alone: OVFCC_OK, OVFCC_EINVAL or OVFCC_EUNSUPPORTED, as ovfcc_weights_create would. */
+int ovfcc_desc_validate(const ovfcc_fc_desc* desc);
+
+/* Sizes of the tiled layout for a descriptor; all zero when the descriptor falls back to the
+ * OpenVINO layout.  w_bytes: 1 KiB tiles of 16 channels x 128 (4-bit) or 64 (8-bit) inputs;
+ * scale_bytes: f16 [N/16][groups][16]; zp_bytes: u8 [N/16][groups][16] (0 without zero-points). */
+int ovfcc_tiled_sizes(const ovfcc_fc_desc* desc, size_t* w_bytes, size_t* scale_bytes, size_t* zp_bytes);
+
+/* The repacker itself, host to host (what ovfcc_weights_create uploads), and its inverse, which
+ * restores OpenVINO's layout bit for bit.  i4 weights are stored as u4 = i4 xor 8 with the
+ * zero-point raised by 8 (the transformation the CPU plugin applies for its unsigned kernels,
+ * src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_utils.cpp:70-97); i8 likewise xor 0x80. */
+int ovfcc_repack_host(const ovfcc_fc_desc* desc, const void* w, const void* scales, const void* zp,
+                      void* w_tiled, void* scale_tiled, void* zp_tiled);
+int ovfcc_unrepack_host(const ovfcc_fc_desc* desc, const void* w_tiled, const void* scale_tiled,
+                        const void* zp_tiled, void* w, void* scales, void* zp);
+
+/* 4-bit element access in OpenVINO order
+ * (src/core/dev_api/openvino/core/type/element_iterator.hpp:76,161-176,248-259). */
+int ovfcc_unpack_u4(const void* src, size_t n, uint8_t* dst);
+int ovfcc_unpack_i4(const void* src, size_t n, int8_t* dst);
+
+/* Last error text of the calling thread ("" when none). */
+const char* ovfcc_last_error(void);
+const char* ovfcc_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OVFCC_H */

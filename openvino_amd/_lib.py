@@ -1,0 +1,105 @@
+"""ctypes binding of the C ABI declared in include/ovfcc.h."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG, "libovfcc.so")
+
+OK, EINVAL, EUNSUPPORTED, EDEVICE, ENOMEM = 0, -1, -2, -3, -4
+NONE, U4, I4, U8, I8, F16, F32 = range(7)
+TYPE = {"none": NONE, "u4": U4, "i4": I4, "u8": U8, "i8": I8, "f16": F16, "f32": F32}
+KERNEL_AUTO, KERNEL_PLAIN, KERNEL_DECODE, KERNEL_PREFILL = range(4)
+
+# every symbol include/ovfcc.h declares
+SYMBOLS = [
+    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_destroy",
+    "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
+    "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_request_sync", "ovfcc_request_force_kernel",
+    "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
+    "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_bench_copy", "ovfcc_desc_validate", "ovfcc_tiled_sizes",
+    "ovfcc_repack_host", "ovfcc_unrepack_host", "ovfcc_unpack_u4", "ovfcc_unpack_i4", "ovfcc_last_error",
+    "ovfcc_version",
+]
+
+
+class FcDesc(ctypes.Structure):
+    _fields_ = [
+        ("N", ctypes.c_int64), ("K", ctypes.c_int64), ("group_size", ctypes.c_int64),
+        ("w_type", ctypes.c_int32), ("scale_type", ctypes.c_int32), ("zp_type", ctypes.c_int32),
+        ("zp_scalar", ctypes.c_int32), ("bias_type", ctypes.c_int32), ("act_type", ctypes.c_int32),
+        ("out_type", ctypes.c_int32), ("flags", ctypes.c_int32),
+    ]
+
+
+class KernelInfo(ctypes.Structure):
+    _fields_ = [
+        ("kernel", ctypes.c_int32), ("grid", ctypes.c_int32 * 3), ("block", ctypes.c_int32),
+        ("split_k", ctypes.c_int32), ("tile_m", ctypes.c_int32), ("tile_n", ctypes.c_int32),
+        ("name", ctypes.c_char * 64),
+    ]
+
+
+class OvfccError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"ovfcc error {code}: {message}")
+        self.code = code
+        self.message = message
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the built library; there is no fallback when it is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise OvfccError(EDEVICE, f"{LIB_PATH} is not built; run python -m openvino_amd.build")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, i64, sz, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_size_t, ctypes.c_int
+    pp = ctypes.POINTER(ctypes.c_void_p)
+    sig = {
+        "ovfcc_init": (ci, [ci, pp]),
+        "ovfcc_destroy": (None, [vp]),
+        "ovfcc_device_count": (ci, []),
+        "ovfcc_weights_create": (ci, [vp, ctypes.POINTER(FcDesc), vp, vp, vp, vp, pp]),
+        "ovfcc_weights_clone": (ci, [vp, pp]),
+        "ovfcc_weights_destroy": (None, [vp]),
+        "ovfcc_weights_device_bytes": (i64, [vp]),
+        "ovfcc_weights_is_tiled": (ci, [vp]),
+        "ovfcc_request_create": (ci, [vp, pp]),
+        "ovfcc_request_destroy": (None, [vp]),
+        "ovfcc_fc_run": (ci, [vp, vp, vp, vp, i64]),
+        "ovfcc_fc_run_device": (ci, [vp, vp, vp, vp, i64]),
+        "ovfcc_request_sync": (ci, [vp]),
+        "ovfcc_request_force_kernel": (ci, [vp, ci, ci]),
+        "ovfcc_last_kernel_info": (ci, [vp, ctypes.POINTER(KernelInfo)]),
+        "ovfcc_bench_layers": (ci, [vp, pp, ci, vp, vp, i64, ci, ci, ci, ctypes.POINTER(ctypes.c_float)]),
+        "ovfcc_device_malloc": (ci, [vp, sz, pp]),
+        "ovfcc_device_free": (ci, [vp, vp]),
+        "ovfcc_memcpy_h2d": (ci, [vp, vp, vp, sz]),
+        "ovfcc_memcpy_d2h": (ci, [vp, vp, vp, sz]),
+        "ovfcc_bench_copy": (ci, [vp, vp, vp, sz, ci, ctypes.POINTER(ctypes.c_float)]),
+        "ovfcc_desc_validate": (ci, [ctypes.POINTER(FcDesc)]),
+        "ovfcc_tiled_sizes": (ci, [ctypes.POINTER(FcDesc), ctypes.POINTER(sz), ctypes.POINTER(sz), ctypes.POINTER(sz)]),
+        "ovfcc_repack_host": (ci, [ctypes.POINTER(FcDesc), vp, vp, vp, vp, vp, vp]),
+        "ovfcc_unrepack_host": (ci, [ctypes.POINTER(FcDesc), vp, vp, vp, vp, vp, vp]),
+        "ovfcc_unpack_u4": (ci, [vp, sz, vp]),
+        "ovfcc_unpack_i4": (ci, [vp, sz, vp]),
+        "ovfcc_last_error": (ctypes.c_char_p, []),
+        "ovfcc_version": (ctypes.c_char_p, []),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = L
+    return L
+
+
+def check(rc: int) -> None:
+    if rc != OK:
+        raise OvfccError(rc, load().ovfcc_last_error().decode())

@@ -1,0 +1,559 @@
+// C ABI over the HIP runtime: contexts, repacked weights, requests, execution, benchmarking loops.
+// Every function returns an OVFCC_* code and records the reason with ovfcc::fail.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "ovfcc_internal.h"
+
+struct ovfcc_ctx {
+    int device = 0;
+    int n_cus = 256;
+    std::string arch;
+};
+
+struct ovfcc_weights {
+    ovfcc_ctx* ctx = nullptr;
+    ovfcc_fc_desc desc{};
+    ovfcc::Layout layout;
+    void* d_w = nullptr;
+    void* d_scale = nullptr;
+    void* d_zp = nullptr;
+    void* d_bias = nullptr;
+    size_t bytes = 0;
+};
+
+struct ovfcc_request {
+    ovfcc_ctx* ctx = nullptr;
+    hipStream_t stream = nullptr;
+    void* d_x = nullptr;
+    void* d_y = nullptr;
+    size_t x_cap = 0, y_cap = 0;
+    float* workspace = nullptr;
+    size_t ws_cap = 0;
+    unsigned* counters = nullptr;
+    size_t counter_cap = 0;
+    int force_kernel = OVFCC_KERNEL_AUTO;
+    int force_split = 0;
+    ovfcc_kernel_info last{};
+};
+
+namespace {
+
+using ovfcc::fail;
+
+int hip_fail(hipError_t e, const char* what) {
+    return fail(e == hipErrorOutOfMemory ? OVFCC_ENOMEM : OVFCC_EDEVICE,
+                std::string(what) + ": " + hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                       \
+    do {                                    \
+        hipError_t _e = (expr);             \
+        if (_e != hipSuccess)               \
+            return hip_fail(_e, #expr);     \
+    } while (0)
+
+int grow(void** p, size_t* cap, size_t need) {
+    if (need <= *cap)
+        return OVFCC_OK;
+    if (*p)
+        HIP_TRY(hipFree(*p));
+    *p = nullptr;
+    *cap = 0;
+    HIP_TRY(hipMalloc(p, need));
+    *cap = need;
+    return OVFCC_OK;
+}
+
+int ensure_split_buffers(ovfcc_request* r, const ovfcc::LaunchPlan& plan) {
+    if (plan.workspace_bytes > r->ws_cap) {
+        HIP_TRY(hipStreamSynchronize(r->stream));
+        int rc = grow(reinterpret_cast<void**>(&r->workspace), &r->ws_cap, plan.workspace_bytes);
+        if (rc)
+            return rc;
+    }
+    if (plan.counter_count > r->counter_cap) {
+        HIP_TRY(hipStreamSynchronize(r->stream));
+        size_t cap_bytes = r->counter_cap * sizeof(unsigned);
+        int rc = grow(reinterpret_cast<void**>(&r->counters), &cap_bytes, plan.counter_count * sizeof(unsigned));
+        if (rc)
+            return rc;
+        r->counter_cap = plan.counter_count;
+        // counters return to zero at the end of every launch; they only need clearing once
+        HIP_TRY(hipMemsetAsync(r->counters, 0, plan.counter_count * sizeof(unsigned), r->stream));
+        HIP_TRY(hipStreamSynchronize(r->stream));
+    }
+    return OVFCC_OK;
+}
+
+void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc::FcDeviceArgs* a) {
+    a->w = w->d_w;
+    a->scale = w->d_scale;
+    a->zp = w->d_zp;
+    a->bias = w->d_bias;
+    a->x = x;
+    a->y = y;
+    a->workspace = nullptr;
+    a->counters = nullptr;
+    a->M = M;
+    a->N = w->desc.N;
+    a->K = w->desc.K;
+    a->group_size = w->desc.group_size;
+    a->w_type = w->desc.w_type;
+    a->zp_type = w->desc.zp_type;
+    a->zp_scalar = w->desc.zp_scalar;
+    a->layout = w->layout;
+}
+
+void record(ovfcc_request* r, const ovfcc::LaunchPlan& p) {
+    ovfcc_kernel_info& i = r->last;
+    std::memset(&i, 0, sizeof(i));
+    i.kernel = p.kernel;
+    i.grid[0] = (int32_t)p.grid[0];
+    i.grid[1] = (int32_t)p.grid[1];
+    i.grid[2] = (int32_t)p.grid[2];
+    i.block = (int32_t)p.block;
+    i.split_k = p.split_k;
+    i.tile_m = p.tile_m;
+    i.tile_n = p.tile_n;
+    std::snprintf(i.name, sizeof(i.name), "%s", p.name);
+}
+
+// Enqueue one node.  Rows beyond what a single launch covers (tiled node whose N is not a multiple
+// of the prefill tile) are run through the decode kernel 32 rows at a time.
+int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M) {
+    if (M == 0)
+        return OVFCC_OK;
+    ovfcc::FcDeviceArgs a;
+    fill_args(w, x, y, M, &a);
+    int force = r->force_kernel;
+    const bool chunked = w->layout.tiled && M > 32 && (w->desc.N % 128) != 0 &&
+                         (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL);
+    if (chunked) {
+        for (int64_t m0 = 0; m0 < M; m0 += 32) {
+            const int64_t rows = M - m0 < 32 ? M - m0 : 32;
+            fill_args(w, static_cast<const char*>(x) + (size_t)m0 * w->desc.K * 2,
+                      static_cast<char*>(y) + (size_t)m0 * w->desc.N * 2, rows, &a);
+            ovfcc::LaunchPlan p;
+            int rc = ovfcc::plan_launch(a, OVFCC_KERNEL_DECODE, r->force_split, r->ctx->n_cus, &p);
+            if (rc)
+                return rc;
+            rc = ensure_split_buffers(r, p);
+            if (rc)
+                return rc;
+            a.workspace = r->workspace;
+            a.counters = r->counters;
+            int e = ovfcc::launch_fc(a, p, r->stream);
+            if (e)
+                return hip_fail((hipError_t)e, "kernel launch");
+            record(r, p);
+        }
+        return OVFCC_OK;
+    }
+    ovfcc::LaunchPlan p;
+    int rc = ovfcc::plan_launch(a, force, r->force_split, r->ctx->n_cus, &p);
+    if (rc)
+        return rc;
+    rc = ensure_split_buffers(r, p);
+    if (rc)
+        return rc;
+    a.workspace = r->workspace;
+    a.counters = r->counters;
+    int e = ovfcc::launch_fc(a, p, r->stream);
+    if (e)
+        return hip_fail((hipError_t)e, "kernel launch");
+    record(r, p);
+    return OVFCC_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ovfcc_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+int ovfcc_init(int device, ovfcc_ctx** out) {
+    if (!out)
+        return fail(OVFCC_EINVAL, "out is null");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0) {
+        (void)hipGetLastError();
+        return fail(OVFCC_EDEVICE, "no HIP device is visible; this library has no CPU path");
+    }
+    if (device < 0 || device >= n)
+        return fail(OVFCC_EINVAL, "device index out of range");
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    std::string arch = prop.gcnArchName;
+    if (arch.rfind("gfx950", 0) != 0)
+        return fail(OVFCC_EDEVICE, "device is " + arch + "; the kernels are built for gfx950 only");
+    ovfcc_ctx* c = new ovfcc_ctx();
+    c->device = device;
+    c->n_cus = prop.multiProcessorCount;
+    c->arch = arch;
+    *out = c;
+    return OVFCC_OK;
+}
+
+void ovfcc_destroy(ovfcc_ctx* ctx) {
+    delete ctx;
+}
+
+int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* w, const void* scales, const void* zp,
+                         const void* bias, ovfcc_weights** out) {
+    if (!ctx || !out)
+        return fail(OVFCC_EINVAL, "ctx or out is null");
+    *out = nullptr;
+    int rc = ovfcc::validate_desc(desc);
+    if (rc)
+        return rc;
+    if (!w || !scales)
+        return fail(OVFCC_EINVAL, "weights and scales are required");
+    if (desc->zp_type != OVFCC_NONE && !zp)
+        return fail(OVFCC_EINVAL, "zero-point type given without a buffer");
+    if (desc->bias_type != OVFCC_NONE && !bias)
+        return fail(OVFCC_EINVAL, "bias type given without a buffer");
+    HIP_TRY(hipSetDevice(ctx->device));
+
+    ovfcc_weights* W = new ovfcc_weights();
+    W->ctx = ctx;
+    W->desc = *desc;
+    W->layout = ovfcc::make_layout(*desc);
+    ovfcc::Layout& L = W->layout;
+    if (desc->zp_type != OVFCC_NONE && desc->zp_scalar)
+        L.zp_const = ovfcc::scalar_zero_point(*desc, zp) + L.zp_offset;
+
+    auto upload = [&](void** dst, const void* src, size_t bytes) -> int {
+        if (bytes == 0)
+            return OVFCC_OK;
+        HIP_TRY(hipMalloc(dst, bytes));
+        HIP_TRY(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+        W->bytes += bytes;
+        return OVFCC_OK;
+    };
+
+    const int64_t N = desc->N, K = desc->K, ng = L.groups;
+    if (L.tiled) {
+        std::vector<uint8_t> wt(L.w_bytes), st(L.scale_bytes), zt(L.zp_bytes);
+        ovfcc::repack_weights(*desc, L, w, wt.data());
+        ovfcc::repack_params(*desc, L, scales, zp, st.data(), zt.data());
+        rc = upload(&W->d_w, wt.data(), wt.size());
+        if (!rc)
+            rc = upload(&W->d_scale, st.data(), st.size());
+        if (!rc && L.zp_table)
+            rc = upload(&W->d_zp, zt.data(), zt.size());
+    } else {
+        const bool four = desc->w_type == OVFCC_U4 || desc->w_type == OVFCC_I4;
+        const size_t wb = four ? (size_t)(N * K + 1) / 2 : (size_t)N * K;
+        rc = upload(&W->d_w, w, wb);
+        if (!rc)
+            rc = upload(&W->d_scale, scales, (size_t)N * ng * 2);
+        if (!rc && desc->zp_type != OVFCC_NONE) {
+            const size_t cnt = desc->zp_scalar ? 1 : (size_t)N * ng;
+            rc = upload(&W->d_zp, zp, desc->zp_type == OVFCC_U4 ? (cnt + 1) / 2 : cnt);
+        }
+    }
+    if (!rc && desc->bias_type != OVFCC_NONE)
+        rc = upload(&W->d_bias, bias, (size_t)N * 2);
+    if (rc) {
+        ovfcc_weights_destroy(W);
+        return rc;
+    }
+    *out = W;
+    return OVFCC_OK;
+}
+
+void ovfcc_weights_destroy(ovfcc_weights* w) {
+    if (!w)
+        return;
+    if (w->d_w) (void)hipFree(w->d_w);
+    if (w->d_scale) (void)hipFree(w->d_scale);
+    if (w->d_zp) (void)hipFree(w->d_zp);
+    if (w->d_bias) (void)hipFree(w->d_bias);
+    delete w;
+}
+
+int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out) {
+    if (!src || !out)
+        return fail(OVFCC_EINVAL, "null argument");
+    *out = nullptr;
+    HIP_TRY(hipSetDevice(src->ctx->device));
+    ovfcc_weights* W = new ovfcc_weights();
+    W->ctx = src->ctx;
+    W->desc = src->desc;
+    W->layout = src->layout;
+    const ovfcc::Layout& L = src->layout;
+    const int64_t N = src->desc.N, K = src->desc.K, ng = L.groups;
+    const bool four = L.bits == 4;
+    size_t wb, sb, zb = 0;
+    if (L.tiled) {
+        wb = L.w_bytes;
+        sb = L.scale_bytes;
+        zb = L.zp_bytes;
+    } else {
+        wb = four ? (size_t)(N * K + 1) / 2 : (size_t)N * K;
+        sb = (size_t)N * ng * 2;
+        if (src->desc.zp_type != OVFCC_NONE) {
+            const size_t cnt = src->desc.zp_scalar ? 1 : (size_t)N * ng;
+            zb = src->desc.zp_type == OVFCC_U4 ? (cnt + 1) / 2 : cnt;
+        }
+    }
+    auto dup = [&](void** dst, const void* from, size_t bytes) -> int {
+        if (!from || bytes == 0)
+            return OVFCC_OK;
+        HIP_TRY(hipMalloc(dst, bytes));
+        HIP_TRY(hipMemcpy(*dst, from, bytes, hipMemcpyDeviceToDevice));
+        W->bytes += bytes;
+        return OVFCC_OK;
+    };
+    int rc = dup(&W->d_w, src->d_w, wb);
+    if (!rc) rc = dup(&W->d_scale, src->d_scale, sb);
+    if (!rc) rc = dup(&W->d_zp, src->d_zp, zb);
+    if (!rc) rc = dup(&W->d_bias, src->d_bias, (size_t)N * 2);
+    if (rc) {
+        ovfcc_weights_destroy(W);
+        return rc;
+    }
+    *out = W;
+    return OVFCC_OK;
+}
+
+int64_t ovfcc_weights_device_bytes(const ovfcc_weights* w) {
+    return w ? (int64_t)w->bytes : 0;
+}
+
+int ovfcc_weights_is_tiled(const ovfcc_weights* w) {
+    return w && w->layout.tiled ? 1 : 0;
+}
+
+int ovfcc_request_create(ovfcc_ctx* ctx, ovfcc_request** out) {
+    if (!ctx || !out)
+        return fail(OVFCC_EINVAL, "ctx or out is null");
+    *out = nullptr;
+    HIP_TRY(hipSetDevice(ctx->device));
+    ovfcc_request* r = new ovfcc_request();
+    r->ctx = ctx;
+    hipError_t e = hipStreamCreateWithFlags(&r->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete r;
+        return hip_fail(e, "hipStreamCreateWithFlags");
+    }
+    *out = r;
+    return OVFCC_OK;
+}
+
+void ovfcc_request_destroy(ovfcc_request* r) {
+    if (!r)
+        return;
+    if (r->stream) {
+        (void)hipStreamSynchronize(r->stream);
+        (void)hipStreamDestroy(r->stream);
+    }
+    if (r->d_x) (void)hipFree(r->d_x);
+    if (r->d_y) (void)hipFree(r->d_y);
+    if (r->workspace) (void)hipFree(r->workspace);
+    if (r->counters) (void)hipFree(r->counters);
+    delete r;
+}
+
+int ovfcc_request_force_kernel(ovfcc_request* r, int kernel, int split_k) {
+    if (!r)
+        return fail(OVFCC_EINVAL, "request is null");
+    if (kernel < OVFCC_KERNEL_AUTO || kernel > OVFCC_KERNEL_PREFILL || split_k < 0)
+        return fail(OVFCC_EINVAL, "unknown kernel or negative split");
+    r->force_kernel = kernel;
+    r->force_split = split_k;
+    return OVFCC_OK;
+}
+
+int ovfcc_last_kernel_info(const ovfcc_request* r, ovfcc_kernel_info* info) {
+    if (!r || !info)
+        return fail(OVFCC_EINVAL, "null argument");
+    *info = r->last;
+    return OVFCC_OK;
+}
+
+int ovfcc_fc_run_device(ovfcc_request* r, const ovfcc_weights* w, const void* x_dev, void* y_dev, int64_t M) {
+    if (!r || !w)
+        return fail(OVFCC_EINVAL, "request or weights is null");
+    if (M < 0)
+        return fail(OVFCC_EINVAL, "M is negative");
+    if (M > 0 && (!x_dev || !y_dev))
+        return fail(OVFCC_EINVAL, "x or y is null");
+    if (w->ctx != r->ctx)
+        return fail(OVFCC_EINVAL, "weights and request belong to different contexts");
+    if (M > ((int64_t)1 << 24))
+        return fail(OVFCC_EUNSUPPORTED, "M is limited to 2^24");
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    return enqueue(r, w, x_dev, y_dev, M);
+}
+
+int ovfcc_request_sync(ovfcc_request* r) {
+    if (!r)
+        return fail(OVFCC_EINVAL, "request is null");
+    HIP_TRY(hipStreamSynchronize(r->stream));
+    return OVFCC_OK;
+}
+
+int ovfcc_fc_run(ovfcc_request* r, const ovfcc_weights* w, const void* x_host, void* y_host, int64_t M) {
+    if (!r || !w)
+        return fail(OVFCC_EINVAL, "request or weights is null");
+    if (M < 0)
+        return fail(OVFCC_EINVAL, "M is negative");
+    if (M == 0)
+        return OVFCC_OK;
+    if (!x_host || !y_host)
+        return fail(OVFCC_EINVAL, "x or y is null");
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    const size_t xb = (size_t)M * w->desc.K * 2, yb = (size_t)M * w->desc.N * 2;
+    if (xb > r->x_cap || yb > r->y_cap)
+        HIP_TRY(hipStreamSynchronize(r->stream));
+    int rc = grow(&r->d_x, &r->x_cap, xb);
+    if (rc)
+        return rc;
+    rc = grow(&r->d_y, &r->y_cap, yb);
+    if (rc)
+        return rc;
+    HIP_TRY(hipMemcpyAsync(r->d_x, x_host, xb, hipMemcpyHostToDevice, r->stream));
+    rc = ovfcc_fc_run_device(r, w, r->d_x, r->d_y, M);
+    if (rc)
+        return rc;
+    HIP_TRY(hipMemcpyAsync(y_host, r->d_y, yb, hipMemcpyDeviceToHost, r->stream));
+    HIP_TRY(hipStreamSynchronize(r->stream));
+    return OVFCC_OK;
+}
+
+int ovfcc_bench_layers(ovfcc_request* r, const ovfcc_weights* const* layers, int n_layers, const void* x_dev,
+                       void* y_dev, int64_t M, int warmup, int iters, int use_graph, float* elapsed_ms) {
+    if (!r || !layers || n_layers <= 0 || !elapsed_ms || iters <= 0 || warmup < 0)
+        return fail(OVFCC_EINVAL, "bad benchmark arguments");
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    // one eager pass first: sizes the split-K buffers so that nothing allocates inside a capture
+    for (int i = 0; i < n_layers; ++i) {
+        int rc = ovfcc_fc_run_device(r, layers[i], x_dev, y_dev, M);
+        if (rc)
+            return rc;
+    }
+    HIP_TRY(hipStreamSynchronize(r->stream));
+
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    if (use_graph) {
+        HIP_TRY(hipStreamBeginCapture(r->stream, hipStreamCaptureModeThreadLocal));
+        int rc = OVFCC_OK;
+        for (int i = 0; i < n_layers && !rc; ++i)
+            rc = ovfcc_fc_run_device(r, layers[i], x_dev, y_dev, M);
+        hipError_t e = hipStreamEndCapture(r->stream, &graph);
+        if (rc)
+            return rc;
+        if (e != hipSuccess)
+            return hip_fail(e, "hipStreamEndCapture");
+        HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    }
+    auto one_pass = [&]() -> int {
+        if (use_graph) {
+            HIP_TRY(hipGraphLaunch(exec, r->stream));
+            return OVFCC_OK;
+        }
+        for (int i = 0; i < n_layers; ++i) {
+            int rc = ovfcc_fc_run_device(r, layers[i], x_dev, y_dev, M);
+            if (rc)
+                return rc;
+        }
+        return OVFCC_OK;
+    };
+    int rc = OVFCC_OK;
+    for (int i = 0; i < warmup && !rc; ++i)
+        rc = one_pass();
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    if (!rc) {
+        HIP_TRY(hipEventCreate(&t0));
+        HIP_TRY(hipEventCreate(&t1));
+        HIP_TRY(hipStreamSynchronize(r->stream));
+        HIP_TRY(hipEventRecord(t0, r->stream));
+        for (int i = 0; i < iters && !rc; ++i)
+            rc = one_pass();
+        HIP_TRY(hipEventRecord(t1, r->stream));
+        HIP_TRY(hipEventSynchronize(t1));
+        HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
+    }
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    return rc;
+}
+
+int ovfcc_device_malloc(ovfcc_ctx* ctx, size_t bytes, void** out) {
+    if (!ctx || !out)
+        return fail(OVFCC_EINVAL, "null argument");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMalloc(out, bytes ? bytes : 1));
+    return OVFCC_OK;
+}
+
+int ovfcc_device_free(ovfcc_ctx* ctx, void* ptr) {
+    if (!ctx)
+        return fail(OVFCC_EINVAL, "null argument");
+    if (ptr)
+        HIP_TRY(hipFree(ptr));
+    return OVFCC_OK;
+}
+
+int ovfcc_memcpy_h2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes) {
+    if (!ctx || ((!dst_dev || !src_host) && bytes))
+        return fail(OVFCC_EINVAL, "null argument");
+    if (bytes)
+        HIP_TRY(hipMemcpy(dst_dev, src_host, bytes, hipMemcpyHostToDevice));
+    return OVFCC_OK;
+}
+
+int ovfcc_memcpy_d2h(ovfcc_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes) {
+    if (!ctx || ((!dst_host || !src_dev) && bytes))
+        return fail(OVFCC_EINVAL, "null argument");
+    if (bytes)
+        HIP_TRY(hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+    return OVFCC_OK;
+}
+
+int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, int iters, float* elapsed_ms) {
+    if (!ctx || !dst_dev || !src_dev || !elapsed_ms || iters <= 0 || bytes % 16)
+        return fail(OVFCC_EINVAL, "bad copy benchmark arguments");
+    HIP_TRY(hipSetDevice(ctx->device));
+    hipStream_t s = nullptr;
+    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    hipEvent_t t0, t1;
+    HIP_TRY(hipEventCreate(&t0));
+    HIP_TRY(hipEventCreate(&t1));
+    int e = ovfcc::launch_copy(dst_dev, src_dev, bytes, s);  // warm-up
+    HIP_TRY(hipStreamSynchronize(s));
+    HIP_TRY(hipEventRecord(t0, s));
+    for (int i = 0; i < iters && !e; ++i)
+        e = ovfcc::launch_copy(dst_dev, src_dev, bytes, s);
+    HIP_TRY(hipEventRecord(t1, s));
+    HIP_TRY(hipEventSynchronize(t1));
+    HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    (void)hipStreamDestroy(s);
+    if (e)
+        return hip_fail((hipError_t)e, "copy kernel launch");
+    return OVFCC_OK;
+}
+
+}  // extern "C"

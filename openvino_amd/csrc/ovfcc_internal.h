@@ -1,0 +1,92 @@
+// Internal declarations shared by the host API, the repacker and the kernel launchers.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+
+#include "ovfcc.h"
+
+namespace ovfcc {
+
+// ---- tiled layout ------------------------------------------------------------------------
+// The unit every fast kernel streams is a 1 KiB tile read by one wave64 with one 128-bit load
+// per lane.  A tile covers 16 output channels; lane l serves channel (l & 15) and k-quarter
+// (l >> 4).  A "k-block" is 128 consecutive input channels: one tile for 4-bit weights, two
+// consecutive tiles (64 inputs each) for 8-bit weights.
+//
+// 4-bit tile, lane l, dword j (0..3), element e (0..7):
+//     k_local = 32*j + 8*(l >> 4) + e          nibble position in the dword = (e >> 1) + 4*(e & 1)
+//   so that masking with 0x000F000F / 0x00F000F0 (and once more after >> 8) yields the element
+//   pairs (0,1) (2,3) (4,5) (6,7) as packed halves, the order one MFMA operand register holds.
+// 8-bit tile, lane l, dword d (0..3), byte b (0..3):
+//     k_local = 32*(d >> 1) + 8*(l >> 4) + 4*(d & 1) + b      (within the tile's 64 inputs)
+// Weights are stored unsigned: i4 xor 8, i8 xor 0x80, with the zero-point raised to match.
+// Tiles are ordered [N/16][K/k_per_tile]; scales f16 and zero-points u8 as [N/16][groups][16].
+constexpr int kTileRows = 16;
+constexpr int kTileBytes = 1024;
+constexpr int kBlockK = 128;
+
+struct Layout {
+    bool tiled = false;
+    int bits = 4;
+    int64_t n_tiles = 0;        // N / 16
+    int64_t k_blocks = 0;       // K / 128
+    int64_t tiles_per_kblock = 1;
+    int64_t groups = 0;         // K / G
+    int64_t kblocks_per_group = 0;
+    bool zp_table = false;      // per-(n, group) zero-points stored as a table
+    int zp_const = 0;           // zero-point used when there is no table (includes the unsigned offset)
+    int zp_offset = 0;          // 8 for i4, 128 for i8, else 0
+    size_t w_bytes = 0, scale_bytes = 0, zp_bytes = 0;
+};
+
+void set_error(const std::string& msg);
+int fail(int code, const std::string& msg);
+
+int validate_desc(const ovfcc_fc_desc* d);
+// Fills the layout for a validated descriptor (tiled == false when the fallback applies).
+Layout make_layout(const ovfcc_fc_desc& d);
+int scalar_zero_point(const ovfcc_fc_desc& d, const void* zp);
+
+void repack_weights(const ovfcc_fc_desc& d, const Layout& L, const void* w, void* w_tiled);
+void repack_params(const ovfcc_fc_desc& d, const Layout& L, const void* scales, const void* zp, void* scale_tiled,
+                   void* zp_tiled);
+void unrepack_weights(const ovfcc_fc_desc& d, const Layout& L, const void* w_tiled, void* w);
+void unrepack_params(const ovfcc_fc_desc& d, const Layout& L, const void* scale_tiled, const void* zp_tiled,
+                     void* scales, void* zp);
+
+// ---- kernel launch parameters ------------------------------------------------------------------
+struct FcDeviceArgs {
+    const void* w;       // tiled or OpenVINO layout
+    const void* scale;
+    const void* zp;      // table, raw zp, or null
+    const void* bias;    // f16 [N] or null
+    const void* x;       // f16 [M,K]
+    void* y;             // f16 [M,N]
+    float* workspace;    // split-K partials
+    unsigned* counters;  // split-K arrival counters, one per 16-channel tile, zero between launches
+    int64_t M, N, K, group_size;
+    int w_type, zp_type, zp_scalar;
+    Layout layout;
+};
+
+struct LaunchPlan {
+    int kernel = OVFCC_KERNEL_AUTO;
+    int split_k = 1;
+    int kblocks_per_split = 0;
+    int tile_m = 0, tile_n = 0;
+    unsigned grid[3] = {1, 1, 1};
+    unsigned block = 256;
+    size_t workspace_bytes = 0;
+    size_t counter_count = 0;
+    const char* name = "";
+};
+
+// Chooses kernel family and decomposition (force_kernel / force_split 0 = policy).
+int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_cus, LaunchPlan* plan);
+// Enqueues on `stream` (a hipStream_t passed as void*); returns a HIP error code (0 = success).
+int launch_fc(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
+
+}  // namespace ovfcc

@@ -1,0 +1,218 @@
+"""Host-side mirror of the FullyConnectedCompressed node over the C ABI.
+
+Argument names and meaning follow ov::op::internal::FullyConnectedCompressed
+(src/common/transformations/include/ov_ops/fully_connected_compressed.hpp:15-37): inputs X, W,
+bias, weight_scales, weight_zero_points; W is [N, K]; an absent input is ``None``.  Everything
+executes in libovfcc.so on the GPU; there is no CPU path here.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Sequence
+
+import numpy as np
+
+from . import _lib
+from ._lib import FcDesc, KernelInfo, OvfccError, check
+
+
+def _vp(a: Optional[np.ndarray]):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
+              has_bias: bool = False) -> FcDesc:
+    d = FcDesc()
+    d.N, d.K, d.group_size = N, K, group_size
+    d.w_type = _lib.TYPE[w_type]
+    d.scale_type = _lib.F16
+    d.zp_type = _lib.TYPE[zp_type]
+    d.zp_scalar = int(zp_scalar)
+    d.bias_type = _lib.F16 if has_bias else _lib.NONE
+    d.act_type = _lib.F16
+    d.out_type = _lib.F16
+    d.flags = 0
+    return d
+
+
+class Device:
+    """One MI355X and its library context (the plugin object's device half)."""
+
+    def __init__(self, index: int = 0):
+        self.lib = _lib.load()
+        h = ctypes.c_void_p()
+        check(self.lib.ovfcc_init(index, ctypes.byref(h)))
+        self.handle = h
+
+    def close(self):
+        if self.handle:
+            self.lib.ovfcc_destroy(self.handle)
+            self.handle = None
+
+    # raw device buffers
+    def malloc(self, nbytes: int) -> int:
+        p = ctypes.c_void_p()
+        check(self.lib.ovfcc_device_malloc(self.handle, nbytes, ctypes.byref(p)))
+        return p.value
+
+    def free(self, ptr: int) -> None:
+        check(self.lib.ovfcc_device_free(self.handle, ctypes.c_void_p(ptr)))
+
+    def upload(self, ptr: int, a: np.ndarray) -> None:
+        a = np.ascontiguousarray(a)
+        check(self.lib.ovfcc_memcpy_h2d(self.handle, ctypes.c_void_p(ptr), _vp(a), a.nbytes))
+
+    def download(self, ptr: int, shape, dtype) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        check(self.lib.ovfcc_memcpy_d2h(self.handle, _vp(out), ctypes.c_void_p(ptr), out.nbytes))
+        return out
+
+    def copy_bandwidth(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
+        """GB/s (read + write) of the plain copy kernel."""
+        src, dst = self.malloc(nbytes), self.malloc(nbytes)
+        ms = ctypes.c_float()
+        try:
+            check(self.lib.ovfcc_bench_copy(self.handle, ctypes.c_void_p(dst), ctypes.c_void_p(src), nbytes, iters,
+                                            ctypes.byref(ms)))
+        finally:
+            self.free(src)
+            self.free(dst)
+        return 2.0 * nbytes * iters / (ms.value * 1e-3) / 1e9
+
+
+class CompressedWeights:
+    """Repacked, device-resident constants of one FullyConnectedCompressed node."""
+
+    def __init__(self, device: Device, W: np.ndarray, weight_scales: np.ndarray, weight_zero_points=None, bias=None, *,
+                 N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False):
+        self.device = device
+        self.N, self.K, self.group_size = N, K, group_size
+        self.desc = make_desc(N, K, group_size, w_type, zp_type if weight_zero_points is not None else "none",
+                              zp_scalar, bias is not None)
+        W = np.ascontiguousarray(W)
+        s = np.ascontiguousarray(weight_scales, dtype=np.float16)
+        z = None if weight_zero_points is None else np.ascontiguousarray(weight_zero_points, dtype=np.uint8)
+        b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float16)
+        h = ctypes.c_void_p()
+        check(device.lib.ovfcc_weights_create(device.handle, ctypes.byref(self.desc), _vp(W), _vp(s), _vp(z), _vp(b),
+                                              ctypes.byref(h)))
+        self.handle = h
+
+    @classmethod
+    def from_case(cls, device: Device, c) -> "CompressedWeights":
+        return cls(device, c.w, c.scale, c.zp, c.bias, N=c.N, K=c.K, group_size=c.group_size, w_type=c.w_type,
+                   zp_type=c.zp_type, zp_scalar=c.zp_scalar)
+
+    def clone(self) -> "CompressedWeights":
+        """Second device copy at distinct addresses (no host work)."""
+        other = object.__new__(CompressedWeights)
+        other.device, other.N, other.K, other.group_size, other.desc = (self.device, self.N, self.K,
+                                                                        self.group_size, self.desc)
+        h = ctypes.c_void_p()
+        check(self.device.lib.ovfcc_weights_clone(self.handle, ctypes.byref(h)))
+        other.handle = h
+        return other
+
+    @property
+    def tiled(self) -> bool:
+        return bool(self.device.lib.ovfcc_weights_is_tiled(self.handle))
+
+    @property
+    def device_bytes(self) -> int:
+        return int(self.device.lib.ovfcc_weights_device_bytes(self.handle))
+
+    def close(self):
+        if self.handle:
+            self.device.lib.ovfcc_weights_destroy(self.handle)
+            self.handle = None
+
+
+class InferRequest:
+    """One stream of execution (ov::ISyncInferRequest for this node)."""
+
+    def __init__(self, device: Device):
+        self.device = device
+        h = ctypes.c_void_p()
+        check(device.lib.ovfcc_request_create(device.handle, ctypes.byref(h)))
+        self.handle = h
+
+    def close(self):
+        if self.handle:
+            self.device.lib.ovfcc_request_destroy(self.handle)
+            self.handle = None
+
+    def force_kernel(self, kernel: int = _lib.KERNEL_AUTO, split_k: int = 0) -> None:
+        check(self.device.lib.ovfcc_request_force_kernel(self.handle, kernel, split_k))
+
+    def infer(self, weights: CompressedWeights, X: np.ndarray) -> np.ndarray:
+        """X float16 [..., K] on the host -> Y float16 [..., N] (MatMul shape rules, transpose_b = true)."""
+        X = np.ascontiguousarray(X, dtype=np.float16)
+        if X.shape[-1] != weights.K:
+            raise OvfccError(_lib.EINVAL, f"last dimension of X is {X.shape[-1]}, expected K = {weights.K}")
+        M = int(np.prod(X.shape[:-1], dtype=np.int64))
+        Y = np.empty(X.shape[:-1] + (weights.N,), dtype=np.float16)
+        check(self.device.lib.ovfcc_fc_run(self.handle, weights.handle, _vp(X), _vp(Y), M))
+        return Y
+
+    def infer_device(self, weights: CompressedWeights, x_ptr: int, y_ptr: int, M: int) -> None:
+        check(self.device.lib.ovfcc_fc_run_device(self.handle, weights.handle, ctypes.c_void_p(x_ptr),
+                                                  ctypes.c_void_p(y_ptr), M))
+
+    def sync(self) -> None:
+        check(self.device.lib.ovfcc_request_sync(self.handle))
+
+    def last_kernel(self) -> dict:
+        info = KernelInfo()
+        check(self.device.lib.ovfcc_last_kernel_info(self.handle, ctypes.byref(info)))
+        return dict(kernel=info.kernel, name=info.name.decode(), grid=tuple(info.grid), block=info.block,
+                    split_k=info.split_k, tile_m=info.tile_m, tile_n=info.tile_n)
+
+    def bench_layers(self, layers: Sequence[CompressedWeights], x_ptr: int, y_ptr: int, M: int, warmup: int,
+                     iters: int, use_graph: bool = True) -> float:
+        """Milliseconds for `iters` passes over `layers`, HIP events on the launching stream."""
+        arr = (ctypes.c_void_p * len(layers))(*[w.handle for w in layers])
+        ms = ctypes.c_float()
+        check(self.device.lib.ovfcc_bench_layers(self.handle, arr, len(layers), ctypes.c_void_p(x_ptr),
+                                                 ctypes.c_void_p(y_ptr), M, warmup, iters, int(use_graph),
+                                                 ctypes.byref(ms)))
+        return ms.value
+
+
+# ---- host-only helpers (no GPU needed) ----
+
+def validate(desc: FcDesc) -> int:
+    return _lib.load().ovfcc_desc_validate(ctypes.byref(desc))
+
+
+def tiled_sizes(desc: FcDesc):
+    L = _lib.load()
+    a, b, c = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    check(L.ovfcc_tiled_sizes(ctypes.byref(desc), ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+    return a.value, b.value, c.value
+
+
+def repack_host(desc: FcDesc, W, scales, zp=None):
+    L = _lib.load()
+    wb, sb, zb = tiled_sizes(desc)
+    if wb == 0:
+        raise OvfccError(_lib.EUNSUPPORTED, "descriptor keeps the OpenVINO layout")
+    wt, st = np.empty(wb, np.uint8), np.empty(sb // 2, np.float16)
+    zt = np.empty(zb, np.uint8) if zb else None
+    W = np.ascontiguousarray(W)
+    scales = np.ascontiguousarray(scales, dtype=np.float16)
+    zp = None if zp is None else np.ascontiguousarray(zp, dtype=np.uint8)
+    check(L.ovfcc_repack_host(ctypes.byref(desc), _vp(W), _vp(scales), _vp(zp), _vp(wt), _vp(st), _vp(zt)))
+    return wt, st, zt
+
+
+def unrepack_host(desc: FcDesc, wt, st, zt=None):
+    L = _lib.load()
+    four = desc.w_type in (_lib.U4, _lib.I4)
+    ng = desc.K // desc.group_size
+    W = np.empty(desc.N * desc.K // 2 if four else desc.N * desc.K, np.uint8)
+    scales = np.empty((desc.N, ng), np.float16)
+    zp = None
+    if zt is not None:
+        zp = np.empty((desc.N * ng + 1) // 2 if desc.zp_type == _lib.U4 else desc.N * ng, np.uint8)
+    check(L.ovfcc_unrepack_host(ctypes.byref(desc), _vp(wt), _vp(st), _vp(zt), _vp(W), _vp(scales), _vp(zp)))
+    return W, scales, zp

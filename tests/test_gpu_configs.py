@@ -1,0 +1,134 @@
+"""GPU parity at the five benchmark configurations (real shapes).
+
+Small-M cases are checked in full against the oracle.  Large-M cases are checked on a seeded sample of
+rows against the oracle (all output channels), and over the full output through properties that do not
+need the oracle: duplicated activation rows give duplicated output rows, and doubling the activations
+doubles every output bit-exactly (a power-of-two scale commutes with every rounding on the path).
+"""
+import sys
+
+import numpy as np
+import pytest
+
+from openvino_amd import _lib, datagen, fc
+from parity import check_parity, oracle_y
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = fc.Device(0)
+    yield d
+    d.close()
+
+
+@pytest.fixture()
+def req(dev):
+    r = fc.InferRequest(dev)
+    yield r
+    r.close()
+
+
+def sampled_check(oracle, req, w, c, rows, what):
+    """GPU on all rows; oracle on `rows` sampled rows, every output channel."""
+    y = req.infer(w, c.x)
+    info = req.last_kernel()
+    rng = np.random.default_rng(99)
+    pick = np.sort(rng.choice(c.M, size=min(rows, c.M), replace=False))
+    ref = oracle_y(oracle, c, x=c.x[pick])
+    r = check_parity(oracle, y[pick], ref, c.K, f"{what} {info}")
+    say(f"   {what}: {info['name']} grid={info['grid']} split={info['split_k']} rel-L2={r[0]:.2e} max-abs={r[1]:.2e}")
+    return y
+
+
+def test_config1_u4_asym(oracle, dev, req):
+    say("config 1")
+    c = datagen.config1()
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        assert w.tiled
+        y = req.infer(w, c.x)
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
+        r = check_parity(oracle, y, oracle_y(oracle, c), c.K, "config1")
+        say(f"   config1 rel-L2={r[0]:.2e} max-abs={r[1]:.2e} {req.last_kernel()}")
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("shape", list(datagen.LLAMA3_8B_SHAPES))
+def test_config2_decode(oracle, dev, req, shape):
+    say(f"config 2 {shape}")
+    c = datagen.config2(shape, 32)
+    w = fc.CompressedWeights.from_case(dev, c)
+    ref = oracle_y(oracle, c)
+    try:
+        for M in (1, 4, 16, 32):
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            assert info["kernel"] == _lib.KERNEL_DECODE
+            r = check_parity(oracle, y, ref[:M], c.K, f"config2 {shape} M={M}")
+            say(f"   M={M}: split={info['split_k']} rel-L2={r[0]:.2e} max-abs={r[1]:.2e}")
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("shape", list(datagen.LLAMA3_8B_SHAPES))
+def test_config3_prefill(oracle, dev, req, shape):
+    say(f"config 3 {shape}")
+    c = datagen.config3(shape, 8192)
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        for M in (512, 2048, 8192):
+            sub = datagen.FcCase(M, c.K, c.N, c.group_size, c.w_type, c.zp_type, c.w, c.scale, c.zp, c.x[:M])
+            y = sampled_check(oracle, req, w, sub, 24, f"config3 {shape} M={M}")
+            assert req.last_kernel()["kernel"] == _lib.KERNEL_PREFILL
+            if M == 2048:
+                # full-output properties
+                y2 = req.infer(w, (sub.x * np.float16(2)))
+                assert np.array_equal((y.astype(np.float32) * 2).astype(np.float16).view(np.uint16),
+                                      y2.view(np.uint16)), "doubling the activations must double every output"
+                xdup = np.repeat(sub.x[:1], M, axis=0)
+                yd = req.infer(w, xdup)
+                assert np.all(yd.view(np.uint16) == yd[:1].view(np.uint16)), "equal rows must give equal outputs"
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("shape", list(datagen.LLAMA3_70B_SHAPES))
+def test_config4_u8_per_channel(oracle, dev, req, shape):
+    say(f"config 4 {shape}")
+    c = datagen.config4(shape, 1024)
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        for M, rows in ((1, 1), (32, 32), (1024, 12)):
+            sub = datagen.FcCase(M, c.K, c.N, c.group_size, c.w_type, c.zp_type, c.w, c.scale, c.zp, c.x[:M])
+            sampled_check(oracle, req, w, sub, rows, f"config4 {shape} M={M}")
+    finally:
+        w.close()
+
+
+def test_config5_moe_experts(oracle, dev, req):
+    say("config 5")
+    routes = datagen.moe_routing()
+    assert sum(len(r) for r in routes) == 512
+    rng = np.random.default_rng(7)
+    for e, tokens in enumerate(routes):
+        M = len(tokens)
+        for which in ("gate", "up", "down"):
+            c = datagen.config5_expert(e, which, M)
+            w = fc.CompressedWeights.from_case(dev, c)
+            try:
+                y = req.infer(w, c.x)
+                info = req.last_kernel()
+                cols = np.sort(rng.choice(c.N, size=192, replace=False))
+                ref = oracle_y(oracle, c, n_index=cols)
+                r = check_parity(oracle, y[:, cols], ref, c.K, f"config5 expert {e} {which} M={M}")
+                say(f"   expert {e} {which} M={M}: {info['name']} rel-L2={r[0]:.2e} max-abs={r[1]:.2e}")
+            finally:
+                w.close()

@@ -1,0 +1,200 @@
+"""GPU parity: the HIP path through the C ABI against the CPU oracle.
+
+Tolerances (float path): relative L2 error <= 1e-3 and max-abs error <= 2e-2*sqrt(K/4096) against the
+fp32 dequantise-then-matmul oracle.  Golden vectors of the reference's own tests must come out exactly.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+from golden_cases import fc_cases
+from openvino_amd import _lib, datagen, fc
+from parity import check_parity, oracle_y, run_case
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = fc.Device(0)
+    yield d
+    d.close()
+
+
+@pytest.fixture()
+def req(dev):
+    r = fc.InferRequest(dev)
+    yield r
+    r.close()
+
+
+GOLD = fc_cases()
+
+
+@pytest.mark.parametrize("g", GOLD, ids=[g["id"] for g in GOLD])
+def test_golden_vectors_exact(dev, req, g):
+    """Every value of these cases is exact in float16, so the f16 device path must reproduce it bit for bit."""
+    say(f"golden {g['id']} N={g['N']} K={g['K']}")
+    c = datagen.FcCase(g["M"], g["K"], g["N"], g["group_size"], g["w_type"], "none" if g["zp"] is None else "u8",
+                       g["w"], g["scale"].astype(np.float16), g["zp"], g["x"].astype(np.float16),
+                       None if g["bias"] is None else g["bias"].astype(np.float16), zp_scalar=g["zp_scalar"])
+    x = c.x.reshape(g["x_shape"])
+    y, info = run_case(dev, req, c, x=x)
+    assert y.shape == tuple(g["x_shape"][:-1]) + (g["N"],)
+    assert np.array_equal(y.reshape(g["M"], g["N"]).astype(np.float32), g["expected"]), (g["source"], info)
+
+
+@pytest.mark.parametrize("n_pad", [16, 128])
+@pytest.mark.parametrize("M", [1, 40])
+def test_golden_accumulation_on_tiled_kernels(dev, req, n_pad, M):
+    """The int4 accumulation vector (all weights 1, all activations 1, K = 4096) widened to a tiled shape:
+    every output is exactly 4096 on the decode and the prefill kernel."""
+    say(f"accumulation N={n_pad} M={M}")
+    c = datagen.FcCase(M, 4096, n_pad, 128, "u4", "none", np.full(n_pad * 2048, 0x11, np.uint8),
+                       np.ones((n_pad, 32), np.float16), None, np.ones((M, 4096), np.float16))
+    y, info = run_case(dev, req, c)
+    assert info["kernel"] != _lib.KERNEL_PLAIN
+    assert np.all(y.astype(np.float32) == 4096.0), info
+
+
+SMALL = [
+    # w_type, zp_type, N, K, G, with_bias
+    ("u4", "u4", 128, 512, 128, False), ("u4", "none", 256, 256, 128, True), ("i4", "none", 128, 1024, 128, False),
+    ("i4", "u4", 128, 512, 256, True), ("u4", "u8", 384, 384, 128, False), ("u8", "u8", 128, 512, 512, False),
+    ("u8", "none", 128, 256, 128, True), ("u8", "u8", 256, 384, 128, False), ("i8", "none", 128, 256, 256, False),
+    ("u4", "u4", 48, 256, 128, False),      # tiled, N not a multiple of 128: decode kernel in 32-row chunks
+    ("u4", "u4", 40, 200, 50, True),        # untiled: plain kernel
+    ("i4", "none", 24, 96, 32, False),      # untiled
+    ("u8", "u8", 8, 6, 6, False),
+]
+MS = [1, 2, 3, 15, 16, 17, 31, 32, 33, 63, 65, 130, 257]
+
+
+@pytest.mark.parametrize("wt,zt,N,K,G,bias", SMALL)
+def test_small_shapes_all_row_counts(oracle, dev, req, wt, zt, N, K, G, bias):
+    c = datagen.make_case(11, max(MS), K, N, wt, G, zt, with_bias=bias)
+    w = fc.CompressedWeights.from_case(dev, c)
+    ref = oracle_y(oracle, c)
+    seen = set()
+    try:
+        for M in MS:
+            say(f"small {wt}/{zt} N={N} K={K} G={G} M={M}")
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            seen.add(info["name"])
+            check_parity(oracle, y, ref[:M], K, f"{wt}/{zt} N={N} K={K} M={M} {info}")
+    finally:
+        w.close()
+    if w.desc.N % 16 == 0 and K % 128 == 0 and G % 128 == 0:
+        assert "fcc_plain" not in seen
+
+
+def test_scalar_zero_point_and_3d_activations(oracle, dev, req):
+    say("scalar zp, 3-D x")
+    c = datagen.make_case(5, 6, 256, 128, "u8", 256, "u8", zp_range=(100, 157))
+    c.zp = c.zp[:1].copy()
+    c.zp_scalar = True
+    x3 = c.x.reshape(2, 3, 256)
+    y, info = run_case(dev, req, c, x=x3)
+    assert y.shape == (2, 3, 128)
+    check_parity(oracle, y.reshape(6, 128), oracle_y(oracle, c), 256, str(info))
+    c4 = datagen.make_case(6, 5, 256, 64, "u4", 128, "u4")
+    c4.zp = np.array([0x07], np.uint8)
+    c4.zp_scalar = True
+    y, info = run_case(dev, req, c4)
+    check_parity(oracle, y, oracle_y(oracle, c4), 256, str(info))
+
+
+def test_zero_rows(dev, req):
+    say("M = 0")
+    c = datagen.make_case(5, 0, 256, 128, "u4", 128, "u4")
+    y, _ = run_case(dev, req, c)
+    assert y.shape == (0, 128)
+
+
+@pytest.mark.parametrize("split", [1, 2, 3, 8, 32])
+@pytest.mark.parametrize("M", [1, 20])
+def test_decode_split_k_is_deterministic(oracle, dev, req, split, M):
+    """Any split gives the oracle's answer, and repeated launches give identical bits (the reduction order is
+    fixed and the arrival counters return to zero)."""
+    say(f"split {split} M={M}")
+    c = datagen.make_case(21, M, 4096, 256, "i4", 128, "none")
+    w = fc.CompressedWeights.from_case(dev, c)
+    ref = oracle_y(oracle, c)
+    try:
+        req.force_kernel(_lib.KERNEL_DECODE, split)
+        first = req.infer(w, c.x)
+        assert req.last_kernel()["split_k"] <= max(1, split)
+        check_parity(oracle, first, ref, 4096, f"split {split}")
+        for _ in range(5):
+            assert np.array_equal(req.infer(w, c.x).view(np.uint16), first.view(np.uint16))
+    finally:
+        req.force_kernel()
+        w.close()
+
+
+def test_kernel_policy(dev, req):
+    say("policy")
+    c = datagen.make_case(3, 64, 256, 128, "u4", 128, "u4")
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        assert w.tiled
+        req.infer(w, c.x[:1])
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
+        req.infer(w, c.x[:32])
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
+        req.infer(w, c.x[:33])
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_PREFILL
+        req.force_kernel(_lib.KERNEL_PLAIN)
+        with pytest.raises(fc.OvfccError):
+            req.infer(w, c.x[:1])
+        req.force_kernel(_lib.KERNEL_DECODE)
+        with pytest.raises(fc.OvfccError):
+            req.infer(w, c.x[:33])
+        req.force_kernel()
+        with pytest.raises(fc.OvfccError):
+            req.infer(w, c.x[:, :100])
+    finally:
+        w.close()
+
+
+def test_decode_and_prefill_agree(oracle, dev, req):
+    """Same inputs through both tiled kernels at M = 32 (full output, every tile)."""
+    say("decode vs prefill")
+    c = datagen.make_case(31, 32, 4096, 1024, "u4", 128, "u4")
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        req.force_kernel(_lib.KERNEL_DECODE)
+        yd = req.infer(w, c.x)
+        req.force_kernel(_lib.KERNEL_PREFILL)
+        yp = req.infer(w, c.x)
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_PREFILL
+    finally:
+        req.force_kernel()
+        w.close()
+    ref = oracle_y(oracle, c)
+    check_parity(oracle, yd, ref, 4096, "decode")
+    check_parity(oracle, yp, ref, 4096, "prefill")
+    assert oracle.rel_l2(yd.astype(np.float32), yp.astype(np.float32)) < 1e-3
+
+
+def test_two_requests_interleaved(oracle, dev):
+    """Two requests (streams) over the same weights give the same bits as one."""
+    say("two requests")
+    c = datagen.make_case(41, 8, 2048, 512, "i4", 128, "none")
+    w = fc.CompressedWeights.from_case(dev, c)
+    a, b = fc.InferRequest(dev), fc.InferRequest(dev)
+    try:
+        ya = a.infer(w, c.x)
+        yb = b.infer(w, c.x[::-1].copy())
+        assert np.array_equal(ya.view(np.uint16), yb[::-1].view(np.uint16))
+    finally:
+        a.close()
+        b.close()
+        w.close()
