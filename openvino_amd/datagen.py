@@ -35,7 +35,7 @@ class FcCase:
     K: int
     N: int
     group_size: int
-    w_type: str                 # "u4" | "i4" | "u8"
+    w_type: str                 # "u4" | "i4" | "u8" | "i8"
     zp_type: str                # "none" | "u4" | "u8"
     w: np.ndarray               # raw bytes
     scale: np.ndarray           # float16 [N, K/G]
@@ -51,7 +51,7 @@ class FcCase:
 
     def algorithmic_bytes(self) -> int:
         """W + S + ZP + X + Y, the traffic one call cannot avoid."""
-        bits = 8 if self.w_type == "u8" else 4
+        bits = 8 if self.w_type in ("u8", "i8") else 4
         ng = self.n_groups
         zp = {"none": 0, "u4": self.N * ng // 2, "u8": self.N * ng}[self.zp_type]
         if self.zp_scalar:
@@ -92,6 +92,8 @@ def make_case(seed: int, M: int, K: int, N: int, w_type: str = "u4", group_size:
         w = pack_nibbles(rng.integers(-8, 8, size=N * K, dtype=np.int8))
     elif w_type == "u8":
         w = rng.integers(0, 256, size=N * K, dtype=np.uint8)
+    elif w_type == "i8":
+        w = rng.integers(-128, 128, size=N * K, dtype=np.int8).view(np.uint8)
     else:
         raise ValueError(w_type)
     scale = rng.uniform(scale_range[0], scale_range[1], size=(N, ng)).astype(np.float16)

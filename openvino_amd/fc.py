@@ -89,7 +89,7 @@ class CompressedWeights:
         self.N, self.K, self.group_size = N, K, group_size
         self.desc = make_desc(N, K, group_size, w_type, zp_type if weight_zero_points is not None else "none",
                               zp_scalar, bias is not None)
-        W = np.ascontiguousarray(W)
+        W = np.ascontiguousarray(W).view(np.uint8)
         s = np.ascontiguousarray(weight_scales, dtype=np.float16)
         z = None if weight_zero_points is None else np.ascontiguousarray(weight_zero_points, dtype=np.uint8)
         b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float16)

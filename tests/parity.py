@@ -21,15 +21,22 @@ def oracle_y(o, c: datagen.FcCase, x=None, n_index=None, acc_f64=False):
                           acc_f64=acc_f64)
 
 
-def check_parity(o, y_gpu, y_ref, K, what=""):
-    """Both north-star bounds; returns (rel_l2, max_abs) for reporting."""
+def check_parity(o, y_gpu, y_ref, K, what="", output_rounding_slack=False):
+    """Both north-star bounds; returns (rel_l2, max_abs) for reporting.
+
+    The max-abs bound 2e-2*sqrt(K/4096) is stated for the benchmark distributions.  Tests on other
+    distributions (small K, large outputs) set output_rounding_slack, which adds half a float16 ulp of the
+    largest reference output: the rounding of the f16 result itself, which no kernel can avoid."""
     y = np.asarray(y_gpu, dtype=np.float32)
     assert y.shape == y_ref.shape, (what, y.shape, y_ref.shape)
     assert np.all(np.isfinite(y)), what
     rl2 = o.rel_l2(y, y_ref)
     mab = o.max_abs(y, y_ref)
+    limit = max_abs_limit(K)
+    if output_rounding_slack and y_ref.size:
+        limit += float(np.max(np.abs(y_ref))) * 2.0 ** -11
     assert rl2 <= REL_L2_MAX, f"{what}: rel-L2 {rl2:.3e} > {REL_L2_MAX}"
-    assert mab <= max_abs_limit(K), f"{what}: max-abs {mab:.3e} > {max_abs_limit(K):.3e}"
+    assert mab <= limit, f"{what}: max-abs {mab:.3e} > {limit:.3e}"
     return rl2, mab
 
 

@@ -88,7 +88,7 @@ def test_small_shapes_all_row_counts(oracle, dev, req, wt, zt, N, K, G, bias):
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
             seen.add(info["name"])
-            check_parity(oracle, y, ref[:M], K, f"{wt}/{zt} N={N} K={K} M={M} {info}")
+            check_parity(oracle, y, ref[:M], K, f"{wt}/{zt} N={N} K={K} M={M} {info}", output_rounding_slack=True)
     finally:
         w.close()
     if w.desc.N % 16 == 0 and K % 128 == 0 and G % 128 == 0:
@@ -103,12 +103,12 @@ def test_scalar_zero_point_and_3d_activations(oracle, dev, req):
     x3 = c.x.reshape(2, 3, 256)
     y, info = run_case(dev, req, c, x=x3)
     assert y.shape == (2, 3, 128)
-    check_parity(oracle, y.reshape(6, 128), oracle_y(oracle, c), 256, str(info))
+    check_parity(oracle, y.reshape(6, 128), oracle_y(oracle, c), 256, str(info), output_rounding_slack=True)
     c4 = datagen.make_case(6, 5, 256, 64, "u4", 128, "u4")
     c4.zp = np.array([0x07], np.uint8)
     c4.zp_scalar = True
     y, info = run_case(dev, req, c4)
-    check_parity(oracle, y, oracle_y(oracle, c4), 256, str(info))
+    check_parity(oracle, y, oracle_y(oracle, c4), 256, str(info), output_rounding_slack=True)
 
 
 def test_zero_rows(dev, req):
