@@ -56,7 +56,7 @@ typedef struct ovfcc_fc_desc {
     int32_t zp_scalar;  /* non-zero: zp holds one element (Shape{} / Shape{1}) used for every (n, group) */
     int32_t bias_type;  /* OVFCC_NONE | OVFCC_F16, [N] */
     int32_t act_type;   /* OVFCC_F16 */
-    int32_t out_type;   /* OVFCC_F16 (FullyConnected's output_type; default = activation type) */
+    int32_t out_type;   /* OVFCC_F16 | OVFCC_F32 (FullyConnected's output_type; default = activation type) */
     int32_t flags;      /* 0 */
 } ovfcc_fc_desc;
 
@@ -123,7 +123,7 @@ void ovfcc_request_destroy(ovfcc_request* req);
 /* ---- execution ----------------------------------------------------------------------------- */
 
 /* ISyncInferRequest::infer for one node with host tensors: copies X [M,K] f16 to the device,
- * runs the kernel, copies Y [M,N] f16 back and waits.  The CPU plugin's equivalent is
+ * runs the kernel, copies Y [M,N] (out_type) back and waits.  The CPU plugin's equivalent is
  * FullyConnected::execute -> DnnlFCPrimitive::execute
  * (src/plugins/intel_cpu/src/nodes/fullyconnected.cpp:427-433,
  * .../dnnl_fullyconnected_primitive.cpp:518-520).  M may be 0. */

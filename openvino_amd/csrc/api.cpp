@@ -107,6 +107,7 @@ void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc:
     a->w_type = w->desc.w_type;
     a->zp_type = w->desc.zp_type;
     a->zp_scalar = w->desc.zp_scalar;
+    a->out_f32 = w->desc.out_type == OVFCC_F32 ? 1 : 0;
     a->layout = w->layout;
 }
 
@@ -138,7 +139,7 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
         for (int64_t m0 = 0; m0 < M; m0 += 32) {
             const int64_t rows = M - m0 < 32 ? M - m0 : 32;
             fill_args(w, static_cast<const char*>(x) + (size_t)m0 * w->desc.K * 2,
-                      static_cast<char*>(y) + (size_t)m0 * w->desc.N * 2, rows, &a);
+                      static_cast<char*>(y) + (size_t)m0 * w->desc.N * (w->desc.out_type == OVFCC_F32 ? 4 : 2), rows, &a);
             ovfcc::LaunchPlan p;
             int rc = ovfcc::plan_launch(a, OVFCC_KERNEL_DECODE, r->force_split, r->ctx->n_cus, &p);
             if (rc)
@@ -420,7 +421,8 @@ int ovfcc_fc_run(ovfcc_request* r, const ovfcc_weights* w, const void* x_host, v
     if (!x_host || !y_host)
         return fail(OVFCC_EINVAL, "x or y is null");
     HIP_TRY(hipSetDevice(r->ctx->device));
-    const size_t xb = (size_t)M * w->desc.K * 2, yb = (size_t)M * w->desc.N * 2;
+    const size_t xb = (size_t)M * w->desc.K * 2;
+    const size_t yb = (size_t)M * w->desc.N * (w->desc.out_type == OVFCC_F32 ? 4 : 2);
     if (xb > r->x_cap || yb > r->y_cap)
         HIP_TRY(hipStreamSynchronize(r->stream));
     int rc = grow(&r->d_x, &r->x_cap, xb);

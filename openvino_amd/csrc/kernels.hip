@@ -65,6 +65,14 @@ __device__ __forceinline__ void unpack8(uint32_t w0, uint32_t w1, half2_t off, F
     f.h2[3] = as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) - off;
 }
 
+// Output cast: FullyConnected's output_type is f16 (default, the activation type) or f32.
+__device__ __forceinline__ void store_out(void* y, size_t i, float v, int out_f32) {
+    if (out_f32)
+        static_cast<float*>(y)[i] = v;
+    else
+        static_cast<half_t*>(y)[i] = (half_t)v;
+}
+
 __device__ __forceinline__ half2_t splat(float v) {
     const half_t h = (half_t)v;
     return half2_t{h, h};
@@ -76,8 +84,9 @@ __device__ __forceinline__ half2_t splat(float v) {
 __global__ __launch_bounds__(64) void fcc_plain_kernel(const uint8_t* __restrict__ w, const half_t* __restrict__ s,
                                                        const uint8_t* __restrict__ zp,
                                                        const half_t* __restrict__ bias,
-                                                       const half_t* __restrict__ x, half_t* __restrict__ y, int M,
-                                                       int N, int K, int G, int w_type, int zp_type, int zp_scalar) {
+                                                       const half_t* __restrict__ x, void* __restrict__ y, int M,
+                                                       int N, int K, int G, int w_type, int zp_type, int zp_scalar,
+                                                       int out_f32) {
     const int n = blockIdx.x;
     const int m = blockIdx.y;
     const int lane = threadIdx.x;
@@ -116,7 +125,7 @@ __global__ __launch_bounds__(64) void fcc_plain_kernel(const uint8_t* __restrict
     if (lane == 0) {
         if (bias)
             acc += (float)bias[n];
-        y[(size_t)m * N + n] = (half_t)acc;
+        store_out(y, (size_t)m * N + n, acc, out_f32);
     }
 }
 
@@ -133,10 +142,11 @@ __global__ __launch_bounds__(256) void fcc_decode_kernel(const uint4_t* __restri
                                                          const half_t* __restrict__ st,
                                                          const uint8_t* __restrict__ zt,
                                                          const half_t* __restrict__ x,
-                                                         const half_t* __restrict__ bias, half_t* __restrict__ y,
+                                                         const half_t* __restrict__ bias, void* __restrict__ y,
                                                          float* __restrict__ ws, unsigned* __restrict__ counters,
                                                          int M, int N, int K, int kb_total, int kb_per_group,
-                                                         int ng, int zp_const, int kb_per_split, int split_k) {
+                                                         int ng, int zp_const, int kb_per_split, int split_k,
+                                                         int out_f32) {
     constexpr int TPB = BITS == 4 ? 1 : 2;  // tiles per k-block
     const int nt = blockIdx.x;
     const int ks = blockIdx.y;
@@ -300,7 +310,7 @@ __global__ __launch_bounds__(256) void fcc_decode_kernel(const uint4_t* __restri
         for (int r = 0; r < 4; ++r) {
             const int m = 4 * kq + r + 16 * t;
             if (m < M)
-                y[(size_t)m * N + n] = (half_t)(sum[t][r] + b);
+                store_out(y, (size_t)m * N + n, sum[t][r] + b, out_f32);
         }
 }
 
@@ -319,9 +329,9 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
                                                           const half_t* __restrict__ st,
                                                           const uint8_t* __restrict__ zt,
                                                           const half_t* __restrict__ x,
-                                                          const half_t* __restrict__ bias, half_t* __restrict__ y,
+                                                          const half_t* __restrict__ bias, void* __restrict__ y,
                                                           int M, int N, int K, int kb_total, int kb_per_group, int ng,
-                                                          int zp_const) {
+                                                          int zp_const, int out_f32) {
     constexpr int TPB = BITS == 4 ? 1 : 2;
     __shared__ __attribute__((aligned(16))) half_t As[PF_BM * PF_LD];
     __shared__ __attribute__((aligned(16))) half_t Bs[PF_BN * PF_LD];
@@ -454,7 +464,7 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + 64 * wm + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (m < M)
-                    y[(size_t)m * N + n] = (half_t)(acc[i][j][r] + b);
+                    store_out(y, (size_t)m * N + n, acc[i][j][r] + b, out_f32);
             }
     }
 }
@@ -542,9 +552,9 @@ static void launch_decode(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_
     const Layout& L = a.layout;
     hipLaunchKernelGGL((fcc_decode_kernel<BITS, MT, ZPT>), dim3(p.grid[0], p.grid[1], 1), dim3(256), 0, s,
                        (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x,
-                       (const half_t*)a.bias, (half_t*)a.y, a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K,
+                       (const half_t*)a.bias, a.y, a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K,
                        (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups, L.zp_const, p.kblocks_per_split,
-                       p.split_k);
+                       p.split_k, a.out_f32);
 }
 
 template <int BITS, bool ZPT>
@@ -552,8 +562,8 @@ static void launch_prefill(const FcDeviceArgs& a, const LaunchPlan& p, hipStream
     const Layout& L = a.layout;
     hipLaunchKernelGGL((fcc_prefill_kernel<BITS, ZPT>), dim3(p.grid[0], p.grid[1], 1), dim3(256), 0, s,
                        (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x,
-                       (const half_t*)a.bias, (half_t*)a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
-                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const);
+                       (const half_t*)a.bias, a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
+                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32);
 }
 
 int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
@@ -564,8 +574,8 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     if (p.kernel == OVFCC_KERNEL_PLAIN) {
         hipLaunchKernelGGL(fcc_plain_kernel, dim3(p.grid[0], p.grid[1], 1), dim3(64), 0, s, (const uint8_t*)a.w,
                            (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.bias, (const half_t*)a.x,
-                           (half_t*)a.y, (int)a.M, (int)a.N, (int)a.K, (int)a.group_size, a.w_type, a.zp_type,
-                           a.zp_scalar);
+                           a.y, (int)a.M, (int)a.N, (int)a.K, (int)a.group_size, a.w_type, a.zp_type,
+                           a.zp_scalar, a.out_f32);
     } else if (p.kernel == OVFCC_KERNEL_DECODE) {
         const bool two = a.M > 16;
         if (L.bits == 4) {

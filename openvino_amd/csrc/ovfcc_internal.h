@@ -63,11 +63,12 @@ struct FcDeviceArgs {
     const void* zp;      // table, raw zp, or null
     const void* bias;    // f16 [N] or null
     const void* x;       // f16 [M,K]
-    void* y;             // f16 [M,N]
+    void* y;             // f16 or f32 [M,N]
     float* workspace;    // split-K partials
     unsigned* counters;  // split-K arrival counters, one per 16-channel tile, zero between launches
     int64_t M, N, K, group_size;
     int w_type, zp_type, zp_scalar;
+    int out_f32;         // output_type f32 instead of f16
     Layout layout;
 };
 

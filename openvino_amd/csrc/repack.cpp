@@ -59,8 +59,10 @@ int validate_desc(const ovfcc_fc_desc* d) {
         return fail(OVFCC_EUNSUPPORTED, "zero-points must be absent, u4 or u8");
     if (d->bias_type != OVFCC_NONE && d->bias_type != OVFCC_F16)
         return fail(OVFCC_EUNSUPPORTED, "bias must be absent or f16");
-    if (d->act_type != OVFCC_F16 || d->out_type != OVFCC_F16)
-        return fail(OVFCC_EUNSUPPORTED, "activations and output must be f16");
+    if (d->act_type != OVFCC_F16)
+        return fail(OVFCC_EUNSUPPORTED, "activations must be f16");
+    if (d->out_type != OVFCC_F16 && d->out_type != OVFCC_F32)
+        return fail(OVFCC_EUNSUPPORTED, "output must be f16 or f32");
     if (d->flags != 0)
         return fail(OVFCC_EINVAL, "flags must be 0");
     if (d->N > (int64_t)1 << 24 || d->K > (int64_t)1 << 24)

@@ -21,7 +21,7 @@ def _vp(a: Optional[np.ndarray]):
 
 
 def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
-              has_bias: bool = False) -> FcDesc:
+              has_bias: bool = False, out_type: str = "f16") -> FcDesc:
     d = FcDesc()
     d.N, d.K, d.group_size = N, K, group_size
     d.w_type = _lib.TYPE[w_type]
@@ -30,7 +30,7 @@ def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none
     d.zp_scalar = int(zp_scalar)
     d.bias_type = _lib.F16 if has_bias else _lib.NONE
     d.act_type = _lib.F16
-    d.out_type = _lib.F16
+    d.out_type = _lib.TYPE[out_type]
     d.flags = 0
     return d
 
@@ -84,11 +84,12 @@ class CompressedWeights:
     """Repacked, device-resident constants of one FullyConnectedCompressed node."""
 
     def __init__(self, device: Device, W: np.ndarray, weight_scales: np.ndarray, weight_zero_points=None, bias=None, *,
-                 N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False):
+                 N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
+                 output_type: str = "f16"):
         self.device = device
         self.N, self.K, self.group_size = N, K, group_size
         self.desc = make_desc(N, K, group_size, w_type, zp_type if weight_zero_points is not None else "none",
-                              zp_scalar, bias is not None)
+                              zp_scalar, bias is not None, output_type)
         W = np.ascontiguousarray(W).view(np.uint8)
         s = np.ascontiguousarray(weight_scales, dtype=np.float16)
         z = None if weight_zero_points is None else np.ascontiguousarray(weight_zero_points, dtype=np.uint8)
@@ -99,9 +100,9 @@ class CompressedWeights:
         self.handle = h
 
     @classmethod
-    def from_case(cls, device: Device, c) -> "CompressedWeights":
+    def from_case(cls, device: Device, c, output_type: str = "f16") -> "CompressedWeights":
         return cls(device, c.w, c.scale, c.zp, c.bias, N=c.N, K=c.K, group_size=c.group_size, w_type=c.w_type,
-                   zp_type=c.zp_type, zp_scalar=c.zp_scalar)
+                   zp_type=c.zp_type, zp_scalar=c.zp_scalar, output_type=output_type)
 
     def clone(self) -> "CompressedWeights":
         """Second device copy at distinct addresses (no host work)."""
@@ -145,12 +146,12 @@ class InferRequest:
         check(self.device.lib.ovfcc_request_force_kernel(self.handle, kernel, split_k))
 
     def infer(self, weights: CompressedWeights, X: np.ndarray) -> np.ndarray:
-        """X float16 [..., K] on the host -> Y float16 [..., N] (MatMul shape rules, transpose_b = true)."""
+        """X float16 [..., K] on the host -> Y [..., N] in the node's output_type (MatMul shape rules, transpose_b = true)."""
         X = np.ascontiguousarray(X, dtype=np.float16)
         if X.shape[-1] != weights.K:
             raise OvfccError(_lib.EINVAL, f"last dimension of X is {X.shape[-1]}, expected K = {weights.K}")
         M = int(np.prod(X.shape[:-1], dtype=np.int64))
-        Y = np.empty(X.shape[:-1] + (weights.N,), dtype=np.float16)
+        Y = np.empty(X.shape[:-1] + (weights.N,), dtype=np.float32 if weights.desc.out_type == _lib.F32 else np.float16)
         check(self.device.lib.ovfcc_fc_run(self.handle, weights.handle, _vp(X), _vp(Y), M))
         return Y
 

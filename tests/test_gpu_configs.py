@@ -35,15 +35,16 @@ def req(dev):
     r.close()
 
 
-def sampled_check(oracle, req, w, c, rows, what):
+def sampled_check(oracle, req, w, c, rows, what, output_rounding_slack=False):
     """GPU on all rows; oracle on `rows` sampled rows, every output channel."""
     y = req.infer(w, c.x)
     info = req.last_kernel()
     rng = np.random.default_rng(99)
     pick = np.sort(rng.choice(c.M, size=min(rows, c.M), replace=False))
     ref = oracle_y(oracle, c, x=c.x[pick])
-    r = check_parity(oracle, y[pick], ref, c.K, f"{what} {info}")
-    say(f"   {what}: {info['name']} grid={info['grid']} split={info['split_k']} rel-L2={r[0]:.2e} max-abs={r[1]:.2e}")
+    r = check_parity(oracle, y[pick], ref, c.K, f"{what} {info}", output_rounding_slack=output_rounding_slack)
+    say(f"   {what}: {info['name']} grid={info['grid']} split={info['split_k']} out={y.dtype} "
+        f"rel-L2={r[0]:.2e} max-abs={r[1]:.2e}")
     return y
 
 
@@ -91,8 +92,11 @@ def test_config3_prefill(oracle, dev, req, shape):
             if M == 2048:
                 # full-output properties
                 y2 = req.infer(w, (sub.x * np.float16(2)))
-                assert np.array_equal((y.astype(np.float32) * 2).astype(np.float16).view(np.uint16),
-                                      y2.view(np.uint16)), "doubling the activations must double every output"
+                normal = np.abs(y.astype(np.float32)) >= 2.0 ** -13   # doubling a subnormal half rounds differently
+                want = (y.astype(np.float32) * 2).astype(np.float16)
+                bad = int(np.count_nonzero((want.view(np.uint16) != y2.view(np.uint16)) & normal))
+                assert bad == 0, f"doubling the activations must double every output ({bad} differ)"
+                assert np.all(np.abs(y2[~normal].astype(np.float32)) <= 2.0 ** -11)
                 xdup = np.repeat(sub.x[:1], M, axis=0)
                 yd = req.infer(w, xdup)
                 assert np.all(yd.view(np.uint16) == yd[:1].view(np.uint16)), "equal rows must give equal outputs"
@@ -102,15 +106,24 @@ def test_config3_prefill(oracle, dev, req, shape):
 
 @pytest.mark.parametrize("shape", list(datagen.LLAMA3_70B_SHAPES))
 def test_config4_u8_per_channel(oracle, dev, req, shape):
+    """Outputs of this distribution reach |y| > 128, where half a float16 ulp (0.0625) alone exceeds the max-abs
+    bound, so the bound proper is checked on the f32 output_type (the kernel's arithmetic before the output
+    cast); the f16 output must be exactly the rounding of that f32 output and meets the bound plus the cast's
+    own half ulp."""
     say(f"config 4 {shape}")
     c = datagen.config4(shape, 1024)
-    w = fc.CompressedWeights.from_case(dev, c)
+    w16 = fc.CompressedWeights.from_case(dev, c)
+    w32 = fc.CompressedWeights.from_case(dev, c, output_type="f32")
     try:
         for M, rows in ((1, 1), (32, 32), (1024, 12)):
             sub = datagen.FcCase(M, c.K, c.N, c.group_size, c.w_type, c.zp_type, c.w, c.scale, c.zp, c.x[:M])
-            sampled_check(oracle, req, w, sub, rows, f"config4 {shape} M={M}")
+            y32 = sampled_check(oracle, req, w32, sub, rows, f"config4 {shape} M={M}")
+            assert y32.dtype == np.float32
+            y16 = sampled_check(oracle, req, w16, sub, rows, f"config4 {shape} M={M}", output_rounding_slack=True)
+            assert np.array_equal(y32.astype(np.float16).view(np.uint16), y16.view(np.uint16))
     finally:
-        w.close()
+        w16.close()
+        w32.close()
 
 
 def test_config5_moe_experts(oracle, dev, req):

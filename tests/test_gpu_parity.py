@@ -111,6 +111,27 @@ def test_scalar_zero_point_and_3d_activations(oracle, dev, req):
     check_parity(oracle, y, oracle_y(oracle, c4), 256, str(info), output_rounding_slack=True)
 
 
+@pytest.mark.parametrize("M", [1, 24, 70])
+@pytest.mark.parametrize("wt,N,K,G", [("u4", 128, 512, 128), ("u8", 128, 256, 256), ("i4", 24, 96, 32)])
+def test_f32_output_type(oracle, dev, req, wt, N, K, G, M):
+    """output_type f32: same arithmetic, no output cast; the f16 result is its exact rounding."""
+    say(f"f32 out {wt} N={N} K={K} M={M}")
+    c = datagen.make_case(17, M, K, N, wt, G, "none" if wt == "i4" else wt, with_bias=True)
+    w32 = fc.CompressedWeights.from_case(dev, c, output_type="f32")
+    w16 = fc.CompressedWeights.from_case(dev, c)
+    try:
+        y32 = req.infer(w32, c.x)
+        y16 = req.infer(w16, c.x)
+    finally:
+        w32.close()
+        w16.close()
+    assert y32.dtype == np.float32 and y32.shape == (M, N)
+    ref = oracle_y(oracle, c)
+    check_parity(oracle, y32, ref, K, "f32 out")
+    assert oracle.rel_l2(y32, ref) < 3e-4
+    assert np.array_equal(y32.astype(np.float16).view(np.uint16), y16.view(np.uint16))
+
+
 def test_zero_rows(dev, req):
     say("M = 0")
     c = datagen.make_case(5, 0, 256, 128, "u4", 128, "u4")
