@@ -15,8 +15,9 @@
 //                       over the four waves of a workgroup (LDS reduction) and over workgroups
 //                       (partials + arrival counter; the last workgroup sums in fixed order).
 //   fcc_prefill_kernel  M > 32, tiled layout: 128x128 output tile per workgroup; weight tiles
-//                       are dequantised to f16 (q - zp) * s into LDS, activations staged in LDS,
-//                       v_mfma_f32_32x32x16_f16 with f32 accumulators.
+//                       are dequantised to f16 into LDS ((q - zp) * s for grouped scales, exact
+//                       q - zp with the scale applied to the f32 result for per-channel scales),
+//                       activations staged in LDS, v_mfma_f32_32x32x16_f16 with f32 accumulators.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -324,7 +325,7 @@ __global__ __launch_bounds__(256) void fcc_decode_kernel(const uint4_t* __restri
 // ------------------------------------------------------------------------------------------------
 constexpr int PF_BM = 128, PF_BN = 128, PF_BK = 64, PF_LD = PF_BK + 8;
 
-template <int BITS, bool ZP_TABLE>
+template <int BITS, bool ZP_TABLE, bool PRESCALE>
 __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restrict__ wt,
                                                           const half_t* __restrict__ st,
                                                           const uint8_t* __restrict__ zt,
@@ -406,9 +407,11 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
                 for (int jj = 0; jj < 2; ++jj) {
                     Frag8 b;
                     unpack4(half_w[jj], off_lo, off_hi, b);
+                    if constexpr (PRESCALE) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        b.h2[e] = b.h2[e] * sc;
+                        for (int e = 0; e < 4; ++e)
+                            b.h2[e] = b.h2[e] * sc;
+                    }
                     *reinterpret_cast<half8_t*>(&Bs[row * PF_LD + 32 * jj + 8 * kq]) = b.v;
                 }
             } else {
@@ -417,9 +420,11 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
                 for (int jj = 0; jj < 2; ++jj) {
                     Frag8 b;
                     unpack8(wd[2 * jj], wd[2 * jj + 1], off, b);
+                    if constexpr (PRESCALE) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        b.h2[e] = b.h2[e] * sc;
+                        for (int e = 0; e < 4; ++e)
+                            b.h2[e] = b.h2[e] * sc;
+                    }
                     *reinterpret_cast<half8_t*>(&Bs[row * PF_LD + 32 * jj + 8 * kq]) = b.v;
                 }
             }
@@ -458,13 +463,15 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
     for (int j = 0; j < 2; ++j) {
         const int n = n0 + 64 * wn + 32 * j + (lane & 31);
         const float b = bias ? (float)bias[n] : 0.f;
+        // one scale per output channel: applied here, to the f32 sum of exact integer products
+        const float cs = PRESCALE ? 1.f : (float)st[(size_t)(n >> 4) * ng * 16 + (n & 15)];
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + 64 * wm + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (m < M)
-                    store_out(y, (size_t)m * N + n, acc[i][j][r] + b, out_f32);
+                    store_out(y, (size_t)m * N + n, acc[i][j][r] * cs + b, out_f32);
             }
     }
 }
@@ -557,13 +564,23 @@ static void launch_decode(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_
                        p.split_k, a.out_f32);
 }
 
-template <int BITS, bool ZPT>
-static void launch_prefill(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+template <int BITS, bool ZPT, bool PRE>
+static void launch_prefill_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
-    hipLaunchKernelGGL((fcc_prefill_kernel<BITS, ZPT>), dim3(p.grid[0], p.grid[1], 1), dim3(256), 0, s,
+    hipLaunchKernelGGL((fcc_prefill_kernel<BITS, ZPT, PRE>), dim3(p.grid[0], p.grid[1], 1), dim3(256), 0, s,
                        (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x,
                        (const half_t*)a.bias, a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
                        (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32);
+}
+
+// Grouped scales are folded into the f16 weights in LDS; a single group per channel (G == K) keeps the
+// weights as exact integers and scales the f32 result once.
+template <int BITS, bool ZPT>
+static void launch_prefill(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    if (a.layout.groups == 1)
+        launch_prefill_impl<BITS, ZPT, false>(a, p, s);
+    else
+        launch_prefill_impl<BITS, ZPT, true>(a, p, s);
 }
 
 int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
