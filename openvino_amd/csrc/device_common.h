@@ -1,0 +1,98 @@
+// Device-side types and the register unpack shared by the tiled kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "ovfcc_internal.h"
+
+namespace ovfcc {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ half2_t as_half2(uint32_t u) {
+    return __builtin_bit_cast(half2_t, u);
+}
+__device__ __forceinline__ uint32_t as_u32(half2_t h) {
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+union Frag8 {
+    half8_t v;
+    uint32_t u[4];
+    half2_t h2[4];
+};
+
+// One dword of the 4-bit tile layout -> 8 exact halves (q - zp), elements 0..7 in order.
+// 0x6400 | q is the half 1024 + q; 0x5400 | (q << 4) is the half 64 + q.  Subtracting
+// (1024 + zp) resp. (64 + zp) is exact in half precision.
+__device__ __forceinline__ void unpack4(uint32_t w, half2_t off_lo, half2_t off_hi, Frag8& f) {
+    const uint32_t w8 = w >> 8;
+    f.h2[0] = as_half2((w & 0x000F000Fu) | 0x64006400u) - off_lo;
+    f.h2[1] = as_half2((w & 0x00F000F0u) | 0x54005400u) - off_hi;
+    f.h2[2] = as_half2((w8 & 0x000F000Fu) | 0x64006400u) - off_lo;
+    f.h2[3] = as_half2((w8 & 0x00F000F0u) | 0x54005400u) - off_hi;
+}
+
+// Two dwords of the 8-bit tile layout (8 consecutive inputs) -> 8 exact halves (q - zp).
+__device__ __forceinline__ void unpack8(uint32_t w0, uint32_t w1, half2_t off, Frag8& f) {
+    // byte permute: result bytes {w.b0, 0x64, w.b1, 0x64} = halves (1024 + b0, 1024 + b1)
+    f.h2[0] = as_half2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u)) - off;
+    f.h2[1] = as_half2(__builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)) - off;
+    f.h2[2] = as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)) - off;
+    f.h2[3] = as_half2(__builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) - off;
+}
+
+// The masks and magic numbers of the 4-bit unpack as values the compiler cannot fold: with register
+// operands (w & mask) | magic selects the single instruction v_and_or_b32, with literals it becomes two.
+// (Plain C on purpose: the compiler must see these VALU writes to keep its MFMA hazard spacing right.)
+struct Unpack4Consts {
+    uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
+};
+__device__ __forceinline__ Unpack4Consts unpack4_consts() {
+    Unpack4Consts c{0x000F000Fu, 0x00F000F0u, 0x64006400u, 0x54005400u};
+    asm volatile("" : "+s"(c.mask_lo), "+s"(c.mask_hi));
+    asm volatile("" : "+v"(c.magic_lo), "+v"(c.magic_hi));
+    return c;
+}
+
+// Biased variants: the halves 1024 + q (elements 0,1,4,5) and 64 + q (elements 2,3,6,7) of a 4-bit dword,
+// resp. 1024 + q for every element of two 8-bit dwords, without removing the bias.  A kernel that uses them
+// cancels bias and zero-point with one extra MFMA whose weight operand is the constant fragment
+// {-(1024 + zp), -(64 + zp), -(1024 + zp), -(64 + zp)} (resp. all -(1024 + zp)): the products are exact and
+// the f32 accumulator sees sum x * (bias + q) - sum x * (bias + zp).
+__device__ __forceinline__ void unpack4_biased(uint32_t w, const Unpack4Consts& c, Frag8& f) {
+    const uint32_t w8 = w >> 8;
+    f.u[0] = (w & c.mask_lo) | c.magic_lo;
+    f.u[1] = (w & c.mask_hi) | c.magic_hi;
+    f.u[2] = (w8 & c.mask_lo) | c.magic_lo;
+    f.u[3] = (w8 & c.mask_hi) | c.magic_hi;
+}
+
+__device__ __forceinline__ void unpack8_biased(uint32_t w0, uint32_t w1, Frag8& f) {
+    f.u[0] = __builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u);
+    f.u[1] = __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u);
+    f.u[2] = __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u);
+    f.u[3] = __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u);
+}
+
+// Output cast: FullyConnected's output_type is f16 (default, the activation type) or f32.
+__device__ __forceinline__ void store_out(void* y, size_t i, float v, int out_f32) {
+    if (out_f32)
+        static_cast<float*>(y)[i] = v;
+    else
+        static_cast<half_t*>(y)[i] = (half_t)v;
+}
+
+__device__ __forceinline__ half2_t splat(float v) {
+    const half_t h = (half_t)v;
+    return half2_t{h, h};
+}
+
+}  // namespace ovfcc

@@ -1,0 +1,287 @@
+// Decode kernel (M <= 32) over the tiled layout: a split-K streaming kernel.
+//
+// grid = (N/16, split_k), block = 64 * NW (NW = 4, 8 or 16 waves).  Workgroup (nt, ks) owns output channels
+// [16 nt, 16 nt + 16) and k-blocks [ks * kb_per_split, min(KB, (ks + 1) * kb_per_split)); wave w takes
+// k-blocks first + w, first + w + NW, ...  Every k-block is one (4-bit) or two (8-bit) 1 KiB tiles, read
+// with one 128-bit load per lane; DEPTH k-blocks per wave are kept in flight in registers together with
+// the matching activation fragments, so a wave never waits for a barrier before it can contract.
+//
+// Arithmetic per k-block: nibbles/bytes are unpacked in registers to the exact halves bias + q and contracted
+// against the activation rows on the matrix cores (A = activations, rows m; B = weights, columns n;
+// v_mfma_f32_16x16x32_f16, f32 result: lane holds column n = lane & 15, rows 4 (lane >> 4) + r); one more
+// MFMA per k-step against the constant fragment -(bias + zp) cancels bias and zero-point in the f32
+// accumulator, which keeps the vector ALU free for the unpack.  The group scale multiplies the f32 partial
+// sum of the k-block, so no weight is ever rounded.
+//
+// Reductions: the waves of a workgroup are summed through LDS in wave order.  With split_k > 1 every
+// workgroup writes its partial tile with device-scope stores, waits for them, and takes a ticket from a
+// per-tile arrival counter; the workgroup that draws the last ticket adds all partials in split order (the
+// result does not depend on arrival order) and returns the counter to zero for the next launch.
+#include "device_common.h"
+
+namespace ovfcc {
+
+template <int TPB, int MT>
+struct DecodeSlot {
+    uint4_t w[TPB];
+    half8_t a[MT][4];
+    half_t scale;
+    uint8_t zp;
+};
+
+template <int BITS, int MT, bool ZP_TABLE>
+__global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restrict__ wt,
+                                                          const half_t* __restrict__ st,
+                                                          const uint8_t* __restrict__ zt,
+                                                          const half_t* __restrict__ x,
+                                                          const half_t* __restrict__ bias, void* __restrict__ y,
+                                                          float* __restrict__ ws, unsigned* __restrict__ counters,
+                                                          int M, int N, int K, int kb_total, int kb_per_group,
+                                                          int ng, int zp_const, int kb_per_split, int split_k,
+                                                          int out_f32) {
+    constexpr int TPB = BITS == 4 ? 1 : 2;    // tiles per k-block
+    constexpr int DEPTH = (MT == 1 ? 4 : 2) / TPB;  // k-blocks in flight per wave (4 KiB of weights for M <= 16)
+    extern __shared__ float red[];            // [NW][MT * 256]
+    __shared__ unsigned ticket_s;
+
+    const int nt = blockIdx.x;
+    const int ks = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nw = blockDim.x >> 6;
+    const int col = lane & 15;
+    const int kq = lane >> 4;
+
+    const int kb_begin = ks * kb_per_split;
+    const int kb_end = min(kb_total, kb_begin + kb_per_split);
+    const int kb_first = kb_begin + wave;
+    const int cnt = kb_first < kb_end ? (kb_end - kb_first + nw - 1) / nw : 0;
+
+    // Every load goes through a buffer descriptor with hardware range checking: a lane whose offset lies
+    // beyond the buffer (an activation row >= M, a k-block past the end of this wave's share) reads zero and
+    // costs no memory traffic, so the loop below has no branches and every wait counts exactly.
+    constexpr unsigned kOob = 0x80000000u;
+    constexpr int kRsrcFlags = 0x00020000;
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint4_t*>(wt + (size_t)nt * kb_total * TPB * 64), 0, kb_total * TPB * kTileBytes, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<half_t*>(st + (size_t)nt * ng * 16), 0, ng * 32, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rz = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(ZP_TABLE ? zt + (size_t)nt * ng * 16 : zt), 0, ZP_TABLE ? ng * 16 : 0, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rx =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, M * K * 2, kRsrcFlags);
+    // activation fragment of this lane: row m = col (+16 for the second tile), inputs 8 kq ..+8 of each k-step
+    unsigned xbase[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = col + 16 * t;
+        xbase[t] = m < M ? (unsigned)(m * K + 8 * kq) * 2u : kOob;
+    }
+
+    // group index of a k-block without a division in the loop: kb_per_group == 1 -> kb, else the high word of
+    // kb * ceil(2^32 / kb_per_group) (exact for kb < 2^16)
+    const unsigned g_mul = kb_per_group == 1 ? 0u : (unsigned)((0x100000000ull + kb_per_group - 1) / kb_per_group);
+    auto issue = [&](int i, DecodeSlot<TPB, MT>& s) {
+        // bit 31 of every offset of a slot past the end of this wave's share is set: out of range, reads zero
+        const unsigned oob = (unsigned)((cnt - 1 - i) >> 31) & kOob;
+        const unsigned kb = (unsigned)(kb_first + nw * i);
+        const unsigned wofs = (kb * (unsigned)(TPB * kTileBytes) + lane * 16u) | oob;
+#pragma unroll
+        for (int t = 0; t < TPB; ++t)
+            s.w[t] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rw, wofs + t * kTileBytes, 0, 2));
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const unsigned xofs = (xbase[t] + kb * 256u) | oob;  // an invalid row keeps bit 31 of its base
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                s.a[t][j] =
+                    __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(rx, xofs + 64u * j, 0, 0));
+        }
+        const unsigned g = kb_per_group == 1 ? kb : __umulhi(kb, g_mul);
+        const unsigned sofs = (g * 16u + col) | oob;
+        s.scale = __builtin_bit_cast(half_t, __builtin_amdgcn_raw_buffer_load_b16(rs, sofs * 2u, 0, 0));
+        if constexpr (ZP_TABLE)
+            s.zp = __builtin_amdgcn_raw_buffer_load_b8(rz, sofs, 0, 0);
+    };
+
+    DecodeSlot<TPB, MT> slot[DEPTH];
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u)
+        issue(u, slot[u]);
+
+    float4_t acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+        acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const Unpack4Consts uc = unpack4_consts();
+    auto consume = [&](const DecodeSlot<TPB, MT>& s) {
+        const float zpv = ZP_TABLE ? (float)s.zp : (float)zp_const;
+        const float scale = (float)s.scale;
+        float4_t part[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+            part[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+        // weights enter the matrix cores with their unpack bias (1024 + q, 64 + q); a second MFMA against the
+        // constant fragment -(bias + zp) removes bias and zero-point inside the f32 accumulator
+        Frag8 bc;
+        if constexpr (BITS == 4) {
+            bc.h2[0] = bc.h2[2] = splat(-(1024.f + zpv));
+            bc.h2[1] = bc.h2[3] = splat(-(64.f + zpv));
+            const uint32_t wd[4] = {s.w[0].x, s.w[0].y, s.w[0].z, s.w[0].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                Frag8 b;
+                unpack4_biased(wd[j], uc, b);
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(s.a[t][j], b.v, part[t], 0, 0, 0);
+                    part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(s.a[t][j], bc.v, part[t], 0, 0, 0);
+                }
+            }
+        } else {
+            bc.h2[0] = bc.h2[1] = bc.h2[2] = bc.h2[3] = splat(-(1024.f + zpv));
+#pragma unroll
+            for (int i2 = 0; i2 < 2; ++i2) {
+                const uint32_t wd[4] = {s.w[i2].x, s.w[i2].y, s.w[i2].z, s.w[i2].w};
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+                    Frag8 b;
+                    unpack8_biased(wd[2 * jj], wd[2 * jj + 1], b);
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) {
+                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(s.a[t][2 * i2 + jj], b.v, part[t], 0, 0, 0);
+                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(s.a[t][2 * i2 + jj], bc.v, part[t], 0, 0, 0);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            acc[t].x += scale * part[t].x;
+            acc[t].y += scale * part[t].y;
+            acc[t].z += scale * part[t].z;
+            acc[t].w += scale * part[t].w;
+        }
+    };
+
+    // slots past the end of this wave's share hold zeros (weights, activations and scale) and add nothing
+    for (int i = 0; i < cnt; i += DEPTH) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            consume(slot[u]);
+            issue(i + u + DEPTH, slot[u]);
+        }
+    }
+
+    // ---- reduce the waves through LDS, in wave order; only rows < M carry data ----
+    float accv[MT][4];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        accv[t][0] = acc[t].x;
+        accv[t][1] = acc[t].y;
+        accv[t][2] = acc[t].z;
+        accv[t][3] = acc[t].w;
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (4 * kq + r + 16 * t < M)
+                red[(wave * MT + t) * 256 + r * 64 + lane] = accv[t][r];
+    __syncthreads();
+    if (wave != 0 && split_k == 1)
+        return;
+
+    float sum[MT][4];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            sum[t][r] = 0.f;
+            if (wave == 0 && 4 * kq + r + 16 * t < M)
+                for (int w = 0; w < nw; ++w)
+                    sum[t][r] += red[(w * MT + t) * 256 + r * 64 + lane];
+        }
+
+    if (split_k > 1) {
+        // partial layout: [nt][ks][MT][4 r][64 lanes] floats; only rows < M are written and read
+        float* mine = ws + ((size_t)nt * split_k + ks) * (MT * 256);
+        if (wave == 0) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (4 * kq + r + 16 * t < M)
+                        __hip_atomic_store(mine + (t * 4 + r) * 64 + lane, sum[t][r], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+            // device-scope stores write through; once they are acknowledged the ticket may be drawn
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        __syncthreads();
+        if (threadIdx.x == 0)
+            ticket_s = __hip_atomic_fetch_add(counters + nt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket_s != (unsigned)(split_k - 1) || wave != 0)
+            return;
+        // last arrival: add all partials in split order with device-scope loads
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                sum[t][r] = 0.f;
+        for (int s = 0; s < split_k; ++s) {
+            const float* p = ws + ((size_t)nt * split_k + s) * (MT * 256);
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (4 * kq + r + 16 * t < M)
+                        sum[t][r] += __hip_atomic_load(p + (t * 4 + r) * 64 + lane, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (lane == 0)
+            __hip_atomic_store(counters + nt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    const int n = nt * 16 + col;
+    const float b = bias ? (float)bias[n] : 0.f;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = 4 * kq + r + 16 * t;
+            if (m < M)
+                store_out(y, (size_t)m * N + n, sum[t][r] + b, out_f32);
+        }
+}
+
+template <int BITS, int MT, bool ZPT>
+static void launch_decode_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    const Layout& L = a.layout;
+    hipLaunchKernelGGL((fcc_decode_kernel<BITS, MT, ZPT>), dim3(p.grid[0], p.grid[1], 1), dim3(p.block),
+                       p.dynamic_lds, s, (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp,
+                       (const half_t*)a.x, (const half_t*)a.bias, a.y, a.workspace, a.counters, (int)a.M, (int)a.N,
+                       (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups, L.zp_const,
+                       p.kblocks_per_split, p.split_k, a.out_f32);
+}
+
+template <int BITS, bool ZPT>
+static void launch_decode_bits(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    if (a.M > 16)
+        launch_decode_impl<BITS, 2, ZPT>(a, p, s);
+    else
+        launch_decode_impl<BITS, 1, ZPT>(a, p, s);
+}
+
+int launch_decode(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Layout& L = a.layout;
+    if (L.bits == 4)
+        L.zp_table ? launch_decode_bits<4, true>(a, p, s) : launch_decode_bits<4, false>(a, p, s);
+    else
+        L.zp_table ? launch_decode_bits<8, true>(a, p, s) : launch_decode_bits<8, false>(a, p, s);
+    return (int)hipGetLastError();
+}
+
+}  // namespace ovfcc

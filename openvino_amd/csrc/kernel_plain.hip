@@ -1,0 +1,86 @@
+// Fallback kernel for shapes that keep OpenVINO's constant layout, and the copy yardstick.
+// Semantics: the scalar reference kernel of the OpenVINO Intel-GPU plugin
+// (src/plugins/intel_gpu/src/kernel_selector/cl_kernels/fully_connected_gpu_bfyx_ref.cl:88-160).
+#include "device_common.h"
+
+namespace ovfcc {
+
+// ------------------------------------------------------------------------------------------------
+// Plain kernel: OpenVINO layout, any N/K/G.  One wave per (n, m); lanes stride over k.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void fcc_plain_kernel(const uint8_t* __restrict__ w, const half_t* __restrict__ s,
+                                                       const uint8_t* __restrict__ zp,
+                                                       const half_t* __restrict__ bias,
+                                                       const half_t* __restrict__ x, void* __restrict__ y, int M,
+                                                       int N, int K, int G, int w_type, int zp_type, int zp_scalar,
+                                                       int out_f32) {
+    const int n = blockIdx.x;
+    const int m = blockIdx.y;
+    const int lane = threadIdx.x;
+    const int ng = K / G;
+    float acc = 0.f;
+    for (int k = lane; k < K; k += 64) {
+        const size_t wi = (size_t)n * K + k;
+        float q;
+        if (w_type == OVFCC_U4 || w_type == OVFCC_I4) {
+            const unsigned b = w[wi >> 1];
+            int v = (wi & 1) ? (b >> 4) : (b & 0xF);
+            if (w_type == OVFCC_I4 && v >= 8)
+                v -= 16;
+            q = (float)v;
+        } else if (w_type == OVFCC_U8) {
+            q = (float)w[wi];
+        } else {
+            q = (float)(int8_t)w[wi];
+        }
+        const int g = k / G;
+        float z = 0.f;
+        if (zp_type != OVFCC_NONE) {
+            const size_t zi = zp_scalar ? 0 : (size_t)n * ng + g;
+            if (zp_type == OVFCC_U4) {
+                const unsigned b = zp[zi >> 1];
+                z = (float)((zi & 1) ? (b >> 4) : (b & 0xF));
+            } else {
+                z = (float)zp[zi];
+            }
+        }
+        const float sc = (float)s[(size_t)n * ng + g];
+        acc += (float)x[(size_t)m * K + k] * ((q - z) * sc);
+    }
+    for (int off = 32; off > 0; off >>= 1)
+        acc += __shfl_down(acc, off, 64);
+    if (lane == 0) {
+        if (bias)
+            acc += (float)bias[n];
+        store_out(y, (size_t)m * N + n, acc, out_f32);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Plain 128-bit copy, the yardstick for bandwidth figures and counter scaling.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fcc_copy_kernel(uint4_t* __restrict__ dst, const uint4_t* __restrict__ src,
+                                                       size_t n16) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n16; i += stride)
+        dst[i] = __builtin_nontemporal_load(src + i);
+}
+
+
+int launch_plain(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
+    hipLaunchKernelGGL(fcc_plain_kernel, dim3(p.grid[0], p.grid[1], 1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       (const uint8_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.bias,
+                       (const half_t*)a.x, a.y, (int)a.M, (int)a.N, (int)a.K, (int)a.group_size, a.w_type, a.zp_type,
+                       a.zp_scalar, a.out_f32);
+    return (int)hipGetLastError();
+}
+
+int launch_copy(void* dst, const void* src, size_t bytes, void* stream) {
+    const size_t n16 = bytes / 16;
+    hipLaunchKernelGGL(fcc_copy_kernel, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream), (uint4_t*)dst,
+                       (const uint4_t*)src, n16);
+    return (int)hipGetLastError();
+}
+
+}  // namespace ovfcc

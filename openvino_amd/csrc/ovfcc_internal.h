@@ -79,6 +79,7 @@ struct LaunchPlan {
     int tile_m = 0, tile_n = 0;
     unsigned grid[3] = {1, 1, 1};
     unsigned block = 256;
+    unsigned dynamic_lds = 0;   // bytes of dynamic LDS (decode kernel: the cross-wave reduction buffer)
     size_t workspace_bytes = 0;
     size_t counter_count = 0;
     const char* name = "";
@@ -88,6 +89,11 @@ struct LaunchPlan {
 int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_cus, LaunchPlan* plan);
 // Enqueues on `stream` (a hipStream_t passed as void*); returns a HIP error code (0 = success).
 int launch_fc(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_plain(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_decode(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
+
+constexpr int kPrefillTileM = 128, kPrefillTileN = 128;
 
 }  // namespace ovfcc

@@ -77,7 +77,9 @@ Layout make_layout(const ovfcc_fc_desc& d) {
     L.zp_offset = d.w_type == OVFCC_I4 ? 8 : (d.w_type == OVFCC_I8 ? 128 : 0);
     L.zp_table = d.zp_type != OVFCC_NONE && !d.zp_scalar;
     L.zp_const = L.zp_offset;
-    L.tiled = (d.N % kTileRows == 0) && (d.K % kBlockK == 0) && (d.group_size % kBlockK == 0);
+    // K / 128 < 2^16 keeps the kernels' 32-bit offsets and reciprocal group index exact
+    L.tiled = (d.N % kTileRows == 0) && (d.K % kBlockK == 0) && (d.group_size % kBlockK == 0) &&
+              (d.K / kBlockK < 65536);
     if (L.tiled) {
         L.n_tiles = d.N / kTileRows;
         L.k_blocks = d.K / kBlockK;
