@@ -77,6 +77,8 @@ struct LaunchPlan {
     int split_k = 1;
     int kblocks_per_split = 0;
     int tile_m = 0, tile_n = 0;
+    int tiles_per_group = 1;    // decode kernel: 16-channel tiles per workgroup
+    bool x_in_lds = false;      // decode kernel: activations staged in LDS
     unsigned grid[3] = {1, 1, 1};
     unsigned block = 256;
     unsigned dynamic_lds = 0;   // bytes of dynamic LDS (decode kernel: the cross-wave reduction buffer)

@@ -9,13 +9,11 @@
 
 namespace ovfcc {
 
-// Tuning override for experiments: OVFCC_DECODE_WAVES = 4 | 8 | 16 fixes the decode workgroup size.
-static int env_decode_waves() {
-    const char* e = std::getenv("OVFCC_DECODE_WAVES");
-    if (!e)
-        return 0;
-    const int v = std::atoi(e);
-    return (v == 4 || v == 8 || v == 16) ? v : 0;
+// Tuning overrides for experiments: OVFCC_DECODE_WAVES = 4 | 8 | 16 (workgroup size),
+// OVFCC_DECODE_RT = 1 | 2 | 4 (channel tiles per workgroup), OVFCC_DECODE_XLDS = 0 | 1 (activations via LDS).
+static int env_int(const char* name, int fallback) {
+    const char* e = std::getenv(name);
+    return e ? std::atoi(e) : fallback;
 }
 
 int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_cus, LaunchPlan* plan) {
@@ -43,12 +41,16 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
     } else if (kernel == OVFCC_KERNEL_DECODE) {
         const int kb = (int)L.k_blocks;
         const int mt = a.M <= 16 ? 1 : 2;
-        // Waves per workgroup: as many as the k-range feeds (one k-block each at least), up to 16, so that
-        // a 16-channel tile is reduced inside one workgroup whenever possible.  K is split over workgroups
-        // only when the grid would otherwise leave compute units idle (few channel tiles, long rows).
+        // Activations go through LDS for M <= 4 when the k-range of one workgroup fits 40 KiB.
+        bool xlds = a.M <= 4;
+        const int x_env = env_int("OVFCC_DECODE_XLDS", -1);
+        if (x_env == 0)
+            xlds = false;
         int split = force_split;
         if (split <= 0) {
             split = 1;
+            // K is split over workgroups only when the grid would otherwise leave compute units idle
+            // (few channel tiles, long rows)
             const int64_t want_waves = (int64_t)16 * n_cus;
             while (split < 8 && L.n_tiles * 16 * split * 2 <= want_waves && kb / (split * 2) >= 32)
                 split *= 2;
@@ -57,21 +59,39 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             split = kb;
         const int per = (kb + split - 1) / split;
         split = (kb + per - 1) / per;  // no empty splits
+        const size_t x_bytes = (size_t)a.M * ((size_t)per * kBlockK + 8) * 2;
+        if (x_bytes > 40 * 1024)  // does not fit beside the reduction buffer: read the operand from L2 instead
+            xlds = false;
+        // Channel tiles per workgroup: one.  More tiles would share a staged activation copy between more
+        // weights, but measured slower at M <= 4 (fewer, longer workgroups); the override stays for experiments.
+        int rt = 1;
+        if (xlds) {
+            const int rt_max = L.bits == 4 ? 4 : 2;
+            const int rt_env = env_int("OVFCC_DECODE_RT", 0);
+            if ((rt_env == 1 || rt_env == 2 || rt_env == 4) && rt_env <= rt_max && L.n_tiles % rt_env == 0)
+                rt = rt_env;
+        }
+        const int64_t groups = L.n_tiles / rt;
+        // waves per workgroup: as many as the k-range feeds with four k-blocks each (the prefetch depth),
+        // at most 16, and no more than about 16 waves per compute unit in total
         int nw = 16;
-        while (nw > 4 && (per < nw || L.n_tiles * split * nw > (int64_t)24 * n_cus))
+        while (nw > 4 && (per < 4 * nw || groups * split * nw > (int64_t)16 * n_cus || nw * rt > 32))
             nw >>= 1;
-        if (const int forced = env_decode_waves())
-            nw = forced;
+        const int nw_env = env_int("OVFCC_DECODE_WAVES", 0);
+        if ((nw_env == 4 || nw_env == 8 || nw_env == 16) && nw_env * rt <= 32)
+            nw = nw_env;
         p.split_k = split;
         p.kblocks_per_split = per;
-        p.grid[0] = (unsigned)L.n_tiles;
+        p.tiles_per_group = rt;
+        p.x_in_lds = xlds;
+        p.grid[0] = (unsigned)groups;
         p.grid[1] = (unsigned)split;
         p.block = 64u * nw;
         p.tile_m = 16 * mt;
-        p.tile_n = 16;
-        p.workspace_bytes = split > 1 ? (size_t)L.n_tiles * split * mt * 256 * sizeof(float) : 0;
-        p.counter_count = split > 1 ? (size_t)L.n_tiles : 0;
-        p.dynamic_lds = (unsigned)(nw * mt * 256 * sizeof(float));
+        p.tile_n = 16 * rt;
+        p.workspace_bytes = split > 1 ? (size_t)groups * split * rt * mt * 256 * sizeof(float) : 0;
+        p.counter_count = split > 1 ? (size_t)groups : 0;
+        p.dynamic_lds = (unsigned)((size_t)nw * rt * mt * 256 * sizeof(float) + (xlds ? x_bytes : 0));
         p.name = L.bits == 4 ? "fcc_decode_w4" : "fcc_decode_w8";
     } else {
         p.grid[0] = (unsigned)(a.N / kPrefillTileN);
