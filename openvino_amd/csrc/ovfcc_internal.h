@@ -94,8 +94,10 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_plain(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_decode(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
 
-constexpr int kPrefillTileM = 128, kPrefillTileN = 128;
+constexpr int kPrefillTileM = 128, kPrefillTileN = 128;  // square prefill kernel
+constexpr int kPrefillWideN = 256;                         // wide prefill kernel: 128 x 256
 
 }  // namespace ovfcc

@@ -94,12 +94,24 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.dynamic_lds = (unsigned)((size_t)nw * rt * mt * 256 * sizeof(float) + (xlds ? x_bytes : 0));
         p.name = L.bits == 4 ? "fcc_decode_w4" : "fcc_decode_w8";
     } else {
-        p.grid[0] = (unsigned)(a.N / kPrefillTileN);
-        p.grid[1] = (unsigned)((a.M + kPrefillTileM - 1) / kPrefillTileM);
-        p.block = 256;
+        // The wide kernel (128 x 256 tiles) runs when its grid still gives every second compute unit
+        // a tile; otherwise, or when N is not a multiple of 256, the square kernel's smaller tiles spread
+        // the work further.  OVFCC_PREFILL_WIDE = 0 | 1 overrides for experiments.
+        const int64_t m_tiles = (a.M + kPrefillTileM - 1) / kPrefillTileM;
+        const bool wide_ok = (a.N % kPrefillWideN) == 0 && (a.K % 256) == 0 && a.M * a.K * 2 < ((int64_t)1 << 31);
+        bool wide = wide_ok && (a.N / kPrefillWideN) * m_tiles * 2 >= n_cus;
+        const int wide_env = env_int("OVFCC_PREFILL_WIDE", -1);
+        if (wide_env == 0)
+            wide = false;
+        if (wide_env == 1 && wide_ok)
+            wide = true;
         p.tile_m = kPrefillTileM;
-        p.tile_n = kPrefillTileN;
-        p.name = L.bits == 4 ? "fcc_prefill_w4" : "fcc_prefill_w8";
+        p.tile_n = wide ? kPrefillWideN : kPrefillTileN;
+        p.grid[0] = (unsigned)(a.N / p.tile_n);
+        p.grid[1] = (unsigned)m_tiles;
+        p.block = wide ? 512 : 256;
+        p.name = L.bits == 4 ? (wide ? "fcc_prefill_wide_w4" : "fcc_prefill_w4")
+                             : (wide ? "fcc_prefill_wide_w8" : "fcc_prefill_w8");
     }
     *plan = p;
     return OVFCC_OK;
@@ -114,7 +126,7 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     case OVFCC_KERNEL_DECODE:
         return launch_decode(a, p, stream);
     default:
-        return launch_prefill(a, p, stream);
+        return p.tile_n == kPrefillWideN ? launch_prefill_wide(a, p, stream) : launch_prefill(a, p, stream);
     }
 }
 
