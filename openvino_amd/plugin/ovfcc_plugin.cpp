@@ -1,0 +1,573 @@
+// OpenVINO device plugin "MI355X": runs weight-compressed FullyConnected nodes on the GPU through the
+// C ABI of libovfcc (include/ovfcc.h).
+//
+//   ov::Core core;
+//   core.register_plugin("/abs/path/libovfcc_plugin.so", "MI355X");
+//   auto compiled = core.compile_model(model, "MI355X");      // unchanged ov::Model
+//
+// What the plugin accepts: models whose Results are MatMuls (transpose_a = false) of a Parameter with a
+// weight-decompression subgraph
+//     Constant(u4|i4|u8|i8) -> Convert -> [Subtract(zp)] -> Multiply(scale) -> [Reshape] -> [Convert] -> MatMul
+// i.e. exactly what ConvertMatMulToFC + ConvertFullyConnectedToFullyConnectedCompressed fold into
+// ov::op::internal::FullyConnectedCompressed on the CPU plugin
+// (src/plugins/intel_cpu/src/transformations/cpu_opset/common/pass/convert_matmul_to_fc.cpp:47-270,
+//  src/common/transformations/src/transformations/op_conversions/convert_fc_to_compressed.cpp:170-225).
+// The pattern is matched on the untouched input model, before any folding pass, so the u4/u8 constants
+// are still there and no MarkDequantization pass is needed.  Everything else is reported as unsupported by
+// query_model (a HETERO device can place it elsewhere) and rejected by compile_model.
+//
+// The interfaces implemented are ov::IPlugin (src/inference/dev_api/openvino/runtime/iplugin.hpp:74-255),
+// ov::ICompiledModel (icompiled_model.hpp:36-190) and ov::ISyncInferRequest (isync_infer_request.hpp:30-175);
+// the template plugin (src/plugins/template/src) is the model for which properties to answer.
+//
+// This file needs OpenVINO's developer headers and libopenvino to build; it is not part of libovfcc.so.
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "openvino/core/model.hpp"
+#include "openvino/core/type/float16.hpp"
+#include "openvino/op/constant.hpp"
+#include "openvino/op/convert.hpp"
+#include "openvino/op/matmul.hpp"
+#include "openvino/op/multiply.hpp"
+#include "openvino/op/parameter.hpp"
+#include "openvino/op/reshape.hpp"
+#include "openvino/op/result.hpp"
+#include "openvino/op/subtract.hpp"
+#include "openvino/op/transpose.hpp"
+#include "openvino/runtime/icompiled_model.hpp"
+#include "openvino/runtime/internal_properties.hpp"
+#include "openvino/runtime/iplugin.hpp"
+#include "openvino/runtime/isync_infer_request.hpp"
+#include "openvino/runtime/make_tensor.hpp"
+#include "openvino/runtime/properties.hpp"
+#include "ovfcc.h"
+
+namespace ovfcc_plugin {
+
+[[noreturn]] void throw_last(const char* what) {
+    OPENVINO_THROW("ovfcc: ", what, ": ", ovfcc_last_error());
+}
+
+// ---- the decompression pattern ------------------------------------------------------------------------
+
+struct CompressedFc {
+    std::shared_ptr<ov::op::v0::MatMul> matmul;
+    std::shared_ptr<ov::op::v0::Parameter> activations;
+    std::shared_ptr<ov::op::v0::Constant> weights, scales, zero_points;  // zero_points may be null
+    ovfcc_fc_desc desc{};
+    std::vector<ov::float16> scales_f16;  // [N, K/G]
+    std::vector<uint8_t> zp_bytes;        // packed u4 / u8 in OpenVINO order, or one element
+};
+
+static std::shared_ptr<ov::op::v0::Constant> constant_behind_convert(const ov::Output<ov::Node>& out) {
+    auto node = out.get_node_shared_ptr();
+    if (auto cvt = ov::as_type_ptr<ov::op::v0::Convert>(node))
+        node = cvt->input_value(0).get_node_shared_ptr();
+    return ov::as_type_ptr<ov::op::v0::Constant>(node);
+}
+
+static int weight_tag(const ov::element::Type& t) {
+    if (t == ov::element::u4) return OVFCC_U4;
+    if (t == ov::element::i4) return OVFCC_I4;
+    if (t == ov::element::u8) return OVFCC_U8;
+    if (t == ov::element::i8) return OVFCC_I8;
+    return OVFCC_NONE;
+}
+
+// Matches MatMul(Parameter, decompression chain) and fills the C-ABI descriptor.  Mirrors the anchors of
+// pattern::op::CompressedWeightsBlock (src/common/transformations/src/transformations/pattern_blocks/
+// compressed_weights_block.cpp:31-84) and the shape algebra of combine_groups
+// (convert_fc_to_compressed.cpp:42-78): W [N, K] or [N, K/G, G]; scale and zero-point [N, 1], [N, K/G, 1],
+// [N], [1] or [].
+static bool match_compressed_fc(const std::shared_ptr<ov::Node>& node, CompressedFc& fc, std::string& why) {
+    auto mm = ov::as_type_ptr<ov::op::v0::MatMul>(node);
+    if (!mm)
+        return false;
+    if (mm->get_transpose_a() || !mm->get_transpose_b()) {
+        why = "MatMul must have transpose_a = false and transpose_b = true (weights [N, K])";
+        return false;
+    }
+    auto param = ov::as_type_ptr<ov::op::v0::Parameter>(mm->input_value(0).get_node_shared_ptr());
+    if (!param) {
+        why = "activations must come straight from a Parameter";
+        return false;
+    }
+    // walk up from the MatMul's weight input: [Convert] <- [Reshape] <- Multiply
+    auto w = mm->input_value(1).get_node_shared_ptr();
+    if (auto cvt = ov::as_type_ptr<ov::op::v0::Convert>(w))
+        w = cvt->input_value(0).get_node_shared_ptr();
+    if (auto rs = ov::as_type_ptr<ov::op::v1::Reshape>(w))
+        w = rs->input_value(0).get_node_shared_ptr();
+    auto mul = ov::as_type_ptr<ov::op::v1::Multiply>(w);
+    if (!mul) {
+        why = "no Multiply(scale) on the weight path";
+        return false;
+    }
+    // one Multiply input is the scale constant, the other Convert(W) or Subtract(Convert(W), zp)
+    std::shared_ptr<ov::op::v0::Constant> scale;
+    ov::Output<ov::Node> body;
+    for (int side = 0; side < 2 && !scale; ++side) {
+        auto c = constant_behind_convert(mul->input_value(side));
+        if (c && c->get_element_type().is_real()) {
+            scale = c;
+            body = mul->input_value(1 - side);
+        }
+    }
+    if (!scale) {
+        why = "scale is not a floating-point constant";
+        return false;
+    }
+    std::shared_ptr<ov::op::v0::Constant> zp;
+    auto body_node = body.get_node_shared_ptr();
+    if (auto sub = ov::as_type_ptr<ov::op::v1::Subtract>(body_node)) {
+        zp = constant_behind_convert(sub->input_value(1));
+        if (!zp) {
+            why = "zero-point is not a constant";
+            return false;
+        }
+        body_node = sub->input_value(0).get_node_shared_ptr();
+    }
+    auto wcvt = ov::as_type_ptr<ov::op::v0::Convert>(body_node);
+    auto wconst = wcvt ? ov::as_type_ptr<ov::op::v0::Constant>(wcvt->input_value(0).get_node_shared_ptr()) : nullptr;
+    if (!wconst || weight_tag(wconst->get_element_type()) == OVFCC_NONE) {
+        why = "weights are not a u4/i4/u8/i8 constant behind a Convert";
+        return false;
+    }
+
+    const auto& ws = wconst->get_shape();
+    int64_t N, K, G;
+    if (ws.size() == 2) {
+        N = (int64_t)ws[0];
+        K = (int64_t)ws[1];
+        G = K;
+    } else if (ws.size() == 3) {
+        N = (int64_t)ws[0];
+        K = (int64_t)(ws[1] * ws[2]);
+        G = (int64_t)ws[2];
+    } else {
+        why = "weights must be [N, K] or [N, K/G, G]";
+        return false;
+    }
+    const int64_t ng = K / G;
+    const size_t scale_count = ov::shape_size(scale->get_shape());
+    if (scale_count != (size_t)(N * ng)) {
+        if (scale_count == (size_t)N && ng == 1) {
+            // per-channel [N] / [N, 1]
+        } else {
+            why = "scale must hold one value per (channel, group)";
+            return false;
+        }
+    }
+    if (mm->get_input_partial_shape(0).rbegin()->is_dynamic() ||
+        mm->get_input_partial_shape(0).rbegin()->get_length() != K) {
+        why = "last activation dimension must equal K";
+        return false;
+    }
+    const auto act_type = param->get_element_type();
+    if (act_type != ov::element::f16 && act_type != ov::element::f32) {
+        why = "activations must be f16 (or f32, converted on the host)";
+        return false;
+    }
+
+    fc.matmul = mm;
+    fc.activations = param;
+    fc.weights = wconst;
+    fc.scales = scale;
+    fc.zero_points = zp;
+    fc.desc.N = N;
+    fc.desc.K = K;
+    fc.desc.group_size = G;
+    fc.desc.w_type = weight_tag(wconst->get_element_type());
+    fc.desc.scale_type = OVFCC_F16;
+    fc.desc.bias_type = OVFCC_NONE;
+    fc.desc.act_type = OVFCC_F16;
+    fc.desc.out_type = mm->get_output_element_type(0) == ov::element::f32 ? OVFCC_F32 : OVFCC_F16;
+    fc.desc.flags = 0;
+    // scales as f16 [N, K/G]
+    fc.scales_f16.resize((size_t)(N * ng));
+    {
+        const auto vals = scale->cast_vector<float>();
+        for (size_t i = 0; i < fc.scales_f16.size(); ++i)
+            fc.scales_f16[i] = ov::float16(vals[i]);
+    }
+    // zero-points: u4/u8 constants are passed through untouched; real-typed ones (NNCF sometimes stores
+    // them as f16) must be integers in 0..255 and become u8
+    fc.desc.zp_type = OVFCC_NONE;
+    fc.desc.zp_scalar = 0;
+    if (zp) {
+        const size_t zc = ov::shape_size(zp->get_shape());
+        if (zc != 1 && zc != (size_t)(N * ng)) {
+            why = "zero-point must be scalar or hold one value per (channel, group)";
+            return false;
+        }
+        fc.desc.zp_scalar = zc == 1 && N * ng != 1;
+        const auto zt = zp->get_element_type();
+        if (zt == ov::element::u4 || zt == ov::element::u8) {
+            fc.desc.zp_type = zt == ov::element::u4 ? OVFCC_U4 : OVFCC_U8;
+            fc.zp_bytes.assign(static_cast<const uint8_t*>(zp->get_data_ptr()),
+                               static_cast<const uint8_t*>(zp->get_data_ptr()) + zp->get_byte_size());
+        } else {
+            const auto vals = zp->cast_vector<float>();
+            fc.desc.zp_type = OVFCC_U8;
+            fc.zp_bytes.resize(vals.size());
+            for (size_t i = 0; i < vals.size(); ++i) {
+                if (vals[i] < 0 || vals[i] > 255 || vals[i] != (float)(int)vals[i]) {
+                    why = "zero-point values must be integers in 0..255";
+                    return false;
+                }
+                fc.zp_bytes[i] = (uint8_t)vals[i];
+            }
+        }
+    }
+    if (ovfcc_desc_validate(&fc.desc) != OVFCC_OK) {
+        why = ovfcc_last_error();
+        return false;
+    }
+    return true;
+}
+
+// Nodes of the decompression chain of a matched MatMul (for query_model)
+static void chain_nodes(const CompressedFc& fc, std::vector<std::shared_ptr<ov::Node>>& out) {
+    std::vector<std::shared_ptr<ov::Node>> stack{fc.matmul->input_value(1).get_node_shared_ptr()};
+    while (!stack.empty()) {
+        auto n = stack.back();
+        stack.pop_back();
+        out.push_back(n);
+        for (const auto& in : n->input_values())
+            stack.push_back(in.get_node_shared_ptr());
+    }
+}
+
+// ---- plugin -------------------------------------------------------------------------------------------------
+
+class Plugin;
+
+class CompiledModel : public ov::ICompiledModel {
+public:
+    struct Node {
+        CompressedFc fc;
+        ovfcc_weights* weights = nullptr;
+        size_t input_index = 0, output_index = 0;
+    };
+
+    CompiledModel(const std::shared_ptr<ov::Model>& model, const std::shared_ptr<const ov::IPlugin>& plugin,
+                  ovfcc_ctx* ctx, bool profiling);
+    ~CompiledModel() override {
+        for (auto& n : m_nodes)
+            ovfcc_weights_destroy(n.weights);
+    }
+
+    void export_model(std::ostream&) const override {
+        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: export_model (caching the repacked weights) is not implemented");
+    }
+    std::shared_ptr<const ov::Model> get_runtime_model() const override {
+        return m_model;
+    }
+    void set_property(const ov::AnyMap&) override {
+        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: compiled model has no mutable properties");
+    }
+    ov::Any get_property(const std::string& name) const override {
+        if (name == ov::supported_properties)
+            return std::vector<ov::PropertyName>{ov::supported_properties, ov::model_name,
+                                                 ov::optimal_number_of_infer_requests, ov::execution_devices,
+                                                 ov::enable_profiling};
+        if (name == ov::model_name)
+            return decltype(ov::model_name)::value_type{m_model->get_friendly_name()};
+        if (name == ov::optimal_number_of_infer_requests)
+            return decltype(ov::optimal_number_of_infer_requests)::value_type{2};
+        if (name == ov::execution_devices)
+            return decltype(ov::execution_devices)::value_type{get_plugin()->get_device_name()};
+        if (name == ov::enable_profiling)
+            return m_profiling;
+        OPENVINO_THROW("MI355X: unsupported compiled-model property ", name);
+    }
+    std::shared_ptr<ov::ISyncInferRequest> create_sync_infer_request() const override;
+
+    const std::vector<Node>& nodes() const {
+        return m_nodes;
+    }
+    ovfcc_ctx* ctx() const {
+        return m_ctx;
+    }
+
+private:
+    std::shared_ptr<ov::Model> m_model;
+    std::vector<Node> m_nodes;
+    ovfcc_ctx* m_ctx;
+    bool m_profiling;
+};
+
+class InferRequest : public ov::ISyncInferRequest {
+public:
+    explicit InferRequest(const std::shared_ptr<const CompiledModel>& compiled)
+        : ov::ISyncInferRequest(compiled), m_compiled(compiled) {
+        if (ovfcc_request_create(compiled->ctx(), &m_request) != OVFCC_OK)
+            throw_last("request_create");
+        // host tensors for every port, as the template plugin does (src/plugins/template/src/sync_infer_request.cpp:94-110)
+        for (const auto& port : get_inputs())
+            allocate_tensor(port, [port](ov::SoPtr<ov::ITensor>& t) {
+                allocate_tensor_impl(t, port.get_element_type(),
+                                     port.get_partial_shape().is_dynamic() ? ov::Shape{0} : port.get_shape());
+            });
+        for (const auto& port : get_outputs())
+            allocate_tensor(port, [port](ov::SoPtr<ov::ITensor>& t) {
+                allocate_tensor_impl(t, port.get_element_type(),
+                                     port.get_partial_shape().is_dynamic() ? ov::Shape{0} : port.get_shape());
+            });
+    }
+    ~InferRequest() override {
+        ovfcc_request_destroy(m_request);
+    }
+
+    void infer() override {
+        check_tensors();
+        m_kernels.clear();
+        for (const auto& node : m_compiled->nodes()) {
+            auto in = get_tensor(get_inputs()[node.input_index]);
+            auto out = get_tensor(get_outputs()[node.output_index]);
+            const ov::Shape in_shape = in->get_shape();
+            int64_t M = 1;  // 3-D activations flatten to [B*S, K] like the CPU path does
+            for (size_t d = 0; d + 1 < in_shape.size(); ++d)
+                M *= (int64_t)in_shape[d];
+            ov::Shape out_shape = in_shape;
+            out_shape.back() = (size_t)node.fc.desc.N;
+            out->set_shape(out_shape);  // dynamic M: the output follows the input
+            const void* x = in->data();
+            if (in->get_element_type() == ov::element::f32) {
+                // the device path computes on f16 activations
+                const float* src = static_cast<const float*>(in->data());
+                m_staging.resize((size_t)M * node.fc.desc.K);
+                for (size_t i = 0; i < m_staging.size(); ++i)
+                    m_staging[i] = ov::float16(src[i]);
+                x = m_staging.data();
+            }
+            if (ovfcc_fc_run(m_request, node.weights, x, out->data(), M) != OVFCC_OK)
+                throw_last("fc_run");
+            ovfcc_kernel_info info;
+            ovfcc_last_kernel_info(m_request, &info);
+            m_kernels.push_back(info);
+        }
+    }
+
+    std::vector<ov::ProfilingInfo> get_profiling_info() const override {
+        std::vector<ov::ProfilingInfo> out;
+        for (size_t i = 0; i < m_kernels.size(); ++i) {
+            ov::ProfilingInfo p;
+            p.status = ov::ProfilingInfo::Status::EXECUTED;
+            p.node_name = m_compiled->nodes()[i].fc.matmul->get_friendly_name();
+            p.node_type = "FullyConnected";
+            p.exec_type = m_kernels[i].name;
+            out.push_back(p);
+        }
+        return out;
+    }
+    std::vector<ov::SoPtr<ov::IVariableState>> query_state() const override {
+        return {};
+    }
+
+private:
+    static void allocate_tensor_impl(ov::SoPtr<ov::ITensor>& tensor, const ov::element::Type& type,
+                                     const ov::Shape& shape) {
+        if (!tensor || tensor->get_element_type() != type)
+            tensor = ov::make_tensor(type, shape);
+        else
+            tensor->set_shape(shape);
+    }
+
+    std::shared_ptr<const CompiledModel> m_compiled;
+    ovfcc_request* m_request = nullptr;
+    std::vector<ov::float16> m_staging;
+    std::vector<ovfcc_kernel_info> m_kernels;
+};
+
+class Plugin : public ov::IPlugin {
+public:
+    Plugin() {
+        set_device_name("MI355X");
+    }
+    ~Plugin() override {
+        ovfcc_destroy(m_ctx);
+    }
+
+    std::shared_ptr<ov::ICompiledModel> compile_model(const std::shared_ptr<const ov::Model>& model,
+                                                      const ov::AnyMap& properties) const override {
+        bool profiling = m_profiling;
+        for (const auto& kv : properties) {
+            if (kv.first == ov::enable_profiling.name())
+                profiling = kv.second.as<bool>();
+            else if (!known_hint(kv.first))
+                OPENVINO_THROW("MI355X: unsupported property ", kv.first);
+        }
+        return std::make_shared<CompiledModel>(model->clone(), shared_from_this(), context(), profiling);
+    }
+    std::shared_ptr<ov::ICompiledModel> compile_model(const std::shared_ptr<const ov::Model>& model,
+                                                      const ov::AnyMap& properties,
+                                                      const ov::SoPtr<ov::IRemoteContext>&) const override {
+        return compile_model(model, properties);
+    }
+
+    void set_property(const ov::AnyMap& properties) override {
+        for (const auto& kv : properties) {
+            if (kv.first == ov::enable_profiling.name())
+                m_profiling = kv.second.as<bool>();
+            else if (!known_hint(kv.first))
+                OPENVINO_THROW("MI355X: unsupported property ", kv.first);
+        }
+    }
+
+    ov::Any get_property(const std::string& name, const ov::AnyMap&) const override {
+        if (name == ov::supported_properties)
+            return std::vector<ov::PropertyName>{
+                {ov::available_devices.name(), ov::PropertyMutability::RO},
+                {ov::supported_properties.name(), ov::PropertyMutability::RO},
+                {ov::device::full_name.name(), ov::PropertyMutability::RO},
+                {ov::device::architecture.name(), ov::PropertyMutability::RO},
+                {ov::device::capabilities.name(), ov::PropertyMutability::RO},
+                {ov::device::type.name(), ov::PropertyMutability::RO},
+                {ov::range_for_async_infer_requests.name(), ov::PropertyMutability::RO},
+                {ov::execution_devices.name(), ov::PropertyMutability::RO},
+                {ov::enable_profiling.name(), ov::PropertyMutability::RW},
+                {ov::hint::performance_mode.name(), ov::PropertyMutability::RW},
+                {ov::hint::inference_precision.name(), ov::PropertyMutability::RW},
+                {ov::hint::num_requests.name(), ov::PropertyMutability::RW},
+                {ov::num_streams.name(), ov::PropertyMutability::RW},
+                {ov::device::id.name(), ov::PropertyMutability::RW},
+            };
+        // no caching_properties: export_model / import_model are not implemented, so Core must not try
+        if (name == ov::internal::supported_properties)
+            return decltype(ov::internal::supported_properties)::value_type{};
+        if (name == ov::available_devices)
+            return decltype(ov::available_devices)::value_type{"0"};
+        if (name == ov::device::full_name)
+            return decltype(ov::device::full_name)::value_type{"AMD Instinct MI355X (gfx950) via ovfcc"};
+        if (name == ov::device::architecture)
+            return decltype(ov::device::architecture)::value_type{"gfx950"};
+        if (name == ov::device::type)
+            return decltype(ov::device::type)::value_type{ov::device::Type::DISCRETE};
+        if (name == ov::device::capabilities)
+            return decltype(ov::device::capabilities)::value_type{ov::device::capability::FP16};
+        if (name == ov::execution_devices)
+            return decltype(ov::execution_devices)::value_type{get_device_name()};
+        if (name == ov::range_for_async_infer_requests)
+            return decltype(ov::range_for_async_infer_requests)::value_type{1, 8, 1};
+        if (name == ov::enable_profiling)
+            return m_profiling;
+        if (name == ov::hint::performance_mode)
+            return ov::hint::PerformanceMode::LATENCY;
+        if (name == ov::hint::inference_precision)
+            return ov::element::f16;
+        if (name == ov::hint::num_requests)
+            return (uint32_t)0;
+        if (name == ov::num_streams)
+            return ov::streams::Num(1);
+        if (name == ov::device::id)
+            return std::string("0");
+        OPENVINO_THROW("MI355X: unsupported property ", name);
+    }
+
+    ov::SoPtr<ov::IRemoteContext> create_context(const ov::AnyMap&) const override {
+        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: remote contexts are not implemented");
+    }
+    ov::SoPtr<ov::IRemoteContext> get_default_context(const ov::AnyMap&) const override {
+        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: remote contexts are not implemented");
+    }
+    std::shared_ptr<ov::ICompiledModel> import_model(std::istream&, const ov::AnyMap&) const override {
+        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: import_model is not implemented");
+    }
+    std::shared_ptr<ov::ICompiledModel> import_model(std::istream&, const ov::SoPtr<ov::IRemoteContext>&,
+                                                     const ov::AnyMap&) const override {
+        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: import_model is not implemented");
+    }
+    std::shared_ptr<ov::ICompiledModel> import_model(const ov::Tensor&, const ov::AnyMap&) const override {
+        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: import_model is not implemented");
+    }
+    std::shared_ptr<ov::ICompiledModel> import_model(const ov::Tensor&, const ov::SoPtr<ov::IRemoteContext>&,
+                                                     const ov::AnyMap&) const override {
+        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: import_model is not implemented");
+    }
+
+    // Supported: each matched MatMul with its whole decompression chain, and the Parameter / Result around it.
+    ov::SupportedOpsMap query_model(const std::shared_ptr<const ov::Model>& model, const ov::AnyMap&) const override {
+        ov::SupportedOpsMap res;
+        for (const auto& node : model->get_ordered_ops()) {
+            CompressedFc fc;
+            std::string why;
+            if (!match_compressed_fc(node, fc, why))
+                continue;
+            std::vector<std::shared_ptr<ov::Node>> nodes;
+            chain_nodes(fc, nodes);
+            nodes.push_back(fc.matmul);
+            nodes.push_back(fc.activations);
+            for (const auto& user : fc.matmul->output(0).get_target_inputs())
+                if (ov::is_type<ov::op::v0::Result>(user.get_node()))
+                    nodes.push_back(user.get_node()->shared_from_this());
+            for (const auto& n : nodes)
+                res[n->get_friendly_name()] = get_device_name();
+        }
+        return res;
+    }
+
+private:
+    static bool known_hint(const std::string& k) {
+        return k == ov::hint::performance_mode.name() || k == ov::hint::inference_precision.name() ||
+               k == ov::hint::num_requests.name() || k == ov::num_streams.name() || k == ov::device::id.name() ||
+               k == ov::hint::execution_mode.name() || k == ov::hint::model_priority.name() ||
+               k == ov::inference_num_threads.name() || k == ov::log::level.name();
+    }
+    // the device context is created on first use: Core constructs plugins on hosts without the device too
+    ovfcc_ctx* context() const {
+        std::lock_guard<std::mutex> lock(m_mutex);
+        if (!m_ctx && ovfcc_init(0, &m_ctx) != OVFCC_OK)
+            throw_last("init");
+        return m_ctx;
+    }
+
+    mutable std::mutex m_mutex;
+    mutable ovfcc_ctx* m_ctx = nullptr;
+    bool m_profiling = false;
+};
+
+CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std::shared_ptr<const ov::IPlugin>& plugin,
+                             ovfcc_ctx* ctx, bool profiling)
+    : ov::ICompiledModel(model, plugin), m_model(model), m_ctx(ctx), m_profiling(profiling) {
+    // every Result must be fed by a matched MatMul; every Parameter must feed one
+    const auto& results = model->get_results();
+    const auto& params = model->get_parameters();
+    for (size_t r = 0; r < results.size(); ++r) {
+        Node n;
+        std::string why = "not a MatMul";
+        auto producer = results[r]->input_value(0).get_node_shared_ptr();
+        if (!match_compressed_fc(producer, n.fc, why))
+            OPENVINO_THROW("MI355X: result ", results[r]->get_friendly_name(),
+                           " is not produced by a weight-compressed FullyConnected: ", why,
+                           " (use HETERO:MI355X,CPU for the rest of the graph)");
+        n.output_index = r;
+        for (size_t p = 0; p < params.size(); ++p)
+            if (params[p] == n.fc.activations)
+                n.input_index = p;
+        const void* zp = n.fc.zp_bytes.empty() ? nullptr : n.fc.zp_bytes.data();
+        if (ovfcc_weights_create(ctx, &n.fc.desc, n.fc.weights->get_data_ptr(), n.fc.scales_f16.data(), zp, nullptr,
+                                 &n.weights) != OVFCC_OK)
+            throw_last("weights_create");
+        // the executed graph shows the same layer type the CPU plugin shows
+        // (src/inference/dev_api/openvino/runtime/exec_model_info.hpp:31-73)
+        n.fc.matmul->get_rt_info()["layerType"] = std::string("FullyConnected");
+        n.fc.matmul->get_rt_info()["primitiveType"] =
+            std::string(ovfcc_weights_is_tiled(n.weights) ? "hip_tiled_w" : "hip_plain_w") +
+            (n.fc.desc.w_type == OVFCC_U8 || n.fc.desc.w_type == OVFCC_I8 ? "8" : "4");
+        m_nodes.push_back(std::move(n));
+    }
+}
+
+std::shared_ptr<ov::ISyncInferRequest> CompiledModel::create_sync_infer_request() const {
+    return std::make_shared<InferRequest>(std::static_pointer_cast<const CompiledModel>(shared_from_this()));
+}
+
+}  // namespace ovfcc_plugin
+
+static const ov::Version version = {"ovfcc-0.1", "openvino_mi355x_plugin"};
+OV_DEFINE_PLUGIN_CREATE_FUNCTION(ovfcc_plugin::Plugin, version)
