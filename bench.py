@@ -122,6 +122,27 @@ def main() -> int:
         log(f"  {name}: " + ", ".join(f"M={m}: {per_shape[f'{name}_M{m}']['us']:.2f} us "
                                       f"{per_shape[f'{name}_M{m}']['GBps']:.0f} GB/s" for m in (1, 4, 16, 32)))
 
+    # horizontal fusion (q,k,v -> one node; gate,up -> one node): 4 launches per block instead of 7
+    fused_base = {
+        "qkv": fc.CompressedWeights.concat([base["qo"], base["kv"], base["kv"]]),
+        "o": base["qo"],
+        "gate_up2": fc.CompressedWeights.concat([base["gate_up"], base["gate_up"]]),
+        "down": base["down"],
+    }
+    fused_layers = []
+    for _ in range(args.layers):
+        for name in ("qkv", "o", "gate_up2", "down"):
+            fused_layers.append(fused_base[name].clone())
+    fms = req.bench_layers(fused_layers, x_dev, y_dev, 1, args.warmup, args.steps, use_graph=not args.no_graph)
+    fused_bytes = sum(w.N * w.K // 2 + w.N * (w.K // 128) * 2 + w.K * 2 + w.N * 2 for w in fused_layers)
+    fused_gbs = fused_bytes / (fms / args.steps * 1e-3) / 1e9
+    log(f"decode M=1 with q/k/v and gate/up fused: {fms / args.steps:.4f} ms/pass, {len(fused_layers)} launches -> "
+        f"{fused_gbs:.1f} GB/s ({100 * fused_gbs / HBM_PEAK_GBS:.1f} % of 8 TB/s)")
+    for w in fused_layers:
+        w.close()
+    for k in ("qkv", "gate_up2"):
+        fused_base[k].close()
+
     copy_gbs = dev.copy_bandwidth(1 << 30, 10)
     log(f"plain copy kernel: {copy_gbs:.0f} GB/s (read + write)")
 
@@ -152,6 +173,10 @@ def main() -> int:
             "avg_launch_us": round(ms_per_step * 1e3 / launches, 3),
         },
         "copy_kernel_GBps": round(copy_gbs, 1),
+        "decode_fused": {"note": "same pass with q/k/v and gate/up concatenated into one node each "
+                                 "(ovfcc_weights_concat), 4 launches per block",
+                         "launches": args.layers * 4, "ms_per_pass": round(fms / args.steps, 5),
+                         "GBps": round(fused_gbs, 1), "pct_of_hbm_peak": round(100 * fused_gbs / HBM_PEAK_GBS, 2)},
         "decode_per_shape": {k: {"us": round(v["us"], 3), "GBps": round(v["GBps"], 1)} for k, v in per_shape.items()},
         "parity": {k: {a: float(f"{b:.3e}") for a, b in v.items()} for k, v in parity.items()},
     }

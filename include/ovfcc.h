@@ -109,6 +109,14 @@ void ovfcc_weights_destroy(ovfcc_weights* w);
  * must own its buffer (shared weights: src/tests/functional/plugin/shared/src/subgraph/
  * shared_matmul_weights_decompression.cpp); the benchmark uses it to build a rotating weight set. */
 int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out);
+/* Horizontal fusion of FullyConnected nodes that read the same activations (Q/K/V, gate/up): one node whose
+ * output channels are the parts' channels in order, N = sum N_i, so that one launch serves them all and the
+ * caller splits Y [M, N] by columns.  What FullyConnectedHorizontalFusion does on the Intel GPU plugin
+ * (src/plugins/intel_gpu/src/plugin/transformations/fc_horizontal_fusion.cpp: Concat of weights, scales and
+ * zero-points along the output-channel axis, VariadicSplit of the result).  Parts must be tiled nodes with
+ * equal K, group size, weight type, zero-point kind, bias presence and output type; the copy is made on the
+ * device and the parts stay valid. */
+int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_weights** out);
 /* device bytes held by the repacked node */
 int64_t ovfcc_weights_device_bytes(const ovfcc_weights* w);
 /* 1 when the node uses the tiled layout (fast kernels), 0 for the OpenVINO-layout fallback */

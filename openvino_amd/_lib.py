@@ -14,7 +14,7 @@ KERNEL_AUTO, KERNEL_PLAIN, KERNEL_DECODE, KERNEL_PREFILL = range(4)
 
 # every symbol include/ovfcc.h declares
 SYMBOLS = [
-    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_destroy",
+    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_destroy",
     "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
     "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_request_sync", "ovfcc_request_force_kernel",
     "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
@@ -67,6 +67,7 @@ def load() -> ctypes.CDLL:
         "ovfcc_device_count": (ci, []),
         "ovfcc_weights_create": (ci, [vp, ctypes.POINTER(FcDesc), vp, vp, vp, vp, pp]),
         "ovfcc_weights_clone": (ci, [vp, pp]),
+        "ovfcc_weights_concat": (ci, [pp, ci, pp]),
         "ovfcc_weights_destroy": (None, [vp]),
         "ovfcc_weights_device_bytes": (i64, [vp]),
         "ovfcc_weights_is_tiled": (ci, [vp]),

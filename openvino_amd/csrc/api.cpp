@@ -334,6 +334,68 @@ int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out) {
     return OVFCC_OK;
 }
 
+int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_weights** out) {
+    if (!parts || n_parts <= 0 || !out)
+        return fail(OVFCC_EINVAL, "null or empty part list");
+    *out = nullptr;
+    const ovfcc_weights* first = parts[0];
+    if (!first)
+        return fail(OVFCC_EINVAL, "part 0 is null");
+    int64_t n_total = 0;
+    for (int i = 0; i < n_parts; ++i) {
+        const ovfcc_weights* p = parts[i];
+        if (!p)
+            return fail(OVFCC_EINVAL, "a part is null");
+        if (!p->layout.tiled)
+            return fail(OVFCC_EUNSUPPORTED, "only tiled nodes can be fused");
+        const bool same = p->ctx == first->ctx && p->desc.K == first->desc.K &&
+                          p->desc.group_size == first->desc.group_size && p->desc.w_type == first->desc.w_type &&
+                          p->desc.zp_type == first->desc.zp_type && p->desc.zp_scalar == first->desc.zp_scalar &&
+                          p->desc.bias_type == first->desc.bias_type && p->desc.out_type == first->desc.out_type &&
+                          p->layout.zp_const == first->layout.zp_const;
+        if (!same)
+            return fail(OVFCC_EUNSUPPORTED,
+                        "parts differ in K, group size, types, scalar zero-point, bias or output type");
+        n_total += p->desc.N;
+    }
+    HIP_TRY(hipSetDevice(first->ctx->device));
+    ovfcc_weights* W = new ovfcc_weights();
+    W->ctx = first->ctx;
+    W->desc = first->desc;
+    W->desc.N = n_total;
+    W->layout = ovfcc::make_layout(W->desc);
+    W->layout.zp_const = first->layout.zp_const;
+    const ovfcc::Layout& L = W->layout;
+    auto gather = [&](void** dst, size_t total, void* ovfcc_weights::*member, auto bytes_of) -> int {
+        if (total == 0)
+            return OVFCC_OK;
+        HIP_TRY(hipMalloc(dst, total));
+        W->bytes += total;
+        size_t at = 0;
+        for (int i = 0; i < n_parts; ++i) {
+            const size_t b = bytes_of(parts[i]);
+            HIP_TRY(hipMemcpy(static_cast<char*>(*dst) + at, parts[i]->*member, b, hipMemcpyDeviceToDevice));
+            at += b;
+        }
+        return OVFCC_OK;
+    };
+    int rc = gather(&W->d_w, L.w_bytes, &ovfcc_weights::d_w, [](const ovfcc_weights* p) { return p->layout.w_bytes; });
+    if (!rc)
+        rc = gather(&W->d_scale, L.scale_bytes, &ovfcc_weights::d_scale,
+                    [](const ovfcc_weights* p) { return p->layout.scale_bytes; });
+    if (!rc)
+        rc = gather(&W->d_zp, L.zp_bytes, &ovfcc_weights::d_zp, [](const ovfcc_weights* p) { return p->layout.zp_bytes; });
+    if (!rc && W->desc.bias_type != OVFCC_NONE)
+        rc = gather(&W->d_bias, (size_t)n_total * 2, &ovfcc_weights::d_bias,
+                    [](const ovfcc_weights* p) { return (size_t)p->desc.N * 2; });
+    if (rc) {
+        ovfcc_weights_destroy(W);
+        return rc;
+    }
+    *out = W;
+    return OVFCC_OK;
+}
+
 int64_t ovfcc_weights_device_bytes(const ovfcc_weights* w) {
     return w ? (int64_t)w->bytes : 0;
 }

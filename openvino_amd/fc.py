@@ -114,6 +114,21 @@ class CompressedWeights:
         other.handle = h
         return other
 
+    @classmethod
+    def concat(cls, parts: Sequence["CompressedWeights"]) -> "CompressedWeights":
+        """Horizontal fusion: one node whose output channels are the parts' channels in order."""
+        first = parts[0]
+        arr = (ctypes.c_void_p * len(parts))(*[p.handle for p in parts])
+        h = ctypes.c_void_p()
+        check(first.device.lib.ovfcc_weights_concat(arr, len(parts), ctypes.byref(h)))
+        other = object.__new__(CompressedWeights)
+        other.device, other.K, other.group_size = first.device, first.K, first.group_size
+        other.N = sum(p.N for p in parts)
+        other.desc = FcDesc.from_buffer_copy(first.desc)
+        other.desc.N = other.N
+        other.handle = h
+        return other
+
     @property
     def tiled(self) -> bool:
         return bool(self.device.lib.ovfcc_weights_is_tiled(self.handle))

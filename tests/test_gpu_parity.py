@@ -219,3 +219,30 @@ def test_two_requests_interleaved(oracle, dev):
         a.close()
         b.close()
         w.close()
+
+
+def test_horizontal_fusion_matches_separate_nodes(oracle, dev, req):
+    """Q/K/V-style fusion: the fused node's columns equal the separate nodes' outputs (up to the last f16 bit:
+    the launch decomposition, and with it the summation order, depends on N) and meet the oracle bounds."""
+    say("concat")
+    K = 1024
+    cases = [datagen.make_case(50 + i, 64, K, n, "u4", 128, "u4", with_bias=True) for i, n in enumerate((256, 128, 128))]
+    x = cases[0].x
+    parts = [fc.CompressedWeights.from_case(dev, c) for c in cases]
+    fused = fc.CompressedWeights.concat(parts)
+    try:
+        assert fused.N == 512 and fused.tiled
+        for M in (1, 4, 64):
+            y = req.infer(fused, x[:M]).astype(np.float32)
+            sep = np.concatenate([req.infer(p, x[:M]) for p in parts], axis=1).astype(np.float32)
+            assert np.all(np.abs(y - sep) <= np.abs(sep) * 2.0 ** -10 + 1e-6)
+            ref = np.concatenate([oracle_y(oracle, c, x=x[:M]) for c in cases], axis=1)
+            check_parity(oracle, y, ref, K, f"fused M={M}", output_rounding_slack=True)
+        other = fc.CompressedWeights.from_case(dev, datagen.make_case(60, 1, 2 * K, 64, "u4", 128, "u4", with_bias=True))
+        with pytest.raises(fc.OvfccError):
+            fc.CompressedWeights.concat([parts[0], other])
+        other.close()
+    finally:
+        fused.close()
+        for p in parts:
+            p.close()
