@@ -26,6 +26,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
+# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/ (counters cannot be
+# read from inside this process): FETCH_SIZE x 2.000 (its reading for a copy kernel of known size) + WRITE_SIZE.
+TRAFFIC_DECODE_M1 = {"qo": 8836096, "kv": 2341888, "gate_up": 30483456, "down": 30626816}
+TRAFFIC_PREFILL_M2048 = {"qo": 85293056, "kv": 38443008, "gate_up": 314969088, "down": 255686656}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -47,6 +52,9 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--profile", choices=["decode", "prefill"], default=None,
+                    help="short run for rocprofv3: one copy-kernel launch of known size (the counter yardstick), "
+                         "then a few eager passes of the chosen kernel family; prints no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU only (the path has no collectives); run with --gpus 1")
@@ -85,6 +93,21 @@ def main() -> int:
     x_dev = dev.malloc(x_host.nbytes)
     y_dev = dev.malloc(m_max * max_n * 2)
     dev.upload(x_dev, x_host)
+
+    if args.profile:
+        # yardstick: one 256 MiB device-to-device copy (reads 256 MiB, writes 256 MiB)
+        dev.copy_bandwidth(256 << 20, 1)
+        if args.profile == "decode":
+            for _ in range(3):
+                for _, w in layers:
+                    req.infer_device(w, x_dev, y_dev, 1)
+        else:
+            for _ in range(3):
+                for name in datagen.LLAMA3_8B_BLOCK:
+                    req.infer_device(base[name], x_dev, y_dev, args.prefill_m)
+        req.sync()
+        log(f"profile run done ({args.profile})")
+        return 0
 
     # ---- correctness of the timed path against the oracle, before timing ----
     from oracle import oracle
@@ -168,7 +191,10 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm", "kernel": "fcc_decode_w4", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS,
-            "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+            "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "traffic": (sum(TRAFFIC_DECODE_M1[name] for name, _ in layers) // launches
+                        if set(n for n, _ in layers) <= set(TRAFFIC_DECODE_M1) else None),
+            "traffic_source": "profiles/fcc_decode_w4_llama3_8b_m1.md",
             "algorithmic_bytes_per_launch": pass_bytes // launches,
             "avg_launch_us": round(ms_per_step * 1e3 / launches, 3),
         },
@@ -196,14 +222,15 @@ def main() -> int:
         out["parity"][f"qo_M{Mp}"] = {"rel_l2": float(f"{oracle.rel_l2(y[pick], ref):.3e}"),
                                       "max_abs": float(f"{oracle.max_abs(y[pick], ref):.3e}")}
         assert out["parity"][f"qo_M{Mp}"]["rel_l2"] < 1e-3, out["parity"]
-        psteps = max(3, args.steps // 5)
-        pms = req.bench_layers(block, x_dev, y_dev, Mp, 2, psteps, use_graph=not args.no_graph)
+        psteps = max(10, args.steps // 2)
+        pwarm = max(10, args.warmup)     # the clocks take some tens of milliseconds of MFMA load to settle
+        pms = req.bench_layers(block, x_dev, y_dev, Mp, pwarm, psteps, use_graph=not args.no_graph)
         tflops = flops * psteps / (pms * 1e-3) / 1e12
         log(f"prefill M={Mp}: {pms / psteps:.3f} ms/block -> {tflops:.1f} TFLOP/s "
             f"({100 * tflops / MFMA_F16_PEAK_TFLOPS:.1f} % of 2.5 PFLOP/s)")
         pshape = {}
         for name, (K, N) in datagen.LLAMA3_8B_SHAPES.items():
-            t = req.bench_layers([base[name]], x_dev, y_dev, Mp, 2, psteps, use_graph=not args.no_graph) / psteps
+            t = req.bench_layers([base[name]], x_dev, y_dev, Mp, pwarm, psteps, use_graph=not args.no_graph) / psteps
             pshape[name] = {"us": round(t * 1e3, 2), "TFLOPs": round(2 * Mp * K * N / (t * 1e-3) / 1e12, 1)}
         log("  " + ", ".join(f"{k}: {v['us']} us {v['TFLOPs']} TFLOP/s" for k, v in pshape.items()))
         out["prefill"] = {
@@ -211,7 +238,10 @@ def main() -> int:
             "ms_per_block": round(pms / psteps, 4), "steps": psteps, "per_shape": pshape,
             "roofline": {"bound": "mfma", "kernel": "fcc_prefill_w4", "achieved": round(tflops, 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+                         "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
+                         "traffic": (sum(TRAFFIC_PREFILL_M2048[n] for n in datagen.LLAMA3_8B_BLOCK)
+                                     // len(datagen.LLAMA3_8B_BLOCK) if Mp == 2048 else None),
+                         "traffic_source": "profiles/fcc_prefill_wide_w4_llama3_8b_m2048.md"},
         }
 
     # ---- CPU baseline: the oracle on the host cores, bounded sample ----

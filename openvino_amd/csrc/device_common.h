@@ -82,6 +82,54 @@ __device__ __forceinline__ void unpack8_biased(uint32_t w0, uint32_t w1, Frag8& 
     f.u[3] = __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u);
 }
 
+// Tile coordinates of this workgroup for a 2-D tile grid, arranged for the chip's eight XCDs.  The dispatcher
+// hands consecutive workgroups to consecutive XCDs (workgroup L runs on XCD L % 8), every XCD has its own L2,
+// and one XCD runs 32 workgroups of a one-per-CU kernel at a time.  Workgroups that run together on an XCD
+// are therefore given one compact sm x sn block of tiles (sm sn <= 32), so that they share activation
+// row-blocks and weight column-blocks through that L2; sm : sn is chosen to minimise the bytes the block
+// fetches, row_cost and col_cost being the relative sizes of one tile's activation and weight strips.
+// Blocks are dealt to the XCDs round-robin; when the number of blocks is no multiple of eight, the blocks
+// of the last, partial round are cut into equal runs of tiles, one run per XCD.
+__device__ __forceinline__ void xcd_tile(int& tile_x, int& tile_y, unsigned row_cost, unsigned col_cost) {
+    const unsigned gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+    const unsigned linear = blockIdx.y * gx + blockIdx.x;
+    tile_x = (int)blockIdx.x;
+    tile_y = (int)blockIdx.y;
+    if (total & 7u)
+        return;
+    unsigned best_sn = 0, best_sm = 0;
+    for (unsigned block = 32; block > 1 && best_sn == 0; block >>= 1) {
+        unsigned best_cost = ~0u;
+        for (unsigned sn = block; sn >= 1; sn >>= 1) {
+            const unsigned sm = block / sn;
+            const unsigned cost = row_cost * sm + col_cost * sn;
+            if (gx % sn == 0 && gy % sm == 0 && cost < best_cost) {
+                best_cost = cost;
+                best_sn = sn;
+                best_sm = sm;
+            }
+        }
+    }
+    if (best_sn == 0)
+        return;
+    const unsigned sn = best_sn, sm = best_sm, block = sn * sm;
+    const unsigned xcd = linear & 7u, slot = linear >> 3;       // slot < total / 8
+    const unsigned full_rounds = (total / block) >> 3;          // rounds in which every XCD owns a whole block
+    unsigned super, within;
+    if (slot < full_rounds * block) {
+        super = (slot / block) * 8 + xcd;
+        within = slot % block;
+    } else {
+        const unsigned share = (total >> 3) - full_rounds * block;    // tiles per XCD in the partial round
+        const unsigned e = xcd * share + (slot - full_rounds * block);
+        super = full_rounds * 8 + e / block;
+        within = e % block;
+    }
+    const unsigned supers_x = gx / sn;
+    tile_x = (int)((super % supers_x) * sn + within % sn);
+    tile_y = (int)((super / supers_x) * sm + within / sn);
+}
+
 // Output cast: FullyConnected's output_type is f16 (default, the activation type) or f32.
 __device__ __forceinline__ void store_out(void* y, size_t i, float v, int out_f32) {
     if (out_f32)

@@ -29,8 +29,10 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int n0 = blockIdx.x * PF_BN;
-    const int m0 = blockIdx.y * PF_BM;
+    int tile_x, tile_y;
+    xcd_tile(tile_x, tile_y, 2 * PF_BM * 2, PF_BN * BITS / 4);
+    const int n0 = tile_x * PF_BN;
+    const int m0 = tile_y * PF_BM;
     const int nt0 = n0 / 16;
     const int col = lane & 15, kq = lane >> 4;
 

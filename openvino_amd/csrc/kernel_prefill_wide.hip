@@ -53,8 +53,10 @@ __global__ __launch_bounds__(512) void fcc_prefill_wide_kernel(const uint4_t* __
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kgrp = wave >> 2;            // which 32 inputs of a stage this wave contracts
     const int wm = (wave >> 1) & 1, wn = wave & 1;
-    const int n0 = blockIdx.x * PW_BN;
-    const int m0 = blockIdx.y * PW_BM;
+    int tile_x, tile_y;
+    xcd_tile(tile_x, tile_y, 2 * PW_BM * 2, PW_BN * BITS / 4);
+    const int n0 = tile_x * PW_BN;
+    const int m0 = tile_y * PW_BM;
     const int col = lane & 15, kq = lane >> 4;
 
     // Global loads run four stages ahead of the MFMAs (register ring), far enough to cover an L2 / HBM
