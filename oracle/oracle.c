@@ -30,6 +30,12 @@
  *                    :1819-1877), an independent numpy float64 restatement, and
  *                    algebraic invariants (zp == q gives 0, scale linearity, unit-vector
  *                    probes, i4 == u4 xor 8 with zp 8, row permutation)
+ *
+ * Parity unpinned: the CPU plugin's numbers come from the oneDNN fork's decompression
+ * inner-product kernel (openvinotoolkit/oneDNN, a submodule whose commit the tree does
+ * not record and whose sources are absent).  Its summation order and intermediate
+ * roundings are not restated here; the reference's own tests hold only tolerance checks
+ * at that boundary, and so does this oracle's use (fp32 accumulation in k order).
  */
 #include <stddef.h>
 #include <stdint.h>
