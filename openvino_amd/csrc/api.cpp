@@ -125,19 +125,22 @@ void record(ovfcc_request* r, const ovfcc::LaunchPlan& p) {
     std::snprintf(i.name, sizeof(i.name), "%s", p.name);
 }
 
-// Enqueue one node.  Rows beyond what a single launch covers (tiled node whose N is not a multiple
-// of the prefill tile) are run through the decode kernel 32 rows at a time.
+// Enqueue one node.  A tiled node is cut into decode-family launches of at most 48 rows when M is small
+// enough that they beat one sparse prefill grid, or when N is not a multiple of the prefill tile.
 int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M) {
     if (M == 0)
         return OVFCC_OK;
     ovfcc::FcDeviceArgs a;
     fill_args(w, x, y, M, &a);
     int force = r->force_kernel;
-    const bool chunked = w->layout.tiled && M > 32 && (w->desc.N % 128) != 0 &&
-                         (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL);
+    const bool chunked = w->layout.tiled && M > ovfcc::kDecodeMaxRows &&
+                         ((force == OVFCC_KERNEL_AUTO && M <= ovfcc::kChunkedMaxRows) ||
+                          ((w->desc.N % 128) != 0 && (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL)));
     if (chunked) {
-        for (int64_t m0 = 0; m0 < M; m0 += 32) {
-            const int64_t rows = M - m0 < 32 ? M - m0 : 32;
+        const int64_t chunks = (M + ovfcc::kDecodeMaxRows - 1) / ovfcc::kDecodeMaxRows;
+        const int64_t step = (M + chunks - 1) / chunks;  // equal shares rather than 48 + remainder
+        for (int64_t m0 = 0; m0 < M; m0 += step) {
+            const int64_t rows = M - m0 < step ? M - m0 : step;
             fill_args(w, static_cast<const char*>(x) + (size_t)m0 * w->desc.K * 2,
                       static_cast<char*>(y) + (size_t)m0 * w->desc.N * (w->desc.out_type == OVFCC_F32 ? 4 : 2), rows, &a);
             ovfcc::LaunchPlan p;

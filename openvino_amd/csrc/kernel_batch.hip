@@ -1,0 +1,312 @@
+// Small-batch decode kernel (M <= 48) over the tiled layout.
+//
+// With more than a few activation rows the streaming decode kernel re-reads X once per 16 output channels,
+// which costs more than the weights.  Here a workgroup owns NW * RT channel tiles and one slice of K instead:
+//
+//   grid = (ceil(N / 16 / (NW RT)), split_k), block = 64 NW.  Workgroup (g, ks) stages X[0:M, its k-range]
+//   in LDS once (rows >= M are zero) and wave w streams the k-range of its own RT channel tiles
+//   (g NW + w) RT .. +RT, one 1 KiB tile per 128-bit load per lane, DEPTH k-blocks in flight, straight
+//   from HBM into the MFMA weight operand.  The activation operand is read from LDS (lanes 0-15 of a
+//   128-bit read hit 16 different rows; the row pitch of 16 bytes more than a multiple of 256 spreads
+//   them over all banks).
+//
+// Arithmetic as in the streaming kernel: exact halves q - zp, v_mfma_f32_16x16x32_f16 with A = activations,
+// f32 partial per k-block multiplied by the group scale.  Bias and zero-point are removed on the vector
+// ALU here (one packed subtract per two weights): with two or more row tiles per weight tile the matrix
+// cores are the scarcer unit.
+//
+// No reduction inside the workgroup.  With split_k > 1 each workgroup publishes its partial tiles with
+// device-scope stores, waits for them, and draws a ticket from the group's arrival counter; the last
+// arrival adds the partials in split order (independent of arrival order) and zeroes the counter.
+#include "device_common.h"
+
+namespace ovfcc {
+
+template <int TPB, int RT>
+struct BatchSlot {
+    uint4_t w[RT][TPB];
+    half_t scale[RT];
+    uint8_t zp[RT];
+};
+
+template <int BITS, int MT, bool ZP_TABLE, int RT>
+__global__ __launch_bounds__(512) void fcc_batch_kernel(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
+                                                        const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
+                                                        const half_t* __restrict__ bias, void* __restrict__ y,
+                                                        float* __restrict__ ws, unsigned* __restrict__ counters,
+                                                        int M, int N, int K, int kb_total, int kb_per_group, int ng,
+                                                        int zp_const, int kb_per_split, int split_k, int n_tiles,
+                                                        int out_f32) {
+    constexpr int TPB = BITS == 4 ? 1 : 2;                    // tiles per k-block
+    constexpr int DEPTH = (RT * TPB >= 4) ? 2 : 4 / TPB;      // k-blocks in flight per wave
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    __shared__ unsigned ticket_s;
+    half_t* xs = reinterpret_cast<half_t*>(lds);              // [16 MT][x_stride]
+
+    const int grp = blockIdx.x;
+    const int ks = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nw = blockDim.x >> 6;
+    const int col = lane & 15;
+    const int kq = lane >> 4;
+
+    const int kb_begin = ks * kb_per_split;
+    const int kb_end = min(kb_total, kb_begin + kb_per_split);
+    const int cnt = kb_end - kb_begin;
+    const int x_stride = cnt * 128 + 8;  // halves
+
+    const int tile0 = (grp * nw + wave) * RT;
+    const int tiles_here = max(0, min(RT, n_tiles - tile0));  // 0: this wave has no channels (ragged last group)
+
+    constexpr unsigned kOob = 0x80000000u;
+    constexpr int kRsrcFlags = 0x00020000;
+    const size_t tile_base = tiles_here ? (size_t)tile0 : 0;
+    const __amdgpu_buffer_rsrc_t rw =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4_t*>(wt + tile_base * kb_total * TPB * 64), 0,
+                                          tiles_here * kb_total * TPB * kTileBytes, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(st + tile_base * ng * 16),
+                                                                        0, tiles_here * ng * 32, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rz = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(ZP_TABLE ? zt + tile_base * ng * 16 : zt), 0, ZP_TABLE ? tiles_here * ng * 16 : 0,
+        kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rx =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, M * K * 2, kRsrcFlags);
+
+    const unsigned g_mul = kb_per_group == 1 ? 0u : (unsigned)((0x100000000ull + kb_per_group - 1) / kb_per_group);
+    using Slot = BatchSlot<TPB, RT>;
+    auto issue = [&](int i, Slot& s) {
+        // bit 31 of every offset of a slot past the end of the k-range is set: out of range, reads zero
+        const unsigned oob = (unsigned)((cnt - 1 - i) >> 31) & kOob;
+        const unsigned kb = (unsigned)(kb_begin + i);
+        const unsigned g = kb_per_group == 1 ? kb : __umulhi(kb, g_mul);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const unsigned wofs = ((r * kb_total + kb) * (unsigned)(TPB * kTileBytes) + lane * 16u) | oob;
+#pragma unroll
+            for (int t = 0; t < TPB; ++t)
+                s.w[r][t] =
+                    __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rw, wofs + t * kTileBytes, 0, 2));
+            const unsigned sidx = (r * ng + g) * 16u + col;
+            s.scale[r] = __builtin_bit_cast(half_t, __builtin_amdgcn_raw_buffer_load_b16(rs, (sidx * 2u) | oob, 0, 0));
+            if constexpr (ZP_TABLE)
+                s.zp[r] = __builtin_amdgcn_raw_buffer_load_b8(rz, sidx | oob, 0, 0);
+        }
+    };
+
+    Slot slot[DEPTH];
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u)
+        issue(u, slot[u]);
+
+    // stage X[0 : 16 MT, k-range] in LDS; 16-byte chunks, coalesced along k; rows >= M read zeros
+    {
+        const int chunks_per_row = cnt * 16;
+        const int total = 16 * MT * chunks_per_row;
+        for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
+            const int m = idx / chunks_per_row, c = idx - m * chunks_per_row;
+            const unsigned ofs = (unsigned)(m * K + kb_begin * 128 + c * 8) * 2u;
+            *reinterpret_cast<uint4_t*>(&xs[m * x_stride + c * 8]) =
+                __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rx, ofs, 0, 0));
+        }
+        __syncthreads();
+    }
+    const half_t* xs_lane = xs + col * x_stride + 8 * kq;
+
+    float4_t acc[RT][MT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+            acc[r][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    auto consume = [&](int i, const Slot& s) {
+        // a slot past the end reads the last valid k-block of LDS; its scale is zero
+        const int kbl = min(i, cnt - 1);
+        half8_t a[MT][4];
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                a[t][j] = *reinterpret_cast<const half8_t*>(xs_lane + 16 * t * x_stride + kbl * 128 + 32 * j);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const float zpv = ZP_TABLE ? (float)s.zp[r] : (float)zp_const;
+            const float scale = (float)s.scale[r];
+            float4_t part[MT];
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                part[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+            if constexpr (BITS == 4) {
+                const half2_t off_lo = splat(1024.f + zpv), off_hi = splat(64.f + zpv);
+                const uint32_t wd[4] = {s.w[r][0].x, s.w[r][0].y, s.w[r][0].z, s.w[r][0].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    Frag8 b;
+                    unpack4(wd[j], off_lo, off_hi, b);
+#pragma unroll
+                    for (int t = 0; t < MT; ++t)
+                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], b.v, part[t], 0, 0, 0);
+                }
+            } else {
+                const half2_t off = splat(1024.f + zpv);
+#pragma unroll
+                for (int i2 = 0; i2 < 2; ++i2) {
+                    const uint32_t wd[4] = {s.w[r][i2].x, s.w[r][i2].y, s.w[r][i2].z, s.w[r][i2].w};
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+                        Frag8 b;
+                        unpack8(wd[2 * jj], wd[2 * jj + 1], off, b);
+#pragma unroll
+                        for (int t = 0; t < MT; ++t)
+                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], b.v, part[t], 0, 0, 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                acc[r][t].x += scale * part[t].x;
+                acc[r][t].y += scale * part[t].y;
+                acc[r][t].z += scale * part[t].z;
+                acc[r][t].w += scale * part[t].w;
+            }
+        }
+    };
+
+    for (int i = 0; i < cnt; i += DEPTH) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            consume(i + u, slot[u]);
+            issue(i + u + DEPTH, slot[u]);
+        }
+    }
+
+    float sum[RT][MT][4];
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            sum[r][t][0] = acc[r][t].x;
+            sum[r][t][1] = acc[r][t].y;
+            sum[r][t][2] = acc[r][t].z;
+            sum[r][t][3] = acc[r][t].w;
+        }
+
+    if (split_k > 1) {
+        // partial layout: [group][ks][wave][RT][MT][4 r][64 lanes] floats; only rows < M are written and read
+        constexpr int kPart = RT * MT * 256;
+        float* mine = ws + (((size_t)grp * split_k + ks) * nw + wave) * kPart;
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (r < tiles_here && 4 * kq + q + 16 * t < M)
+                        __hip_atomic_store(mine + ((r * MT + t) * 4 + q) * 64 + lane, sum[r][t][q], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+        // device-scope stores write through; once every wave's are acknowledged the ticket may be drawn
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0)
+            ticket_s = __hip_atomic_fetch_add(counters + grp, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket_s != (unsigned)(split_k - 1))
+            return;
+        // last arrival: every wave adds the partials of its own tiles in split order.  The loads are
+        // device-scope buffer loads (they must not hit a stale line of this XCD's L2), eight splits in flight;
+        // a split index past split_k falls outside the descriptor's range and reads zero.
+        constexpr int kAuxDeviceScope = 16;  // sc1
+        const unsigned s_stride = (unsigned)nw * kPart * 4u;
+        const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(
+            ws + ((size_t)grp * split_k * nw + wave) * kPart, 0, (split_k - 1) * (int)s_stride + kPart * 4, kRsrcFlags);
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                float tot[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int s0 = 0; s0 < split_k; s0 += 8) {
+                    float v[8][4];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const bool live = r < tiles_here && 4 * kq + q + 16 * t < M;
+                            const unsigned ofs =
+                                (unsigned)(s0 + u) * s_stride + (unsigned)(((r * MT + t) * 4 + q) * 64 + lane) * 4u;
+                            v[u][q] = __builtin_bit_cast(
+                                float, __builtin_amdgcn_raw_buffer_load_b32(rp, live ? ofs : kOob, 0, kAuxDeviceScope));
+                        }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q)
+                            tot[q] += v[u][q];
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    sum[r][t][q] = tot[q];
+            }
+        if (threadIdx.x == 0)
+            __hip_atomic_store(counters + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+        if (r >= tiles_here)
+            break;
+        const int n = (tile0 + r) * 16 + col;
+        const float b = bias ? (float)bias[n] : 0.f;
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int m = 4 * kq + q + 16 * t;
+                if (m < M)
+                    store_out(y, (size_t)m * N + n, sum[r][t][q] + b, out_f32);
+            }
+    }
+}
+
+template <int BITS, int MT, bool ZPT, int RT>
+static int launch_batch_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    const Layout& L = a.layout;
+    auto kern = fcc_batch_kernel<BITS, MT, ZPT, RT>;
+    if (p.dynamic_lds > 48 * 1024) {
+        static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+            if (e != hipSuccess)
+                return (int)e;
+            attr_set = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], 1), dim3(p.block), p.dynamic_lds, s, (const uint4_t*)a.w,
+                       (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
+                       a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
+                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, p.kblocks_per_split, p.split_k,
+                       (int)L.n_tiles, a.out_f32);
+    return (int)hipGetLastError();
+}
+
+template <int BITS, bool ZPT>
+static int launch_batch_bits(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    const int mt = (int)(a.M + 15) / 16;
+    const int rt = p.tiles_per_group;
+    if (mt <= 1)
+        return rt == 2 ? launch_batch_impl<BITS, 1, ZPT, 2>(a, p, s) : launch_batch_impl<BITS, 1, ZPT, 1>(a, p, s);
+    if (mt == 2)
+        return rt == 2 ? launch_batch_impl<BITS, 2, ZPT, 2>(a, p, s) : launch_batch_impl<BITS, 2, ZPT, 1>(a, p, s);
+    return rt == 2 ? launch_batch_impl<BITS, 3, ZPT, 2>(a, p, s) : launch_batch_impl<BITS, 3, ZPT, 1>(a, p, s);
+}
+
+int launch_batch(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Layout& L = a.layout;
+    if (L.bits == 4)
+        return L.zp_table ? launch_batch_bits<4, true>(a, p, s) : launch_batch_bits<4, false>(a, p, s);
+    return L.zp_table ? launch_batch_bits<8, true>(a, p, s) : launch_batch_bits<8, false>(a, p, s);
+}
+
+}  // namespace ovfcc

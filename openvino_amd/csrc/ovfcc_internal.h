@@ -79,6 +79,7 @@ struct LaunchPlan {
     int tile_m = 0, tile_n = 0;
     int tiles_per_group = 1;    // decode kernel: 16-channel tiles per workgroup
     bool x_in_lds = false;      // decode kernel: activations staged in LDS
+    bool batch = false;         // decode family: the small-batch kernel (waves own channel tiles)
     unsigned grid[3] = {1, 1, 1};
     unsigned block = 256;
     unsigned dynamic_lds = 0;   // bytes of dynamic LDS (decode kernel: the cross-wave reduction buffer)
@@ -93,10 +94,13 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
 int launch_fc(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_plain(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_decode(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_batch(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
 
+constexpr int kDecodeMaxRows = 48;                       // rows one decode-family launch covers
+constexpr int kChunkedMaxRows = 128;                     // up to here M is cut into decode launches
 constexpr int kPrefillTileM = 128, kPrefillTileN = 128;  // square prefill kernel
 constexpr int kPrefillWideN = 256;                         // wide prefill kernel: 128 x 256
 

@@ -1,8 +1,9 @@
 // Kernel choice and launch decomposition (host only).
 //
-// Policy: shapes that keep OpenVINO's layout run the plain kernel; tiled nodes run the decode kernel
-// for M <= 32 and the prefill kernel above (the roofline ridge of int4 g128 sits near M = 83; the
-// decode kernel's activation operand stops scaling at two 16-row tiles).
+// Policy: shapes that keep OpenVINO's layout run the plain kernel; tiled nodes run a decode kernel for
+// M <= 48 (the streaming kernel for a few rows, the small-batch kernel above) and the prefill kernel for more
+// (the roofline ridge of int4 g128 sits near M = 83).  The caller cuts 48 < M <= 128 into decode launches:
+// a single 128-row prefill tile per column block leaves most of the chip idle.
 #include <cstdlib>
 
 #include "ovfcc_internal.h"
@@ -10,7 +11,8 @@
 namespace ovfcc {
 
 // Tuning overrides for experiments: OVFCC_DECODE_WAVES = 4 | 8 | 16 (workgroup size),
-// OVFCC_DECODE_RT = 1 | 2 | 4 (channel tiles per workgroup), OVFCC_DECODE_XLDS = 0 | 1 (activations via LDS).
+// OVFCC_DECODE_RT = 1 | 2 | 4 (channel tiles per workgroup or wave), OVFCC_DECODE_XLDS = 0 | 1 (activations
+// via LDS), OVFCC_DECODE_BATCH = 0 | 1 (small-batch kernel instead of the streaming kernel).
 static int env_int(const char* name, int fallback) {
     const char* e = std::getenv(name);
     return e ? std::atoi(e) : fallback;
@@ -21,13 +23,13 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
     const Layout& L = a.layout;
     int kernel = force_kernel;
     if (kernel == OVFCC_KERNEL_AUTO)
-        kernel = !L.tiled ? OVFCC_KERNEL_PLAIN : (a.M <= 32 ? OVFCC_KERNEL_DECODE : OVFCC_KERNEL_PREFILL);
+        kernel = !L.tiled ? OVFCC_KERNEL_PLAIN : (a.M <= kDecodeMaxRows ? OVFCC_KERNEL_DECODE : OVFCC_KERNEL_PREFILL);
     if (kernel != OVFCC_KERNEL_PLAIN && !L.tiled)
         return fail(OVFCC_EUNSUPPORTED, "this node keeps the OpenVINO layout; only the plain kernel can run it");
     if (kernel == OVFCC_KERNEL_PLAIN && L.tiled)
         return fail(OVFCC_EUNSUPPORTED, "this node was repacked into tiles; the plain kernel needs the OpenVINO layout");
-    if (kernel == OVFCC_KERNEL_DECODE && a.M > 32)
-        return fail(OVFCC_EUNSUPPORTED, "the decode kernel handles at most 32 rows");
+    if (kernel == OVFCC_KERNEL_DECODE && a.M > kDecodeMaxRows)
+        return fail(OVFCC_EUNSUPPORTED, "the decode kernels handle at most 48 rows per launch");
     if (kernel == OVFCC_KERNEL_PREFILL && (a.N % kPrefillTileN) != 0)
         return fail(OVFCC_EUNSUPPORTED, "the prefill kernel needs N % 128 == 0");
     p.kernel = kernel;
@@ -38,7 +40,54 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.grid[1] = (unsigned)a.M;
         p.block = 64;
         p.name = "fcc_plain";
+    } else if (kernel == OVFCC_KERNEL_DECODE &&
+               env_int("OVFCC_DECODE_BATCH", (a.M > 16 || (a.M > 4 && L.w_bytes >= ((size_t)16 << 20))) ? 1 : 0) != 0) {
+        // Small-batch kernel: waves own channel tiles, the workgroup shares one staged slice of X.  It pays
+        // for its split-K epilogue, so the streaming kernel keeps M <= 4 and, for small nodes, M <= 16.
+        const int kb = (int)L.k_blocks;
+        const int mt = (int)((a.M + 15) / 16);
+        int rt = 1;
+        const int rt_env = env_int("OVFCC_DECODE_RT", 0);
+        if (rt_env == 1 || rt_env == 2)
+            rt = rt_env;
+        int nw = 8;
+        const int nw_env = env_int("OVFCC_DECODE_WAVES", 0);
+        if (nw_env == 4 || nw_env == 8)
+            nw = nw_env;
+        const int64_t groups = (L.n_tiles + nw * rt - 1) / (nw * rt);
+        auto x_bytes = [&](int per) { return (size_t)16 * mt * ((size_t)per * kBlockK + 8) * 2; };
+        const size_t lds_budget = 96 * 1024;
+        int split = force_split;
+        if (split <= 0) {
+            // split K until the grid covers the compute units (keeping at least two k-blocks per workgroup)
+            split = 1;
+            while (groups * split < n_cus && split < 8 && kb / (split * 2) >= 2)
+                split *= 2;
+        }
+        if (split > kb)
+            split = kb;
+        while (split < kb && x_bytes((kb + split - 1) / split) > lds_budget)
+            split = split * 2 < kb ? split * 2 : kb;  // the staged slice of X has to fit in LDS
+        const int per = (kb + split - 1) / split;
+        split = (kb + per - 1) / per;  // no empty splits
+        if (x_bytes(per) > lds_budget)
+            return fail(OVFCC_EUNSUPPORTED, "one k-block of the activations does not fit in LDS");
+        p.batch = true;
+        p.split_k = split;
+        p.kblocks_per_split = per;
+        p.tiles_per_group = rt;
+        p.grid[0] = (unsigned)groups;
+        p.grid[1] = (unsigned)split;
+        p.block = 64u * nw;
+        p.tile_m = 16 * mt;
+        p.tile_n = 16 * rt * nw;
+        p.workspace_bytes = split > 1 ? (size_t)groups * split * nw * rt * mt * 256 * sizeof(float) : 0;
+        p.counter_count = split > 1 ? (size_t)groups : 0;
+        p.dynamic_lds = (unsigned)x_bytes(per);
+        p.name = L.bits == 4 ? "fcc_batch_w4" : "fcc_batch_w8";
     } else if (kernel == OVFCC_KERNEL_DECODE) {
+        if (a.M > 32)
+            return fail(OVFCC_EUNSUPPORTED, "the streaming decode kernel handles at most 32 rows");
         const int kb = (int)L.k_blocks;
         const int mt = a.M <= 16 ? 1 : 2;
         // Activations go through LDS for M <= 4 when the k-range of one workgroup fits 40 KiB.
@@ -124,7 +173,7 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     case OVFCC_KERNEL_PLAIN:
         return launch_plain(a, p, stream);
     case OVFCC_KERNEL_DECODE:
-        return launch_decode(a, p, stream);
+        return p.batch ? launch_batch(a, p, stream) : launch_decode(a, p, stream);
     default:
         return p.tile_n == kPrefillWideN ? launch_prefill_wide(a, p, stream) : launch_prefill(a, p, stream);
     }

@@ -151,7 +151,9 @@ def test_decode_split_k_is_deterministic(oracle, dev, req, split, M):
     try:
         req.force_kernel(_lib.KERNEL_DECODE, split)
         first = req.infer(w, c.x)
-        assert req.last_kernel()["split_k"] <= max(1, split)
+        info = req.last_kernel()
+        # the small-batch kernel raises a forced split until its slice of X fits in LDS
+        assert info["split_k"] <= max(1, split) or info["name"].startswith("fcc_batch")
         check_parity(oracle, first, ref, 4096, f"split {split}")
         for _ in range(5):
             assert np.array_equal(req.infer(w, c.x).view(np.uint16), first.view(np.uint16))
@@ -162,26 +164,57 @@ def test_decode_split_k_is_deterministic(oracle, dev, req, split, M):
 
 def test_kernel_policy(dev, req):
     say("policy")
-    c = datagen.make_case(3, 64, 256, 128, "u4", 128, "u4")
+    c = datagen.make_case(3, 130, 256, 128, "u4", 128, "u4")
     w = fc.CompressedWeights.from_case(dev, c)
     try:
         assert w.tiled
         req.infer(w, c.x[:1])
-        assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
+        assert req.last_kernel()["name"] == "fcc_decode_w4"
         req.infer(w, c.x[:32])
+        assert req.last_kernel()["name"] == "fcc_batch_w4"
+        req.infer(w, c.x[:48])
         assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
-        req.infer(w, c.x[:33])
+        req.infer(w, c.x[:128])          # three launches of the small-batch kernel
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE and req.last_kernel()["tile_m"] == 48
+        req.infer(w, c.x[:129])
         assert req.last_kernel()["kernel"] == _lib.KERNEL_PREFILL
         req.force_kernel(_lib.KERNEL_PLAIN)
         with pytest.raises(fc.OvfccError):
             req.infer(w, c.x[:1])
         req.force_kernel(_lib.KERNEL_DECODE)
         with pytest.raises(fc.OvfccError):
-            req.infer(w, c.x[:33])
+            req.infer(w, c.x[:49])
         req.force_kernel()
         with pytest.raises(fc.OvfccError):
             req.infer(w, c.x[:, :100])
     finally:
+        w.close()
+
+
+@pytest.mark.parametrize("batch", ["0", "1"])
+@pytest.mark.parametrize("wt,zt,N,K,G", [("u4", "u4", 272, 1024, 128), ("i4", "none", 128, 2048, 256),
+                                         ("u8", "u8", 144, 512, 512), ("u8", "none", 256, 1024, 128)])
+def test_both_decode_kernels_every_row_count(oracle, dev, req, monkeypatch, wt, zt, N, K, G, batch):
+    """The streaming kernel (M <= 32) and the small-batch kernel (M <= 48) each forced over their whole range of
+    row counts, with channel-tile counts that leave the last workgroup ragged, with and without a forced split."""
+    monkeypatch.setenv("OVFCC_DECODE_BATCH", batch)
+    top = 48 if batch == "1" else 32
+    c = datagen.make_case(41, top, K, N, wt, G, zt, with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c)
+    ref = oracle_y(oracle, c)
+    try:
+        for split in (0, 1, 3):
+            req.force_kernel(_lib.KERNEL_DECODE, split)
+            for M in (1, 4, 5, 15, 16, 17, 31, 32, 33, 47, 48):
+                if M > top:
+                    continue
+                say(f"decode batch={batch} {wt}/{zt} N={N} K={K} split={split} M={M}")
+                y = req.infer(w, c.x[:M])
+                info = req.last_kernel()
+                assert info["name"].startswith("fcc_batch" if batch == "1" else "fcc_decode"), info
+                check_parity(oracle, y, ref[:M], K, f"{info}", output_rounding_slack=True)
+    finally:
+        req.force_kernel()
         w.close()
 
 
