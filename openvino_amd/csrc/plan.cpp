@@ -140,27 +140,32 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.tile_n = 16 * rt;
         p.workspace_bytes = split > 1 ? (size_t)groups * split * rt * mt * 256 * sizeof(float) : 0;
         p.counter_count = split > 1 ? (size_t)groups : 0;
-        p.dynamic_lds = (unsigned)((size_t)nw * rt * mt * 256 * sizeof(float) + (xlds ? x_bytes : 0));
+        // reduction buffer, then (LDS-staged activations) the rows of X and two sums per k-block and row
+        p.dynamic_lds = (unsigned)((size_t)nw * rt * mt * 256 * sizeof(float) + (xlds ? x_bytes + (size_t)per * 32 : 0));
         p.name = L.bits == 4 ? "fcc_decode_w4" : "fcc_decode_w8";
     } else {
-        // The wide kernel (128 x 256 tiles) runs when its grid still gives every second compute unit
-        // a tile; otherwise, or when N is not a multiple of 256, the square kernel's smaller tiles spread
-        // the work further.  OVFCC_PREFILL_WIDE = 0 | 1 overrides for experiments.
+        // The kernels with 128 x 256 tiles run when their grid still gives every second compute unit a tile;
+        // otherwise, or when N is not a multiple of 256, the square kernel's smaller tiles spread the work
+        // further.  Of the two, the register-fed kernel is the faster one; the LDS-dequantising one also needs
+        // K % 256 == 0.  OVFCC_PREFILL_WIDE = 0 | 1 and OVFCC_PREFILL_DIRECT = 0 | 1 override for experiments.
         const int64_t m_tiles = (a.M + kPrefillTileM - 1) / kPrefillTileM;
-        const bool wide_ok = (a.N % kPrefillWideN) == 0 && (a.K % 256) == 0 && a.M * a.K * 2 < ((int64_t)1 << 31);
-        bool wide = wide_ok && (a.N / kPrefillWideN) * m_tiles * 2 >= n_cus;
+        const int tiles_per_kb = L.bits == 4 ? 1 : 2;
+        const bool direct_ok = (a.N % kPrefillWideN) == 0 && a.M * a.K * 2 < ((int64_t)1 << 31) &&
+                               (int64_t)16 * L.k_blocks * tiles_per_kb * kTileBytes < ((int64_t)1 << 31);
+        const bool wide_ok = direct_ok && (a.K % 256) == 0;
+        bool big = (a.N / kPrefillWideN) * m_tiles * 2 >= n_cus;
         const int wide_env = env_int("OVFCC_PREFILL_WIDE", -1);
-        if (wide_env == 0)
-            wide = false;
-        if (wide_env == 1 && wide_ok)
-            wide = true;
+        if (wide_env >= 0)
+            big = wide_env != 0;
+        p.direct = big && direct_ok && env_int("OVFCC_PREFILL_DIRECT", 1) != 0;
+        const bool wide = p.direct || (big && wide_ok);
         p.tile_m = kPrefillTileM;
         p.tile_n = wide ? kPrefillWideN : kPrefillTileN;
         p.grid[0] = (unsigned)(a.N / p.tile_n);
         p.grid[1] = (unsigned)m_tiles;
         p.block = wide ? 512 : 256;
-        p.name = L.bits == 4 ? (wide ? "fcc_prefill_wide_w4" : "fcc_prefill_w4")
-                             : (wide ? "fcc_prefill_wide_w8" : "fcc_prefill_w8");
+        p.name = L.bits == 4 ? (p.direct ? "fcc_prefill_direct_w4" : wide ? "fcc_prefill_wide_w4" : "fcc_prefill_w4")
+                             : (p.direct ? "fcc_prefill_direct_w8" : wide ? "fcc_prefill_wide_w8" : "fcc_prefill_w8");
     }
     *plan = p;
     return OVFCC_OK;
@@ -175,6 +180,8 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     case OVFCC_KERNEL_DECODE:
         return p.batch ? launch_batch(a, p, stream) : launch_decode(a, p, stream);
     default:
+        if (p.direct)
+            return launch_prefill_direct(a, p, stream);
         return p.tile_n == kPrefillWideN ? launch_prefill_wide(a, p, stream) : launch_prefill(a, p, stream);
     }
 }
