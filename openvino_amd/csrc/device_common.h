@@ -15,6 +15,10 @@ typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_void_ptr;            // destination of a direct-to-LDS load
+typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;  // arithmetic stays in the LDS address space
 
 __device__ __forceinline__ half2_t as_half2(uint32_t u) {
     return __builtin_bit_cast(half2_t, u);
@@ -141,6 +145,11 @@ __device__ __forceinline__ void store_out(void* y, size_t i, float v, int out_f3
 __device__ __forceinline__ half2_t splat(float v) {
     const half_t h = (half_t)v;
     return half2_t{h, h};
+}
+
+// s_waitcnt vmcnt(n) alone (export and LDS/scalar counters left at their maxima); n <= 63
+constexpr int wait_vmcnt_imm(int n) {
+    return (n & 15) | ((n >> 4) << 14) | 0x0F70;
 }
 
 }  // namespace ovfcc

@@ -1,0 +1,385 @@
+// Prefill kernel for 4-bit weights with register-fed matrix-core operands and fully asynchronous data
+// movement (M > 128): 128 x 256 output tile per workgroup, 8 waves.
+//
+// grid = (N/256, ceil(M/128)), block = 512.  K advances one k-block (128 inputs) per step.
+//
+// Every operand of a k-block travels HBM/L2 -> LDS with buffer loads that write LDS directly (no registers,
+// no LDS store instructions), 16 bytes per lane:
+//   - the activation tile, 128 rows x 128 inputs f16 = 32 KiB, two k-blocks ahead, three stages; rows are
+//     256 bytes without padding and the sixteen 16-byte chunks of row r sit at chunk ^ (r & 15), so the 16
+//     rows of one 128-bit read phase hit 16 different bank groups (the swizzle is applied on the global
+//     side: a lane fetches the chunk that belongs in its linear LDS slot);
+//   - the 16 packed weight tiles of the workgroup's 256 channels (16 KiB), copied verbatim three k-blocks
+//     ahead, three stages.  A tile already has the matrix cores' operand layout (lane = channel (lane & 15),
+//     eight consecutive inputs per dword at 8 (lane >> 4)): a wave reads its 8 bytes per tile back with one
+//     LDS read and unpacks them in registers -- dequantised weights never exist in memory;
+//   - the group scales (and zero-points) of the k-block, 512 (+256) bytes, with the weights.
+// That is 6 to 7 vector-memory instructions per wave and k-block; each one costs the compute unit some
+// 15 cycles that nothing overlaps, which is why weights do not come as four 8-byte register loads per wave.
+// A wave waits for its own loads (the vector-memory counter is in order); one bare barrier per k-block
+// publishes the activations of this k-block and the weights of the next, and frees the oldest stages (a fence
+// would also wait for the loads meant to stay in flight).
+//
+// Waves: wn = wave & 3 picks 64 of the 256 channels, kg = wave >> 2 picks which two of the four 32-input
+// steps of every k-block the wave contracts.  A wave unpacks every weight it uses exactly once and multiplies
+// it with all 128 rows (eight 16-row operands read from LDS): 32 v_mfma_f32_16x16x32_f16 per step and 4
+// unpacked dwords.  After the last k-block k-group 1 hands its f32 accumulators to k-group 0 through LDS,
+// which adds, applies per-channel scale and bias and stores.
+//
+// The inner loop is software-pipelined by hand and pinned with scheduling barriers: between every two MFMAs
+// of a step sit one or two vector-ALU operations of the *next* step's unpack, and every few MFMAs one memory
+// instruction.  Left to itself the compiler emits these in bursts; the two waves of a SIMD run in lockstep
+// between barriers, so a burst in one is a burst in both and the matrix pipe idles.
+//
+// MFMA roles: A = weights (rows = channels), B = activations (columns = rows m of X); result lane holds
+// column m = lane & 15, channels 4 (lane >> 4) + r, so a lane stores four consecutive outputs of one row.
+//
+// Weights: (q - zp) * s rounded once to f16 for grouped scales; with one group per channel the exact
+// integers q - zp go to the matrix cores and the scale multiplies the f32 result.
+#include "device_common.h"
+
+namespace ovfcc {
+
+constexpr int PA_BM = 128, PA_BN = 256, PA_BK = 128;
+constexpr int PA_STAGES = 3;
+constexpr int PA_XQ = 3;  // activation operands in registers: the one in use and PA_XQ - 1 on their way from LDS
+constexpr int PA_A_BYTES = PA_BM * PA_BK * 2;  // 32 KiB per stage
+constexpr int PA_W_BYTES = 16 * kTileBytes;    // 16 KiB per stage
+constexpr int PA_P_BYTES = 1024;               // scales (512) + zero-points (256)
+constexpr int PA_W_OFF = PA_STAGES * PA_A_BYTES;
+constexpr int PA_P_OFF = PA_W_OFF + PA_STAGES * PA_W_BYTES;
+constexpr unsigned PA_LDS_BYTES = (unsigned)(PA_P_OFF + PA_STAGES * PA_P_BYTES);  // 147 KiB
+
+template <bool ZP_TABLE, bool PRESCALE>
+__global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* __restrict__ wt,
+                                                                const half_t* __restrict__ st,
+                                                                const uint8_t* __restrict__ zt,
+                                                                const half_t* __restrict__ x,
+                                                                const half_t* __restrict__ bias,
+                                                                void* __restrict__ y, int M, int N, int K,
+                                                                int kb_total, int kb_per_group, int ng, int zp_const,
+                                                                int out_f32) {
+    constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave & 3, kg = wave >> 2;
+    int tile_x, tile_y;
+    xcd_tile(tile_x, tile_y, 2 * PA_BM, PA_BN / 2);
+    const int n0 = tile_x * PA_BN;
+    const int m0 = tile_y * PA_BM;
+    const int col = lane & 15, kq = lane >> 4;
+
+    constexpr unsigned kOob = 0x80000000u;
+    constexpr int kRsrcFlags = 0x00020000;
+    // Every offset goes through the vector operand: the scalar offset of a buffer load is not range-checked.
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, M * K * 2, kRsrcFlags);
+    const int nt0 = n0 / 16;  // the workgroup's 16 channel tiles
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint4_t*>(wt + (size_t)nt0 * kb_total * 64), 0, 16 * kb_total * kTileBytes, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rs =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(st + (size_t)nt0 * ng * 16), 0, 16 * ng * 32, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rz = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(ZP_TABLE ? zt + (size_t)nt0 * ng * 16 : zt), 0, ZP_TABLE ? 16 * ng * 16 : 0, kRsrcFlags);
+    const unsigned g_mul = kb_per_group == 1 ? 0u : (unsigned)((0x100000000ull + kb_per_group - 1) / kb_per_group);
+
+    // ---- activations: direct-to-LDS load i of the wave covers rows 16 wave + 4 i .. +3 of the tile; lane ->
+    // row 4 i + (lane >> 4) of those, LDS slot lane & 15 of that row, which holds global chunk
+    // (lane & 15) ^ (row & 15).  Rows >= M lie beyond the descriptor's range and arrive as zeros.
+    // (row & 15 = 4 i + (lane >> 4) = 4 i ^ (lane >> 4), so the chunk of load i is c0 ^ 4 i.) ----
+    const unsigned a_row0 = (unsigned)((m0 + 16 * wave + (lane >> 4)) * K) * 2u;
+    const unsigned a_c0 = (unsigned)((lane & 15) ^ (lane >> 4));
+    auto dma_a = [&](int kb, int stage, int i) {
+        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(4 * i * K + kb * PA_BK) * 2u);
+        const unsigned voff = a_row0 + sterm + ((a_c0 ^ (unsigned)(4 * i)) << 4);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void_ptr)(lds3 + stage * PA_A_BYTES + (4 * wave + i) * 1024), 16,
+                                                 voff | oob, 0, 0, 0);
+    };
+    // ---- weights: the wave copies tiles 2 wave, 2 wave + 1 of the workgroup's 16 ----
+    auto dma_w = [&](int kb, int stage, int i) {
+        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const int t = 2 * wave + i;
+        const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(t * kb_total + kb) * kTileBytes);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void_ptr)(lds3 + PA_W_OFF + stage * PA_W_BYTES + t * kTileBytes),
+                                                 16, (sterm + lane * 16u) | oob, 0, 0, 0);
+    };
+    // ---- parameters: waves 0 and 1 fetch the scales of eight channel tiles each (32 bytes per tile, 4 per
+    // lane), wave 2 the zero-points of all sixteen (16 bytes per tile, 4 per lane); other waves fetch nothing ----
+    const bool has_p = (PRESCALE && wave < 2) || (ZP_TABLE && wave == 2);
+    auto dma_p = [&](int kb, int stage) {
+        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned g = kb_per_group == 1 ? (unsigned)kb : __umulhi((unsigned)kb, g_mul);
+        if (PRESCALE && wave < 2) {
+            const unsigned tile = 8u * wave + (lane >> 3);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_ptr)(lds3 + PA_P_OFF + stage * PA_P_BYTES + 256 * wave), 4,
+                                                     ((tile * ng + g) * 32u + (lane & 7) * 4u) | oob, 0, 0, 0);
+        } else if (ZP_TABLE && wave == 2) {
+            const unsigned tile = lane >> 2;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(lds3 + PA_P_OFF + stage * PA_P_BYTES + 512), 4,
+                                                     ((tile * ng + g) * 16u + (lane & 3) * 4u) | oob, 0, 0, 0);
+        }
+    };
+    // Per k-block a wave issues, in this order: 4 activation loads (for k-block + 2), then 2 weight loads and at
+    // most one parameter load (for k-block + 3).  The wait at the top of a k-block needs the activations of this
+    // k-block and the weights and parameters of the next; the instructions issued after those are one k-block's
+    // worth, at least 6.
+    constexpr int kWaitTop = 6;
+
+    // ---- the wave's share of a staged k-block of weights: 8 bytes per tile, plus scale and zero-point ----
+    typedef __attribute__((address_space(3))) const uint2_t* lds_u2_ptr;
+    typedef __attribute__((address_space(3))) const half_t* lds_half_ptr;
+    uint32_t wraw[2][4][2];
+    uint32_t wscale[2][4];  // f16 scale in both halves
+    uint32_t wzp[2][4];
+    auto read_w = [&](int par, int stage, int r) {
+        const uint2_t v = *(lds_u2_ptr)(lds3 + PA_W_OFF + stage * PA_W_BYTES + (4 * wn + r) * kTileBytes + lane * 16 + kg * 8);
+        wraw[par][r][0] = v.x, wraw[par][r][1] = v.y;
+    };
+    auto read_p = [&](int par, int stage, int r) {
+        if constexpr (PRESCALE)
+        {
+            const half_t h = *(lds_half_ptr)(lds3 + PA_P_OFF + stage * PA_P_BYTES + (4 * wn + r) * 32 + col * 2);
+            wscale[par][r] = as_u32(half2_t{h, h});
+        }
+        if constexpr (ZP_TABLE)
+            wzp[par][r] = lds3[PA_P_OFF + stage * PA_P_BYTES + 512 + (4 * wn + r) * 16 + col];
+    };
+
+    // ---- unpack, one micro-operation at a time: dword js of tile r of parity par -> f ----
+    const Unpack4Consts uc = unpack4_consts();
+    // uniform values the vector ALU can take as its one scalar operand are kept in scalar registers
+    const half2_t off_lo_c = as_half2(__builtin_amdgcn_readfirstlane(as_u32(splat(1024.f + (float)zp_const))));
+    const half2_t off_hi_c = as_half2(__builtin_amdgcn_readfirstlane(as_u32(splat(64.f + (float)zp_const))));
+    auto unpack_op = [&](int par, int r, int js, int op, Frag8& f) {
+        const uint32_t w = wraw[par][r][js];
+        if (op == 0)
+            f.u[3] = w >> 8;
+        else if (op == 1)
+            f.u[0] = (w & uc.mask_lo) | uc.magic_lo;
+        else if (op == 2)
+            f.u[1] = (w & uc.mask_hi) | uc.magic_hi;
+        else if (op == 3)
+            f.u[2] = (f.u[3] & uc.mask_lo) | uc.magic_lo;
+        else if (op == 4)
+            f.u[3] = (f.u[3] & uc.mask_hi) | uc.magic_hi;
+        else if (op < 9) {
+            const int k = op - 5;
+            half2_t off;
+            if constexpr (ZP_TABLE) {
+                const float zpv = (float)wzp[par][r];
+                off = (k & 1) ? splat(64.f + zpv) : splat(1024.f + zpv);
+            } else {
+                off = (k & 1) ? off_hi_c : off_lo_c;
+            }
+            f.h2[k] = f.h2[k] - off;
+        } else if constexpr (PRESCALE) {
+            f.h2[op - 9] *= as_half2(wscale[par][r]);
+        }
+    };
+
+    float4_t acc[4][8];  // [channel tile][row tile]
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+            acc[r][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // One k-block: 64 MFMAs -- step 0 with operand wf0 while the unpack of (par_a, dword 1) fills wf1, then
+    // step 1 with wf1 while the unpack of (par_b, dword 0) refills wf0 -- against the eight row tiles of this
+    // wave's two k-steps in activation stage `stage`; mem(i) adds the memory instructions of slot i.  The
+    // activation operands run PA_XQ - 1 row tiles ahead of the MFMAs, across the boundary between the steps.
+    auto block = [&](int stage, Frag8 (&wf0)[4], Frag8 (&wf1)[4], int par_a, int par_b, auto&& mem) {
+        typedef __attribute__((address_space(3))) const half8_t* lds_frag_ptr;
+        // operand of row tile t and step js: row 16 t + col, chunk (4 (2 kg + js) + kq) ^ col
+        const lds_byte_ptr xa0 = lds3 + stage * PA_A_BYTES + col * 256 + (((8 * kg + kq) ^ col) << 4);
+        const lds_byte_ptr xa1 = lds3 + stage * PA_A_BYTES + col * 256 + (((8 * kg + 4 + kq) ^ col) << 4);
+        auto x_at = [&](int tt) { return *(lds_frag_ptr)((tt < 8 ? xa0 : xa1) + (tt & 7) * 16 * 256); };
+        half8_t xq[PA_XQ];
+#pragma unroll
+        for (int tt = 0; tt < PA_XQ - 1; ++tt)
+            xq[tt] = x_at(tt);
+        auto slot = [&](int i) {
+            const int tt = i >> 2, r = i & 3;  // tt = 8 js + t
+            if (r == 0 && tt + PA_XQ - 1 < 16)
+                xq[(tt + PA_XQ - 1) % PA_XQ] = x_at(tt + PA_XQ - 1);
+            const int t = tt & 7;
+            if (i < 32) {
+                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf0[r].v, xq[tt % PA_XQ], acc[r][t], 0, 0, 0);
+#pragma unroll
+                for (int g = i * 4 * NOPS / 32; g < (i + 1) * 4 * NOPS / 32; ++g)
+                    unpack_op(par_a, g / NOPS, 1, g % NOPS, wf1[g / NOPS]);
+            } else {
+                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf1[r].v, xq[tt % PA_XQ], acc[r][t], 0, 0, 0);
+#pragma unroll
+                for (int g = (i - 32) * 4 * NOPS / 32; g < (i - 31) * 4 * NOPS / 32; ++g)
+                    unpack_op(par_b, g / NOPS, 0, g % NOPS, wf0[g / NOPS]);
+            }
+            mem(i);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+#pragma unroll
+        for (int i = 0; i < 32; ++i)
+            slot(i);
+#pragma unroll
+        for (int i = 32; i < 64; ++i)
+            slot(i);
+    };
+
+    // ---- prologue: activations of k-blocks 0, 1; weights and parameters of k-blocks 0, 1, 2; everything
+    // landed and published; first operand unpacked ----
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            dma_a(kb, kb, i);
+#pragma unroll
+    for (int kb = 0; kb < 3; ++kb) {
+        dma_w(kb, kb, 0);
+        dma_w(kb, kb, 1);
+        if (has_p)
+            dma_p(kb, kb);
+    }
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    Frag8 wf0[4], wf1[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        read_w(0, 0, r);
+        read_p(0, 0, r);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int op = 0; op < NOPS; ++op)
+            unpack_op(0, r, 0, op, wf0[r]);
+
+    // ---- main loop: two k-blocks per trip so that the parity of the weight registers is static.  k-blocks
+    // past the end are loaded out of range (zeros) and add nothing. ----
+    int s0 = 0;  // stage of k-block kb (activations, weights and parameters cycle alike): kb % 3
+    for (int kb0 = 0; kb0 < kb_total; kb0 += 2) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int kb = kb0 + u;
+            const int s1 = s0 == 2 ? 0 : s0 + 1;  // stage of k-block kb + 1 and kb - 2
+            const int s2 = s1 == 2 ? 0 : s1 + 1;  // stage of k-block kb + 2 and kb - 1
+            // own loads landed: activations of kb, weights and parameters of kb + 1
+            __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(kWaitTop));
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();  // everyone's have; everyone is done with k-block kb - 1
+            asm volatile("" ::: "memory");
+            // Slots 0-31 (first step): request the activations of k-block kb + 2 into the stage k-block kb - 1
+            // used; towards the end fetch the next k-block's weight bits and parameters from LDS.  Slots 32-63:
+            // request the weights and parameters of k-block kb + 3 into the stage those of k-block kb used
+            // (every wave read them before the barrier above).
+            block(s0, wf0, wf1, u, u ^ 1, [&](int i) {
+                if (i < 32 && (i & 7) == 2)
+                    dma_a(kb + 2, s2, i >> 3);
+                if (i >= 24 && i < 28)
+                    read_p(u ^ 1, s1, i - 24);
+                if (i >= 28 && i < 32)
+                    read_w(u ^ 1, s1, i - 28);
+                if (i == 36)
+                    dma_w(kb + 3, s0, 0);
+                if (i == 52)
+                    dma_w(kb + 3, s0, 1);
+                if (i == 44 && has_p)
+                    dma_p(kb + 3, s0);
+            });
+            s0 = s1;
+        }
+    }
+
+    // ---- epilogue: k-group 1 -> k-group 0 through LDS, two channel tiles at a time ----
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));  // the out-of-range loads of the last trips still target LDS
+    __syncthreads();
+    float* ex = reinterpret_cast<float*>(lds_raw);  // [wn][2 x 8 x 4][64 lanes]
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+        if (kg == 1) {
+#pragma unroll
+            for (int r2 = 0; r2 < 2; ++r2)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const float4_t v = acc[2 * hh + r2][t];
+                    float* p = ex + ((wn * 64 + (r2 * 8 + t) * 4) * 64) + lane;
+                    p[0] = v.x, p[64] = v.y, p[128] = v.z, p[192] = v.w;
+                }
+        }
+        __syncthreads();
+        if (kg == 0) {
+#pragma unroll
+            for (int r2 = 0; r2 < 2; ++r2) {
+                const int r = 2 * hh + r2;
+                const int n = n0 + 64 * wn + 16 * r + 4 * kq;  // four consecutive channels
+                float sc[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (!PRESCALE) {  // one group per channel: scales are st[n]
+                    const half4_t s4 = *reinterpret_cast<const half4_t*>(st + n);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        sc[q] = (float)s4[q];
+                }
+                if (bias) {
+                    const half4_t b4 = *reinterpret_cast<const half4_t*>(bias + n);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        bs[q] = (float)b4[q];
+                }
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const float* p = ex + ((wn * 64 + (r2 * 8 + t) * 4) * 64) + lane;
+                    const float4_t a = acc[r][t];
+                    const float v[4] = {(a.x + p[0]) * sc[0] + bs[0], (a.y + p[64]) * sc[1] + bs[1],
+                                        (a.z + p[128]) * sc[2] + bs[2], (a.w + p[192]) * sc[3] + bs[3]};
+                    const int m = m0 + 16 * t + col;
+                    if (m < M) {
+                        if (out_f32) {
+                            *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * N + n) =
+                                float4_t{v[0], v[1], v[2], v[3]};
+                        } else {
+                            *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * N + n) =
+                                half4_t{(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <bool ZPT, bool PRE>
+static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    const Layout& L = a.layout;
+    auto kern = fcc_prefill_async_kernel<ZPT, PRE>;
+    static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)PA_LDS_BYTES);
+        if (e != hipSuccess)
+            return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], 1), dim3(512), PA_LDS_BYTES, s, (const uint4_t*)a.w,
+                       (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
+                       (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
+                       L.zp_const, a.out_f32);
+    return (int)hipGetLastError();
+}
+
+int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Layout& L = a.layout;
+    if (L.bits != 4)
+        return (int)hipErrorInvalidValue;  // the planner sends 8-bit nodes to the register-ring kernel
+    if (L.groups == 1)
+        return L.zp_table ? launch_async_impl<true, false>(a, p, s) : launch_async_impl<false, false>(a, p, s);
+    return L.zp_table ? launch_async_impl<true, true>(a, p, s) : launch_async_impl<false, true>(a, p, s);
+}
+
+}  // namespace ovfcc

@@ -41,12 +41,6 @@ constexpr int PD_XQ = 2;  // activation operands in registers: the one in use an
 constexpr int PD_A_BYTES = PD_BM * PD_BK * 2;                        // 32 KiB per stage
 constexpr unsigned PD_LDS_BYTES = (unsigned)(PD_STAGES * PD_A_BYTES);  // 96 KiB (the epilogue needs 64)
 
-typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-
-// s_waitcnt vmcnt(n) alone (export and LDS/scalar counters left at their maxima); n <= 63
-constexpr int pd_wait_vm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
 template <int BITS, bool ZP_TABLE, bool PRESCALE>
 __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* __restrict__ wt,
@@ -63,7 +57,6 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
     // memory instructions a wave issues per k-block, in this order: 4 direct-to-LDS, then weights and parameters
     constexpr int RING_LOADS = 4 + (PRESCALE ? 4 : 0) + (ZP_TABLE ? 4 : 0);
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;  // arithmetic stays in the LDS address space (no null checks)
 
     const int tid = threadIdx.x;
@@ -251,7 +244,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
             const int stage = kb % PD_STAGES;
             // This wave's direct-to-LDS loads of k-block kb have landed once at most the memory instructions
             // issued after them are outstanding: the ring loads of that k-block, and all of the next one's.
-            __builtin_amdgcn_s_waitcnt(pd_wait_vm(4 + 2 * RING_LOADS));
+            __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(4 + 2 * RING_LOADS));
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();  // everyone's have; everyone is done with the stage k-block kb - 1 used
             asm volatile("" ::: "memory");
@@ -276,7 +269,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
     }
 
     // ---- epilogue: k-group 1 -> k-group 0 through LDS, two channel tiles at a time ----
-    __builtin_amdgcn_s_waitcnt(pd_wait_vm(0));  // the out-of-range loads of the last trips still target LDS
+    __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));  // the out-of-range loads of the last trips still target LDS
     __syncthreads();
     float* ex = reinterpret_cast<float*>(lds_raw);  // [wn][2 x 8 x 4][64 lanes]
 #pragma unroll

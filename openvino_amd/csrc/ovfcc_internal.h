@@ -79,7 +79,8 @@ struct LaunchPlan {
     int tile_m = 0, tile_n = 0;
     int tiles_per_group = 1;    // decode kernel: 16-channel tiles per workgroup
     bool x_in_lds = false;      // decode kernel: activations staged in LDS
-    bool direct = false;        // prefill family: the kernel that feeds weights from registers
+    bool direct = false;        // prefill family: the kernels that feed weights from registers
+    bool async_dma = false;     // ... and of those the one whose operands all travel by direct-to-LDS loads
     bool batch = false;         // decode family: the small-batch kernel (waves own channel tiles)
     unsigned grid[3] = {1, 1, 1};
     unsigned block = 256;
@@ -99,6 +100,7 @@ int launch_batch(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
 
 constexpr int kDecodeMaxRows = 48;                       // rows one decode-family launch covers

@@ -159,12 +159,14 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             big = wide_env != 0;
         p.direct = big && direct_ok && env_int("OVFCC_PREFILL_DIRECT", 1) != 0;
         const bool wide = p.direct || (big && wide_ok);
+        // 4-bit nodes take the variant whose operands all travel by direct-to-LDS loads
+        p.async_dma = p.direct && L.bits == 4 && env_int("OVFCC_PREFILL_ASYNC", 1) != 0;
         p.tile_m = kPrefillTileM;
         p.tile_n = wide ? kPrefillWideN : kPrefillTileN;
         p.grid[0] = (unsigned)(a.N / p.tile_n);
         p.grid[1] = (unsigned)m_tiles;
         p.block = wide ? 512 : 256;
-        p.name = L.bits == 4 ? (p.direct ? "fcc_prefill_direct_w4" : wide ? "fcc_prefill_wide_w4" : "fcc_prefill_w4")
+        p.name = L.bits == 4 ? (p.async_dma ? "fcc_prefill_async_w4" : p.direct ? "fcc_prefill_direct_w4" : wide ? "fcc_prefill_wide_w4" : "fcc_prefill_w4")
                              : (p.direct ? "fcc_prefill_direct_w8" : wide ? "fcc_prefill_wide_w8" : "fcc_prefill_w8");
     }
     *plan = p;
@@ -180,6 +182,8 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     case OVFCC_KERNEL_DECODE:
         return p.batch ? launch_batch(a, p, stream) : launch_decode(a, p, stream);
     default:
+        if (p.async_dma)
+            return launch_prefill_async(a, p, stream);
         if (p.direct)
             return launch_prefill_direct(a, p, stream);
         return p.tile_n == kPrefillWideN ? launch_prefill_wide(a, p, stream) : launch_prefill(a, p, stream);

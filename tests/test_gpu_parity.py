@@ -218,29 +218,34 @@ def test_both_decode_kernels_every_row_count(oracle, dev, req, monkeypatch, wt, 
         w.close()
 
 
-@pytest.mark.parametrize("direct", ["1", "0"])
+@pytest.mark.parametrize("variant", ["async", "ring", "lds"])
 @pytest.mark.parametrize("wt,zt,N,K,G,out", [
     ("u4", "u4", 256, 512, 128, "f16"), ("i4", "none", 512, 1024, 256, "f16"), ("u4", "u8", 256, 768, 128, "f32"),
     ("u4", "none", 256, 512, 512, "f16"),            # one group per channel: exact integers, scale in the epilogue
     ("u8", "u8", 256, 512, 512, "f32"), ("u8", "u8", 256, 512, 128, "f16"), ("i8", "none", 512, 256, 128, "f16"),
     ("u8", "none", 256, 1024, 256, "f16"),
 ])
-def test_256_wide_prefill_kernels_small_shapes(oracle, dev, req, monkeypatch, wt, zt, N, K, G, out, direct):
-    """The two prefill kernels with 256-channel tiles (the register-fed one and the LDS-dequantising one), forced
+def test_256_wide_prefill_kernels_small_shapes(oracle, dev, req, monkeypatch, wt, zt, N, K, G, out, variant):
+    """The prefill kernels with 256-channel tiles -- register-fed weights with every operand loaded straight into
+    LDS (4-bit only), register-fed weights through a register ring, and weights dequantised into LDS -- forced
     onto shapes small enough for the oracle to cover every output: every weight type, zero-point form, scale
     grouping, bias, both output types, row counts that leave the last row tile ragged, odd k-block counts."""
+    four_bit = wt in ("u4", "i4")
+    if variant == "async" and not four_bit:
+        pytest.skip("the all-asynchronous kernel takes 4-bit weights; 8-bit nodes run the register-ring kernel")
     monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
-    monkeypatch.setenv("OVFCC_PREFILL_DIRECT", direct)
+    monkeypatch.setenv("OVFCC_PREFILL_DIRECT", "0" if variant == "lds" else "1")
+    monkeypatch.setenv("OVFCC_PREFILL_ASYNC", "1" if variant == "async" else "0")
     c = datagen.make_case(51, 300, K, N, wt, G, zt, with_bias=True)
     w = fc.CompressedWeights.from_case(dev, c, output_type=out)
     ref = oracle_y(oracle, c)
-    want = "fcc_prefill_direct" if direct == "1" else "fcc_prefill_wide"
+    want = {"async": "fcc_prefill_async", "ring": "fcc_prefill_direct", "lds": "fcc_prefill_wide"}[variant]
     try:
         for M in (129, 256, 300):
-            say(f"wide prefill direct={direct} {wt}/{zt} N={N} K={K} G={G} out={out} M={M}")
+            say(f"256-wide prefill {variant} {wt}/{zt} N={N} K={K} G={G} out={out} M={M}")
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
-            if direct == "1" or K % 256 == 0:
+            if variant != "lds" or K % 256 == 0:
                 assert info["name"].startswith(want), info
             # grouped scales: these kernels round (q - zp) * s once to f16, an error of the same size as the
             # rounding of an f16 output, so the slack applies to the f32 output as well
