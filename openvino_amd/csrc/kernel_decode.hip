@@ -15,12 +15,10 @@
 //
 // Arithmetic per k-block: nibbles/bytes are unpacked in registers to the exact halves bias + q and
 // contracted against the activation rows on the matrix cores (A = activations, rows m; B = weights,
-// columns n; v_mfma_f32_16x16x32_f16, f32 result: lane holds column n = lane & 15, rows 4 (lane >> 4) + r).
-// Bias and zero-point leave the f32 partial sum as -(bias + zp) * sum_k x[m,k]: with LDS-staged activations
-// the sums over each k-block (one for the inputs unpacked with bias 1024, one for those with bias 64) are
-// computed once while staging, otherwise one more MFMA per k-step against the constant fragment
-// -(bias + zp) does it; either way the vector ALU only unpacks.  The group scale multiplies the f32 partial
-// sum of the k-block, so no weight is ever rounded.
+// columns n; v_mfma_f32_16x16x32_f16, f32 result: lane holds column n = lane & 15, rows 4 (lane >> 4) + r);
+// one more MFMA per k-step against the constant fragment -(bias + zp) cancels bias and zero-point in the
+// f32 accumulator, which keeps the vector ALU free for the unpack.  The group scale multiplies the f32
+// partial sum of the k-block, so no weight is ever rounded.
 //
 // Reductions: the waves of a workgroup are summed through LDS in wave order.  With split_k > 1 every
 // workgroup writes its partial tiles with device-scope stores, waits for them, and takes a ticket from a
@@ -125,67 +123,19 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
         }
     };
 
-    // Staging of X[0:M, k-range] (M <= 4): 16-byte chunks, coalesced along k.  The loads of the first
-    // XR rounds are issued ahead of the weights, so that they return first and the first k-block can be
-    // consumed while later ones are still in flight.  Sixteen consecutive chunks are one k-block: their
-    // lanes also add up its two activation sums (inputs 0,1,4,5 of every eight carry the unpack bias 1024,
-    // inputs 2,3,6,7 the bias 64; 8-bit weights use 1024 throughout and add the two sums).
-    constexpr int XR = XLDS ? 4 : 0;
-    const int chunks_per_row = (kb_end - kb_begin) * 16;
-    const int x_total = XLDS ? M * chunks_per_row : 0;
-    float* xsum = reinterpret_cast<float*>(xs + (size_t)M * x_stride);  // [k-block][4 rows][lo, hi]
-    uint4_t xr[XR > 0 ? XR : 1];
-    auto x_coord = [&](int idx, int& m, int& c) {
-        m = (idx >= chunks_per_row) + (idx >= 2 * chunks_per_row) + (idx >= 3 * chunks_per_row);
-        c = idx - m * chunks_per_row;
-    };
-    auto x_store = [&](int idx, uint4_t v) {
-        int m, c;
-        x_coord(idx, m, c);
-        Frag8 f;
-        f.u[0] = v.x, f.u[1] = v.y, f.u[2] = v.z, f.u[3] = v.w;
-        float lo = ((float)f.v[0] + (float)f.v[1]) + ((float)f.v[4] + (float)f.v[5]);
-        float hi = ((float)f.v[2] + (float)f.v[3]) + ((float)f.v[6] + (float)f.v[7]);
-#pragma unroll
-        for (int d = 1; d < 16; d <<= 1) {
-            lo += __shfl_xor(lo, d, 64);
-            hi += __shfl_xor(hi, d, 64);
-        }
-        if (idx < x_total) {
-            *reinterpret_cast<uint4_t*>(&xs[m * x_stride + c * 8]) = v;
-            if ((lane & 15) == 0) {
-                xsum[((c >> 4) * 4 + m) * 2] = lo;
-                xsum[((c >> 4) * 4 + m) * 2 + 1] = hi;
-            }
-        }
-    };
-    if constexpr (XLDS) {
-#pragma unroll
-        for (int r = 0; r < XR; ++r) {
-            const int idx = threadIdx.x + r * blockDim.x;
-            int m, c;
-            x_coord(idx, m, c);
-            const unsigned ofs = idx < x_total ? (unsigned)(m * K + kb_begin * 128 + c * 8) * 2u : kOob;
-            xr[r] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rx, ofs, 0, 0));
-        }
-    }
-
     Slot slot[DEPTH];
 #pragma unroll
     for (int u = 0; u < DEPTH; ++u)
         issue(u, slot[u]);
 
     if constexpr (XLDS) {
-#pragma unroll
-        for (int r = 0; r < XR; ++r)
-            x_store(threadIdx.x + r * blockDim.x, xr[r]);
-        // rounds beyond the prefetched ones (x_total is a multiple of 16, so the sixteen lanes that share a
-        // k-block enter or leave together)
-        for (int idx = threadIdx.x + XR * blockDim.x; idx < x_total; idx += blockDim.x) {
-            int m, c;
-            x_coord(idx, m, c);
-            const unsigned ofs = (unsigned)(m * K + kb_begin * 128 + c * 8) * 2u;
-            x_store(idx, __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rx, ofs, 0, 0)));
+        // stage X[0:M, k-range of this workgroup] once; 16-byte chunks, coalesced along k
+        const int chunks_per_row = (kb_end - kb_begin) * 16;
+        const int total = M * chunks_per_row;
+        for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
+            const int m = idx / chunks_per_row, c = idx - m * chunks_per_row;
+            *reinterpret_cast<uint4_t*>(&xs[m * x_stride + c * 8]) =
+                *reinterpret_cast<const uint4_t*>(x + (size_t)m * K + (size_t)kb_begin * 128 + c * 8);
         }
         __syncthreads();
     }
@@ -215,22 +165,16 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
                 for (int j = 0; j < 4; ++j)
                     a[t][j] = s.a[t][j];
         }
-        // activation sums of this k-block, rows 0..3 (every lane reads the same 32 bytes)
-        float4_t xs_lo_hi[2];
-        if constexpr (XLDS) {
-            const int kbl = i < cnt ? wave + nw * i : 0;
-            xs_lo_hi[0] = *reinterpret_cast<const float4_t*>(xsum + kbl * 8);
-            xs_lo_hi[1] = *reinterpret_cast<const float4_t*>(xsum + kbl * 8 + 4);
-        }
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
             const float zpv = ZP_TABLE ? (float)s.zp[r] : (float)zp_const;
             const float scale = (float)s.scale[r];
-            float4_t part[MT], part2[MT];  // two accumulators: independent MFMA chains
+            float4_t part[MT];
 #pragma unroll
             for (int t = 0; t < MT; ++t)
-                part[t] = part2[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-            // weights enter the matrix cores with their unpack bias (1024 + q, 64 + q)
+                part[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+            // weights enter the matrix cores with their unpack bias (1024 + q, 64 + q); a second MFMA against
+            // the constant fragment -(bias + zp) removes bias and zero-point inside the f32 accumulator
             Frag8 bc;
             if constexpr (BITS == 4) {
                 bc.h2[0] = bc.h2[2] = splat(-(1024.f + zpv));
@@ -242,12 +186,8 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
                     unpack4_biased(wd[j], uc, b);
 #pragma unroll
                     for (int t = 0; t < MT; ++t) {
-                        if (j & 1)
-                            part2[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], b.v, part2[t], 0, 0, 0);
-                        else
-                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], b.v, part[t], 0, 0, 0);
-                        if constexpr (!XLDS)
-                            part2[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], bc.v, part2[t], 0, 0, 0);
+                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], b.v, part[t], 0, 0, 0);
+                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], bc.v, part[t], 0, 0, 0);
                     }
                 }
             } else {
@@ -261,30 +201,18 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
                         unpack8_biased(wd[2 * jj], wd[2 * jj + 1], b);
 #pragma unroll
                         for (int t = 0; t < MT; ++t) {
-                            if (jj & 1)
-                                part2[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], b.v, part2[t], 0, 0, 0);
-                            else
-                                part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], b.v, part[t], 0, 0, 0);
-                            if constexpr (!XLDS)
-                                part2[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], bc.v, part2[t], 0, 0, 0);
+                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], b.v, part[t], 0, 0, 0);
+                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], bc.v, part[t], 0, 0, 0);
                         }
                     }
                 }
             }
-            if constexpr (XLDS) {
-                // remove bias and zero-point: -(1024 + zp) * sum_lo - (64 + zp) * sum_hi per row
-                const float c_lo = -(1024.f + zpv), c_hi = BITS == 4 ? -(64.f + zpv) : c_lo;
-                part2[0].x += c_lo * xs_lo_hi[0].x + c_hi * xs_lo_hi[0].y;
-                part2[0].y += c_lo * xs_lo_hi[0].z + c_hi * xs_lo_hi[0].w;
-                part2[0].z += c_lo * xs_lo_hi[1].x + c_hi * xs_lo_hi[1].y;
-                part2[0].w += c_lo * xs_lo_hi[1].z + c_hi * xs_lo_hi[1].w;
-            }
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                acc[r][t].x += scale * (part[t].x + part2[t].x);
-                acc[r][t].y += scale * (part[t].y + part2[t].y);
-                acc[r][t].z += scale * (part[t].z + part2[t].z);
-                acc[r][t].w += scale * (part[t].w + part2[t].w);
+                acc[r][t].x += scale * part[t].x;
+                acc[r][t].y += scale * part[t].y;
+                acc[r][t].z += scale * part[t].z;
+                acc[r][t].w += scale * part[t].w;
             }
         }
     };

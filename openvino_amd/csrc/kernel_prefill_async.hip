@@ -56,9 +56,10 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
                                                                 const uint8_t* __restrict__ zt,
                                                                 const half_t* __restrict__ x,
                                                                 const half_t* __restrict__ bias,
-                                                                void* __restrict__ y, int M, int N, int K,
+                                                                void* __restrict__ y, float* __restrict__ ws,
+                                                                unsigned* __restrict__ counters, int M, int N, int K,
                                                                 int kb_total, int kb_per_group, int ng, int zp_const,
-                                                                int out_f32) {
+                                                                int kb_per_split, int split_k, int out_f32) {
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
@@ -72,6 +73,9 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
     const int n0 = tile_x * PA_BN;
     const int m0 = tile_y * PA_BM;
     const int col = lane & 15, kq = lane >> 4;
+    // split-K: workgroup z contracts k-blocks [kb_lo, kb_hi); loads of k-blocks past kb_hi are sent out of range
+    const int kb_lo = blockIdx.z * kb_per_split;
+    const int kb_hi = min(kb_total, kb_lo + kb_per_split);
 
     constexpr unsigned kOob = 0x80000000u;
     constexpr int kRsrcFlags = 0x00020000;
@@ -93,7 +97,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
     const unsigned a_row0 = (unsigned)((m0 + 16 * wave + (lane >> 4)) * K) * 2u;
     const unsigned a_c0 = (unsigned)((lane & 15) ^ (lane >> 4));
     auto dma_a = [&](int kb, int stage, int i) {
-        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(4 * i * K + kb * PA_BK) * 2u);
         const unsigned voff = a_row0 + sterm + ((a_c0 ^ (unsigned)(4 * i)) << 4);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void_ptr)(lds3 + stage * PA_A_BYTES + (4 * wave + i) * 1024), 16,
@@ -101,7 +105,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
     };
     // ---- weights: the wave copies tiles 2 wave, 2 wave + 1 of the workgroup's 16 ----
     auto dma_w = [&](int kb, int stage, int i) {
-        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         const int t = 2 * wave + i;
         const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(t * kb_total + kb) * kTileBytes);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void_ptr)(lds3 + PA_W_OFF + stage * PA_W_BYTES + t * kTileBytes),
@@ -111,7 +115,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
     // lane), wave 2 the zero-points of all sixteen (16 bytes per tile, 4 per lane); other waves fetch nothing ----
     const bool has_p = (PRESCALE && wave < 2) || (ZP_TABLE && wave == 2);
     auto dma_p = [&](int kb, int stage) {
-        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         const unsigned g = kb_per_group == 1 ? (unsigned)kb : __umulhi((unsigned)kb, g_mul);
         if (PRESCALE && wave < 2) {
             const unsigned tile = 8u * wave + (lane >> 3);
@@ -232,16 +236,16 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
     // ---- prologue: activations of k-blocks 0, 1; weights and parameters of k-blocks 0, 1, 2; everything
     // landed and published; first operand unpacked ----
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            dma_a(kb, kb, i);
+            dma_a(kb_lo + j, j, i);
 #pragma unroll
-    for (int kb = 0; kb < 3; ++kb) {
-        dma_w(kb, kb, 0);
-        dma_w(kb, kb, 1);
+    for (int j = 0; j < 3; ++j) {
+        dma_w(kb_lo + j, j, 0);
+        dma_w(kb_lo + j, j, 1);
         if (has_p)
-            dma_p(kb, kb);
+            dma_p(kb_lo + j, j);
     }
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));
     asm volatile("" ::: "memory");
@@ -262,7 +266,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
     // ---- main loop: two k-blocks per trip so that the parity of the weight registers is static.  k-blocks
     // past the end are loaded out of range (zeros) and add nothing. ----
     int s0 = 0;  // stage of k-block kb (activations, weights and parameters cycle alike): kb % 3
-    for (int kb0 = 0; kb0 < kb_total; kb0 += 2) {
+    for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += 2) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int kb = kb0 + u;
@@ -295,10 +299,53 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
         }
     }
 
-    // ---- epilogue: k-group 1 -> k-group 0 through LDS, two channel tiles at a time ----
+    // ---- epilogue: k-group 1 -> k-group 0 through LDS, two channel tiles at a time.  Without split-K k-group 0
+    // finishes the outputs; with split-K it parks the f32 tile in the workspace with device-scope stores and
+    // waits for them, the workgroup draws a ticket from the tile's arrival counter, and the last arrival adds
+    // the parked tiles in split order with device-scope loads (the result does not depend on arrival order),
+    // finishes the outputs and returns the counter to zero.  No fences: a device-scope fence writes back and
+    // invalidates whole caches, which costs more than the kernel. ----
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));  // the out-of-range loads of the last trips still target LDS
     __syncthreads();
     float* ex = reinterpret_cast<float*>(lds_raw);  // [wn][2 x 8 x 4][64 lanes]
+    __shared__ unsigned ticket_s;
+    const int tile_id = tile_y * gridDim.x + tile_x;
+    // parked tile layout: [tile][split][wn][channel tile r][row tile t][lane] float4
+    constexpr int kAuxDeviceScope = 16;              // sc1: write through to / read from memory shared by all XCDs
+    constexpr unsigned kParkBytes = 4 * 32 * 64 * 16;  // one workgroup's f32 tile
+    const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<char*>(ws) + (size_t)tile_id * split_k * kParkBytes, 0, split_k * (int)kParkBytes, kRsrcFlags);
+    auto finish = [&](int r, int t, float4_t v, const float (&sc)[4], const float (&bs)[4]) {
+        const int n = n0 + 64 * wn + 16 * r + 4 * kq;  // four consecutive channels
+        const int m = m0 + 16 * t + col;
+        const float o[4] = {v.x * sc[0] + bs[0], v.y * sc[1] + bs[1], v.z * sc[2] + bs[2], v.w * sc[3] + bs[3]};
+        if (m < M) {
+            if (out_f32) {
+                *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * N + n) = float4_t{o[0], o[1], o[2], o[3]};
+            } else {
+                *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * N + n) =
+                    half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
+            }
+        }
+    };
+    auto channel_params = [&](int r, float (&sc)[4], float (&bs)[4]) {
+        const int n = n0 + 64 * wn + 16 * r + 4 * kq;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            sc[q] = 1.f, bs[q] = 0.f;
+        if constexpr (!PRESCALE) {  // one group per channel: scales are st[n]
+            const half4_t s4 = *reinterpret_cast<const half4_t*>(st + n);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                sc[q] = (float)s4[q];
+        }
+        if (bias) {
+            const half4_t b4 = *reinterpret_cast<const half4_t*>(bias + n);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                bs[q] = (float)b4[q];
+        }
+    };
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh) {
         if (kg == 1) {
@@ -316,41 +363,55 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
 #pragma unroll
             for (int r2 = 0; r2 < 2; ++r2) {
                 const int r = 2 * hh + r2;
-                const int n = n0 + 64 * wn + 16 * r + 4 * kq;  // four consecutive channels
-                float sc[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (!PRESCALE) {  // one group per channel: scales are st[n]
-                    const half4_t s4 = *reinterpret_cast<const half4_t*>(st + n);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        sc[q] = (float)s4[q];
-                }
-                if (bias) {
-                    const half4_t b4 = *reinterpret_cast<const half4_t*>(bias + n);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        bs[q] = (float)b4[q];
-                }
+                float sc[4], bs[4];
+                channel_params(r, sc, bs);
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
                     const float* p = ex + ((wn * 64 + (r2 * 8 + t) * 4) * 64) + lane;
                     const float4_t a = acc[r][t];
-                    const float v[4] = {(a.x + p[0]) * sc[0] + bs[0], (a.y + p[64]) * sc[1] + bs[1],
-                                        (a.z + p[128]) * sc[2] + bs[2], (a.w + p[192]) * sc[3] + bs[3]};
-                    const int m = m0 + 16 * t + col;
-                    if (m < M) {
-                        if (out_f32) {
-                            *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * N + n) =
-                                float4_t{v[0], v[1], v[2], v[3]};
-                        } else {
-                            *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * N + n) =
-                                half4_t{(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                        }
-                    }
+                    const float4_t v = float4_t{a.x + p[0], a.y + p[64], a.z + p[128], a.w + p[192]};
+                    if (split_k == 1)
+                        finish(r, t, v, sc, bs);
+                    else
+                        __builtin_amdgcn_raw_buffer_store_b128(
+                            __builtin_bit_cast(uint4_t, v), rp,
+                            blockIdx.z * kParkBytes + (unsigned)(((wn * 4 + r) * 8 + t) * 64 + lane) * 16u, 0,
+                            kAuxDeviceScope);
                 }
             }
         }
         __syncthreads();
     }
+    if (split_k == 1)
+        return;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the parked tile has reached memory before the ticket is drawn
+    __syncthreads();
+    if (tid == 0)
+        ticket_s = __hip_atomic_fetch_add(counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket_s != (unsigned)(split_k - 1))
+        return;
+    if (kg == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float sc[4], bs[4];
+            channel_params(r, sc, bs);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                float4_t v = float4_t{0.f, 0.f, 0.f, 0.f};
+                for (int z = 0; z < split_k; ++z) {
+                    const float4_t pz = __builtin_bit_cast(
+                        float4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                      rp, z * kParkBytes + (unsigned)(((wn * 4 + r) * 8 + t) * 64 + lane) * 16u, 0,
+                                      kAuxDeviceScope));
+                    v.x += pz.x, v.y += pz.y, v.z += pz.z, v.w += pz.w;
+                }
+                finish(r, t, v, sc, bs);
+            }
+        }
+    }
+    if (tid == 0)
+        __hip_atomic_store(counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <bool ZPT, bool PRE>
@@ -365,10 +426,10 @@ static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
             return (int)e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], 1), dim3(512), PA_LDS_BYTES, s, (const uint4_t*)a.w,
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), PA_LDS_BYTES, s, (const uint4_t*)a.w,
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
-                       (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
-                       L.zp_const, a.out_f32);
+                       a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
+                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, p.kblocks_per_split, p.split_k, a.out_f32);
     return (int)hipGetLastError();
 }
 

@@ -140,8 +140,7 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.tile_n = 16 * rt;
         p.workspace_bytes = split > 1 ? (size_t)groups * split * rt * mt * 256 * sizeof(float) : 0;
         p.counter_count = split > 1 ? (size_t)groups : 0;
-        // reduction buffer, then (LDS-staged activations) the rows of X and two sums per k-block and row
-        p.dynamic_lds = (unsigned)((size_t)nw * rt * mt * 256 * sizeof(float) + (xlds ? x_bytes + (size_t)per * 32 : 0));
+        p.dynamic_lds = (unsigned)((size_t)nw * rt * mt * 256 * sizeof(float) + (xlds ? x_bytes : 0));
         p.name = L.bits == 4 ? "fcc_decode_w4" : "fcc_decode_w8";
     } else {
         // The kernels with 128 x 256 tiles run when their grid still gives every second compute unit a tile;
@@ -153,7 +152,14 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         const bool direct_ok = (a.N % kPrefillWideN) == 0 && a.M * a.K * 2 < ((int64_t)1 << 31) &&
                                (int64_t)16 * L.k_blocks * tiles_per_kb * kTileBytes < ((int64_t)1 << 31);
         const bool wide_ok = direct_ok && (a.K % 256) == 0;
-        bool big = (a.N / kPrefillWideN) * m_tiles * 2 >= n_cus;
+        // (the 4-bit register-fed kernel can also split K, which multiplies its grid by up to eight)
+        const bool may_split = direct_ok && L.bits == 4 && env_int("OVFCC_PREFILL_DIRECT", 1) != 0 &&
+                               env_int("OVFCC_PREFILL_ASYNC", 1) != 0;
+        int64_t reach = (a.N / kPrefillWideN) * m_tiles;
+        if (may_split)
+            for (int split = 1; split < 8 && reach * 2 <= n_cus && L.k_blocks / (split * 2) >= 8; split *= 2)
+                reach *= 2;
+        bool big = reach * 2 >= n_cus;
         const int wide_env = env_int("OVFCC_PREFILL_WIDE", -1);
         if (wide_env >= 0)
             big = wide_env != 0;
@@ -165,6 +171,25 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.tile_n = wide ? kPrefillWideN : kPrefillTileN;
         p.grid[0] = (unsigned)(a.N / p.tile_n);
         p.grid[1] = (unsigned)m_tiles;
+        p.kblocks_per_split = (int)L.k_blocks;
+        if (p.async_dma) {
+            // split K while the tiles alone leave compute units idle (at least eight k-blocks per workgroup);
+            // the f32 tiles are parked in the workspace and added by the last workgroup to arrive
+            const int64_t tiles = (int64_t)p.grid[0] * p.grid[1];
+            int split = force_split > 0 ? force_split : 1;
+            if (force_split <= 0)
+                while (split < 8 && tiles * split * 2 <= n_cus && L.k_blocks / (split * 2) >= 8)
+                    split *= 2;
+            if (split > L.k_blocks)
+                split = (int)L.k_blocks;
+            const int per = (int)((L.k_blocks + split - 1) / split);
+            split = (int)((L.k_blocks + per - 1) / per);
+            p.split_k = split;
+            p.kblocks_per_split = per;
+            p.grid[2] = (unsigned)split;
+            p.workspace_bytes = split > 1 ? (size_t)tiles * split * kPrefillTileM * kPrefillWideN * sizeof(float) : 0;
+            p.counter_count = split > 1 ? (size_t)tiles : 0;
+        }
         p.block = wide ? 512 : 256;
         p.name = L.bits == 4 ? (p.async_dma ? "fcc_prefill_async_w4" : p.direct ? "fcc_prefill_direct_w4" : wide ? "fcc_prefill_wide_w4" : "fcc_prefill_w4")
                              : (p.direct ? "fcc_prefill_direct_w8" : wide ? "fcc_prefill_wide_w8" : "fcc_prefill_w8");

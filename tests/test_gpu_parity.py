@@ -254,6 +254,35 @@ def test_256_wide_prefill_kernels_small_shapes(oracle, dev, req, monkeypatch, wt
         w.close()
 
 
+@pytest.mark.parametrize("wt,zt,N,K,G", [("i4", "none", 256, 2048, 128), ("u4", "u4", 512, 1280, 256),
+                                         ("u4", "none", 256, 1024, 1024)])
+@pytest.mark.parametrize("split", [2, 3, 8])
+def test_prefill_split_k_is_deterministic(oracle, dev, req, monkeypatch, wt, zt, N, K, G, split):
+    """The 4-bit register-fed prefill kernel with K split over workgroups: any split gives the oracle's answer
+    (ragged last split, ragged last row tile, bias, per-channel scale in the fix-up), repeated launches give
+    identical bits, and the arrival counters return to zero."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    c = datagen.make_case(61, 200, K, N, wt, G, zt, with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c)
+    ref = oracle_y(oracle, c)
+    try:
+        req.force_kernel(_lib.KERNEL_PREFILL, split)
+        say(f"prefill split {split} {wt}/{zt} N={N} K={K} G={G}")
+        first = req.infer(w, c.x)
+        info = req.last_kernel()
+        assert info["name"] == "fcc_prefill_async_w4" and info["split_k"] > 1, info
+        check_parity(oracle, first, ref, K, f"{info}", output_rounding_slack=True)
+        for _ in range(4):
+            assert np.array_equal(req.infer(w, c.x).view(np.uint16), first.view(np.uint16))
+        req.force_kernel(_lib.KERNEL_PREFILL, 1)
+        one = req.infer(w, c.x)
+        assert req.last_kernel()["split_k"] == 1
+        check_parity(oracle, one, ref, K, "unsplit", output_rounding_slack=True)
+    finally:
+        req.force_kernel()
+        w.close()
+
+
 def test_decode_and_prefill_agree(oracle, dev, req):
     """Same inputs through both tiled kernels at M = 32 (full output, every tile)."""
     say("decode vs prefill")
