@@ -68,6 +68,29 @@ __global__ __launch_bounds__(256) void fcc_copy_kernel(uint4_t* __restrict__ dst
 }
 
 
+// ------------------------------------------------------------------------------------------------
+// Read-only sweep over a weight buffer: pulls it through L2 into the memory-side Infinity Cache ahead of
+// the kernel that will consume it.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fcc_touch_kernel(const uint4_t* __restrict__ src, size_t n16) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint4_t acc = {0, 0, 0, 0};
+    for (; i < n16; i += stride) {
+        const uint4_t v = src[i];
+        acc.x ^= v.x, acc.y ^= v.y, acc.z ^= v.z, acc.w ^= v.w;
+    }
+    asm volatile("" ::"v"(acc.x), "v"(acc.y), "v"(acc.z), "v"(acc.w));  // keeps the loads alive
+}
+
+int launch_touch(const void* src, size_t bytes, void* stream) {
+    const size_t n16 = bytes / 16;
+    const unsigned blocks = (unsigned)((n16 + 256 * 4 - 1) / (256 * 4));  // four loads per thread
+    hipLaunchKernelGGL(fcc_touch_kernel, dim3(blocks ? blocks : 1), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       (const uint4_t*)src, n16);
+    return (int)hipGetLastError();
+}
+
 int launch_plain(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipLaunchKernelGGL(fcc_plain_kernel, dim3(p.grid[0], p.grid[1], 1), dim3(64), 0, static_cast<hipStream_t>(stream),
                        (const uint8_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.bias,

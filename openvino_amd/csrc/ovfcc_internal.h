@@ -102,6 +102,7 @@ int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* str
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
+int launch_touch(const void* src, size_t bytes, void* stream);
 
 constexpr int kDecodeMaxRows = 48;                       // rows one decode-family launch covers
 constexpr int kChunkedMaxRows = 128;                     // up to here M is cut into decode launches
