@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/ (counters cannot be
 # read from inside this process): FETCH_SIZE x 2.000 (its reading for a copy kernel of known size) + WRITE_SIZE.
 TRAFFIC_DECODE_M1 = {"qo": 8836096, "kv": 2341888, "gate_up": 30483456, "down": 30626816}
-TRAFFIC_PREFILL_M2048 = {"qo": 85293056, "kv": 38443008, "gate_up": 314969088, "down": 255686656}
+TRAFFIC_PREFILL_M2048 = {"qo": 90240000, "kv": 110650368, "gate_up": 363849728, "down": 260682752}
 
 
 def log(*a):
@@ -39,6 +39,77 @@ def log(*a):
 def algorithmic_bytes(K, N, M, bits=4, group=128, zp_bytes_per_group=0.0):
     ng = K // group
     return N * K * bits // 8 + N * ng * 2 + int(N * ng * zp_bytes_per_group) + M * K * 2 + M * N * 2
+
+
+def results_table(dev, req, args) -> int:
+    """All five benchmark configurations: kernel time with device-resident operands (HIP graph over a rotating set of
+    weight copies larger than the caches), derived GB/s and TFLOP/s, and parity against the CPU oracle on a seeded
+    sample of rows (every output channel)."""
+    from openvino_amd import datagen, fc
+    from oracle import oracle
+
+    type_tag = {"u4": oracle.U4, "i4": oracle.I4, "u8": oracle.U8, "i8": oracle.I8, "none": oracle.NONE}
+    rows = []
+
+    def run(cfg, label, c, Ms, bits, zp_bytes_per_group, dtype):
+        w = fc.CompressedWeights.from_case(dev, c)
+        copies = [w]
+        while sum(h.device_bytes for h in copies) < (600 << 20) and len(copies) < 48:
+            copies.append(w.clone())
+        x_dev = dev.malloc(c.x.nbytes)
+        y_dev = dev.malloc(c.M * c.N * 2)
+        for M in Ms:
+            xs = np.ascontiguousarray(c.x[:M])
+            y = req.infer(w, xs).astype(np.float32)
+            info = req.last_kernel()
+            pick = np.sort(np.random.default_rng(99).choice(M, size=min(16, M), replace=False))
+            ref = oracle.fc_reference(xs[pick], c.w, type_tag[c.w_type], c.scale, c.zp, type_tag[c.zp_type], None,
+                                      N=c.N, K=c.K, group_size=c.group_size)
+            rl2, mab = oracle.rel_l2(y[pick], ref), oracle.max_abs(y[pick], ref)
+            dev.upload(x_dev, xs)
+            hs = copies if M <= 128 else copies[:1]
+            reps = 20 if M <= 128 else 10
+            best = min(req.bench_layers(hs, x_dev, y_dev, M, 3, reps, use_graph=True) for _ in range(2))
+            us = best / reps / len(hs) * 1e3
+            nbytes = algorithmic_bytes(c.K, c.N, M, bits, c.group_size, zp_bytes_per_group)
+            gbs, tfs = nbytes / us / 1e3, 2.0 * M * c.N * c.K / us / 1e6
+            rows.append(f"| {cfg} | {label} {c.K}->{c.N} | {M} | {dtype} | {info['name']} | {us:.1f} | "
+                        f"{gbs:.0f} ({100 * gbs / HBM_PEAK_GBS:.1f} %) | {tfs:.1f} ({100 * tfs / 1000 / 2.5:.1f} %) | "
+                        f"{rl2:.1e} | {mab:.1e} |")
+            log(rows[-1])
+        for h in copies:
+            h.close()
+        dev.free(x_dev)
+        dev.free(y_dev)
+
+    run(1, "q/o", datagen.config1(), [1], 4, 0.5, "u4 g128 asym")
+    for shape in datagen.LLAMA3_8B_SHAPES:
+        run(2, shape, datagen.config2(shape, 32), [1, 4, 16, 32], 4, 0.0, "i4 g128 sym")
+    for shape in datagen.LLAMA3_8B_SHAPES:
+        run(3, shape, datagen.config3(shape, 8192), [512, 2048, 8192], 4, 0.0, "i4 g128 sym")
+    for shape in datagen.LLAMA3_70B_SHAPES:
+        run(4, shape, datagen.config4(shape, 1024), [1, 32, 1024], 8, 1.0, "u8 per-channel asym")
+    routes = datagen.moe_routing()
+    t_total, flops_total = 0.0, 0.0
+    for e, tokens in enumerate(routes):
+        for which in ("gate", "up", "down"):
+            n0 = len(rows)
+            run(5, f"expert {e} {which}", datagen.config5_expert(e, which, len(tokens)), [len(tokens)], 4, 0.5,
+                "u4 g128 asym")
+            us = float(rows[n0].split("|")[6])
+            K, N = (4096, 14336) if which != "down" else (14336, 4096)
+            t_total += us
+            flops_total += 2.0 * len(tokens) * K * N
+    log(f"config 5 as 24 separate launches: {t_total:.1f} us in total, {flops_total / t_total / 1e6:.1f} TFLOP/s")
+    print("| Config | Shape (K->N) | M | dtype | GPU kernel | us | GB/s (% of 8 TB/s) | TFLOP/s (% of 2.5 PF) | "
+          "rel-L2 vs fp32 | max-abs |")
+    print("|---|---|---|---|---|---|---|---|---|---|")
+    for r in rows:
+        print(r)
+    print(f"\nconfig 5 as 24 separate launches: {t_total:.1f} us in total, {flops_total / t_total / 1e6:.1f} TFLOP/s")
+    req.close()
+    dev.close()
+    return 0
 
 
 def main() -> int:
@@ -52,6 +123,9 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--table", action="store_true",
+                    help="time and parity-check every benchmark configuration (1-5) and print a markdown table on "
+                         "stdout instead of the JSON line")
     ap.add_argument("--profile", choices=["decode", "prefill"], default=None,
                     help="short run for rocprofv3: one copy-kernel launch of known size (the counter yardstick), "
                          "then a few eager passes of the chosen kernel family; prints no JSON")
@@ -68,6 +142,8 @@ def main() -> int:
 
     dev = fc.Device(0)
     req = fc.InferRequest(dev)
+    if args.table:
+        return results_table(dev, req, args)
 
     # ---- weights: one host tensor set per shape, one device copy per use ----
     t0 = time.perf_counter()
@@ -236,12 +312,12 @@ def main() -> int:
         out["prefill"] = {
             "M": Mp, "TFLOPs": round(tflops, 2), "pct_of_mfma_peak": round(100 * tflops / MFMA_F16_PEAK_TFLOPS, 2),
             "ms_per_block": round(pms / psteps, 4), "steps": psteps, "per_shape": pshape,
-            "roofline": {"bound": "mfma", "kernel": "fcc_prefill_w4", "achieved": round(tflops, 2),
+            "roofline": {"bound": "mfma", "kernel": "fcc_prefill_async_w4", "achieved": round(tflops, 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": (sum(TRAFFIC_PREFILL_M2048[n] for n in datagen.LLAMA3_8B_BLOCK)
                                      // len(datagen.LLAMA3_8B_BLOCK) if Mp == 2048 else None),
-                         "traffic_source": "profiles/fcc_prefill_wide_w4_llama3_8b_m2048.md"},
+                         "traffic_source": "profiles/fcc_prefill_async_w4_llama3_8b_m2048.md"},
         }
 
     # ---- CPU baseline: the oracle on the host cores, bounded sample ----
