@@ -101,12 +101,49 @@ def results_table(dev, req, args) -> int:
             t_total += us
             flops_total += 2.0 * len(tokens) * K * N
     log(f"config 5 as 24 separate launches: {t_total:.1f} us in total, {flops_total / t_total / 1e6:.1f} TFLOP/s")
+
+    # The same 24 nodes as grouped runs: gate and up of all experts in one call (16 nodes of one shape), down in another.
+    t_grouped = 0.0
+    for label, names in (("experts gate+up, 16 nodes grouped", ("gate", "up")), ("experts down, 8 nodes grouped", ("down",))):
+        cases = [datagen.config5_expert(e, which, len(routes[e])) for which in names for e in range(len(routes))]
+        ws = [fc.CompressedWeights.from_case(dev, c) for c in cases]
+        bufs = [(dev.malloc(c.x.nbytes), dev.malloc(c.M * c.N * 2)) for c in cases]
+        for c, (xp, _) in zip(cases, bufs):
+            dev.upload(xp, c.x)
+        items = [(w, xp, yp, c.M) for w, c, (xp, yp) in zip(ws, cases, bufs)]
+        req.infer_grouped_device(items)
+        req.sync()
+        info = req.last_kernel()
+        rl2 = mab = 0.0
+        for c, (_, yp) in zip(cases, bufs):
+            y = dev.download(yp, (c.M, c.N), np.float16).astype(np.float32)
+            pick = np.array([0, c.M // 2, c.M - 1])
+            ref = oracle.fc_reference(c.x[pick], c.w, type_tag[c.w_type], c.scale, c.zp, type_tag[c.zp_type], None,
+                                      N=c.N, K=c.K, group_size=c.group_size)
+            rl2, mab = max(rl2, oracle.rel_l2(y[pick], ref)), max(mab, oracle.max_abs(y[pick], ref))
+        us = min(req.bench_grouped(items, 3, 20) for _ in range(2)) / 20 * 1e3
+        t_grouped += us
+        nbytes = sum(algorithmic_bytes(c.K, c.N, c.M, 4, c.group_size, 0.5) for c in cases)
+        gbs, tfs = nbytes / us / 1e3, sum(2.0 * c.M * c.N * c.K for c in cases) / us / 1e6
+        rows.append(f"| 5 | {label} {cases[0].K}->{cases[0].N} | {'+'.join(str(len(t)) for t in routes)} | u4 g128 asym | "
+                    f"{info['name']} | {us:.1f} | {gbs:.0f} ({100 * gbs / HBM_PEAK_GBS:.1f} %) | "
+                    f"{tfs:.1f} ({100 * tfs / 1000 / 2.5:.1f} %) | {rl2:.1e} | {mab:.1e} |")
+        log(rows[-1])
+        for w in ws:
+            w.close()
+        for xp, yp in bufs:
+            dev.free(xp)
+            dev.free(yp)
+    grouped_line = (f"config 5 as 2 grouped runs: {t_grouped:.1f} us in total, "
+                    f"{flops_total / t_grouped / 1e6:.1f} TFLOP/s")
+    log(grouped_line)
     print("| Config | Shape (K->N) | M | dtype | GPU kernel | us | GB/s (% of 8 TB/s) | TFLOP/s (% of 2.5 PF) | "
           "rel-L2 vs fp32 | max-abs |")
     print("|---|---|---|---|---|---|---|---|---|---|")
     for r in rows:
         print(r)
     print(f"\nconfig 5 as 24 separate launches: {t_total:.1f} us in total, {flops_total / t_total / 1e6:.1f} TFLOP/s")
+    print(grouped_line)
     req.close()
     dev.close()
     return 0

@@ -142,6 +142,28 @@ int ovfcc_fc_run(ovfcc_request* req, const ovfcc_weights* w, const void* x_host,
  * stream and returns without waiting. */
 int ovfcc_fc_run_device(ovfcc_request* req, const ovfcc_weights* w, const void* x_dev, void* y_dev, int64_t M);
 
+/* Several independent nodes of one shape and weight format in one launch: the experts of a
+ * mixture-of-experts layer, each with its own gathered rows.  Stands in for the grouped forms of the op,
+ * ov::op::internal::GatherMatmulCompressed (src/common/transformations/include/ov_ops/
+ * gather_matmul_compressed.hpp:17-33; shape contract src/common/transformations/src/ov_ops/gather_matmul.cpp:38-110:
+ * B = [n_experts, N, K], one row set per expert) and GroupedMatMulCompressed
+ * (include/ov_ops/grouped_matmul_compressed.hpp), with the gather already done by the caller: item i multiplies its
+ * M_i rows x_dev [M_i, K] with its own weights into y_dev [M_i, N].  Device pointers, no copies, enqueued on the
+ * request's stream.  Items with M = 0 are skipped; items that differ in shape or format, untiled nodes and small
+ * nodes with few rows run one by one, with the same results. */
+typedef struct ovfcc_group_item {
+    const ovfcc_weights* weights;
+    const void* x_dev;
+    void* y_dev;
+    int64_t M;
+} ovfcc_group_item;
+int ovfcc_fc_run_grouped_device(ovfcc_request* req, const ovfcc_group_item* items, int n_items);
+
+/* Benchmark twin of ovfcc_bench_layers for grouped runs: `iters` eager calls of ovfcc_fc_run_grouped_device on the
+ * request's stream, bracketed by HIP events on that stream. */
+int ovfcc_bench_grouped(ovfcc_request* req, const ovfcc_group_item* items, int n_items, int warmup, int iters,
+                        float* elapsed_ms);
+
 /* Wait for everything enqueued on the request (IAsyncInferRequest::wait). */
 int ovfcc_request_sync(ovfcc_request* req);
 

@@ -16,12 +16,18 @@ KERNEL_AUTO, KERNEL_PLAIN, KERNEL_DECODE, KERNEL_PREFILL = range(4)
 SYMBOLS = [
     "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_destroy",
     "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
-    "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_request_sync", "ovfcc_request_force_kernel",
+    "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_grouped_device", "ovfcc_bench_grouped", "ovfcc_request_sync", "ovfcc_request_force_kernel",
     "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
     "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_bench_copy", "ovfcc_desc_validate", "ovfcc_tiled_sizes",
     "ovfcc_repack_host", "ovfcc_unrepack_host", "ovfcc_unpack_u4", "ovfcc_unpack_i4", "ovfcc_last_error",
     "ovfcc_version",
 ]
+
+
+class GroupItem(ctypes.Structure):
+    """struct ovfcc_group_item"""
+    _fields_ = [("weights", ctypes.c_void_p), ("x_dev", ctypes.c_void_p), ("y_dev", ctypes.c_void_p),
+                ("M", ctypes.c_int64)]
 
 
 class FcDesc(ctypes.Structure):
@@ -75,6 +81,8 @@ def load() -> ctypes.CDLL:
         "ovfcc_request_destroy": (None, [vp]),
         "ovfcc_fc_run": (ci, [vp, vp, vp, vp, i64]),
         "ovfcc_fc_run_device": (ci, [vp, vp, vp, vp, i64]),
+        "ovfcc_fc_run_grouped_device": (ci, [vp, ctypes.POINTER(GroupItem), ci]),
+        "ovfcc_bench_grouped": (ci, [vp, ctypes.POINTER(GroupItem), ci, ci, ci, ctypes.POINTER(ctypes.c_float)]),
         "ovfcc_request_sync": (ci, [vp]),
         "ovfcc_request_force_kernel": (ci, [vp, ci, ci]),
         "ovfcc_last_kernel_info": (ci, [vp, ctypes.POINTER(KernelInfo)]),

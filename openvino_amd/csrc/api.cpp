@@ -2,6 +2,7 @@
 // Every function returns an OVFCC_* code and records the reason with ovfcc::fail.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -470,6 +471,121 @@ int ovfcc_fc_run_device(ovfcc_request* r, const ovfcc_weights* w, const void* x_
     return enqueue(r, w, x_dev, y_dev, M);
 }
 
+int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items, int n_items) {
+    if (!r || (!items && n_items > 0) || n_items < 0)
+        return fail(OVFCC_EINVAL, "bad grouped-run arguments");
+    if (n_items == 0)
+        return OVFCC_OK;
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    const ovfcc_weights* w0 = items[0].weights;
+    if (!w0)
+        return fail(OVFCC_EINVAL, "an item has no weights");
+    bool same = true;
+    for (int i = 0; i < n_items && same; ++i) {
+        const ovfcc_weights* w = items[i].weights;
+        if (!w || w->ctx != r->ctx)
+            return fail(OVFCC_EINVAL, "an item's weights are null or belong to another context");
+        if (items[i].M < 0 || (items[i].M > 0 && (!items[i].x_dev || !items[i].y_dev)))
+            return fail(OVFCC_EINVAL, "an item has a negative row count or a null buffer");
+        same = std::memcmp(&w->desc, &w0->desc, sizeof(ovfcc_fc_desc)) == 0 && (w->d_bias != nullptr) == (w0->d_bias != nullptr);
+    }
+    // one launch needs a common shape and format, the tiled layout and no forced kernel; otherwise item by item
+    bool grouped = same && w0->layout.tiled && r->force_kernel == OVFCC_KERNEL_AUTO;
+    int64_t rows_max = 0;
+    for (int i = 0; i < n_items; ++i)
+        rows_max = std::max<int64_t>(rows_max, items[i].M);
+    if (rows_max == 0)
+        return OVFCC_OK;
+    // Few rows everywhere: the small-batch decode kernel; otherwise the prefill kernel, one 128-row tile per slice.
+    const bool decode = rows_max <= ovfcc::kDecodeMaxRows;
+    const int64_t rows_cap = decode ? ovfcc::kDecodeMaxRows : ovfcc::kPrefillGroupRows;
+    ovfcc::FcDeviceArgs a;
+    std::vector<ovfcc::BatchGroupItem> work;
+    if (grouped) {
+        // cut every item into equal slices of at most rows_cap rows
+        const size_t out_bytes = w0->desc.out_type == OVFCC_F32 ? 4 : 2;
+        rows_max = 0;
+        for (int i = 0; i < n_items; ++i) {
+            const int64_t M = items[i].M;
+            if (M == 0)
+                continue;
+            const int64_t slices = (M + rows_cap - 1) / rows_cap;
+            const int64_t step = (M + slices - 1) / slices;
+            const ovfcc_weights* w = items[i].weights;
+            for (int64_t m0 = 0; m0 < M; m0 += step) {
+                ovfcc::BatchGroupItem it{};
+                it.w = w->d_w, it.scale = w->d_scale, it.zp = w->d_zp, it.bias = w->d_bias;
+                it.x = static_cast<const char*>(items[i].x_dev) + (size_t)m0 * w->desc.K * 2;
+                it.y = static_cast<char*>(items[i].y_dev) + (size_t)m0 * w->desc.N * out_bytes;
+                it.M = (int)std::min(M - m0, step);
+                rows_max = std::max<int64_t>(rows_max, it.M);
+                work.push_back(it);
+            }
+        }
+    }
+    for (size_t first = 0; grouped && first < work.size(); first += ovfcc::kMaxGroupItems) {
+        const int n = (int)std::min<size_t>(ovfcc::kMaxGroupItems, work.size() - first);
+        ovfcc::BatchGroupTable tab{};
+        for (int i = 0; i < n; ++i)
+            tab.item[i] = work[first + i];
+        ovfcc::LaunchPlan p;
+        int rc;
+        if (decode) {
+            // planned for one slice; the other slices fill the chip, so K is split only as far as LDS demands
+            // unless the slices together still leave compute units idle
+            fill_args(w0, work[0].x, work[0].y, rows_max, &a);
+            int split = r->force_split;
+            if (split <= 0) {
+                const int64_t per_slice = (w0->layout.n_tiles + 7) / 8;
+                const int kb = (int)w0->layout.k_blocks;
+                split = 1;
+                while (per_slice * n * split < r->ctx->n_cus && split < 8 && kb / (split * 2) >= 2)
+                    split *= 2;
+            }
+            rc = ovfcc::plan_launch(a, OVFCC_KERNEL_DECODE, split, r->ctx->n_cus, &p);
+            grouped = !rc && p.batch && p.tiles_per_group == 1;  // small nodes with few rows plan the streaming kernel
+        } else {
+            // planned as one node whose 128-row tiles are the slices: tile counts and split-K come out right
+            fill_args(w0, work[0].x, work[0].y, (int64_t)n * ovfcc::kPrefillGroupRows, &a);
+            rc = ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, r->force_split, r->ctx->n_cus, &p);
+            grouped = !rc && p.async_dma && p.grid[1] == (unsigned)n;
+        }
+        if (!grouped) {
+            if (first != 0)
+                return fail(OVFCC_EUNSUPPORTED, "grouped launch plan changed between batches of slices");
+            break;
+        }
+        ovfcc::LaunchPlan all = p;  // split-K buffers for n slices
+        if (decode) {
+            all.workspace_bytes = p.workspace_bytes * n;
+            all.counter_count = p.counter_count * n;
+        }
+        rc = ensure_split_buffers(r, all);
+        if (rc)
+            return rc;
+        a.workspace = r->workspace;
+        a.counters = r->counters;
+        const int e = decode ? ovfcc::launch_batch_grouped(tab, n, a, p, r->stream)
+                             : ovfcc::launch_prefill_async_grouped(tab, n, a, p, r->stream);
+        if (e)
+            return hip_fail((hipError_t)e, "grouped kernel launch");
+        ovfcc::LaunchPlan shown = p;
+        if (decode)
+            shown.grid[2] = (unsigned)n;
+        shown.name = decode ? (w0->layout.bits == 4 ? "fcc_batch_grouped_w4" : "fcc_batch_grouped_w8")
+                            : "fcc_prefill_async_grouped_w4";
+        record(r, shown);
+    }
+    if (!grouped) {
+        for (int i = 0; i < n_items; ++i) {
+            int rc = enqueue(r, items[i].weights, items[i].x_dev, items[i].y_dev, items[i].M);
+            if (rc)
+                return rc;
+        }
+    }
+    return OVFCC_OK;
+}
+
 int ovfcc_request_sync(ovfcc_request* r) {
     if (!r)
         return fail(OVFCC_EINVAL, "request is null");
@@ -564,6 +680,31 @@ int ovfcc_bench_layers(ovfcc_request* r, const ovfcc_weights* const* layers, int
     if (t1) (void)hipEventDestroy(t1);
     if (exec) (void)hipGraphExecDestroy(exec);
     if (graph) (void)hipGraphDestroy(graph);
+    return rc;
+}
+
+int ovfcc_bench_grouped(ovfcc_request* r, const ovfcc_group_item* items, int n_items, int warmup, int iters,
+                        float* elapsed_ms) {
+    if (!r || !items || n_items <= 0 || !elapsed_ms || iters <= 0 || warmup < 0)
+        return fail(OVFCC_EINVAL, "bad benchmark arguments");
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    int rc = OVFCC_OK;
+    for (int i = 0; i < warmup + 1 && !rc; ++i)
+        rc = ovfcc_fc_run_grouped_device(r, items, n_items);
+    if (rc)
+        return rc;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    HIP_TRY(hipEventCreate(&t0));
+    HIP_TRY(hipEventCreate(&t1));
+    HIP_TRY(hipStreamSynchronize(r->stream));
+    HIP_TRY(hipEventRecord(t0, r->stream));
+    for (int i = 0; i < iters && !rc; ++i)
+        rc = ovfcc_fc_run_grouped_device(r, items, n_items);
+    HIP_TRY(hipEventRecord(t1, r->stream));
+    HIP_TRY(hipEventSynchronize(t1));
+    HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
     return rc;
 }
 

@@ -30,13 +30,12 @@ struct BatchSlot {
 };
 
 template <int BITS, int MT, bool ZP_TABLE, int RT>
-__global__ __launch_bounds__(512) void fcc_batch_kernel(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
-                                                        const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
-                                                        const half_t* __restrict__ bias, void* __restrict__ y,
-                                                        float* __restrict__ ws, unsigned* __restrict__ counters,
-                                                        int M, int N, int K, int kb_total, int kb_per_group, int ng,
-                                                        int zp_const, int kb_per_split, int split_k, int n_tiles,
-                                                        int out_f32) {
+__device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
+                                           const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
+                                           const half_t* __restrict__ bias, void* __restrict__ y,
+                                           float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N, int K,
+                                           int kb_total, int kb_per_group, int ng, int zp_const, int kb_per_split,
+                                           int split_k, int n_tiles, int out_f32) {
     constexpr int TPB = BITS == 4 ? 1 : 2;                    // tiles per k-block
     constexpr int DEPTH = (RT * TPB >= 4) ? 2 : 4 / TPB;      // k-blocks in flight per wave
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -268,6 +267,38 @@ __global__ __launch_bounds__(512) void fcc_batch_kernel(const uint4_t* __restric
     }
 }
 
+template <int BITS, int MT, bool ZP_TABLE, int RT>
+__global__ __launch_bounds__(512) void fcc_batch_kernel(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
+                                                        const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
+                                                        const half_t* __restrict__ bias, void* __restrict__ y,
+                                                        float* __restrict__ ws, unsigned* __restrict__ counters,
+                                                        int M, int N, int K, int kb_total, int kb_per_group, int ng,
+                                                        int zp_const, int kb_per_split, int split_k, int n_tiles,
+                                                        int out_f32) {
+    batch_body<BITS, MT, ZP_TABLE, RT>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
+                                       zp_const, kb_per_split, split_k, n_tiles, out_f32);
+}
+
+// Grouped launch: blockIdx.z picks one of up to kMaxGroupItems independent problems that share N, K and the weight
+// format (the experts of a mixture-of-experts layer, each with its own rows): one launch instead of one per expert.
+// The table travels in the kernel arguments; every problem has its own slice of the split-K workspace and counters.
+template <int BITS, int MT, bool ZP_TABLE, int RT>
+__global__ __launch_bounds__(512) void fcc_batch_grouped_kernel(BatchGroupTable tab, float* __restrict__ ws,
+                                                                unsigned* __restrict__ counters, size_t ws_per_item,
+                                                                int counters_per_item, int N, int K, int kb_total,
+                                                                int kb_per_group, int ng, int zp_const,
+                                                                int kb_per_split, int split_k, int n_tiles,
+                                                                int out_f32) {
+    const BatchGroupItem& it = tab.item[blockIdx.z];
+    if (it.M == 0)
+        return;
+    batch_body<BITS, MT, ZP_TABLE, RT>(static_cast<const uint4_t*>(it.w), static_cast<const half_t*>(it.scale),
+                                       static_cast<const uint8_t*>(it.zp), static_cast<const half_t*>(it.x),
+                                       static_cast<const half_t*>(it.bias), it.y, ws + blockIdx.z * ws_per_item,
+                                       counters + blockIdx.z * counters_per_item, it.M, N, K, kb_total, kb_per_group,
+                                       ng, zp_const, kb_per_split, split_k, n_tiles, out_f32);
+}
+
 template <int BITS, int MT, bool ZPT, int RT>
 static int launch_batch_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
@@ -299,6 +330,45 @@ static int launch_batch_bits(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
     if (mt == 2)
         return rt == 2 ? launch_batch_impl<BITS, 2, ZPT, 2>(a, p, s) : launch_batch_impl<BITS, 2, ZPT, 1>(a, p, s);
     return rt == 2 ? launch_batch_impl<BITS, 3, ZPT, 2>(a, p, s) : launch_batch_impl<BITS, 3, ZPT, 1>(a, p, s);
+}
+
+template <int BITS, int MT, bool ZPT>
+static int launch_grouped_impl(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
+                               hipStream_t s) {
+    const Layout& L = a.layout;
+    auto kern = fcc_batch_grouped_kernel<BITS, MT, ZPT, 1>;
+    if (p.dynamic_lds > 48 * 1024) {
+        static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+            if (e != hipSuccess)
+                return (int)e;
+            attr_set = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], (unsigned)n_items), dim3(p.block), p.dynamic_lds, s, tab,
+                       a.workspace, a.counters, p.workspace_bytes / sizeof(float), (int)p.counter_count, (int)a.N,
+                       (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups, L.zp_const,
+                       p.kblocks_per_split, p.split_k, (int)L.n_tiles, a.out_f32);
+    return (int)hipGetLastError();
+}
+
+// `a` describes the shared shape (M = the largest row count of any item, at most 48); `p` is its small-batch plan
+// with one channel tile per wave; workspace and counters hold n_items slices of p.workspace_bytes / p.counter_count.
+int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
+                         void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Layout& L = a.layout;
+    const int mt = (int)(a.M + 15) / 16;
+#define OVFCC_GROUPED(B, Z)                                                         \
+    (mt <= 1   ? launch_grouped_impl<B, 1, Z>(tab, n_items, a, p, s)                \
+     : mt == 2 ? launch_grouped_impl<B, 2, Z>(tab, n_items, a, p, s)                \
+               : launch_grouped_impl<B, 3, Z>(tab, n_items, a, p, s))
+    if (L.bits == 4)
+        return L.zp_table ? OVFCC_GROUPED(4, true) : OVFCC_GROUPED(4, false);
+    return L.zp_table ? OVFCC_GROUPED(8, true) : OVFCC_GROUPED(8, false);
+#undef OVFCC_GROUPED
 }
 
 int launch_batch(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {

@@ -50,16 +50,16 @@ constexpr int PA_W_OFF = PA_STAGES * PA_A_BYTES;
 constexpr int PA_P_OFF = PA_W_OFF + PA_STAGES * PA_W_BYTES;
 constexpr unsigned PA_LDS_BYTES = (unsigned)(PA_P_OFF + PA_STAGES * PA_P_BYTES);  // 147 KiB
 
+// The whole kernel for output tile (tile_x, tile_y) of one node; m0 is the tile's first row and tile_id its slot
+// in the split-K workspace.  The two kernels below differ only in where these come from.
 template <bool ZP_TABLE, bool PRESCALE>
-__global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* __restrict__ wt,
-                                                                const half_t* __restrict__ st,
-                                                                const uint8_t* __restrict__ zt,
-                                                                const half_t* __restrict__ x,
-                                                                const half_t* __restrict__ bias,
-                                                                void* __restrict__ y, float* __restrict__ ws,
-                                                                unsigned* __restrict__ counters, int M, int N, int K,
-                                                                int kb_total, int kb_per_group, int ng, int zp_const,
-                                                                int kb_per_split, int split_k, int out_f32) {
+__device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
+                                                   const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
+                                                   const half_t* __restrict__ bias, void* __restrict__ y,
+                                                   float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N,
+                                                   int K, int kb_total, int kb_per_group, int ng, int zp_const,
+                                                   int kb_per_split, int split_k, int out_f32, int tile_x, int m0,
+                                                   int tile_id) {
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
@@ -68,10 +68,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave & 3, kg = wave >> 2;
-    int tile_x, tile_y;
-    xcd_tile(tile_x, tile_y, 2 * PA_BM, PA_BN / 2);
     const int n0 = tile_x * PA_BN;
-    const int m0 = tile_y * PA_BM;
     const int col = lane & 15, kq = lane >> 4;
     // split-K: workgroup z contracts k-blocks [kb_lo, kb_hi); loads of k-blocks past kb_hi are sent out of range
     const int kb_lo = blockIdx.z * kb_per_split;
@@ -309,7 +306,6 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
     __syncthreads();
     float* ex = reinterpret_cast<float*>(lds_raw);  // [wn][2 x 8 x 4][64 lanes]
     __shared__ unsigned ticket_s;
-    const int tile_id = tile_y * gridDim.x + tile_x;
     // parked tile layout: [tile][split][wn][channel tile r][row tile t][lane] float4
     constexpr int kAuxDeviceScope = 16;              // sc1: write through to / read from memory shared by all XCDs
     constexpr unsigned kParkBytes = 4 * 32 * 64 * 16;  // one workgroup's f32 tile
@@ -414,22 +410,80 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
         __hip_atomic_store(counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+template <bool ZP_TABLE, bool PRESCALE>
+__global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* __restrict__ wt,
+                                                                const half_t* __restrict__ st,
+                                                                const uint8_t* __restrict__ zt,
+                                                                const half_t* __restrict__ x,
+                                                                const half_t* __restrict__ bias,
+                                                                void* __restrict__ y, float* __restrict__ ws,
+                                                                unsigned* __restrict__ counters, int M, int N, int K,
+                                                                int kb_total, int kb_per_group, int ng, int zp_const,
+                                                                int kb_per_split, int split_k, int out_f32) {
+    int tile_x, tile_y;
+    xcd_tile(tile_x, tile_y, 2 * PA_BM, PA_BN / 2);
+    prefill_async_body<ZP_TABLE, PRESCALE>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
+                                           zp_const, kb_per_split, split_k, out_f32, tile_x, tile_y * PA_BM,
+                                           tile_y * gridDim.x + tile_x);
+}
+
+// Grouped launch: grid row tile_y is item tile_y of the table, a node of the common shape and format with at most
+// 128 rows of its own (the experts of a mixture-of-experts layer over their gathered rows).  grid =
+// (N/256, items, split).  Workgroups of one item sit together in a super-tile and share its activations in L2.
+template <bool ZP_TABLE, bool PRESCALE>
+__global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const BatchGroupTable tab,
+                                                                        float* __restrict__ ws,
+                                                                        unsigned* __restrict__ counters, int N, int K,
+                                                                        int kb_total, int kb_per_group, int ng,
+                                                                        int zp_const, int kb_per_split, int split_k,
+                                                                        int out_f32) {
+    int tile_x, tile_y;
+    xcd_tile(tile_x, tile_y, 2 * PA_BM, PA_BN / 2);
+    const BatchGroupItem& it = tab.item[tile_y];
+    if (it.M <= 0)
+        return;
+    prefill_async_body<ZP_TABLE, PRESCALE>((const uint4_t*)it.w, (const half_t*)it.scale, (const uint8_t*)it.zp,
+                                           (const half_t*)it.x, (const half_t*)it.bias, it.y, ws, counters, it.M, N, K,
+                                           kb_total, kb_per_group, ng, zp_const, kb_per_split, split_k, out_f32, tile_x,
+                                           0, tile_y * gridDim.x + tile_x);
+}
+
+template <typename Kern>
+static int allow_lds(Kern kern, bool* done) {
+    if (*done)
+        return 0;  // the attribute is idempotent, a race only repeats it
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)PA_LDS_BYTES);
+    if (e == hipSuccess)
+        *done = true;
+    return (int)e;
+}
+
 template <bool ZPT, bool PRE>
 static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
     auto kern = fcc_prefill_async_kernel<ZPT, PRE>;
-    static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)PA_LDS_BYTES);
-        if (e != hipSuccess)
-            return (int)e;
-        attr_set = true;
-    }
+    static bool attr_set = false;  // per instantiation
+    if (int e = allow_lds(kern, &attr_set))
+        return e;
     hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), PA_LDS_BYTES, s, (const uint4_t*)a.w,
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
                        a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
                        (int)L.kblocks_per_group, (int)L.groups, L.zp_const, p.kblocks_per_split, p.split_k, a.out_f32);
+    return (int)hipGetLastError();
+}
+
+template <bool ZPT, bool PRE>
+static int launch_async_grouped_impl(const BatchGroupTable& tab, const FcDeviceArgs& a, const LaunchPlan& p,
+                                     hipStream_t s) {
+    const Layout& L = a.layout;
+    auto kern = fcc_prefill_async_grouped_kernel<ZPT, PRE>;
+    static bool attr_set = false;  // per instantiation
+    if (int e = allow_lds(kern, &attr_set))
+        return e;
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), PA_LDS_BYTES, s, tab, a.workspace,
+                       a.counters, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
+                       L.zp_const, p.kblocks_per_split, p.split_k, a.out_f32);
     return (int)hipGetLastError();
 }
 
@@ -441,6 +495,23 @@ int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& p, void* strea
     if (L.groups == 1)
         return L.zp_table ? launch_async_impl<true, false>(a, p, s) : launch_async_impl<false, false>(a, p, s);
     return L.zp_table ? launch_async_impl<true, true>(a, p, s) : launch_async_impl<false, true>(a, p, s);
+}
+
+// p plans one node of n_items * 128 rows: its grid rows are the items of the table.
+int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
+                                 void* stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const Layout& L = a.layout;
+    if (L.bits != 4 || n_items < 1 || n_items > kMaxGroupItems || p.grid[1] != (unsigned)n_items)
+        return (int)hipErrorInvalidValue;
+    for (int i = 0; i < n_items; ++i)
+        if (tab.item[i].M < 1 || tab.item[i].M > PA_BM)
+            return (int)hipErrorInvalidValue;
+    if (L.groups == 1)
+        return L.zp_table ? launch_async_grouped_impl<true, false>(tab, a, p, s)
+                          : launch_async_grouped_impl<false, false>(tab, a, p, s);
+    return L.zp_table ? launch_async_grouped_impl<true, true>(tab, a, p, s)
+                      : launch_async_grouped_impl<false, true>(tab, a, p, s);
 }
 
 }  // namespace ovfcc

@@ -97,6 +97,27 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_plain(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_decode(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_batch(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+
+// Problems of one grouped launch (passed in the kernel arguments: at most 4 KiB)
+constexpr int kMaxGroupItems = 64;
+struct BatchGroupItem {
+    const void* w;
+    const void* scale;
+    const void* zp;
+    const void* bias;
+    const void* x;
+    void* y;
+    int M;  // rows of this problem (0 = skip), at most kDecodeMaxRows (decode) or kPrefillGroupRows (prefill)
+    int reserved;
+};
+struct BatchGroupTable {
+    BatchGroupItem item[kMaxGroupItems];
+};
+int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& plan,
+                         void* stream);
+// Same table, items of at most 128 rows, 4-bit async prefill kernel; plan is that of one node of 128 * n_items rows.
+int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& plan,
+                                 void* stream);
 int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
@@ -105,6 +126,7 @@ int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
 int launch_touch(const void* src, size_t bytes, void* stream);
 
 constexpr int kDecodeMaxRows = 48;                       // rows one decode-family launch covers
+constexpr int kPrefillGroupRows = 128;                   // rows per slice of a grouped prefill launch (one tile)
 constexpr int kChunkedMaxRows = 128;                     // up to here M is cut into decode launches
 constexpr int kPrefillTileM = 128, kPrefillTileN = 128;  // square prefill kernel
 constexpr int kPrefillWideN = 256;                         // wide prefill kernel: 128 x 256

@@ -174,6 +174,50 @@ class InferRequest:
         check(self.device.lib.ovfcc_fc_run_device(self.handle, weights.handle, ctypes.c_void_p(x_ptr),
                                                   ctypes.c_void_p(y_ptr), M))
 
+    def _group_items(self, items):
+        arr = (_lib.GroupItem * len(items))()
+        for a, (w, x_ptr, y_ptr, M) in zip(arr, items):
+            a.weights, a.x_dev, a.y_dev, a.M = w.handle, x_ptr, y_ptr, M
+        return arr
+
+    def infer_grouped_device(self, items: Sequence[tuple]) -> None:
+        """items: (weights, x_ptr, y_ptr, M) per independent node of one shape and format (e.g. the experts of a
+        mixture-of-experts layer with their gathered rows); one launch where possible."""
+        arr = self._group_items(items)
+        check(self.device.lib.ovfcc_fc_run_grouped_device(self.handle, arr, len(items)))
+
+    def infer_grouped(self, items: Sequence[tuple]) -> list:
+        """items: (weights, X float16 [M_i, K] on the host) per node; returns the list of Y [M_i, N].  Stages the
+        operands in device memory, runs infer_grouped_device, copies back."""
+        dev, xs, ptrs = self.device, [], []
+        try:
+            for w, X in items:
+                X = np.ascontiguousarray(X, dtype=np.float16)
+                if X.ndim != 2 or X.shape[1] != w.K:
+                    raise OvfccError(_lib.EINVAL, f"X has shape {X.shape}, expected [M, {w.K}]")
+                xs.append(X)
+                itemsize = 4 if w.desc.out_type == _lib.F32 else 2
+                x_ptr, y_ptr = dev.malloc(max(X.nbytes, 16)), dev.malloc(max(X.shape[0] * w.N * itemsize, 16))
+                ptrs.append((x_ptr, y_ptr))
+                if X.size:
+                    dev.upload(x_ptr, X)
+            self.infer_grouped_device([(w, xp, yp, X.shape[0]) for (w, _), X, (xp, yp) in zip(items, xs, ptrs)])
+            self.sync()
+            return [dev.download(yp, (X.shape[0], w.N), np.float32 if w.desc.out_type == _lib.F32 else np.float16)
+                    if X.shape[0] else np.empty((0, w.N), np.float32 if w.desc.out_type == _lib.F32 else np.float16)
+                    for (w, _), X, (_, yp) in zip(items, xs, ptrs)]
+        finally:
+            for xp, yp in ptrs:
+                dev.free(xp)
+                dev.free(yp)
+
+    def bench_grouped(self, items: Sequence[tuple], warmup: int, iters: int) -> float:
+        """Milliseconds for `iters` grouped runs, HIP events on the launching stream."""
+        arr = self._group_items(items)
+        ms = ctypes.c_float()
+        check(self.device.lib.ovfcc_bench_grouped(self.handle, arr, len(items), warmup, iters, ctypes.byref(ms)))
+        return ms.value
+
     def sync(self) -> None:
         check(self.device.lib.ovfcc_request_sync(self.handle))
 

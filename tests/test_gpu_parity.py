@@ -344,3 +344,89 @@ def test_horizontal_fusion_matches_separate_nodes(oracle, dev, req):
         fused.close()
         for p in parts:
             p.close()
+
+
+GROUPED = [
+    # w_type, zp_type, N, K, G, bias, rows per item
+    ("u4", "u4", 256, 1024, 128, True, [5, 0, 48, 17, 1]),            # few rows everywhere: small-batch kernel
+    ("u8", "u8", 128, 512, 512, False, [3, 33, 16]),                  # 8-bit, per-channel
+    ("u4", "u4", 512, 1280, 128, False, [70, 3, 0, 129, 48, 300]),    # more rows: prefill kernel, slices of <= 128 rows
+    ("i4", "none", 256, 2048, 2048, True, [64, 65]),                  # per-channel scale in the epilogue
+    ("u4", "none", 256, 512, 128, False, [1] * 70 + [100]),           # more slices than one launch holds
+]
+
+
+@pytest.mark.parametrize("wt,zt,N,K,G,bias,rows", GROUPED)
+def test_grouped_run_matches_oracle_and_separate_runs(oracle, dev, req, monkeypatch, wt, zt, N, K, G, bias, rows):
+    """A grouped run over nodes of one shape (mixture-of-experts layers: one node per expert, its own weights and
+    gathered rows): every item meets the oracle bounds, and repeated runs give identical bits.  (The planner
+    would give grids this small to the square prefill kernel, which has no grouped form: the 256-wide one is
+    forced.)"""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    say(f"grouped {wt}/{zt} N={N} K={K} G={G} rows={rows[:8]}")
+    n_weights = min(len(rows), 6)
+    cases = [datagen.make_case(700 + i, max(rows), K, N, wt, G, zt, with_bias=bias) for i in range(n_weights)]
+    ws = [fc.CompressedWeights.from_case(dev, c) for c in cases]
+    try:
+        items = [(ws[i % n_weights], cases[i % n_weights].x[:m]) for i, m in enumerate(rows)]
+        ys = req.infer_grouped(items)
+        info = req.last_kernel()
+        assert "grouped" in info["name"], info
+        assert ("prefill" in info["name"]) == (max(rows) > 48), info
+        for i, (m, y) in enumerate(zip(rows, ys)):
+            assert y.shape == (m, N)
+            if m:
+                c = cases[i % n_weights]
+                check_parity(oracle, y, oracle_y(oracle, c, x=c.x[:m]), K, f"item {i} M={m} {info}",
+                             output_rounding_slack=True)
+        again = req.infer_grouped(items)
+        for y, z in zip(ys, again):
+            assert np.array_equal(y.view(np.uint16), z.view(np.uint16))
+    finally:
+        for w in ws:
+            w.close()
+
+
+def test_grouped_run_falls_back_item_by_item(oracle, dev, req):
+    """Items of different shapes, an untiled node, or a forced kernel cannot share a launch: the run still gives
+    every item's result (through the ordinary per-node path)."""
+    say("grouped fallback")
+    a = datagen.make_case(720, 20, 512, 128, "u4", 128, "u4")
+    b = datagen.make_case(721, 7, 256, 256, "u8", 128, "u8")
+    c = datagen.make_case(722, 9, 200, 40, "u4", 50, "u4")  # untiled
+    ws = [fc.CompressedWeights.from_case(dev, k) for k in (a, b, c)]
+    try:
+        ys = req.infer_grouped([(w, k.x) for w, k in zip(ws, (a, b, c))])
+        assert "grouped" not in req.last_kernel()["name"]
+        for y, k in zip(ys, (a, b, c)):
+            check_parity(oracle, y, oracle_y(oracle, k), k.K, "mixed", output_rounding_slack=True)
+        req.force_kernel(_lib.KERNEL_PREFILL)
+        y = req.infer_grouped([(ws[0], a.x), (ws[0], a.x[:3])])
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_PREFILL and "grouped" not in req.last_kernel()["name"]
+        check_parity(oracle, y[0], oracle_y(oracle, a), a.K, "forced", output_rounding_slack=True)
+        assert req.infer_grouped([]) == []
+        with pytest.raises(fc.OvfccError):
+            req.infer_grouped_device([(ws[0], 0, 0, 4)])
+    finally:
+        req.force_kernel()
+        for w in ws:
+            w.close()
+
+
+def test_grouped_run_mixtral_experts(oracle, dev, req):
+    """Benchmark configuration 5 at its real shape: the gate matrices of all eight experts over their routed
+    tokens in one launch, sampled rows against the oracle."""
+    say("grouped mixtral gate")
+    routes = datagen.moe_routing()
+    cases = [datagen.config5_expert(e, "gate", len(t)) for e, t in enumerate(routes)]
+    ws = [fc.CompressedWeights.from_case(dev, c) for c in cases]
+    try:
+        ys = req.infer_grouped([(w, c.x) for w, c in zip(ws, cases)])
+        info = req.last_kernel()
+        assert info["name"] == "fcc_prefill_async_grouped_w4", info
+        for e, (c, y) in enumerate(zip(cases, ys)):
+            pick = np.array([0, c.M // 2, c.M - 1])
+            check_parity(oracle, y[pick], oracle_y(oracle, c, x=c.x[pick]), c.K, f"expert {e}")
+    finally:
+        for w in ws:
+            w.close()
