@@ -57,8 +57,27 @@ typedef struct ovfcc_fc_desc {
     int32_t bias_type;  /* OVFCC_NONE | OVFCC_F16, [N] */
     int32_t act_type;   /* OVFCC_F16 */
     int32_t out_type;   /* OVFCC_F16 | OVFCC_F32 (FullyConnected's output_type; default = activation type) */
-    int32_t flags;      /* 0 */
+    int32_t flags;      /* 0, or a gated-linear-unit epilogue: OVFCC_GLU_* [| OVFCC_GLU_GATE_SECOND] */
 } ovfcc_fc_desc;
+
+/* Gated linear unit fused into the node (flags).  The reference fuses ov::op::internal::GLU
+ * (src/common/transformations/include/ov_ops/glu.hpp:16-40: axis = -1, split_lengths = N/2, glu_type,
+ * split_to_glu_idx) into the FullyConnected that produces its input when gate and up projection were fused
+ * horizontally (src/plugins/intel_gpu/src/kernel_selector/kernels/fully_connected/
+ * fully_connected_kernel_bf_tiled.cpp:223-236,661-666; epilogue cl_kernels/fully_connected_gpu_bf_tiled.cl:764-780;
+ * stand-alone formula cl_kernels/swiglu_gpu_ref.cl:66-85).  With Y = X W^T (+ bias) of shape [M, N], L = N / 2:
+ *     out[m, f] = act(Y[m, g + f]) * Y[m, u + f],  f in [0, L)
+ * where (g, u) = (0, L), or (L, 0) with OVFCC_GLU_GATE_SECOND (split_to_glu_idx = 1), and act is
+ * Swish x / (1 + exp(-x)), Gelu x (1 + erf(x / sqrt 2)) / 2 or Gelu_Tanh
+ * x (1 + tanh(sqrt(2 / pi) x (1 + 0.044715 x^2))) / 2, evaluated in f32 on the f32 sums.  The node's output is
+ * [M, L] in out_type; N, W, scales, zero-points and bias keep their [N, ...] shapes.  N must be even; the fast
+ * (tiled) kernels also need N % 32 == 0. */
+#define OVFCC_GLU_NONE 0
+#define OVFCC_GLU_SWISH 1
+#define OVFCC_GLU_GELU 2
+#define OVFCC_GLU_GELU_TANH 3
+#define OVFCC_GLU_TYPE_MASK 3
+#define OVFCC_GLU_GATE_SECOND 4
 
 typedef struct ovfcc_ctx ovfcc_ctx;         /* one device + its kernels */
 typedef struct ovfcc_weights ovfcc_weights; /* repacked, device-resident W/S/ZP/bias of one node */
@@ -117,6 +136,11 @@ int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out);
  * equal K, group size, weight type, zero-point kind, bias presence and output type; the copy is made on the
  * device and the parts stay valid. */
 int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_weights** out);
+/* Gate and up projection of a gated linear unit as one node: out[m, f] = act(gate(x)[m, f]) * up(x)[m, f]
+ * (see OVFCC_GLU_*; gate first).  The device-side counterpart of creating the node from concatenated constants
+ * with desc.flags = glu_type: both parts must be tiled nodes equal in shape, types, bias presence and output type;
+ * they stay valid.  The result reports N = 2 * N_part and produces [M, N_part]. */
+int ovfcc_weights_glu(const ovfcc_weights* gate, const ovfcc_weights* up, int glu_type, ovfcc_weights** out);
 /* device bytes held by the repacked node */
 int64_t ovfcc_weights_device_bytes(const ovfcc_weights* w);
 /* 1 when the node uses the tiled layout (fast kernels), 0 for the OpenVINO-layout fallback */

@@ -11,10 +11,12 @@ OK, EINVAL, EUNSUPPORTED, EDEVICE, ENOMEM = 0, -1, -2, -3, -4
 NONE, U4, I4, U8, I8, F16, F32 = range(7)
 TYPE = {"none": NONE, "u4": U4, "i4": I4, "u8": U8, "i8": I8, "f16": F16, "f32": F32}
 KERNEL_AUTO, KERNEL_PLAIN, KERNEL_DECODE, KERNEL_PREFILL = range(4)
+GLU = {None: 0, "none": 0, "swish": 1, "gelu": 2, "gelu_tanh": 3}      # OVFCC_GLU_*
+GLU_GATE_SECOND = 4
 
 # every symbol include/ovfcc.h declares
 SYMBOLS = [
-    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_destroy",
+    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_glu", "ovfcc_weights_destroy",
     "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
     "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_grouped_device", "ovfcc_bench_grouped", "ovfcc_request_sync", "ovfcc_request_force_kernel",
     "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
@@ -74,6 +76,7 @@ def load() -> ctypes.CDLL:
         "ovfcc_weights_create": (ci, [vp, ctypes.POINTER(FcDesc), vp, vp, vp, vp, pp]),
         "ovfcc_weights_clone": (ci, [vp, pp]),
         "ovfcc_weights_concat": (ci, [pp, ci, pp]),
+        "ovfcc_weights_glu": (ci, [vp, vp, ci, pp]),
         "ovfcc_weights_destroy": (None, [vp]),
         "ovfcc_weights_device_bytes": (i64, [vp]),
         "ovfcc_weights_is_tiled": (ci, [vp]),

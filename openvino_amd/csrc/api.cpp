@@ -93,6 +93,11 @@ int ensure_split_buffers(ovfcc_request* r, const ovfcc::LaunchPlan& plan) {
     return OVFCC_OK;
 }
 
+// row length of the node's output
+int64_t out_channels(const ovfcc_weights* w) {
+    return w->layout.glu ? w->desc.N / 2 : w->desc.N;
+}
+
 void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc::FcDeviceArgs* a) {
     a->w = w->d_w;
     a->scale = w->d_scale;
@@ -110,6 +115,9 @@ void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc:
     a->zp_type = w->desc.zp_type;
     a->zp_scalar = w->desc.zp_scalar;
     a->out_f32 = w->desc.out_type == OVFCC_F32 ? 1 : 0;
+    a->N_out = out_channels(w);
+    a->gate_offset = w->layout.glu_gate_second ? (int)(w->desc.N / 2) : 0;
+    a->up_offset = w->layout.glu_gate_second ? 0 : (int)(w->desc.N / 2);
     a->layout = w->layout;
 }
 
@@ -144,7 +152,7 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
         for (int64_t m0 = 0; m0 < M; m0 += step) {
             const int64_t rows = M - m0 < step ? M - m0 : step;
             fill_args(w, static_cast<const char*>(x) + (size_t)m0 * w->desc.K * 2,
-                      static_cast<char*>(y) + (size_t)m0 * w->desc.N * (w->desc.out_type == OVFCC_F32 ? 4 : 2), rows, &a);
+                      static_cast<char*>(y) + (size_t)m0 * out_channels(w) * (w->desc.out_type == OVFCC_F32 ? 4 : 2), rows, &a);
             ovfcc::LaunchPlan p;
             int rc = ovfcc::plan_launch(a, OVFCC_KERNEL_DECODE, r->force_split, r->ctx->n_cus, &p);
             if (rc)
@@ -274,8 +282,18 @@ int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* 
             rc = upload(&W->d_zp, zp, desc->zp_type == OVFCC_U4 ? (cnt + 1) / 2 : cnt);
         }
     }
-    if (!rc && desc->bias_type != OVFCC_NONE)
-        rc = upload(&W->d_bias, bias, (size_t)N * 2);
+    if (!rc && desc->bias_type != OVFCC_NONE) {
+        if (L.tiled && L.glu) {  // bias follows the channel order of the tiles
+            const uint16_t* b = static_cast<const uint16_t*>(bias);
+            std::vector<uint16_t> bt((size_t)N);
+            for (int64_t nt = 0; nt < L.n_tiles; ++nt)
+                std::memcpy(&bt[(size_t)nt * ovfcc::kTileRows], b + L.source_tile(nt) * ovfcc::kTileRows,
+                            ovfcc::kTileRows * 2);
+            rc = upload(&W->d_bias, bt.data(), (size_t)N * 2);
+        } else {
+            rc = upload(&W->d_bias, bias, (size_t)N * 2);
+        }
+    }
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;
@@ -353,6 +371,8 @@ int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_w
             return fail(OVFCC_EINVAL, "a part is null");
         if (!p->layout.tiled)
             return fail(OVFCC_EUNSUPPORTED, "only tiled nodes can be fused");
+        if (p->layout.glu)
+            return fail(OVFCC_EUNSUPPORTED, "a node with a gated-linear-unit epilogue cannot be a part");
         const bool same = p->ctx == first->ctx && p->desc.K == first->desc.K &&
                           p->desc.group_size == first->desc.group_size && p->desc.w_type == first->desc.w_type &&
                           p->desc.zp_type == first->desc.zp_type && p->desc.zp_scalar == first->desc.zp_scalar &&
@@ -393,6 +413,55 @@ int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_w
     if (!rc && W->desc.bias_type != OVFCC_NONE)
         rc = gather(&W->d_bias, (size_t)n_total * 2, &ovfcc_weights::d_bias,
                     [](const ovfcc_weights* p) { return (size_t)p->desc.N * 2; });
+    if (rc) {
+        ovfcc_weights_destroy(W);
+        return rc;
+    }
+    *out = W;
+    return OVFCC_OK;
+}
+
+int ovfcc_weights_glu(const ovfcc_weights* gate, const ovfcc_weights* up, int glu_type, ovfcc_weights** out) {
+    if (!gate || !up || !out)
+        return fail(OVFCC_EINVAL, "null argument");
+    *out = nullptr;
+    if (glu_type != OVFCC_GLU_SWISH && glu_type != OVFCC_GLU_GELU && glu_type != OVFCC_GLU_GELU_TANH)
+        return fail(OVFCC_EINVAL, "unknown gated-linear-unit type");
+    if (!gate->layout.tiled || !up->layout.tiled)
+        return fail(OVFCC_EUNSUPPORTED, "only tiled nodes can be fused");
+    if (gate->layout.glu || up->layout.glu)
+        return fail(OVFCC_EUNSUPPORTED, "a node with a gated-linear-unit epilogue cannot be a part");
+    ovfcc_fc_desc want = gate->desc;
+    if (std::memcmp(&want, &up->desc, sizeof(want)) != 0 || gate->ctx != up->ctx ||
+        gate->layout.zp_const != up->layout.zp_const)
+        return fail(OVFCC_EUNSUPPORTED, "gate and up projection differ in shape, types, bias or output type");
+    HIP_TRY(hipSetDevice(gate->ctx->device));
+    ovfcc_weights* W = new ovfcc_weights();
+    W->ctx = gate->ctx;
+    W->desc = gate->desc;
+    W->desc.N = 2 * gate->desc.N;
+    W->desc.flags = glu_type;
+    W->layout = ovfcc::make_layout(W->desc);
+    W->layout.zp_const = gate->layout.zp_const;
+    const ovfcc::Layout& L = W->layout;
+    const size_t tiles = (size_t)gate->layout.n_tiles;
+    // rows of one tile in each array; gate tiles land on even rows of the fused arrays, up tiles on odd rows
+    auto weave = [&](void** dst, const void* g, const void* u, size_t row) -> int {
+        if (!g || row == 0)
+            return OVFCC_OK;
+        HIP_TRY(hipMalloc(dst, 2 * tiles * row));
+        W->bytes += 2 * tiles * row;
+        HIP_TRY(hipMemcpy2D(*dst, 2 * row, g, row, row, tiles, hipMemcpyDeviceToDevice));
+        HIP_TRY(hipMemcpy2D(static_cast<char*>(*dst) + row, 2 * row, u, row, row, tiles, hipMemcpyDeviceToDevice));
+        return OVFCC_OK;
+    };
+    int rc = weave(&W->d_w, gate->d_w, up->d_w, gate->layout.w_bytes / tiles);
+    if (!rc)
+        rc = weave(&W->d_scale, gate->d_scale, up->d_scale, gate->layout.scale_bytes / tiles);
+    if (!rc && L.zp_table)
+        rc = weave(&W->d_zp, gate->d_zp, up->d_zp, gate->layout.zp_bytes / tiles);
+    if (!rc && W->desc.bias_type != OVFCC_NONE)
+        rc = weave(&W->d_bias, gate->d_bias, up->d_bias, (size_t)ovfcc::kTileRows * 2);
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;
@@ -516,7 +585,7 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
                 ovfcc::BatchGroupItem it{};
                 it.w = w->d_w, it.scale = w->d_scale, it.zp = w->d_zp, it.bias = w->d_bias;
                 it.x = static_cast<const char*>(items[i].x_dev) + (size_t)m0 * w->desc.K * 2;
-                it.y = static_cast<char*>(items[i].y_dev) + (size_t)m0 * w->desc.N * out_bytes;
+                it.y = static_cast<char*>(items[i].y_dev) + (size_t)m0 * out_channels(w) * out_bytes;
                 it.M = (int)std::min(M - m0, step);
                 rows_max = std::max<int64_t>(rows_max, it.M);
                 work.push_back(it);
@@ -548,7 +617,7 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
             // planned as one node whose 128-row tiles are the slices: tile counts and split-K come out right
             fill_args(w0, work[0].x, work[0].y, (int64_t)n * ovfcc::kPrefillGroupRows, &a);
             rc = ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, r->force_split, r->ctx->n_cus, &p);
-            grouped = !rc && p.async_dma && p.grid[1] == (unsigned)n;
+            grouped = !rc && p.async_dma && p.tiles_y == n;
         }
         if (!grouped) {
             if (first != 0)
@@ -604,7 +673,7 @@ int ovfcc_fc_run(ovfcc_request* r, const ovfcc_weights* w, const void* x_host, v
         return fail(OVFCC_EINVAL, "x or y is null");
     HIP_TRY(hipSetDevice(r->ctx->device));
     const size_t xb = (size_t)M * w->desc.K * 2;
-    const size_t yb = (size_t)M * w->desc.N * (w->desc.out_type == OVFCC_F32 ? 4 : 2);
+    const size_t yb = (size_t)M * out_channels(w) * (w->desc.out_type == OVFCC_F32 ? 4 : 2);
     if (xb > r->x_cap || yb > r->y_cap)
         HIP_TRY(hipStreamSynchronize(r->stream));
     int rc = grow(&r->d_x, &r->x_cap, xb);

@@ -94,11 +94,12 @@ __device__ __forceinline__ void unpack8_biased(uint32_t w0, uint32_t w1, Frag8& 
 // fetches, row_cost and col_cost being the relative sizes of one tile's activation and weight strips.
 // Blocks are dealt to the XCDs round-robin; when the number of blocks is no multiple of eight, the blocks
 // of the last, partial round are cut into equal runs of tiles, one run per XCD.
-__device__ __forceinline__ void xcd_tile(int& tile_x, int& tile_y, unsigned row_cost, unsigned col_cost) {
-    const unsigned gx = gridDim.x, gy = gridDim.y, total = gx * gy;
-    const unsigned linear = blockIdx.y * gx + blockIdx.x;
-    tile_x = (int)blockIdx.x;
-    tile_y = (int)blockIdx.y;
+// xcd_tile_at: the tile of position `linear` (< gx gy) in that order, for a gx x gy tile grid.
+__device__ __forceinline__ void xcd_tile_at(unsigned linear, unsigned gx, unsigned gy, int& tile_x, int& tile_y,
+                                            unsigned row_cost, unsigned col_cost) {
+    const unsigned total = gx * gy;
+    tile_x = (int)(linear % gx);
+    tile_y = (int)(linear / gx);
     if (total & 7u)
         return;
     unsigned best_sn = 0, best_sm = 0;
@@ -132,6 +133,30 @@ __device__ __forceinline__ void xcd_tile(int& tile_x, int& tile_y, unsigned row_
     const unsigned supers_x = gx / sn;
     tile_x = (int)((super % supers_x) * sn + within % sn);
     tile_y = (int)((super / supers_x) * sm + within / sn);
+}
+
+// The launch's own 2-D grid as the tile grid.
+__device__ __forceinline__ void xcd_tile(int& tile_x, int& tile_y, unsigned row_cost, unsigned col_cost) {
+    xcd_tile_at(blockIdx.y * gridDim.x + blockIdx.x, gridDim.x, gridDim.y, tile_x, tile_y, row_cost, col_cost);
+}
+
+// Gated-linear-unit epilogue on f32 values: act(gate) * up with act = Swish (1), Gelu (2), Gelu_Tanh (3), the
+// formulas of the OpenVINO Intel-GPU plugin (cl_kernels/swiglu_gpu_ref.cl:74-85, swish beta = 1).  Exponential
+// and reciprocal are the hardware's (about 1e-6 relative, far inside the f16 result): the epilogue of a prefill
+// tile runs with the matrix cores idle, so its length is paid in full.  Both saturate correctly:
+// exp -> inf gives 1 / inf = 0, exp -> 0 gives 1.
+__device__ __forceinline__ float glu_value(int type, float gate, float up) {
+    float a;
+    if (type == 1) {
+        a = gate * __builtin_amdgcn_rcpf(1.f + __expf(-gate));
+    } else if (type == 2) {
+        a = 0.5f * gate * (1.f + erff(gate * 0.70710678118654752440f));
+    } else {
+        // tanh z = 1 - 2 / (1 + exp 2 z)
+        const float z = 0.79788456080286535588f * gate * (1.f + 0.044715f * gate * gate);
+        a = gate * (1.f - __builtin_amdgcn_rcpf(1.f + __expf(2.f * z)));
+    }
+    return a * up;
 }
 
 // Output cast: FullyConnected's output_type is f16 (default, the activation type) or f32.

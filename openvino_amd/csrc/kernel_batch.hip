@@ -35,7 +35,7 @@ __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const
                                            const half_t* __restrict__ bias, void* __restrict__ y,
                                            float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N, int K,
                                            int kb_total, int kb_per_group, int ng, int zp_const, int kb_per_split,
-                                           int split_k, int n_tiles, int out_f32) {
+                                           int split_k, int n_tiles, int out_f32, int glu) {
     constexpr int TPB = BITS == 4 ? 1 : 2;                    // tiles per k-block
     constexpr int DEPTH = (RT * TPB >= 4) ? 2 : 4 / TPB;      // k-blocks in flight per wave
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -250,6 +250,54 @@ __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const
             __hip_atomic_store(counters + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
+    if (glu) {
+        // gated linear unit: the wave's two tiles are the gate and up channels 16 (tile0 / 2) .. of the
+        // [M, N / 2] output
+        if constexpr (RT == 1) {
+            // one tile per wave: even waves own gate tiles, the next wave the matching up tile, handed over
+            // through LDS (the staged activations are no longer needed once every wave is here)
+            float* hand = reinterpret_cast<float*>(lds);  // [nw / 2][MT][4][64 lanes]
+            const int n = tile0 * 16 + col;
+            const float b = bias && tiles_here ? (float)bias[n] : 0.f;
+            __syncthreads();
+            if (wave & 1) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        hand[(((wave >> 1) * MT + t) * 4 + q) * 64 + lane] = sum[0][t][q] + b;
+            }
+            __syncthreads();
+            if (!(wave & 1) && tiles_here) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int m = 4 * kq + q + 16 * t;
+                        if (m < M)
+                            store_out(y, (size_t)m * (N / 2) + (tile0 >> 1) * 16 + col,
+                                      glu_value(glu, sum[0][t][q] + b,
+                                                hand[(((wave >> 1) * MT + t) * 4 + q) * 64 + lane]),
+                                      out_f32);
+                    }
+            }
+        } else {
+            if (tiles_here == 2) {
+                const int n = tile0 * 16 + col;
+                const float bg = bias ? (float)bias[n] : 0.f, bu = bias ? (float)bias[n + 16] : 0.f;
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int m = 4 * kq + q + 16 * t;
+                        if (m < M)
+                            store_out(y, (size_t)m * (N / 2) + (tile0 >> 1) * 16 + col,
+                                      glu_value(glu, sum[0][t][q] + bg, sum[1][t][q] + bu), out_f32);
+                    }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
         if (r >= tiles_here)
@@ -274,9 +322,9 @@ __global__ __launch_bounds__(512) void fcc_batch_kernel(const uint4_t* __restric
                                                         float* __restrict__ ws, unsigned* __restrict__ counters,
                                                         int M, int N, int K, int kb_total, int kb_per_group, int ng,
                                                         int zp_const, int kb_per_split, int split_k, int n_tiles,
-                                                        int out_f32) {
+                                                        int out_f32, int glu) {
     batch_body<BITS, MT, ZP_TABLE, RT>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
-                                       zp_const, kb_per_split, split_k, n_tiles, out_f32);
+                                       zp_const, kb_per_split, split_k, n_tiles, out_f32, glu);
 }
 
 // Grouped launch: blockIdx.z picks one of up to kMaxGroupItems independent problems that share N, K and the weight
@@ -296,7 +344,7 @@ __global__ __launch_bounds__(512) void fcc_batch_grouped_kernel(BatchGroupTable 
                                        static_cast<const uint8_t*>(it.zp), static_cast<const half_t*>(it.x),
                                        static_cast<const half_t*>(it.bias), it.y, ws + blockIdx.z * ws_per_item,
                                        counters + blockIdx.z * counters_per_item, it.M, N, K, kb_total, kb_per_group,
-                                       ng, zp_const, kb_per_split, split_k, n_tiles, out_f32);
+                                       ng, zp_const, kb_per_split, split_k, n_tiles, out_f32, 0);
 }
 
 template <int BITS, int MT, bool ZPT, int RT>
@@ -317,7 +365,7 @@ static int launch_batch_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
                        a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
                        (int)L.kblocks_per_group, (int)L.groups, L.zp_const, p.kblocks_per_split, p.split_k,
-                       (int)L.n_tiles, a.out_f32);
+                       (int)L.n_tiles, a.out_f32, L.glu);
     return (int)hipGetLastError();
 }
 
@@ -360,6 +408,8 @@ int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDevice
                          void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
+    if (L.glu || p.tiles_per_group != 1)
+        return (int)hipErrorInvalidValue;  // the grouped kernel is built for one tile per wave
     const int mt = (int)(a.M + 15) / 16;
 #define OVFCC_GROUPED(B, Z)                                                         \
     (mt <= 1   ? launch_grouped_impl<B, 1, Z>(tab, n_items, a, p, s)                \
@@ -374,6 +424,8 @@ int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDevice
 int launch_batch(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
+    if (L.glu && ((p.tiles_per_group == 1 && ((p.block >> 6) & 1)) || p.dynamic_lds < (p.block >> 7) * (unsigned)p.tile_m * 64u))
+        return (int)hipErrorInvalidValue;  // gate and up tile: one wave, or two neighbours with room for the hand-over
     if (L.bits == 4)
         return L.zp_table ? launch_batch_bits<4, true>(a, p, s) : launch_batch_bits<4, false>(a, p, s);
     return L.zp_table ? launch_batch_bits<8, true>(a, p, s) : launch_batch_bits<8, false>(a, p, s);

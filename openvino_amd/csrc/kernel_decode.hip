@@ -45,7 +45,7 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
                                                           float* __restrict__ ws, unsigned* __restrict__ counters,
                                                           int M, int N, int K, int kb_total, int kb_per_group,
                                                           int ng, int zp_const, int kb_per_split, int split_k,
-                                                          int out_f32) {
+                                                          int out_f32, int glu) {
     static_assert(!XLDS || MT == 1, "LDS-staged activations serve one 16-row tile");
     constexpr int TPB = BITS == 4 ? 1 : 2;                                            // tiles per k-block
     constexpr int DEPTH = XLDS ? (RT * TPB >= 4 ? 2 : 4) : (MT == 1 ? 4 : 2) / TPB;  // k-blocks in flight
@@ -301,6 +301,26 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
             __hip_atomic_store(counters + grp, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
+    if (glu) {
+        // gated linear unit: tiles 2 j and 2 j + 1 are the gate and up channels 16 j .. of the [M, N / 2] output
+        if constexpr (RT % 2 == 0) {
+#pragma unroll
+            for (int r = 0; r < RT; r += 2) {
+                const int n = (grp * RT + r) * 16 + col;
+                const float bg = bias ? (float)bias[n] : 0.f, bu = bias ? (float)bias[n + 16] : 0.f;
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int m = 4 * kq + q + 16 * t;
+                        if (m < M)
+                            store_out(y, (size_t)m * (N / 2) + (n >> 5) * 16 + col,
+                                      glu_value(glu, sum[r][t][q] + bg, sum[r + 1][t][q] + bu), out_f32);
+                    }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
         const int n = (grp * RT + r) * 16 + col;
@@ -323,7 +343,7 @@ static void launch_decode_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipSt
                        p.dynamic_lds, s, (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp,
                        (const half_t*)a.x, (const half_t*)a.bias, a.y, a.workspace, a.counters, (int)a.M, (int)a.N,
                        (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups, L.zp_const,
-                       p.kblocks_per_split, p.split_k, a.out_f32);
+                       p.kblocks_per_split, p.split_k, a.out_f32, L.glu);
 }
 
 template <int BITS, bool ZPT>
@@ -352,6 +372,8 @@ static void launch_decode_bits(const FcDeviceArgs& a, const LaunchPlan& p, hipSt
 int launch_decode(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
+    if (L.glu && (!p.x_in_lds || a.M > 16 || (p.tiles_per_group & 1)))
+        return (int)hipErrorInvalidValue;  // gate and up tile must share a workgroup
     if (L.bits == 4)
         L.zp_table ? launch_decode_bits<4, true>(a, p, s) : launch_decode_bits<4, false>(a, p, s);
     else

@@ -8,14 +8,9 @@ namespace ovfcc {
 // ------------------------------------------------------------------------------------------------
 // Plain kernel: OpenVINO layout, any N/K/G.  One wave per (n, m); lanes stride over k.
 // ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(64) void fcc_plain_kernel(const uint8_t* __restrict__ w, const half_t* __restrict__ s,
-                                                       const uint8_t* __restrict__ zp,
-                                                       const half_t* __restrict__ bias,
-                                                       const half_t* __restrict__ x, void* __restrict__ y, int M,
-                                                       int N, int K, int G, int w_type, int zp_type, int zp_scalar,
-                                                       int out_f32) {
-    const int n = blockIdx.x;
-    const int m = blockIdx.y;
+__device__ __forceinline__ float plain_dot(const uint8_t* __restrict__ w, const half_t* __restrict__ s,
+                                           const uint8_t* __restrict__ zp, const half_t* __restrict__ x, int n, int m,
+                                           int K, int G, int w_type, int zp_type, int zp_scalar) {
     const int lane = threadIdx.x;
     const int ng = K / G;
     float acc = 0.f;
@@ -49,11 +44,31 @@ __global__ __launch_bounds__(64) void fcc_plain_kernel(const uint8_t* __restrict
     }
     for (int off = 32; off > 0; off >>= 1)
         acc += __shfl_down(acc, off, 64);
-    if (lane == 0) {
+    return acc;  // lane 0 holds the sum
+}
+
+// grid = (output channels, M).  With a gated linear unit (glu != 0) output channel f is
+// act(channel gate_offset + f) * (channel up_offset + f) and N_out = N / 2.
+__global__ __launch_bounds__(64) void fcc_plain_kernel(const uint8_t* __restrict__ w, const half_t* __restrict__ s,
+                                                       const uint8_t* __restrict__ zp,
+                                                       const half_t* __restrict__ bias,
+                                                       const half_t* __restrict__ x, void* __restrict__ y, int M,
+                                                       int N_out, int K, int G, int w_type, int zp_type, int zp_scalar,
+                                                       int out_f32, int glu, int gate_offset, int up_offset) {
+    const int f = blockIdx.x;
+    const int m = blockIdx.y;
+    const int n = glu ? gate_offset + f : f;
+    float acc = plain_dot(w, s, zp, x, n, m, K, G, w_type, zp_type, zp_scalar);
+    if (bias)
+        acc += (float)bias[n];
+    if (glu) {
+        float up = plain_dot(w, s, zp, x, up_offset + f, m, K, G, w_type, zp_type, zp_scalar);
         if (bias)
-            acc += (float)bias[n];
-        store_out(y, (size_t)m * N + n, acc, out_f32);
+            up += (float)bias[up_offset + f];
+        acc = glu_value(glu, acc, up);
     }
+    if (threadIdx.x == 0)
+        store_out(y, (size_t)m * N_out + f, acc, out_f32);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -94,8 +109,8 @@ int launch_touch(const void* src, size_t bytes, void* stream) {
 int launch_plain(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipLaunchKernelGGL(fcc_plain_kernel, dim3(p.grid[0], p.grid[1], 1), dim3(64), 0, static_cast<hipStream_t>(stream),
                        (const uint8_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.bias,
-                       (const half_t*)a.x, a.y, (int)a.M, (int)a.N, (int)a.K, (int)a.group_size, a.w_type, a.zp_type,
-                       a.zp_scalar, a.out_f32);
+                       (const half_t*)a.x, a.y, (int)a.M, (int)a.N_out, (int)a.K, (int)a.group_size, a.w_type,
+                       a.zp_type, a.zp_scalar, a.out_f32, a.layout.glu, a.gate_offset, a.up_offset);
     return (int)hipGetLastError();
 }
 

@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
                                                           const half_t* __restrict__ x,
                                                           const half_t* __restrict__ bias, void* __restrict__ y,
                                                           int M, int N, int K, int kb_total, int kb_per_group, int ng,
-                                                          int zp_const, int out_f32) {
+                                                          int zp_const, int out_f32, int glu) {
     constexpr int TPB = BITS == 4 ? 1 : 2;
     __shared__ __attribute__((aligned(16))) half_t As[PF_BM * PF_LD];
     __shared__ __attribute__((aligned(16))) half_t Bs[PF_BN * PF_LD];
@@ -160,8 +160,15 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + 64 * wm + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m < M)
-                    store_out(y, (size_t)m * N + n, acc[i][j][r] * cs + b, out_f32);
+                const float v = acc[i][j][r] * cs + b;
+                if (glu) {
+                    // gated linear unit: the 32 channels are a gate tile (lanes & 16 == 0) and its up tile
+                    const float up = __shfl_xor(v, 16, 64);
+                    if (m < M && !(lane & 16))
+                        store_out(y, (size_t)m * (N / 2) + (n >> 5) * 16 + (lane & 15), glu_value(glu, v, up), out_f32);
+                } else if (m < M) {
+                    store_out(y, (size_t)m * N + n, v, out_f32);
+                }
             }
     }
 }
@@ -172,7 +179,7 @@ static void launch_prefill_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipS
     hipLaunchKernelGGL((fcc_prefill_kernel<BITS, ZPT, PRE>), dim3(p.grid[0], p.grid[1], 1), dim3(256), 0, s,
                        (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x,
                        (const half_t*)a.bias, a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
-                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32);
+                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32, L.glu);
 }
 
 // Grouped scales are folded into the f16 weights in LDS; a single group per channel (G == K) keeps the

@@ -50,16 +50,44 @@ constexpr int PA_W_OFF = PA_STAGES * PA_A_BYTES;
 constexpr int PA_P_OFF = PA_W_OFF + PA_STAGES * PA_W_BYTES;
 constexpr unsigned PA_LDS_BYTES = (unsigned)(PA_P_OFF + PA_STAGES * PA_P_BYTES);  // 147 KiB
 
-// The whole kernel for output tile (tile_x, tile_y) of one node; m0 is the tile's first row and tile_id its slot
-// in the split-K workspace.  The two kernels below differ only in where these come from.
+// What one workgroup does: k-blocks [kb_lo, kb_hi) of the output tile at column block tile_x and rows m0.. of its
+// node, as part z of split_k parts of that tile (split_k == 1: the whole tile), parked in workspace slot park_slot.
+struct AsyncWork {
+    int tile_x, tile_y, m0, z, split_k, kb_lo, kb_hi, park_slot;
+};
+
+// Work of workgroup blockIdx.x for a tiles_x x tiles_y tile grid (1-D launch).  The first full_tiles workgroups
+// take one whole tile each, in the XCD-aware order of xcd_tile_at; the remaining tiles are cut into tail_split
+// parts along K, part by part (all first parts, then all second parts, ...), so that a launch whose tile count
+// is a little more than a multiple of the compute units ends with a full round of shorter workgroups instead
+// of a mostly idle round of whole tiles.  full_tiles = 0 splits every tile (few tiles, long K).
+__device__ __forceinline__ AsyncWork async_work(int tiles_x, int tiles_y, int full_tiles, int tail_split,
+                                                int kb_per_split, int kb_total) {
+    AsyncWork wk;
+    const int L = (int)blockIdx.x;
+    int slot;
+    if (L < full_tiles) {
+        slot = L, wk.z = 0, wk.split_k = 1, wk.kb_lo = 0, wk.kb_hi = kb_total, wk.park_slot = 0;
+    } else {
+        const int tail = tiles_x * tiles_y - full_tiles, j = L - full_tiles;
+        wk.z = j / tail, slot = full_tiles + j % tail, wk.split_k = tail_split;
+        wk.kb_lo = wk.z * kb_per_split, wk.kb_hi = min(kb_total, wk.kb_lo + kb_per_split);
+        wk.park_slot = j % tail;
+    }
+    xcd_tile_at((unsigned)slot, (unsigned)tiles_x, (unsigned)tiles_y, wk.tile_x, wk.tile_y, 2 * PA_BM, PA_BN / 2);
+    wk.m0 = wk.tile_y * PA_BM;
+    return wk;
+}
+
+// The whole kernel for one workgroup's share of one node.  The two kernels below differ only in where the node's
+// operands come from.
 template <bool ZP_TABLE, bool PRESCALE>
 __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
                                                    const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
                                                    const half_t* __restrict__ bias, void* __restrict__ y,
                                                    float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N,
                                                    int K, int kb_total, int kb_per_group, int ng, int zp_const,
-                                                   int kb_per_split, int split_k, int out_f32, int tile_x, int m0,
-                                                   int tile_id) {
+                                                   int out_f32, int glu, const AsyncWork wk) {
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
@@ -68,11 +96,10 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave & 3, kg = wave >> 2;
-    const int n0 = tile_x * PA_BN;
+    const int n0 = wk.tile_x * PA_BN, m0 = wk.m0, tile_id = wk.park_slot, split_k = wk.split_k;
     const int col = lane & 15, kq = lane >> 4;
-    // split-K: workgroup z contracts k-blocks [kb_lo, kb_hi); loads of k-blocks past kb_hi are sent out of range
-    const int kb_lo = blockIdx.z * kb_per_split;
-    const int kb_hi = min(kb_total, kb_lo + kb_per_split);
+    // split-K: this workgroup contracts k-blocks [kb_lo, kb_hi); loads of k-blocks past kb_hi are sent out of range
+    const int kb_lo = wk.kb_lo, kb_hi = wk.kb_hi;
 
     constexpr unsigned kOob = 0x80000000u;
     constexpr int kRsrcFlags = 0x00020000;
@@ -324,6 +351,26 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             }
         }
     };
+    // gated linear unit: channel tiles 2 j and 2 j + 1 of the wave are gate and up of output channels
+    // (n0 + 64 wn) / 2 + 16 j .. of the [M, N / 2] result
+    auto finish_glu = [&](int j, int t, float4_t g, float4_t u, const float (&scg)[4], const float (&bsg)[4],
+                          const float (&scu)[4], const float (&bsu)[4]) {
+        const int n = (n0 + 64 * wn) / 2 + 16 * j + 4 * kq;
+        const int m = m0 + 16 * t + col;
+        const float o[4] = {glu_value(glu, g.x * scg[0] + bsg[0], u.x * scu[0] + bsu[0]),
+                            glu_value(glu, g.y * scg[1] + bsg[1], u.y * scu[1] + bsu[1]),
+                            glu_value(glu, g.z * scg[2] + bsg[2], u.z * scu[2] + bsu[2]),
+                            glu_value(glu, g.w * scg[3] + bsg[3], u.w * scu[3] + bsu[3])};
+        if (m < M) {
+            if (out_f32) {
+                *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * (N / 2) + n) =
+                    float4_t{o[0], o[1], o[2], o[3]};
+            } else {
+                *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * (N / 2) + n) =
+                    half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
+            }
+        }
+    };
     auto channel_params = [&](int r, float (&sc)[4], float (&bs)[4]) {
         const int n = n0 + 64 * wn + 16 * r + 4 * kq;
 #pragma unroll
@@ -355,7 +402,19 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                 }
         }
         __syncthreads();
-        if (kg == 0) {
+        if (kg == 0 && glu && split_k == 1) {
+            float scg[4], bsg[4], scu[4], bsu[4];
+            channel_params(2 * hh, scg, bsg);
+            channel_params(2 * hh + 1, scu, bsu);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const float* pg = ex + ((wn * 64 + t * 4) * 64) + lane;
+                const float* pu = ex + ((wn * 64 + (8 + t) * 4) * 64) + lane;
+                const float4_t a = acc[2 * hh][t], b = acc[2 * hh + 1][t];
+                finish_glu(hh, t, float4_t{a.x + pg[0], a.y + pg[64], a.z + pg[128], a.w + pg[192]},
+                           float4_t{b.x + pu[0], b.y + pu[64], b.z + pu[128], b.w + pu[192]}, scg, bsg, scu, bsu);
+            }
+        } else if (kg == 0) {
 #pragma unroll
             for (int r2 = 0; r2 < 2; ++r2) {
                 const int r = 2 * hh + r2;
@@ -371,7 +430,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                     else
                         __builtin_amdgcn_raw_buffer_store_b128(
                             __builtin_bit_cast(uint4_t, v), rp,
-                            blockIdx.z * kParkBytes + (unsigned)(((wn * 4 + r) * 8 + t) * 64 + lane) * 16u, 0,
+                            wk.z * kParkBytes + (unsigned)(((wn * 4 + r) * 8 + t) * 64 + lane) * 16u, 0,
                             kAuxDeviceScope);
                 }
             }
@@ -387,23 +446,35 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     __syncthreads();
     if (ticket_s != (unsigned)(split_k - 1))
         return;
-    if (kg == 0) {
+    auto parked_sum = [&](int r, int t) {
+        float4_t v = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int z = 0; z < split_k; ++z) {
+            const float4_t pz = __builtin_bit_cast(
+                float4_t,
+                __builtin_amdgcn_raw_buffer_load_b128(
+                    rp, z * kParkBytes + (unsigned)(((wn * 4 + r) * 8 + t) * 64 + lane) * 16u, 0, kAuxDeviceScope));
+            v.x += pz.x, v.y += pz.y, v.z += pz.z, v.w += pz.w;
+        }
+        return v;
+    };
+    if (kg == 0 && glu) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            float scg[4], bsg[4], scu[4], bsu[4];
+            channel_params(2 * j, scg, bsg);
+            channel_params(2 * j + 1, scu, bsu);
+#pragma unroll
+            for (int t = 0; t < 8; ++t)
+                finish_glu(j, t, parked_sum(2 * j, t), parked_sum(2 * j + 1, t), scg, bsg, scu, bsu);
+        }
+    } else if (kg == 0) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             float sc[4], bs[4];
             channel_params(r, sc, bs);
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                float4_t v = float4_t{0.f, 0.f, 0.f, 0.f};
-                for (int z = 0; z < split_k; ++z) {
-                    const float4_t pz = __builtin_bit_cast(
-                        float4_t, __builtin_amdgcn_raw_buffer_load_b128(
-                                      rp, z * kParkBytes + (unsigned)(((wn * 4 + r) * 8 + t) * 64 + lane) * 16u, 0,
-                                      kAuxDeviceScope));
-                    v.x += pz.x, v.y += pz.y, v.z += pz.z, v.w += pz.w;
-                }
-                finish(r, t, v, sc, bs);
-            }
+            for (int t = 0; t < 8; ++t)
+                finish(r, t, parked_sum(r, t), sc, bs);
         }
     }
     if (tid == 0)
@@ -419,33 +490,32 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
                                                                 void* __restrict__ y, float* __restrict__ ws,
                                                                 unsigned* __restrict__ counters, int M, int N, int K,
                                                                 int kb_total, int kb_per_group, int ng, int zp_const,
-                                                                int kb_per_split, int split_k, int out_f32) {
-    int tile_x, tile_y;
-    xcd_tile(tile_x, tile_y, 2 * PA_BM, PA_BN / 2);
+                                                                int out_f32, int glu, int tiles_x, int tiles_y,
+                                                                int full_tiles, int tail_split, int kb_per_split) {
+    const AsyncWork wk = async_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total);
     prefill_async_body<ZP_TABLE, PRESCALE>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
-                                           zp_const, kb_per_split, split_k, out_f32, tile_x, tile_y * PA_BM,
-                                           tile_y * gridDim.x + tile_x);
+                                           zp_const, out_f32, glu, wk);
 }
 
-// Grouped launch: grid row tile_y is item tile_y of the table, a node of the common shape and format with at most
-// 128 rows of its own (the experts of a mixture-of-experts layer over their gathered rows).  grid =
-// (N/256, items, split).  Workgroups of one item sit together in a super-tile and share its activations in L2.
+// Grouped launch: tile row tile_y is item tile_y of the table, a node of the common shape and format with at most
+// 128 rows of its own (the experts of a mixture-of-experts layer over their gathered rows).  Workgroups of one
+// item sit together in a super-tile and share its activations in L2.
 template <bool ZP_TABLE, bool PRESCALE>
 __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const BatchGroupTable tab,
                                                                         float* __restrict__ ws,
                                                                         unsigned* __restrict__ counters, int N, int K,
                                                                         int kb_total, int kb_per_group, int ng,
-                                                                        int zp_const, int kb_per_split, int split_k,
-                                                                        int out_f32) {
-    int tile_x, tile_y;
-    xcd_tile(tile_x, tile_y, 2 * PA_BM, PA_BN / 2);
-    const BatchGroupItem& it = tab.item[tile_y];
+                                                                        int zp_const, int out_f32, int glu,
+                                                                        int tiles_x, int tiles_y, int full_tiles,
+                                                                        int tail_split, int kb_per_split) {
+    AsyncWork wk = async_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total);
+    const BatchGroupItem& it = tab.item[wk.tile_y];
     if (it.M <= 0)
         return;
+    wk.m0 = 0;
     prefill_async_body<ZP_TABLE, PRESCALE>((const uint4_t*)it.w, (const half_t*)it.scale, (const uint8_t*)it.zp,
                                            (const half_t*)it.x, (const half_t*)it.bias, it.y, ws, counters, it.M, N, K,
-                                           kb_total, kb_per_group, ng, zp_const, kb_per_split, split_k, out_f32, tile_x,
-                                           0, tile_y * gridDim.x + tile_x);
+                                           kb_total, kb_per_group, ng, zp_const, out_f32, glu, wk);
 }
 
 template <typename Kern>
@@ -459,6 +529,16 @@ static int allow_lds(Kern kern, bool* done) {
     return (int)e;
 }
 
+// The launch must be what async_work assumes: a 1-D grid of full_tiles whole tiles plus split_k parts of each
+// remaining tile, parts that cover K.
+static bool async_plan_ok(const FcDeviceArgs& a, const LaunchPlan& p) {
+    const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
+    return p.tiles_x == a.N / PA_BN && p.tiles_y >= 1 && p.full_tiles >= 0 && p.full_tiles <= tiles && p.split_k >= 1 &&
+           (int64_t)p.kblocks_per_split * p.split_k >= a.layout.k_blocks && (p.full_tiles == tiles || p.kblocks_per_split >= 1) &&
+           p.grid[0] == (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) && p.grid[1] == 1 && p.grid[2] == 1 &&
+           (p.split_k == 1 || (a.workspace && a.counters));
+}
+
 template <bool ZPT, bool PRE>
 static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
@@ -469,7 +549,8 @@ static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
     hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), PA_LDS_BYTES, s, (const uint4_t*)a.w,
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
                        a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
-                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, p.kblocks_per_split, p.split_k, a.out_f32);
+                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32, L.glu, p.tiles_x,
+                       p.tiles_y, p.full_tiles, p.split_k, p.kblocks_per_split);
     return (int)hipGetLastError();
 }
 
@@ -483,14 +564,15 @@ static int launch_async_grouped_impl(const BatchGroupTable& tab, const FcDeviceA
         return e;
     hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), PA_LDS_BYTES, s, tab, a.workspace,
                        a.counters, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
-                       L.zp_const, p.kblocks_per_split, p.split_k, a.out_f32);
+                       L.zp_const, a.out_f32, L.glu, p.tiles_x, p.tiles_y, p.full_tiles, p.split_k,
+                       p.kblocks_per_split);
     return (int)hipGetLastError();
 }
 
 int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
-    if (L.bits != 4)
+    if (L.bits != 4 || !async_plan_ok(a, p))
         return (int)hipErrorInvalidValue;  // the planner sends 8-bit nodes to the register-ring kernel
     if (L.groups == 1)
         return L.zp_table ? launch_async_impl<true, false>(a, p, s) : launch_async_impl<false, false>(a, p, s);
@@ -502,7 +584,7 @@ int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const 
                                  void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
-    if (L.bits != 4 || n_items < 1 || n_items > kMaxGroupItems || p.grid[1] != (unsigned)n_items)
+    if (L.bits != 4 || !async_plan_ok(a, p) || n_items < 1 || n_items > kMaxGroupItems || p.tiles_y != n_items)
         return (int)hipErrorInvalidValue;
     for (int i = 0; i < n_items; ++i)
         if (tab.item[i].M < 1 || tab.item[i].M > PA_BM)

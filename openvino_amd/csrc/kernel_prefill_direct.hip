@@ -50,7 +50,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
                                                                  const half_t* __restrict__ bias,
                                                                  void* __restrict__ y, int M, int N, int K,
                                                                  int kb_total, int kb_per_group, int ng, int zp_const,
-                                                                 int out_f32) {
+                                                                 int out_f32, int glu) {
     constexpr int TPB = BITS == 4 ? 1 : 2;   // tiles per k-block and channel tile
     constexpr int WD = BITS == 4 ? 2 : 4;    // packed dwords per lane, channel tile and k-block for this k-group
     constexpr int NOPS = (BITS == 4 ? 5 : 4) + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword (pair)
@@ -285,7 +285,38 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
                 }
         }
         __syncthreads();
-        if (kg == 0) {
+        if (kg == 0 && glu) {
+            // gated linear unit: channel tiles 2 hh and 2 hh + 1 of the wave are gate and up of output channels
+            // (n0 + 64 wn) / 2 + 16 hh .. of the [M, N / 2] result
+            const int ng_ch = n0 + 64 * wn + 32 * hh + 4 * kq;  // gate channels; up channels are 16 further
+            float sc[2][4], bs[2][4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    sc[h][q] = PRESCALE ? 1.f : (float)st[ng_ch + 16 * h + q];
+                    bs[h][q] = bias ? (float)bias[ng_ch + 16 * h + q] : 0.f;
+                }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                float o[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float g = acc[2 * hh][t][q] + ex[((wn * 64 + t * 4 + q) * 64) + lane];
+                    const float u = acc[2 * hh + 1][t][q] + ex[((wn * 64 + (8 + t) * 4 + q) * 64) + lane];
+                    o[q] = glu_value(glu, g * sc[0][q] + bs[0][q], u * sc[1][q] + bs[1][q]);
+                }
+                const int m = m0 + 16 * t + col;
+                const size_t at = (size_t)m * (N / 2) + (n0 + 64 * wn) / 2 + 16 * hh + 4 * kq;
+                if (m < M) {
+                    if (out_f32)
+                        *reinterpret_cast<float4_t*>(static_cast<float*>(y) + at) = float4_t{o[0], o[1], o[2], o[3]};
+                    else
+                        *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + at) =
+                            half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
+                }
+            }
+        } else if (kg == 0) {
 #pragma unroll
             for (int r2 = 0; r2 < 2; ++r2) {
                 const int r = 2 * hh + r2;
@@ -341,7 +372,7 @@ static int launch_direct_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStr
     hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], 1), dim3(512), PD_LDS_BYTES, s, (const uint4_t*)a.w,
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
                        (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
-                       L.zp_const, a.out_f32);
+                       L.zp_const, a.out_f32, L.glu);
     return (int)hipGetLastError();
 }
 

@@ -43,7 +43,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_wide_kernel(const uint4_t* __
                                                                const half_t* __restrict__ bias,
                                                                void* __restrict__ y, int M, int N, int K,
                                                                int kb_total, int kb_per_group, int ng, int zp_const,
-                                                               int out_f32) {
+                                                               int out_f32, int glu) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     half_t* As = reinterpret_cast<half_t*>(lds_raw);  // [2][128 x 64]
     half_t* Bs = As + PW_RING * PW_A_HALVES;          // [2][256 x 64]
@@ -248,9 +248,15 @@ __global__ __launch_bounds__(512) void fcc_prefill_wide_kernel(const uint4_t* __
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + 64 * wm + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                const float v = acc[i][j][r] + hand[((i * 4 + j) * 16 + r) * 64 + lane];
-                if (m < M)
-                    store_out(y, (size_t)m * N + n, v * cs + b, out_f32);
+                const float v = (acc[i][j][r] + hand[((i * 4 + j) * 16 + r) * 64 + lane]) * cs + b;
+                if (glu) {
+                    // gated linear unit: the 32 channels are a gate tile (lanes & 16 == 0) and its up tile
+                    const float up = __shfl_xor(v, 16, 64);
+                    if (m < M && !(lane & 16))
+                        store_out(y, (size_t)m * (N / 2) + (n >> 5) * 16 + (lane & 15), glu_value(glu, v, up), out_f32);
+                } else if (m < M) {
+                    store_out(y, (size_t)m * N + n, v, out_f32);
+                }
             }
     }
 }
@@ -270,7 +276,7 @@ static int launch_wide_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStrea
     hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], 1), dim3(512), PW_LDS_BYTES, s, (const uint4_t*)a.w,
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
                        (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
-                       L.zp_const, a.out_f32);
+                       L.zp_const, a.out_f32, L.glu);
     return (int)hipGetLastError();
 }
 

@@ -39,6 +39,18 @@ struct Layout {
     int zp_const = 0;           // zero-point used when there is no table (includes the unsigned offset)
     int zp_offset = 0;          // 8 for i4, 128 for i8, else 0
     size_t w_bytes = 0, scale_bytes = 0, zp_bytes = 0;
+    // Gated-linear-unit epilogue (OVFCC_GLU_*, 0 = none).  In the tiled layout the 16-channel tiles of gate and up
+    // projection alternate (tile 2 j = gate channels 16 j .., tile 2 j + 1 = up channels 16 j ..; bias likewise),
+    // so that the wave that finishes a gate tile also holds the matching up tile.
+    int glu = 0;
+    bool glu_gate_second = false;
+    // 16-channel block of the OpenVINO-order channel axis that tile nt holds
+    int64_t source_tile(int64_t nt) const {
+        if (!glu)
+            return nt;
+        const bool is_gate = (nt & 1) == 0;
+        return (is_gate != glu_gate_second ? 0 : n_tiles / 2) + (nt >> 1);
+    }
 };
 
 void set_error(const std::string& msg);
@@ -69,6 +81,8 @@ struct FcDeviceArgs {
     int64_t M, N, K, group_size;
     int w_type, zp_type, zp_scalar;
     int out_f32;         // output_type f32 instead of f16
+    int64_t N_out;       // row length of y: N, or N / 2 with a gated-linear-unit epilogue
+    int gate_offset, up_offset;  // untiled layout with such an epilogue: first gate / up channel
     Layout layout;
 };
 
@@ -82,6 +96,8 @@ struct LaunchPlan {
     bool direct = false;        // prefill family: the kernels that feed weights from registers
     bool async_dma = false;     // ... and of those the one whose operands all travel by direct-to-LDS loads
     bool batch = false;         // decode family: the small-batch kernel (waves own channel tiles)
+    int tiles_x = 0, tiles_y = 0;  // async prefill kernel: the tile grid; its launch is 1-D
+    int full_tiles = 0;         // ... of which this many run unsplit (the rest in split_k parts each)
     unsigned grid[3] = {1, 1, 1};
     unsigned block = 256;
     unsigned dynamic_lds = 0;   // bytes of dynamic LDS (decode kernel: the cross-wave reduction buffer)

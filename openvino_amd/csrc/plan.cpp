@@ -33,17 +33,11 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
     if (kernel == OVFCC_KERNEL_PREFILL && (a.N % kPrefillTileN) != 0)
         return fail(OVFCC_EUNSUPPORTED, "the prefill kernel needs N % 128 == 0");
     p.kernel = kernel;
-    if (kernel == OVFCC_KERNEL_PLAIN) {
-        if (a.M > 65535)
-            return fail(OVFCC_EUNSUPPORTED, "the plain kernel handles at most 65535 rows");
-        p.grid[0] = (unsigned)a.N;
-        p.grid[1] = (unsigned)a.M;
-        p.block = 64;
-        p.name = "fcc_plain";
-    } else if (kernel == OVFCC_KERNEL_DECODE &&
-               env_int("OVFCC_DECODE_BATCH", (a.M > 16 || (a.M > 4 && L.w_bytes >= ((size_t)16 << 20))) ? 1 : 0) != 0) {
-        // Small-batch kernel: waves own channel tiles, the workgroup shares one staged slice of X.  It pays
-        // for its split-K epilogue, so the streaming kernel keeps M <= 4 and, for small nodes, M <= 16.
+    // Small-batch kernel: waves own channel tiles, the workgroup shares one staged slice of X.  It pays
+    // for its split-K epilogue, so the streaming kernel keeps M <= 4 and, for small nodes, M <= 16.
+    const bool want_batch =
+        env_int("OVFCC_DECODE_BATCH", (a.M > 16 || (a.M > 4 && L.w_bytes >= ((size_t)16 << 20))) ? 1 : 0) != 0;
+    auto plan_batch = [&]() -> int {
         const int kb = (int)L.k_blocks;
         const int mt = (int)((a.M + 15) / 16);
         int rt = 1;
@@ -85,6 +79,18 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.counter_count = split > 1 ? (size_t)groups : 0;
         p.dynamic_lds = (unsigned)x_bytes(per);
         p.name = L.bits == 4 ? "fcc_batch_w4" : "fcc_batch_w8";
+        return OVFCC_OK;
+    };
+    if (kernel == OVFCC_KERNEL_PLAIN) {
+        if (a.M > 65535)
+            return fail(OVFCC_EUNSUPPORTED, "the plain kernel handles at most 65535 rows");
+        p.grid[0] = (unsigned)a.N_out;
+        p.grid[1] = (unsigned)a.M;
+        p.block = 64;
+        p.name = "fcc_plain";
+    } else if (kernel == OVFCC_KERNEL_DECODE && want_batch) {
+        if (int rc = plan_batch())
+            return rc;
     } else if (kernel == OVFCC_KERNEL_DECODE) {
         if (a.M > 32)
             return fail(OVFCC_EUNSUPPORTED, "the streaming decode kernel handles at most 32 rows");
@@ -120,6 +126,16 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             if ((rt_env == 1 || rt_env == 2 || rt_env == 4) && rt_env <= rt_max && L.n_tiles % rt_env == 0)
                 rt = rt_env;
         }
+        // A gated linear unit needs a gate tile and its up tile in one workgroup, which only the LDS-staged form
+        // of this kernel offers; otherwise the small-batch kernel takes the node.
+        if (L.glu && !xlds) {
+            if (int rc = plan_batch())
+                return rc;
+            *plan = p;
+            return OVFCC_OK;
+        }
+        if (L.glu && rt < 2)
+            rt = 2;
         const int64_t groups = L.n_tiles / rt;
         // waves per workgroup: as many as the k-range feeds with four k-blocks each (the prefetch depth),
         // at most 16, and no more than about 16 waves per compute unit in total
@@ -173,22 +189,41 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.grid[1] = (unsigned)m_tiles;
         p.kblocks_per_split = (int)L.k_blocks;
         if (p.async_dma) {
-            // split K while the tiles alone leave compute units idle (at least eight k-blocks per workgroup);
-            // the f32 tiles are parked in the workspace and added by the last workgroup to arrive
+            // Split K while the tiles alone leave compute units idle (at least eight k-blocks per workgroup): the
+            // f32 tiles are parked in the workspace and added by the last workgroup to arrive.
+            // OVFCC_PREFILL_TAIL = 1 (an experiment, off by default) also splits, with more tiles than compute
+            // units, the tiles of the last, partial round.  It does not pay: the chip is power-limited, a
+            // half-empty round runs at a higher clock, and time is linear in tiles rather than in rounds.
             const int64_t tiles = (int64_t)p.grid[0] * p.grid[1];
             int split = force_split > 0 ? force_split : 1;
-            if (force_split <= 0)
+            int64_t full = 0;
+            if (force_split <= 0) {
                 while (split < 8 && tiles * split * 2 <= n_cus && L.k_blocks / (split * 2) >= 8)
                     split *= 2;
+                const int64_t rest = tiles % n_cus;
+                if (split == 1 && tiles > n_cus && rest * 2 <= n_cus && rest > 0 && L.k_blocks >= 16 &&
+                    env_int("OVFCC_PREFILL_TAIL", 0) != 0) {
+                    full = tiles - rest;
+                    split = 2;
+                    while (split < 8 && rest * split * 2 <= n_cus && L.k_blocks / (split * 2) >= 8)
+                        split *= 2;
+                }
+            }
             if (split > L.k_blocks)
                 split = (int)L.k_blocks;
             const int per = (int)((L.k_blocks + split - 1) / split);
             split = (int)((L.k_blocks + per - 1) / per);
+            if (split == 1)
+                full = tiles;
             p.split_k = split;
             p.kblocks_per_split = per;
-            p.grid[2] = (unsigned)split;
-            p.workspace_bytes = split > 1 ? (size_t)tiles * split * kPrefillTileM * kPrefillWideN * sizeof(float) : 0;
-            p.counter_count = split > 1 ? (size_t)tiles : 0;
+            p.tiles_x = (int)p.grid[0];
+            p.tiles_y = (int)p.grid[1];
+            p.full_tiles = (int)full;
+            p.grid[0] = (unsigned)(full + (tiles - full) * split);
+            p.grid[1] = 1;
+            p.workspace_bytes = split > 1 ? (size_t)(tiles - full) * split * kPrefillTileM * kPrefillWideN * sizeof(float) : 0;
+            p.counter_count = split > 1 ? (size_t)(tiles - full) : 0;
         }
         p.block = wide ? 512 : 256;
         p.name = L.bits == 4 ? (p.async_dma ? "fcc_prefill_async_w4" : p.direct ? "fcc_prefill_direct_w4" : wide ? "fcc_prefill_wide_w4" : "fcc_prefill_w4")

@@ -63,8 +63,12 @@ int validate_desc(const ovfcc_fc_desc* d) {
         return fail(OVFCC_EUNSUPPORTED, "activations must be f16");
     if (d->out_type != OVFCC_F16 && d->out_type != OVFCC_F32)
         return fail(OVFCC_EUNSUPPORTED, "output must be f16 or f32");
-    if (d->flags != 0)
-        return fail(OVFCC_EINVAL, "flags must be 0");
+    if (d->flags & ~(OVFCC_GLU_TYPE_MASK | OVFCC_GLU_GATE_SECOND))
+        return fail(OVFCC_EINVAL, "unknown bits in flags");
+    if ((d->flags & OVFCC_GLU_GATE_SECOND) && (d->flags & OVFCC_GLU_TYPE_MASK) == OVFCC_GLU_NONE)
+        return fail(OVFCC_EINVAL, "OVFCC_GLU_GATE_SECOND without a gated-linear-unit type");
+    if ((d->flags & OVFCC_GLU_TYPE_MASK) != OVFCC_GLU_NONE && (d->N % 2) != 0)
+        return fail(OVFCC_EINVAL, "a gated linear unit splits N in two: N must be even");
     if (d->N > (int64_t)1 << 24 || d->K > (int64_t)1 << 24)
         return fail(OVFCC_EUNSUPPORTED, "N and K are limited to 2^24");
     return OVFCC_OK;
@@ -78,8 +82,10 @@ Layout make_layout(const ovfcc_fc_desc& d) {
     L.zp_table = d.zp_type != OVFCC_NONE && !d.zp_scalar;
     L.zp_const = L.zp_offset;
     // K / 128 < 2^16 keeps the kernels' 32-bit offsets and reciprocal group index exact
-    L.tiled = (d.N % kTileRows == 0) && (d.K % kBlockK == 0) && (d.group_size % kBlockK == 0) &&
-              (d.K / kBlockK < 65536);
+    L.glu = d.flags & OVFCC_GLU_TYPE_MASK;
+    L.glu_gate_second = (d.flags & OVFCC_GLU_GATE_SECOND) != 0;
+    L.tiled = (d.N % (L.glu ? 2 * kTileRows : kTileRows) == 0) && (d.K % kBlockK == 0) &&
+              (d.group_size % kBlockK == 0) && (d.K / kBlockK < 65536);
     if (L.tiled) {
         L.n_tiles = d.N / kTileRows;
         L.k_blocks = d.K / kBlockK;
@@ -155,7 +161,7 @@ void repack_weights(const ovfcc_fc_desc& d, const Layout& L, const void* w, void
             for (int64_t kb = 0; kb < L.k_blocks; ++kb) {
                 uint8_t* tile = dst + (size_t)(nt * L.k_blocks + kb) * kTileBytes;
                 for (int lane = 0; lane < 64; ++lane) {
-                    const int64_t n = nt * kTileRows + (lane & 15);
+                    const int64_t n = L.source_tile(nt) * kTileRows + (lane & 15);
                     const int kq = lane >> 4;
                     for (int j = 0; j < 4; ++j) {
                         const int64_t k = kb * kBlockK + 32 * j + 8 * kq;
@@ -174,7 +180,7 @@ void repack_weights(const ovfcc_fc_desc& d, const Layout& L, const void* w, void
             for (int64_t kt = 0; kt < k_tiles; ++kt) {
                 uint8_t* tile = dst + (size_t)(nt * k_tiles + kt) * kTileBytes;
                 for (int lane = 0; lane < 64; ++lane) {
-                    const int64_t n = nt * kTileRows + (lane & 15);
+                    const int64_t n = L.source_tile(nt) * kTileRows + (lane & 15);
                     const int kq = lane >> 4;
                     for (int dw = 0; dw < 4; ++dw) {
                         const int64_t k = kt * 64 + 32 * (dw >> 1) + 8 * kq + 4 * (dw & 1);
@@ -197,7 +203,7 @@ void unrepack_weights(const ovfcc_fc_desc& d, const Layout& L, const void* w_til
             for (int64_t kb = 0; kb < L.k_blocks; ++kb) {
                 const uint8_t* tile = src + (size_t)(nt * L.k_blocks + kb) * kTileBytes;
                 for (int lane = 0; lane < 64; ++lane) {
-                    const int64_t n = nt * kTileRows + (lane & 15);
+                    const int64_t n = L.source_tile(nt) * kTileRows + (lane & 15);
                     const int kq = lane >> 4;
                     for (int j = 0; j < 4; ++j) {
                         const int64_t k = kb * kBlockK + 32 * j + 8 * kq;
@@ -216,7 +222,7 @@ void unrepack_weights(const ovfcc_fc_desc& d, const Layout& L, const void* w_til
             for (int64_t kt = 0; kt < k_tiles; ++kt) {
                 const uint8_t* tile = src + (size_t)(nt * k_tiles + kt) * kTileBytes;
                 for (int lane = 0; lane < 64; ++lane) {
-                    const int64_t n = nt * kTileRows + (lane & 15);
+                    const int64_t n = L.source_tile(nt) * kTileRows + (lane & 15);
                     const int kq = lane >> 4;
                     for (int dw = 0; dw < 4; ++dw) {
                         const int64_t k = kt * 64 + 32 * (dw >> 1) + 8 * kq + 4 * (dw & 1);
@@ -239,7 +245,7 @@ void repack_params(const ovfcc_fc_desc& d, const Layout& L, const void* scales, 
     for (int64_t nt = 0; nt < L.n_tiles; ++nt)
         for (int64_t g = 0; g < ng; ++g)
             for (int r = 0; r < kTileRows; ++r) {
-                const int64_t n = nt * kTileRows + r;
+                const int64_t n = L.source_tile(nt) * kTileRows + r;
                 const size_t o = (size_t)(nt * ng + g) * kTileRows + r;
                 st[o] = s[n * ng + g];
                 if (L.zp_table) {
@@ -261,7 +267,7 @@ void unrepack_params(const ovfcc_fc_desc& d, const Layout& L, const void* scale_
     for (int64_t nt = 0; nt < L.n_tiles; ++nt)
         for (int64_t g = 0; g < ng; ++g)
             for (int r = 0; r < kTileRows; ++r) {
-                const int64_t n = nt * kTileRows + r;
+                const int64_t n = L.source_tile(nt) * kTileRows + r;
                 const size_t o = (size_t)(nt * ng + g) * kTileRows + r;
                 s[n * ng + g] = st[o];
                 if (L.zp_table) {

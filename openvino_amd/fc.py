@@ -21,7 +21,8 @@ def _vp(a: Optional[np.ndarray]):
 
 
 def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
-              has_bias: bool = False, out_type: str = "f16") -> FcDesc:
+              has_bias: bool = False, out_type: str = "f16", glu: Optional[str] = None,
+              glu_gate_second: bool = False) -> FcDesc:
     d = FcDesc()
     d.N, d.K, d.group_size = N, K, group_size
     d.w_type = _lib.TYPE[w_type]
@@ -31,7 +32,7 @@ def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none
     d.bias_type = _lib.F16 if has_bias else _lib.NONE
     d.act_type = _lib.F16
     d.out_type = _lib.TYPE[out_type]
-    d.flags = 0
+    d.flags = _lib.GLU[glu] | (_lib.GLU_GATE_SECOND if glu_gate_second else 0)
     return d
 
 
@@ -85,11 +86,13 @@ class CompressedWeights:
 
     def __init__(self, device: Device, W: np.ndarray, weight_scales: np.ndarray, weight_zero_points=None, bias=None, *,
                  N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
-                 output_type: str = "f16"):
+                 output_type: str = "f16", glu: Optional[str] = None, glu_gate_second: bool = False):
+        """glu = "swish" | "gelu" | "gelu_tanh": W holds gate and up projection ([N, K], first and second half of
+        the rows, or the other way round with glu_gate_second) and the node computes act(gate) * up, [M, N / 2]."""
         self.device = device
         self.N, self.K, self.group_size = N, K, group_size
         self.desc = make_desc(N, K, group_size, w_type, zp_type if weight_zero_points is not None else "none",
-                              zp_scalar, bias is not None, output_type)
+                              zp_scalar, bias is not None, output_type, glu, glu_gate_second)
         W = np.ascontiguousarray(W).view(np.uint8)
         s = np.ascontiguousarray(weight_scales, dtype=np.float16)
         z = None if weight_zero_points is None else np.ascontiguousarray(weight_zero_points, dtype=np.uint8)
@@ -100,9 +103,30 @@ class CompressedWeights:
         self.handle = h
 
     @classmethod
-    def from_case(cls, device: Device, c, output_type: str = "f16") -> "CompressedWeights":
+    def from_case(cls, device: Device, c, output_type: str = "f16", glu: Optional[str] = None,
+                  glu_gate_second: bool = False) -> "CompressedWeights":
         return cls(device, c.w, c.scale, c.zp, c.bias, N=c.N, K=c.K, group_size=c.group_size, w_type=c.w_type,
-                   zp_type=c.zp_type, zp_scalar=c.zp_scalar, output_type=output_type)
+                   zp_type=c.zp_type, zp_scalar=c.zp_scalar, output_type=output_type, glu=glu,
+                   glu_gate_second=glu_gate_second)
+
+    @property
+    def N_out(self) -> int:
+        """Row length of the node's output: N, or N / 2 with a gated-linear-unit epilogue."""
+        return self.N // 2 if self.desc.flags & 3 else self.N
+
+    @classmethod
+    def glu(cls, gate: "CompressedWeights", up: "CompressedWeights", kind: str = "swish") -> "CompressedWeights":
+        """Gate and up projection fused into one node that computes act(gate(x)) * up(x)."""
+        h = ctypes.c_void_p()
+        check(gate.device.lib.ovfcc_weights_glu(gate.handle, up.handle, _lib.GLU[kind], ctypes.byref(h)))
+        other = object.__new__(CompressedWeights)
+        other.device, other.K, other.group_size = gate.device, gate.K, gate.group_size
+        other.N = 2 * gate.N
+        other.desc = FcDesc.from_buffer_copy(gate.desc)
+        other.desc.N = other.N
+        other.desc.flags = _lib.GLU[kind]
+        other.handle = h
+        return other
 
     def clone(self) -> "CompressedWeights":
         """Second device copy at distinct addresses (no host work)."""
@@ -166,7 +190,8 @@ class InferRequest:
         if X.shape[-1] != weights.K:
             raise OvfccError(_lib.EINVAL, f"last dimension of X is {X.shape[-1]}, expected K = {weights.K}")
         M = int(np.prod(X.shape[:-1], dtype=np.int64))
-        Y = np.empty(X.shape[:-1] + (weights.N,), dtype=np.float32 if weights.desc.out_type == _lib.F32 else np.float16)
+        Y = np.empty(X.shape[:-1] + (weights.N_out,),
+                     dtype=np.float32 if weights.desc.out_type == _lib.F32 else np.float16)
         check(self.device.lib.ovfcc_fc_run(self.handle, weights.handle, _vp(X), _vp(Y), M))
         return Y
 
@@ -197,14 +222,14 @@ class InferRequest:
                     raise OvfccError(_lib.EINVAL, f"X has shape {X.shape}, expected [M, {w.K}]")
                 xs.append(X)
                 itemsize = 4 if w.desc.out_type == _lib.F32 else 2
-                x_ptr, y_ptr = dev.malloc(max(X.nbytes, 16)), dev.malloc(max(X.shape[0] * w.N * itemsize, 16))
+                x_ptr, y_ptr = dev.malloc(max(X.nbytes, 16)), dev.malloc(max(X.shape[0] * w.N_out * itemsize, 16))
                 ptrs.append((x_ptr, y_ptr))
                 if X.size:
                     dev.upload(x_ptr, X)
             self.infer_grouped_device([(w, xp, yp, X.shape[0]) for (w, _), X, (xp, yp) in zip(items, xs, ptrs)])
             self.sync()
-            return [dev.download(yp, (X.shape[0], w.N), np.float32 if w.desc.out_type == _lib.F32 else np.float16)
-                    if X.shape[0] else np.empty((0, w.N), np.float32 if w.desc.out_type == _lib.F32 else np.float16)
+            return [dev.download(yp, (X.shape[0], w.N_out), np.float32 if w.desc.out_type == _lib.F32 else np.float16)
+                    if X.shape[0] else np.empty((0, w.N_out), np.float32 if w.desc.out_type == _lib.F32 else np.float16)
                     for (w, _), X, (_, yp) in zip(items, xs, ptrs)]
         finally:
             for xp, yp in ptrs:

@@ -31,12 +31,24 @@
  *                    algebraic invariants (zp == q gives 0, scale linearity, unit-vector
  *                    probes, i4 == u4 xor 8 with zp 8, row permutation)
  *
+ *   glu              the stand-alone formula of the Intel-GPU plugin,
+ *                    src/plugins/intel_gpu/src/kernel_selector/cl_kernels/swiglu_gpu_ref.cl:46-90
+ *                    (split form, GATE_IDX, the three GLU_TYPEs), the op's attributes
+ *                    src/common/transformations/include/ov_ops/glu.hpp:16-40 and the host
+ *                    restatement in the reference's own test,
+ *                    src/plugins/intel_gpu/tests/unit/test_cases/swiglu_gpu_test.cpp:55-72.
+ *                    The reference holds no numeric vector for it (its tests recompute the
+ *                    formula); pinned against library routines (torch silu / gelu, exact and
+ *                    tanh form), the identities act(x) - act(-x) = x, act(0) = 0, and the
+ *                    roles of the two halves on one-hot inputs.
+ *
  * Parity unpinned: the CPU plugin's numbers come from the oneDNN fork's decompression
  * inner-product kernel (openvinotoolkit/oneDNN, a submodule whose commit the tree does
  * not record and whose sources are absent).  Its summation order and intermediate
  * roundings are not restated here; the reference's own tests hold only tolerance checks
  * at that boundary, and so does this oracle's use (fp32 accumulation in k order).
  */
+#include <math.h>
 #include <stddef.h>
 #include <stdint.h>
 #include <string.h>
@@ -283,6 +295,28 @@ int ovo_fc_reference(const ovo_fc_args* a, float* y) {
     }
     __builtin_free(xf);
     return status;
+}
+
+/* Gated linear unit over the last axis of y [M, 2 L]: out[m, f] = act(y[m, g + f]) * y[m, u + f] with
+ * (g, u) = (0, L), or (L, 0) when gate_second (the op's split_to_glu_idx = 1).  type: 1 Swish (beta = 1),
+ * 2 Gelu (erf), 3 Gelu_Tanh.  Evaluated in double, returned as float. */
+int ovo_glu(const float* y, int64_t M, int64_t L, int32_t type, int32_t gate_second, float* out) {
+    if (!y || !out || M < 0 || L <= 0 || type < 1 || type > 3)
+        return -1;
+    const int64_t g0 = gate_second ? L : 0, u0 = gate_second ? 0 : L;
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t f = 0; f < L; ++f) {
+            const double gate = y[m * 2 * L + g0 + f], up = y[m * 2 * L + u0 + f];
+            double a;
+            if (type == 1)
+                a = gate / (1.0 + exp(-gate));
+            else if (type == 2)
+                a = 0.5 * gate * (1.0 + erf(gate * 0.70710678118654752440));
+            else
+                a = 0.5 * gate * (1.0 + tanh(0.79788456080286535588 * gate * (1.0 + 0.044715 * gate * gate)));
+            out[m * L + f] = (float)(a * up);
+        }
+    return 0;
 }
 
 int ovo_num_threads(void) {

@@ -196,6 +196,24 @@ def fc_reference(x, w, w_type, scale, zp=None, zp_type=NONE, bias=None, *, N, K,
     return y
 
 
+GLU_SWISH, GLU_GELU, GLU_GELU_TANH = 1, 2, 3
+
+
+def glu(y, glu_type, gate_second=False) -> np.ndarray:
+    """C oracle of the gated linear unit over the last axis of y [M, 2 L]: act(gate half) * up half, float32 [M, L]."""
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    M, N = y.shape
+    if N % 2:
+        raise ValueError("the last axis must be even")
+    out = np.empty((M, N // 2), dtype=np.float32)
+    f = lib().ovo_glu
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+    if f(_ptr(y), M, N // 2, int(glu_type), int(bool(gate_second)), _ptr(out)) != 0:
+        raise ValueError("ovo_glu rejected its arguments")
+    return out
+
+
 # ---- independent numpy restatement (bit operations and float64 matmul) ----
 
 def np_unpack_nibbles(packed: np.ndarray, n: int, signed: bool) -> np.ndarray:

@@ -40,7 +40,8 @@ def test_version_and_error_string():
     (dict(group_size=96), _lib.EINVAL), (dict(w_type=_lib.F16), _lib.EUNSUPPORTED),
     (dict(scale_type=_lib.F32), _lib.EUNSUPPORTED), (dict(zp_type=_lib.I4), _lib.EUNSUPPORTED),
     (dict(act_type=_lib.F32), _lib.EUNSUPPORTED), (dict(out_type=_lib.U8), _lib.EUNSUPPORTED),
-    (dict(bias_type=_lib.F32), _lib.EUNSUPPORTED), (dict(flags=1), _lib.EINVAL),
+    (dict(bias_type=_lib.F32), _lib.EUNSUPPORTED), (dict(flags=8), _lib.EINVAL),
+    (dict(flags=4), _lib.EINVAL), (dict(flags=1, N=63), _lib.EINVAL),
 ])
 def test_descriptor_gate(mutate, code):
     d = fc.make_desc(64, 256, 128, "u4", "u4")
@@ -49,6 +50,33 @@ def test_descriptor_gate(mutate, code):
         setattr(d, k, v)
     assert fc.validate(d) == code
     assert _lib.load().ovfcc_last_error() != b""
+
+
+def test_glu_descriptor_and_layout():
+    """A gated-linear-unit node keeps the tiled layout when its halves are whole tiles (N % 32 == 0), and the
+    repacker alternates gate and up tiles: unrepacking restores the OpenVINO order."""
+    assert fc.validate(fc.make_desc(64, 256, 128, "u4", "u4", glu="swish")) == _lib.OK
+    assert fc.validate(fc.make_desc(64, 256, 128, "u4", "u4", glu="gelu_tanh", glu_gate_second=True)) == _lib.OK
+    assert fc.tiled_sizes(fc.make_desc(64, 256, 128, "u4", "u4", glu="swish"))[0] == 64 * 256 // 2
+    assert fc.tiled_sizes(fc.make_desc(48, 256, 128, "u4", "u4"))[0] == 48 * 256 // 2
+    assert fc.tiled_sizes(fc.make_desc(48, 256, 128, "u4", "u4", glu="swish"))[0] == 0      # halves of 24 channels
+    rng = np.random.default_rng(5)
+    N, K = 64, 256
+    W = rng.integers(0, 256, N * K // 2, dtype=np.uint8)
+    S = rng.uniform(0.01, 0.02, (N, 2)).astype(np.float16)
+    Z = rng.integers(0, 256, N * 2 // 2, dtype=np.uint8)
+    plain = fc.make_desc(N, K, 128, "u4", "u4")
+    wt0, st0, zt0 = fc.repack_host(plain, W, S, Z)
+    for second in (False, True):
+        d = fc.make_desc(N, K, 128, "u4", "u4", glu="swish", glu_gate_second=second)
+        wt, st, zt = fc.repack_host(d, W, S, Z)
+        tile_w = wt0.size // 4                          # bytes of one 16-channel tile row
+        order = [2, 0, 3, 1] if second else [0, 2, 1, 3]  # tiles: gate j, up j, ...
+        assert np.array_equal(wt.reshape(4, tile_w), wt0.reshape(4, tile_w)[order])
+        assert np.array_equal(st.reshape(4, -1), st0.reshape(4, -1)[order])
+        assert np.array_equal(zt.reshape(4, -1), zt0.reshape(4, -1)[order])
+        w2, s2, z2 = fc.unrepack_host(d, wt, st, zt)
+        assert np.array_equal(w2, W) and np.array_equal(s2, S) and np.array_equal(z2, Z)
 
 
 def test_null_descriptor_and_null_outputs():

@@ -430,3 +430,30 @@ def test_grouped_run_mixtral_experts(oracle, dev, req):
     finally:
         for w in ws:
             w.close()
+
+
+def test_prefill_splits_only_the_last_partial_round(oracle, dev, req, monkeypatch):
+    """More tiles than compute units with a small remainder, OVFCC_PREFILL_TAIL = 1: the whole rounds run unsplit,
+    the remaining tiles are cut along K so that the last round fills the chip.  Every row against the numpy oracle
+    (itself pinned against the C oracle in the CPU tests), identical bits on repeats, and the unsplit launch."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    monkeypatch.setenv("OVFCC_PREFILL_TAIL", "1")
+    M, K, N = 3400, 2048, 2560          # 10 x 27 = 270 tiles of 128 x 256
+    say(f"tail split M={M} K={K} N={N}")
+    c = datagen.make_case(810, M, K, N, "u4", 128, "u4", with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        y = req.infer(w, c.x)
+        info = req.last_kernel()
+        n_cus = info["grid"][0] - 270   # (270 - full) * (split - 1) extra workgroups
+        assert info["name"] == "fcc_prefill_async_w4" and info["split_k"] > 1 and n_cus > 0, info
+        ref = oracle.fc_reference_numpy(c.x, c.w, oracle.U4, c.scale, c.zp, oracle.U4, c.bias, N=N, K=K, group_size=128)
+        check_parity(oracle, y, ref, K, f"{info}", output_rounding_slack=True)
+        for _ in range(3):
+            assert np.array_equal(req.infer(w, c.x).view(np.uint16), y.view(np.uint16))
+        monkeypatch.setenv("OVFCC_PREFILL_TAIL", "0")
+        whole = req.infer(w, c.x)
+        assert req.last_kernel()["split_k"] == 1 and req.last_kernel()["grid"][0] == 270
+        check_parity(oracle, whole, ref, K, "unsplit", output_rounding_slack=True)
+    finally:
+        w.close()
