@@ -146,6 +146,18 @@ int64_t ovfcc_weights_device_bytes(const ovfcc_weights* w);
 /* 1 when the node uses the tiled layout (fast kernels), 0 for the OpenVINO-layout fallback */
 int ovfcc_weights_is_tiled(const ovfcc_weights* w);
 
+/* The node in its device form as one relocatable host blob, and back: what ICompiledModel::export_model /
+ * IPlugin::import_model (src/inference/dev_api/openvino/runtime/icompiled_model.hpp:105, iplugin.hpp:173-208; the
+ * template plugin's pair: src/plugins/template/src/compiled_model.cpp:173-192, plugin.cpp:230-311) store per node so
+ * that a cached model skips the repack (ov::cache_dir, src/inference/src/dev/core_impl.cpp:858-897).
+ * ovfcc_weights_export_size gives the blob's size; ovfcc_weights_export fills a host buffer of at least that size;
+ * ovfcc_weights_import rebuilds the node on ctx's device.  A blob is valid for this library version only: import
+ * checks magic, version, descriptor and every size against what the descriptor implies and fails with
+ * OVFCC_EINVAL otherwise. */
+int ovfcc_weights_export_size(const ovfcc_weights* w, size_t* bytes);
+int ovfcc_weights_export(const ovfcc_weights* w, void* blob, size_t bytes);
+int ovfcc_weights_import(ovfcc_ctx* ctx, const void* blob, size_t bytes, ovfcc_weights** out);
+
 /* One infer request: ov::ISyncInferRequest
  * (src/inference/dev_api/openvino/runtime/isync_infer_request.hpp:30-175).  Different requests
  * may run concurrently from different threads; one request is used by one thread at a time. */

@@ -16,7 +16,7 @@ GLU_GATE_SECOND = 4
 
 # every symbol include/ovfcc.h declares
 SYMBOLS = [
-    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_glu", "ovfcc_weights_destroy",
+    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_glu", "ovfcc_weights_export_size", "ovfcc_weights_export", "ovfcc_weights_import", "ovfcc_weights_destroy",
     "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
     "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_grouped_device", "ovfcc_bench_grouped", "ovfcc_request_sync", "ovfcc_request_force_kernel",
     "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
@@ -77,6 +77,9 @@ def load() -> ctypes.CDLL:
         "ovfcc_weights_clone": (ci, [vp, pp]),
         "ovfcc_weights_concat": (ci, [pp, ci, pp]),
         "ovfcc_weights_glu": (ci, [vp, vp, ci, pp]),
+        "ovfcc_weights_export_size": (ci, [vp, ctypes.POINTER(ctypes.c_size_t)]),
+        "ovfcc_weights_export": (ci, [vp, vp, ctypes.c_size_t]),
+        "ovfcc_weights_import": (ci, [vp, vp, ctypes.c_size_t, pp]),
         "ovfcc_weights_destroy": (None, [vp]),
         "ovfcc_weights_device_bytes": (i64, [vp]),
         "ovfcc_weights_is_tiled": (ci, [vp]),

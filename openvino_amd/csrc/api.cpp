@@ -478,6 +478,133 @@ int ovfcc_weights_is_tiled(const ovfcc_weights* w) {
     return w && w->layout.tiled ? 1 : 0;
 }
 
+namespace {
+
+// Blob of one node: header, then the device arrays in this order, each padded to 16 bytes.
+struct BlobHeader {
+    char magic[8];        // "OVFCCW\0\0"
+    uint32_t version;     // layout version of blob and tiles
+    uint32_t header_bytes;
+    ovfcc_fc_desc desc;
+    int32_t zp_const;
+    int32_t tiled;
+    uint64_t w_bytes, scale_bytes, zp_bytes, bias_bytes;
+};
+constexpr uint32_t kBlobVersion = 2;
+const char kBlobMagic[8] = {'O', 'V', 'F', 'C', 'C', 'W', 0, 0};
+
+size_t pad16(size_t n) {
+    return (n + 15) & ~(size_t)15;
+}
+
+// sizes of the four device arrays of a node
+void device_sizes(const ovfcc_fc_desc& d, const ovfcc::Layout& L, uint64_t out[4]) {
+    const int64_t N = d.N, K = d.K, ng = L.groups;
+    if (L.tiled) {
+        out[0] = L.w_bytes, out[1] = L.scale_bytes, out[2] = L.zp_bytes;
+    } else {
+        out[0] = L.bits == 4 ? (uint64_t)(N * K + 1) / 2 : (uint64_t)N * K;
+        out[1] = (uint64_t)N * ng * 2;
+        out[2] = 0;
+        if (d.zp_type != OVFCC_NONE) {
+            const uint64_t cnt = d.zp_scalar ? 1 : (uint64_t)N * ng;
+            out[2] = d.zp_type == OVFCC_U4 ? (cnt + 1) / 2 : cnt;
+        }
+    }
+    out[3] = d.bias_type != OVFCC_NONE ? (uint64_t)N * 2 : 0;
+}
+
+}  // namespace
+
+int ovfcc_weights_export_size(const ovfcc_weights* w, size_t* bytes) {
+    if (!w || !bytes)
+        return fail(OVFCC_EINVAL, "null argument");
+    uint64_t sz[4];
+    device_sizes(w->desc, w->layout, sz);
+    *bytes = pad16(sizeof(BlobHeader)) + pad16(sz[0]) + pad16(sz[1]) + pad16(sz[2]) + pad16(sz[3]);
+    return OVFCC_OK;
+}
+
+int ovfcc_weights_export(const ovfcc_weights* w, void* blob, size_t bytes) {
+    size_t need = 0;
+    int rc = ovfcc_weights_export_size(w, &need);
+    if (rc)
+        return rc;
+    if (!blob || bytes < need)
+        return fail(OVFCC_EINVAL, "blob buffer is null or too small");
+    HIP_TRY(hipSetDevice(w->ctx->device));
+    uint64_t sz[4];
+    device_sizes(w->desc, w->layout, sz);
+    BlobHeader h{};
+    std::memcpy(h.magic, kBlobMagic, 8);
+    h.version = kBlobVersion;
+    h.header_bytes = (uint32_t)sizeof(BlobHeader);
+    h.desc = w->desc;
+    h.zp_const = w->layout.zp_const;
+    h.tiled = w->layout.tiled ? 1 : 0;
+    h.w_bytes = sz[0], h.scale_bytes = sz[1], h.zp_bytes = sz[2], h.bias_bytes = sz[3];
+    char* at = static_cast<char*>(blob);
+    std::memset(at, 0, need);
+    std::memcpy(at, &h, sizeof(h));
+    at += pad16(sizeof(BlobHeader));
+    const void* src[4] = {w->d_w, w->d_scale, w->d_zp, w->d_bias};
+    for (int i = 0; i < 4; ++i) {
+        if (sz[i] && src[i])
+            HIP_TRY(hipMemcpy(at, src[i], sz[i], hipMemcpyDeviceToHost));
+        at += pad16(sz[i]);
+    }
+    return OVFCC_OK;
+}
+
+int ovfcc_weights_import(ovfcc_ctx* ctx, const void* blob, size_t bytes, ovfcc_weights** out) {
+    if (!ctx || !blob || !out)
+        return fail(OVFCC_EINVAL, "null argument");
+    *out = nullptr;
+    if (bytes < pad16(sizeof(BlobHeader)))
+        return fail(OVFCC_EINVAL, "blob is shorter than its header");
+    BlobHeader h;
+    std::memcpy(&h, blob, sizeof(h));
+    if (std::memcmp(h.magic, kBlobMagic, 8) != 0 || h.version != kBlobVersion || h.header_bytes != sizeof(BlobHeader))
+        return fail(OVFCC_EINVAL, "not a weight blob of this library version");
+    int rc = ovfcc::validate_desc(&h.desc);
+    if (rc)
+        return rc;
+    ovfcc::Layout L = ovfcc::make_layout(h.desc);
+    uint64_t sz[4];
+    device_sizes(h.desc, L, sz);
+    // a scalar zero-point lives in zp_const; everything else must be exactly what the descriptor implies
+    const int zp_lo = L.zp_offset, zp_hi = L.zp_offset + 255;
+    if ((h.tiled != 0) != L.tiled || h.w_bytes != sz[0] || h.scale_bytes != sz[1] || h.zp_bytes != sz[2] ||
+        h.bias_bytes != sz[3] || h.zp_const < zp_lo || h.zp_const > zp_hi ||
+        bytes < pad16(sizeof(BlobHeader)) + pad16(sz[0]) + pad16(sz[1]) + pad16(sz[2]) + pad16(sz[3]))
+        return fail(OVFCC_EINVAL, "blob sizes do not match its descriptor");
+    L.zp_const = h.zp_const;
+    HIP_TRY(hipSetDevice(ctx->device));
+    ovfcc_weights* W = new ovfcc_weights();
+    W->ctx = ctx;
+    W->desc = h.desc;
+    W->layout = L;
+    const char* at = static_cast<const char*>(blob) + pad16(sizeof(BlobHeader));
+    void** dst[4] = {&W->d_w, &W->d_scale, &W->d_zp, &W->d_bias};
+    for (int i = 0; i < 4 && !rc; ++i) {
+        if (sz[i]) {
+            hipError_t e = hipMalloc(dst[i], sz[i]);
+            if (e == hipSuccess)
+                e = hipMemcpy(*dst[i], at, sz[i], hipMemcpyHostToDevice);
+            if (e != hipSuccess)
+                rc = hip_fail(e, "weight blob upload");
+            W->bytes += sz[i];
+        }
+        at += pad16(sz[i]);
+    }
+    if (rc) {
+        ovfcc_weights_destroy(W);
+        return rc;
+    }
+    *out = W;
+    return OVFCC_OK;
+}
+
 int ovfcc_request_create(ovfcc_ctx* ctx, ovfcc_request** out) {
     if (!ctx || !out)
         return fail(OVFCC_EINVAL, "ctx or out is null");

@@ -153,6 +153,26 @@ class CompressedWeights:
         other.handle = h
         return other
 
+    def export_blob(self) -> np.ndarray:
+        """The node in its device form as one host blob (what a model cache stores instead of repacking again)."""
+        n = ctypes.c_size_t()
+        check(self.device.lib.ovfcc_weights_export_size(self.handle, ctypes.byref(n)))
+        blob = np.empty(n.value, np.uint8)
+        check(self.device.lib.ovfcc_weights_export(self.handle, _vp(blob), blob.nbytes))
+        return blob
+
+    @classmethod
+    def import_blob(cls, device: Device, blob: np.ndarray) -> "CompressedWeights":
+        blob = np.ascontiguousarray(blob, dtype=np.uint8)
+        h = ctypes.c_void_p()
+        check(device.lib.ovfcc_weights_import(device.handle, _vp(blob), blob.nbytes, ctypes.byref(h)))
+        other = object.__new__(CompressedWeights)
+        other.device = device
+        other.desc = FcDesc.from_buffer_copy(blob[16:16 + ctypes.sizeof(FcDesc)].tobytes())
+        other.N, other.K, other.group_size = other.desc.N, other.desc.K, other.desc.group_size
+        other.handle = h
+        return other
+
     @property
     def tiled(self) -> bool:
         return bool(self.device.lib.ovfcc_weights_is_tiled(self.handle))

@@ -457,3 +457,47 @@ def test_prefill_splits_only_the_last_partial_round(oracle, dev, req, monkeypatc
         check_parity(oracle, whole, ref, K, "unsplit", output_rounding_slack=True)
     finally:
         w.close()
+
+
+def test_weight_blob_export_import(oracle, dev, req):
+    """A node exported as a host blob and imported again gives identical bits (tiled, untiled, fused and
+    gated nodes); damaged blobs are refused."""
+    say("weight blob")
+    tiled = datagen.make_case(830, 40, 512, 256, "u4", 128, "u4", with_bias=True)
+    plain = datagen.make_case(831, 9, 200, 40, "u8", 50, "u8")
+    scalar = datagen.make_case(832, 5, 256, 64, "u8", 128, "u8")
+    scalar.zp, scalar.zp_scalar = np.array([131], np.uint8), True
+    ws = [fc.CompressedWeights.from_case(dev, tiled), fc.CompressedWeights.from_case(dev, plain),
+          fc.CompressedWeights.from_case(dev, scalar), fc.CompressedWeights.from_case(dev, tiled, glu="swish")]
+    ws.append(fc.CompressedWeights.concat([ws[0], ws[0]]))
+    xs = [tiled.x, plain.x, scalar.x, tiled.x, tiled.x]
+    try:
+        for w, x in zip(ws, xs):
+            blob = w.export_blob()
+            back = fc.CompressedWeights.import_blob(dev, blob)
+            try:
+                assert (back.N, back.K, back.N_out, back.tiled) == (w.N, w.K, w.N_out, w.tiled)
+                assert back.device_bytes == w.device_bytes
+                for M in (1, x.shape[0]):
+                    assert np.array_equal(req.infer(back, x[:M]).view(np.uint16), req.infer(w, x[:M]).view(np.uint16))
+                assert np.array_equal(back.export_blob(), blob)
+            finally:
+                back.close()
+        blob = ws[0].export_blob()
+        for damage in ("magic", "version", "short", "shape", "size"):
+            bad = blob.copy()
+            if damage == "magic":
+                bad[0] ^= 1
+            elif damage == "version":
+                bad[8] += 1
+            elif damage == "short":
+                bad = bad[:-16]
+            elif damage == "shape":
+                bad[16:24] = np.frombuffer(np.int64(512).tobytes(), np.uint8)       # N: 256 -> 512
+            else:
+                bad[16 + 56 + 8:16 + 56 + 16] = np.frombuffer(np.uint64(1 << 40).tobytes(), np.uint8)  # w_bytes
+            with pytest.raises(fc.OvfccError):
+                fc.CompressedWeights.import_blob(dev, bad)
+    finally:
+        for w in ws:
+            w.close()
