@@ -1,0 +1,167 @@
+// Host-logic check, built with AddressSanitizer and UBSan by tests/test_host_logic.py: descriptor gate, layout,
+// repack round trips on exactly sized buffers, and the invariants every launch plan must satisfy before a kernel
+// may be launched with it.  No GPU: the kernel launchers are stubbed out below and never called.
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "ovfcc_internal.h"
+
+namespace ovfcc {
+int launch_plain(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_decode(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_batch(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_prefill(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_prefill_wide(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_prefill_direct(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_prefill_async(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+}  // namespace ovfcc
+
+static int g_failures = 0;
+#define CHECK(cond, ...)                                   \
+    do {                                                   \
+        if (!(cond)) {                                     \
+            std::printf("FAILED %s: ", #cond);             \
+            std::printf(__VA_ARGS__);                      \
+            std::printf("\n");                             \
+            ++g_failures;                                  \
+        }                                                  \
+    } while (0)
+
+static ovfcc_fc_desc desc(int64_t N, int64_t K, int64_t G, int w_type, int zp_type, int flags) {
+    ovfcc_fc_desc d{};
+    d.N = N, d.K = K, d.group_size = G, d.w_type = w_type, d.scale_type = OVFCC_F16, d.zp_type = zp_type;
+    d.bias_type = OVFCC_NONE, d.act_type = OVFCC_F16, d.out_type = OVFCC_F16, d.flags = flags;
+    return d;
+}
+
+static void round_trip(const ovfcc_fc_desc& d, std::mt19937& rng) {
+    const ovfcc::Layout L = ovfcc::make_layout(d);
+    if (!L.tiled)
+        return;
+    const bool four = L.bits == 4;
+    const size_t wb = four ? (size_t)d.N * d.K / 2 : (size_t)d.N * d.K, cnt = (size_t)d.N * L.groups;
+    const size_t zb = d.zp_type == OVFCC_NONE ? 0 : (d.zp_type == OVFCC_U4 ? (cnt + 1) / 2 : cnt);
+    std::vector<uint8_t> w(wb), z(zb), w2(wb), z2(zb), wt(L.w_bytes), zt(L.zp_bytes);
+    std::vector<uint16_t> s(cnt), s2(cnt), st(L.scale_bytes / 2);
+    for (auto& v : w) v = (uint8_t)rng();
+    for (auto& v : z) v = (uint8_t)rng();
+    for (auto& v : s) v = (uint16_t)rng();
+    ovfcc::repack_weights(d, L, w.data(), wt.data());
+    ovfcc::repack_params(d, L, s.data(), zb ? z.data() : nullptr, st.data(), zt.data());
+    ovfcc::unrepack_weights(d, L, wt.data(), w2.data());
+    ovfcc::unrepack_params(d, L, st.data(), zt.data(), s2.data(), zb ? z2.data() : nullptr);
+    CHECK(w == w2 && s == s2 && z == z2, "round trip N=%ld K=%ld G=%ld type=%d zp=%d flags=%d", (long)d.N, (long)d.K,
+          (long)d.group_size, d.w_type, d.zp_type, d.flags);
+}
+
+static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_split, int n_cus) {
+    ovfcc::FcDeviceArgs a{};
+    a.M = M, a.N = d.N, a.K = d.K, a.group_size = d.group_size, a.w_type = d.w_type, a.zp_type = d.zp_type;
+    a.layout = ovfcc::make_layout(d);
+    a.N_out = a.layout.glu ? d.N / 2 : d.N;
+    const ovfcc::Layout& L = a.layout;
+    ovfcc::LaunchPlan p;
+    const int rc = ovfcc::plan_launch(a, force, force_split, n_cus, &p);
+    if (rc != 0)
+        return;  // refusals are legitimate; the API turns them into errors or falls back
+    char what[160];
+    std::snprintf(what, sizeof(what), "%s M=%ld N=%ld K=%ld G=%ld bits=%d glu=%d force=%d/%d", p.name, (long)M, (long)d.N,
+                  (long)d.K, (long)d.group_size, L.bits, L.glu, force, force_split);
+    CHECK(p.grid[0] >= 1 && p.grid[1] >= 1 && p.grid[2] >= 1, "%s", what);
+    CHECK((uint64_t)p.grid[0] * p.grid[1] * p.grid[2] < (1ull << 31) && p.grid[1] < 65536 && p.grid[2] < 65536, "%s", what);
+    CHECK(p.block >= 64 && p.block <= 1024 && p.block % 64 == 0, "%s block=%u", what, p.block);
+    CHECK(p.dynamic_lds <= 160 * 1024, "%s lds=%u", what, p.dynamic_lds);
+    CHECK(p.split_k >= 1, "%s", what);
+    CHECK((p.split_k > 1) == (p.workspace_bytes > 0) && (p.split_k > 1) == (p.counter_count > 0), "%s ws=%zu counters=%zu split=%d",
+          what, p.workspace_bytes, p.counter_count, p.split_k);
+    if (p.kernel == OVFCC_KERNEL_PLAIN) {
+        CHECK(!L.tiled && p.grid[0] == (unsigned)a.N_out && p.grid[1] == (unsigned)M, "%s", what);
+        return;
+    }
+    CHECK(L.tiled, "%s", what);
+    const int kb = (int)L.k_blocks;
+    if (p.kernel == OVFCC_KERNEL_DECODE || p.async_dma) {
+        CHECK((int64_t)p.split_k * p.kblocks_per_split >= kb, "%s split=%d per=%d kb=%d", what, p.split_k, p.kblocks_per_split, kb);
+        CHECK((int64_t)(p.split_k - 1) * p.kblocks_per_split < kb, "%s empty split: split=%d per=%d kb=%d", what, p.split_k,
+              p.kblocks_per_split, kb);
+    }
+    if (p.kernel == OVFCC_KERNEL_DECODE) {
+        CHECK(M <= ovfcc::kDecodeMaxRows, "%s", what);
+        const int nw = (int)p.block / 64, rt = p.tiles_per_group;
+        if (p.batch) {
+            const int mt = (int)(M + 15) / 16;
+            CHECK(p.tile_m == 16 * mt && (rt == 1 || rt == 2), "%s", what);
+            CHECK((int64_t)p.grid[0] * nw * rt >= L.n_tiles && p.grid[1] == (unsigned)p.split_k, "%s", what);
+            CHECK(p.dynamic_lds <= 96 * 1024 && p.dynamic_lds == (unsigned)(16 * mt * ((size_t)p.kblocks_per_split * 128 + 8) * 2),
+                  "%s lds=%u", what, p.dynamic_lds);
+            CHECK(p.workspace_bytes == (p.split_k > 1 ? (size_t)p.grid[0] * p.split_k * nw * rt * mt * 1024 : 0), "%s", what);
+            if (L.glu)  // gate and up tile in one wave, or in neighbouring waves with room for the hand-over
+                CHECK((rt == 2 || nw % 2 == 0) && p.dynamic_lds >= (unsigned)(nw / 2) * p.tile_m * 64u, "%s", what);
+        } else {
+            CHECK(M <= 32 && (int64_t)p.grid[0] * rt == L.n_tiles && p.grid[1] == (unsigned)p.split_k, "%s rt=%d", what, rt);
+            CHECK(!L.glu || (p.x_in_lds && rt % 2 == 0 && M <= 16), "%s rt=%d xlds=%d", what, rt, (int)p.x_in_lds);
+            CHECK(p.dynamic_lds <= 64 * 1024, "%s lds=%u", what, p.dynamic_lds);
+        }
+        return;
+    }
+    CHECK(d.N % 128 == 0, "%s", what);
+    if (p.async_dma) {
+        const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
+        CHECK(L.bits == 4 && d.N % 256 == 0 && p.tiles_x == d.N / 256 && p.tiles_y == (M + 127) / 128, "%s", what);
+        CHECK(p.full_tiles >= 0 && p.full_tiles <= tiles && (p.split_k > 1 || p.full_tiles == tiles), "%s full=%d", what, p.full_tiles);
+        CHECK(p.grid[0] == (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) && p.grid[1] == 1 && p.grid[2] == 1, "%s", what);
+        CHECK(p.workspace_bytes == (p.split_k > 1 ? (size_t)(tiles - p.full_tiles) * p.split_k * 128 * 256 * 4 : 0), "%s", what);
+        CHECK(M * d.K * 2 < (1ll << 31), "%s", what);
+    } else {
+        CHECK(p.split_k == 1, "%s", what);
+        CHECK(p.grid[0] == (unsigned)(d.N / p.tile_n) && p.grid[1] == (unsigned)((M + 127) / 128), "%s", what);
+        CHECK(p.tile_n == 128 || (d.N % 256 == 0 && (p.direct || d.K % 256 == 0)), "%s", what);
+    }
+}
+
+int main() {
+    std::mt19937 rng(12345);
+    const int64_t Ns[] = {16, 32, 48, 96, 128, 256, 272, 1024, 4096, 14336};
+    const int64_t Ks[] = {128, 256, 384, 1024, 4096, 14336};
+    const int64_t Ms[] = {1, 2, 4, 5, 15, 16, 17, 31, 32, 33, 47, 48, 49, 127, 128, 129, 300, 2048, 8192};
+    const int types[] = {OVFCC_U4, OVFCC_I4, OVFCC_U8, OVFCC_I8};
+    const int flags[] = {0, OVFCC_GLU_SWISH, OVFCC_GLU_GELU | OVFCC_GLU_GATE_SECOND};
+    int plans = 0;
+    for (int64_t N : Ns)
+        for (int64_t K : Ks)
+            for (int64_t G : {(int64_t)128, K})
+                for (int t : types)
+                    for (int fl : flags) {
+                        const int zp = (t == OVFCC_U4) ? OVFCC_U4 : (t == OVFCC_U8 ? OVFCC_U8 : OVFCC_NONE);
+                        const ovfcc_fc_desc d = desc(N, K, G, t, zp, fl);
+                        if (ovfcc::validate_desc(&d) != 0)
+                            continue;
+                        if (N <= 1024 && K <= 1024)
+                            round_trip(d, rng);
+                        for (int64_t M : Ms)
+                            for (int force : {OVFCC_KERNEL_AUTO, OVFCC_KERNEL_DECODE, OVFCC_KERNEL_PREFILL})
+                                for (int split : {0, 1, 3, 8, 64})
+                                    for (int cus : {256, 64}) {
+                                        check_plan(d, M, force, split, cus);
+                                        ++plans;
+                                    }
+                    }
+    // untiled shapes: plain kernel only
+    for (int fl : flags) {
+        const ovfcc_fc_desc d = desc(40, 200, 50, OVFCC_U4, OVFCC_U4, fl);
+        CHECK(ovfcc::validate_desc(&d) == 0 && !ovfcc::make_layout(d).tiled, "untiled");
+        for (int64_t M : Ms)
+            check_plan(d, M, OVFCC_KERNEL_AUTO, 0, 256);
+    }
+    // the gate refuses what the kernels cannot index
+    ovfcc_fc_desc bad = desc(64, 256, 96, OVFCC_U4, OVFCC_NONE, 0);
+    CHECK(ovfcc::validate_desc(&bad) != 0, "group size must divide K");
+    bad = desc(63, 256, 128, OVFCC_U4, OVFCC_NONE, OVFCC_GLU_SWISH);
+    CHECK(ovfcc::validate_desc(&bad) != 0, "odd N with a gated linear unit");
+    std::printf("%d plans checked, %d failures\n", plans, g_failures);
+    return g_failures ? 1 : 0;
+}
