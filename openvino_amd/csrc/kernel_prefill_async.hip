@@ -40,7 +40,7 @@
 
 namespace ovfcc {
 
-constexpr int PA_BM = 128, PA_BN = 256, PA_BK = 128;
+constexpr int PA_BM = 128, PA_BN = 256, PA_BK = 128;  // PA_BM: rows of the full tile (NT = 8 row tiles of 16)
 constexpr int PA_STAGES = 3;
 constexpr int PA_XQ = 3;  // activation operands in registers: the one in use and PA_XQ - 1 on their way from LDS
 constexpr int PA_A_BYTES = PA_BM * PA_BK * 2;  // 32 KiB per stage
@@ -62,7 +62,7 @@ struct AsyncWork {
 // is a little more than a multiple of the compute units ends with a full round of shorter workgroups instead
 // of a mostly idle round of whole tiles.  full_tiles = 0 splits every tile (few tiles, long K).
 __device__ __forceinline__ AsyncWork async_work(int tiles_x, int tiles_y, int full_tiles, int tail_split,
-                                                int kb_per_split, int kb_total) {
+                                                int kb_per_split, int kb_total, int tile_rows) {
     AsyncWork wk;
     const int L = (int)blockIdx.x;
     int slot;
@@ -74,21 +74,24 @@ __device__ __forceinline__ AsyncWork async_work(int tiles_x, int tiles_y, int fu
         wk.kb_lo = wk.z * kb_per_split, wk.kb_hi = min(kb_total, wk.kb_lo + kb_per_split);
         wk.park_slot = j % tail;
     }
-    xcd_tile_at((unsigned)slot, (unsigned)tiles_x, (unsigned)tiles_y, wk.tile_x, wk.tile_y, 2 * PA_BM, PA_BN / 2);
-    wk.m0 = wk.tile_y * PA_BM;
+    xcd_tile_at((unsigned)slot, (unsigned)tiles_x, (unsigned)tiles_y, wk.tile_x, wk.tile_y, 2 * tile_rows, PA_BN / 2);
+    wk.m0 = wk.tile_y * tile_rows;
     return wk;
 }
 
 // The whole kernel for one workgroup's share of one node.  The two kernels below differ only in where the node's
 // operands come from.
-template <bool ZP_TABLE, bool PRESCALE>
+template <bool ZP_TABLE, bool PRESCALE, int NT>
 __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
                                                    const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
                                                    const half_t* __restrict__ bias, void* __restrict__ y,
                                                    float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N,
                                                    int K, int kb_total, int kb_per_group, int ng, int zp_const,
                                                    int out_f32, int glu, const AsyncWork wk) {
+    static_assert(NT == 8 || NT == 4, "tiles of 128 or 64 rows");
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
+    constexpr int AL = NT / 2;                          // activation loads per wave and k-block
+    constexpr int S = 4 * NT;                           // MFMA slots per step (a wave's two steps make a k-block)
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
 
@@ -118,13 +121,14 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     // row 4 i + (lane >> 4) of those, LDS slot lane & 15 of that row, which holds global chunk
     // (lane & 15) ^ (row & 15).  Rows >= M lie beyond the descriptor's range and arrive as zeros.
     // (row & 15 = 4 i + (lane >> 4) = 4 i ^ (lane >> 4), so the chunk of load i is c0 ^ 4 i.) ----
-    const unsigned a_row0 = (unsigned)((m0 + 16 * wave + (lane >> 4)) * K) * 2u;
-    const unsigned a_c0 = (unsigned)((lane & 15) ^ (lane >> 4));
+    // (64-row tiles: two loads per wave, rows 8 wave + 4 i + (lane >> 4); row & 15 = 8 (wave & 1) ^ 4 i ^ (lane >> 4).)
+    const unsigned a_row0 = (unsigned)((m0 + 4 * AL * wave + (lane >> 4)) * K) * 2u;
+    const unsigned a_c0 = (unsigned)((lane & 15) ^ (lane >> 4) ^ (NT == 4 ? 8 * (wave & 1) : 0));
     auto dma_a = [&](int kb, int stage, int i) {
         const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(4 * i * K + kb * PA_BK) * 2u);
         const unsigned voff = a_row0 + sterm + ((a_c0 ^ (unsigned)(4 * i)) << 4);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void_ptr)(lds3 + stage * PA_A_BYTES + (4 * wave + i) * 1024), 16,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void_ptr)(lds3 + stage * PA_A_BYTES + (AL * wave + i) * 1024), 16,
                                                  voff | oob, 0, 0, 0);
     };
     // ---- weights: the wave copies tiles 2 wave, 2 wave + 1 of the workgroup's 16 ----
@@ -151,11 +155,11 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                                                      ((tile * ng + g) * 16u + (lane & 3) * 4u) | oob, 0, 0, 0);
         }
     };
-    // Per k-block a wave issues, in this order: 4 activation loads (for k-block + 2), then 2 weight loads and at
-    // most one parameter load (for k-block + 3).  The wait at the top of a k-block needs the activations of this
-    // k-block and the weights and parameters of the next; the instructions issued after those are one k-block's
-    // worth, at least 6.
-    constexpr int kWaitTop = 6;
+    // Per k-block a wave issues, in this order: AL (4 or 2) activation loads (for k-block + 2), then 2 weight
+    // loads and at most one parameter load (for k-block + 3).  The wait at the top of a k-block needs the
+    // activations of this k-block and the weights and parameters of the next; the instructions issued after those
+    // are one k-block's worth, at least AL + 2.
+    constexpr int kWaitTop = AL + 2;
 
     // ---- the wave's share of a staged k-block of weights: 8 bytes per tile, plus scale and zero-point ----
     typedef __attribute__((address_space(3))) const uint2_t* lds_u2_ptr;
@@ -209,11 +213,11 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
         }
     };
 
-    float4_t acc[4][8];  // [channel tile][row tile]
+    float4_t acc[4][NT];  // [channel tile][row tile]
 #pragma unroll
     for (int r = 0; r < 4; ++r)
 #pragma unroll
-        for (int t = 0; t < 8; ++t)
+        for (int t = 0; t < NT; ++t)
             acc[r][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // One k-block: 64 MFMAs -- step 0 with operand wf0 while the unpack of (par_a, dword 1) fills wf1, then
@@ -225,35 +229,35 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
         // operand of row tile t and step js: row 16 t + col, chunk (4 (2 kg + js) + kq) ^ col
         const lds_byte_ptr xa0 = lds3 + stage * PA_A_BYTES + col * 256 + (((8 * kg + kq) ^ col) << 4);
         const lds_byte_ptr xa1 = lds3 + stage * PA_A_BYTES + col * 256 + (((8 * kg + 4 + kq) ^ col) << 4);
-        auto x_at = [&](int tt) { return *(lds_frag_ptr)((tt < 8 ? xa0 : xa1) + (tt & 7) * 16 * 256); };
+        auto x_at = [&](int tt) { return *(lds_frag_ptr)((tt < NT ? xa0 : xa1) + (tt % NT) * 16 * 256); };
         half8_t xq[PA_XQ];
 #pragma unroll
         for (int tt = 0; tt < PA_XQ - 1; ++tt)
             xq[tt] = x_at(tt);
         auto slot = [&](int i) {
-            const int tt = i >> 2, r = i & 3;  // tt = 8 js + t
-            if (r == 0 && tt + PA_XQ - 1 < 16)
+            const int tt = i >> 2, r = i & 3;  // tt = NT js + t
+            if (r == 0 && tt + PA_XQ - 1 < 2 * NT)
                 xq[(tt + PA_XQ - 1) % PA_XQ] = x_at(tt + PA_XQ - 1);
-            const int t = tt & 7;
-            if (i < 32) {
+            const int t = tt % NT;
+            if (i < S) {
                 acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf0[r].v, xq[tt % PA_XQ], acc[r][t], 0, 0, 0);
 #pragma unroll
-                for (int g = i * 4 * NOPS / 32; g < (i + 1) * 4 * NOPS / 32; ++g)
+                for (int g = i * 4 * NOPS / S; g < (i + 1) * 4 * NOPS / S; ++g)
                     unpack_op(par_a, g / NOPS, 1, g % NOPS, wf1[g / NOPS]);
             } else {
                 acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf1[r].v, xq[tt % PA_XQ], acc[r][t], 0, 0, 0);
 #pragma unroll
-                for (int g = (i - 32) * 4 * NOPS / 32; g < (i - 31) * 4 * NOPS / 32; ++g)
+                for (int g = (i - S) * 4 * NOPS / S; g < (i - S + 1) * 4 * NOPS / S; ++g)
                     unpack_op(par_b, g / NOPS, 0, g % NOPS, wf0[g / NOPS]);
             }
             mem(i);
             __builtin_amdgcn_sched_barrier(0);
         };
 #pragma unroll
-        for (int i = 0; i < 32; ++i)
+        for (int i = 0; i < S; ++i)
             slot(i);
 #pragma unroll
-        for (int i = 32; i < 64; ++i)
+        for (int i = S; i < 2 * S; ++i)
             slot(i);
     };
 
@@ -262,7 +266,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < AL; ++i)
             dma_a(kb_lo + j, j, i);
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
@@ -306,17 +310,17 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             // request the weights and parameters of k-block kb + 3 into the stage those of k-block kb used
             // (every wave read them before the barrier above).
             block(s0, wf0, wf1, u, u ^ 1, [&](int i) {
-                if (i < 32 && (i & 7) == 2)
+                if (i < S && (i & 7) == 2)
                     dma_a(kb + 2, s2, i >> 3);
-                if (i >= 24 && i < 28)
-                    read_p(u ^ 1, s1, i - 24);
-                if (i >= 28 && i < 32)
-                    read_w(u ^ 1, s1, i - 28);
-                if (i == 36)
+                if (i >= S - 8 && i < S - 4)
+                    read_p(u ^ 1, s1, i - (S - 8));
+                if (i >= S - 4 && i < S)
+                    read_w(u ^ 1, s1, i - (S - 4));
+                if (i == S + 4)
                     dma_w(kb + 3, s0, 0);
-                if (i == 52)
+                if (i == S + 4 + S / 2)
                     dma_w(kb + 3, s0, 1);
-                if (i == 44 && has_p)
+                if (i == S + 4 + S / 4 && has_p)
                     dma_p(kb + 3, s0);
             });
             s0 = s1;
@@ -335,7 +339,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     __shared__ unsigned ticket_s;
     // parked tile layout: [tile][split][wn][channel tile r][row tile t][lane] float4
     constexpr int kAuxDeviceScope = 16;              // sc1: write through to / read from memory shared by all XCDs
-    constexpr unsigned kParkBytes = 4 * 32 * 64 * 16;  // one workgroup's f32 tile
+    constexpr unsigned kParkBytes = 4 * (4 * NT) * 64 * 16;  // one workgroup's f32 tile
     const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(
         reinterpret_cast<char*>(ws) + (size_t)tile_id * split_k * kParkBytes, 0, split_k * (int)kParkBytes, kRsrcFlags);
     auto finish = [&](int r, int t, float4_t v, const float (&sc)[4], const float (&bs)[4]) {
@@ -395,9 +399,9 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
 #pragma unroll
             for (int r2 = 0; r2 < 2; ++r2)
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
+                for (int t = 0; t < NT; ++t) {
                     const float4_t v = acc[2 * hh + r2][t];
-                    float* p = ex + ((wn * 64 + (r2 * 8 + t) * 4) * 64) + lane;
+                    float* p = ex + ((wn * 8 * NT + (r2 * NT + t) * 4) * 64) + lane;
                     p[0] = v.x, p[64] = v.y, p[128] = v.z, p[192] = v.w;
                 }
         }
@@ -407,9 +411,9 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             channel_params(2 * hh, scg, bsg);
             channel_params(2 * hh + 1, scu, bsu);
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                const float* pg = ex + ((wn * 64 + t * 4) * 64) + lane;
-                const float* pu = ex + ((wn * 64 + (8 + t) * 4) * 64) + lane;
+            for (int t = 0; t < NT; ++t) {
+                const float* pg = ex + ((wn * 8 * NT + t * 4) * 64) + lane;
+                const float* pu = ex + ((wn * 8 * NT + (NT + t) * 4) * 64) + lane;
                 const float4_t a = acc[2 * hh][t], b = acc[2 * hh + 1][t];
                 finish_glu(hh, t, float4_t{a.x + pg[0], a.y + pg[64], a.z + pg[128], a.w + pg[192]},
                            float4_t{b.x + pu[0], b.y + pu[64], b.z + pu[128], b.w + pu[192]}, scg, bsg, scu, bsu);
@@ -421,8 +425,8 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                 float sc[4], bs[4];
                 channel_params(r, sc, bs);
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const float* p = ex + ((wn * 64 + (r2 * 8 + t) * 4) * 64) + lane;
+                for (int t = 0; t < NT; ++t) {
+                    const float* p = ex + ((wn * 8 * NT + (r2 * NT + t) * 4) * 64) + lane;
                     const float4_t a = acc[r][t];
                     const float4_t v = float4_t{a.x + p[0], a.y + p[64], a.z + p[128], a.w + p[192]};
                     if (split_k == 1)
@@ -430,7 +434,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                     else
                         __builtin_amdgcn_raw_buffer_store_b128(
                             __builtin_bit_cast(uint4_t, v), rp,
-                            wk.z * kParkBytes + (unsigned)(((wn * 4 + r) * 8 + t) * 64 + lane) * 16u, 0,
+                            wk.z * kParkBytes + (unsigned)(((wn * 4 + r) * NT + t) * 64 + lane) * 16u, 0,
                             kAuxDeviceScope);
                 }
             }
@@ -452,7 +456,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             const float4_t pz = __builtin_bit_cast(
                 float4_t,
                 __builtin_amdgcn_raw_buffer_load_b128(
-                    rp, z * kParkBytes + (unsigned)(((wn * 4 + r) * 8 + t) * 64 + lane) * 16u, 0, kAuxDeviceScope));
+                    rp, z * kParkBytes + (unsigned)(((wn * 4 + r) * NT + t) * 64 + lane) * 16u, 0, kAuxDeviceScope));
             v.x += pz.x, v.y += pz.y, v.z += pz.z, v.w += pz.w;
         }
         return v;
@@ -464,7 +468,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             channel_params(2 * j, scg, bsg);
             channel_params(2 * j + 1, scu, bsu);
 #pragma unroll
-            for (int t = 0; t < 8; ++t)
+            for (int t = 0; t < NT; ++t)
                 finish_glu(j, t, parked_sum(2 * j, t), parked_sum(2 * j + 1, t), scg, bsg, scu, bsu);
         }
     } else if (kg == 0) {
@@ -473,7 +477,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             float sc[4], bs[4];
             channel_params(r, sc, bs);
 #pragma unroll
-            for (int t = 0; t < 8; ++t)
+            for (int t = 0; t < NT; ++t)
                 finish(r, t, parked_sum(r, t), sc, bs);
         }
     }
@@ -481,7 +485,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
         __hip_atomic_store(counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <bool ZP_TABLE, bool PRESCALE>
+template <bool ZP_TABLE, bool PRESCALE, int NT>
 __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* __restrict__ wt,
                                                                 const half_t* __restrict__ st,
                                                                 const uint8_t* __restrict__ zt,
@@ -492,15 +496,15 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
                                                                 int kb_total, int kb_per_group, int ng, int zp_const,
                                                                 int out_f32, int glu, int tiles_x, int tiles_y,
                                                                 int full_tiles, int tail_split, int kb_per_split) {
-    const AsyncWork wk = async_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total);
-    prefill_async_body<ZP_TABLE, PRESCALE>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
+    const AsyncWork wk = async_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT);
+    prefill_async_body<ZP_TABLE, PRESCALE, NT>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
                                            zp_const, out_f32, glu, wk);
 }
 
 // Grouped launch: tile row tile_y is item tile_y of the table, a node of the common shape and format with at most
 // 128 rows of its own (the experts of a mixture-of-experts layer over their gathered rows).  Workgroups of one
 // item sit together in a super-tile and share its activations in L2.
-template <bool ZP_TABLE, bool PRESCALE>
+template <bool ZP_TABLE, bool PRESCALE, int NT>
 __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const BatchGroupTable tab,
                                                                         float* __restrict__ ws,
                                                                         unsigned* __restrict__ counters, int N, int K,
@@ -508,12 +512,12 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const Ba
                                                                         int zp_const, int out_f32, int glu,
                                                                         int tiles_x, int tiles_y, int full_tiles,
                                                                         int tail_split, int kb_per_split) {
-    AsyncWork wk = async_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total);
+    AsyncWork wk = async_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT);
     const BatchGroupItem& it = tab.item[wk.tile_y];
     if (it.M <= 0)
         return;
     wk.m0 = 0;
-    prefill_async_body<ZP_TABLE, PRESCALE>((const uint4_t*)it.w, (const half_t*)it.scale, (const uint8_t*)it.zp,
+    prefill_async_body<ZP_TABLE, PRESCALE, NT>((const uint4_t*)it.w, (const half_t*)it.scale, (const uint8_t*)it.zp,
                                            (const half_t*)it.x, (const half_t*)it.bias, it.y, ws, counters, it.M, N, K,
                                            kb_total, kb_per_group, ng, zp_const, out_f32, glu, wk);
 }
@@ -533,16 +537,16 @@ static int allow_lds(Kern kern, bool* done) {
 // remaining tile, parts that cover K.
 static bool async_plan_ok(const FcDeviceArgs& a, const LaunchPlan& p) {
     const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
-    return p.tiles_x == a.N / PA_BN && p.tiles_y >= 1 && p.full_tiles >= 0 && p.full_tiles <= tiles && p.split_k >= 1 &&
+    return (p.tile_m == PA_BM || p.tile_m == PA_BM / 2) && p.tiles_x == a.N / PA_BN && p.tiles_y >= 1 && p.full_tiles >= 0 && p.full_tiles <= tiles && p.split_k >= 1 &&
            (int64_t)p.kblocks_per_split * p.split_k >= a.layout.k_blocks && (p.full_tiles == tiles || p.kblocks_per_split >= 1) &&
            p.grid[0] == (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) && p.grid[1] == 1 && p.grid[2] == 1 &&
            (p.split_k == 1 || (a.workspace && a.counters));
 }
 
-template <bool ZPT, bool PRE>
+template <bool ZPT, bool PRE, int NT>
 static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_prefill_async_kernel<ZPT, PRE>;
+    auto kern = fcc_prefill_async_kernel<ZPT, PRE, NT>;
     static bool attr_set = false;  // per instantiation
     if (int e = allow_lds(kern, &attr_set))
         return e;
@@ -554,11 +558,11 @@ static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
     return (int)hipGetLastError();
 }
 
-template <bool ZPT, bool PRE>
+template <bool ZPT, bool PRE, int NT>
 static int launch_async_grouped_impl(const BatchGroupTable& tab, const FcDeviceArgs& a, const LaunchPlan& p,
                                      hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_prefill_async_grouped_kernel<ZPT, PRE>;
+    auto kern = fcc_prefill_async_grouped_kernel<ZPT, PRE, NT>;
     static bool attr_set = false;  // per instantiation
     if (int e = allow_lds(kern, &attr_set))
         return e;
@@ -569,17 +573,24 @@ static int launch_async_grouped_impl(const BatchGroupTable& tab, const FcDeviceA
     return (int)hipGetLastError();
 }
 
+// dispatch on zero-point table, per-group scales and tile height
+#define OVFCC_ASYNC_DISPATCH(FN, ...)                                                                    \
+    (L.groups == 1 ? (L.zp_table ? (nt8 ? FN<true, false, 8>(__VA_ARGS__) : FN<true, false, 4>(__VA_ARGS__))    \
+                                 : (nt8 ? FN<false, false, 8>(__VA_ARGS__) : FN<false, false, 4>(__VA_ARGS__)))  \
+                   : (L.zp_table ? (nt8 ? FN<true, true, 8>(__VA_ARGS__) : FN<true, true, 4>(__VA_ARGS__))      \
+                                 : (nt8 ? FN<false, true, 8>(__VA_ARGS__) : FN<false, true, 4>(__VA_ARGS__))))
+
 int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
-    if (L.bits != 4 || !async_plan_ok(a, p))
-        return (int)hipErrorInvalidValue;  // the planner sends 8-bit nodes to the register-ring kernel
-    if (L.groups == 1)
-        return L.zp_table ? launch_async_impl<true, false>(a, p, s) : launch_async_impl<false, false>(a, p, s);
-    return L.zp_table ? launch_async_impl<true, true>(a, p, s) : launch_async_impl<false, true>(a, p, s);
+    // (the planner sends 8-bit nodes to the register-ring kernel)
+    if (L.bits != 4 || !async_plan_ok(a, p) || (int64_t)p.tiles_y * p.tile_m < a.M)
+        return (int)hipErrorInvalidValue;
+    const bool nt8 = p.tile_m == PA_BM;
+    return OVFCC_ASYNC_DISPATCH(launch_async_impl, a, p, s);
 }
 
-// p plans one node of n_items * 128 rows: its grid rows are the items of the table.
+// p plans one node of n_items * tile_m rows: its tile rows are the items of the table.
 int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
                                  void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -587,13 +598,11 @@ int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const 
     if (L.bits != 4 || !async_plan_ok(a, p) || n_items < 1 || n_items > kMaxGroupItems || p.tiles_y != n_items)
         return (int)hipErrorInvalidValue;
     for (int i = 0; i < n_items; ++i)
-        if (tab.item[i].M < 1 || tab.item[i].M > PA_BM)
+        if (tab.item[i].M < 1 || tab.item[i].M > p.tile_m)
             return (int)hipErrorInvalidValue;
-    if (L.groups == 1)
-        return L.zp_table ? launch_async_grouped_impl<true, false>(tab, a, p, s)
-                          : launch_async_grouped_impl<false, false>(tab, a, p, s);
-    return L.zp_table ? launch_async_grouped_impl<true, true>(tab, a, p, s)
-                      : launch_async_grouped_impl<false, true>(tab, a, p, s);
+    const bool nt8 = p.tile_m == PA_BM;
+    return OVFCC_ASYNC_DISPATCH(launch_async_grouped_impl, tab, a, p, s);
 }
+#undef OVFCC_ASYNC_DISPATCH
 
 }  // namespace ovfcc

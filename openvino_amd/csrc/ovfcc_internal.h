@@ -83,6 +83,7 @@ struct FcDeviceArgs {
     int out_f32;         // output_type f32 instead of f16
     int64_t N_out;       // row length of y: N, or N / 2 with a gated-linear-unit epilogue
     int gate_offset, up_offset;  // untiled layout with such an epilogue: first gate / up channel
+    int tile_rows = 0;   // async prefill kernel: 64 or 128 forces the tile height, 0 leaves it to the planner
     Layout layout;
 };
 

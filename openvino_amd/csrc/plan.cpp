@@ -187,6 +187,19 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.tile_n = wide ? kPrefillWideN : kPrefillTileN;
         p.grid[0] = (unsigned)(a.N / p.tile_n);
         p.grid[1] = (unsigned)m_tiles;
+        if (p.async_dma) {
+            // 64-row tiles while they still fit the compute units in one round: a 64-row tile takes two thirds of
+            // the time of a 128-row tile (same weight traffic and unpack work, half the MFMAs), so it pays only
+            // where 128-row tiles would leave half the chip idle.  (OVFCC_PREFILL_ROWS = 64 | 128 overrides;
+            // a.tile_rows, set by the grouped run, wins over both.)
+            int rows = env_int("OVFCC_PREFILL_ROWS", (int64_t)p.grid[0] * ((a.M + 63) / 64) <= n_cus ? 64 : 128);
+            if (a.tile_rows == 64 || a.tile_rows == 128)
+                rows = a.tile_rows;
+            if (rows == 64) {
+                p.tile_m = 64;
+                p.grid[1] = (unsigned)((a.M + 63) / 64);
+            }
+        }
         p.kblocks_per_split = (int)L.k_blocks;
         if (p.async_dma) {
             // Split K while the tiles alone leave compute units idle (at least eight k-blocks per workgroup): the
@@ -222,7 +235,7 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             p.full_tiles = (int)full;
             p.grid[0] = (unsigned)(full + (tiles - full) * split);
             p.grid[1] = 1;
-            p.workspace_bytes = split > 1 ? (size_t)(tiles - full) * split * kPrefillTileM * kPrefillWideN * sizeof(float) : 0;
+            p.workspace_bytes = split > 1 ? (size_t)(tiles - full) * split * p.tile_m * kPrefillWideN * sizeof(float) : 0;
             p.counter_count = split > 1 ? (size_t)(tiles - full) : 0;
         }
         p.block = wide ? 512 : 256;

@@ -111,10 +111,11 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     CHECK(d.N % 128 == 0, "%s", what);
     if (p.async_dma) {
         const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
-        CHECK(L.bits == 4 && d.N % 256 == 0 && p.tiles_x == d.N / 256 && p.tiles_y == (M + 127) / 128, "%s", what);
+        CHECK(p.tile_m == 128 || p.tile_m == 64, "%s tile_m=%d", what, p.tile_m);
+        CHECK(L.bits == 4 && d.N % 256 == 0 && p.tiles_x == d.N / 256 && p.tiles_y == (M + p.tile_m - 1) / p.tile_m, "%s", what);
         CHECK(p.full_tiles >= 0 && p.full_tiles <= tiles && (p.split_k > 1 || p.full_tiles == tiles), "%s full=%d", what, p.full_tiles);
         CHECK(p.grid[0] == (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) && p.grid[1] == 1 && p.grid[2] == 1, "%s", what);
-        CHECK(p.workspace_bytes == (p.split_k > 1 ? (size_t)(tiles - p.full_tiles) * p.split_k * 128 * 256 * 4 : 0), "%s", what);
+        CHECK(p.workspace_bytes == (p.split_k > 1 ? (size_t)(tiles - p.full_tiles) * p.split_k * p.tile_m * 256 * 4 : 0), "%s", what);
         CHECK(M * d.K * 2 < (1ll << 31), "%s", what);
     } else {
         CHECK(p.split_k == 1, "%s", what);

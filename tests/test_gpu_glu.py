@@ -68,12 +68,17 @@ def test_glu_every_row_count(oracle, dev, req, wt, zt, N, K, G, bias, kind, seco
         w.close()
 
 
-@pytest.mark.parametrize("variant", ["async", "ring", "lds"])
+@pytest.mark.parametrize("variant", ["async", "async128", "ring", "lds"])
 @pytest.mark.parametrize("wt,zt,N,K,G,kind", [("u4", "u4", 512, 1024, 128, "swish"), ("i4", "none", 512, 512, 512, "gelu"),
                                              ("u8", "u8", 512, 512, 128, "swish"), ("u8", "none", 256, 512, 512, "gelu_tanh")])
 def test_glu_256_wide_prefill_kernels(oracle, dev, req, monkeypatch, wt, zt, N, K, G, kind, variant):
     """The three prefill kernels with 128 x 256 tiles, forced on small shapes (the planner would pick the square one)."""
     monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    if variant == "async128":     # the planner gives grids this small 64-row tiles; cover the 128-row form too
+        if wt[1] == "8":
+            pytest.skip("8-bit nodes run the register-ring kernel")
+        monkeypatch.setenv("OVFCC_PREFILL_ROWS", "128")
+        variant = "async"
     if variant == "ring":
         monkeypatch.setenv("OVFCC_PREFILL_ASYNC", "0")
     if variant == "lds":

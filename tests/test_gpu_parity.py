@@ -218,7 +218,7 @@ def test_both_decode_kernels_every_row_count(oracle, dev, req, monkeypatch, wt, 
         w.close()
 
 
-@pytest.mark.parametrize("variant", ["async", "ring", "lds"])
+@pytest.mark.parametrize("variant", ["async", "async64", "ring", "lds"])
 @pytest.mark.parametrize("wt,zt,N,K,G,out", [
     ("u4", "u4", 256, 512, 128, "f16"), ("i4", "none", 512, 1024, 256, "f16"), ("u4", "u8", 256, 768, 128, "f32"),
     ("u4", "none", 256, 512, 512, "f16"),            # one group per channel: exact integers, scale in the epilogue
@@ -231,22 +231,31 @@ def test_256_wide_prefill_kernels_small_shapes(oracle, dev, req, monkeypatch, wt
     onto shapes small enough for the oracle to cover every output: every weight type, zero-point form, scale
     grouping, bias, both output types, row counts that leave the last row tile ragged, odd k-block counts."""
     four_bit = wt in ("u4", "i4")
-    if variant == "async" and not four_bit:
+    if variant.startswith("async") and not four_bit:
         pytest.skip("the all-asynchronous kernel takes 4-bit weights; 8-bit nodes run the register-ring kernel")
     monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
     monkeypatch.setenv("OVFCC_PREFILL_DIRECT", "0" if variant == "lds" else "1")
-    monkeypatch.setenv("OVFCC_PREFILL_ASYNC", "1" if variant == "async" else "0")
+    monkeypatch.setenv("OVFCC_PREFILL_ASYNC", "1" if variant.startswith("async") else "0")
+    monkeypatch.setenv("OVFCC_PREFILL_ROWS", "64" if variant == "async64" else "128")   # tile height of the async kernel
     c = datagen.make_case(51, 300, K, N, wt, G, zt, with_bias=True)
     w = fc.CompressedWeights.from_case(dev, c, output_type=out)
     ref = oracle_y(oracle, c)
-    want = {"async": "fcc_prefill_async", "ring": "fcc_prefill_direct", "lds": "fcc_prefill_wide"}[variant]
+    want = {"async": "fcc_prefill_async", "async64": "fcc_prefill_async", "ring": "fcc_prefill_direct",
+            "lds": "fcc_prefill_wide"}[variant]
     try:
-        for M in (129, 256, 300):
+        for M in (129, 256, 300) + ((49, 64, 65) if variant == "async64" else ()):
             say(f"256-wide prefill {variant} {wt}/{zt} N={N} K={K} G={G} out={out} M={M}")
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
+            if M <= 128:
+                req.force_kernel(_lib.KERNEL_PREFILL)      # the policy would cut these rows into decode launches
+                y = req.infer(w, c.x[:M])
+                info = req.last_kernel()
+                req.force_kernel()
             if variant != "lds" or K % 256 == 0:
                 assert info["name"].startswith(want), info
+            if variant.startswith("async"):
+                assert info["tile_m"] == (64 if variant == "async64" else 128), info
             # grouped scales: these kernels round (q - zp) * s once to f16, an error of the same size as the
             # rounding of an f16 output, so the slack applies to the f32 output as well
             check_parity(oracle, y, ref[:M], K, f"{info}", output_rounding_slack=True)
@@ -257,11 +266,13 @@ def test_256_wide_prefill_kernels_small_shapes(oracle, dev, req, monkeypatch, wt
 @pytest.mark.parametrize("wt,zt,N,K,G", [("i4", "none", 256, 2048, 128), ("u4", "u4", 512, 1280, 256),
                                          ("u4", "none", 256, 1024, 1024)])
 @pytest.mark.parametrize("split", [2, 3, 8])
-def test_prefill_split_k_is_deterministic(oracle, dev, req, monkeypatch, wt, zt, N, K, G, split):
+@pytest.mark.parametrize("rows", ["128", "64"])
+def test_prefill_split_k_is_deterministic(oracle, dev, req, monkeypatch, wt, zt, N, K, G, split, rows):
     """The 4-bit register-fed prefill kernel with K split over workgroups: any split gives the oracle's answer
     (ragged last split, ragged last row tile, bias, per-channel scale in the fix-up), repeated launches give
     identical bits, and the arrival counters return to zero."""
     monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    monkeypatch.setenv("OVFCC_PREFILL_ROWS", rows)
     c = datagen.make_case(61, 200, K, N, wt, G, zt, with_bias=True)
     w = fc.CompressedWeights.from_case(dev, c)
     ref = oracle_y(oracle, c)
