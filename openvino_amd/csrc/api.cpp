@@ -143,9 +143,16 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
     ovfcc::FcDeviceArgs a;
     fill_args(w, x, y, M, &a);
     int force = r->force_kernel;
-    const bool chunked = w->layout.tiled && M > ovfcc::kDecodeMaxRows &&
-                         ((force == OVFCC_KERNEL_AUTO && M <= ovfcc::kChunkedMaxRows) ||
-                          ((w->desc.N % 128) != 0 && (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL)));
+    bool chunked = w->layout.tiled && M > ovfcc::kDecodeMaxRows &&
+                   ((force == OVFCC_KERNEL_AUTO && M <= ovfcc::kChunkedMaxRows) ||
+                    ((w->desc.N % 128) != 0 && (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL)));
+    if (chunked && force == OVFCC_KERNEL_AUTO && M > ovfcc::kChunkedMinPrefillRows && (w->desc.N % 128) == 0) {
+        // above 64 rows the 4-bit async prefill kernel (64-row tiles, K split) beats two or three decode launches
+        // wherever its grid fills the chip; measured on the Llama-3-8B shapes
+        ovfcc::LaunchPlan p;
+        if (ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, r->force_split, r->ctx->n_cus, &p) == OVFCC_OK && p.async_dma)
+            chunked = false;
+    }
     if (chunked) {
         const int64_t chunks = (M + ovfcc::kDecodeMaxRows - 1) / ovfcc::kDecodeMaxRows;
         const int64_t step = (M + chunks - 1) / chunks;  // equal shares rather than 48 + remainder

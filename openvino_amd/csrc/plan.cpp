@@ -171,10 +171,15 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         // (the 4-bit register-fed kernel can also split K, which multiplies its grid by up to eight)
         const bool may_split = direct_ok && L.bits == 4 && env_int("OVFCC_PREFILL_DIRECT", 1) != 0 &&
                                env_int("OVFCC_PREFILL_ASYNC", 1) != 0;
+        // (and it has a form with 64-row tiles, which doubles the tile count of a grid that fits one round)
         int64_t reach = (a.N / kPrefillWideN) * m_tiles;
-        if (may_split)
+        if (may_split) {
+            const int64_t tiles64 = (a.N / kPrefillWideN) * ((a.M + 63) / 64);
+            if (tiles64 <= n_cus)
+                reach = tiles64;
             for (int split = 1; split < 8 && reach * 2 <= n_cus && L.k_blocks / (split * 2) >= 8; split *= 2)
                 reach *= 2;
+        }
         bool big = reach * 2 >= n_cus;
         const int wide_env = env_int("OVFCC_PREFILL_WIDE", -1);
         if (wide_env >= 0)

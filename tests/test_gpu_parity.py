@@ -191,6 +191,26 @@ def test_kernel_policy(dev, req):
         w.close()
 
 
+def test_mid_row_counts_on_a_wide_node(oracle, dev, req):
+    """49..128 rows on a node wide enough for the async prefill kernel to fill the chip: up to 64 rows run as decode
+    launches, above as one prefill launch with 64-row tiles and K split; all within the oracle bounds."""
+    say("mid row counts")
+    c = datagen.make_case(840, 128, 2048, 8192, "u4", 128, "u4", with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c)
+    ref = oracle_y(oracle, c)
+    try:
+        for M, family in ((49, _lib.KERNEL_DECODE), (64, _lib.KERNEL_DECODE), (65, _lib.KERNEL_PREFILL),
+                          (96, _lib.KERNEL_PREFILL), (128, _lib.KERNEL_PREFILL)):
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            assert info["kernel"] == family, (M, info)
+            if family == _lib.KERNEL_PREFILL:
+                assert info["name"] == "fcc_prefill_async_w4" and info["tile_m"] == 64 and info["split_k"] > 1, info
+            check_parity(oracle, y, ref[:M], c.K, f"M={M} {info}", output_rounding_slack=True)
+    finally:
+        w.close()
+
+
 @pytest.mark.parametrize("batch", ["0", "1"])
 @pytest.mark.parametrize("wt,zt,N,K,G", [("u4", "u4", 272, 1024, 128), ("i4", "none", 128, 2048, 256),
                                          ("u8", "u8", 144, 512, 512), ("u8", "none", 256, 1024, 128)])
