@@ -140,6 +140,37 @@ __device__ __forceinline__ void xcd_tile(int& tile_x, int& tile_y, unsigned row_
     xcd_tile_at(blockIdx.y * gridDim.x + blockIdx.x, gridDim.x, gridDim.y, tile_x, tile_y, row_cost, col_cost);
 }
 
+// What one workgroup does: k-blocks [kb_lo, kb_hi) of the output tile at column block tile_x and rows m0.. of its
+// node, as part z of split_k parts of that tile (split_k == 1: the whole tile), parked in workspace slot park_slot.
+struct TileWork {
+    int tile_x, tile_y, m0, z, split_k, kb_lo, kb_hi, park_slot;
+};
+
+// Work of workgroup blockIdx.x for a tiles_x x tiles_y tile grid (1-D launch) of the prefill kernels with
+// 256-channel tiles; col_cost is the relative size of a tile's weight strip against 2 * tile_rows for its
+// activation strip.  The first full_tiles workgroups take one whole tile each, in the XCD-aware order of
+// xcd_tile_at; the remaining tiles are cut into tail_split
+// parts along K, part by part (all first parts, then all second parts, ...), so that a launch whose tile count
+// is a little more than a multiple of the compute units ends with a full round of shorter workgroups instead
+// of a mostly idle round of whole tiles.  full_tiles = 0 splits every tile (few tiles, long K).
+__device__ __forceinline__ TileWork tile_work(int tiles_x, int tiles_y, int full_tiles, int tail_split,
+                                              int kb_per_split, int kb_total, int tile_rows, int col_cost) {
+    TileWork wk;
+    const int L = (int)blockIdx.x;
+    int slot;
+    if (L < full_tiles) {
+        slot = L, wk.z = 0, wk.split_k = 1, wk.kb_lo = 0, wk.kb_hi = kb_total, wk.park_slot = 0;
+    } else {
+        const int tail = tiles_x * tiles_y - full_tiles, j = L - full_tiles;
+        wk.z = j / tail, slot = full_tiles + j % tail, wk.split_k = tail_split;
+        wk.kb_lo = wk.z * kb_per_split, wk.kb_hi = min(kb_total, wk.kb_lo + kb_per_split);
+        wk.park_slot = j % tail;
+    }
+    xcd_tile_at((unsigned)slot, (unsigned)tiles_x, (unsigned)tiles_y, wk.tile_x, wk.tile_y, 2 * tile_rows, col_cost);
+    wk.m0 = wk.tile_y * tile_rows;
+    return wk;
+}
+
 // Gated-linear-unit epilogue on f32 values: act(gate) * up with act = Swish (1), Gelu (2), Gelu_Tanh (3), the
 // formulas of the OpenVINO Intel-GPU plugin (cl_kernels/swiglu_gpu_ref.cl:74-85, swish beta = 1).  Exponential
 // and reciprocal are the hardware's (about 1e-6 relative, far inside the f16 result): the epilogue of a prefill

@@ -37,6 +37,7 @@
 // Weights: (q - zp) * s rounded once to f16 for grouped scales; with one group per channel the exact
 // integers q - zp go to the matrix cores and the scale multiplies the f32 result.
 #include "device_common.h"
+#include "prefill_epilogue.h"
 
 namespace ovfcc {
 
@@ -50,35 +51,6 @@ constexpr int PA_W_OFF = PA_STAGES * PA_A_BYTES;
 constexpr int PA_P_OFF = PA_W_OFF + PA_STAGES * PA_W_BYTES;
 constexpr unsigned PA_LDS_BYTES = (unsigned)(PA_P_OFF + PA_STAGES * PA_P_BYTES);  // 147 KiB
 
-// What one workgroup does: k-blocks [kb_lo, kb_hi) of the output tile at column block tile_x and rows m0.. of its
-// node, as part z of split_k parts of that tile (split_k == 1: the whole tile), parked in workspace slot park_slot.
-struct AsyncWork {
-    int tile_x, tile_y, m0, z, split_k, kb_lo, kb_hi, park_slot;
-};
-
-// Work of workgroup blockIdx.x for a tiles_x x tiles_y tile grid (1-D launch).  The first full_tiles workgroups
-// take one whole tile each, in the XCD-aware order of xcd_tile_at; the remaining tiles are cut into tail_split
-// parts along K, part by part (all first parts, then all second parts, ...), so that a launch whose tile count
-// is a little more than a multiple of the compute units ends with a full round of shorter workgroups instead
-// of a mostly idle round of whole tiles.  full_tiles = 0 splits every tile (few tiles, long K).
-__device__ __forceinline__ AsyncWork async_work(int tiles_x, int tiles_y, int full_tiles, int tail_split,
-                                                int kb_per_split, int kb_total, int tile_rows) {
-    AsyncWork wk;
-    const int L = (int)blockIdx.x;
-    int slot;
-    if (L < full_tiles) {
-        slot = L, wk.z = 0, wk.split_k = 1, wk.kb_lo = 0, wk.kb_hi = kb_total, wk.park_slot = 0;
-    } else {
-        const int tail = tiles_x * tiles_y - full_tiles, j = L - full_tiles;
-        wk.z = j / tail, slot = full_tiles + j % tail, wk.split_k = tail_split;
-        wk.kb_lo = wk.z * kb_per_split, wk.kb_hi = min(kb_total, wk.kb_lo + kb_per_split);
-        wk.park_slot = j % tail;
-    }
-    xcd_tile_at((unsigned)slot, (unsigned)tiles_x, (unsigned)tiles_y, wk.tile_x, wk.tile_y, 2 * tile_rows, PA_BN / 2);
-    wk.m0 = wk.tile_y * tile_rows;
-    return wk;
-}
-
 // The whole kernel for one workgroup's share of one node.  The two kernels below differ only in where the node's
 // operands come from.
 template <bool ZP_TABLE, bool PRESCALE, int NT>
@@ -87,7 +59,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                                                    const half_t* __restrict__ bias, void* __restrict__ y,
                                                    float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N,
                                                    int K, int kb_total, int kb_per_group, int ng, int zp_const,
-                                                   int out_f32, int glu, const AsyncWork wk) {
+                                                   int out_f32, int glu, const TileWork wk) {
     static_assert(NT == 8 || NT == 4, "tiles of 128 or 64 rows");
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
     constexpr int AL = NT / 2;                          // activation loads per wave and k-block
@@ -327,162 +299,9 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
         }
     }
 
-    // ---- epilogue: k-group 1 -> k-group 0 through LDS, two channel tiles at a time.  Without split-K k-group 0
-    // finishes the outputs; with split-K it parks the f32 tile in the workspace with device-scope stores and
-    // waits for them, the workgroup draws a ticket from the tile's arrival counter, and the last arrival adds
-    // the parked tiles in split order with device-scope loads (the result does not depend on arrival order),
-    // finishes the outputs and returns the counter to zero.  No fences: a device-scope fence writes back and
-    // invalidates whole caches, which costs more than the kernel. ----
+    // ---- epilogue (prefill_epilogue.h): k-group hand-over, scale / bias / gated linear unit, split-K fix-up ----
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));  // the out-of-range loads of the last trips still target LDS
-    __syncthreads();
-    float* ex = reinterpret_cast<float*>(lds_raw);  // [wn][2 x 8 x 4][64 lanes]
-    __shared__ unsigned ticket_s;
-    // parked tile layout: [tile][split][wn][channel tile r][row tile t][lane] float4
-    constexpr int kAuxDeviceScope = 16;              // sc1: write through to / read from memory shared by all XCDs
-    constexpr unsigned kParkBytes = 4 * (4 * NT) * 64 * 16;  // one workgroup's f32 tile
-    const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(
-        reinterpret_cast<char*>(ws) + (size_t)tile_id * split_k * kParkBytes, 0, split_k * (int)kParkBytes, kRsrcFlags);
-    auto finish = [&](int r, int t, float4_t v, const float (&sc)[4], const float (&bs)[4]) {
-        const int n = n0 + 64 * wn + 16 * r + 4 * kq;  // four consecutive channels
-        const int m = m0 + 16 * t + col;
-        const float o[4] = {v.x * sc[0] + bs[0], v.y * sc[1] + bs[1], v.z * sc[2] + bs[2], v.w * sc[3] + bs[3]};
-        if (m < M) {
-            if (out_f32) {
-                *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * N + n) = float4_t{o[0], o[1], o[2], o[3]};
-            } else {
-                *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * N + n) =
-                    half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
-            }
-        }
-    };
-    // gated linear unit: channel tiles 2 j and 2 j + 1 of the wave are gate and up of output channels
-    // (n0 + 64 wn) / 2 + 16 j .. of the [M, N / 2] result
-    auto finish_glu = [&](int j, int t, float4_t g, float4_t u, const float (&scg)[4], const float (&bsg)[4],
-                          const float (&scu)[4], const float (&bsu)[4]) {
-        const int n = (n0 + 64 * wn) / 2 + 16 * j + 4 * kq;
-        const int m = m0 + 16 * t + col;
-        const float o[4] = {glu_value(glu, g.x * scg[0] + bsg[0], u.x * scu[0] + bsu[0]),
-                            glu_value(glu, g.y * scg[1] + bsg[1], u.y * scu[1] + bsu[1]),
-                            glu_value(glu, g.z * scg[2] + bsg[2], u.z * scu[2] + bsu[2]),
-                            glu_value(glu, g.w * scg[3] + bsg[3], u.w * scu[3] + bsu[3])};
-        if (m < M) {
-            if (out_f32) {
-                *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * (N / 2) + n) =
-                    float4_t{o[0], o[1], o[2], o[3]};
-            } else {
-                *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * (N / 2) + n) =
-                    half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
-            }
-        }
-    };
-    auto channel_params = [&](int r, float (&sc)[4], float (&bs)[4]) {
-        const int n = n0 + 64 * wn + 16 * r + 4 * kq;
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-            sc[q] = 1.f, bs[q] = 0.f;
-        if constexpr (!PRESCALE) {  // one group per channel: scales are st[n]
-            const half4_t s4 = *reinterpret_cast<const half4_t*>(st + n);
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                sc[q] = (float)s4[q];
-        }
-        if (bias) {
-            const half4_t b4 = *reinterpret_cast<const half4_t*>(bias + n);
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                bs[q] = (float)b4[q];
-        }
-    };
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-        if (kg == 1) {
-#pragma unroll
-            for (int r2 = 0; r2 < 2; ++r2)
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const float4_t v = acc[2 * hh + r2][t];
-                    float* p = ex + ((wn * 8 * NT + (r2 * NT + t) * 4) * 64) + lane;
-                    p[0] = v.x, p[64] = v.y, p[128] = v.z, p[192] = v.w;
-                }
-        }
-        __syncthreads();
-        if (kg == 0 && glu && split_k == 1) {
-            float scg[4], bsg[4], scu[4], bsu[4];
-            channel_params(2 * hh, scg, bsg);
-            channel_params(2 * hh + 1, scu, bsu);
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const float* pg = ex + ((wn * 8 * NT + t * 4) * 64) + lane;
-                const float* pu = ex + ((wn * 8 * NT + (NT + t) * 4) * 64) + lane;
-                const float4_t a = acc[2 * hh][t], b = acc[2 * hh + 1][t];
-                finish_glu(hh, t, float4_t{a.x + pg[0], a.y + pg[64], a.z + pg[128], a.w + pg[192]},
-                           float4_t{b.x + pu[0], b.y + pu[64], b.z + pu[128], b.w + pu[192]}, scg, bsg, scu, bsu);
-            }
-        } else if (kg == 0) {
-#pragma unroll
-            for (int r2 = 0; r2 < 2; ++r2) {
-                const int r = 2 * hh + r2;
-                float sc[4], bs[4];
-                channel_params(r, sc, bs);
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const float* p = ex + ((wn * 8 * NT + (r2 * NT + t) * 4) * 64) + lane;
-                    const float4_t a = acc[r][t];
-                    const float4_t v = float4_t{a.x + p[0], a.y + p[64], a.z + p[128], a.w + p[192]};
-                    if (split_k == 1)
-                        finish(r, t, v, sc, bs);
-                    else
-                        __builtin_amdgcn_raw_buffer_store_b128(
-                            __builtin_bit_cast(uint4_t, v), rp,
-                            wk.z * kParkBytes + (unsigned)(((wn * 4 + r) * NT + t) * 64 + lane) * 16u, 0,
-                            kAuxDeviceScope);
-                }
-            }
-        }
-        __syncthreads();
-    }
-    if (split_k == 1)
-        return;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the parked tile has reached memory before the ticket is drawn
-    __syncthreads();
-    if (tid == 0)
-        ticket_s = __hip_atomic_fetch_add(counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (ticket_s != (unsigned)(split_k - 1))
-        return;
-    auto parked_sum = [&](int r, int t) {
-        float4_t v = float4_t{0.f, 0.f, 0.f, 0.f};
-        for (int z = 0; z < split_k; ++z) {
-            const float4_t pz = __builtin_bit_cast(
-                float4_t,
-                __builtin_amdgcn_raw_buffer_load_b128(
-                    rp, z * kParkBytes + (unsigned)(((wn * 4 + r) * NT + t) * 64 + lane) * 16u, 0, kAuxDeviceScope));
-            v.x += pz.x, v.y += pz.y, v.z += pz.z, v.w += pz.w;
-        }
-        return v;
-    };
-    if (kg == 0 && glu) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            float scg[4], bsg[4], scu[4], bsu[4];
-            channel_params(2 * j, scg, bsg);
-            channel_params(2 * j + 1, scu, bsu);
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-                finish_glu(j, t, parked_sum(2 * j, t), parked_sum(2 * j + 1, t), scg, bsg, scu, bsu);
-        }
-    } else if (kg == 0) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float sc[4], bs[4];
-            channel_params(r, sc, bs);
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-                finish(r, t, parked_sum(r, t), sc, bs);
-        }
-    }
-    if (tid == 0)
-        __hip_atomic_store(counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    tile_epilogue<PRESCALE, NT>(acc, lds_raw, st, bias, y, ws, counters, M, N, n0, m0, split_k, wk.z, tile_id, out_f32, glu);
 }
 
 template <bool ZP_TABLE, bool PRESCALE, int NT>
@@ -496,7 +315,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
                                                                 int kb_total, int kb_per_group, int ng, int zp_const,
                                                                 int out_f32, int glu, int tiles_x, int tiles_y,
                                                                 int full_tiles, int tail_split, int kb_per_split) {
-    const AsyncWork wk = async_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT);
+    const TileWork wk = tile_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT, PA_BN / 2);
     prefill_async_body<ZP_TABLE, PRESCALE, NT>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
                                            zp_const, out_f32, glu, wk);
 }
@@ -512,7 +331,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const Ba
                                                                         int zp_const, int out_f32, int glu,
                                                                         int tiles_x, int tiles_y, int full_tiles,
                                                                         int tail_split, int kb_per_split) {
-    AsyncWork wk = async_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT);
+    TileWork wk = tile_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT, PA_BN / 2);
     const BatchGroupItem& it = tab.item[wk.tile_y];
     if (it.M <= 0)
         return;

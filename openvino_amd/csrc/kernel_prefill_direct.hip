@@ -32,6 +32,7 @@
 // Weights: (q - zp) * s rounded once to f16 for grouped scales; with one group per channel the exact
 // integers q - zp go to the matrix cores and the scale multiplies the f32 result.
 #include "device_common.h"
+#include "prefill_epilogue.h"
 
 namespace ovfcc {
 
@@ -48,9 +49,11 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
                                                                  const uint8_t* __restrict__ zt,
                                                                  const half_t* __restrict__ x,
                                                                  const half_t* __restrict__ bias,
-                                                                 void* __restrict__ y, int M, int N, int K,
+                                                                 void* __restrict__ y, float* __restrict__ ws,
+                                                                 unsigned* __restrict__ counters, int M, int N, int K,
                                                                  int kb_total, int kb_per_group, int ng, int zp_const,
-                                                                 int out_f32, int glu) {
+                                                                 int out_f32, int glu, int tiles_x, int tiles_y,
+                                                                 int full_tiles, int tail_split, int kb_per_split) {
     constexpr int TPB = BITS == 4 ? 1 : 2;   // tiles per k-block and channel tile
     constexpr int WD = BITS == 4 ? 2 : 4;    // packed dwords per lane, channel tile and k-block for this k-group
     constexpr int NOPS = (BITS == 4 ? 5 : 4) + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword (pair)
@@ -63,10 +66,11 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wn = wave & 3, kg = wave >> 2;
-    int tile_x, tile_y;
-    xcd_tile(tile_x, tile_y, 2 * PD_BM, PD_BN * BITS / 8);
-    const int n0 = tile_x * PD_BN;
-    const int m0 = tile_y * PD_BM;
+    // split-K: this workgroup contracts k-blocks [kb_lo, kb_hi); loads of k-blocks past kb_hi are sent out of range
+    const TileWork wk = tile_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, PD_BM, PD_BN * BITS / 8);
+    const int n0 = wk.tile_x * PD_BN;
+    const int m0 = wk.m0;
+    const int kb_lo = wk.kb_lo, kb_hi = wk.kb_hi;
     const int col = lane & 15, kq = lane >> 4;
 
     constexpr unsigned kOob = 0x80000000u;
@@ -89,7 +93,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
     const unsigned a_row0 = (unsigned)((m0 + 16 * wave + (lane >> 4)) * K) * 2u;
     const unsigned a_c0 = (unsigned)((lane & 15) ^ (lane >> 4));
     auto dma_a = [&](int kb, int i) {
-        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         const int stage = kb % PD_STAGES;
         const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(4 * i * K + kb * PD_BK) * 2u);
         const unsigned voff = a_row0 + sterm + ((a_c0 ^ (unsigned)(4 * i)) << 4);
@@ -103,7 +107,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
     uint32_t rzp[2][4];
     const unsigned w_voff = BITS == 4 ? lane * 16u + kg * 8u : lane * 16u;
     auto load_w = [&](int kb, int slot, int r) {
-        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         if constexpr (BITS == 4) {
             const unsigned sofs = __builtin_amdgcn_readfirstlane((unsigned)(r * kb_total + kb) * kTileBytes);
             const uint2_t v =
@@ -120,14 +124,14 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
     // into both halves of a register when the scale is used
     const uint32_t scale_sel = (col & 1) ? 0x03020302u : 0x01000100u;
     auto load_s = [&](int kb, int slot, int r) {
-        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         const unsigned g = kb_per_group == 1 ? (unsigned)kb : __umulhi((unsigned)kb, g_mul);
         rscale[slot][r] =
             __builtin_amdgcn_raw_buffer_load_b32(
                 rs, (__builtin_amdgcn_readfirstlane((r * ng + g) * 32u) + (unsigned)(col & ~1) * 2u) | oob, 0, 0);
     };
     auto load_z = [&](int kb, int slot, int r) {
-        const unsigned oob = (unsigned)((kb_total - 1 - kb) >> 31) & kOob;
+        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         const unsigned g = kb_per_group == 1 ? (unsigned)kb : __umulhi((unsigned)kb, g_mul);
         rzp[slot][r] = (uint8_t)__builtin_amdgcn_raw_buffer_load_b8(
             rz, (__builtin_amdgcn_readfirstlane((r * ng + g) * 16u) + (unsigned)col) | oob, 0, 0);
@@ -210,23 +214,23 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
     // ---- prologue.  Memory instructions are issued in the same order as in the main loop (direct-to-LDS
     // loads of a k-block, then its ring loads), which the wait below counts on. ----
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            dma_a(kb, i);
+            dma_a(kb_lo + j, i);
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    for (int j = 0; j < 2; ++j) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-            load_w(kb, kb, r);
+            load_w(kb_lo + j, j, r);
         if constexpr (PRESCALE)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                load_s(kb, kb, r);
+                load_s(kb_lo + j, j, r);
         if constexpr (ZP_TABLE)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                load_z(kb, kb, r);
+                load_z(kb_lo + j, j, r);
     }
     Frag8 wf0[4], wf1[4];
 #pragma unroll
@@ -237,7 +241,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
 
     // ---- main loop: two k-blocks per trip so that ring slots are static.  k-blocks past the end are loaded
     // out of range (zeros) and add nothing. ----
-    for (int kb0 = 0; kb0 < kb_total; kb0 += 2) {
+    for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += 2) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int kb = kb0 + u;
@@ -268,93 +272,10 @@ __global__ __launch_bounds__(512) void fcc_prefill_direct_kernel(const uint4_t* 
         }
     }
 
-    // ---- epilogue: k-group 1 -> k-group 0 through LDS, two channel tiles at a time ----
+    // ---- epilogue (prefill_epilogue.h): k-group hand-over, scale / bias / gated linear unit, split-K fix-up ----
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));  // the out-of-range loads of the last trips still target LDS
-    __syncthreads();
-    float* ex = reinterpret_cast<float*>(lds_raw);  // [wn][2 x 8 x 4][64 lanes]
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh) {
-        if (kg == 1) {
-#pragma unroll
-            for (int r2 = 0; r2 < 2; ++r2)
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const float4_t v = acc[2 * hh + r2][t];
-                    float* p = ex + ((wn * 64 + (r2 * 8 + t) * 4) * 64) + lane;
-                    p[0] = v.x, p[64] = v.y, p[128] = v.z, p[192] = v.w;
-                }
-        }
-        __syncthreads();
-        if (kg == 0 && glu) {
-            // gated linear unit: channel tiles 2 hh and 2 hh + 1 of the wave are gate and up of output channels
-            // (n0 + 64 wn) / 2 + 16 hh .. of the [M, N / 2] result
-            const int ng_ch = n0 + 64 * wn + 32 * hh + 4 * kq;  // gate channels; up channels are 16 further
-            float sc[2][4], bs[2][4];
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    sc[h][q] = PRESCALE ? 1.f : (float)st[ng_ch + 16 * h + q];
-                    bs[h][q] = bias ? (float)bias[ng_ch + 16 * h + q] : 0.f;
-                }
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                float o[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float g = acc[2 * hh][t][q] + ex[((wn * 64 + t * 4 + q) * 64) + lane];
-                    const float u = acc[2 * hh + 1][t][q] + ex[((wn * 64 + (8 + t) * 4 + q) * 64) + lane];
-                    o[q] = glu_value(glu, g * sc[0][q] + bs[0][q], u * sc[1][q] + bs[1][q]);
-                }
-                const int m = m0 + 16 * t + col;
-                const size_t at = (size_t)m * (N / 2) + (n0 + 64 * wn) / 2 + 16 * hh + 4 * kq;
-                if (m < M) {
-                    if (out_f32)
-                        *reinterpret_cast<float4_t*>(static_cast<float*>(y) + at) = float4_t{o[0], o[1], o[2], o[3]};
-                    else
-                        *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + at) =
-                            half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
-                }
-            }
-        } else if (kg == 0) {
-#pragma unroll
-            for (int r2 = 0; r2 < 2; ++r2) {
-                const int r = 2 * hh + r2;
-                const int n = n0 + 64 * wn + 16 * r + 4 * kq;  // four consecutive channels
-                float sc[4] = {1.f, 1.f, 1.f, 1.f}, bs[4] = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (!PRESCALE) {  // one group per channel: scales are st[n]
-                    const half4_t s4 = *reinterpret_cast<const half4_t*>(st + n);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        sc[q] = (float)s4[q];
-                }
-                if (bias) {
-                    const half4_t b4 = *reinterpret_cast<const half4_t*>(bias + n);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        bs[q] = (float)b4[q];
-                }
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const float* p = ex + ((wn * 64 + (r2 * 8 + t) * 4) * 64) + lane;
-                    const float4_t a = acc[r][t];
-                    const float v[4] = {(a.x + p[0]) * sc[0] + bs[0], (a.y + p[64]) * sc[1] + bs[1],
-                                        (a.z + p[128]) * sc[2] + bs[2], (a.w + p[192]) * sc[3] + bs[3]};
-                    const int m = m0 + 16 * t + col;
-                    if (m < M) {
-                        if (out_f32) {
-                            *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * N + n) =
-                                float4_t{v[0], v[1], v[2], v[3]};
-                        } else {
-                            *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * N + n) =
-                                half4_t{(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
-                        }
-                    }
-                }
-            }
-        }
-        __syncthreads();
-    }
+    tile_epilogue<PRESCALE, 8>(acc, lds_raw, st, bias, y, ws, counters, M, N, n0, m0, wk.split_k, wk.z, wk.park_slot,
+                               out_f32, glu);
 }
 
 template <int BITS, bool ZPT, bool PRE>
@@ -369,10 +290,11 @@ static int launch_direct_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStr
             return (int)e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], 1), dim3(512), PD_LDS_BYTES, s, (const uint4_t*)a.w,
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), PD_LDS_BYTES, s, (const uint4_t*)a.w,
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
-                       (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
-                       L.zp_const, a.out_f32, L.glu);
+                       a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
+                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32, L.glu, p.tiles_x, p.tiles_y,
+                       p.full_tiles, p.split_k, p.kblocks_per_split);
     return (int)hipGetLastError();
 }
 
@@ -385,6 +307,14 @@ static int launch_direct_bits(const FcDeviceArgs& a, const LaunchPlan& p, hipStr
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
+    // the launch must be what tile_work assumes: a 1-D grid of full_tiles whole tiles plus split_k parts of each
+    // remaining tile, parts that cover K and rows that cover M
+    const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
+    if (p.tile_m != PD_BM || p.tiles_x != a.N / PD_BN || (int64_t)p.tiles_y * PD_BM < a.M || p.full_tiles < 0 ||
+        p.full_tiles > tiles || p.split_k < 1 || (int64_t)p.kblocks_per_split * p.split_k < L.k_blocks ||
+        p.grid[0] != (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) || p.grid[1] != 1 || p.grid[2] != 1 ||
+        (p.split_k > 1 && !(a.workspace && a.counters)))
+        return (int)hipErrorInvalidValue;
     if (L.bits == 4)
         return L.zp_table ? launch_direct_bits<4, true>(a, p, s) : launch_direct_bits<4, false>(a, p, s);
     return L.zp_table ? launch_direct_bits<8, true>(a, p, s) : launch_direct_bits<8, false>(a, p, s);

@@ -168,14 +168,14 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         const bool direct_ok = (a.N % kPrefillWideN) == 0 && a.M * a.K * 2 < ((int64_t)1 << 31) &&
                                (int64_t)16 * L.k_blocks * tiles_per_kb * kTileBytes < ((int64_t)1 << 31);
         const bool wide_ok = direct_ok && (a.K % 256) == 0;
-        // (the 4-bit register-fed kernel can also split K, which multiplies its grid by up to eight)
-        const bool may_split = direct_ok && L.bits == 4 && env_int("OVFCC_PREFILL_DIRECT", 1) != 0 &&
-                               env_int("OVFCC_PREFILL_ASYNC", 1) != 0;
-        // (and it has a form with 64-row tiles, which doubles the tile count of a grid that fits one round)
+        // (the register-fed kernels can also split K, which multiplies their grid by up to eight)
+        const bool may_split = direct_ok && env_int("OVFCC_PREFILL_DIRECT", 1) != 0;
+        const bool may_async = may_split && L.bits == 4 && env_int("OVFCC_PREFILL_ASYNC", 1) != 0;
+        // (and the 4-bit one has a form with 64-row tiles, which doubles the tile count of a grid that fits one round)
         int64_t reach = (a.N / kPrefillWideN) * m_tiles;
         if (may_split) {
             const int64_t tiles64 = (a.N / kPrefillWideN) * ((a.M + 63) / 64);
-            if (tiles64 <= n_cus)
+            if (may_async && tiles64 <= n_cus)
                 reach = tiles64;
             for (int split = 1; split < 8 && reach * 2 <= n_cus && L.k_blocks / (split * 2) >= 8; split *= 2)
                 reach *= 2;
@@ -206,7 +206,7 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             }
         }
         p.kblocks_per_split = (int)L.k_blocks;
-        if (p.async_dma) {
+        if (p.direct) {
             // Split K while the tiles alone leave compute units idle (at least eight k-blocks per workgroup): the
             // f32 tiles are parked in the workspace and added by the last workgroup to arrive.
             // OVFCC_PREFILL_TAIL = 1 (an experiment, off by default) also splits, with more tiles than compute

@@ -1,0 +1,183 @@
+// Epilogue shared by the prefill kernels with 256-channel tiles and 8 waves (wn = wave & 3 owns 64 channels as four
+// 16-channel tiles, kg = wave >> 2 owns half of every k-block): acc[r][t] is the wave's f32 result for channel tile r
+// and row tile t in the 16x16 MFMA layout (lane: column m = lane & 15, channels 4 (lane >> 4) + q).
+#pragma once
+
+#include "device_common.h"
+
+namespace ovfcc {
+
+// k-group 1 -> k-group 0 through LDS, two channel tiles at a time.  Without split-K k-group 0
+// finishes the outputs; with split-K it parks the f32 tile in the workspace with device-scope stores and
+// waits for them, the workgroup draws a ticket from the tile's arrival counter, and the last arrival adds
+// the parked tiles in split order with device-scope loads (the result does not depend on arrival order),
+// finishes the outputs and returns the counter to zero.  No fences: a device-scope fence writes back and
+// invalidates whole caches, which costs more than the kernel.
+// The caller has waited for its own outstanding loads into LDS; lds_raw is the workgroup's dynamic LDS (at least
+// NT * 8 KiB), n0 / m0 the tile's first channel and row, z_part this workgroup's part of split_k, park_slot the
+// tile's slot in workspace and counters.
+template <bool PRESCALE, int NT>
+__device__ __forceinline__ void tile_epilogue(float4_t (&acc)[4][NT], unsigned char* lds_raw,
+                                              const half_t* __restrict__ st, const half_t* __restrict__ bias,
+                                              void* __restrict__ y, float* __restrict__ ws,
+                                              unsigned* __restrict__ counters, int M, int N, int n0, int m0, int split_k,
+                                              int z_part, int park_slot, int out_f32, int glu) {
+    constexpr int kRsrcFlags = 0x00020000;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave & 3, kg = wave >> 2;
+    const int col = lane & 15, kq = lane >> 4;
+    const int tile_id = park_slot;
+    __syncthreads();
+    float* ex = reinterpret_cast<float*>(lds_raw);  // [wn][2 x 8 x 4][64 lanes]
+    __shared__ unsigned ticket_s;
+    // parked tile layout: [tile][split][wn][channel tile r][row tile t][lane] float4
+    constexpr int kAuxDeviceScope = 16;              // sc1: write through to / read from memory shared by all XCDs
+    constexpr unsigned kParkBytes = 4 * (4 * NT) * 64 * 16;  // one workgroup's f32 tile
+    const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<char*>(ws) + (size_t)tile_id * split_k * kParkBytes, 0, split_k * (int)kParkBytes, kRsrcFlags);
+    auto finish = [&](int r, int t, float4_t v, const float (&sc)[4], const float (&bs)[4]) {
+        const int n = n0 + 64 * wn + 16 * r + 4 * kq;  // four consecutive channels
+        const int m = m0 + 16 * t + col;
+        const float o[4] = {v.x * sc[0] + bs[0], v.y * sc[1] + bs[1], v.z * sc[2] + bs[2], v.w * sc[3] + bs[3]};
+        if (m < M) {
+            if (out_f32) {
+                *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * N + n) = float4_t{o[0], o[1], o[2], o[3]};
+            } else {
+                *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * N + n) =
+                    half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
+            }
+        }
+    };
+    // gated linear unit: channel tiles 2 j and 2 j + 1 of the wave are gate and up of output channels
+    // (n0 + 64 wn) / 2 + 16 j .. of the [M, N / 2] result
+    auto finish_glu = [&](int j, int t, float4_t g, float4_t u, const float (&scg)[4], const float (&bsg)[4],
+                          const float (&scu)[4], const float (&bsu)[4]) {
+        const int n = (n0 + 64 * wn) / 2 + 16 * j + 4 * kq;
+        const int m = m0 + 16 * t + col;
+        const float o[4] = {glu_value(glu, g.x * scg[0] + bsg[0], u.x * scu[0] + bsu[0]),
+                            glu_value(glu, g.y * scg[1] + bsg[1], u.y * scu[1] + bsu[1]),
+                            glu_value(glu, g.z * scg[2] + bsg[2], u.z * scu[2] + bsu[2]),
+                            glu_value(glu, g.w * scg[3] + bsg[3], u.w * scu[3] + bsu[3])};
+        if (m < M) {
+            if (out_f32) {
+                *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * (N / 2) + n) =
+                    float4_t{o[0], o[1], o[2], o[3]};
+            } else {
+                *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * (N / 2) + n) =
+                    half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
+            }
+        }
+    };
+    auto channel_params = [&](int r, float (&sc)[4], float (&bs)[4]) {
+        const int n = n0 + 64 * wn + 16 * r + 4 * kq;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            sc[q] = 1.f, bs[q] = 0.f;
+        if constexpr (!PRESCALE) {  // one group per channel: scales are st[n]
+            const half4_t s4 = *reinterpret_cast<const half4_t*>(st + n);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                sc[q] = (float)s4[q];
+        }
+        if (bias) {
+            const half4_t b4 = *reinterpret_cast<const half4_t*>(bias + n);
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                bs[q] = (float)b4[q];
+        }
+    };
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+        if (kg == 1) {
+#pragma unroll
+            for (int r2 = 0; r2 < 2; ++r2)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const float4_t v = acc[2 * hh + r2][t];
+                    float* p = ex + ((wn * 8 * NT + (r2 * NT + t) * 4) * 64) + lane;
+                    p[0] = v.x, p[64] = v.y, p[128] = v.z, p[192] = v.w;
+                }
+        }
+        __syncthreads();
+        if (kg == 0 && glu && split_k == 1) {
+            float scg[4], bsg[4], scu[4], bsu[4];
+            channel_params(2 * hh, scg, bsg);
+            channel_params(2 * hh + 1, scu, bsu);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const float* pg = ex + ((wn * 8 * NT + t * 4) * 64) + lane;
+                const float* pu = ex + ((wn * 8 * NT + (NT + t) * 4) * 64) + lane;
+                const float4_t a = acc[2 * hh][t], b = acc[2 * hh + 1][t];
+                finish_glu(hh, t, float4_t{a.x + pg[0], a.y + pg[64], a.z + pg[128], a.w + pg[192]},
+                           float4_t{b.x + pu[0], b.y + pu[64], b.z + pu[128], b.w + pu[192]}, scg, bsg, scu, bsu);
+            }
+        } else if (kg == 0) {
+#pragma unroll
+            for (int r2 = 0; r2 < 2; ++r2) {
+                const int r = 2 * hh + r2;
+                float sc[4], bs[4];
+                channel_params(r, sc, bs);
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const float* p = ex + ((wn * 8 * NT + (r2 * NT + t) * 4) * 64) + lane;
+                    const float4_t a = acc[r][t];
+                    const float4_t v = float4_t{a.x + p[0], a.y + p[64], a.z + p[128], a.w + p[192]};
+                    if (split_k == 1)
+                        finish(r, t, v, sc, bs);
+                    else
+                        __builtin_amdgcn_raw_buffer_store_b128(
+                            __builtin_bit_cast(uint4_t, v), rp,
+                            z_part * kParkBytes + (unsigned)(((wn * 4 + r) * NT + t) * 64 + lane) * 16u, 0,
+                            kAuxDeviceScope);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (split_k == 1)
+        return;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the parked tile has reached memory before the ticket is drawn
+    __syncthreads();
+    if (tid == 0)
+        ticket_s = __hip_atomic_fetch_add(counters + tile_id, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket_s != (unsigned)(split_k - 1))
+        return;
+    auto parked_sum = [&](int r, int t) {
+        float4_t v = float4_t{0.f, 0.f, 0.f, 0.f};
+        for (int z = 0; z < split_k; ++z) {
+            const float4_t pz = __builtin_bit_cast(
+                float4_t,
+                __builtin_amdgcn_raw_buffer_load_b128(
+                    rp, z * kParkBytes + (unsigned)(((wn * 4 + r) * NT + t) * 64 + lane) * 16u, 0, kAuxDeviceScope));
+            v.x += pz.x, v.y += pz.y, v.z += pz.z, v.w += pz.w;
+        }
+        return v;
+    };
+    if (kg == 0 && glu) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            float scg[4], bsg[4], scu[4], bsu[4];
+            channel_params(2 * j, scg, bsg);
+            channel_params(2 * j + 1, scu, bsu);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                finish_glu(j, t, parked_sum(2 * j, t), parked_sum(2 * j + 1, t), scg, bsg, scu, bsu);
+        }
+    } else if (kg == 0) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float sc[4], bs[4];
+            channel_params(r, sc, bs);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                finish(r, t, parked_sum(r, t), sc, bs);
+        }
+    }
+    if (tid == 0)
+        __hip_atomic_store(counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace ovfcc

@@ -84,7 +84,7 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     }
     CHECK(L.tiled, "%s", what);
     const int kb = (int)L.k_blocks;
-    if (p.kernel == OVFCC_KERNEL_DECODE || p.async_dma) {
+    if (p.kernel == OVFCC_KERNEL_DECODE || p.direct) {
         CHECK((int64_t)p.split_k * p.kblocks_per_split >= kb, "%s split=%d per=%d kb=%d", what, p.split_k, p.kblocks_per_split, kb);
         CHECK((int64_t)(p.split_k - 1) * p.kblocks_per_split < kb, "%s empty split: split=%d per=%d kb=%d", what, p.split_k,
               p.kblocks_per_split, kb);
@@ -109,10 +109,11 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
         return;
     }
     CHECK(d.N % 128 == 0, "%s", what);
-    if (p.async_dma) {
+    CHECK(!p.async_dma || (p.direct && L.bits == 4), "%s", what);
+    if (p.direct) {
         const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
-        CHECK(p.tile_m == 128 || p.tile_m == 64, "%s tile_m=%d", what, p.tile_m);
-        CHECK(L.bits == 4 && d.N % 256 == 0 && p.tiles_x == d.N / 256 && p.tiles_y == (M + p.tile_m - 1) / p.tile_m, "%s", what);
+        CHECK(p.tile_m == 128 || (p.async_dma && p.tile_m == 64), "%s tile_m=%d", what, p.tile_m);
+        CHECK(d.N % 256 == 0 && p.tiles_x == d.N / 256 && p.tiles_y == (M + p.tile_m - 1) / p.tile_m, "%s", what);
         CHECK(p.full_tiles >= 0 && p.full_tiles <= tiles && (p.split_k > 1 || p.full_tiles == tiles), "%s full=%d", what, p.full_tiles);
         CHECK(p.grid[0] == (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) && p.grid[1] == 1 && p.grid[2] == 1, "%s", what);
         CHECK(p.workspace_bytes == (p.split_k > 1 ? (size_t)(tiles - p.full_tiles) * p.split_k * p.tile_m * 256 * 4 : 0), "%s", what);
@@ -120,7 +121,7 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     } else {
         CHECK(p.split_k == 1, "%s", what);
         CHECK(p.grid[0] == (unsigned)(d.N / p.tile_n) && p.grid[1] == (unsigned)((M + 127) / 128), "%s", what);
-        CHECK(p.tile_n == 128 || (d.N % 256 == 0 && (p.direct || d.K % 256 == 0)), "%s", what);
+        CHECK(p.tile_n == 128 || (d.N % 256 == 0 && d.K % 256 == 0), "%s", what);
     }
 }
 

@@ -284,11 +284,12 @@ def test_256_wide_prefill_kernels_small_shapes(oracle, dev, req, monkeypatch, wt
 
 
 @pytest.mark.parametrize("wt,zt,N,K,G", [("i4", "none", 256, 2048, 128), ("u4", "u4", 512, 1280, 256),
-                                         ("u4", "none", 256, 1024, 1024)])
+                                         ("u4", "none", 256, 1024, 1024), ("u8", "u8", 256, 1536, 128),
+                                         ("i8", "none", 512, 1024, 1024)])
 @pytest.mark.parametrize("split", [2, 3, 8])
 @pytest.mark.parametrize("rows", ["128", "64"])
 def test_prefill_split_k_is_deterministic(oracle, dev, req, monkeypatch, wt, zt, N, K, G, split, rows):
-    """The 4-bit register-fed prefill kernel with K split over workgroups: any split gives the oracle's answer
+    """The register-fed prefill kernels with K split over workgroups: any split gives the oracle's answer
     (ragged last split, ragged last row tile, bias, per-channel scale in the fix-up), repeated launches give
     identical bits, and the arrival counters return to zero."""
     monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
@@ -301,7 +302,8 @@ def test_prefill_split_k_is_deterministic(oracle, dev, req, monkeypatch, wt, zt,
         say(f"prefill split {split} {wt}/{zt} N={N} K={K} G={G}")
         first = req.infer(w, c.x)
         info = req.last_kernel()
-        assert info["name"] == "fcc_prefill_async_w4" and info["split_k"] > 1, info
+        want = "fcc_prefill_async_w4" if wt in ("u4", "i4") else "fcc_prefill_direct_w8"
+        assert info["name"] == want and info["split_k"] > 1, info
         check_parity(oracle, first, ref, K, f"{info}", output_rounding_slack=True)
         for _ in range(4):
             assert np.array_equal(req.infer(w, c.x).view(np.uint16), first.view(np.uint16))
