@@ -147,10 +147,10 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
                    ((force == OVFCC_KERNEL_AUTO && M <= ovfcc::kChunkedMaxRows) ||
                     ((w->desc.N % 128) != 0 && (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL)));
     if (chunked && force == OVFCC_KERNEL_AUTO && M > ovfcc::kChunkedMinPrefillRows && (w->desc.N % 128) == 0) {
-        // above 64 rows the 4-bit async prefill kernel (64-row tiles, K split) beats two or three decode launches
-        // wherever its grid fills the chip; measured on the Llama-3-8B shapes
+        // a register-fed prefill kernel (K split; 64-row tiles for 4-bit weights) beats two or three decode
+        // launches wherever its grid fills the chip; measured on the Llama-3-8B and -70B shapes
         ovfcc::LaunchPlan p;
-        if (ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, r->force_split, r->ctx->n_cus, &p) == OVFCC_OK && p.async_dma)
+        if (ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, r->force_split, r->ctx->n_cus, &p) == OVFCC_OK && p.direct)
             chunked = false;
     }
     if (chunked) {

@@ -144,7 +144,7 @@ int launch_touch(const void* src, size_t bytes, void* stream);
 
 constexpr int kDecodeMaxRows = 48;                       // rows one decode-family launch covers
 constexpr int kPrefillGroupRows = 128;                   // rows per slice of a grouped prefill launch (one tile)
-constexpr int kChunkedMinPrefillRows = 64;                // ... unless, above this, the async prefill kernel fills the chip
+constexpr int kChunkedMinPrefillRows = 48;                // ... unless, above this, the async prefill kernel fills the chip
 constexpr int kChunkedMaxRows = 128;                     // up to here M is cut into decode launches
 constexpr int kPrefillTileM = 128, kPrefillTileN = 128;  // square prefill kernel
 constexpr int kPrefillWideN = 256;                         // wide prefill kernel: 128 x 256

@@ -145,35 +145,54 @@ __device__ __forceinline__ void tile_epilogue(float4_t (&acc)[4][NT], unsigned c
     __syncthreads();
     if (ticket_s != (unsigned)(split_k - 1))
         return;
-    auto parked_sum = [&](int r, int t) {
-        float4_t v = float4_t{0.f, 0.f, 0.f, 0.f};
-        for (int z = 0; z < split_k; ++z) {
-            const float4_t pz = __builtin_bit_cast(
-                float4_t,
-                __builtin_amdgcn_raw_buffer_load_b128(
-                    rp, z * kParkBytes + (unsigned)(((wn * 4 + r) * NT + t) * 64 + lane) * 16u, 0, kAuxDeviceScope));
-            v.x += pz.x, v.y += pz.y, v.z += pz.z, v.w += pz.w;
-        }
-        return v;
-    };
-    if (kg == 0 && glu) {
+    // Last arrival: every wave adds up two of its k-group pair's four channel tiles (k-group kg takes tiles 2 kg and
+    // 2 kg + 1 -- a gate tile and its up tile), all row tiles, parts in ascending order.  The loads of two parts,
+    // 2 x 2 NT of them, are in flight together (a part index past split_k falls outside the descriptor's range
+    // and reads zero); issued one at a time behind their additions they cost 9 us per part.
+    float4_t sum[2][NT];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            float scg[4], bsg[4], scu[4], bsu[4];
-            channel_params(2 * j, scg, bsg);
-            channel_params(2 * j + 1, scu, bsu);
+    for (int r2 = 0; r2 < 2; ++r2)
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
-                finish_glu(j, t, parked_sum(2 * j, t), parked_sum(2 * j + 1, t), scg, bsg, scu, bsu);
-        }
-    } else if (kg == 0) {
+        for (int t = 0; t < NT; ++t)
+            sum[r2][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int z0 = 0; z0 < split_k; z0 += 2) {
+        float4_t part[2][2][NT];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r2 = 0; r2 < 2; ++r2)
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    part[u][r2][t] = __builtin_bit_cast(
+                        float4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                      rp, (unsigned)(z0 + u) * kParkBytes +
+                                              (unsigned)(((wn * 4 + 2 * kg + r2) * NT + t) * 64 + lane) * 16u,
+                                      0, kAuxDeviceScope));
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r2 = 0; r2 < 2; ++r2)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    sum[r2][t].x += part[u][r2][t].x, sum[r2][t].y += part[u][r2][t].y;
+                    sum[r2][t].z += part[u][r2][t].z, sum[r2][t].w += part[u][r2][t].w;
+                }
+    }
+    if (glu) {
+        float scg[4], bsg[4], scu[4], bsu[4];
+        channel_params(2 * kg, scg, bsg);
+        channel_params(2 * kg + 1, scu, bsu);
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            finish_glu(kg, t, sum[0][t], sum[1][t], scg, bsg, scu, bsu);
+    } else {
+#pragma unroll
+        for (int r2 = 0; r2 < 2; ++r2) {
             float sc[4], bs[4];
-            channel_params(r, sc, bs);
+            channel_params(2 * kg + r2, sc, bs);
 #pragma unroll
             for (int t = 0; t < NT; ++t)
-                finish(r, t, parked_sum(r, t), sc, bs);
+                finish(2 * kg + r2, t, sum[r2][t], sc, bs);
         }
     }
     if (tid == 0)

@@ -192,15 +192,15 @@ def test_kernel_policy(dev, req):
 
 
 def test_mid_row_counts_on_a_wide_node(oracle, dev, req):
-    """49..128 rows on a node wide enough for the async prefill kernel to fill the chip: up to 64 rows run as decode
-    launches, above as one prefill launch with 64-row tiles and K split; all within the oracle bounds."""
+    """49..128 rows: where the async prefill kernel's grid (64-row tiles, K split) fills the chip -- here from two
+    row tiles on -- one prefill launch, otherwise two or three decode launches; all within the oracle bounds."""
     say("mid row counts")
     c = datagen.make_case(840, 128, 2048, 8192, "u4", 128, "u4", with_bias=True)
     w = fc.CompressedWeights.from_case(dev, c)
     ref = oracle_y(oracle, c)
     try:
-        for M, family in ((49, _lib.KERNEL_DECODE), (64, _lib.KERNEL_DECODE), (65, _lib.KERNEL_PREFILL),
-                          (96, _lib.KERNEL_PREFILL), (128, _lib.KERNEL_PREFILL)):
+        for M, family in ((48, _lib.KERNEL_DECODE), (49, _lib.KERNEL_DECODE), (64, _lib.KERNEL_DECODE),
+                          (65, _lib.KERNEL_PREFILL), (96, _lib.KERNEL_PREFILL), (128, _lib.KERNEL_PREFILL)):
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
             assert info["kernel"] == family, (M, info)
