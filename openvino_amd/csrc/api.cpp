@@ -760,7 +760,8 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
                     split *= 2;
             }
             rc = ovfcc::plan_launch(a, OVFCC_KERNEL_DECODE, split, r->ctx->n_cus, &p);
-            grouped = !rc && p.batch && p.tiles_per_group == 1;  // small nodes with few rows plan the streaming kernel
+            // (small nodes with few rows plan the streaming kernel; the grouped kernel has no gated-linear-unit form)
+            grouped = !rc && p.batch && p.tiles_per_group == 1 && !w0->layout.glu;
         } else {
             // planned as one node whose row tiles are the slices: tile counts and split-K come out right
             fill_args(w0, work[0].x, work[0].y, (int64_t)n * rows_cap, &a);

@@ -157,3 +157,25 @@ def test_glu_llama_gate_up(oracle, dev, req):
     finally:
         for w in (wg, wu, fused):
             w.close()
+
+
+def test_glu_grouped_run(oracle, dev, req, monkeypatch):
+    """Experts with fused SwiGLU in one grouped launch (prefill kernel), and with few rows (item-by-item fallback:
+    the grouped small-batch kernel has no gated form)."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    say("glu grouped")
+    K, N = 1024, 512
+    cases = [datagen.make_case(940 + i, 100, K, N, "u4", 128, "u4", with_bias=True) for i in range(3)]
+    ws = [fc.CompressedWeights.from_case(dev, c, glu="swish") for c in cases]
+    try:
+        for rows, grouped in (([100, 7, 64], True), ([5, 20, 1], False)):
+            ys = req.infer_grouped([(w, c.x[:m]) for w, c, m in zip(ws, cases, rows)])
+            info = req.last_kernel()
+            assert ("grouped" in info["name"]) == grouped, info
+            for c, m, y in zip(cases, rows, ys):
+                assert y.shape == (m, N // 2)
+                ref, amp = glu_reference(oracle, c, "swish", x=c.x[:m])
+                check_parity(oracle, y, ref, K, f"rows {rows} {info}", output_rounding_slack=True, limit_scale=amp)
+    finally:
+        for w in ws:
+            w.close()
