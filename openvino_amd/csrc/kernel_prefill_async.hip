@@ -1,7 +1,11 @@
 // Prefill kernel for 4-bit weights with register-fed matrix-core operands and fully asynchronous data
-// movement (M > 128): 128 x 256 output tile per workgroup, 8 waves.
+// movement: 128 x 256 output tile per workgroup (NT = 8 row tiles of 16), 8 waves; also built with 64 x 256
+// tiles (NT = 4) for grids that 128-row tiles would underfill.  The text below describes NT = 8.
 //
-// grid = (N/256, ceil(M/128)), block = 512.  K advances one k-block (128 inputs) per step.
+// 1-D grid, block = 512: workgroup -> (tile, part of K) by tile_work (device_common.h); the first full_tiles
+// workgroups own whole tiles in XCD-aware order, the others one of split_k parts of a tile (deterministic
+// split-K, prefill_epilogue.h).  K advances one k-block (128 inputs) per step.  The grouped kernel at the end of
+// the file runs the same body over a table of nodes, one tile row per node.
 //
 // Every operand of a k-block travels HBM/L2 -> LDS with buffer loads that write LDS directly (no registers,
 // no LDS store instructions), 16 bytes per lane:
@@ -24,7 +28,7 @@
 // steps of every k-block the wave contracts.  A wave unpacks every weight it uses exactly once and multiplies
 // it with all 128 rows (eight 16-row operands read from LDS): 32 v_mfma_f32_16x16x32_f16 per step and 4
 // unpacked dwords.  After the last k-block k-group 1 hands its f32 accumulators to k-group 0 through LDS,
-// which adds, applies per-channel scale and bias and stores.
+// which adds, applies per-channel scale, bias and the gated linear unit and stores (prefill_epilogue.h).
 //
 // The inner loop is software-pipelined by hand and pinned with scheduling barriers: between every two MFMAs
 // of a step sit one or two vector-ALU operations of the *next* step's unpack, and every few MFMAs one memory

@@ -1,6 +1,9 @@
-// Prefill kernel with register-fed weights (M > 128): 128 x 256 output tile per workgroup, 8 waves.
+// Prefill kernel with register-fed weights: 128 x 256 output tile per workgroup, 8 waves.  Runs the 8-bit
+// nodes (three stages of an 8-bit k-block of tiles do not fit in LDS beside the activations, so the 4-bit
+// kernel's all-asynchronous form does not carry over) and, on request, 4-bit ones.
 //
-// grid = (N/256, ceil(M/128)), block = 512.  K advances one k-block (128 inputs) per step.
+// 1-D grid, block = 512: workgroup -> (tile, part of K) by tile_work (device_common.h), deterministic split-K
+// and the rest of the epilogue in prefill_epilogue.h.  K advances one k-block (128 inputs) per step.
 //
 // Weights never pass through LDS as f16.  A packed weight tile already has the matrix cores' operand layout
 // (lane = channel (lane & 15), eight consecutive inputs per dword at 8 (lane >> 4)), so every wave loads the
@@ -18,7 +21,8 @@
 // steps of every k-block the wave contracts (for 8-bit weights: which of the k-block's two 64-input tiles).
 // A wave unpacks every weight it uses exactly once and multiplies it with all 128 rows (eight 16-row operands
 // read from LDS): 32 MFMAs per step and 4 unpacked dwords.  After the last k-block k-group 1 hands its f32
-// accumulators to k-group 0 through LDS, which adds, applies per-channel scale and bias and stores.
+// accumulators to k-group 0 through LDS, which adds, applies per-channel scale, bias and the gated linear unit
+// and stores.
 //
 // The inner loop is software-pipelined by hand and pinned with scheduling barriers: between every two MFMAs
 // of a step sit one or two vector-ALU operations of the *next* step's unpack, and every few MFMAs one memory
