@@ -87,8 +87,8 @@ typedef struct ovfcc_request ovfcc_request; /* one HIP stream + staging + split-
 enum ovfcc_kernel {
     OVFCC_KERNEL_AUTO = 0,
     OVFCC_KERNEL_PLAIN = 1,  /* any shape, OpenVINO layout, one wave per output channel */
-    OVFCC_KERNEL_DECODE = 2, /* M <= 32: split-K streaming kernel over the tiled layout */
-    OVFCC_KERNEL_PREFILL = 3 /* M > 32: LDS-dequantise + MFMA tiles over the tiled layout */
+    OVFCC_KERNEL_DECODE = 2, /* M <= 48: the streaming and the small-batch kernel over the tiled layout */
+    OVFCC_KERNEL_PREFILL = 3 /* more rows: MFMA tile kernels over the tiled layout (N % 128 == 0) */
 };
 
 typedef struct ovfcc_kernel_info {
