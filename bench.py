@@ -137,6 +137,56 @@ def results_table(dev, req, args) -> int:
     grouped_line = (f"config 5 as 2 grouped runs: {t_grouped:.1f} us in total, "
                     f"{flops_total / t_grouped / 1e6:.1f} TFLOP/s")
     log(grouped_line)
+
+    # The same layer through the GatherMatmulCompressed entry point (routing indices in, gather and scatter on the
+    # device): wall time per call over 20 back-to-back calls, host work included.
+    import time
+    tokens = 256
+    indices = np.full((tokens, 2), -1, np.int32)
+    for e, rows_e in enumerate(routes):
+        for t in rows_e:
+            indices[t, 0 if indices[t, 0] < 0 else 1] = e
+    t_op = 0.0
+    for label, which, batches in (("gate", "gate", 1), ("up", "up", 1), ("down", "down", 2)):
+        cases = [datagen.config5_expert(e, which, 1) for e in range(len(routes))]
+        ws = [fc.CompressedWeights.from_case(dev, c) for c in cases]
+        K, N = cases[0].K, cases[0].N
+        A = np.random.default_rng(5).standard_normal((batches, tokens, K)).astype(np.float16)
+        a_ptr, y_ptr = dev.malloc(A.nbytes), dev.malloc(2 * tokens * N * 2)
+        dev.upload(a_ptr, A)
+        req.gather_matmul_device(ws, a_ptr, batches, indices, y_ptr)
+        req.sync()
+        y = dev.download(y_ptr, (2, tokens, N), np.float16).astype(np.float32)
+        info = req.last_kernel()
+        rl2 = mab = 0.0
+        for t in (0, 101, 255):
+            for i in range(2):
+                c = cases[indices[t, i]]
+                ref = oracle.fc_reference(A[i if batches > 1 else 0, t:t + 1], c.w, type_tag[c.w_type], c.scale, c.zp,
+                                          type_tag[c.zp_type], None, N=N, K=K, group_size=c.group_size)
+                rl2 = max(rl2, oracle.rel_l2(y[i, t:t + 1], ref))
+                mab = max(mab, oracle.max_abs(y[i, t:t + 1], ref))
+        best = 1e30
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _ in range(20):
+                req.gather_matmul_device(ws, a_ptr, batches, indices, y_ptr)
+            req.sync()
+            best = min(best, (time.perf_counter() - t0) / 20 * 1e6)
+        t_op += best
+        nbytes = sum(algorithmic_bytes(K, N, len(r_e), 4, 128, 0.5) for r_e in routes)
+        gbs, tfs = nbytes / best / 1e3, 2.0 * 2 * tokens * N * K / best / 1e6
+        rows.append(f"| 5 | gather-matmul op, {label} {K}->{N} (8 experts, top-2) | {tokens} tokens | u4 g128 asym | "
+                    f"rows gather + {info['name']} + scatter | {best:.1f} | {gbs:.0f} ({100 * gbs / HBM_PEAK_GBS:.1f} %) | "
+                    f"{tfs:.1f} ({100 * tfs / 1000 / 2.5:.1f} %) | {rl2:.1e} | {mab:.1e} |")
+        log(rows[-1])
+        for w in ws:
+            w.close()
+        dev.free(a_ptr)
+        dev.free(y_ptr)
+    op_line = (f"config 5 as 3 gather-matmul calls (wall time, gather and scatter included): {t_op:.1f} us in total, "
+               f"{flops_total / t_op / 1e6:.1f} TFLOP/s")
+    log(op_line)
     print("| Config | Shape (K->N) | M | dtype | GPU kernel | us | GB/s (% of 8 TB/s) | TFLOP/s (% of 2.5 PF) | "
           "rel-L2 vs fp32 | max-abs |")
     print("|---|---|---|---|---|---|---|---|---|---|")
@@ -144,6 +194,7 @@ def results_table(dev, req, args) -> int:
         print(r)
     print(f"\nconfig 5 as 24 separate launches: {t_total:.1f} us in total, {flops_total / t_total / 1e6:.1f} TFLOP/s")
     print(grouped_line)
+    print(op_line)
     req.close()
     dev.close()
     return 0

@@ -195,6 +195,21 @@ typedef struct ovfcc_group_item {
 } ovfcc_group_item;
 int ovfcc_fc_run_grouped_device(ovfcc_request* req, const ovfcc_group_item* items, int n_items);
 
+/* GatherMatmulCompressed (src/common/transformations/include/ov_ops/gather_matmul.hpp:17-41,
+ * gather_matmul_compressed.hpp:17-33; shapes src/common/transformations/src/ov_ops/gather_matmul.cpp:38-130; CPU
+ * executor src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_gathermatmul_executor.cpp:470-600): the expert
+ * matrices of a mixture-of-experts layer applied to routed rows.  experts[e] is expert e's node (B[e] of the op's
+ * [n_experts, N, K] constant, all of one shape and format); a_dev is A [a_batches, M, K] f16 in device memory with
+ * a_batches = 1 (every selected expert reads the same row) or top_k; indices [M, top_k] int32 in host memory names
+ * the experts of each row; y_dev receives [top_k, M, N_out]:
+ *     Y[i, m, :] = experts[indices[m, i]](A[a_batches == 1 ? 0 : i, m, :]).
+ * Rows are gathered per expert on the device, all experts run as one grouped launch
+ * (ovfcc_fc_run_grouped_device) and the results are scattered back; everything is enqueued on the request's
+ * stream.  An index outside [0, n_experts) is OVFCC_EINVAL. */
+int ovfcc_gather_matmul_device(ovfcc_request* req, const ovfcc_weights* const* experts, int n_experts,
+                               const void* a_dev, int a_batches, const int32_t* indices, int64_t M, int top_k,
+                               void* y_dev);
+
 /* Benchmark twin of ovfcc_bench_layers for grouped runs: `iters` eager calls of ovfcc_fc_run_grouped_device on the
  * request's stream, bracketed by HIP events on that stream. */
 int ovfcc_bench_grouped(ovfcc_request* req, const ovfcc_group_item* items, int n_items, int warmup, int iters,

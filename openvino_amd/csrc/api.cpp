@@ -39,6 +39,11 @@ struct ovfcc_request {
     size_t ws_cap = 0;
     unsigned* counters = nullptr;
     size_t counter_cap = 0;
+    void* d_gather = nullptr;  // gather-matmul: gathered rows, results before the scatter, row maps
+    size_t gather_cap = 0;
+    int* h_maps = nullptr;     // ... and the pinned host copy of the row maps, reused once its upload has finished
+    size_t h_maps_cap = 0;
+    hipEvent_t maps_uploaded = nullptr;
     int force_kernel = OVFCC_KERNEL_AUTO;
     int force_split = 0;
     ovfcc_kernel_info last{};
@@ -639,6 +644,9 @@ void ovfcc_request_destroy(ovfcc_request* r) {
     if (r->d_y) (void)hipFree(r->d_y);
     if (r->workspace) (void)hipFree(r->workspace);
     if (r->counters) (void)hipFree(r->counters);
+    if (r->d_gather) (void)hipFree(r->d_gather);
+    if (r->h_maps) (void)hipHostFree(r->h_maps);
+    if (r->maps_uploaded) (void)hipEventDestroy(r->maps_uploaded);
     delete r;
 }
 
@@ -802,6 +810,99 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
                 return rc;
         }
     }
+    return OVFCC_OK;
+}
+
+int ovfcc_gather_matmul_device(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, const void* a_dev,
+                               int a_batches, const int32_t* indices, int64_t M, int top_k, void* y_dev) {
+    if (!r || !experts || n_experts <= 0 || !indices || M < 0 || top_k <= 0)
+        return fail(OVFCC_EINVAL, "bad gather-matmul arguments");
+    if (a_batches != 1 && a_batches != top_k)
+        return fail(OVFCC_EINVAL, "A must have one batch or one batch per selected expert");
+    if (top_k > n_experts)
+        return fail(OVFCC_EINVAL, "more selected experts per row than experts");
+    if (M == 0)
+        return OVFCC_OK;
+    if (!a_dev || !y_dev)
+        return fail(OVFCC_EINVAL, "A or Y is null");
+    if (M * top_k > ((int64_t)1 << 24))
+        return fail(OVFCC_EUNSUPPORTED, "M * top_k is limited to 2^24");
+    const ovfcc_weights* w0 = experts[0];
+    for (int e = 0; e < n_experts; ++e) {
+        const ovfcc_weights* w = experts[e];
+        if (!w || w->ctx != r->ctx)
+            return fail(OVFCC_EINVAL, "an expert's weights are null or belong to another context");
+        if (std::memcmp(&w->desc, &w0->desc, sizeof(ovfcc_fc_desc)) != 0 || (w->d_bias != nullptr) != (w0->d_bias != nullptr))
+            return fail(OVFCC_EUNSUPPORTED, "experts differ in shape, types, bias or output type");
+    }
+    const int64_t K = w0->desc.K, N_out = out_channels(w0);
+    const size_t out_bytes = w0->desc.out_type == OVFCC_F32 ? 4 : 2;
+    if ((K * 2) % 16 != 0 || (N_out * out_bytes) % 16 != 0)
+        return fail(OVFCC_EUNSUPPORTED, "rows of A and Y must be multiples of 16 bytes");
+    HIP_TRY(hipSetDevice(r->ctx->device));
+
+    // rows of each expert, in row order: the bucketing of the reference's CPU executor
+    // (src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_gathermatmul_executor.cpp:492-509)
+    const int64_t R = M * top_k;
+    std::vector<int> count(n_experts, 0), start(n_experts + 1, 0);
+    for (int64_t m = 0; m < M; ++m)
+        for (int i = 0; i < top_k; ++i) {
+            const int32_t e = indices[m * top_k + i];
+            if (e < 0 || e >= n_experts)
+                return fail(OVFCC_EINVAL, "an expert index is out of range");
+            ++count[e];
+        }
+    for (int e = 0; e < n_experts; ++e)
+        start[e + 1] = start[e] + count[e];
+    // the maps go through pinned host memory owned by the request; the previous call's upload must have left it
+    const size_t map_bytes = (size_t)2 * R * sizeof(int);
+    if (!r->maps_uploaded)
+        HIP_TRY(hipEventCreateWithFlags(&r->maps_uploaded, hipEventDisableTiming));
+    else
+        HIP_TRY(hipEventSynchronize(r->maps_uploaded));
+    if (map_bytes > r->h_maps_cap) {
+        if (r->h_maps)
+            HIP_TRY(hipHostFree(r->h_maps));
+        r->h_maps = nullptr, r->h_maps_cap = 0;
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->h_maps), map_bytes, hipHostMallocDefault));
+        r->h_maps_cap = map_bytes;
+    }
+    std::vector<int> at(start.begin(), start.end() - 1);
+    int* src_row = r->h_maps;
+    int* dst_row = r->h_maps + R;
+    for (int64_t m = 0; m < M; ++m)
+        for (int i = 0; i < top_k; ++i) {
+            const int slot = at[indices[m * top_k + i]]++;
+            src_row[slot] = (int)(a_batches == 1 ? m : (int64_t)i * M + m);
+            dst_row[slot] = (int)((int64_t)i * M + m);
+        }
+
+    // one scratch allocation: gathered rows | results | row maps
+    const size_t x_bytes = (size_t)R * K * 2, y_bytes = (size_t)R * N_out * out_bytes;
+    const size_t x_off = 0, y_off = (x_bytes + 255) & ~(size_t)255, m_off = (y_off + y_bytes + 255) & ~(size_t)255;
+    if (m_off + map_bytes > r->gather_cap)
+        HIP_TRY(hipStreamSynchronize(r->stream));
+    int rc = grow(&r->d_gather, &r->gather_cap, m_off + map_bytes);
+    if (rc)
+        return rc;
+    char* base = static_cast<char*>(r->d_gather);
+    int* d_maps = reinterpret_cast<int*>(base + m_off);
+    HIP_TRY(hipMemcpyAsync(d_maps, r->h_maps, map_bytes, hipMemcpyHostToDevice, r->stream));
+    HIP_TRY(hipEventRecord(r->maps_uploaded, r->stream));
+    int e1 = ovfcc::launch_rows(base + x_off, a_dev, d_maps, nullptr, (int)R, (int)(K * 2), r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "row gather launch");
+    std::vector<ovfcc_group_item> items;
+    for (int e = 0; e < n_experts; ++e)
+        if (count[e])
+            items.push_back({experts[e], base + x_off + (size_t)start[e] * K * 2,
+                             base + y_off + (size_t)start[e] * N_out * out_bytes, (int64_t)count[e]});
+    rc = ovfcc_fc_run_grouped_device(r, items.data(), (int)items.size());
+    if (rc)
+        return rc;
+    e1 = ovfcc::launch_rows(y_dev, base + y_off, nullptr, d_maps + R, (int)R, (int)(N_out * out_bytes), r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "row scatter launch");
     return OVFCC_OK;
 }
 

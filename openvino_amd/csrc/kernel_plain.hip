@@ -98,6 +98,32 @@ __global__ __launch_bounds__(256) void fcc_touch_kernel(const uint4_t* __restric
     asm volatile("" ::"v"(acc.x), "v"(acc.y), "v"(acc.z), "v"(acc.w));  // keeps the loads alive
 }
 
+// ------------------------------------------------------------------------------------------------
+// Row gather / scatter for the mixture-of-experts entry point: dst row r = src row src_row[r] (gather, dst_row
+// null) or dst row dst_row[r] = src row r (scatter, src_row null); rows of row_bytes (a multiple of 16) bytes.
+// One workgroup per row.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fcc_rows_kernel(uint4_t* __restrict__ dst, const uint4_t* __restrict__ src,
+                                                       const int* __restrict__ src_row,
+                                                       const int* __restrict__ dst_row, int row_bytes) {
+    const int r = blockIdx.x;
+    const size_t from = (size_t)(src_row ? src_row[r] : r) * (row_bytes / 16);
+    const size_t to = (size_t)(dst_row ? dst_row[r] : r) * (row_bytes / 16);
+    for (int i = threadIdx.x; i < row_bytes / 16; i += blockDim.x)
+        dst[to + i] = src[from + i];
+}
+
+int launch_rows(void* dst, const void* src, const int* src_row, const int* dst_row, int rows, int row_bytes,
+                void* stream) {
+    if (rows <= 0)
+        return 0;
+    if (row_bytes <= 0 || (row_bytes & 15) || (!src_row == !dst_row))
+        return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(fcc_rows_kernel, dim3((unsigned)rows), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       (uint4_t*)dst, (const uint4_t*)src, src_row, dst_row, row_bytes);
+    return (int)hipGetLastError();
+}
+
 int launch_touch(const void* src, size_t bytes, void* stream) {
     const size_t n16 = bytes / 16;
     const unsigned blocks = (unsigned)((n16 + 256 * 4 - 1) / (256 * 4));  // four loads per thread

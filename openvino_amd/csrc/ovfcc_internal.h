@@ -140,6 +140,10 @@ int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* str
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
+// dst[r] = src[src_row[r]] (dst_row null) or dst[dst_row[r]] = src[r] (src_row null), rows of row_bytes % 16 == 0 bytes;
+// the caller guarantees that every index is a row of the buffer it addresses
+int launch_rows(void* dst, const void* src, const int* src_row, const int* dst_row, int rows, int row_bytes,
+                void* stream);
 int launch_touch(const void* src, size_t bytes, void* stream);
 
 constexpr int kDecodeMaxRows = 48;                       // rows one decode-family launch covers

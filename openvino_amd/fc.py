@@ -256,6 +256,39 @@ class InferRequest:
                 dev.free(xp)
                 dev.free(yp)
 
+    def gather_matmul_device(self, experts: Sequence[CompressedWeights], a_ptr: int, a_batches: int,
+                             indices: np.ndarray, y_ptr: int) -> None:
+        """GatherMatmulCompressed on device buffers: A [a_batches, M, K] at a_ptr, indices int32 [M, top_k] on the
+        host, Y [top_k, M, N_out] at y_ptr."""
+        idx = np.ascontiguousarray(indices, dtype=np.int32)
+        M, top_k = idx.shape
+        arr = (ctypes.c_void_p * len(experts))(*[w.handle for w in experts])
+        check(self.device.lib.ovfcc_gather_matmul_device(self.handle, arr, len(experts), ctypes.c_void_p(a_ptr), a_batches,
+                                                         idx.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), M, top_k,
+                                                         ctypes.c_void_p(y_ptr)))
+
+    def gather_matmul(self, experts: Sequence[CompressedWeights], A: np.ndarray, indices: np.ndarray) -> np.ndarray:
+        """Host convenience: A float16 [a_batches, M, K] (a_batches 1 or top_k), indices [M, top_k] -> Y [top_k, M, N_out]."""
+        A = np.ascontiguousarray(A, dtype=np.float16)
+        idx = np.ascontiguousarray(indices, dtype=np.int32)
+        M, top_k = idx.shape
+        w = experts[0]
+        if A.ndim != 3 or A.shape[1] != M or A.shape[2] != w.K:
+            raise OvfccError(_lib.EINVAL, f"A has shape {A.shape}, expected [1 or {top_k}, {M}, {w.K}]")
+        dt = np.float32 if w.desc.out_type == _lib.F32 else np.float16
+        if M == 0:
+            return np.empty((top_k, 0, w.N_out), dt)
+        dev = self.device
+        a_ptr, y_ptr = dev.malloc(A.nbytes), dev.malloc(top_k * M * w.N_out * np.dtype(dt).itemsize)
+        try:
+            dev.upload(a_ptr, A)
+            self.gather_matmul_device(experts, a_ptr, A.shape[0], idx, y_ptr)
+            self.sync()
+            return dev.download(y_ptr, (top_k, M, w.N_out), dt)
+        finally:
+            dev.free(a_ptr)
+            dev.free(y_ptr)
+
     def bench_grouped(self, items: Sequence[tuple], warmup: int, iters: int) -> float:
         """Milliseconds for `iters` grouped runs, HIP events on the launching stream."""
         arr = self._group_items(items)

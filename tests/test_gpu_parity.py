@@ -534,3 +534,48 @@ def test_weight_blob_export_import(oracle, dev, req):
     finally:
         for w in ws:
             w.close()
+
+
+def gather_matmul_reference(oracle, cases, A, indices):
+    """Y[i, m] = expert indices[m, i] applied to A[i or 0, m]: the op's definition
+    (src/common/transformations/src/ov_ops/gather_matmul.cpp:38-130), expert by expert with the FC oracle."""
+    M, top_k = indices.shape
+    N = cases[0].N
+    ref = np.zeros((top_k, M, N), np.float32)
+    for e, c in enumerate(cases):
+        for i in range(top_k):
+            rows = np.nonzero(indices[:, i] == e)[0]
+            if rows.size:
+                ref[i, rows] = oracle_y(oracle, c, x=A[i if A.shape[0] > 1 else 0, rows])
+    return ref
+
+
+@pytest.mark.parametrize("M,a_batches", [(1, 1), (5, 1), (64, 2), (200, 1), (200, 2)])
+def test_gather_matmul(oracle, dev, req, monkeypatch, M, a_batches):
+    """GatherMatmulCompressed: eight experts, top-2 routing from seeded logits (uneven loads, some experts idle at
+    small M); every output row against the oracle of the expert that the indices name."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    say(f"gather matmul M={M} a_batches={a_batches}")
+    E, top_k, K, N = 8, 2, 512, 256
+    cases = [datagen.make_case(860 + e, 1, K, N, "u4", 128, "u4", with_bias=True) for e in range(E)]
+    ws = [fc.CompressedWeights.from_case(dev, c) for c in cases]
+    rng = np.random.default_rng(870 + M)
+    logits = rng.standard_normal((M, E))
+    indices = np.argsort(-logits, axis=1, kind="stable")[:, :top_k].astype(np.int32)
+    A = rng.standard_normal((a_batches, M, K)).astype(np.float16)
+    try:
+        y = req.gather_matmul(ws, A, indices)
+        assert y.shape == (top_k, M, N)
+        ref = gather_matmul_reference(oracle, cases, A, indices)
+        check_parity(oracle, y.reshape(-1, N), ref.reshape(-1, N), K, f"M={M} {req.last_kernel()}",
+                     output_rounding_slack=True)
+        assert np.array_equal(req.gather_matmul(ws, A, indices).view(np.uint16), y.view(np.uint16))
+        bad = indices.copy()
+        bad[0, 0] = E
+        with pytest.raises(fc.OvfccError):
+            req.gather_matmul(ws, A, bad)
+        with pytest.raises(fc.OvfccError):
+            req.gather_matmul_device(ws, 0, 3, indices, 0)        # a_batches neither 1 nor top_k
+    finally:
+        for w in ws:
+            w.close()
