@@ -179,3 +179,28 @@ def test_glu_grouped_run(oracle, dev, req, monkeypatch):
     finally:
         for w in ws:
             w.close()
+
+
+def test_glu_gather_matmul(oracle, dev, req, monkeypatch):
+    """A mixture-of-experts gate/up stage with fused SwiGLU through the GatherMatmulCompressed entry point."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    say("glu gather matmul")
+    E, top_k, K, N, M = 4, 2, 512, 512, 150
+    cases = [datagen.make_case(950 + e, 1, K, N, "i4", 128, "none") for e in range(E)]
+    ws = [fc.CompressedWeights.from_case(dev, c, glu="swish") for c in cases]
+    rng = np.random.default_rng(951)
+    indices = np.argsort(-rng.standard_normal((M, E)), axis=1, kind="stable")[:, :top_k].astype(np.int32)
+    A = rng.standard_normal((1, M, K)).astype(np.float16)
+    try:
+        y = req.gather_matmul(ws, A, indices)
+        assert y.shape == (top_k, M, N // 2)
+        for e, c in enumerate(cases):
+            for i in range(top_k):
+                rows = np.nonzero(indices[:, i] == e)[0]
+                if rows.size:
+                    ref, amp = glu_reference(oracle, c, "swish", x=A[0, rows])
+                    check_parity(oracle, y[i, rows], ref, K, f"expert {e} slot {i}", output_rounding_slack=True,
+                                 limit_scale=amp)
+    finally:
+        for w in ws:
+            w.close()
