@@ -579,3 +579,49 @@ def test_gather_matmul(oracle, dev, req, monkeypatch, M, a_batches):
     finally:
         for w in ws:
             w.close()
+
+
+def test_requests_on_concurrent_threads(oracle, dev):
+    """Different requests may run concurrently from different threads (the reference runs infer requests on a
+    task executor): four threads, one request each, shared weights, mixed row counts; every result bit-equal to
+    the single-threaded one, errors stay on the thread that caused them."""
+    import threading
+    say("concurrent threads")
+    c = datagen.make_case(880, 300, 1024, 512, "u4", 128, "u4", with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c)
+    rows = [1, 7, 40, 100, 300]
+    one = fc.InferRequest(dev)
+    want = {m: one.infer(w, c.x[:m]) for m in rows}
+    one.close()
+    failures = []
+
+    def work(tid):
+        req = fc.InferRequest(dev)
+        try:
+            for it in range(20):
+                m = rows[(it + tid) % len(rows)]
+                y = req.infer(w, c.x[:m])
+                if not np.array_equal(y.view(np.uint16), want[m].view(np.uint16)):
+                    failures.append((tid, it, m))
+                if it % 7 == 3:
+                    try:
+                        req.infer(w, c.x[:m, :100])
+                        failures.append((tid, it, "no error"))
+                    except fc.OvfccError as e:
+                        if "K" not in str(e):
+                            failures.append((tid, it, str(e)))
+        except Exception as e:  # noqa: BLE001 - reported below
+            failures.append((tid, repr(e)))
+        finally:
+            req.close()
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    try:
+        assert not any(t.is_alive() for t in threads)
+        assert not failures, failures[:5]
+    finally:
+        w.close()
