@@ -42,6 +42,19 @@
  *                    tanh form), the identities act(x) - act(-x) = x, act(0) = 0, and the
  *                    roles of the two halves on one-hot inputs.
  *
+ *   dynquant         per-token symmetric int8 quantisation of activations and the integer
+ *                    FullyConnected on top of it, as the Intel-GPU plugin does for large batches:
+ *                    src/plugins/intel_gpu/src/kernel_selector/cl_kernels/dynamic_quantize_gpu_ref.cl:100-250
+ *                    (max |x| clamped below at 0.003, scale = 127 / max in half, q = rte(half(x * scale)),
+ *                    stored scale 1 / scale, sum of q), fully_connected_gpu_bf_tiled.cl:1283-1284
+ *                    ((acc - zp * sum) * weight scale * stored scale); attributes
+ *                    src/common/transformations/include/ov_ops/dynamic_quantize.hpp:16-60.  The reference
+ *                    holds no numeric vector for it (its tests compare against the unquantised result with
+ *                    absolute tolerances 0.1-0.2).  Pinned by: exact round trip on rows that are integer
+ *                    multiples of max / 127; |x - q * stored scale| <= stored scale / 2 (+ half rounding);
+ *                    sum and range of q; an independent numpy restatement; and, for the FC, equality with
+ *                    ovo_fc_reference applied to the dequantised activations q * stored scale.
+ *
  * Parity unpinned: the CPU plugin's numbers come from the oneDNN fork's decompression
  * inner-product kernel (openvinotoolkit/oneDNN, a submodule whose commit the tree does
  * not record and whose sources are absent).  Its summation order and intermediate
@@ -315,6 +328,57 @@ int ovo_glu(const float* y, int64_t M, int64_t L, int32_t type, int32_t gate_sec
             else
                 a = 0.5 * gate * (1.0 + tanh(0.79788456080286535588 * gate * (1.0 + 0.044715 * gate * gate)));
             out[m * L + f] = (float)(a * up);
+        }
+    return 0;
+}
+
+/* Per-token symmetric int8 quantisation of x [M, K] (f16 bit patterns): q [M, K], inv_scale [M] (the f16 value
+ * the reference stores, returned as float), qsum [M] = sum_k q.  Half arithmetic as in the reference kernel:
+ * max and product are exact half operations; 127 / max is one f32 division rounded to half, which equals the half
+ * division (a quotient of two 11-bit significands cannot lie within 2^-24 of a 12-bit tie). */
+int ovo_dynquant_rows(const uint16_t* x, int64_t M, int64_t K, int8_t* q, float* inv_scale, int32_t* qsum) {
+    if (!x || !q || !inv_scale || !qsum || M < 0 || K <= 0)
+        return -1;
+    for (int64_t m = 0; m < M; ++m) {
+        float mx = ovo_f16_to_f32(ovo_f32_to_f16(0.003f));
+        for (int64_t k = 0; k < K; ++k) {
+            const float a = fabsf(ovo_f16_to_f32(x[m * K + k]));
+            if (a > mx)
+                mx = a;
+        }
+        const float scale = ovo_f16_to_f32(ovo_f32_to_f16(127.0f / mx));
+        int32_t sum = 0;
+        for (int64_t k = 0; k < K; ++k) {
+            const float v = ovo_f16_to_f32(ovo_f32_to_f16(ovo_f16_to_f32(x[m * K + k]) * scale));
+            const float r = nearbyintf(v);  /* round to nearest even, the default mode */
+            const int32_t i = (int32_t)(r > 127.f ? 127.f : (r < -128.f ? -128.f : r));
+            q[m * K + k] = (int8_t)i;
+            sum += i;
+        }
+        inv_scale[m] = ovo_f16_to_f32(ovo_f32_to_f16(1.0f / scale));
+        qsum[m] = sum;
+    }
+    return 0;
+}
+
+/* FullyConnected over dynamically quantised activations, 8-bit weights, one scale (and zero-point) per output
+ * channel: y[m, n] = (sum_k q[m, k] w[n, k] - zp[n] qsum[m]) * (scale[n] * inv_scale[m]) (+ bias[n]), integers
+ * exact, the rest in f32.  w_signed: weights are i8 instead of u8.  zp may be null (0), bias may be null. */
+int ovo_fc_dynquant_reference(const int8_t* q, const float* inv_scale, const int32_t* qsum, int64_t M, int64_t K,
+                              int64_t N, const uint8_t* w, int32_t w_signed, const float* scale, const float* zp,
+                              const float* bias, float* y) {
+    if (!q || !inv_scale || !qsum || !w || !scale || !y || M < 0 || K <= 0 || N <= 0)
+        return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t m = 0; m < M; ++m) {
+            int64_t acc = 0;
+            for (int64_t k = 0; k < K; ++k) {
+                const int32_t wv = w_signed ? (int32_t)(int8_t)w[n * K + k] : (int32_t)w[n * K + k];
+                acc += (int32_t)q[m * K + k] * wv;
+            }
+            acc -= (int64_t)(zp ? (int32_t)zp[n] : 0) * qsum[m];
+            y[m * N + n] = (float)(int32_t)acc * (scale[n] * inv_scale[m]) + (bias ? bias[n] : 0.f);
         }
     return 0;
 }
