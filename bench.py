@@ -89,6 +89,33 @@ def results_table(dev, req, args) -> int:
         run(3, shape, datagen.config3(shape, 8192), [512, 2048, 8192], 4, 0.0, "i4 g128 sym")
     for shape in datagen.LLAMA3_70B_SHAPES:
         run(4, shape, datagen.config4(shape, 1024), [1, 32, 1024], 8, 1.0, "u8 per-channel asym")
+    # Config 4's prefill row again with the node's activations allowed to be quantised per token to int8 (W8A8):
+    # checked against the oracle of that arithmetic (exact integers) and, for reference, against the f16 oracle.
+    for shape in datagen.LLAMA3_70B_SHAPES:
+        c = datagen.config4(shape, 1024)
+        w = fc.CompressedWeights.from_case(dev, c, dynamic_quantization=True)
+        x_dev, y_dev = dev.malloc(c.x.nbytes), dev.malloc(c.M * c.N * 2)
+        dev.upload(x_dev, c.x)
+        y = req.infer(w, c.x).astype(np.float32)
+        info = req.last_kernel()
+        pick = np.sort(np.random.default_rng(99).choice(c.M, size=8, replace=False))
+        zp = c.zp.astype(np.float32)
+        ref_q = oracle.fc_dynquant_reference(c.x[pick], c.w, type_tag[c.w_type], c.scale, zp, None, N=c.N, K=c.K)
+        ref_f = oracle.fc_reference(c.x[pick], c.w, type_tag[c.w_type], c.scale, c.zp, type_tag[c.zp_type], None,
+                                    N=c.N, K=c.K, group_size=c.group_size)
+        us = min(req.bench_layers([w], x_dev, y_dev, c.M, 3, 10, use_graph=True) for _ in range(2)) / 10 * 1e3
+        nbytes = algorithmic_bytes(c.K, c.N, c.M, 8, c.group_size, 1.0)
+        gbs, tfs = nbytes / us / 1e3, 2.0 * c.M * c.N * c.K / us / 1e6
+        quantised = info["name"] == "fcc_prefill_i8_w8"
+        rows.append(f"| 4 | {shape} {c.K}->{c.N}, int8 activations allowed | {c.M} | u8 per-channel asym"
+                    f"{' x i8 per token' if quantised else ''} | {'fcc_dynquant + ' if quantised else ''}{info['name']} | "
+                    f"{us:.1f} | {gbs:.0f} ({100 * gbs / HBM_PEAK_GBS:.1f} %) | {tfs:.1f} ({100 * tfs / 1000 / 2.5:.1f} % of f16 peak) | "
+                    f"{oracle.rel_l2(y[pick], ref_q if quantised else ref_f):.1e} vs its own oracle, "
+                    f"{oracle.rel_l2(y[pick], ref_f):.1e} vs f16 | {oracle.max_abs(y[pick], ref_q if quantised else ref_f):.1e} |")
+        log(rows[-1])
+        w.close()
+        dev.free(x_dev)
+        dev.free(y_dev)
     routes = datagen.moe_routing()
     t_total, flops_total = 0.0, 0.0
     for e, tokens in enumerate(routes):

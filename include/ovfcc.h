@@ -79,6 +79,20 @@ typedef struct ovfcc_fc_desc {
 #define OVFCC_GLU_TYPE_MASK 3
 #define OVFCC_GLU_GATE_SECOND 4
 
+/* Dynamic quantisation of the activations (flags), the counterpart of ov::hint::dynamic_quantization_group_size
+ * with per-token groups: the reference's plugins quantise FullyConnected activations to int8 on the fly
+ * (ov::op::internal::DynamicQuantize, src/common/transformations/include/ov_ops/dynamic_quantize.hpp:16-60; Intel
+ * GPU: cl_kernels/dynamic_quantize_gpu_ref.cl:100-250 and the integer path of
+ * cl_kernels/fully_connected_gpu_bf_tiled.cl:1257-1291, for batches above a threshold only).  The flag is a
+ * permission, not a request for a specific kernel: it takes effect for 8-bit weights with one scale per output
+ * channel, N % 256 == 0, K % 128 == 0, no gated linear unit, and more than 48 rows; every other call of the node
+ * computes in f16 as without the flag.  Where it takes effect,
+ *     q[m, k] = rte(half(x[m, k] * half(127 / max(0.003, max_k |x[m, k]|)))),
+ *     y[m, n] = (sum_k q[m, k] W[n, k] - ZP[n] sum_k q[m, k]) * (S[n] * half(1 / scale_m)) + bias[n],
+ * integers exact, which differs from the f16 result by the quantisation noise (about 1e-2 relative; the
+ * reference tests such nodes with absolute tolerances of 0.1-0.2). */
+#define OVFCC_DYNQUANT_I8 8
+
 typedef struct ovfcc_ctx ovfcc_ctx;         /* one device + its kernels */
 typedef struct ovfcc_weights ovfcc_weights; /* repacked, device-resident W/S/ZP/bias of one node */
 typedef struct ovfcc_request ovfcc_request; /* one HIP stream + staging + split-K workspace */

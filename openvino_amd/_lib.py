@@ -13,6 +13,7 @@ TYPE = {"none": NONE, "u4": U4, "i4": I4, "u8": U8, "i8": I8, "f16": F16, "f32":
 KERNEL_AUTO, KERNEL_PLAIN, KERNEL_DECODE, KERNEL_PREFILL = range(4)
 GLU = {None: 0, "none": 0, "swish": 1, "gelu": 2, "gelu_tanh": 3}      # OVFCC_GLU_*
 GLU_GATE_SECOND = 4
+DYNQUANT_I8 = 8                                                        # OVFCC_DYNQUANT_I8
 
 # every symbol include/ovfcc.h declares
 SYMBOLS = [

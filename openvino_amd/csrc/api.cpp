@@ -41,6 +41,8 @@ struct ovfcc_request {
     size_t counter_cap = 0;
     void* d_gather = nullptr;  // gather-matmul: gathered rows, results before the scatter, row maps
     size_t gather_cap = 0;
+    void* d_quant = nullptr;   // dynamic quantisation: int8 activations, inverse scales, sums
+    size_t quant_cap = 0;
     int* h_maps = nullptr;     // ... and the pinned host copy of the row maps, reused once its upload has finished
     size_t h_maps_cap = 0;
     hipEvent_t maps_uploaded = nullptr;
@@ -148,6 +150,39 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
     ovfcc::FcDeviceArgs a;
     fill_args(w, x, y, M, &a);
     int force = r->force_kernel;
+    // Per-token int8 activations where the node allows them and the integer kernel applies: prefill row counts,
+    // 8-bit weights with one scale per channel, whole 256-channel tiles.
+    const ovfcc::Layout& L0 = w->layout;
+    if (L0.dynquant && L0.tiled && L0.bits == 8 && L0.groups == 1 && !L0.glu && (w->desc.N % 256) == 0 &&
+        M > ovfcc::kDecodeMaxRows && (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL) &&
+        M * w->desc.K < ((int64_t)1 << 31) && (M + 127) / 128 <= 65535 &&
+        // (it has no split-K: a grid that leaves half the chip idle stays with the f16 kernels, which have;
+        // OVFCC_PREFILL_WIDE = 1 forces the 256-wide kernels onto small shapes, for tests)
+        ((w->desc.N / 256) * ((M + 127) / 128) * 2 >= r->ctx->n_cus ||
+         (std::getenv("OVFCC_PREFILL_WIDE") && std::atoi(std::getenv("OVFCC_PREFILL_WIDE")) == 1))) {
+        const size_t q_bytes = ((size_t)M * w->desc.K + 255) & ~(size_t)255;
+        const size_t need = q_bytes + (size_t)M * 8;
+        if (need > r->quant_cap)
+            HIP_TRY(hipStreamSynchronize(r->stream));
+        int rc = grow(&r->d_quant, &r->quant_cap, need);
+        if (rc)
+            return rc;
+        char* base = static_cast<char*>(r->d_quant);
+        float* inv_scale = reinterpret_cast<float*>(base + q_bytes);
+        int* qsum = reinterpret_cast<int*>(base + q_bytes + (size_t)M * 4);
+        int e = ovfcc::launch_dynquant(x, base, inv_scale, qsum, M, w->desc.K, r->stream);
+        if (!e)
+            e = ovfcc::launch_prefill_i8(a, base, inv_scale, qsum, r->stream);
+        if (e)
+            return hip_fail((hipError_t)e, "integer kernel launch");
+        ovfcc::LaunchPlan shown;
+        shown.kernel = OVFCC_KERNEL_PREFILL;
+        shown.tile_m = 128, shown.tile_n = 256, shown.block = 512;
+        shown.grid[0] = (unsigned)(w->desc.N / 256), shown.grid[1] = (unsigned)((M + 127) / 128);
+        shown.name = "fcc_prefill_i8_w8";
+        record(r, shown);
+        return OVFCC_OK;
+    }
     bool chunked = w->layout.tiled && M > ovfcc::kDecodeMaxRows &&
                    ((force == OVFCC_KERNEL_AUTO && M <= ovfcc::kChunkedMaxRows) ||
                     ((w->desc.N % 128) != 0 && (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL)));
@@ -645,6 +680,7 @@ void ovfcc_request_destroy(ovfcc_request* r) {
     if (r->workspace) (void)hipFree(r->workspace);
     if (r->counters) (void)hipFree(r->counters);
     if (r->d_gather) (void)hipFree(r->d_gather);
+    if (r->d_quant) (void)hipFree(r->d_quant);
     if (r->h_maps) (void)hipHostFree(r->h_maps);
     if (r->maps_uploaded) (void)hipEventDestroy(r->maps_uploaded);
     delete r;

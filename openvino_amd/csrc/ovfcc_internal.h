@@ -44,6 +44,7 @@ struct Layout {
     // so that the wave that finishes a gate tile also holds the matching up tile.
     int glu = 0;
     bool glu_gate_second = false;
+    bool dynquant = false;  // the node allows per-token int8 activations (OVFCC_DYNQUANT_I8) where a kernel exists
     // 16-channel block of the OpenVINO-order channel axis that tile nt holds
     int64_t source_tile(int64_t nt) const {
         if (!glu)
@@ -139,6 +140,11 @@ int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+// Per-row int8 quantisation of x [M, K] f16 (K % 128 == 0): xq [M, K] in the weight tiles' input order, one
+// inverse scale and one sum of quantised values per row.
+int launch_dynquant(const void* x, void* xq, float* inv_scale, int* qsum, int64_t M, int64_t K, void* stream);
+// Integer prefill kernel over launch_dynquant's outputs: tiled 8-bit weights, one group per channel, N % 256 == 0.
+int launch_prefill_i8(const FcDeviceArgs& a, const void* xq, const float* inv_scale, const int* qsum, void* stream);
 int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
 // dst[r] = src[src_row[r]] (dst_row null) or dst[dst_row[r]] = src[r] (src_row null), rows of row_bytes % 16 == 0 bytes;
 // the caller guarantees that every index is a row of the buffer it addresses

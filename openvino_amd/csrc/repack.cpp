@@ -63,7 +63,7 @@ int validate_desc(const ovfcc_fc_desc* d) {
         return fail(OVFCC_EUNSUPPORTED, "activations must be f16");
     if (d->out_type != OVFCC_F16 && d->out_type != OVFCC_F32)
         return fail(OVFCC_EUNSUPPORTED, "output must be f16 or f32");
-    if (d->flags & ~(OVFCC_GLU_TYPE_MASK | OVFCC_GLU_GATE_SECOND))
+    if (d->flags & ~(OVFCC_GLU_TYPE_MASK | OVFCC_GLU_GATE_SECOND | OVFCC_DYNQUANT_I8))
         return fail(OVFCC_EINVAL, "unknown bits in flags");
     if ((d->flags & OVFCC_GLU_GATE_SECOND) && (d->flags & OVFCC_GLU_TYPE_MASK) == OVFCC_GLU_NONE)
         return fail(OVFCC_EINVAL, "OVFCC_GLU_GATE_SECOND without a gated-linear-unit type");
@@ -82,6 +82,7 @@ Layout make_layout(const ovfcc_fc_desc& d) {
     L.zp_table = d.zp_type != OVFCC_NONE && !d.zp_scalar;
     L.zp_const = L.zp_offset;
     // K / 128 < 2^16 keeps the kernels' 32-bit offsets and reciprocal group index exact
+    L.dynquant = (d.flags & OVFCC_DYNQUANT_I8) != 0;
     L.glu = d.flags & OVFCC_GLU_TYPE_MASK;
     L.glu_gate_second = (d.flags & OVFCC_GLU_GATE_SECOND) != 0;
     L.tiled = (d.N % (L.glu ? 2 * kTileRows : kTileRows) == 0) && (d.K % kBlockK == 0) &&

@@ -22,7 +22,7 @@ def _vp(a: Optional[np.ndarray]):
 
 def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
               has_bias: bool = False, out_type: str = "f16", glu: Optional[str] = None,
-              glu_gate_second: bool = False) -> FcDesc:
+              glu_gate_second: bool = False, dynamic_quantization: bool = False) -> FcDesc:
     d = FcDesc()
     d.N, d.K, d.group_size = N, K, group_size
     d.w_type = _lib.TYPE[w_type]
@@ -32,7 +32,8 @@ def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none
     d.bias_type = _lib.F16 if has_bias else _lib.NONE
     d.act_type = _lib.F16
     d.out_type = _lib.TYPE[out_type]
-    d.flags = _lib.GLU[glu] | (_lib.GLU_GATE_SECOND if glu_gate_second else 0)
+    d.flags = (_lib.GLU[glu] | (_lib.GLU_GATE_SECOND if glu_gate_second else 0) |
+               (_lib.DYNQUANT_I8 if dynamic_quantization else 0))
     return d
 
 
@@ -86,13 +87,14 @@ class CompressedWeights:
 
     def __init__(self, device: Device, W: np.ndarray, weight_scales: np.ndarray, weight_zero_points=None, bias=None, *,
                  N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
-                 output_type: str = "f16", glu: Optional[str] = None, glu_gate_second: bool = False):
+                 output_type: str = "f16", glu: Optional[str] = None, glu_gate_second: bool = False,
+                 dynamic_quantization: bool = False):
         """glu = "swish" | "gelu" | "gelu_tanh": W holds gate and up projection ([N, K], first and second half of
         the rows, or the other way round with glu_gate_second) and the node computes act(gate) * up, [M, N / 2]."""
         self.device = device
         self.N, self.K, self.group_size = N, K, group_size
         self.desc = make_desc(N, K, group_size, w_type, zp_type if weight_zero_points is not None else "none",
-                              zp_scalar, bias is not None, output_type, glu, glu_gate_second)
+                              zp_scalar, bias is not None, output_type, glu, glu_gate_second, dynamic_quantization)
         W = np.ascontiguousarray(W).view(np.uint8)
         s = np.ascontiguousarray(weight_scales, dtype=np.float16)
         z = None if weight_zero_points is None else np.ascontiguousarray(weight_zero_points, dtype=np.uint8)
@@ -104,10 +106,10 @@ class CompressedWeights:
 
     @classmethod
     def from_case(cls, device: Device, c, output_type: str = "f16", glu: Optional[str] = None,
-                  glu_gate_second: bool = False) -> "CompressedWeights":
+                  glu_gate_second: bool = False, dynamic_quantization: bool = False) -> "CompressedWeights":
         return cls(device, c.w, c.scale, c.zp, c.bias, N=c.N, K=c.K, group_size=c.group_size, w_type=c.w_type,
                    zp_type=c.zp_type, zp_scalar=c.zp_scalar, output_type=output_type, glu=glu,
-                   glu_gate_second=glu_gate_second)
+                   glu_gate_second=glu_gate_second, dynamic_quantization=dynamic_quantization)
 
     @property
     def N_out(self) -> int:
