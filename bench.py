@@ -241,7 +241,7 @@ def main() -> int:
     ap.add_argument("--table", action="store_true",
                     help="time and parity-check every benchmark configuration (1-5) and print a markdown table on "
                          "stdout instead of the JSON line")
-    ap.add_argument("--profile", choices=["decode", "prefill"], default=None,
+    ap.add_argument("--profile", choices=["decode", "prefill", "w8a8"], default=None,
                     help="short run for rocprofv3: one copy-kernel launch of known size (the counter yardstick), "
                          "then a few eager passes of the chosen kernel family; prints no JSON")
     args = ap.parse_args()
@@ -288,7 +288,20 @@ def main() -> int:
     if args.profile:
         # yardstick: one 256 MiB device-to-device copy (reads 256 MiB, writes 256 MiB)
         dev.copy_bandwidth(256 << 20, 1)
-        if args.profile == "decode":
+        if args.profile == "w8a8":
+            # Llama-3-70B u8 per-channel projections at M = 1024, int8 activations allowed (config 4 of the table)
+            for shape in ("qo", "gate_up", "down"):
+                c = datagen.config4(shape, 1024)
+                w = fc.CompressedWeights.from_case(dev, c, dynamic_quantization=True)
+                xq_dev, yq_dev = dev.malloc(c.x.nbytes), dev.malloc(c.M * c.N * 2)
+                dev.upload(xq_dev, c.x)
+                for _ in range(3):
+                    req.infer_device(w, xq_dev, yq_dev, c.M)
+                req.sync()
+                w.close()
+                dev.free(xq_dev)
+                dev.free(yq_dev)
+        elif args.profile == "decode":
             for _ in range(3):
                 for _, w in layers:
                     req.infer_device(w, x_dev, y_dev, 1)
