@@ -22,8 +22,11 @@
 //
 // This file needs OpenVINO's developer headers and libopenvino to build; it is not part of libovfcc.so.
 #include <cstring>
+#include <istream>
 #include <memory>
 #include <mutex>
+#include <ostream>
+#include <sstream>
 #include <string>
 #include <vector>
 
@@ -38,6 +41,7 @@
 #include "openvino/op/result.hpp"
 #include "openvino/op/subtract.hpp"
 #include "openvino/op/transpose.hpp"
+#include "openvino/pass/serialize.hpp"
 #include "openvino/runtime/icompiled_model.hpp"
 #include "openvino/runtime/internal_properties.hpp"
 #include "openvino/runtime/iplugin.hpp"
@@ -254,16 +258,45 @@ public:
         size_t input_index = 0, output_index = 0;
     };
 
+    // node_flags: OVFCC_* flags for every node's descriptor (OVFCC_DYNQUANT_I8 when the caller allows dynamic
+    // quantisation); blobs: the repacked nodes of an exported model, in result order, instead of a fresh repack
     CompiledModel(const std::shared_ptr<ov::Model>& model, const std::shared_ptr<const ov::IPlugin>& plugin,
-                  ovfcc_ctx* ctx, bool profiling);
+                  ovfcc_ctx* ctx, bool profiling, int node_flags,
+                  const std::vector<std::vector<uint8_t>>* blobs = nullptr);
     ~CompiledModel() override {
         for (auto& n : m_nodes)
             ovfcc_weights_destroy(n.weights);
     }
 
-    void export_model(std::ostream&) const override {
-        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: export_model (caching the repacked weights) is not implemented");
+    // Stream layout: magic, node flags, the model as the template plugin stores it (xml and constants from
+    // ov::pass::Serialize, each behind its size; src/plugins/template/src/compiled_model.cpp:173-192), then the
+    // number of nodes and every node's repacked device image (ovfcc_weights_export) behind its size.
+    void export_model(std::ostream& out) const override {
+        std::stringstream xml, bin;
+        ov::pass::Serialize(xml, bin).run_on_model(m_model);
+        const std::string x = xml.str(), b = bin.str();
+        auto put = [&out](const void* p, uint64_t n) {
+            out.write(reinterpret_cast<const char*>(&n), sizeof(n));
+            out.write(static_cast<const char*>(p), static_cast<std::streamsize>(n));
+        };
+        out.write(kExportMagic, sizeof(kExportMagic));
+        const int32_t flags = m_node_flags;
+        out.write(reinterpret_cast<const char*>(&flags), sizeof(flags));
+        put(x.data(), x.size());
+        put(b.data(), b.size());
+        const uint64_t count = m_nodes.size();
+        out.write(reinterpret_cast<const char*>(&count), sizeof(count));
+        for (const auto& n : m_nodes) {
+            size_t bytes = 0;
+            if (ovfcc_weights_export_size(n.weights, &bytes) != OVFCC_OK)
+                throw_last("weights_export_size");
+            std::vector<uint8_t> blob(bytes);
+            if (ovfcc_weights_export(n.weights, blob.data(), bytes) != OVFCC_OK)
+                throw_last("weights_export");
+            put(blob.data(), blob.size());
+        }
     }
+    static constexpr char kExportMagic[8] = {'O', 'V', 'F', 'C', 'C', 'M', '0', '1'};
     std::shared_ptr<const ov::Model> get_runtime_model() const override {
         return m_model;
     }
@@ -298,6 +331,7 @@ private:
     std::shared_ptr<ov::Model> m_model;
     std::vector<Node> m_nodes;
     ovfcc_ctx* m_ctx;
+    int m_node_flags = 0;
     bool m_profiling;
 };
 
@@ -396,13 +430,17 @@ public:
     std::shared_ptr<ov::ICompiledModel> compile_model(const std::shared_ptr<const ov::Model>& model,
                                                       const ov::AnyMap& properties) const override {
         bool profiling = m_profiling;
+        uint64_t dq_group = m_dq_group;
         for (const auto& kv : properties) {
             if (kv.first == ov::enable_profiling.name())
                 profiling = kv.second.as<bool>();
+            else if (kv.first == ov::hint::dynamic_quantization_group_size.name())
+                dq_group = kv.second.as<uint64_t>();
             else if (!known_hint(kv.first))
                 OPENVINO_THROW("MI355X: unsupported property ", kv.first);
         }
-        return std::make_shared<CompiledModel>(model->clone(), shared_from_this(), context(), profiling);
+        return std::make_shared<CompiledModel>(model->clone(), shared_from_this(), context(), profiling,
+                                               dq_group != 0 ? OVFCC_DYNQUANT_I8 : 0);
     }
     std::shared_ptr<ov::ICompiledModel> compile_model(const std::shared_ptr<const ov::Model>& model,
                                                       const ov::AnyMap& properties,
@@ -414,6 +452,8 @@ public:
         for (const auto& kv : properties) {
             if (kv.first == ov::enable_profiling.name())
                 m_profiling = kv.second.as<bool>();
+            else if (kv.first == ov::hint::dynamic_quantization_group_size.name())
+                m_dq_group = kv.second.as<uint64_t>();  // non-zero: activations may be quantised per token
             else if (!known_hint(kv.first))
                 OPENVINO_THROW("MI355X: unsupported property ", kv.first);
         }
@@ -431,15 +471,22 @@ public:
                 {ov::range_for_async_infer_requests.name(), ov::PropertyMutability::RO},
                 {ov::execution_devices.name(), ov::PropertyMutability::RO},
                 {ov::enable_profiling.name(), ov::PropertyMutability::RW},
+                {ov::hint::dynamic_quantization_group_size.name(), ov::PropertyMutability::RW},
                 {ov::hint::performance_mode.name(), ov::PropertyMutability::RW},
                 {ov::hint::inference_precision.name(), ov::PropertyMutability::RW},
                 {ov::hint::num_requests.name(), ov::PropertyMutability::RW},
                 {ov::num_streams.name(), ov::PropertyMutability::RW},
                 {ov::device::id.name(), ov::PropertyMutability::RW},
             };
-        // no caching_properties: export_model / import_model are not implemented, so Core must not try
+        // caching_properties tells Core which properties key a cache entry (src/inference/src/dev/plugin.cpp:115-118)
         if (name == ov::internal::supported_properties)
-            return decltype(ov::internal::supported_properties)::value_type{};
+            return decltype(ov::internal::supported_properties)::value_type{
+                {ov::internal::caching_properties.name(), ov::PropertyMutability::RO}};
+        if (name == ov::internal::caching_properties)
+            return std::vector<ov::PropertyName>{ov::device::architecture.name(),
+                                                 ov::hint::dynamic_quantization_group_size.name()};
+        if (name == ov::hint::dynamic_quantization_group_size)
+            return m_dq_group;
         if (name == ov::available_devices)
             return decltype(ov::available_devices)::value_type{"0"};
         if (name == ov::device::full_name)
@@ -449,7 +496,8 @@ public:
         if (name == ov::device::type)
             return decltype(ov::device::type)::value_type{ov::device::Type::DISCRETE};
         if (name == ov::device::capabilities)
-            return decltype(ov::device::capabilities)::value_type{ov::device::capability::FP16};
+            return decltype(ov::device::capabilities)::value_type{ov::device::capability::FP16,
+                                                                  ov::device::capability::EXPORT_IMPORT};
         if (name == ov::execution_devices)
             return decltype(ov::execution_devices)::value_type{get_device_name()};
         if (name == ov::range_for_async_infer_requests)
@@ -475,19 +523,55 @@ public:
     ov::SoPtr<ov::IRemoteContext> get_default_context(const ov::AnyMap&) const override {
         OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: remote contexts are not implemented");
     }
-    std::shared_ptr<ov::ICompiledModel> import_model(std::istream&, const ov::AnyMap&) const override {
-        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: import_model is not implemented");
+    // The reverse of CompiledModel::export_model: the model is read back through Core, the nodes are rebuilt from
+    // their device images without repacking (template: src/plugins/template/src/plugin.cpp:230-311).
+    std::shared_ptr<ov::ICompiledModel> import_model(std::istream& in, const ov::AnyMap& properties) const override {
+        char magic[sizeof(CompiledModel::kExportMagic)];
+        in.read(magic, sizeof(magic));
+        if (!in || std::memcmp(magic, CompiledModel::kExportMagic, sizeof(magic)) != 0)
+            OPENVINO_THROW("MI355X: the stream does not hold a model exported by this plugin");
+        int32_t flags = 0;
+        in.read(reinterpret_cast<char*>(&flags), sizeof(flags));
+        auto get = [&in](std::vector<uint8_t>& v) {
+            uint64_t n = 0;
+            in.read(reinterpret_cast<char*>(&n), sizeof(n));
+            if (!in || n > (uint64_t(1) << 40))
+                OPENVINO_THROW("MI355X: damaged model stream");
+            v.resize(n);
+            in.read(reinterpret_cast<char*>(v.data()), static_cast<std::streamsize>(n));
+            if (!in)
+                OPENVINO_THROW("MI355X: truncated model stream");
+        };
+        std::vector<uint8_t> xml, bin;
+        get(xml);
+        get(bin);
+        uint64_t count = 0;
+        in.read(reinterpret_cast<char*>(&count), sizeof(count));
+        if (!in || count > 65536)
+            OPENVINO_THROW("MI355X: damaged model stream");
+        std::vector<std::vector<uint8_t>> blobs(count);
+        for (auto& b : blobs)
+            get(b);
+        ov::Tensor weights(ov::element::u8, ov::Shape{bin.size()});
+        std::memcpy(weights.data(), bin.data(), bin.size());
+        auto model = get_core()->read_model(std::string(xml.begin(), xml.end()), weights);
+        bool profiling = m_profiling;
+        for (const auto& kv : properties)
+            if (kv.first == ov::enable_profiling.name())
+                profiling = kv.second.as<bool>();
+        return std::make_shared<CompiledModel>(model, shared_from_this(), context(), profiling, flags, &blobs);
     }
-    std::shared_ptr<ov::ICompiledModel> import_model(std::istream&, const ov::SoPtr<ov::IRemoteContext>&,
-                                                     const ov::AnyMap&) const override {
-        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: import_model is not implemented");
+    std::shared_ptr<ov::ICompiledModel> import_model(std::istream& in, const ov::SoPtr<ov::IRemoteContext>&,
+                                                     const ov::AnyMap& properties) const override {
+        return import_model(in, properties);
     }
-    std::shared_ptr<ov::ICompiledModel> import_model(const ov::Tensor&, const ov::AnyMap&) const override {
-        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: import_model is not implemented");
+    std::shared_ptr<ov::ICompiledModel> import_model(const ov::Tensor& blob, const ov::AnyMap& properties) const override {
+        std::istringstream in(std::string(static_cast<const char*>(blob.data()), blob.get_byte_size()));
+        return import_model(in, properties);
     }
-    std::shared_ptr<ov::ICompiledModel> import_model(const ov::Tensor&, const ov::SoPtr<ov::IRemoteContext>&,
-                                                     const ov::AnyMap&) const override {
-        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: import_model is not implemented");
+    std::shared_ptr<ov::ICompiledModel> import_model(const ov::Tensor& blob, const ov::SoPtr<ov::IRemoteContext>&,
+                                                     const ov::AnyMap& properties) const override {
+        return import_model(blob, properties);
     }
 
     // Supported: each matched MatMul with its whole decompression chain, and the Parameter / Result around it.
@@ -529,11 +613,15 @@ private:
     mutable std::mutex m_mutex;
     mutable ovfcc_ctx* m_ctx = nullptr;
     bool m_profiling = false;
+    uint64_t m_dq_group = 0;  // ov::hint::dynamic_quantization_group_size; 0 = off
 };
 
 CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std::shared_ptr<const ov::IPlugin>& plugin,
-                             ovfcc_ctx* ctx, bool profiling)
-    : ov::ICompiledModel(model, plugin), m_model(model), m_ctx(ctx), m_profiling(profiling) {
+                             ovfcc_ctx* ctx, bool profiling, int node_flags,
+                             const std::vector<std::vector<uint8_t>>* blobs)
+    : ov::ICompiledModel(model, plugin), m_model(model), m_ctx(ctx), m_node_flags(node_flags), m_profiling(profiling) {
+    if (blobs && blobs->size() != model->get_results().size())
+        OPENVINO_THROW("MI355X: the imported blob holds ", blobs->size(), " nodes, the model ", model->get_results().size());
     // every Result must be fed by a matched MatMul; every Parameter must feed one
     const auto& results = model->get_results();
     const auto& params = model->get_parameters();
@@ -549,10 +637,17 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
         for (size_t p = 0; p < params.size(); ++p)
             if (params[p] == n.fc.activations)
                 n.input_index = p;
-        const void* zp = n.fc.zp_bytes.empty() ? nullptr : n.fc.zp_bytes.data();
-        if (ovfcc_weights_create(ctx, &n.fc.desc, n.fc.weights->get_data_ptr(), n.fc.scales_f16.data(), zp, nullptr,
-                                 &n.weights) != OVFCC_OK)
-            throw_last("weights_create");
+        n.fc.desc.flags |= node_flags;
+        if (blobs) {
+            // the cached device image; the library checks it against its own descriptor
+            if (ovfcc_weights_import(ctx, (*blobs)[r].data(), (*blobs)[r].size(), &n.weights) != OVFCC_OK)
+                throw_last("weights_import");
+        } else {
+            const void* zp = n.fc.zp_bytes.empty() ? nullptr : n.fc.zp_bytes.data();
+            if (ovfcc_weights_create(ctx, &n.fc.desc, n.fc.weights->get_data_ptr(), n.fc.scales_f16.data(), zp,
+                                     nullptr, &n.weights) != OVFCC_OK)
+                throw_last("weights_create");
+        }
         // the executed graph shows the same layer type the CPU plugin shows
         // (src/inference/dev_api/openvino/runtime/exec_model_info.hpp:31-73)
         n.fc.matmul->get_rt_info()["layerType"] = std::string("FullyConnected");
