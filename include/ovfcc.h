@@ -85,7 +85,8 @@ typedef struct ovfcc_fc_desc {
  * GPU: cl_kernels/dynamic_quantize_gpu_ref.cl:100-250 and the integer path of
  * cl_kernels/fully_connected_gpu_bf_tiled.cl:1257-1291, for batches above a threshold only).  The flag is a
  * permission, not a request for a specific kernel: it takes effect for 8-bit weights with one scale per output
- * channel, N % 256 == 0, K % 128 == 0, no gated linear unit, and more than 48 rows; every other call of the node
+ * channel, N % 256 == 0, K % 128 == 0 and more than 48 rows (a gated linear unit, if any, is applied to the
+ * results as usual); every other call of the node
  * computes in f16 as without the flag.  Where it takes effect,
  *     q[m, k] = rte(half(x[m, k] * half(127 / max(0.003, max_k |x[m, k]|)))),
  *     y[m, n] = (sum_k q[m, k] W[n, k] - ZP[n] sum_k q[m, k]) * (S[n] * half(1 / scale_m)) + bias[n],

@@ -153,7 +153,7 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
     // Per-token int8 activations where the node allows them and the integer kernel applies: prefill row counts,
     // 8-bit weights with one scale per channel, whole 256-channel tiles.
     const ovfcc::Layout& L0 = w->layout;
-    if (L0.dynquant && L0.tiled && L0.bits == 8 && L0.groups == 1 && !L0.glu && (w->desc.N % 256) == 0 &&
+    if (L0.dynquant && L0.tiled && L0.bits == 8 && L0.groups == 1 && (w->desc.N % 256) == 0 &&
         M > ovfcc::kDecodeMaxRows && (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL) &&
         M * w->desc.K < ((int64_t)1 << 31) && (M + 127) / 128 <= 65535 &&
         // (it has no split-K: a grid that leaves half the chip idle stays with the f16 kernels, which have;

@@ -104,7 +104,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_i8_kernel(const uint4_t* __re
                                                              const int* __restrict__ qsum,
                                                              const half_t* __restrict__ bias, void* __restrict__ y,
                                                              int M, int N, int K, int kb_total, int zp_const,
-                                                             int out_f32) {
+                                                             int out_f32, int glu) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
 
@@ -228,7 +228,43 @@ __global__ __launch_bounds__(512) void fcc_prefill_i8_kernel(const uint4_t* __re
                 }
         }
         __syncthreads();
-        if (kg == 0) {
+        if (kg == 0 && glu) {
+            // gated linear unit: channel tiles 2 hh and 2 hh + 1 of the wave are gate and up of output channels
+            // (n0 + 64 wn) / 2 + 16 hh .. of the [M, N / 2] result
+            const int ng_ch = n0 + 64 * wn + 32 * hh + 4 * kq;  // gate channels; up channels are 16 further
+            int zadj[2][4];
+            float sc[2][4], bs[2][4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    zadj[h][q] = (ZP_TABLE ? (int)zt[ng_ch + 16 * h + q] : zp_const) - 128;
+                    sc[h][q] = (float)st[ng_ch + 16 * h + q];
+                    bs[h][q] = bias ? (float)bias[ng_ch + 16 * h + q] : 0.f;
+                }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int m = m0 + 16 * t + col;
+                if (m < M) {
+                    const int rs = qsum[m];
+                    const float inv = inv_scale[m];
+                    float o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int g = acc[2 * hh][t][q] + ex[((wn * 64 + t * 4 + q) * 64) + lane];
+                        const int u = acc[2 * hh + 1][t][q] + ex[((wn * 64 + (8 + t) * 4 + q) * 64) + lane];
+                        o[q] = glu_value(glu, (float)(g - zadj[0][q] * rs) * (sc[0][q] * inv) + bs[0][q],
+                                         (float)(u - zadj[1][q] * rs) * (sc[1][q] * inv) + bs[1][q]);
+                    }
+                    const size_t at = (size_t)m * (N / 2) + (n0 + 64 * wn) / 2 + 16 * hh + 4 * kq;
+                    if (out_f32)
+                        *reinterpret_cast<float4_t*>(static_cast<float*>(y) + at) = float4_t{o[0], o[1], o[2], o[3]};
+                    else
+                        *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + at) =
+                            half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
+                }
+            }
+        } else if (kg == 0) {
 #pragma unroll
             for (int r2 = 0; r2 < 2; ++r2) {
                 const int r = 2 * hh + r2;
@@ -291,7 +327,7 @@ static int launch_i8_impl(const FcDeviceArgs& a, const void* xq, const float* in
     hipLaunchKernelGGL(kern, dim3((unsigned)(a.N / PI_BN), (unsigned)((a.M + PI_BM - 1) / PI_BM), 1), dim3(512),
                        PI_LDS_BYTES, s, (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp,
                        (const int8_t*)xq, inv_scale, qsum, (const half_t*)a.bias, a.y, (int)a.M, (int)a.N, (int)a.K,
-                       (int)L.k_blocks, L.zp_const, a.out_f32);
+                       (int)L.k_blocks, L.zp_const, a.out_f32, L.glu);
     return (int)hipGetLastError();
 }
 
@@ -299,8 +335,8 @@ static int launch_i8_impl(const FcDeviceArgs& a, const void* xq, const float* in
 int launch_prefill_i8(const FcDeviceArgs& a, const void* xq, const float* inv_scale, const int* qsum, void* stream) {
     const Layout& L = a.layout;
     // what the kernel's indexing assumes: tiled 8-bit weights, one group per channel, whole 256-channel tiles,
-    // 32-bit byte offsets into the quantised activations and into one wave's weight strip, no gated linear unit
-    if (!L.tiled || L.bits != 8 || L.groups != 1 || L.glu || (a.N % PI_BN) != 0 || a.M < 1 ||
+    // 32-bit byte offsets into the quantised activations and into one wave's weight strip
+    if (!L.tiled || L.bits != 8 || L.groups != 1 || (a.N % PI_BN) != 0 || a.M < 1 ||
         a.M * a.K >= ((int64_t)1 << 31) || (int64_t)4 * L.k_blocks * 2 * kTileBytes >= ((int64_t)1 << 31) ||
         (a.M + PI_BM - 1) / PI_BM > 65535 || !xq || !inv_scale || !qsum)
         return (int)hipErrorInvalidValue;

@@ -112,3 +112,20 @@ def test_dynquant_llama70b_shape(oracle, dev, req):
         assert r < 2e-2
     finally:
         w.close()
+
+
+def test_dynquant_with_gated_linear_unit(oracle, dev, req, monkeypatch):
+    """SwiGLU on top of the integer path: the unit applied to the integer oracle's gate and up halves."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    say("dynquant + glu")
+    c = datagen.make_case(1120, 200, 512, 512, "u8", 512, "u8", with_bias=True)
+    for kind, second in (("swish", False), ("gelu_tanh", True)):
+        w = fc.CompressedWeights.from_case(dev, c, output_type="f32", glu=kind, glu_gate_second=second,
+                                           dynamic_quantization=True)
+        try:
+            y = req.infer(w, c.x)
+            assert req.last_kernel()["name"] == "fcc_prefill_i8_w8" and y.shape == (200, 256)
+            ref = oracle.glu(dq_reference(oracle, c), {"swish": 1, "gelu_tanh": 3}[kind], second)
+            assert oracle.rel_l2(y, ref) < 2e-6, oracle.rel_l2(y, ref)
+        finally:
+            w.close()
