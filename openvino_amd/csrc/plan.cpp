@@ -117,6 +117,15 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         const size_t x_bytes = (size_t)a.M * ((size_t)per * kBlockK + 8) * 2;
         if (x_bytes > 40 * 1024)  // does not fit beside the reduction buffer: read the operand from L2 instead
             xlds = false;
+        // Two to four rows of a long-K, large node whose activations do not fit: the small-batch kernel's
+        // shared staged slice beats per-lane reads of X from L2 (measured on K = 14336, N = 4096).
+        if (!xlds && x_env != 0 && a.M > 1 && a.M <= 4 && L.w_bytes >= ((size_t)16 << 20) &&
+            env_int("OVFCC_DECODE_BATCH", -1) < 0 && force_split <= 0) {
+            if (int rc = plan_batch())
+                return rc;
+            *plan = p;
+            return OVFCC_OK;
+        }
         // Channel tiles per workgroup: one.  More tiles would share a staged activation copy between more
         // weights, but measured slower at M <= 4 (fewer, longer workgroups); the override stays for experiments.
         int rt = 1;
