@@ -22,20 +22,23 @@
 
 namespace ovfcc {
 
-template <int TPB, int RT>
+template <int TPB, int RT, int GPB>
 struct BatchSlot {
     uint4_t w[RT][TPB];
-    half_t scale[RT];
-    uint8_t zp[RT];
+    uint32_t scale[RT][GPB == 4 ? 2 : 1];  // GPB f16 scales, packed
+    uint32_t zp[RT];                       // GPB zero-points, one per byte
 };
 
-template <int BITS, int MT, bool ZP_TABLE, int RT>
+// GPB: groups per k-block (2 or 4 for groups of 64 or 32 inputs, 4-bit weights only); MFMA j of a k-block
+// covers inputs 32 j ..+32 and adds into the partial sum of group j GPB / 4.
+template <int BITS, int MT, bool ZP_TABLE, int RT, int GPB>
 __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
                                            const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
                                            const half_t* __restrict__ bias, void* __restrict__ y,
                                            float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N, int K,
                                            int kb_total, int kb_per_group, int ng, int zp_const, int kb_per_split,
                                            int split_k, int n_tiles, int out_f32, int glu) {
+    static_assert(GPB == 1 || ((GPB == 2 || GPB == 4) && BITS == 4), "groups below 128 inputs: 4-bit weights only");
     constexpr int TPB = BITS == 4 ? 1 : 2;                    // tiles per k-block
     constexpr int DEPTH = (RT * TPB >= 4) ? 2 : 4 / TPB;      // k-blocks in flight per wave
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -73,7 +76,7 @@ __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const
         __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, M * K * 2, kRsrcFlags);
 
     const unsigned g_mul = kb_per_group == 1 ? 0u : (unsigned)((0x100000000ull + kb_per_group - 1) / kb_per_group);
-    using Slot = BatchSlot<TPB, RT>;
+    using Slot = BatchSlot<TPB, RT, GPB>;
     auto issue = [&](int i, Slot& s) {
         // bit 31 of every offset of a slot past the end of the k-range is set: out of range, reads zero
         const unsigned oob = (unsigned)((cnt - 1 - i) >> 31) & kOob;
@@ -86,10 +89,24 @@ __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const
             for (int t = 0; t < TPB; ++t)
                 s.w[r][t] =
                     __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rw, wofs + t * kTileBytes, 0, 2));
-            const unsigned sidx = (r * ng + g) * 16u + col;
-            s.scale[r] = __builtin_bit_cast(half_t, __builtin_amdgcn_raw_buffer_load_b16(rs, (sidx * 2u) | oob, 0, 0));
-            if constexpr (ZP_TABLE)
-                s.zp[r] = __builtin_amdgcn_raw_buffer_load_b8(rz, sidx | oob, 0, 0);
+            if constexpr (GPB == 1) {
+                const unsigned sidx = (r * ng + g) * 16u + col;
+                s.scale[r][0] = __builtin_amdgcn_raw_buffer_load_b16(rs, (sidx * 2u) | oob, 0, 0);
+                if constexpr (ZP_TABLE)
+                    s.zp[r] = __builtin_amdgcn_raw_buffer_load_b8(rz, sidx | oob, 0, 0);
+            } else {
+                const unsigned sidx = ((r * kb_total + kb) * 16u + col) * GPB;
+                if constexpr (GPB == 2) {
+                    s.scale[r][0] = __builtin_amdgcn_raw_buffer_load_b32(rs, (sidx * 2u) | oob, 0, 0);
+                    if constexpr (ZP_TABLE)
+                        s.zp[r] = __builtin_amdgcn_raw_buffer_load_b16(rz, sidx | oob, 0, 0);
+                } else {
+                    const uint2_t v = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(rs, (sidx * 2u) | oob, 0, 0));
+                    s.scale[r][0] = v.x, s.scale[r][1] = v.y;
+                    if constexpr (ZP_TABLE)
+                        s.zp[r] = __builtin_amdgcn_raw_buffer_load_b32(rz, sidx | oob, 0, 0);
+                }
+            }
         }
     };
 
@@ -130,24 +147,44 @@ __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const
                 a[t][j] = *reinterpret_cast<const half8_t*>(xs_lane + 16 * t * x_stride + kbl * 128 + 32 * j);
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
-            const float zpv = ZP_TABLE ? (float)s.zp[r] : (float)zp_const;
-            const float scale = (float)s.scale[r];
-            float4_t part[MT];
+            auto add_scaled = [&](int gi, const float4_t(&part)[MT]) {
+                const uint32_t sbits = s.scale[r][gi >> 1] >> (16 * (gi & 1));
+                const float scale = (float)__builtin_bit_cast(half_t, (uint16_t)sbits);
 #pragma unroll
-            for (int t = 0; t < MT; ++t)
-                part[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+                for (int t = 0; t < MT; ++t) {
+                    acc[r][t].x += scale * part[t].x;
+                    acc[r][t].y += scale * part[t].y;
+                    acc[r][t].z += scale * part[t].z;
+                    acc[r][t].w += scale * part[t].w;
+                }
+            };
             if constexpr (BITS == 4) {
-                const half2_t off_lo = splat(1024.f + zpv), off_hi = splat(64.f + zpv);
                 const uint32_t wd[4] = {s.w[r][0].x, s.w[r][0].y, s.w[r][0].z, s.w[r][0].w};
+                constexpr int kPerGroup = 4 / GPB;  // MFMAs per group
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    Frag8 b;
-                    unpack4(wd[j], off_lo, off_hi, b);
+                for (int gi = 0; gi < GPB; ++gi) {
+                    const float zpv = ZP_TABLE ? (float)((s.zp[r] >> (8 * gi)) & 0xFFu) : (float)zp_const;
+                    const half2_t off_lo = splat(1024.f + zpv), off_hi = splat(64.f + zpv);
+                    float4_t part[MT];
 #pragma unroll
                     for (int t = 0; t < MT; ++t)
-                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], b.v, part[t], 0, 0, 0);
+                        part[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int j = gi * kPerGroup; j < (gi + 1) * kPerGroup; ++j) {
+                        Frag8 b;
+                        unpack4(wd[j], off_lo, off_hi, b);
+#pragma unroll
+                        for (int t = 0; t < MT; ++t)
+                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], b.v, part[t], 0, 0, 0);
+                    }
+                    add_scaled(gi, part);
                 }
             } else {
+                const float zpv = ZP_TABLE ? (float)s.zp[r] : (float)zp_const;
+                float4_t part0[MT];
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    part0[t] = float4_t{0.f, 0.f, 0.f, 0.f};
                 const half2_t off = splat(1024.f + zpv);
 #pragma unroll
                 for (int i2 = 0; i2 < 2; ++i2) {
@@ -158,16 +195,10 @@ __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const
                         unpack8(wd[2 * jj], wd[2 * jj + 1], off, b);
 #pragma unroll
                         for (int t = 0; t < MT; ++t)
-                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], b.v, part[t], 0, 0, 0);
+                            part0[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], b.v, part0[t], 0, 0, 0);
                     }
                 }
-            }
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                acc[r][t].x += scale * part[t].x;
-                acc[r][t].y += scale * part[t].y;
-                acc[r][t].z += scale * part[t].z;
-                acc[r][t].w += scale * part[t].w;
+                add_scaled(0, part0);
             }
         }
     };
@@ -315,7 +346,7 @@ __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const
     }
 }
 
-template <int BITS, int MT, bool ZP_TABLE, int RT>
+template <int BITS, int MT, bool ZP_TABLE, int RT, int GPB>
 __global__ __launch_bounds__(512) void fcc_batch_kernel(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
                                                         const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
                                                         const half_t* __restrict__ bias, void* __restrict__ y,
@@ -323,14 +354,14 @@ __global__ __launch_bounds__(512) void fcc_batch_kernel(const uint4_t* __restric
                                                         int M, int N, int K, int kb_total, int kb_per_group, int ng,
                                                         int zp_const, int kb_per_split, int split_k, int n_tiles,
                                                         int out_f32, int glu) {
-    batch_body<BITS, MT, ZP_TABLE, RT>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
+    batch_body<BITS, MT, ZP_TABLE, RT, GPB>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
                                        zp_const, kb_per_split, split_k, n_tiles, out_f32, glu);
 }
 
 // Grouped launch: blockIdx.z picks one of up to kMaxGroupItems independent problems that share N, K and the weight
 // format (the experts of a mixture-of-experts layer, each with its own rows): one launch instead of one per expert.
 // The table travels in the kernel arguments; every problem has its own slice of the split-K workspace and counters.
-template <int BITS, int MT, bool ZP_TABLE, int RT>
+template <int BITS, int MT, bool ZP_TABLE, int RT, int GPB>
 __global__ __launch_bounds__(512) void fcc_batch_grouped_kernel(BatchGroupTable tab, float* __restrict__ ws,
                                                                 unsigned* __restrict__ counters, size_t ws_per_item,
                                                                 int counters_per_item, int N, int K, int kb_total,
@@ -340,17 +371,17 @@ __global__ __launch_bounds__(512) void fcc_batch_grouped_kernel(BatchGroupTable 
     const BatchGroupItem& it = tab.item[blockIdx.z];
     if (it.M == 0)
         return;
-    batch_body<BITS, MT, ZP_TABLE, RT>(static_cast<const uint4_t*>(it.w), static_cast<const half_t*>(it.scale),
+    batch_body<BITS, MT, ZP_TABLE, RT, GPB>(static_cast<const uint4_t*>(it.w), static_cast<const half_t*>(it.scale),
                                        static_cast<const uint8_t*>(it.zp), static_cast<const half_t*>(it.x),
                                        static_cast<const half_t*>(it.bias), it.y, ws + blockIdx.z * ws_per_item,
                                        counters + blockIdx.z * counters_per_item, it.M, N, K, kb_total, kb_per_group,
                                        ng, zp_const, kb_per_split, split_k, n_tiles, out_f32, 0);
 }
 
-template <int BITS, int MT, bool ZPT, int RT>
-static int launch_batch_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+template <int BITS, int MT, bool ZPT, int RT, int GPB>
+static int launch_batch_gpb(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_batch_kernel<BITS, MT, ZPT, RT>;
+    auto kern = fcc_batch_kernel<BITS, MT, ZPT, RT, GPB>;
     if (p.dynamic_lds > 48 * 1024) {
         static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
         if (!attr_set) {
@@ -369,6 +400,17 @@ static int launch_batch_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
     return (int)hipGetLastError();
 }
 
+template <int BITS, int MT, bool ZPT, int RT>
+static int launch_batch_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    if constexpr (BITS == 4) {
+        if (a.layout.groups_per_kblock == 2)
+            return launch_batch_gpb<BITS, MT, ZPT, RT, 2>(a, p, s);
+        if (a.layout.groups_per_kblock == 4)
+            return launch_batch_gpb<BITS, MT, ZPT, RT, 4>(a, p, s);
+    }
+    return launch_batch_gpb<BITS, MT, ZPT, RT, 1>(a, p, s);
+}
+
 template <int BITS, bool ZPT>
 static int launch_batch_bits(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const int mt = (int)(a.M + 15) / 16;
@@ -380,11 +422,11 @@ static int launch_batch_bits(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
     return rt == 2 ? launch_batch_impl<BITS, 3, ZPT, 2>(a, p, s) : launch_batch_impl<BITS, 3, ZPT, 1>(a, p, s);
 }
 
-template <int BITS, int MT, bool ZPT>
-static int launch_grouped_impl(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
-                               hipStream_t s) {
+template <int BITS, int MT, bool ZPT, int GPB>
+static int launch_grouped_gpb(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
+                              hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_batch_grouped_kernel<BITS, MT, ZPT, 1>;
+    auto kern = fcc_batch_grouped_kernel<BITS, MT, ZPT, 1, GPB>;
     if (p.dynamic_lds > 48 * 1024) {
         static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
         if (!attr_set) {
@@ -402,6 +444,18 @@ static int launch_grouped_impl(const BatchGroupTable& tab, int n_items, const Fc
     return (int)hipGetLastError();
 }
 
+template <int BITS, int MT, bool ZPT>
+static int launch_grouped_impl(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
+                               hipStream_t s) {
+    if constexpr (BITS == 4) {
+        if (a.layout.groups_per_kblock == 2)
+            return launch_grouped_gpb<BITS, MT, ZPT, 2>(tab, n_items, a, p, s);
+        if (a.layout.groups_per_kblock == 4)
+            return launch_grouped_gpb<BITS, MT, ZPT, 4>(tab, n_items, a, p, s);
+    }
+    return launch_grouped_gpb<BITS, MT, ZPT, 1>(tab, n_items, a, p, s);
+}
+
 // `a` describes the shared shape (M = the largest row count of any item, at most 48); `p` is its small-batch plan
 // with one channel tile per wave; workspace and counters hold n_items slices of p.workspace_bytes / p.counter_count.
 int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
@@ -410,6 +464,8 @@ int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDevice
     const Layout& L = a.layout;
     if (L.glu || p.tiles_per_group != 1)
         return (int)hipErrorInvalidValue;  // the grouped kernel is built for one tile per wave
+    if (L.groups_per_kblock != 1 && L.bits != 4)
+        return (int)hipErrorInvalidValue;
     const int mt = (int)(a.M + 15) / 16;
 #define OVFCC_GROUPED(B, Z)                                                         \
     (mt <= 1   ? launch_grouped_impl<B, 1, Z>(tab, n_items, a, p, s)                \
@@ -426,6 +482,8 @@ int launch_batch(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     const Layout& L = a.layout;
     if (L.glu && ((p.tiles_per_group == 1 && ((p.block >> 6) & 1)) || p.dynamic_lds < (p.block >> 7) * (unsigned)p.tile_m * 64u))
         return (int)hipErrorInvalidValue;  // gate and up tile: one wave, or two neighbours with room for the hand-over
+    if (L.groups_per_kblock != 1 && L.bits != 4)
+        return (int)hipErrorInvalidValue;
     if (L.bits == 4)
         return L.zp_table ? launch_batch_bits<4, true>(a, p, s) : launch_batch_bits<4, false>(a, p, s);
     return L.zp_table ? launch_batch_bits<8, true>(a, p, s) : launch_batch_bits<8, false>(a, p, s);

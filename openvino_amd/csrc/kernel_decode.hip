@@ -18,7 +18,8 @@
 // columns n; v_mfma_f32_16x16x32_f16, f32 result: lane holds column n = lane & 15, rows 4 (lane >> 4) + r);
 // one more MFMA per k-step against the constant fragment -(bias + zp) cancels bias and zero-point in the
 // f32 accumulator, which keeps the vector ALU free for the unpack.  The group scale multiplies the f32
-// partial sum of the k-block, so no weight is ever rounded.
+// partial sum of the k-block, so no weight is ever rounded.  Groups of 64 or 32 inputs (GPB = 2 or 4 groups
+// per k-block, 4-bit weights) keep one partial sum per group: MFMA j of a k-block covers inputs 32 j ..+32.
 //
 // Reductions: the waves of a workgroup are summed through LDS in wave order.  With split_k > 1 every
 // workgroup writes its partial tiles with device-scope stores, waits for them, and takes a ticket from a
@@ -28,15 +29,15 @@
 
 namespace ovfcc {
 
-template <int TPB, int MT, int RT, bool XLDS>
+template <int TPB, int MT, int RT, bool XLDS, int GPB>
 struct DecodeSlot {
     uint4_t w[RT][TPB];
     half8_t a[XLDS ? 1 : MT][XLDS ? 1 : 4];  // unused when the activations come from LDS
-    half_t scale[RT];
-    uint8_t zp[RT];
+    uint32_t scale[RT][GPB == 4 ? 2 : 1];    // GPB f16 scales, packed
+    uint32_t zp[RT];                         // GPB zero-points, one per byte
 };
 
-template <int BITS, int MT, bool ZP_TABLE, int RT, bool XLDS>
+template <int BITS, int MT, bool ZP_TABLE, int RT, bool XLDS, int GPB>
 __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restrict__ wt,
                                                           const half_t* __restrict__ st,
                                                           const uint8_t* __restrict__ zt,
@@ -47,6 +48,7 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
                                                           int ng, int zp_const, int kb_per_split, int split_k,
                                                           int out_f32, int glu) {
     static_assert(!XLDS || MT == 1, "LDS-staged activations serve one 16-row tile");
+    static_assert(GPB == 1 || ((GPB == 2 || GPB == 4) && BITS == 4), "groups below 128 inputs: 4-bit weights only");
     constexpr int TPB = BITS == 4 ? 1 : 2;                                            // tiles per k-block
     constexpr int DEPTH = XLDS ? (RT * TPB >= 4 ? 2 : 4) : (MT == 1 ? 4 : 2) / TPB;  // k-blocks in flight
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];              // [red][xs]
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
     // group index of a k-block without a division in the loop: kb_per_group == 1 -> kb, else the high word of
     // kb * ceil(2^32 / kb_per_group) (exact for kb < 2^16)
     const unsigned g_mul = kb_per_group == 1 ? 0u : (unsigned)((0x100000000ull + kb_per_group - 1) / kb_per_group);
-    using Slot = DecodeSlot<TPB, MT, RT, XLDS>;
+    using Slot = DecodeSlot<TPB, MT, RT, XLDS, GPB>;
     auto issue = [&](int i, Slot& s) {
         // bit 31 of every offset of a slot past the end of this wave's share is set: out of range, reads zero
         const unsigned oob = (unsigned)((cnt - 1 - i) >> 31) & kOob;
@@ -116,10 +118,25 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
         }
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
-            const unsigned sidx = (r * ng + g) * 16u + col;
-            s.scale[r] = __builtin_bit_cast(half_t, __builtin_amdgcn_raw_buffer_load_b16(rs, (sidx * 2u) | oob, 0, 0));
-            if constexpr (ZP_TABLE)
-                s.zp[r] = __builtin_amdgcn_raw_buffer_load_b8(rz, sidx | oob, 0, 0);
+            if constexpr (GPB == 1) {
+                const unsigned sidx = (r * ng + g) * 16u + col;
+                s.scale[r][0] = __builtin_amdgcn_raw_buffer_load_b16(rs, (sidx * 2u) | oob, 0, 0);
+                if constexpr (ZP_TABLE)
+                    s.zp[r] = __builtin_amdgcn_raw_buffer_load_b8(rz, sidx | oob, 0, 0);
+            } else {
+                // the GPB groups of this k-block for the lane's channel lie side by side
+                const unsigned sidx = ((r * kb_total + kb) * 16u + col) * GPB;
+                if constexpr (GPB == 2) {
+                    s.scale[r][0] = __builtin_amdgcn_raw_buffer_load_b32(rs, (sidx * 2u) | oob, 0, 0);
+                    if constexpr (ZP_TABLE)
+                        s.zp[r] = __builtin_amdgcn_raw_buffer_load_b16(rz, sidx | oob, 0, 0);
+                } else {
+                    const uint2_t v = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(rs, (sidx * 2u) | oob, 0, 0));
+                    s.scale[r][0] = v.x, s.scale[r][1] = v.y;
+                    if constexpr (ZP_TABLE)
+                        s.zp[r] = __builtin_amdgcn_raw_buffer_load_b32(rz, sidx | oob, 0, 0);
+                }
+            }
         }
     };
 
@@ -167,30 +184,51 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
         }
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
-            const float zpv = ZP_TABLE ? (float)s.zp[r] : (float)zp_const;
-            const float scale = (float)s.scale[r];
-            float4_t part[MT];
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-                part[t] = float4_t{0.f, 0.f, 0.f, 0.f};
             // weights enter the matrix cores with their unpack bias (1024 + q, 64 + q); a second MFMA against
             // the constant fragment -(bias + zp) removes bias and zero-point inside the f32 accumulator
-            Frag8 bc;
+            auto add_scaled = [&](int gi, const float4_t(&part)[MT]) {
+                const uint32_t sbits = s.scale[r][gi >> 1] >> (16 * (gi & 1));
+                const float scale = (float)__builtin_bit_cast(half_t, (uint16_t)sbits);
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    acc[r][t].x += scale * part[t].x;
+                    acc[r][t].y += scale * part[t].y;
+                    acc[r][t].z += scale * part[t].z;
+                    acc[r][t].w += scale * part[t].w;
+                }
+            };
             if constexpr (BITS == 4) {
-                bc.h2[0] = bc.h2[2] = splat(-(1024.f + zpv));
-                bc.h2[1] = bc.h2[3] = splat(-(64.f + zpv));
                 const uint32_t wd[4] = {s.w[r][0].x, s.w[r][0].y, s.w[r][0].z, s.w[r][0].w};
+                constexpr int kPerGroup = 4 / GPB;  // MFMAs per group
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    Frag8 b;
-                    unpack4_biased(wd[j], uc, b);
+                for (int gi = 0; gi < GPB; ++gi) {
+                    const float zpv = ZP_TABLE ? (float)((s.zp[r] >> (8 * gi)) & 0xFFu) : (float)zp_const;
+                    Frag8 bc;
+                    bc.h2[0] = bc.h2[2] = splat(-(1024.f + zpv));
+                    bc.h2[1] = bc.h2[3] = splat(-(64.f + zpv));
+                    float4_t part[MT];
 #pragma unroll
-                    for (int t = 0; t < MT; ++t) {
-                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], b.v, part[t], 0, 0, 0);
-                        part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], bc.v, part[t], 0, 0, 0);
+                    for (int t = 0; t < MT; ++t)
+                        part[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int j = gi * kPerGroup; j < (gi + 1) * kPerGroup; ++j) {
+                        Frag8 b;
+                        unpack4_biased(wd[j], uc, b);
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) {
+                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], b.v, part[t], 0, 0, 0);
+                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][j], bc.v, part[t], 0, 0, 0);
+                        }
                     }
+                    add_scaled(gi, part);
                 }
             } else {
+                const float zpv = ZP_TABLE ? (float)s.zp[r] : (float)zp_const;
+                float4_t part0[MT];
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    part0[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+                Frag8 bc;
                 bc.h2[0] = bc.h2[1] = bc.h2[2] = bc.h2[3] = splat(-(1024.f + zpv));
 #pragma unroll
                 for (int i2 = 0; i2 < 2; ++i2) {
@@ -201,18 +239,12 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
                         unpack8_biased(wd[2 * jj], wd[2 * jj + 1], b);
 #pragma unroll
                         for (int t = 0; t < MT; ++t) {
-                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], b.v, part[t], 0, 0, 0);
-                            part[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], bc.v, part[t], 0, 0, 0);
+                            part0[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], b.v, part0[t], 0, 0, 0);
+                            part0[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][2 * i2 + jj], bc.v, part0[t], 0, 0, 0);
                         }
                     }
                 }
-            }
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                acc[r][t].x += scale * part[t].x;
-                acc[r][t].y += scale * part[t].y;
-                acc[r][t].z += scale * part[t].z;
-                acc[r][t].w += scale * part[t].w;
+                add_scaled(0, part0);
             }
         }
     };
@@ -336,14 +368,25 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
     }
 }
 
+template <int BITS, int MT, bool ZPT, int RT, bool XLDS, int GPB>
+static void launch_decode_gpb(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    const Layout& L = a.layout;
+    hipLaunchKernelGGL((fcc_decode_kernel<BITS, MT, ZPT, RT, XLDS, GPB>), dim3(p.grid[0], p.grid[1], 1),
+                       dim3(p.block), p.dynamic_lds, s, (const uint4_t*)a.w, (const half_t*)a.scale,
+                       (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y, a.workspace, a.counters,
+                       (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
+                       L.zp_const, p.kblocks_per_split, p.split_k, a.out_f32, L.glu);
+}
+
 template <int BITS, int MT, bool ZPT, int RT, bool XLDS>
 static void launch_decode_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
-    const Layout& L = a.layout;
-    hipLaunchKernelGGL((fcc_decode_kernel<BITS, MT, ZPT, RT, XLDS>), dim3(p.grid[0], p.grid[1], 1), dim3(p.block),
-                       p.dynamic_lds, s, (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp,
-                       (const half_t*)a.x, (const half_t*)a.bias, a.y, a.workspace, a.counters, (int)a.M, (int)a.N,
-                       (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups, L.zp_const,
-                       p.kblocks_per_split, p.split_k, a.out_f32, L.glu);
+    if constexpr (BITS == 4) {
+        if (a.layout.groups_per_kblock == 2)
+            return launch_decode_gpb<BITS, MT, ZPT, RT, XLDS, 2>(a, p, s);
+        if (a.layout.groups_per_kblock == 4)
+            return launch_decode_gpb<BITS, MT, ZPT, RT, XLDS, 4>(a, p, s);
+    }
+    launch_decode_gpb<BITS, MT, ZPT, RT, XLDS, 1>(a, p, s);
 }
 
 template <int BITS, bool ZPT>
@@ -374,6 +417,8 @@ int launch_decode(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     const Layout& L = a.layout;
     if (L.glu && (!p.x_in_lds || a.M > 16 || (p.tiles_per_group & 1)))
         return (int)hipErrorInvalidValue;  // gate and up tile must share a workgroup
+    if (L.groups_per_kblock != 1 && (L.bits != 4 || (L.groups_per_kblock != 2 && L.groups_per_kblock != 4)))
+        return (int)hipErrorInvalidValue;
     if (L.bits == 4)
         L.zp_table ? launch_decode_bits<4, true>(a, p, s) : launch_decode_bits<4, false>(a, p, s);
     else

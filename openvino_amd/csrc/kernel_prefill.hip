@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
                                                           const half_t* __restrict__ x,
                                                           const half_t* __restrict__ bias, void* __restrict__ y,
                                                           int M, int N, int K, int kb_total, int kb_per_group, int ng,
-                                                          int zp_const, int out_f32, int glu) {
+                                                          int zp_const, int out_f32, int glu, int gpb) {
     constexpr int TPB = BITS == 4 ? 1 : 2;
     __shared__ __attribute__((aligned(16))) half_t As[PF_BM * PF_LD];
     __shared__ __attribute__((aligned(16))) half_t Bs[PF_BN * PF_LD];
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
     uint4_t a_reg[4];
     // weight staging: wave covers channel tiles 2 wave, 2 wave + 1 of the 8 in this workgroup
     uint4_t w_reg[2];
-    float w_scale[2], w_zp[2];
+    float w_scale[2][2], w_zp[2][2];  // [tile][32-input half of the step]
 
     float16_t acc[2][2];
 #pragma unroll
@@ -65,18 +65,35 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
         }
     };
     auto load_w = [&](int step) {
+        const int kb = step >> 1;
+        if (gpb > 1) {
+            // groups of 64 or 32 inputs (4-bit weights): the step's two 32-input halves are dwords 2 h, 2 h + 1
+            // of the tile, groups (2 h + jj) gpb / 4 of the k-block
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int nt = nt0 + 2 * wave + i;
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+                    const int gi = (2 * (step & 1) + jj) * gpb / 4;
+                    const size_t idx = (((size_t)nt * kb_total + kb) * 16 + col) * gpb + gi;
+                    w_scale[i][jj] = (float)st[idx];
+                    w_zp[i][jj] = ZP_TABLE ? (float)zt[idx] : (float)zp_const;
+                }
+            }
+        }
         // 4-bit: a new 128-input tile every second step; 8-bit: a new 64-input tile every step
         if (BITS == 4 && (step & 1))
             return;
-        const int kb = step >> 1;
         const int g = kb / kb_per_group;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int nt = nt0 + 2 * wave + i;
             const size_t tile = BITS == 4 ? ((size_t)nt * kb_total + kb) : ((size_t)nt * kb_total * 2 + step);
             w_reg[i] = wt[tile * 64 + lane];
-            w_scale[i] = (float)st[((size_t)nt * ng + g) * 16 + col];
-            w_zp[i] = ZP_TABLE ? (float)zt[((size_t)nt * ng + g) * 16 + col] : (float)zp_const;
+            if (gpb == 1) {
+                w_scale[i][0] = w_scale[i][1] = (float)st[((size_t)nt * ng + g) * 16 + col];
+                w_zp[i][0] = w_zp[i][1] = ZP_TABLE ? (float)zt[((size_t)nt * ng + g) * 16 + col] : (float)zp_const;
+            }
         }
     };
     auto store_tiles = [&](int step) {
@@ -86,15 +103,15 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
             const int row = 16 * (2 * wave + i) + col;
-            const half2_t sc = splat(w_scale[i]);
             const uint32_t wd[4] = {w_reg[i].x, w_reg[i].y, w_reg[i].z, w_reg[i].w};
             if constexpr (BITS == 4) {
-                const half2_t off_lo = splat(1024.f + w_zp[i]);
-                const half2_t off_hi = splat(64.f + w_zp[i]);
                 const bool h = step & 1;
                 const uint32_t half_w[2] = {h ? wd[2] : wd[0], h ? wd[3] : wd[1]};
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
+                    const half2_t sc = splat(w_scale[i][jj]);
+                    const half2_t off_lo = splat(1024.f + w_zp[i][jj]);
+                    const half2_t off_hi = splat(64.f + w_zp[i][jj]);
                     Frag8 b;
                     unpack4(half_w[jj], off_lo, off_hi, b);
                     if constexpr (PRESCALE) {
@@ -105,7 +122,8 @@ __global__ __launch_bounds__(256) void fcc_prefill_kernel(const uint4_t* __restr
                     *reinterpret_cast<half8_t*>(&Bs[row * PF_LD + 32 * jj + 8 * kq]) = b.v;
                 }
             } else {
-                const half2_t off = splat(1024.f + w_zp[i]);
+                const half2_t sc = splat(w_scale[i][0]);
+                const half2_t off = splat(1024.f + w_zp[i][0]);
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
                     Frag8 b;
@@ -179,7 +197,7 @@ static void launch_prefill_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipS
     hipLaunchKernelGGL((fcc_prefill_kernel<BITS, ZPT, PRE>), dim3(p.grid[0], p.grid[1], 1), dim3(256), 0, s,
                        (const uint4_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x,
                        (const half_t*)a.bias, a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
-                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32, L.glu);
+                       (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32, L.glu, L.groups_per_kblock);
 }
 
 // Grouped scales are folded into the f16 weights in LDS; a single group per channel (G == K) keeps the
@@ -195,6 +213,8 @@ static void launch_prefill(const FcDeviceArgs& a, const LaunchPlan& p, hipStream
 int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
+    if (L.groups_per_kblock != 1 && (L.bits != 4 || L.groups == 1))
+        return (int)hipErrorInvalidValue;
     if (L.bits == 4)
         L.zp_table ? launch_prefill<4, true>(a, p, s) : launch_prefill<4, false>(a, p, s);
     else

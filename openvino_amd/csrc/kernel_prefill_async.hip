@@ -50,14 +50,20 @@ constexpr int PA_STAGES = 3;
 constexpr int PA_XQ = 3;  // activation operands in registers: the one in use and PA_XQ - 1 on their way from LDS
 constexpr int PA_A_BYTES = PA_BM * PA_BK * 2;  // 32 KiB per stage
 constexpr int PA_W_BYTES = 16 * kTileBytes;    // 16 KiB per stage
-constexpr int PA_P_BYTES = 1024;               // scales (512) + zero-points (256)
+constexpr int PA_P_BYTES = 1024;               // per group of a k-block: scales (512) + zero-points (256)
 constexpr int PA_W_OFF = PA_STAGES * PA_A_BYTES;
 constexpr int PA_P_OFF = PA_W_OFF + PA_STAGES * PA_W_BYTES;
-constexpr unsigned PA_LDS_BYTES = (unsigned)(PA_P_OFF + PA_STAGES * PA_P_BYTES);  // 147 KiB
+// 147 KiB with one group per k-block, 150 and 156 KiB with two and four
+constexpr unsigned pa_lds_bytes(int gpb) {
+    return (unsigned)(PA_P_OFF + PA_STAGES * PA_P_BYTES * gpb);
+}
 
 // The whole kernel for one workgroup's share of one node.  The two kernels below differ only in where the node's
 // operands come from.
-template <bool ZP_TABLE, bool PRESCALE, int NT>
+// GPB: groups per k-block.  With groups of 64 or 32 inputs (GPB = 2 or 4) a staged k-block carries GPB scales and
+// zero-points per channel, stored [tile][channel][group]; a wave's k-group kg and step js contract inputs
+// 32 (2 kg + js) ..+32 of the k-block, that is group kg (GPB = 2) or 2 kg + js (GPB = 4).
+template <bool ZP_TABLE, bool PRESCALE, int NT, int GPB>
 __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ wt, const half_t* __restrict__ st,
                                                    const uint8_t* __restrict__ zt, const half_t* __restrict__ x,
                                                    const half_t* __restrict__ bias, void* __restrict__ y,
@@ -65,6 +71,9 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                                                    int K, int kb_total, int kb_per_group, int ng, int zp_const,
                                                    int out_f32, int glu, const TileWork wk) {
     static_assert(NT == 8 || NT == 4, "tiles of 128 or 64 rows");
+    static_assert(GPB == 1 || ((GPB == 2 || GPB == 4) && PRESCALE), "several groups per k-block: scales go into the weights");
+    constexpr int PB = PA_P_BYTES * GPB;  // parameter bytes per stage
+    constexpr int ZOFF = 512 * GPB;       // zero-points follow the scales
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
     constexpr int AL = NT / 2;                          // activation loads per wave and k-block
     constexpr int S = 4 * NT;                           // MFMA slots per step (a wave's two steps make a k-block)
@@ -117,18 +126,46 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     };
     // ---- parameters: waves 0 and 1 fetch the scales of eight channel tiles each (32 bytes per tile, 4 per
     // lane), wave 2 the zero-points of all sixteen (16 bytes per tile, 4 per lane); other waves fetch nothing ----
-    const bool has_p = (PRESCALE && wave < 2) || (ZP_TABLE && wave == 2);
+    // With two groups per k-block (64 and 32 bytes per tile): wave 0 the scales, 16 bytes per lane; waves 2 and 3
+    // the zero-points of eight tiles each.  With four (128 and 64 bytes per tile): waves 0 and 1 the scales of
+    // eight tiles each and wave 2 the zero-points, 16 bytes per lane.  No wave issues more than one such load.
+    const bool has_p = GPB == 1   ? (PRESCALE && wave < 2) || (ZP_TABLE && wave == 2)
+                       : GPB == 2 ? wave == 0 || (ZP_TABLE && (wave == 2 || wave == 3))
+                                  : wave < 2 || (ZP_TABLE && wave == 2);
     auto dma_p = [&](int kb, int stage) {
         const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
-        const unsigned g = kb_per_group == 1 ? (unsigned)kb : __umulhi((unsigned)kb, g_mul);
-        if (PRESCALE && wave < 2) {
-            const unsigned tile = 8u * wave + (lane >> 3);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_ptr)(lds3 + PA_P_OFF + stage * PA_P_BYTES + 256 * wave), 4,
-                                                     ((tile * ng + g) * 32u + (lane & 7) * 4u) | oob, 0, 0, 0);
-        } else if (ZP_TABLE && wave == 2) {
-            const unsigned tile = lane >> 2;
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(lds3 + PA_P_OFF + stage * PA_P_BYTES + 512), 4,
-                                                     ((tile * ng + g) * 16u + (lane & 3) * 4u) | oob, 0, 0, 0);
+        const lds_byte_ptr pbase = lds3 + PA_P_OFF + stage * PB;
+        if constexpr (GPB == 1) {
+            const unsigned g = kb_per_group == 1 ? (unsigned)kb : __umulhi((unsigned)kb, g_mul);
+            if (PRESCALE && wave < 2) {
+                const unsigned tile = 8u * wave + (lane >> 3);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_ptr)(pbase + 256 * wave), 4,
+                                                         ((tile * ng + g) * 32u + (lane & 7) * 4u) | oob, 0, 0, 0);
+            } else if (ZP_TABLE && wave == 2) {
+                const unsigned tile = lane >> 2;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(pbase + ZOFF), 4,
+                                                         ((tile * ng + g) * 16u + (lane & 3) * 4u) | oob, 0, 0, 0);
+            }
+        } else if constexpr (GPB == 2) {
+            if (wave == 0) {
+                const unsigned tile = lane >> 2;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_ptr)pbase, 16,
+                                                         ((tile * kb_total + kb) * 64u + (lane & 3) * 16u) | oob, 0, 0, 0);
+            } else if (ZP_TABLE && (wave == 2 || wave == 3)) {
+                const unsigned tile = 8u * (wave - 2) + (lane >> 3);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(pbase + ZOFF + 256 * (wave - 2)), 4,
+                                                         ((tile * kb_total + kb) * 32u + (lane & 7) * 4u) | oob, 0, 0, 0);
+            }
+        } else {
+            if (wave < 2) {
+                const unsigned tile = 8u * wave + (lane >> 3);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_ptr)(pbase + 1024 * wave), 16,
+                                                         ((tile * kb_total + kb) * 128u + (lane & 7) * 16u) | oob, 0, 0, 0);
+            } else if (ZP_TABLE && wave == 2) {
+                const unsigned tile = lane >> 2;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(pbase + ZOFF), 16,
+                                                         ((tile * kb_total + kb) * 64u + (lane & 3) * 16u) | oob, 0, 0, 0);
+            }
         }
     };
     // Per k-block a wave issues, in this order: AL (4 or 2) activation loads (for k-block + 2), then 2 weight
@@ -141,20 +178,31 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     typedef __attribute__((address_space(3))) const uint2_t* lds_u2_ptr;
     typedef __attribute__((address_space(3))) const half_t* lds_half_ptr;
     uint32_t wraw[2][4][2];
-    uint32_t wscale[2][4];  // f16 scale in both halves
-    uint32_t wzp[2][4];
+    typedef __attribute__((address_space(3))) const uint32_t* lds_u32_ptr;
+    typedef __attribute__((address_space(3))) const uint16_t* lds_u16_ptr;
+    uint32_t wscale[2][4];  // f16 scale in both halves; GPB == 4: the scales of step 0 and step 1
+    uint32_t wzp[2][4];     // zero-point; GPB == 4: those of step 0 and step 1 in bytes 0 and 1
     auto read_w = [&](int par, int stage, int r) {
         const uint2_t v = *(lds_u2_ptr)(lds3 + PA_W_OFF + stage * PA_W_BYTES + (4 * wn + r) * kTileBytes + lane * 16 + kg * 8);
         wraw[par][r][0] = v.x, wraw[par][r][1] = v.y;
     };
     auto read_p = [&](int par, int stage, int r) {
-        if constexpr (PRESCALE)
-        {
-            const half_t h = *(lds_half_ptr)(lds3 + PA_P_OFF + stage * PA_P_BYTES + (4 * wn + r) * 32 + col * 2);
-            wscale[par][r] = as_u32(half2_t{h, h});
+        const lds_byte_ptr pbase = lds3 + PA_P_OFF + stage * PB;
+        if constexpr (GPB == 4) {
+            // groups 2 kg (step 0) and 2 kg + 1 (step 1) of the lane's channel
+            const uint32_t v = *(lds_u32_ptr)(pbase + (4 * wn + r) * 128 + col * 8 + kg * 4);
+            wscale[par][r] = v;
+            if constexpr (ZP_TABLE)
+                wzp[par][r] = *(lds_u16_ptr)(pbase + ZOFF + (4 * wn + r) * 64 + col * 4 + kg * 2);
+        } else {
+            // GPB == 2: group kg of the lane's channel
+            if constexpr (PRESCALE) {
+                const half_t h = *(lds_half_ptr)(pbase + (4 * wn + r) * 32 * GPB + col * 2 * GPB + (GPB == 2 ? kg * 2 : 0));
+                wscale[par][r] = as_u32(half2_t{h, h});
+            }
+            if constexpr (ZP_TABLE)
+                wzp[par][r] = pbase[ZOFF + (4 * wn + r) * 16 * GPB + col * GPB + (GPB == 2 ? kg : 0)];
         }
-        if constexpr (ZP_TABLE)
-            wzp[par][r] = lds3[PA_P_OFF + stage * PA_P_BYTES + 512 + (4 * wn + r) * 16 + col];
     };
 
     // ---- unpack, one micro-operation at a time: dword js of tile r of parity par -> f ----
@@ -178,14 +226,15 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             const int k = op - 5;
             half2_t off;
             if constexpr (ZP_TABLE) {
-                const float zpv = (float)wzp[par][r];
+                const float zpv = GPB == 4 ? (float)((wzp[par][r] >> (8 * js)) & 0xFFu) : (float)wzp[par][r];
                 off = (k & 1) ? splat(64.f + zpv) : splat(1024.f + zpv);
             } else {
                 off = (k & 1) ? off_hi_c : off_lo_c;
             }
             f.h2[k] = f.h2[k] - off;
         } else if constexpr (PRESCALE) {
-            f.h2[op - 9] *= as_half2(wscale[par][r]);
+            const half2_t sv = as_half2(wscale[par][r]);
+            f.h2[op - 9] *= GPB == 4 ? half2_t{sv[js], sv[js]} : sv;
         }
     };
 
@@ -308,7 +357,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     tile_epilogue<PRESCALE, NT>(acc, lds_raw, st, bias, y, ws, counters, M, N, n0, m0, split_k, wk.z, tile_id, out_f32, glu);
 }
 
-template <bool ZP_TABLE, bool PRESCALE, int NT>
+template <bool ZP_TABLE, bool PRESCALE, int NT, int GPB>
 __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* __restrict__ wt,
                                                                 const half_t* __restrict__ st,
                                                                 const uint8_t* __restrict__ zt,
@@ -320,14 +369,14 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
                                                                 int out_f32, int glu, int tiles_x, int tiles_y,
                                                                 int full_tiles, int tail_split, int kb_per_split) {
     const TileWork wk = tile_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT, PA_BN / 2);
-    prefill_async_body<ZP_TABLE, PRESCALE, NT>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total, kb_per_group, ng,
-                                           zp_const, out_f32, glu, wk);
+    prefill_async_body<ZP_TABLE, PRESCALE, NT, GPB>(wt, st, zt, x, bias, y, ws, counters, M, N, K, kb_total,
+                                                    kb_per_group, ng, zp_const, out_f32, glu, wk);
 }
 
 // Grouped launch: tile row tile_y is item tile_y of the table, a node of the common shape and format with at most
 // 128 rows of its own (the experts of a mixture-of-experts layer over their gathered rows).  Workgroups of one
 // item sit together in a super-tile and share its activations in L2.
-template <bool ZP_TABLE, bool PRESCALE, int NT>
+template <bool ZP_TABLE, bool PRESCALE, int NT, int GPB>
 __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const BatchGroupTable tab,
                                                                         float* __restrict__ ws,
                                                                         unsigned* __restrict__ counters, int N, int K,
@@ -340,17 +389,18 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const Ba
     if (it.M <= 0)
         return;
     wk.m0 = 0;
-    prefill_async_body<ZP_TABLE, PRESCALE, NT>((const uint4_t*)it.w, (const half_t*)it.scale, (const uint8_t*)it.zp,
-                                           (const half_t*)it.x, (const half_t*)it.bias, it.y, ws, counters, it.M, N, K,
-                                           kb_total, kb_per_group, ng, zp_const, out_f32, glu, wk);
+    prefill_async_body<ZP_TABLE, PRESCALE, NT, GPB>((const uint4_t*)it.w, (const half_t*)it.scale,
+                                                    (const uint8_t*)it.zp, (const half_t*)it.x, (const half_t*)it.bias,
+                                                    it.y, ws, counters, it.M, N, K, kb_total, kb_per_group, ng, zp_const,
+                                                    out_f32, glu, wk);
 }
 
 template <typename Kern>
-static int allow_lds(Kern kern, bool* done) {
+static int allow_lds(Kern kern, bool* done, unsigned bytes) {
     if (*done)
         return 0;  // the attribute is idempotent, a race only repeats it
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)PA_LDS_BYTES);
+                                       (int)bytes);
     if (e == hipSuccess)
         *done = true;
     return (int)e;
@@ -366,14 +416,14 @@ static bool async_plan_ok(const FcDeviceArgs& a, const LaunchPlan& p) {
            (p.split_k == 1 || (a.workspace && a.counters));
 }
 
-template <bool ZPT, bool PRE, int NT>
-static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+template <bool ZPT, bool PRE, int NT, int GPB>
+static int launch_async_gpb(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_prefill_async_kernel<ZPT, PRE, NT>;
+    auto kern = fcc_prefill_async_kernel<ZPT, PRE, NT, GPB>;
     static bool attr_set = false;  // per instantiation
-    if (int e = allow_lds(kern, &attr_set))
+    if (int e = allow_lds(kern, &attr_set, pa_lds_bytes(GPB)))
         return e;
-    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), PA_LDS_BYTES, s, (const uint4_t*)a.w,
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(GPB), s, (const uint4_t*)a.w,
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
                        a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
                        (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32, L.glu, p.tiles_x,
@@ -382,18 +432,41 @@ static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
 }
 
 template <bool ZPT, bool PRE, int NT>
-static int launch_async_grouped_impl(const BatchGroupTable& tab, const FcDeviceArgs& a, const LaunchPlan& p,
-                                     hipStream_t s) {
+static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    if constexpr (PRE) {
+        if (a.layout.groups_per_kblock == 2)
+            return launch_async_gpb<ZPT, PRE, NT, 2>(a, p, s);
+        if (a.layout.groups_per_kblock == 4)
+            return launch_async_gpb<ZPT, PRE, NT, 4>(a, p, s);
+    }
+    return launch_async_gpb<ZPT, PRE, NT, 1>(a, p, s);
+}
+
+template <bool ZPT, bool PRE, int NT, int GPB>
+static int launch_async_grouped_gpb(const BatchGroupTable& tab, const FcDeviceArgs& a, const LaunchPlan& p,
+                                    hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_prefill_async_grouped_kernel<ZPT, PRE, NT>;
+    auto kern = fcc_prefill_async_grouped_kernel<ZPT, PRE, NT, GPB>;
     static bool attr_set = false;  // per instantiation
-    if (int e = allow_lds(kern, &attr_set))
+    if (int e = allow_lds(kern, &attr_set, pa_lds_bytes(GPB)))
         return e;
-    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), PA_LDS_BYTES, s, tab, a.workspace,
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(GPB), s, tab, a.workspace,
                        a.counters, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
                        L.zp_const, a.out_f32, L.glu, p.tiles_x, p.tiles_y, p.full_tiles, p.split_k,
                        p.kblocks_per_split);
     return (int)hipGetLastError();
+}
+
+template <bool ZPT, bool PRE, int NT>
+static int launch_async_grouped_impl(const BatchGroupTable& tab, const FcDeviceArgs& a, const LaunchPlan& p,
+                                     hipStream_t s) {
+    if constexpr (PRE) {
+        if (a.layout.groups_per_kblock == 2)
+            return launch_async_grouped_gpb<ZPT, PRE, NT, 2>(tab, a, p, s);
+        if (a.layout.groups_per_kblock == 4)
+            return launch_async_grouped_gpb<ZPT, PRE, NT, 4>(tab, a, p, s);
+    }
+    return launch_async_grouped_gpb<ZPT, PRE, NT, 1>(tab, a, p, s);
 }
 
 // dispatch on zero-point table, per-group scales and tile height

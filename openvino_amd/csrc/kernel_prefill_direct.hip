@@ -314,6 +314,8 @@ int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& p, void* stre
     // the launch must be what tile_work assumes: a 1-D grid of full_tiles whole tiles plus split_k parts of each
     // remaining tile, parts that cover K and rows that cover M
     const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
+    if (L.groups_per_kblock != 1)
+        return (int)hipErrorInvalidValue;  // groups below 128 inputs: the planner picks another kernel
     if (p.tile_m != PD_BM || p.tiles_x != a.N / PD_BN || (int64_t)p.tiles_y * PD_BM < a.M || p.full_tiles < 0 ||
         p.full_tiles > tiles || p.split_k < 1 || (int64_t)p.kblocks_per_split * p.split_k < L.k_blocks ||
         p.grid[0] != (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) || p.grid[1] != 1 || p.grid[2] != 1 ||

@@ -289,6 +289,8 @@ static int launch_wide_bits(const FcDeviceArgs& a, const LaunchPlan& p, hipStrea
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
+    if (L.groups_per_kblock != 1)
+        return (int)hipErrorInvalidValue;  // groups below 128 inputs: the planner picks another kernel
     if (L.bits == 4)
         return L.zp_table ? launch_wide_bits<4, true>(a, p, s) : launch_wide_bits<4, false>(a, p, s);
     return L.zp_table ? launch_wide_bits<8, true>(a, p, s) : launch_wide_bits<8, false>(a, p, s);

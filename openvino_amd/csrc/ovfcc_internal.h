@@ -23,6 +23,9 @@ namespace ovfcc {
 //     k_local = 32*(d >> 1) + 8*(l >> 4) + 4*(d & 1) + b      (within the tile's 64 inputs)
 // Weights are stored unsigned: i4 xor 8, i8 xor 0x80, with the zero-point raised to match.
 // Tiles are ordered [N/16][K/k_per_tile]; scales f16 and zero-points u8 as [N/16][groups][16].
+// Groups of 32 or 64 inputs (4-bit weights only) divide a k-block in four or two: their parameters are
+// stored [N/16][K/128][16][groups per k-block], so that a lane finds the scales of its channel for one
+// k-block in one 4- or 8-byte load; group i of a k-block scales the inputs of dwords 4 i / gpb .. of a tile.
 constexpr int kTileRows = 16;
 constexpr int kTileBytes = 1024;
 constexpr int kBlockK = 128;
@@ -35,6 +38,7 @@ struct Layout {
     int64_t tiles_per_kblock = 1;
     int64_t groups = 0;         // K / G
     int64_t kblocks_per_group = 0;
+    int groups_per_kblock = 1;  // 2 or 4 when G is 64 or 32
     bool zp_table = false;      // per-(n, group) zero-points stored as a table
     int zp_const = 0;           // zero-point used when there is no table (includes the unsigned offset)
     int zp_offset = 0;          // 8 for i4, 128 for i8, else 0
@@ -45,6 +49,13 @@ struct Layout {
     int glu = 0;
     bool glu_gate_second = false;
     bool dynquant = false;  // the node allows per-token int8 activations (OVFCC_DYNQUANT_I8) where a kernel exists
+    // element index of the scale / zero-point of channel r of tile nt for group g
+    size_t param_index(int64_t nt, int64_t g, int r) const {
+        if (groups_per_kblock == 1)
+            return (size_t)(nt * groups + g) * kTileRows + r;
+        const int64_t kb = g / groups_per_kblock, gi = g % groups_per_kblock;
+        return ((size_t)(nt * k_blocks + kb) * kTileRows + r) * groups_per_kblock + gi;
+    }
     // 16-channel block of the OpenVINO-order channel axis that tile nt holds
     int64_t source_tile(int64_t nt) const {
         if (!glu)

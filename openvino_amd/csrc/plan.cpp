@@ -193,8 +193,11 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         const int wide_env = env_int("OVFCC_PREFILL_WIDE", -1);
         if (wide_env >= 0)
             big = wide_env != 0;
-        p.direct = big && direct_ok && env_int("OVFCC_PREFILL_DIRECT", 1) != 0;
-        const bool wide = p.direct || (big && wide_ok);
+        // Groups of 32 or 64 inputs: only the all-asynchronous kernel and the square kernel carry several groups
+        // per k-block.
+        const bool small_groups = L.groups_per_kblock != 1;
+        p.direct = big && direct_ok && env_int("OVFCC_PREFILL_DIRECT", 1) != 0 && (!small_groups || may_async);
+        const bool wide = p.direct || (big && wide_ok && !small_groups);
         // 4-bit nodes take the variant whose operands all travel by direct-to-LDS loads
         p.async_dma = p.direct && L.bits == 4 && env_int("OVFCC_PREFILL_ASYNC", 1) != 0;
         p.tile_m = kPrefillTileM;

@@ -85,13 +85,15 @@ Layout make_layout(const ovfcc_fc_desc& d) {
     L.dynquant = (d.flags & OVFCC_DYNQUANT_I8) != 0;
     L.glu = d.flags & OVFCC_GLU_TYPE_MASK;
     L.glu_gate_second = (d.flags & OVFCC_GLU_GATE_SECOND) != 0;
+    const bool small_groups = L.bits == 4 && (d.group_size == 32 || d.group_size == 64);
     L.tiled = (d.N % (L.glu ? 2 * kTileRows : kTileRows) == 0) && (d.K % kBlockK == 0) &&
-              (d.group_size % kBlockK == 0) && (d.K / kBlockK < 65536);
+              (d.group_size % kBlockK == 0 || small_groups) && (d.K / kBlockK < 65536);
     if (L.tiled) {
         L.n_tiles = d.N / kTileRows;
         L.k_blocks = d.K / kBlockK;
         L.tiles_per_kblock = L.bits == 4 ? 1 : 2;
-        L.kblocks_per_group = d.group_size / kBlockK;
+        L.kblocks_per_group = small_groups ? 1 : d.group_size / kBlockK;
+        L.groups_per_kblock = small_groups ? kBlockK / (int)d.group_size : 1;
         L.w_bytes = (size_t)L.n_tiles * L.k_blocks * L.tiles_per_kblock * kTileBytes;
         L.scale_bytes = (size_t)L.n_tiles * L.groups * kTileRows * 2;
         L.zp_bytes = L.zp_table ? (size_t)L.n_tiles * L.groups * kTileRows : 0;
@@ -247,7 +249,7 @@ void repack_params(const ovfcc_fc_desc& d, const Layout& L, const void* scales, 
         for (int64_t g = 0; g < ng; ++g)
             for (int r = 0; r < kTileRows; ++r) {
                 const int64_t n = L.source_tile(nt) * kTileRows + r;
-                const size_t o = (size_t)(nt * ng + g) * kTileRows + r;
+                const size_t o = L.param_index(nt, g, r);
                 st[o] = s[n * ng + g];
                 if (L.zp_table) {
                     const unsigned v = d.zp_type == OVFCC_U4 ? nibble(z, (size_t)(n * ng + g)) : z[n * ng + g];
@@ -269,7 +271,7 @@ void unrepack_params(const ovfcc_fc_desc& d, const Layout& L, const void* scale_
         for (int64_t g = 0; g < ng; ++g)
             for (int r = 0; r < kTileRows; ++r) {
                 const int64_t n = L.source_tile(nt) * kTileRows + r;
-                const size_t o = (size_t)(nt * ng + g) * kTileRows + r;
+                const size_t o = L.param_index(nt, g, r);
                 s[n * ng + g] = st[o];
                 if (L.zp_table) {
                     const unsigned v = (unsigned)zt[o] - L.zp_offset;
@@ -324,7 +326,7 @@ int ovfcc_repack_host(const ovfcc_fc_desc* desc, const void* w, const void* scal
         return rc;
     const ovfcc::Layout L = ovfcc::make_layout(*desc);
     if (!L.tiled)
-        return ovfcc::fail(OVFCC_EUNSUPPORTED, "shape keeps the OpenVINO layout (needs N%16==0, K%128==0, G%128==0)");
+        return ovfcc::fail(OVFCC_EUNSUPPORTED, "shape keeps the OpenVINO layout (needs N%16==0, K%128==0, G%128==0 or 4-bit weights with G of 32 or 64)");
     if (!w || !scales || !w_tiled || !scale_tiled || (L.zp_table && (!zp || !zp_tiled)))
         return ovfcc::fail(OVFCC_EINVAL, "null buffer");
     ovfcc::repack_weights(*desc, L, w, w_tiled);
@@ -339,7 +341,7 @@ int ovfcc_unrepack_host(const ovfcc_fc_desc* desc, const void* w_tiled, const vo
         return rc;
     const ovfcc::Layout L = ovfcc::make_layout(*desc);
     if (!L.tiled)
-        return ovfcc::fail(OVFCC_EUNSUPPORTED, "shape keeps the OpenVINO layout (needs N%16==0, K%128==0, G%128==0)");
+        return ovfcc::fail(OVFCC_EUNSUPPORTED, "shape keeps the OpenVINO layout (needs N%16==0, K%128==0, G%128==0 or 4-bit weights with G of 32 or 64)");
     if (!w || !scales || !w_tiled || !scale_tiled || (L.zp_table && (!zp || !zp_tiled)))
         return ovfcc::fail(OVFCC_EINVAL, "null buffer");
     ovfcc::unrepack_weights(*desc, L, w_tiled, w);

@@ -110,6 +110,8 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     }
     CHECK(d.N % 128 == 0, "%s", what);
     CHECK(!p.async_dma || (p.direct && L.bits == 4), "%s", what);
+    // several groups per k-block: only the all-asynchronous and the square kernel carry them
+    CHECK(L.groups_per_kblock == 1 || (L.bits == 4 && (p.async_dma || p.tile_n == 128)), "%s gpb=%d", what, L.groups_per_kblock);
     if (p.direct) {
         const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
         CHECK(p.tile_m == 128 || (p.async_dma && p.tile_m == 64), "%s tile_m=%d", what, p.tile_m);
@@ -135,7 +137,7 @@ int main() {
     int plans = 0;
     for (int64_t N : Ns)
         for (int64_t K : Ks)
-            for (int64_t G : {(int64_t)128, K})
+            for (int64_t G : {(int64_t)32, (int64_t)64, (int64_t)128, K})
                 for (int t : types)
                     for (int fl : flags) {
                         const int zp = (t == OVFCC_U4) ? OVFCC_U4 : (t == OVFCC_U8 ? OVFCC_U8 : OVFCC_NONE);

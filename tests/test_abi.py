@@ -92,14 +92,17 @@ def test_null_descriptor_and_null_outputs():
 
 
 def test_layout_choice_and_sizes():
-    # tiled: N % 16 == 0, K % 128 == 0, G % 128 == 0
+    # tiled: N % 16 == 0, K % 128 == 0, G % 128 == 0 -- or G of 32 or 64 under 4-bit weights
     assert fc.tiled_sizes(fc.make_desc(4096, 4096, 128, "u4", "u4")) == (4096 * 4096 // 2, 4096 * 32 * 2, 4096 * 32)
     assert fc.tiled_sizes(fc.make_desc(4096, 4096, 128, "i4")) == (4096 * 4096 // 2, 4096 * 32 * 2, 0)
     assert fc.tiled_sizes(fc.make_desc(1024, 8192, 8192, "u8", "u8")) == (1024 * 8192, 1024 * 2, 1024)
     assert fc.tiled_sizes(fc.make_desc(64, 256, 256, "u8", "u8", zp_scalar=True)) == (64 * 256, 64 * 2, 0)
     # fallbacks keep the OpenVINO layout
+    assert fc.tiled_sizes(fc.make_desc(16, 256, 64, "u4", "u4")) == (16 * 256 // 2, 16 * 4 * 2, 16 * 4)
+    assert fc.tiled_sizes(fc.make_desc(32, 128, 32, "i4")) == (32 * 128 // 2, 32 * 4 * 2, 0)
+    # fallbacks keep the OpenVINO layout
     for d in (fc.make_desc(8, 4, 4, "u8"), fc.make_desc(24, 128, 128, "u4"), fc.make_desc(16, 192, 64, "u4"),
-              fc.make_desc(16, 256, 64, "u4")):
+              fc.make_desc(16, 256, 64, "u8"), fc.make_desc(16, 256, 16, "u4")):
         assert fc.tiled_sizes(d) == (0, 0, 0)
 
 

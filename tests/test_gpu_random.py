@@ -36,6 +36,8 @@ def test_random_nodes(oracle, dev, seed, monkeypatch):
             G = K if rng.random() < 0.3 else (int(rng.choice([128, 256])) if K % 256 == 0 else (128 if K % 128 == 0 else 50))
             if K % G:
                 G = K
+            if wt in ("u4", "i4") and K % 128 == 0 and rng.random() < 0.3:
+                G = int(rng.choice([32, 64]))      # two or four groups per k-block
             N = int(rng.choice([16, 32, 48, 96, 128, 256, 272, 512, 768, 40]))
             glu = str(rng.choice(["none", "none", "swish", "gelu", "gelu_tanh"]))
             second = bool(rng.integers(0, 2)) if glu != "none" else False

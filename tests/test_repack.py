@@ -13,6 +13,8 @@ SHAPES = [
     ("u8", "none", 16, 128, 128), ("u8", "u8", 16, 512, 128),
     ("u4", "u4", 16, 14336, 128),           # 112 groups per channel
     ("i4", "none", 1024, 4096, 128),        # a real k/v projection
+    # groups of 64 and 32 inputs (4-bit weights): two and four groups per k-block
+    ("u4", "u4", 32, 256, 64), ("u4", "u8", 16, 384, 32), ("i4", "none", 48, 128, 64), ("i4", "u4", 32, 512, 32),
 ]
 
 
@@ -68,19 +70,28 @@ def test_round_trip_and_unpack_emulation(oracle, wt_, zt_, N, K, G):
         q = c.w.astype(np.int32)
     assert np.array_equal(emulate_unpack(desc, wt, N, K), q.reshape(N, K) + offset)
 
-    # scale / zero-point tables: [N/16][groups][16]
+    # scale / zero-point tables: [N/16][groups][16]; with G < 128, [N/16][K/128][16][groups per k-block]
     ng = K // G
-    assert np.array_equal(st.reshape(N // 16, ng, 16).transpose(0, 2, 1).reshape(N, ng).view(np.uint16),
-                          c.scale.view(np.uint16))
+
+    def channel_major(t):
+        if G >= 128:
+            return t.reshape(N // 16, ng, 16).transpose(0, 2, 1).reshape(N, ng)
+        return t.reshape(N // 16, K // 128, 16, 128 // G).transpose(0, 2, 1, 3).reshape(N, ng)
+
+    assert np.array_equal(channel_major(st).view(np.uint16), c.scale.view(np.uint16))
     if zt is not None:
         zq = (oracle.unpack_u4(c.zp, N * ng) if zt_ == "u4" else c.zp).astype(np.int32).reshape(N, ng)
-        assert np.array_equal(zt.reshape(N // 16, ng, 16).transpose(0, 2, 1).reshape(N, ng), zq + offset)
+        assert np.array_equal(channel_major(zt), zq + offset)
 
 
 def test_repack_rejects_untiled_shapes():
     desc = fc.make_desc(24, 128, 128, "u4")
     with pytest.raises(fc.OvfccError):
         fc.repack_host(desc, np.zeros(24 * 64, np.uint8), np.zeros((24, 1), np.float16))
+    # groups of 16 inputs, and groups below 128 inputs with 8-bit weights, keep OpenVINO's layout
+    for wt_, G in (("u4", 16), ("u8", 64), ("u8", 32)):
+        desc = fc.make_desc(16, 128, G, wt_)
+        assert fc.tiled_sizes(desc) == (0, 0, 0)
 
 
 def test_half_magic_numbers_are_exact():
