@@ -265,7 +265,8 @@ int ovfcc_desc_validate(const ovfcc_fc_desc* desc);
 
 /* Sizes of the tiled layout for a descriptor; all zero when the descriptor falls back to the
  * OpenVINO layout.  w_bytes: 1 KiB tiles of 16 channels x 128 (4-bit) or 64 (8-bit) inputs;
- * scale_bytes: f16 [N/16][groups][16]; zp_bytes: u8 [N/16][groups][16] (0 without zero-points). */
+ * scale_bytes: f16 [N/16][groups][16]; zp_bytes: u8 [N/16][groups][16] (0 without zero-points).
+ * With 4-bit weights and groups of 32 or 64 inputs both tables are [N/16][K/128][16][128/group_size]. */
 int ovfcc_tiled_sizes(const ovfcc_fc_desc* desc, size_t* w_bytes, size_t* scale_bytes, size_t* zp_bytes);
 
 /* The repacker itself, host to host (what ovfcc_weights_create uploads), and its inverse, which
