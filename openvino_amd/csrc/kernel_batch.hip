@@ -110,23 +110,53 @@ __device__ __forceinline__ void batch_body(const uint4_t* __restrict__ wt, const
         }
     };
 
+    // Stage X[0 : 16 MT, k-range] in LDS; 16-byte chunks, coalesced along k; rows >= M read zeros.  The loads go
+    // out BEFORE the first weight loads: the memory counter retires in order, so a wave that asked for its weights
+    // first could not write the staged activations until all of those weights had landed, and the workgroup would
+    // start computing only after the first DEPTH k-blocks of every wave were in.  (Twelve chunks per thread cover
+    // the 96 KiB budget with eight waves; a workgroup of four waves stages the rest afterwards.)
+    constexpr int kXChunks = 12;
+    uint4_t xr[kXChunks];
+    const int x_cpr = cnt * 16;  // chunks per row
+    const int x_total = 16 * MT * x_cpr;
+    const int x_iters = (x_total + (int)blockDim.x - 1) / (int)blockDim.x;
+    const unsigned x_rcp = (unsigned)((0x100000000ull + x_cpr - 1) / x_cpr);  // idx / x_cpr for idx < 2^16
+    auto x_chunk = [&](int it, int& m, int& c) {
+        const int idx = (int)threadIdx.x + it * (int)blockDim.x;
+        m = (int)__umulhi((unsigned)idx, x_rcp);
+        c = idx - m * x_cpr;
+        return idx < x_total;
+    };
+#pragma unroll
+    for (int it = 0; it < kXChunks; ++it)
+        if (it < x_iters) {
+            int m, c;
+            const bool ok = x_chunk(it, m, c);
+            const unsigned ofs = ok ? (unsigned)(m * K + kb_begin * 128 + c * 8) * 2u : kOob;
+            xr[it] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rx, ofs, 0, 0));
+        }
+
     Slot slot[DEPTH];
 #pragma unroll
     for (int u = 0; u < DEPTH; ++u)
         issue(u, slot[u]);
 
-    // stage X[0 : 16 MT, k-range] in LDS; 16-byte chunks, coalesced along k; rows >= M read zeros
-    {
-        const int chunks_per_row = cnt * 16;
-        const int total = 16 * MT * chunks_per_row;
-        for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
-            const int m = idx / chunks_per_row, c = idx - m * chunks_per_row;
+#pragma unroll
+    for (int it = 0; it < kXChunks; ++it)
+        if (it < x_iters) {
+            int m, c;
+            if (x_chunk(it, m, c))
+                *reinterpret_cast<uint4_t*>(&xs[m * x_stride + c * 8]) = xr[it];
+        }
+    for (int it = kXChunks; it < x_iters; ++it) {
+        int m, c;
+        if (x_chunk(it, m, c)) {
             const unsigned ofs = (unsigned)(m * K + kb_begin * 128 + c * 8) * 2u;
             *reinterpret_cast<uint4_t*>(&xs[m * x_stride + c * 8]) =
                 __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rx, ofs, 0, 0));
         }
-        __syncthreads();
     }
+    __syncthreads();
     const half_t* xs_lane = xs + col * x_stride + 8 * kq;
 
     float4_t acc[RT][MT];

@@ -37,7 +37,8 @@ struct DecodeSlot {
     uint32_t zp[RT];                         // GPB zero-points, one per byte
 };
 
-template <int BITS, int MT, bool ZP_TABLE, int RT, bool XLDS, int GPB>
+// XLEAD (with XLDS): the activation loads go out before the first weight slot instead of right after it.
+template <int BITS, int MT, bool ZP_TABLE, int RT, bool XLDS, int GPB, bool XLEAD>
 __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restrict__ wt,
                                                           const half_t* __restrict__ st,
                                                           const uint8_t* __restrict__ zt,
@@ -140,20 +141,51 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
         }
     };
 
+    // Stage X[0:M, k-range of this workgroup] in LDS once, in 16-byte chunks coalesced along k.  The loads go out
+    // BEFORE most of the first weight loads: the memory counter retires in order, so a wave that asked for all
+    // its weights first could not write (or read) the staged activations until all of those weights had landed,
+    // and no workgroup would start computing before the first DEPTH k-blocks of every wave were in.
+    constexpr int kXChunks = 10;  // per thread: 40 KiB of activations over at least 256 threads
+    uint4_t xr[XLDS ? kXChunks : 1];
+    const int x_cpr = (kb_end - kb_begin) * 16;  // chunks per row
+    const int x_total = M * x_cpr;
+    const int x_iters = (x_total + (int)blockDim.x - 1) / (int)blockDim.x;
+    auto x_chunk = [&](int it, int& m, int& c) {
+        const int idx = (int)threadIdx.x + it * (int)blockDim.x;
+        m = (idx >= x_cpr) + (idx >= 2 * x_cpr) + (idx >= 3 * x_cpr);  // M <= 4
+        c = idx - m * x_cpr;
+        return idx < x_total;
+    };
+    // (When every wave's whole share of k-blocks is in flight from the start, the activations go out before all
+    // of it -- XLEAD; with more k-blocks than slots the first weight slot, which is needed first in any case,
+    // leads.  Measured: 2-4 % either way on the nodes of the other kind; the launcher picks.)
     Slot slot[DEPTH];
+    if constexpr (!XLEAD)
+        issue(0, slot[0]);
+    if constexpr (XLDS) {
 #pragma unroll
-    for (int u = 0; u < DEPTH; ++u)
+        for (int it = 0; it < kXChunks; ++it)
+            if (it < x_iters) {
+                int m, c;
+                const bool ok = x_chunk(it, m, c);
+                const unsigned ofs = ok ? (unsigned)(m * K + kb_begin * 128 + c * 8) * 2u : kOob;
+                xr[it] = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rx, ofs, 0, 0));
+            }
+    }
+    if constexpr (XLEAD)
+        issue(0, slot[0]);
+#pragma unroll
+    for (int u = 1; u < DEPTH; ++u)
         issue(u, slot[u]);
 
     if constexpr (XLDS) {
-        // stage X[0:M, k-range of this workgroup] once; 16-byte chunks, coalesced along k
-        const int chunks_per_row = (kb_end - kb_begin) * 16;
-        const int total = M * chunks_per_row;
-        for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
-            const int m = idx / chunks_per_row, c = idx - m * chunks_per_row;
-            *reinterpret_cast<uint4_t*>(&xs[m * x_stride + c * 8]) =
-                *reinterpret_cast<const uint4_t*>(x + (size_t)m * K + (size_t)kb_begin * 128 + c * 8);
-        }
+#pragma unroll
+        for (int it = 0; it < kXChunks; ++it)
+            if (it < x_iters) {
+                int m, c;
+                if (x_chunk(it, m, c))
+                    *reinterpret_cast<uint4_t*>(&xs[m * x_stride + c * 8]) = xr[it];
+            }
         __syncthreads();
     }
     // LDS operand address of this lane: rows >= M repeat row 0 (their output rows are never stored)
@@ -368,14 +400,25 @@ __global__ __launch_bounds__(1024) void fcc_decode_kernel(const uint4_t* __restr
     }
 }
 
-template <int BITS, int MT, bool ZPT, int RT, bool XLDS, int GPB>
-static void launch_decode_gpb(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+template <int BITS, int MT, bool ZPT, int RT, bool XLDS, int GPB, bool XLEAD>
+static void launch_decode_lead(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
-    hipLaunchKernelGGL((fcc_decode_kernel<BITS, MT, ZPT, RT, XLDS, GPB>), dim3(p.grid[0], p.grid[1], 1),
+    hipLaunchKernelGGL((fcc_decode_kernel<BITS, MT, ZPT, RT, XLDS, GPB, XLEAD>), dim3(p.grid[0], p.grid[1], 1),
                        dim3(p.block), p.dynamic_lds, s, (const uint4_t*)a.w, (const half_t*)a.scale,
                        (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y, a.workspace, a.counters,
                        (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
                        L.zp_const, p.kblocks_per_split, p.split_k, a.out_f32, L.glu);
+}
+
+template <int BITS, int MT, bool ZPT, int RT, bool XLDS, int GPB>
+static void launch_decode_gpb(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    if constexpr (XLDS && RT == 1) {
+        // four k-blocks per wave are in flight from the start: does a wave have more?
+        const int waves = (int)p.block / 64;
+        if ((p.kblocks_per_split + waves - 1) / waves > 4)
+            return launch_decode_lead<BITS, MT, ZPT, RT, XLDS, GPB, false>(a, p, s);
+    }
+    launch_decode_lead<BITS, MT, ZPT, RT, XLDS, GPB, XLDS>(a, p, s);
 }
 
 template <int BITS, int MT, bool ZPT, int RT, bool XLDS>
@@ -418,6 +461,9 @@ int launch_decode(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     if (L.glu && (!p.x_in_lds || a.M > 16 || (p.tiles_per_group & 1)))
         return (int)hipErrorInvalidValue;  // gate and up tile must share a workgroup
     if (L.groups_per_kblock != 1 && (L.bits != 4 || (L.groups_per_kblock != 2 && L.groups_per_kblock != 4)))
+        return (int)hipErrorInvalidValue;
+    // the staged activations: at most four rows, at most ten 16-byte chunks per thread
+    if (p.x_in_lds && (a.M > 4 || (int64_t)a.M * p.kblocks_per_split * 16 > (int64_t)10 * p.block))
         return (int)hipErrorInvalidValue;
     if (L.bits == 4)
         L.zp_table ? launch_decode_bits<4, true>(a, p, s) : launch_decode_bits<4, false>(a, p, s);
