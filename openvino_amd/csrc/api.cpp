@@ -142,9 +142,33 @@ void record(ovfcc_request* r, const ovfcc::LaunchPlan& p) {
     std::snprintf(i.name, sizeof(i.name), "%s", p.name);
 }
 
-// Enqueue one node.  A tiled node is cut into decode-family launches of at most 48 rows when M is small
-// enough that they beat one sparse prefill grid, or when N is not a multiple of the prefill tile.
+int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M);
+
+// Enqueue one node.  The fast kernels address the activations with 32-bit byte offsets and the plain kernel puts
+// the rows on a 16-bit grid axis: a longer node runs as consecutive row blocks on the same stream.
 int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M) {
+    int64_t block = M;
+    if (w->layout.tiled) {
+        const int64_t lim = ((((int64_t)1 << 31) - 1) / (2 * w->desc.K)) & ~(int64_t)127;
+        if (M > lim && lim >= 128)
+            block = lim;
+    } else if (M > 65535) {
+        block = 65535;
+    }
+    const size_t out_row = (size_t)out_channels(w) * (w->desc.out_type == OVFCC_F32 ? 4 : 2);
+    for (int64_t m0 = 0; m0 < M; m0 += block) {
+        const int64_t rows = M - m0 < block ? M - m0 : block;
+        int rc = enqueue_rows(r, w, static_cast<const char*>(x) + (size_t)m0 * w->desc.K * 2,
+                              static_cast<char*>(y) + (size_t)m0 * out_row, rows);
+        if (rc)
+            return rc;
+    }
+    return OVFCC_OK;
+}
+
+// One block of rows.  A tiled node is cut into decode-family launches of at most 48 rows when M is small
+// enough that they beat one sparse prefill grid, or when N is not a multiple of the prefill tile.
+int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M) {
     if (M == 0)
         return OVFCC_OK;
     ovfcc::FcDeviceArgs a;

@@ -625,3 +625,42 @@ def test_requests_on_concurrent_threads(oracle, dev):
         assert not failures, failures[:5]
     finally:
         w.close()
+
+
+def test_more_rows_than_32_bit_offsets_reach(oracle, dev, req):
+    """M K 2 >= 2^31 bytes of activations: the fast kernels address them with 32-bit offsets, so the node runs as
+    consecutive row blocks; rows on both sides of the block boundary, the first and the last against the oracle."""
+    K, N = 8192, 256
+    block = (((1 << 31) - 1) // (2 * K)) & ~127          # 130 944 rows
+    M = block + 128 + 300
+    say(f"long node M={M} K={K} (block {block})")
+    c = datagen.make_case(880, 4096, K, N, "i4", 128, "none", with_bias=True)
+    reps = (M + 4095) // 4096
+    x = np.tile(c.x, (reps, 1))[:M]
+    x[block - 1] *= np.float16(0.5)                      # distinct rows around the boundary
+    x[block] *= np.float16(-1.0)
+    x[M - 1] *= np.float16(0.25)
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        y = req.infer(w, x)
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_PREFILL
+        pick = np.array([0, 1, 4095, 4096, block - 2, block - 1, block, block + 1, block + 127, block + 128, M - 2, M - 1])
+        check_parity(oracle, y[pick], oracle_y(oracle, c, x=x[pick]), K, "long node")
+        assert np.array_equal(y[:4096].view(np.uint16), y[4096:8192].view(np.uint16))     # equal rows, equal results
+    finally:
+        w.close()
+
+
+def test_plain_kernel_beyond_its_row_axis(oracle, dev, req):
+    """More than 65 535 rows on a node that keeps OpenVINO's layout: row blocks again."""
+    say("plain kernel, 70 000 rows")
+    c = datagen.make_case(881, 1000, 200, 40, "u4", 50, "u4")
+    x = np.tile(c.x, (70, 1))
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        y = req.infer(w, x)
+        assert req.last_kernel()["name"] == "fcc_plain" and y.shape == (70000, 40)
+        pick = np.array([0, 999, 65534, 65535, 65536, 69999])
+        check_parity(oracle, y[pick], oracle_y(oracle, c, x=x[pick]), 200, "plain long", output_rounding_slack=True)
+    finally:
+        w.close()
