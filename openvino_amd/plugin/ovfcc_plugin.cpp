@@ -246,6 +246,145 @@ static void chain_nodes(const CompressedFc& fc, std::vector<std::shared_ptr<ov::
     }
 }
 
+// ---- device-resident tensors -------------------------------------------------------------------------------
+// The plugin's remote context hands out tensors that live in HBM (src/inference/dev_api/openvino/runtime/
+// iremote_context.hpp:24-62, iremote_tensor.hpp:18-78; template: src/plugins/template/src/remote_context.cpp:17-140).
+// An infer request whose input and output are such tensors runs without any host copy.
+
+class RemoteTensor : public ov::IRemoteTensor {
+public:
+    RemoteTensor(std::shared_ptr<const ov::IPlugin> plugin, ovfcc_ctx* ctx, const ov::element::Type& type,
+                 const ov::Shape& shape)
+        : m_plugin(std::move(plugin)), m_ctx(ctx), m_type(type), m_shape(shape), m_device_name("MI355X") {
+        OPENVINO_ASSERT(type.bitwidth() >= 8, "MI355X: remote tensors hold whole-byte element types, got ", type);
+        reserve(byte_size_of(shape));
+        update_strides();
+    }
+    ~RemoteTensor() override {
+        if (m_ptr)
+            ovfcc_device_free(m_ctx, m_ptr);
+    }
+
+    const ov::element::Type& get_element_type() const override {
+        return m_type;
+    }
+    const ov::Shape& get_shape() const override {
+        return m_shape;
+    }
+    const ov::Strides& get_strides() const override {
+        return m_strides;
+    }
+    // A larger shape takes a fresh allocation (the old contents are dropped), a smaller one keeps the memory.
+    void set_shape(ov::Shape shape) override {
+        reserve(byte_size_of(shape));
+        m_shape = std::move(shape);
+        update_strides();
+    }
+    const ov::AnyMap& get_properties() const override {
+        return m_properties;
+    }
+    const std::string& get_device_name() const override {
+        return m_device_name;
+    }
+    // Whole-tensor copies only (offsets 0, empty region): what Tensor::copy_to / copy_from of the public API issue.
+    void copy_from(const std::shared_ptr<const ov::ITensor>& src, size_t src_offset, size_t dst_offset,
+                   const ov::Shape& roi_shape) override {
+        OPENVINO_ASSERT(src_offset == 0 && dst_offset == 0 && roi_shape.empty(), "MI355X: region copies are not implemented");
+        OPENVINO_ASSERT(src->get_element_type() == m_type && src->is_continuous(),
+                        "MI355X: copy_from needs a dense tensor of type ", m_type);
+        set_shape(src->get_shape());
+        if (auto remote = std::dynamic_pointer_cast<const RemoteTensor>(src)) {
+            // device to device through the host would be wasteful; the library's copy kernel does it in place
+            float ms = 0.f;
+            const size_t bytes = (get_byte_size() + 15) / 16 * 16;  // allocations are padded to 16 bytes
+            if (bytes && ovfcc_bench_copy(m_ctx, m_ptr, remote->device_ptr(), bytes, 1, &ms) != OVFCC_OK)
+                throw_last("device copy");
+        } else if (get_byte_size() && ovfcc_memcpy_h2d(m_ctx, m_ptr, src->data(), get_byte_size()) != OVFCC_OK) {
+            throw_last("memcpy_h2d");
+        }
+    }
+    void copy_to(const std::shared_ptr<ov::ITensor>& dst, size_t src_offset, size_t dst_offset,
+                 const ov::Shape& roi_shape) const override {
+        OPENVINO_ASSERT(src_offset == 0 && dst_offset == 0 && roi_shape.empty(), "MI355X: region copies are not implemented");
+        OPENVINO_ASSERT(dst->get_element_type() == m_type, "MI355X: copy_to needs a tensor of type ", m_type);
+        if (auto remote = std::dynamic_pointer_cast<RemoteTensor>(dst)) {
+            remote->copy_from(std::static_pointer_cast<const ov::ITensor>(shared_from_this_tensor()), 0, 0, {});
+            return;
+        }
+        dst->set_shape(m_shape);
+        OPENVINO_ASSERT(dst->is_continuous(), "MI355X: copy_to needs a dense destination");
+        if (get_byte_size() && ovfcc_memcpy_d2h(m_ctx, dst->data(), m_ptr, get_byte_size()) != OVFCC_OK)
+            throw_last("memcpy_d2h");
+    }
+
+    void* device_ptr() const {
+        return m_ptr;
+    }
+
+private:
+    size_t byte_size_of(const ov::Shape& shape) const {
+        return ov::shape_size(shape) * m_type.size();
+    }
+    // copy_to(remote) needs `this` as a shared tensor; a non-owning alias is enough for the duration of the call
+    std::shared_ptr<const RemoteTensor> shared_from_this_tensor() const {
+        return std::shared_ptr<const RemoteTensor>(std::shared_ptr<const RemoteTensor>{}, this);
+    }
+    void reserve(size_t bytes) {
+        bytes = (std::max<size_t>(bytes, 16) + 15) / 16 * 16;
+        if (bytes <= m_capacity)
+            return;
+        if (m_ptr)
+            ovfcc_device_free(m_ctx, m_ptr);
+        m_ptr = nullptr;
+        m_capacity = 0;
+        if (ovfcc_device_malloc(m_ctx, bytes, &m_ptr) != OVFCC_OK)
+            throw_last("device_malloc");
+        m_capacity = bytes;
+        m_properties = {{ov::device::full_name.name(), m_device_name}, {"DEV_MEM_PTR", m_ptr}};
+    }
+    void update_strides() {
+        m_strides.assign(m_shape.size(), 0);
+        size_t stride = m_type.size();
+        for (size_t d = m_shape.size(); d-- > 0;) {
+            m_strides[d] = stride;
+            stride *= m_shape[d];
+        }
+    }
+
+    std::shared_ptr<const ov::IPlugin> m_plugin;  // keeps the device context alive
+    ovfcc_ctx* m_ctx;
+    ov::element::Type m_type;
+    ov::Shape m_shape;
+    ov::Strides m_strides;
+    std::string m_device_name;
+    ov::AnyMap m_properties;
+    void* m_ptr = nullptr;
+    size_t m_capacity = 0;
+};
+
+class RemoteContext : public ov::IRemoteContext {
+public:
+    RemoteContext(std::shared_ptr<const ov::IPlugin> plugin, ovfcc_ctx* ctx)
+        : m_plugin(std::move(plugin)), m_ctx(ctx), m_name("MI355X"),
+          m_property{{ov::device::full_name.name(), std::string("AMD Instinct MI355X (gfx950) via ovfcc")}} {}
+    const std::string& get_device_name() const override {
+        return m_name;
+    }
+    const ov::AnyMap& get_property() const override {
+        return m_property;
+    }
+    ov::SoPtr<ov::IRemoteTensor> create_tensor(const ov::element::Type& type, const ov::Shape& shape,
+                                               const ov::AnyMap&) override {
+        return {std::make_shared<RemoteTensor>(m_plugin, m_ctx, type, shape), nullptr};
+    }
+
+private:
+    std::shared_ptr<const ov::IPlugin> m_plugin;
+    ovfcc_ctx* m_ctx;
+    std::string m_name;
+    ov::AnyMap m_property;
+};
+
 // ---- plugin -------------------------------------------------------------------------------------------------
 
 class Plugin;
@@ -354,6 +493,9 @@ public:
             });
     }
     ~InferRequest() override {
+        for (auto& b : m_device_staging)
+            if (b.ptr)
+                ovfcc_device_free(m_compiled->ctx(), b.ptr);
         ovfcc_request_destroy(m_request);
     }
 
@@ -370,17 +512,38 @@ public:
             ov::Shape out_shape = in_shape;
             out_shape.back() = (size_t)node.fc.desc.N;
             out->set_shape(out_shape);  // dynamic M: the output follows the input
-            const void* x = in->data();
-            if (in->get_element_type() == ov::element::f32) {
-                // the device path computes on f16 activations
-                const float* src = static_cast<const float*>(in->data());
-                m_staging.resize((size_t)M * node.fc.desc.K);
-                for (size_t i = 0; i < m_staging.size(); ++i)
-                    m_staging[i] = ov::float16(src[i]);
-                x = m_staging.data();
+            auto rin = std::dynamic_pointer_cast<RemoteTensor>(in._ptr);
+            auto rout = std::dynamic_pointer_cast<RemoteTensor>(out._ptr);
+            if (rin || rout) {
+                // Device-resident tensors: no copy on their side.  A host tensor on the other side goes through a
+                // device buffer of the request.
+                OPENVINO_ASSERT(in->get_element_type() == ov::element::f16,
+                                "MI355X: a device-resident input must be f16, got ", in->get_element_type());
+                const size_t x_bytes = (size_t)M * node.fc.desc.K * sizeof(ov::float16);
+                const size_t y_bytes = out->get_byte_size();
+                void* x_dev = rin ? rin->device_ptr() : device_staging(0, x_bytes);
+                void* y_dev = rout ? rout->device_ptr() : device_staging(1, y_bytes);
+                if (!rin && x_bytes && ovfcc_memcpy_h2d(m_compiled->ctx(), x_dev, in->data(), x_bytes) != OVFCC_OK)
+                    throw_last("memcpy_h2d");
+                if (ovfcc_fc_run_device(m_request, node.weights, x_dev, y_dev, M) != OVFCC_OK)
+                    throw_last("fc_run_device");
+                if (ovfcc_request_sync(m_request) != OVFCC_OK)
+                    throw_last("request_sync");
+                if (!rout && y_bytes && ovfcc_memcpy_d2h(m_compiled->ctx(), out->data(), y_dev, y_bytes) != OVFCC_OK)
+                    throw_last("memcpy_d2h");
+            } else {
+                const void* x = in->data();
+                if (in->get_element_type() == ov::element::f32) {
+                    // the device path computes on f16 activations
+                    const float* src = static_cast<const float*>(in->data());
+                    m_staging.resize((size_t)M * node.fc.desc.K);
+                    for (size_t i = 0; i < m_staging.size(); ++i)
+                        m_staging[i] = ov::float16(src[i]);
+                    x = m_staging.data();
+                }
+                if (ovfcc_fc_run(m_request, node.weights, x, out->data(), M) != OVFCC_OK)
+                    throw_last("fc_run");
             }
-            if (ovfcc_fc_run(m_request, node.weights, x, out->data(), M) != OVFCC_OK)
-                throw_last("fc_run");
             ovfcc_kernel_info info;
             ovfcc_last_kernel_info(m_request, &info);
             m_kernels.push_back(info);
@@ -412,8 +575,27 @@ private:
             tensor->set_shape(shape);
     }
 
+    // device buffer `which` (0 = activations, 1 = outputs) of at least `bytes`, kept and grown across calls
+    void* device_staging(int which, size_t bytes) {
+        auto& b = m_device_staging[which];
+        if (bytes > b.bytes) {
+            if (b.ptr)
+                ovfcc_device_free(m_compiled->ctx(), b.ptr);
+            b.ptr = nullptr, b.bytes = 0;
+            if (ovfcc_device_malloc(m_compiled->ctx(), bytes, &b.ptr) != OVFCC_OK)
+                throw_last("device_malloc");
+            b.bytes = bytes;
+        }
+        return b.ptr;
+    }
+
+    struct DeviceBuffer {
+        void* ptr = nullptr;
+        size_t bytes = 0;
+    };
     std::shared_ptr<const CompiledModel> m_compiled;
     ovfcc_request* m_request = nullptr;
+    DeviceBuffer m_device_staging[2];
     std::vector<ov::float16> m_staging;
     std::vector<ovfcc_kernel_info> m_kernels;
 };
@@ -517,11 +699,14 @@ public:
         OPENVINO_THROW("MI355X: unsupported property ", name);
     }
 
+    // One kind of context: the device's own memory (template: src/plugins/template/src/plugin.cpp:115-124).
     ov::SoPtr<ov::IRemoteContext> create_context(const ov::AnyMap&) const override {
-        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: remote contexts are not implemented");
+        return {std::make_shared<RemoteContext>(shared_from_this(), context()), nullptr};
     }
+    // (Contexts hold no state of their own, so the default one is not cached: a cached context would keep the
+    // plugin alive, which it points back to.)
     ov::SoPtr<ov::IRemoteContext> get_default_context(const ov::AnyMap&) const override {
-        OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: remote contexts are not implemented");
+        return {std::make_shared<RemoteContext>(shared_from_this(), context()), nullptr};
     }
     // The reverse of CompiledModel::export_model: the model is read back through Core, the nodes are rebuilt from
     // their device images without repacking (template: src/plugins/template/src/plugin.cpp:230-311).
