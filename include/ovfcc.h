@@ -57,7 +57,7 @@ typedef struct ovfcc_fc_desc {
     int32_t bias_type;  /* OVFCC_NONE | OVFCC_F16, [N] */
     int32_t act_type;   /* OVFCC_F16 */
     int32_t out_type;   /* OVFCC_F16 | OVFCC_F32 (FullyConnected's output_type; default = activation type) */
-    int32_t flags;      /* 0, or a gated-linear-unit epilogue: OVFCC_GLU_* [| OVFCC_GLU_GATE_SECOND] */
+    int32_t flags;      /* 0, or OVFCC_GLU_* [| OVFCC_GLU_GATE_SECOND] | OVFCC_DYNQUANT_I8 | OVFCC_W_INPUT_MAJOR */
 } ovfcc_fc_desc;
 
 /* Gated linear unit fused into the node (flags).  The reference fuses ov::op::internal::GLU
@@ -93,6 +93,16 @@ typedef struct ovfcc_fc_desc {
  * integers exact, which differs from the f16 result by the quantisation noise (about 1e-2 relative; the
  * reference tests such nodes with absolute tolerances of 0.1-0.2). */
 #define OVFCC_DYNQUANT_I8 8
+
+/* Input-major constants (flags): W is given as [K, N] (grouped: [K/G, G, N]) and scales / zero-points as
+ * [K/G, N], each packed over its own flattened index -- the form in which a MatMul with transpose_b = false holds
+ * its weights.  The reference brings such a node to [N, K] by a constant-folded Transpose that
+ * ConvertMatMulToFC inserts (src/plugins/intel_cpu/src/transformations/cpu_opset/common/pass/
+ * convert_matmul_to_fc.cpp:47-270) and ConvertFullyConnectedToFullyConnectedCompressed replays on scales and
+ * zero-points (convert_fc_to_compressed.cpp:170-225); here ovfcc_weights_create (and ovfcc_repack_host) do that
+ * transposition once on the host.  The node that results is the [N, K] node: ovfcc_weights_export never carries
+ * the flag.  A scalar zero-point and the bias [N] are not affected. */
+#define OVFCC_W_INPUT_MAJOR 16
 
 typedef struct ovfcc_ctx ovfcc_ctx;         /* one device + its kernels */
 typedef struct ovfcc_weights ovfcc_weights; /* repacked, device-resident W/S/ZP/bias of one node */

@@ -315,6 +315,16 @@ int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* 
         return fail(OVFCC_EINVAL, "bias type given without a buffer");
     HIP_TRY(hipSetDevice(ctx->device));
 
+    // Input-major constants are transposed once, here; from then on the node is the [N, K] node.
+    ovfcc::OutputMajorCopy nk;
+    ovfcc_fc_desc own = *desc;
+    if (own.flags & OVFCC_W_INPUT_MAJOR) {
+        ovfcc::transpose_input_major(own, w, scales, zp, &nk);
+        w = nk.w.data(), scales = nk.scales.data(), zp = nk.zp.empty() ? zp : nk.zp.data();
+        own.flags &= ~OVFCC_W_INPUT_MAJOR;
+    }
+    desc = &own;
+
     ovfcc_weights* W = new ovfcc_weights();
     W->ctx = ctx;
     W->desc = *desc;

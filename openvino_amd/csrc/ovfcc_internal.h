@@ -4,6 +4,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <string>
+#include <vector>
 
 #include "ovfcc.h"
 
@@ -72,6 +73,16 @@ int validate_desc(const ovfcc_fc_desc* d);
 // Fills the layout for a validated descriptor (tiled == false when the fallback applies).
 Layout make_layout(const ovfcc_fc_desc& d);
 int scalar_zero_point(const ovfcc_fc_desc& d, const void* zp);
+
+// Input-major constants (OVFCC_W_INPUT_MAJOR) brought to the node's own order: W [K, N] -> [N, K], scales and
+// zero-point tables [K/G, N] -> [N, K/G], each packed over its flattened index.  A scalar zero-point (one element)
+// is copied.  Vectors that the descriptor does not use stay empty.
+struct OutputMajorCopy {
+    std::vector<uint8_t> w, zp;
+    std::vector<uint16_t> scales;
+};
+void transpose_input_major(const ovfcc_fc_desc& d, const void* w, const void* scales, const void* zp,
+                           OutputMajorCopy* out);
 
 void repack_weights(const ovfcc_fc_desc& d, const Layout& L, const void* w, void* w_tiled);
 void repack_params(const ovfcc_fc_desc& d, const Layout& L, const void* scales, const void* zp, void* scale_tiled,

@@ -63,7 +63,7 @@ int validate_desc(const ovfcc_fc_desc* d) {
         return fail(OVFCC_EUNSUPPORTED, "activations must be f16");
     if (d->out_type != OVFCC_F16 && d->out_type != OVFCC_F32)
         return fail(OVFCC_EUNSUPPORTED, "output must be f16 or f32");
-    if (d->flags & ~(OVFCC_GLU_TYPE_MASK | OVFCC_GLU_GATE_SECOND | OVFCC_DYNQUANT_I8))
+    if (d->flags & ~(OVFCC_GLU_TYPE_MASK | OVFCC_GLU_GATE_SECOND | OVFCC_DYNQUANT_I8 | OVFCC_W_INPUT_MAJOR))
         return fail(OVFCC_EINVAL, "unknown bits in flags");
     if ((d->flags & OVFCC_GLU_GATE_SECOND) && (d->flags & OVFCC_GLU_TYPE_MASK) == OVFCC_GLU_NONE)
         return fail(OVFCC_EINVAL, "OVFCC_GLU_GATE_SECOND without a gated-linear-unit type");
@@ -152,6 +152,49 @@ static inline uint32_t permute_nibbles_from_tile(uint32_t t) {
         out |= ((t >> (4 * p)) & 0xFu) << (4 * e);
     }
     return out;
+}
+
+static inline void set_nibble(uint8_t* p, size_t i, unsigned v) {
+    uint8_t& b = p[i >> 1];
+    b = (i & 1) ? (uint8_t)((b & 0x0F) | (v << 4)) : (uint8_t)((b & 0xF0) | v);
+}
+
+// rows x cols (row-major, `bits` per element, packed over the flattened index) -> cols x rows
+static void transpose_elements(const uint8_t* src, uint8_t* dst, int64_t rows, int64_t cols, int bits) {
+    if (bits == 4) {
+        // Two output rows share a byte where `rows` is odd, so workers own pairs of output rows.
+        parallel_for((cols + 1) / 2, [&](int64_t pair) {
+            for (int64_t c = 2 * pair; c < std::min(cols, 2 * pair + 2); ++c)
+                for (int64_t r = 0; r < rows; ++r)
+                    set_nibble(dst, (size_t)(c * rows + r), nibble(src, (size_t)(r * cols + c)));
+        });
+    } else {
+        const int bytes = bits / 8;
+        parallel_for(cols, [&](int64_t c) {
+            for (int64_t r = 0; r < rows; ++r)
+                std::memcpy(dst + (size_t)(c * rows + r) * bytes, src + (size_t)(r * cols + c) * bytes, bytes);
+        });
+    }
+}
+
+void transpose_input_major(const ovfcc_fc_desc& d, const void* w, const void* scales, const void* zp,
+                           OutputMajorCopy* out) {
+    const int64_t N = d.N, K = d.K, ng = K / d.group_size;
+    const int wbits = is4(d.w_type) ? 4 : 8;
+    out->w.assign(((size_t)N * K * wbits + 7) / 8, 0);
+    transpose_elements(static_cast<const uint8_t*>(w), out->w.data(), K, N, wbits);
+    out->scales.assign((size_t)N * ng, 0);
+    transpose_elements(static_cast<const uint8_t*>(scales), reinterpret_cast<uint8_t*>(out->scales.data()), ng, N, 16);
+    out->zp.clear();
+    if (d.zp_type != OVFCC_NONE && zp) {
+        const int zbits = d.zp_type == OVFCC_U4 ? 4 : 8;
+        if (d.zp_scalar) {
+            out->zp.assign(1, static_cast<const uint8_t*>(zp)[0]);
+        } else {
+            out->zp.assign(((size_t)N * ng * zbits + 7) / 8, 0);
+            transpose_elements(static_cast<const uint8_t*>(zp), out->zp.data(), ng, N, zbits);
+        }
+    }
 }
 
 void repack_weights(const ovfcc_fc_desc& d, const Layout& L, const void* w, void* w_tiled) {
@@ -329,6 +372,11 @@ int ovfcc_repack_host(const ovfcc_fc_desc* desc, const void* w, const void* scal
         return ovfcc::fail(OVFCC_EUNSUPPORTED, "shape keeps the OpenVINO layout (needs N%16==0, K%128==0, G%128==0 or 4-bit weights with G of 32 or 64)");
     if (!w || !scales || !w_tiled || !scale_tiled || (L.zp_table && (!zp || !zp_tiled)))
         return ovfcc::fail(OVFCC_EINVAL, "null buffer");
+    ovfcc::OutputMajorCopy nk;
+    if (desc->flags & OVFCC_W_INPUT_MAJOR) {
+        ovfcc::transpose_input_major(*desc, w, scales, zp, &nk);
+        w = nk.w.data(), scales = nk.scales.data(), zp = nk.zp.empty() ? zp : nk.zp.data();
+    }
     ovfcc::repack_weights(*desc, L, w, w_tiled);
     ovfcc::repack_params(*desc, L, scales, zp, scale_tiled, zp_tiled);
     return OVFCC_OK;
@@ -339,6 +387,8 @@ int ovfcc_unrepack_host(const ovfcc_fc_desc* desc, const void* w_tiled, const vo
     int rc = ovfcc::validate_desc(desc);
     if (rc != OVFCC_OK)
         return rc;
+    if (desc->flags & OVFCC_W_INPUT_MAJOR)
+        return ovfcc::fail(OVFCC_EINVAL, "tiles unpack to the [N, K] order; clear OVFCC_W_INPUT_MAJOR");
     const ovfcc::Layout L = ovfcc::make_layout(*desc);
     if (!L.tiled)
         return ovfcc::fail(OVFCC_EUNSUPPORTED, "shape keeps the OpenVINO layout (needs N%16==0, K%128==0, G%128==0 or 4-bit weights with G of 32 or 64)");

@@ -28,6 +28,33 @@ def pack_nibbles(values: np.ndarray) -> np.ndarray:
     return (v[0::2] | (v[1::2] << 4)).astype(np.uint8)
 
 
+def unpack_nibbles(packed: np.ndarray, count: int) -> np.ndarray:
+    """Bytes -> the first `count` 4-bit values (0..15), low nibble first."""
+    b = np.asarray(packed, dtype=np.uint8).ravel()
+    v = np.empty(b.size * 2, np.uint8)
+    v[0::2] = b & 0x0F
+    v[1::2] = b >> 4
+    return v[:count]
+
+
+def to_input_major(c: "FcCase"):
+    """The constants of a case as a MatMul with transpose_b = false holds them: W [K, N], scales and zero-point
+    table [K / G, N], each packed over its own flattened index.  Returns (w, scale, zp)."""
+    N, K, ng = c.N, c.K, c.K // c.group_size
+    if c.w_type in ("u4", "i4"):
+        w = pack_nibbles(unpack_nibbles(c.w, N * K).reshape(N, K).T)
+    else:
+        w = np.ascontiguousarray(np.asarray(c.w, dtype=np.uint8).reshape(N, K).T).ravel()
+    scale = np.ascontiguousarray(np.asarray(c.scale).reshape(N, ng).T)
+    zp = c.zp
+    if zp is not None and not c.zp_scalar:
+        if c.zp_type == "u4":
+            zp = pack_nibbles(unpack_nibbles(zp, N * ng).reshape(N, ng).T)
+        else:
+            zp = np.ascontiguousarray(np.asarray(zp, dtype=np.uint8).reshape(N, ng).T).ravel()
+    return w, scale, zp
+
+
 @dataclass
 class FcCase:
     """One FullyConnectedCompressed problem in OpenVINO's constant layout."""

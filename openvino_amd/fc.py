@@ -22,7 +22,8 @@ def _vp(a: Optional[np.ndarray]):
 
 def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
               has_bias: bool = False, out_type: str = "f16", glu: Optional[str] = None,
-              glu_gate_second: bool = False, dynamic_quantization: bool = False) -> FcDesc:
+              glu_gate_second: bool = False, dynamic_quantization: bool = False,
+              input_major: bool = False) -> FcDesc:
     d = FcDesc()
     d.N, d.K, d.group_size = N, K, group_size
     d.w_type = _lib.TYPE[w_type]
@@ -33,7 +34,7 @@ def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none
     d.act_type = _lib.F16
     d.out_type = _lib.TYPE[out_type]
     d.flags = (_lib.GLU[glu] | (_lib.GLU_GATE_SECOND if glu_gate_second else 0) |
-               (_lib.DYNQUANT_I8 if dynamic_quantization else 0))
+               (_lib.DYNQUANT_I8 if dynamic_quantization else 0) | (_lib.W_INPUT_MAJOR if input_major else 0))
     return d
 
 
@@ -88,13 +89,15 @@ class CompressedWeights:
     def __init__(self, device: Device, W: np.ndarray, weight_scales: np.ndarray, weight_zero_points=None, bias=None, *,
                  N: int, K: int, group_size: int, w_type: str, zp_type: str = "none", zp_scalar: bool = False,
                  output_type: str = "f16", glu: Optional[str] = None, glu_gate_second: bool = False,
-                 dynamic_quantization: bool = False):
+                 dynamic_quantization: bool = False, input_major: bool = False):
         """glu = "swish" | "gelu" | "gelu_tanh": W holds gate and up projection ([N, K], first and second half of
-        the rows, or the other way round with glu_gate_second) and the node computes act(gate) * up, [M, N / 2]."""
+        the rows, or the other way round with glu_gate_second) and the node computes act(gate) * up, [M, N / 2].
+        input_major: W is [K, N] and scales / zero-points [K / G, N] (a MatMul with transpose_b = false)."""
         self.device = device
         self.N, self.K, self.group_size = N, K, group_size
         self.desc = make_desc(N, K, group_size, w_type, zp_type if weight_zero_points is not None else "none",
-                              zp_scalar, bias is not None, output_type, glu, glu_gate_second, dynamic_quantization)
+                              zp_scalar, bias is not None, output_type, glu, glu_gate_second, dynamic_quantization,
+                              input_major)
         W = np.ascontiguousarray(W).view(np.uint8)
         s = np.ascontiguousarray(weight_scales, dtype=np.float16)
         z = None if weight_zero_points is None else np.ascontiguousarray(weight_zero_points, dtype=np.uint8)

@@ -7,7 +7,10 @@
 //
 // What the plugin accepts: models whose Results are MatMuls (transpose_a = false) of a Parameter with a
 // weight-decompression subgraph
-//     Constant(u4|i4|u8|i8) -> Convert -> [Subtract(zp)] -> Multiply(scale) -> [Reshape] -> [Convert] -> MatMul
+//     Constant(u4|i4|u8|i8) -> Convert -> [Subtract(zp)] -> Multiply(scale) -> [Reshape] -> [Convert] ->
+//     [Transpose] -> [Convert] -> MatMul
+// with the constants either output-major ([N, K]: transpose_b = true, or a Transpose node under transpose_b = false)
+// or input-major ([K, N]: transpose_b = false and no Transpose node),
 // i.e. exactly what ConvertMatMulToFC + ConvertFullyConnectedToFullyConnectedCompressed fold into
 // ov::op::internal::FullyConnectedCompressed on the CPU plugin
 // (src/plugins/intel_cpu/src/transformations/cpu_opset/common/pass/convert_matmul_to_fc.cpp:47-270,
@@ -63,7 +66,7 @@ struct CompressedFc {
     std::shared_ptr<ov::op::v0::Parameter> activations;
     std::shared_ptr<ov::op::v0::Constant> weights, scales, zero_points;  // zero_points may be null
     ovfcc_fc_desc desc{};
-    std::vector<ov::float16> scales_f16;  // [N, K/G]
+    std::vector<ov::float16> scales_f16;  // [N, K/G] ([K/G, N] with OVFCC_W_INPUT_MAJOR)
     std::vector<uint8_t> zp_bytes;        // packed u4 / u8 in OpenVINO order, or one element
 };
 
@@ -86,13 +89,15 @@ static int weight_tag(const ov::element::Type& t) {
 // pattern::op::CompressedWeightsBlock (src/common/transformations/src/transformations/pattern_blocks/
 // compressed_weights_block.cpp:31-84) and the shape algebra of combine_groups
 // (convert_fc_to_compressed.cpp:42-78): W [N, K] or [N, K/G, G]; scale and zero-point [N, 1], [N, K/G, 1],
-// [N], [1] or [].
+// [N], [1] or []; or all of them input-major ([K, N], [K/G, G, N], [K/G, 1, N], ...) under a MatMul with
+// transpose_b = false, the form of the reference's decompression tests without transpose_weights
+// (src/tests/test_utils/common_test_utils/src/subgraph_builders/weights_decompression_builders.cpp:60-204).
 static bool match_compressed_fc(const std::shared_ptr<ov::Node>& node, CompressedFc& fc, std::string& why) {
     auto mm = ov::as_type_ptr<ov::op::v0::MatMul>(node);
     if (!mm)
         return false;
-    if (mm->get_transpose_a() || !mm->get_transpose_b()) {
-        why = "MatMul must have transpose_a = false and transpose_b = true (weights [N, K])";
+    if (mm->get_transpose_a()) {
+        why = "MatMul must have transpose_a = false";
         return false;
     }
     auto param = ov::as_type_ptr<ov::op::v0::Parameter>(mm->input_value(0).get_node_shared_ptr());
@@ -100,10 +105,27 @@ static bool match_compressed_fc(const std::shared_ptr<ov::Node>& node, Compresse
         why = "activations must come straight from a Parameter";
         return false;
     }
-    // walk up from the MatMul's weight input: [Convert] <- [Reshape] <- Multiply
+    // walk up from the MatMul's weight input: [Convert] <- [Transpose of the last two axes] <- [Convert] <-
+    // [Reshape] <- Multiply
     auto w = mm->input_value(1).get_node_shared_ptr();
     if (auto cvt = ov::as_type_ptr<ov::op::v0::Convert>(w))
         w = cvt->input_value(0).get_node_shared_ptr();
+    bool transposed_in_graph = false;
+    if (auto tr = ov::as_type_ptr<ov::op::v1::Transpose>(w)) {
+        auto order = ov::as_type_ptr<ov::op::v0::Constant>(tr->input_value(1).get_node_shared_ptr());
+        if (!order || order->cast_vector<int64_t>() != std::vector<int64_t>{1, 0}) {
+            why = "a Transpose on the weight path must swap the two axes of a 2-D constant";
+            return false;
+        }
+        transposed_in_graph = true;
+        w = tr->input_value(0).get_node_shared_ptr();
+        if (auto cvt = ov::as_type_ptr<ov::op::v0::Convert>(w))
+            w = cvt->input_value(0).get_node_shared_ptr();
+    }
+    // The constants are output-major ([N, K], what FullyConnected wants) when exactly one of transpose_b and the
+    // Transpose node turns them; otherwise they are input-major ([K, N]) and the library transposes them once,
+    // as the Transpose that ConvertMatMulToFC inserts does in the reference (convert_matmul_to_fc.cpp:47-270).
+    const bool input_major = mm->get_transpose_b() == transposed_in_graph;
     if (auto rs = ov::as_type_ptr<ov::op::v1::Reshape>(w))
         w = rs->input_value(0).get_node_shared_ptr();
     auto mul = ov::as_type_ptr<ov::op::v1::Multiply>(w);
@@ -145,15 +167,19 @@ static bool match_compressed_fc(const std::shared_ptr<ov::Node>& node, Compresse
     const auto& ws = wconst->get_shape();
     int64_t N, K, G;
     if (ws.size() == 2) {
-        N = (int64_t)ws[0];
-        K = (int64_t)ws[1];
+        N = (int64_t)ws[input_major ? 1 : 0];
+        K = (int64_t)ws[input_major ? 0 : 1];
         G = K;
-    } else if (ws.size() == 3) {
+    } else if (ws.size() == 3 && !input_major) {
         N = (int64_t)ws[0];
         K = (int64_t)(ws[1] * ws[2]);
         G = (int64_t)ws[2];
+    } else if (ws.size() == 3) {
+        N = (int64_t)ws[2];
+        K = (int64_t)(ws[0] * ws[1]);
+        G = (int64_t)ws[1];
     } else {
-        why = "weights must be [N, K] or [N, K/G, G]";
+        why = "weights must be [N, K] or [N, K/G, G] (or [K, N], [K/G, G, N] for a MatMul that does not transpose them)";
         return false;
     }
     const int64_t ng = K / G;
@@ -190,8 +216,8 @@ static bool match_compressed_fc(const std::shared_ptr<ov::Node>& node, Compresse
     fc.desc.bias_type = OVFCC_NONE;
     fc.desc.act_type = OVFCC_F16;
     fc.desc.out_type = mm->get_output_element_type(0) == ov::element::f32 ? OVFCC_F32 : OVFCC_F16;
-    fc.desc.flags = 0;
-    // scales as f16 [N, K/G]
+    fc.desc.flags = input_major ? OVFCC_W_INPUT_MAJOR : 0;
+    // scales as f16 in the constant's own order: [N, K/G], or [K/G, N] for input-major constants
     fc.scales_f16.resize((size_t)(N * ng));
     {
         const auto vals = scale->cast_vector<float>();

@@ -664,3 +664,34 @@ def test_plain_kernel_beyond_its_row_axis(oracle, dev, req):
         check_parity(oracle, y[pick], oracle_y(oracle, c, x=x[pick]), 200, "plain long", output_rounding_slack=True)
     finally:
         w.close()
+
+
+@pytest.mark.parametrize("wt,zt,N,K,G,scalar_zp", [
+    ("u4", "u4", 256, 512, 128, False),      # tiled, zero-point table
+    ("i4", "none", 512, 256, 64, False),     # tiled, two groups per k-block
+    ("u8", "u8", 64, 256, 256, False),       # tiled, one group per channel
+    ("u8", "u8", 128, 256, 128, True),       # scalar zero-point: untouched by the transposition
+    ("u4", "u4", 25, 100, 50, False),        # OpenVINO layout (plain kernel), odd N: rows share bytes
+    ("i8", "none", 7, 96, 32, False),
+])
+def test_input_major_constants(oracle, dev, req, wt, zt, N, K, G, scalar_zp):
+    """W [K, N] with scales / zero-points [K / G, N] (OVFCC_W_INPUT_MAJOR, a MatMul with transpose_b = false): the
+    node is the [N, K] node -- same outputs bit for bit, same exported image -- and meets the oracle bounds."""
+    say(f"input-major {wt}/{zt} N={N} K={K} G={G} scalar_zp={scalar_zp}")
+    c = datagen.make_case(870, 70, K, N, wt, G, zt, with_bias=True)
+    if scalar_zp:
+        c.zp, c.zp_scalar = np.array([119], np.uint8), True
+    w_kn, s_kn, z_kn = datagen.to_input_major(c)
+    a = fc.CompressedWeights.from_case(dev, c)
+    b = fc.CompressedWeights(dev, w_kn, s_kn, z_kn, c.bias, N=N, K=K, group_size=G, w_type=wt, zp_type=zt,
+                             zp_scalar=c.zp_scalar, input_major=True)
+    ref = oracle_y(oracle, c)
+    try:
+        assert np.array_equal(a.export_blob(), b.export_blob())
+        for M in (1, 5, 33, 70):
+            ya, yb = req.infer(a, c.x[:M]), req.infer(b, c.x[:M])
+            assert np.array_equal(ya.view(np.uint16), yb.view(np.uint16)), M
+            check_parity(oracle, yb, ref[:M], K, f"M={M} {req.last_kernel()}", output_rounding_slack=True)
+    finally:
+        a.close()
+        b.close()

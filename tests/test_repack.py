@@ -107,3 +107,33 @@ def test_half_magic_numbers_are_exact():
     by = (b | 0x6400).view(np.float16)
     for zp in (0, 100, 156, 255, 383):
         assert np.array_equal((by - np.float16(1024 + zp)).astype(np.float32), b.astype(np.float32) - zp)
+
+
+@pytest.mark.parametrize("wt_,zt_,N,K,G", [s for s in SHAPES if s[2] * s[3] <= 1 << 20] + [("u4", "u4", 48, 128, 128)])
+def test_input_major_constants_give_the_same_tiles(wt_, zt_, N, K, G):
+    """OVFCC_W_INPUT_MAJOR: W [K, N] and scales / zero-points [K / G, N] (a MatMul with transpose_b = false) are
+    transposed once on the host; the tiles are those of the [N, K] constants.  The transposed inputs come from
+    numpy, not from the library."""
+    c = datagen.make_case(321, 0, K, N, wt_, G, zt_)
+    plain = fc.repack_host(fc.make_desc(N, K, G, wt_, zt_), c.w, c.scale, c.zp)
+    w_kn, s_kn, z_kn = datagen.to_input_major(c)
+    if N != K:
+        assert not np.array_equal(w_kn, c.w)
+    turned = fc.repack_host(fc.make_desc(N, K, G, wt_, zt_, input_major=True), w_kn, s_kn, z_kn)
+    for a, b in zip(plain, turned):
+        assert (a is None) == (b is None)
+        if a is not None:
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+    # tiles unpack to the [N, K] order only
+    with pytest.raises(fc.OvfccError):
+        fc.unrepack_host(fc.make_desc(N, K, G, wt_, zt_, input_major=True), *plain)
+
+
+def test_input_major_nibble_transpose_known_answer():
+    """A 2 x 3 u4 matrix by hand: [[1, 2, 3], [4, 5, 6]] packs low nibble first to 21 43 65; its transpose
+    [[1, 4], [2, 5], [3, 6]] packs to 41 52 63."""
+    from openvino_amd import datagen as d
+    rows = np.array([[1, 2, 3], [4, 5, 6]], np.uint8)
+    assert d.pack_nibbles(rows).tolist() == [0x21, 0x43, 0x65]
+    assert d.pack_nibbles(rows.T).tolist() == [0x41, 0x52, 0x63]
+    assert d.unpack_nibbles(d.pack_nibbles(rows.T), 6).reshape(3, 2).T.tolist() == rows.tolist()
