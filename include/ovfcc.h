@@ -235,6 +235,23 @@ int ovfcc_gather_matmul_device(ovfcc_request* req, const ovfcc_weights* const* e
                                const void* a_dev, int a_batches, const int32_t* indices, int64_t M, int top_k,
                                void* y_dev);
 
+/* The expert block of a mixture-of-experts layer as one call: ov::op::internal::MOECompressed with
+ * Expert_type::GEMM3_SWIGLU (src/common/transformations/include/ov_ops/moe_compressed.hpp:15-75,
+ * src/core/dev_api/openvino/op/moe.hpp:17-45), the node that MoE op fusion folds three GatherMatmulCompressed, the
+ * gate activation, the Multiply by the routing weights and the ReduceSum over the selected experts into
+ * (src/common/transformations/src/transformations/common_optimizations/moe_op_fusion.cpp:55-105):
+ *     y[m, :] = sum_{j < top_k} routing[m, j] * down_e( act(gate_e(x[m, :])) * up_e(x[m, :]) ),  e = indices[m, j].
+ * gate_up[e] is expert e's gate and up projection as one node with a gated linear unit (W [2 I, H] created with
+ * OVFCC_GLU_*, or ovfcc_weights_glu of the op's w0 and w1 slices; f16 output), down[e] its down projection
+ * (w2: [H, I]); the experts agree in shape and format.  x_dev is [M, H] f16 and routing_dev [M, top_k] f16 in device
+ * memory, indices [M, top_k] int32 in host memory; y_dev receives [M, H] in the down nodes' output type.  Rows are
+ * bucketed per expert as in ovfcc_gather_matmul_device, every projection runs as one grouped launch over all
+ * experts, the intermediate activations stay f16 in device memory, and the weighted sum over a row's experts is
+ * taken in f32 in the order j = 0, 1, ....  Everything is enqueued on the request's stream. */
+int ovfcc_moe_device(ovfcc_request* req, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down,
+                     int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices_host, int64_t M,
+                     int top_k, void* y_dev);
+
 /* Benchmark twin of ovfcc_bench_layers for grouped runs: `iters` eager calls of ovfcc_fc_run_grouped_device on the
  * request's stream, bracketed by HIP events on that stream. */
 int ovfcc_bench_grouped(ovfcc_request* req, const ovfcc_group_item* items, int n_items, int warmup, int iters,

@@ -128,6 +128,54 @@ void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc:
     a->layout = w->layout;
 }
 
+// Buckets the (row, selected expert) pairs of a routed batch by expert, rows in ascending order inside a bucket:
+// the bucketing of the reference's CPU executor
+// (src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_gathermatmul_executor.cpp:492-509).  count / start receive
+// the bucket sizes and offsets.  Two maps of R = M * top_k entries each are left in the request's pinned buffer for
+// upload: first[slot] = the row of A that bucket slot `slot` reads (m, or i * M + m when A has one batch per
+// selection), and second[slot] = i * M + m, the row of a [top_k, M, .] result (inverse == false), or
+// second[m * top_k + i] = slot (inverse == true).  Waits for the previous call's upload to have left the buffer.
+int bucket_rows(ovfcc_request* r, const int32_t* indices, int64_t M, int top_k, int n_experts, int a_batches,
+                bool inverse, std::vector<int>* count, std::vector<int>* start) {
+    const int64_t R = M * top_k;
+    count->assign(n_experts, 0);
+    start->assign(n_experts + 1, 0);
+    for (int64_t m = 0; m < M; ++m)
+        for (int i = 0; i < top_k; ++i) {
+            const int32_t e = indices[m * top_k + i];
+            if (e < 0 || e >= n_experts)
+                return fail(OVFCC_EINVAL, "an expert index is out of range");
+            ++(*count)[e];
+        }
+    for (int e = 0; e < n_experts; ++e)
+        (*start)[e + 1] = (*start)[e] + (*count)[e];
+    const size_t map_bytes = (size_t)2 * R * sizeof(int);
+    if (!r->maps_uploaded)
+        HIP_TRY(hipEventCreateWithFlags(&r->maps_uploaded, hipEventDisableTiming));
+    else
+        HIP_TRY(hipEventSynchronize(r->maps_uploaded));
+    if (map_bytes > r->h_maps_cap) {
+        if (r->h_maps)
+            HIP_TRY(hipHostFree(r->h_maps));
+        r->h_maps = nullptr, r->h_maps_cap = 0;
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->h_maps), map_bytes, hipHostMallocDefault));
+        r->h_maps_cap = map_bytes;
+    }
+    std::vector<int> at(start->begin(), start->end() - 1);
+    int* first = r->h_maps;
+    int* second = r->h_maps + R;
+    for (int64_t m = 0; m < M; ++m)
+        for (int i = 0; i < top_k; ++i) {
+            const int slot = at[indices[m * top_k + i]]++;
+            first[slot] = (int)(a_batches == 1 ? m : (int64_t)i * M + m);
+            if (inverse)
+                second[m * top_k + i] = slot;
+            else
+                second[slot] = (int)((int64_t)i * M + m);
+        }
+    return OVFCC_OK;
+}
+
 void record(ovfcc_request* r, const ovfcc::LaunchPlan& p) {
     ovfcc_kernel_info& i = r->last;
     std::memset(&i, 0, sizeof(i));
@@ -911,48 +959,19 @@ int ovfcc_gather_matmul_device(ovfcc_request* r, const ovfcc_weights* const* exp
         return fail(OVFCC_EUNSUPPORTED, "rows of A and Y must be multiples of 16 bytes");
     HIP_TRY(hipSetDevice(r->ctx->device));
 
-    // rows of each expert, in row order: the bucketing of the reference's CPU executor
-    // (src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_gathermatmul_executor.cpp:492-509)
     const int64_t R = M * top_k;
-    std::vector<int> count(n_experts, 0), start(n_experts + 1, 0);
-    for (int64_t m = 0; m < M; ++m)
-        for (int i = 0; i < top_k; ++i) {
-            const int32_t e = indices[m * top_k + i];
-            if (e < 0 || e >= n_experts)
-                return fail(OVFCC_EINVAL, "an expert index is out of range");
-            ++count[e];
-        }
-    for (int e = 0; e < n_experts; ++e)
-        start[e + 1] = start[e] + count[e];
-    // the maps go through pinned host memory owned by the request; the previous call's upload must have left it
+    std::vector<int> count, start;
+    int rc = bucket_rows(r, indices, M, top_k, n_experts, a_batches, false, &count, &start);
+    if (rc)
+        return rc;
     const size_t map_bytes = (size_t)2 * R * sizeof(int);
-    if (!r->maps_uploaded)
-        HIP_TRY(hipEventCreateWithFlags(&r->maps_uploaded, hipEventDisableTiming));
-    else
-        HIP_TRY(hipEventSynchronize(r->maps_uploaded));
-    if (map_bytes > r->h_maps_cap) {
-        if (r->h_maps)
-            HIP_TRY(hipHostFree(r->h_maps));
-        r->h_maps = nullptr, r->h_maps_cap = 0;
-        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->h_maps), map_bytes, hipHostMallocDefault));
-        r->h_maps_cap = map_bytes;
-    }
-    std::vector<int> at(start.begin(), start.end() - 1);
-    int* src_row = r->h_maps;
-    int* dst_row = r->h_maps + R;
-    for (int64_t m = 0; m < M; ++m)
-        for (int i = 0; i < top_k; ++i) {
-            const int slot = at[indices[m * top_k + i]]++;
-            src_row[slot] = (int)(a_batches == 1 ? m : (int64_t)i * M + m);
-            dst_row[slot] = (int)((int64_t)i * M + m);
-        }
 
     // one scratch allocation: gathered rows | results | row maps
     const size_t x_bytes = (size_t)R * K * 2, y_bytes = (size_t)R * N_out * out_bytes;
     const size_t x_off = 0, y_off = (x_bytes + 255) & ~(size_t)255, m_off = (y_off + y_bytes + 255) & ~(size_t)255;
     if (m_off + map_bytes > r->gather_cap)
         HIP_TRY(hipStreamSynchronize(r->stream));
-    int rc = grow(&r->d_gather, &r->gather_cap, m_off + map_bytes);
+    rc = grow(&r->d_gather, &r->gather_cap, m_off + map_bytes);
     if (rc)
         return rc;
     char* base = static_cast<char*>(r->d_gather);
@@ -973,6 +992,86 @@ int ovfcc_gather_matmul_device(ovfcc_request* r, const ovfcc_weights* const* exp
     e1 = ovfcc::launch_rows(y_dev, base + y_off, nullptr, d_maps + R, (int)R, (int)(N_out * out_bytes), r->stream);
     if (e1)
         return hip_fail((hipError_t)e1, "row scatter launch");
+    return OVFCC_OK;
+}
+
+int ovfcc_moe_device(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down,
+                     int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices, int64_t M,
+                     int top_k, void* y_dev) {
+    if (!r || !gate_up || !down || n_experts <= 0 || !indices || M < 0 || top_k <= 0)
+        return fail(OVFCC_EINVAL, "bad mixture-of-experts arguments");
+    if (top_k > n_experts)
+        return fail(OVFCC_EINVAL, "more selected experts per row than experts");
+    if (M == 0)
+        return OVFCC_OK;
+    if (!x_dev || !routing_dev || !y_dev)
+        return fail(OVFCC_EINVAL, "hidden states, routing weights or output is null");
+    if (M * top_k > ((int64_t)1 << 24))
+        return fail(OVFCC_EUNSUPPORTED, "M * top_k is limited to 2^24");
+    const ovfcc_weights *g0 = gate_up[0], *d0 = down[0];
+    for (int e = 0; e < n_experts; ++e) {
+        const ovfcc_weights *g = gate_up[e], *d = down[e];
+        if (!g || !d || g->ctx != r->ctx || d->ctx != r->ctx)
+            return fail(OVFCC_EINVAL, "an expert's weights are null or belong to another context");
+        if (std::memcmp(&g->desc, &g0->desc, sizeof(ovfcc_fc_desc)) != 0 ||
+            std::memcmp(&d->desc, &d0->desc, sizeof(ovfcc_fc_desc)) != 0 ||
+            (g->d_bias != nullptr) != (g0->d_bias != nullptr) || (d->d_bias != nullptr) != (d0->d_bias != nullptr))
+            return fail(OVFCC_EUNSUPPORTED, "experts differ in shape, types, bias or output type");
+    }
+    // gate/up: [2 I, H] with a gated linear unit, f16 out (it feeds the down projection); down: [H, I], no unit
+    const int64_t H = g0->desc.K, I = out_channels(g0);
+    if (!g0->layout.glu || g0->desc.out_type != OVFCC_F16)
+        return fail(OVFCC_EINVAL, "the gate/up nodes must carry a gated linear unit and write f16");
+    if (d0->layout.glu || d0->desc.K != I || d0->desc.N != H)
+        return fail(OVFCC_EINVAL, "the down nodes must map the gate/up output back to the hidden size, without a unit");
+    const int d_f32 = d0->desc.out_type == OVFCC_F32 ? 1 : 0;
+    if ((H * 2) % 16 != 0 || (I * 2) % 16 != 0)
+        return fail(OVFCC_EUNSUPPORTED, "hidden and intermediate rows must be multiples of 16 bytes");
+    HIP_TRY(hipSetDevice(r->ctx->device));
+
+    const int64_t R = M * top_k;
+    std::vector<int> count, start;
+    int rc = bucket_rows(r, indices, M, top_k, n_experts, 1, true, &count, &start);
+    if (rc)
+        return rc;
+    const size_t map_bytes = (size_t)2 * R * sizeof(int);
+
+    // one scratch allocation: gathered rows | gate/up results | down results | row maps
+    auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t x_bytes = (size_t)R * H * 2, h_bytes = (size_t)R * I * 2, d_bytes = (size_t)R * H * (d_f32 ? 4 : 2);
+    const size_t h_off = up256(x_bytes), d_off = up256(h_off + h_bytes), m_off = up256(d_off + d_bytes);
+    if (m_off + map_bytes > r->gather_cap)
+        HIP_TRY(hipStreamSynchronize(r->stream));
+    rc = grow(&r->d_gather, &r->gather_cap, m_off + map_bytes);
+    if (rc)
+        return rc;
+    char* base = static_cast<char*>(r->d_gather);
+    int* d_maps = reinterpret_cast<int*>(base + m_off);
+    HIP_TRY(hipMemcpyAsync(d_maps, r->h_maps, map_bytes, hipMemcpyHostToDevice, r->stream));
+    HIP_TRY(hipEventRecord(r->maps_uploaded, r->stream));
+    int e1 = ovfcc::launch_rows(base, x_dev, d_maps, nullptr, (int)R, (int)(H * 2), r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "row gather launch");
+    std::vector<ovfcc_group_item> items;
+    for (int e = 0; e < n_experts; ++e)
+        if (count[e])
+            items.push_back({gate_up[e], base + (size_t)start[e] * H * 2, base + h_off + (size_t)start[e] * I * 2,
+                             (int64_t)count[e]});
+    rc = ovfcc_fc_run_grouped_device(r, items.data(), (int)items.size());
+    if (rc)
+        return rc;
+    items.clear();
+    for (int e = 0; e < n_experts; ++e)
+        if (count[e])
+            items.push_back({down[e], base + h_off + (size_t)start[e] * I * 2,
+                             base + d_off + (size_t)start[e] * H * (d_f32 ? 4 : 2), (int64_t)count[e]});
+    rc = ovfcc_fc_run_grouped_device(r, items.data(), (int)items.size());
+    if (rc)
+        return rc;
+    e1 = ovfcc::launch_moe_combine(y_dev, base + d_off, routing_dev, d_maps + R, (int)M, top_k, (int)H, d_f32, d_f32,
+                                   r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "expert combine launch");
     return OVFCC_OK;
 }
 

@@ -124,6 +124,58 @@ int launch_rows(void* dst, const void* src, const int* src_row, const int* dst_r
     return (int)hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------------
+// Last step of a mixture-of-experts block: y[m, :] = sum_j routing[m, j] * d[pos[m, j], :] over the top_k experts
+// of row m, in the order j = 0, 1, ... (the Multiply by the routing weights and the ReduceSum over the expert
+// axis that MOE fuses, src/common/transformations/src/transformations/common_optimizations/moe_op_fusion.cpp:97-104).
+// d holds one result row per (row, expert) pair in bucket order, pos maps (m, j) to it.  f32 sums; one workgroup
+// per row, four channels per thread and step.
+// ------------------------------------------------------------------------------------------------
+template <bool IN_F32>
+__global__ __launch_bounds__(256) void fcc_moe_combine_kernel(void* __restrict__ y, const void* __restrict__ d,
+                                                              const half_t* __restrict__ routing,
+                                                              const int* __restrict__ pos, int top_k, int H,
+                                                              int out_f32) {
+    const int m = blockIdx.x;
+    for (int c = 4 * threadIdx.x; c < H; c += 4 * blockDim.x) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < top_k; ++j) {
+            const float wgt = (float)routing[(size_t)m * top_k + j];
+            const size_t row = (size_t)pos[(size_t)m * top_k + j] * H + c;
+            if constexpr (IN_F32) {
+                const float4_t v = *reinterpret_cast<const float4_t*>(static_cast<const float*>(d) + row);
+                acc[0] += wgt * v.x, acc[1] += wgt * v.y, acc[2] += wgt * v.z, acc[3] += wgt * v.w;
+            } else {
+                const half4_t v = *reinterpret_cast<const half4_t*>(static_cast<const half_t*>(d) + row);
+                acc[0] += wgt * (float)v[0], acc[1] += wgt * (float)v[1], acc[2] += wgt * (float)v[2],
+                    acc[3] += wgt * (float)v[3];
+            }
+        }
+        if (out_f32)
+            *reinterpret_cast<float4_t*>(static_cast<float*>(y) + (size_t)m * H + c) =
+                float4_t{acc[0], acc[1], acc[2], acc[3]};
+        else
+            *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * H + c) =
+                half4_t{(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
+    }
+}
+
+int launch_moe_combine(void* y, const void* d, const void* routing, const int* pos, int rows, int top_k, int H,
+                       int d_f32, int out_f32, void* stream) {
+    if (rows <= 0)
+        return 0;
+    if (top_k <= 0 || H <= 0 || (H & 3))
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (d_f32)
+        hipLaunchKernelGGL(fcc_moe_combine_kernel<true>, dim3((unsigned)rows), dim3(256), 0, s, y, d,
+                           (const half_t*)routing, pos, top_k, H, out_f32);
+    else
+        hipLaunchKernelGGL(fcc_moe_combine_kernel<false>, dim3((unsigned)rows), dim3(256), 0, s, y, d,
+                           (const half_t*)routing, pos, top_k, H, out_f32);
+    return (int)hipGetLastError();
+}
+
 int launch_touch(const void* src, size_t bytes, void* stream) {
     const size_t n16 = bytes / 16;
     const unsigned blocks = (unsigned)((n16 + 256 * 4 - 1) / (256 * 4));  // four loads per thread

@@ -173,6 +173,9 @@ int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
 int launch_rows(void* dst, const void* src, const int* src_row, const int* dst_row, int rows, int row_bytes,
                 void* stream);
 int launch_touch(const void* src, size_t bytes, void* stream);
+// y[m, :] = sum_j routing[m, j] * d[pos[m * top_k + j], :], rows of H (a multiple of 4) channels; d f16 or f32
+int launch_moe_combine(void* y, const void* d, const void* routing, const int* pos, int rows, int top_k, int H,
+                       int d_f32, int out_f32, void* stream);
 
 constexpr int kDecodeMaxRows = 48;                       // rows one decode-family launch covers
 constexpr int kPrefillGroupRows = 128;                   // rows per slice of a grouped prefill launch (one tile)

@@ -294,6 +294,46 @@ class InferRequest:
             dev.free(a_ptr)
             dev.free(y_ptr)
 
+    def moe_device(self, gate_up: Sequence[CompressedWeights], down: Sequence[CompressedWeights], x_ptr: int,
+                   routing_ptr: int, indices: np.ndarray, y_ptr: int) -> None:
+        """MOECompressed (three projections per expert, gated linear unit) on device buffers: hidden states
+        [M, H] f16 at x_ptr, routing weights [M, top_k] f16 at routing_ptr, indices int32 [M, top_k] on the host,
+        Y [M, H] at y_ptr."""
+        idx = np.ascontiguousarray(indices, dtype=np.int32)
+        M, top_k = idx.shape
+        g = (ctypes.c_void_p * len(gate_up))(*[w.handle for w in gate_up])
+        d = (ctypes.c_void_p * len(down))(*[w.handle for w in down])
+        check(self.device.lib.ovfcc_moe_device(self.handle, g, d, len(gate_up), ctypes.c_void_p(x_ptr),
+                                               ctypes.c_void_p(routing_ptr),
+                                               idx.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), M, top_k,
+                                               ctypes.c_void_p(y_ptr)))
+
+    def moe(self, gate_up: Sequence[CompressedWeights], down: Sequence[CompressedWeights], x: np.ndarray,
+            routing: np.ndarray, indices: np.ndarray) -> np.ndarray:
+        """Host convenience: x float16 [M, H], routing float16 [M, top_k], indices [M, top_k] -> Y [M, H]."""
+        x = np.ascontiguousarray(x, dtype=np.float16)
+        routing = np.ascontiguousarray(routing, dtype=np.float16)
+        idx = np.ascontiguousarray(indices, dtype=np.int32)
+        M, top_k = idx.shape
+        H = down[0].N
+        if x.shape != (M, gate_up[0].K) or routing.shape != (M, top_k) or len(gate_up) != len(down):
+            raise OvfccError(_lib.EINVAL, f"x {x.shape}, routing {routing.shape}, indices {idx.shape} do not fit")
+        dt = np.float32 if down[0].desc.out_type == _lib.F32 else np.float16
+        if M == 0:
+            return np.empty((0, H), dt)
+        dev = self.device
+        x_ptr, r_ptr, y_ptr = dev.malloc(x.nbytes), dev.malloc(max(routing.nbytes, 16)), dev.malloc(M * H * np.dtype(dt).itemsize)
+        try:
+            dev.upload(x_ptr, x)
+            dev.upload(r_ptr, routing)
+            self.moe_device(gate_up, down, x_ptr, r_ptr, idx, y_ptr)
+            self.sync()
+            return dev.download(y_ptr, (M, H), dt)
+        finally:
+            dev.free(x_ptr)
+            dev.free(r_ptr)
+            dev.free(y_ptr)
+
     def bench_grouped(self, items: Sequence[tuple], warmup: int, iters: int) -> float:
         """Milliseconds for `iters` grouped runs, HIP events on the launching stream."""
         arr = self._group_items(items)

@@ -214,6 +214,33 @@ def glu(y, glu_type, gate_second=False) -> np.ndarray:
     return out
 
 
+def moe_reference(x, routing, indices, gate_up, down, glu_type) -> np.ndarray:
+    """Mixture-of-experts block with three projections per expert (ov::op::internal::MOE, GEMM3_SWIGLU), as the
+    graph that MoE op fusion folds computes it (moe_op_fusion.cpp:55-105):
+
+        y[m] = sum_j routing[m, j] * down_e(act(gate_e(x[m])) * up_e(x[m])),   e = indices[m, j]
+
+    x float16 [M, H], routing [M, top_k], indices int [M, top_k].  gate_up[e] and down[e] are the keyword
+    arguments of fc_reference for expert e's concatenated gate/up node ([2 I, H], gate rows first) and its down
+    node ([H, I]).  Composed of fc_reference and glu; the activations between the two projections are rounded to
+    float16 (they are a float16 tensor in the graph), the sum over a row's experts runs in float64.  float32 [M, H]."""
+    x = np.ascontiguousarray(x, dtype=np.float16)
+    routing = np.asarray(routing, dtype=np.float64)
+    indices = np.asarray(indices)
+    M, top_k = indices.shape
+    H = down[0]["N"]
+    y = np.zeros((M, H), np.float64)
+    for e in range(len(gate_up)):
+        for j in range(top_k):
+            rows = np.nonzero(indices[:, j] == e)[0]
+            if not rows.size:
+                continue
+            h = glu(fc_reference(x[rows], **gate_up[e]), glu_type).astype(np.float16)
+            d = fc_reference(h, **down[e])
+            y[rows] += routing[rows, j, None] * d.astype(np.float64)
+    return y.astype(np.float32)
+
+
 def dynquant_rows(x):
     """C oracle: per-token symmetric int8 quantisation of x [M, K] float16 -> (q int8 [M, K], inv_scale float32 [M],
     qsum int32 [M])."""
