@@ -35,6 +35,8 @@ struct ovfcc_request {
     void* d_x = nullptr;
     void* d_y = nullptr;
     size_t x_cap = 0, y_cap = 0;
+    void* h_stage = nullptr;   // pinned host memory that small host transfers of ovfcc_fc_run go through: x | y
+    size_t h_stage_cap = 0;
     float* workspace = nullptr;
     size_t ws_cap = 0;
     unsigned* counters = nullptr;
@@ -54,6 +56,8 @@ struct ovfcc_request {
 namespace {
 
 using ovfcc::fail;
+
+constexpr size_t kHostStageMax = (size_t)1 << 20;  // host transfers up to this size (x and y together) are staged
 
 int hip_fail(hipError_t e, const char* what) {
     return fail(e == hipErrorOutOfMemory ? OVFCC_ENOMEM : OVFCC_EDEVICE,
@@ -764,6 +768,7 @@ void ovfcc_request_destroy(ovfcc_request* r) {
     if (r->d_gather) (void)hipFree(r->d_gather);
     if (r->d_quant) (void)hipFree(r->d_quant);
     if (r->h_maps) (void)hipHostFree(r->h_maps);
+    if (r->h_stage) (void)hipHostFree(r->h_stage);
     if (r->maps_uploaded) (void)hipEventDestroy(r->maps_uploaded);
     delete r;
 }
@@ -1102,12 +1107,33 @@ int ovfcc_fc_run(ovfcc_request* r, const ovfcc_weights* w, const void* x_host, v
     rc = grow(&r->d_y, &r->y_cap, yb);
     if (rc)
         return rc;
-    HIP_TRY(hipMemcpyAsync(r->d_x, x_host, xb, hipMemcpyHostToDevice, r->stream));
-    rc = ovfcc_fc_run_device(r, w, r->d_x, r->d_y, M);
+    // Small transfers go through pinned memory of the request: a copy from or to pageable memory makes the runtime
+    // stage, pin and synchronise per call, which at decode sizes costs more than the copy and the kernel together.
+    // (The request is idle here: the previous call ended with a synchronisation.)  Large ones go directly.
+    const size_t y_off = (xb + 255) & ~(size_t)255;
+    const bool staged = y_off + yb <= kHostStageMax;
+    if (staged && y_off + yb > r->h_stage_cap) {
+        if (r->h_stage)
+            HIP_TRY(hipHostFree(r->h_stage));
+        r->h_stage = nullptr, r->h_stage_cap = 0;
+        const size_t cap = std::max<size_t>(y_off + yb, 64 << 10);
+        HIP_TRY(hipHostMalloc(&r->h_stage, cap, hipHostMallocDefault));
+        r->h_stage_cap = cap;
+    }
+    char* hs = static_cast<char*>(r->h_stage);
+    if (staged)
+        std::memcpy(hs, x_host, xb);
+    HIP_TRY(hipMemcpyAsync(r->d_x, staged ? hs : x_host, xb, hipMemcpyHostToDevice, r->stream));
+    // ... and the kernel writes its (write-once) output straight into the pinned memory, which is mapped into the
+    // device's address space: one copy operation less.  The activations are copied: every workgroup reads them.
+    rc = ovfcc_fc_run_device(r, w, r->d_x, staged ? static_cast<void*>(hs + y_off) : r->d_y, M);
     if (rc)
         return rc;
-    HIP_TRY(hipMemcpyAsync(y_host, r->d_y, yb, hipMemcpyDeviceToHost, r->stream));
+    if (!staged)
+        HIP_TRY(hipMemcpyAsync(y_host, r->d_y, yb, hipMemcpyDeviceToHost, r->stream));
     HIP_TRY(hipStreamSynchronize(r->stream));
+    if (staged)
+        std::memcpy(y_host, hs + y_off, yb);
     return OVFCC_OK;
 }
 
