@@ -281,6 +281,7 @@ int ovfcc_device_malloc(ovfcc_ctx* ctx, size_t bytes, void** out);
 int ovfcc_device_free(ovfcc_ctx* ctx, void* ptr);
 int ovfcc_memcpy_h2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
 int ovfcc_memcpy_d2h(ovfcc_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
+int ovfcc_memcpy_d2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes);
 /* Plain device-to-device copy kernel of `bytes` (multiple of 16) repeated `iters` times, timed with
  * HIP events: the yardstick the HBM counters and the achieved-bandwidth figures are scaled by. */
 int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, int iters, float* elapsed_ms);

@@ -1255,6 +1255,14 @@ int ovfcc_memcpy_d2h(ovfcc_ctx* ctx, void* dst_host, const void* src_dev, size_t
     return OVFCC_OK;
 }
 
+int ovfcc_memcpy_d2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes) {
+    if (!ctx || ((!dst_dev || !src_dev) && bytes))
+        return fail(OVFCC_EINVAL, "null argument");
+    if (bytes)
+        HIP_TRY(hipMemcpy(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice));
+    return OVFCC_OK;
+}
+
 int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, int iters, float* elapsed_ms) {
     if (!ctx || !dst_dev || !src_dev || !elapsed_ms || iters <= 0 || bytes % 16)
         return fail(OVFCC_EINVAL, "bad copy benchmark arguments");

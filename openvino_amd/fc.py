@@ -70,6 +70,10 @@ class Device:
         check(self.lib.ovfcc_memcpy_d2h(self.handle, _vp(out), ctypes.c_void_p(ptr), out.nbytes))
         return out
 
+    def copy(self, dst_ptr: int, src_ptr: int, nbytes: int) -> None:
+        """Device-to-device copy (blocking)."""
+        check(self.lib.ovfcc_memcpy_d2d(self.handle, ctypes.c_void_p(dst_ptr), ctypes.c_void_p(src_ptr), nbytes))
+
     def copy_bandwidth(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
         """GB/s (read + write) of the plain copy kernel."""
         src, dst = self.malloc(nbytes), self.malloc(nbytes)

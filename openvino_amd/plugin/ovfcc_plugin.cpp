@@ -320,11 +320,8 @@ public:
                         "MI355X: copy_from needs a dense tensor of type ", m_type);
         set_shape(src->get_shape());
         if (auto remote = std::dynamic_pointer_cast<const RemoteTensor>(src)) {
-            // device to device through the host would be wasteful; the library's copy kernel does it in place
-            float ms = 0.f;
-            const size_t bytes = (get_byte_size() + 15) / 16 * 16;  // allocations are padded to 16 bytes
-            if (bytes && ovfcc_bench_copy(m_ctx, m_ptr, remote->device_ptr(), bytes, 1, &ms) != OVFCC_OK)
-                throw_last("device copy");
+            if (get_byte_size() && ovfcc_memcpy_d2d(m_ctx, m_ptr, remote->device_ptr(), get_byte_size()) != OVFCC_OK)
+                throw_last("memcpy_d2d");
         } else if (get_byte_size() && ovfcc_memcpy_h2d(m_ctx, m_ptr, src->data(), get_byte_size()) != OVFCC_OK) {
             throw_last("memcpy_h2d");
         }

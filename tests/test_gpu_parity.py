@@ -695,3 +695,18 @@ def test_input_major_constants(oracle, dev, req, wt, zt, N, K, G, scalar_zp):
     finally:
         a.close()
         b.close()
+
+
+def test_device_memory_helpers(dev):
+    """malloc / upload / device-to-device copy / download round trip, odd sizes included."""
+    say("device memory helpers")
+    for n in (1, 17, 4096, (1 << 20) + 3):
+        a = np.random.default_rng(n).integers(0, 256, size=n, dtype=np.uint8)
+        p, q = dev.malloc(n), dev.malloc(n)
+        try:
+            dev.upload(p, a)
+            dev.copy(q, p, n)
+            assert np.array_equal(dev.download(q, (n,), np.uint8), a)
+        finally:
+            dev.free(p)
+            dev.free(q)
