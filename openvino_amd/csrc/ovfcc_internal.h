@@ -119,6 +119,7 @@ struct LaunchPlan {
     bool x_in_lds = false;      // decode kernel: activations staged in LDS
     bool direct = false;        // prefill family: the kernels that feed weights from registers
     bool async_dma = false;     // ... and of those the one whose operands all travel by direct-to-LDS loads
+    bool big = false;           // prefill family: the 4-bit kernel with 256 x 256 tiles (whole tiles, no split-K)
     bool batch = false;         // decode family: the small-batch kernel (waves own channel tiles)
     int tiles_x = 0, tiles_y = 0;  // async prefill kernel: the tile grid; its launch is 1-D
     int full_tiles = 0;         // ... of which this many run unsplit (the rest in split_k parts each)
@@ -162,6 +163,7 @@ int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_prefill_big(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 // Per-row int8 quantisation of x [M, K] f16 (K % 128 == 0): xq [M, K] in the weight tiles' input order, one
 // inverse scale and one sum of quantised values per row.
 int launch_dynquant(const void* x, void* xq, float* inv_scale, int* qsum, int64_t M, int64_t K, void* stream);

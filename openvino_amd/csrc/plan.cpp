@@ -256,6 +256,24 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             p.counter_count = split > 1 ? (size_t)(tiles - full) : 0;
         }
         p.block = wide ? 512 : 256;
+        // 256 x 256 tiles (four waves with 512 registers each) where whole tiles of that size still give every
+        // compute unit one: every unpacked weight then meets twice the rows.  OVFCC_PREFILL_BIG = 0 | 1 overrides
+        // (1: whenever the kernel can run the node).
+        if (p.async_dma && p.split_k == 1 && p.tile_m == kPrefillTileM && L.groups_per_kblock == 1 && force_split <= 0) {
+            const int64_t big_tiles = (a.N / kPrefillWideN) * ((a.M + 255) / 256);
+            const int big_env = env_int("OVFCC_PREFILL_BIG", 0);
+            if (big_env != 0 && (big_env > 0 || big_tiles >= n_cus)) {
+                p.big = true;
+                p.tile_m = 256;
+                p.tiles_y = (int)((a.M + 255) / 256);
+                p.full_tiles = p.tiles_x * p.tiles_y;
+                p.grid[0] = (unsigned)p.full_tiles;
+                p.block = 256;
+            }
+        }
+        if (p.big)
+            p.name = "fcc_prefill_big_w4";
+        else
         p.name = L.bits == 4 ? (p.async_dma ? "fcc_prefill_async_w4" : p.direct ? "fcc_prefill_direct_w4" : wide ? "fcc_prefill_wide_w4" : "fcc_prefill_w4")
                              : (p.direct ? "fcc_prefill_direct_w8" : wide ? "fcc_prefill_wide_w8" : "fcc_prefill_w8");
     }
@@ -272,6 +290,8 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     case OVFCC_KERNEL_DECODE:
         return p.batch ? launch_batch(a, p, stream) : launch_decode(a, p, stream);
     default:
+        if (p.big)
+            return launch_prefill_big(a, p, stream);
         if (p.async_dma)
             return launch_prefill_async(a, p, stream);
         if (p.direct)

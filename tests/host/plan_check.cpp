@@ -18,6 +18,7 @@ int launch_prefill(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_wide(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_direct(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_async(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_prefill_big(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 }  // namespace ovfcc
 
 static int g_failures = 0;
