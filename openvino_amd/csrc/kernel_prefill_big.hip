@@ -167,7 +167,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // weights into the other set, a few micro-operations after every MFMA: dword ja of `sa` during step 0 (into wb),
     // dword jb of `sb` during step 1 (into wa).  The activation operands run PB_XQ - 1 row tiles ahead of the
     // MFMAs, across the boundary between the steps; mem(i) adds the memory instructions of slot i (0 .. 127).
-    constexpr int PB_XQ = 4;
+    constexpr int PB_XQ = 6;
     auto half = [&](int stage, Frag8 (&wa)[4], Frag8 (&wb)[4], const WSlot& sa, int ja, WSlot& sb, int jb,
                     auto&& mem) {
         // operand of row tile t and step js: row 16 t + col, chunk (4 js + kq) ^ ((col >> 1) & 7)

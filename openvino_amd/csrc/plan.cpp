@@ -256,13 +256,17 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             p.counter_count = split > 1 ? (size_t)(tiles - full) : 0;
         }
         p.block = wide ? 512 : 256;
-        // 256 x 256 tiles (four waves with 512 registers each) where whole tiles of that size still give every
-        // compute unit one: every unpacked weight then meets twice the rows.  OVFCC_PREFILL_BIG = 0 | 1 overrides
-        // (1: whenever the kernel can run the node).
+        // 256 x 256 tiles (four waves with 512 registers each), where every unpacked weight meets twice the rows:
+        // measured, such a tile costs 1.7 to 1.8 times a 128 x 256 tile.  It is whole tiles only, so it pays where
+        // its rounds of tiles over the compute units, at that price, are no more than the rounds of the smaller
+        // tiles: 256, 448, 512, 896, 1792 tiles yes; 128 or 300 no.  OVFCC_PREFILL_BIG = 0 | 1 overrides (1: whenever
+        // the kernel can run the node).
         if (p.async_dma && p.split_k == 1 && p.tile_m == kPrefillTileM && L.groups_per_kblock == 1 && force_split <= 0) {
             const int64_t big_tiles = (a.N / kPrefillWideN) * ((a.M + 255) / 256);
-            const int big_env = env_int("OVFCC_PREFILL_BIG", 0);
-            if (big_env != 0 && (big_env > 0 || big_tiles >= n_cus)) {
+            const int64_t big_rounds = (big_tiles + n_cus - 1) / n_cus;
+            const int64_t small_rounds = ((int64_t)p.tiles_x * p.tiles_y + n_cus - 1) / n_cus;
+            const int big_env = env_int("OVFCC_PREFILL_BIG", -1);
+            if (big_env > 0 || (big_env < 0 && big_tiles >= n_cus && big_rounds * 100 <= small_rounds * 58)) {
                 p.big = true;
                 p.tile_m = 256;
                 p.tiles_y = (int)((a.M + 255) / 256);

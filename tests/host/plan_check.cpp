@@ -115,7 +115,12 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     CHECK(L.groups_per_kblock == 1 || (L.bits == 4 && (p.async_dma || p.tile_n == 128)), "%s gpb=%d", what, L.groups_per_kblock);
     if (p.direct) {
         const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
-        CHECK(p.tile_m == 128 || (p.async_dma && p.tile_m == 64), "%s tile_m=%d", what, p.tile_m);
+        CHECK(p.tile_m == 128 || (p.async_dma && p.tile_m == 64) || (p.big && p.tile_m == 256), "%s tile_m=%d", what, p.tile_m);
+        // 256 x 256 tiles: 4-bit nodes with one group per k-block at most, whole tiles, a tile for every compute unit
+        if (p.big)
+            CHECK(p.async_dma && L.bits == 4 && L.groups_per_kblock == 1 && p.split_k == 1 && p.block == 256 &&
+                      p.tiles_x == (int)(d.N / 256) && p.tiles_y == (int)((M + 255) / 256) &&
+                      p.full_tiles == p.tiles_x * p.tiles_y && p.full_tiles >= n_cus, "%s big", what);
         CHECK(d.N % 256 == 0 && p.tiles_x == d.N / 256 && p.tiles_y == (M + p.tile_m - 1) / p.tile_m, "%s", what);
         CHECK(p.full_tiles >= 0 && p.full_tiles <= tiles && (p.split_k > 1 || p.full_tiles == tiles), "%s full=%d", what, p.full_tiles);
         CHECK(p.grid[0] == (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) && p.grid[1] == 1 && p.grid[2] == 1, "%s", what);
