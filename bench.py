@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/ (counters cannot be
 # read from inside this process): FETCH_SIZE x 2.000 (its reading for a copy kernel of known size) + WRITE_SIZE.
 TRAFFIC_DECODE_M1 = {"qo": 8869888, "kv": 2375680, "gate_up": 30526464, "down": 30669824}
-TRAFFIC_PREFILL_M2048 = {"qo": 85495808, "kv": 72139776, "gate_up": 347048960, "down": 255927296}
+TRAFFIC_PREFILL_M2048 = {"qo": 85494784, "kv": 72139776, "gate_up": 328939520, "down": 255920128}
 
 
 def log(*a):
@@ -495,12 +495,12 @@ def main() -> int:
         out["prefill"] = {
             "M": Mp, "TFLOPs": round(tflops, 2), "pct_of_mfma_peak": round(100 * tflops / MFMA_F16_PEAK_TFLOPS, 2),
             "ms_per_block": round(pms / psteps, 4), "steps": psteps, "per_shape": pshape,
-            "roofline": {"bound": "mfma", "kernel": "fcc_prefill_async_w4", "achieved": round(tflops, 2),
+            "roofline": {"bound": "mfma", "kernel": "fcc_prefill_big_w4 (gate, up) + fcc_prefill_async_w4", "achieved": round(tflops, 2),
                          "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
                          "traffic": (sum(TRAFFIC_PREFILL_M2048[n] for n in datagen.LLAMA3_8B_BLOCK)
                                      // len(datagen.LLAMA3_8B_BLOCK) if Mp == 2048 else None),
-                         "traffic_source": "profiles/fcc_prefill_async_w4_llama3_8b_m2048.md"},
+                         "traffic_source": "profiles/fcc_prefill_w4_llama3_8b_m2048.md"},
         }
 
     # ---- CPU baseline: the oracle on the host cores, bounded sample ----
