@@ -110,7 +110,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
     };
     constexpr int kWLoads = 4 + (PRESCALE ? 4 : 0) + (ZP_TABLE ? 4 : 0);  // vector-memory loads of load_w
-    constexpr int kWaitTop = 2 * PB_AL + kWLoads;  // see the wait at the top of a half
 
     // ---- unpack, one micro-operation at a time: dword j of tile r of slot s -> f (the 128 x 256 kernel's scheme) ----
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // per dword
@@ -167,22 +166,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // weights into the other set, a few micro-operations after every MFMA: dword ja of `sa` during step 0 (into wb),
     // dword jb of `sb` during step 1 (into wa).  The activation operands run PB_XQ - 1 row tiles ahead of the
     // MFMAs, across the boundary between the steps; mem(i) adds the memory instructions of slot i (0 .. 127).
-    constexpr int PB_XQ = 6;
+    // Ring of activation operands, eight deep (a divisor of the 32 operands of a half, so ring positions repeat from
+    // half to half): operand n of a half is row tile n & 15 of step n >> 4.  The ring runs seven operands ahead of
+    // the MFMAs and carries on into the next half's stage, so no half starts with an empty ring.
+    constexpr int PB_XQ = 8;
+    constexpr int PB_SYNC_SLOT = 100;  // the first slot whose ring read belongs to the next half
+    half8_t xq[PB_XQ];
+    const int x_sw = (col >> 1) & 7;
+    // operand n of the half in `stage`: row 16 (n & 15) + col, chunk (4 (n >> 4) + kq) ^ ((col >> 1) & 7)
+    auto x_at = [&](int stage, int n) {
+        return *(lds_frag_ptr)(lds3 + stage * PB_STAGE_BYTES + ((n & 15) * 16 + col) * 128 + ((((n >> 4) * 4 + kq) ^ x_sw) << 4));
+    };
     auto half = [&](int stage, Frag8 (&wa)[4], Frag8 (&wb)[4], const WSlot& sa, int ja, WSlot& sb, int jb,
-                    auto&& mem) {
-        // operand of row tile t and step js: row 16 t + col, chunk (4 js + kq) ^ ((col >> 1) & 7)
-        const int sw = (col >> 1) & 7;
-        const lds_byte_ptr xa0 = lds3 + stage * PB_STAGE_BYTES + col * 128 + ((kq ^ sw) << 4);
-        const lds_byte_ptr xa1 = lds3 + stage * PB_STAGE_BYTES + col * 128 + (((4 + kq) ^ sw) << 4);
-        auto x_at = [&](int tt) { return *(lds_frag_ptr)((tt < 16 ? xa0 : xa1) + (tt & 15) * 16 * 128); };
-        half8_t xq[PB_XQ];
-#pragma unroll
-        for (int tt = 0; tt < PB_XQ - 1; ++tt)
-            xq[tt] = x_at(tt);
+                    auto&& sync_next, auto&& mem) {
         auto slot = [&](int i) {
             const int tt = i >> 2, r = i & 3;  // tt = 16 js + t
-            if (r == 0 && tt + PB_XQ - 1 < 32)
-                xq[(tt + PB_XQ - 1) % PB_XQ] = x_at(tt + PB_XQ - 1);
+            if (i == PB_SYNC_SLOT)
+                sync_next();  // the next half's activations are in LDS for every wave
+            if (r == 0) {
+                constexpr int ahead = PB_XQ - 1;
+                xq[(tt + ahead) % PB_XQ] = tt + ahead < 32 ? x_at(stage, tt + ahead) : x_at((stage + 1) & 3, tt + ahead - 32);
+            }
             const int t = tt & 15;
             if (i < 64) {
                 mfma_in_place(acc[r][t], wa[r].v, xq[tt % PB_XQ]);
@@ -245,6 +249,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             unpack_op(ws0, r, 0, op, wf0[r]);
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(2 * PB_AL));  // half 0 has landed
     asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < PB_XQ - 1; ++n)
+        xq[n] = x_at(0, n);
 
     // ---- main loop: two k-blocks (four halves, the four stages) per trip so that stages and weight slots are
     // static.  Halves and k-blocks past the end are loaded out of range (zeros) and add nothing. ----
@@ -252,18 +261,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int hh = 2 * kb0 + u;
-            // At the top of a half the wave needs the activations of that half.  Issued after them: the activation
-            // loads of the next two halves and, in one of those two, a k-block's weight loads.  (Half 0 was waited
-            // for above; behind half 1's loads lie two halves' activation loads only.)
-            if (kb0 == 0 && u < 2) {
-                if (u == 1)
-                    __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(2 * PB_AL));
-            } else {
-                __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(kWaitTop));
-            }
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();  // everyone's loads of this half are in; everyone is done with half hh - 1
-            asm volatile("" ::: "memory");
+            // The one barrier of a half sits where the operand ring first reaches into the next half: by then the
+            // wave needs that half's activations.  Issued after them by this wave: the rest of the activation loads
+            // of the half before this one and seven of this half's (fifteen in all) and, in one of the two halves, a
+            // k-block's weight loads (none yet in the very first half).  Past the barrier no wave reads this half's
+            // stage any more (its last operand was fetched four slots earlier, and the wave's own LDS reads are
+            // waited for here), so the loads of half hh + 4, which start in the next half, may overwrite it.
+            auto sync_next = [&]() {
+                constexpr int lds_reads_done = ~0x0F00;
+                if (u == 0)  // (later trips: this also waits for loads issued more than a half ago, long since in)
+                    __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(2 * PB_AL - 1) & lds_reads_done);
+                else
+                    __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(2 * PB_AL - 1 + kWLoads) & lds_reads_done);
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            };
             // Memory instructions between the MFMAs: the stage that half hh - 1 used takes half hh + 3 (slots 1, 17,
             // ..).  A k-block's weight slot is free once the last step that unpacks from it has run -- step 0 of its
             // second half -- so the loads of the k-block after next go out at the start of step 1 of that half.
@@ -278,13 +291,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             // steps of this half: dwords 2 (u & 1), 2 (u & 1) + 1 of the k-block's slot; unpacked meanwhile: the
             // next step's dword -- of the same slot, or dword 0 of the other slot at the end of a k-block
             if (u == 0)
-                half(0, wf0, wf1, ws0, 1, ws0, 2, mem);
+                half(0, wf0, wf1, ws0, 1, ws0, 2, sync_next, mem);
             else if (u == 1)
-                half(1, wf0, wf1, ws0, 3, ws1, 0, mem);
+                half(1, wf0, wf1, ws0, 3, ws1, 0, sync_next, mem);
             else if (u == 2)
-                half(2, wf0, wf1, ws1, 1, ws1, 2, mem);
+                half(2, wf0, wf1, ws1, 1, ws1, 2, sync_next, mem);
             else
-                half(3, wf0, wf1, ws1, 3, ws0, 0, mem);
+                half(3, wf0, wf1, ws1, 3, ws0, 0, sync_next, mem);
         }
     }
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));  // the out-of-range loads of the last trips still target LDS

@@ -260,8 +260,9 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         // measured, such a tile costs 1.7 to 1.8 times a 128 x 256 tile.  It is whole tiles only, so it pays where
         // its rounds of tiles over the compute units, at that price, are no more than the rounds of the smaller
         // tiles: 256, 448, 512, 896, 1792 tiles yes; 128 or 300 no.  OVFCC_PREFILL_BIG = 0 | 1 overrides (1: whenever
-        // the kernel can run the node).
-        if (p.async_dma && p.split_k == 1 && p.tile_m == kPrefillTileM && L.groups_per_kblock == 1 && force_split <= 0) {
+        // the kernel can run the node).  A grouped run (a.tile_rows set) keeps its one row tile per slice.
+        if (p.async_dma && p.split_k == 1 && p.tile_m == kPrefillTileM && L.groups_per_kblock == 1 && force_split <= 0 &&
+            a.tile_rows == 0) {
             const int64_t big_tiles = (a.N / kPrefillWideN) * ((a.M + 255) / 256);
             const int64_t big_rounds = (big_tiles + n_cus - 1) / n_cus;
             const int64_t small_rounds = ((int64_t)p.tiles_x * p.tiles_y + n_cus - 1) / n_cus;

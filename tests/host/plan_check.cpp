@@ -167,6 +167,19 @@ int main() {
         for (int64_t M : Ms)
             check_plan(d, M, OVFCC_KERNEL_AUTO, 0, 256);
     }
+    // a grouped run fixes the tile height: its plan keeps one row tile per slice whatever the tile counts say
+    {
+        const ovfcc_fc_desc d = desc(14336, 4096, 128, OVFCC_U4, OVFCC_U4, 0);
+        ovfcc::FcDeviceArgs a{};
+        a.M = 16 * 128, a.N = d.N, a.K = d.K, a.group_size = d.group_size, a.w_type = d.w_type, a.zp_type = d.zp_type;
+        a.layout = ovfcc::make_layout(d);
+        a.N_out = d.N;
+        ovfcc::LaunchPlan p;
+        CHECK(ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, 0, 256, &p) == 0 && p.big && p.tiles_y == 8, "one node: 256-row tiles");
+        a.tile_rows = 128;
+        CHECK(ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, 0, 256, &p) == 0 && !p.big && p.async_dma && p.tiles_y == 16,
+              "grouped: 128-row tiles");
+    }
     // the gate refuses what the kernels cannot index
     ovfcc_fc_desc bad = desc(64, 256, 96, OVFCC_U4, OVFCC_NONE, 0);
     CHECK(ovfcc::validate_desc(&bad) != 0, "group size must divide K");

@@ -386,6 +386,7 @@ GROUPED = [
     ("u4", "u4", 512, 1280, 128, False, [70, 3, 0, 129, 48, 300]),    # more rows: prefill kernel, slices of <= 128 rows
     ("i4", "none", 256, 2048, 2048, True, [64, 65]),                  # per-channel scale in the epilogue
     ("u4", "none", 256, 512, 128, False, [1] * 70 + [100]),           # more slices than one launch holds
+    ("u4", "u4", 4096, 256, 128, False, [128] * 32),                  # as one node it would take 256-row tiles
 ]
 
 
