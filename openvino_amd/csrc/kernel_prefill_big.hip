@@ -333,36 +333,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     };
     if (glu) {
         // channel tiles 2 j and 2 j + 1 of the wave are gate and up of output channels (n0 + 64 wave) / 2 + 16 j ..
+        float scg[2][4], bsg[2][4], scu[2][4], bsu[2][4];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            float scg[4], bsg[4], scu[4], bsu[4];
-            channel_params(2 * j, scg, bsg);
-            channel_params(2 * j + 1, scu, bsu);
-            const int n = (n0 + 64 * wave) / 2 + 16 * j + 4 * kq;
+            channel_params(2 * j, scg[j], bsg[j]);
+            channel_params(2 * j + 1, scu[j], bsu[j]);
+        }
 #pragma unroll
-            for (int t = 0; t < 16; ++t) {
-                const int m = m0 + 16 * t + col;
+        for (int t = 0; t < 16; ++t) {
+            const int m = m0 + 16 * t + col;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {  // the two pairs' results are neighbours in the output row
+                const int n = (n0 + 64 * wave) / 2 + 16 * j + 4 * kq;
                 const float4_t g = acc[2 * j][t], u = acc[2 * j + 1][t];
-                const float o[4] = {glu_value(glu, g.x * scg[0] + bsg[0], u.x * scu[0] + bsu[0]),
-                                    glu_value(glu, g.y * scg[1] + bsg[1], u.y * scu[1] + bsu[1]),
-                                    glu_value(glu, g.z * scg[2] + bsg[2], u.z * scu[2] + bsu[2]),
-                                    glu_value(glu, g.w * scg[3] + bsg[3], u.w * scu[3] + bsu[3])};
+                const float o[4] = {glu_value(glu, g.x * scg[j][0] + bsg[j][0], u.x * scu[j][0] + bsu[j][0]),
+                                    glu_value(glu, g.y * scg[j][1] + bsg[j][1], u.y * scu[j][1] + bsu[j][1]),
+                                    glu_value(glu, g.z * scg[j][2] + bsg[j][2], u.z * scu[j][2] + bsu[j][2]),
+                                    glu_value(glu, g.w * scg[j][3] + bsg[j][3], u.w * scu[j][3] + bsu[j][3])};
                 if (m < M)
                     put((size_t)m * (N / 2) + n, o);
             }
         }
         return;
     }
+    // Row tile by row tile, the four channel tiles one after the other: a wave's 64 channels are one 128-byte line
+    // of an f16 output row, written as four 32-byte pieces by consecutive store instructions.
+    float sc[4][4], bs[4][4];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        float sc[4], bs[4];
-        channel_params(r, sc, bs);
-        const int n = n0 + 64 * wave + 16 * r + 4 * kq;  // four consecutive channels
+    for (int r = 0; r < 4; ++r)
+        channel_params(r, sc[r], bs[r]);
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
-            const int m = m0 + 16 * t + col;
+    for (int t = 0; t < 16; ++t) {
+        const int m = m0 + 16 * t + col;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = n0 + 64 * wave + 16 * r + 4 * kq;  // four consecutive channels
             const float4_t v = acc[r][t];
-            const float o[4] = {v.x * sc[0] + bs[0], v.y * sc[1] + bs[1], v.z * sc[2] + bs[2], v.w * sc[3] + bs[3]};
+            const float o[4] = {v.x * sc[r][0] + bs[r][0], v.y * sc[r][1] + bs[r][1], v.z * sc[r][2] + bs[r][2],
+                                v.w * sc[r][3] + bs[r][3]};
             if (m < M)
                 put((size_t)m * N + n, o);
         }

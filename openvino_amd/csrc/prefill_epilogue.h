@@ -114,18 +114,21 @@ __device__ __forceinline__ void tile_epilogue(float4_t (&acc)[4][NT], unsigned c
                            float4_t{b.x + pu[0], b.y + pu[64], b.z + pu[128], b.w + pu[192]}, scg, bsg, scu, bsu);
             }
         } else if (kg == 0) {
+            // row tile by row tile, the two channel tiles back to back: their pieces of an output row are
+            // neighbours in one 128-byte line, and stores to a line that follow each other closely merge
+            float sc[2][4], bs[2][4];
+            channel_params(2 * hh, sc[0], bs[0]);
+            channel_params(2 * hh + 1, sc[1], bs[1]);
 #pragma unroll
-            for (int r2 = 0; r2 < 2; ++r2) {
-                const int r = 2 * hh + r2;
-                float sc[4], bs[4];
-                channel_params(r, sc, bs);
+            for (int t = 0; t < NT; ++t) {
 #pragma unroll
-                for (int t = 0; t < NT; ++t) {
+                for (int r2 = 0; r2 < 2; ++r2) {
+                    const int r = 2 * hh + r2;
                     const float* p = ex + ((wn * 8 * NT + (r2 * NT + t) * 4) * 64) + lane;
                     const float4_t a = acc[r][t];
                     const float4_t v = float4_t{a.x + p[0], a.y + p[64], a.z + p[128], a.w + p[192]};
                     if (split_k == 1)
-                        finish(r, t, v, sc, bs);
+                        finish(r, t, v, sc[r2], bs[r2]);
                     else
                         __builtin_amdgcn_raw_buffer_store_b128(
                             __builtin_bit_cast(uint4_t, v), rp,
@@ -186,14 +189,14 @@ __device__ __forceinline__ void tile_epilogue(float4_t (&acc)[4][NT], unsigned c
         for (int t = 0; t < NT; ++t)
             finish_glu(kg, t, sum[0][t], sum[1][t], scg, bsg, scu, bsu);
     } else {
+        float sc[2][4], bs[2][4];
+        channel_params(2 * kg, sc[0], bs[0]);
+        channel_params(2 * kg + 1, sc[1], bs[1]);
 #pragma unroll
-        for (int r2 = 0; r2 < 2; ++r2) {
-            float sc[4], bs[4];
-            channel_params(2 * kg + r2, sc, bs);
+        for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int t = 0; t < NT; ++t)
-                finish(2 * kg + r2, t, sum[r2][t], sc, bs);
-        }
+            for (int r2 = 0; r2 < 2; ++r2)
+                finish(2 * kg + r2, t, sum[r2][t], sc[r2], bs[r2]);
     }
     if (tid == 0)
         __hip_atomic_store(counters + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
