@@ -356,6 +356,48 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
         return;
     }
+    if (!out_f32 && (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+        // f16 output: the four lanes of a row (lane bits 4 and 5 = kq) hold four channels of each of the wave's four
+        // channel tiles.  A 4 x 4 exchange between them -- halves of the wave swapped, then neighbouring rows of 16
+        // lanes -- leaves lane kq with all 16 channels of tile kq: 32 contiguous bytes per lane, and the four lanes
+        // of a row write its whole 128-byte line with two store instructions.
+        float sc[4][4], bs[4][4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            channel_params(r, sc[r], bs[r]);
+        half_t* yh = static_cast<half_t*>(y);
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            uint32_t p[4][2];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float4_t v = acc[r][t];
+                const half4_t h = half4_t{(half_t)(v.x * sc[r][0] + bs[r][0]), (half_t)(v.y * sc[r][1] + bs[r][1]),
+                                          (half_t)(v.z * sc[r][2] + bs[r][2]), (half_t)(v.w * sc[r][3] + bs[r][3])};
+                const uint2_t u = __builtin_bit_cast(uint2_t, h);
+                p[r][0] = u.x, p[r][1] = u.y;
+            }
+            uint32_t q[8];  // channels 4 k' .. 4 k' + 3 of tile kq, from lane k' of the row: dwords 2 k', 2 k' + 1
+#pragma unroll
+            for (int d = 0; d < 2; ++d) {
+                // lanes 0-31 keep tiles 0 and 1, lanes 32-63 tiles 2 and 3; .x comes from the lane with kq bit 1
+                // clear, .y from the one with it set
+                const uint2_t s02 = __builtin_amdgcn_permlane32_swap(p[0][d], p[2][d], false, false);
+                const uint2_t s13 = __builtin_amdgcn_permlane32_swap(p[1][d], p[3][d], false, false);
+                // even rows of 16 lanes keep the even tile, odd rows the odd one; .x from kq bit 0 clear, .y set
+                const uint2_t lo = __builtin_amdgcn_permlane16_swap(s02.x, s13.x, false, false);
+                const uint2_t hi = __builtin_amdgcn_permlane16_swap(s02.y, s13.y, false, false);
+                q[d] = lo.x, q[2 + d] = lo.y, q[4 + d] = hi.x, q[6 + d] = hi.y;
+            }
+            const int m = m0 + 16 * t + col;
+            if (m < M) {
+                uint4_t* dst = reinterpret_cast<uint4_t*>(yh + (size_t)m * N + n0 + 64 * wave + 16 * kq);
+                dst[0] = uint4_t{q[0], q[1], q[2], q[3]};
+                dst[1] = uint4_t{q[4], q[5], q[6], q[7]};
+            }
+        }
+        return;
+    }
     // Row tile by row tile, the four channel tiles one after the other: a wave's 64 channels are one 128-byte line
     // of an f16 output row, written as four 32-byte pieces by consecutive store instructions.
     float sc[4][4], bs[4][4];
