@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/ (counters cannot be
 # read from inside this process): FETCH_SIZE x 2.000 (its reading for a copy kernel of known size) + WRITE_SIZE.
 TRAFFIC_DECODE_M1 = {"qo": 8869888, "kv": 2375680, "gate_up": 30526464, "down": 30669824}
-TRAFFIC_PREFILL_M2048 = {"qo": 85494784, "kv": 72139776, "gate_up": 328939520, "down": 255920128}
+TRAFFIC_PREFILL_M2048 = {"qo": 85494784, "kv": 72139776, "gate_up": 264916992, "down": 255920128}
 
 
 def log(*a):
