@@ -26,6 +26,8 @@ struct ovfcc_weights {
     void* d_scale = nullptr;
     void* d_zp = nullptr;
     void* d_bias = nullptr;
+    void* d_scale_cm = nullptr;  // channel-major copies of the group parameters for the matrix-vector kernel
+    void* d_zp_cm = nullptr;
     size_t bytes = 0;
 };
 
@@ -114,6 +116,8 @@ void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc:
     a->scale = w->d_scale;
     a->zp = w->d_zp;
     a->bias = w->d_bias;
+    a->scale_cm = w->d_scale_cm;
+    a->zp_cm = w->d_zp_cm;
     a->x = x;
     a->y = y;
     a->workspace = nullptr;
@@ -130,6 +134,31 @@ void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc:
     a->gate_offset = w->layout.glu_gate_second ? (int)(w->desc.N / 2) : 0;
     a->up_offset = w->layout.glu_gate_second ? 0 : (int)(w->desc.N / 2);
     a->layout = w->layout;
+}
+
+// Last step of every way a node comes into being: tiled 4-bit nodes with groups of 128 inputs get channel-major
+// copies of their scales and zero-point table, [N/16][16][K/128], which the matrix-vector kernel reads.
+int finish_weights(ovfcc_weights* W) {
+    ovfcc::Layout& L = W->layout;
+    L.gemv_c = 0;
+    if (!L.tiled || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 || !W->d_scale)
+        return OVFCC_OK;
+    const int c = ovfcc::gemv_kblocks_per_wave(L, W->ctx->n_cus);
+    if (c == 0)
+        return OVFCC_OK;
+    HIP_TRY(hipMalloc(&W->d_scale_cm, L.scale_bytes));
+    W->bytes += L.scale_bytes;
+    if (L.zp_table) {
+        HIP_TRY(hipMalloc(&W->d_zp_cm, L.zp_bytes));
+        W->bytes += L.zp_bytes;
+    }
+    int e = ovfcc::launch_gemv_params(W->d_scale, L.zp_table ? W->d_zp : nullptr, W->d_scale_cm, W->d_zp_cm, L.n_tiles,
+                                      L.groups, c, nullptr);
+    if (e)
+        return hip_fail((hipError_t)e, "parameter transposition launch");
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    L.gemv_c = c;
+    return OVFCC_OK;
 }
 
 // Buckets the (row, selected expert) pairs of a routed batch by expert, rows in ascending order inside a bucket:
@@ -427,6 +456,8 @@ int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* 
             rc = upload(&W->d_bias, bias, (size_t)N * 2);
         }
     }
+    if (!rc)
+        rc = finish_weights(W);
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;
@@ -442,6 +473,8 @@ void ovfcc_weights_destroy(ovfcc_weights* w) {
     if (w->d_scale) (void)hipFree(w->d_scale);
     if (w->d_zp) (void)hipFree(w->d_zp);
     if (w->d_bias) (void)hipFree(w->d_bias);
+    if (w->d_scale_cm) (void)hipFree(w->d_scale_cm);
+    if (w->d_zp_cm) (void)hipFree(w->d_zp_cm);
     delete w;
 }
 
@@ -482,6 +515,8 @@ int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out) {
     if (!rc) rc = dup(&W->d_scale, src->d_scale, sb);
     if (!rc) rc = dup(&W->d_zp, src->d_zp, zb);
     if (!rc) rc = dup(&W->d_bias, src->d_bias, (size_t)N * 2);
+    if (!rc)
+        rc = finish_weights(W);
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;
@@ -546,6 +581,8 @@ int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_w
     if (!rc && W->desc.bias_type != OVFCC_NONE)
         rc = gather(&W->d_bias, (size_t)n_total * 2, &ovfcc_weights::d_bias,
                     [](const ovfcc_weights* p) { return (size_t)p->desc.N * 2; });
+    if (!rc)
+        rc = finish_weights(W);
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;
@@ -595,6 +632,8 @@ int ovfcc_weights_glu(const ovfcc_weights* gate, const ovfcc_weights* up, int gl
         rc = weave(&W->d_zp, gate->d_zp, up->d_zp, gate->layout.zp_bytes / tiles);
     if (!rc && W->desc.bias_type != OVFCC_NONE)
         rc = weave(&W->d_bias, gate->d_bias, up->d_bias, (size_t)ovfcc::kTileRows * 2);
+    if (!rc)
+        rc = finish_weights(W);
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;
@@ -730,6 +769,8 @@ int ovfcc_weights_import(ovfcc_ctx* ctx, const void* blob, size_t bytes, ovfcc_w
         }
         at += pad16(sz[i]);
     }
+    if (!rc)
+        rc = finish_weights(W);
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;

@@ -49,6 +49,8 @@ struct Layout {
     // so that the wave that finishes a gate tile also holds the matching up tile.
     int glu = 0;
     bool glu_gate_second = false;
+    int gemv_c = 0;         // k-blocks per wave of the matrix-vector kernel, fixed when the node's channel-major
+                            // parameter tables are written (0: the node has none)
     bool dynquant = false;  // the node allows per-token int8 activations (OVFCC_DYNQUANT_I8) where a kernel exists
     // element index of the scale / zero-point of channel r of tile nt for group g
     size_t param_index(int64_t nt, int64_t g, int r) const {
@@ -97,6 +99,8 @@ struct FcDeviceArgs {
     const void* scale;
     const void* zp;      // table, raw zp, or null
     const void* bias;    // f16 [N] or null
+    const void* scale_cm = nullptr;  // channel-major copies [N/16][16][wave][slot] of scales and zero-point table,
+    const void* zp_cm = nullptr;     // where the node has them (tiled 4-bit weights, groups of 128 inputs)
     const void* x;       // f16 [M,K]
     void* y;             // f16 or f32 [M,N]
     float* workspace;    // split-K partials
@@ -121,6 +125,8 @@ struct LaunchPlan {
     bool async_dma = false;     // ... and of those the one whose operands all travel by direct-to-LDS loads
     bool big = false;           // prefill family: the 4-bit kernel with 256 x 256 tiles (whole tiles, no split-K)
     bool batch = false;         // decode family: the small-batch kernel (waves own channel tiles)
+    bool gemv = false;          // decode family: the matrix-vector kernel for M <= 4 (4-bit weights, G = 128)
+    int gemv_c = 0;             // ... and its k-blocks per wave (2, 4 or 8)
     int tiles_x = 0, tiles_y = 0;  // async prefill kernel: the tile grid; its launch is 1-D
     int full_tiles = 0;         // ... of which this many run unsplit (the rest in split_k parts each)
     unsigned grid[3] = {1, 1, 1};
@@ -138,6 +144,14 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_plain(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_decode(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_batch(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_gemv(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+// dynamic LDS of the matrix-vector kernel: c k-blocks per wave, m rows, `waves` waves per workgroup
+size_t gemv_lds_bytes(int c, int m, int waves);
+// [N/16][groups][16] scales f16 (and zero-points u8, or null) -> channel-major [N/16][16][groups]
+int launch_gemv_params(const void* scale_tiled, const void* zp_tiled, void* scale_cm, void* zp_cm, int64_t n_tiles,
+                       int64_t groups, int c_slots, void* stream);
+// k-blocks per wave of the matrix-vector kernel for a node (0: the kernel does not fit it)
+int gemv_kblocks_per_wave(const Layout& L, int n_cus);
 
 // Problems of one grouped launch (passed in the kernel arguments: at most 4 KiB)
 constexpr int kMaxGroupItems = 64;

@@ -18,6 +18,25 @@ static int env_int(const char* name, int fallback) {
     return e ? std::atoi(e) : fallback;
 }
 
+// k-blocks per wave of the matrix-vector kernel for this node (0: the kernel does not fit it).  The waves of one
+// channel tile (of a gate / up tile pair) share a workgroup of at most 16 waves and each takes 2, 4 or 8 whole
+// k-blocks; of the divisions that fit, the coarsest one that still gives every SIMD of the chip about two waves.
+// OVFCC_GEMV_C overrides for experiments.
+int gemv_kblocks_per_wave(const Layout& L, int n_cus) {
+    const int tiles_per_wg = L.glu ? 2 : 1;
+    if (L.glu && (L.n_tiles & 1))
+        return 0;
+    auto fits = [&](int c) { return L.k_blocks % c == 0 && (L.k_blocks / c) * tiles_per_wg <= 16; };
+    const int forced = env_int("OVFCC_GEMV_C", 0);
+    if ((forced == 2 || forced == 4 || forced == 8) && fits(forced))
+        return forced;
+    int best = 0;
+    for (int c : {2, 4, 8})
+        if (fits(c) && (best == 0 || L.n_tiles * (L.k_blocks / c) >= (int64_t)8 * n_cus))
+            best = c;
+    return best;
+}
+
 int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_cus, LaunchPlan* plan) {
     LaunchPlan p;
     const Layout& L = a.layout;
@@ -91,6 +110,23 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
     } else if (kernel == OVFCC_KERNEL_DECODE && want_batch) {
         if (int rc = plan_batch())
             return rc;
+    } else if (kernel == OVFCC_KERNEL_DECODE && a.M <= 4 && a.scale_cm && L.bits == 4 && L.groups_per_kblock == 1 &&
+               L.kblocks_per_group == 1 && force_split <= 0 && env_int("OVFCC_GEMV", 1) != 0 && L.gemv_c != 0) {
+        // One to four rows of a 4-bit node with groups of 128 inputs: the matrix-vector kernel.
+        const int c = L.gemv_c;
+        const int tiles_per_wg = L.glu ? 2 : 1;
+        const int waves = (int)(L.k_blocks / c) * tiles_per_wg;
+        p.gemv = true;
+        p.gemv_c = c;
+        p.split_k = 1;
+        p.kblocks_per_split = (int)L.k_blocks;
+        p.tiles_per_group = tiles_per_wg;
+        p.grid[0] = (unsigned)(L.n_tiles / tiles_per_wg);
+        p.block = 64u * waves;
+        p.tile_m = 16;
+        p.tile_n = 16 * tiles_per_wg;
+        p.dynamic_lds = (unsigned)gemv_lds_bytes(c, (int)a.M, waves);
+        p.name = "fcc_gemv_w4";
     } else if (kernel == OVFCC_KERNEL_DECODE) {
         if (a.M > 32)
             return fail(OVFCC_EUNSUPPORTED, "the streaming decode kernel handles at most 32 rows");
@@ -293,7 +329,7 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     case OVFCC_KERNEL_PLAIN:
         return launch_plain(a, p, stream);
     case OVFCC_KERNEL_DECODE:
-        return p.batch ? launch_batch(a, p, stream) : launch_decode(a, p, stream);
+        return p.gemv ? launch_gemv(a, p, stream) : p.batch ? launch_batch(a, p, stream) : launch_decode(a, p, stream);
     default:
         if (p.big)
             return launch_prefill_big(a, p, stream);

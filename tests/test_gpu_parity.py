@@ -169,6 +169,8 @@ def test_kernel_policy(dev, req):
     try:
         assert w.tiled
         req.infer(w, c.x[:1])
+        assert req.last_kernel()["name"] == "fcc_gemv_w4"    # one to four rows, 4-bit weights, groups of 128
+        req.infer(w, c.x[:5])
         assert req.last_kernel()["name"] == "fcc_decode_w4"
         req.infer(w, c.x[:32])
         assert req.last_kernel()["name"] == "fcc_batch_w4"
@@ -218,6 +220,7 @@ def test_both_decode_kernels_every_row_count(oracle, dev, req, monkeypatch, wt, 
     """The streaming kernel (M <= 32) and the small-batch kernel (M <= 48) each forced over their whole range of
     row counts, with channel-tile counts that leave the last workgroup ragged, with and without a forced split."""
     monkeypatch.setenv("OVFCC_DECODE_BATCH", batch)
+    monkeypatch.setenv("OVFCC_GEMV", "0")     # one to four rows would otherwise take the matrix-vector kernel
     top = 48 if batch == "1" else 32
     c = datagen.make_case(41, top, K, N, wt, G, zt, with_bias=True)
     w = fc.CompressedWeights.from_case(dev, c)
