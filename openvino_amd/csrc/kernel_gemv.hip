@@ -338,11 +338,6 @@ static void launch_gemv_rows(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
         launch_gemv_impl<C, 4, ZPT>(a, p, s);
 }
 
-size_t gemv_lds_bytes(int c, int m, int waves) {
-    const int mr = m == 1 ? 1 : m == 2 ? 2 : 4;
-    return (size_t)waves * mr * (c * 256 + 64) + (size_t)waves * mr * 16 * sizeof(float);
-}
-
 int launch_gemv(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;

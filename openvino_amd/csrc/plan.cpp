@@ -37,6 +37,13 @@ int gemv_kblocks_per_wave(const Layout& L, int n_cus) {
     return best;
 }
 
+// Dynamic LDS of the matrix-vector kernel: every wave stages its rows (1, 2 or 4 carried; c k-blocks of 256 bytes
+// each plus a 64-byte pad per row) and leaves 16 partial sums per row.
+size_t gemv_lds_bytes(int c, int m, int waves) {
+    const int mr = m == 1 ? 1 : m == 2 ? 2 : 4;
+    return (size_t)waves * mr * (c * 256 + 64) + (size_t)waves * mr * 16 * sizeof(float);
+}
+
 int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_cus, LaunchPlan* plan) {
     LaunchPlan p;
     const Layout& L = a.layout;

@@ -14,6 +14,7 @@ namespace ovfcc {
 int launch_plain(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_decode(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_batch(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_gemv(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_wide(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_direct(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
@@ -64,6 +65,13 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     a.M = M, a.N = d.N, a.K = d.K, a.group_size = d.group_size, a.w_type = d.w_type, a.zp_type = d.zp_type;
     a.layout = ovfcc::make_layout(d);
     a.N_out = a.layout.glu ? d.N / 2 : d.N;
+    // what the API does when a node is created: nodes the matrix-vector kernel fits carry its parameter tables
+    static const int placeholder = 0;
+    if (a.layout.tiled && a.layout.bits == 4 && a.layout.groups_per_kblock == 1 && a.layout.kblocks_per_group == 1) {
+        a.layout.gemv_c = ovfcc::gemv_kblocks_per_wave(a.layout, n_cus);
+        if (a.layout.gemv_c)
+            a.scale_cm = &placeholder, a.zp_cm = a.layout.zp_table ? &placeholder : nullptr;
+    }
     const ovfcc::Layout& L = a.layout;
     ovfcc::LaunchPlan p;
     const int rc = ovfcc::plan_launch(a, force, force_split, n_cus, &p);
@@ -93,7 +101,13 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     if (p.kernel == OVFCC_KERNEL_DECODE) {
         CHECK(M <= ovfcc::kDecodeMaxRows, "%s", what);
         const int nw = (int)p.block / 64, rt = p.tiles_per_group;
-        if (p.batch) {
+        if (p.gemv) {
+            const int c = p.gemv_c, per_wg = L.glu ? 2 : 1;
+            CHECK(M <= 4 && L.bits == 4 && L.groups_per_kblock == 1 && L.kblocks_per_group == 1 && c == L.gemv_c, "%s", what);
+            CHECK((c == 2 || c == 4 || c == 8) && kb % c == 0 && nw == (kb / c) * per_wg && nw <= 16, "%s c=%d nw=%d", what, c, nw);
+            CHECK((int64_t)p.grid[0] * per_wg == L.n_tiles && p.grid[1] == 1 && p.split_k == 1, "%s", what);
+            CHECK(p.dynamic_lds == ovfcc::gemv_lds_bytes(c, (int)M, nw) && p.dynamic_lds <= 150 * 1024, "%s lds=%u", what, p.dynamic_lds);
+        } else if (p.batch) {
             const int mt = (int)(M + 15) / 16;
             CHECK(p.tile_m == 16 * mt && (rt == 1 || rt == 2), "%s", what);
             CHECK((int64_t)p.grid[0] * nw * rt >= L.n_tiles && p.grid[1] == (unsigned)p.split_k, "%s", what);
