@@ -203,6 +203,17 @@ int ovfcc_fc_run(ovfcc_request* req, const ovfcc_weights* w, const void* x_host,
  * stream and returns without waiting. */
 int ovfcc_fc_run_device(ovfcc_request* req, const ovfcc_weights* w, const void* x_dev, void* y_dev, int64_t M);
 
+/* ovfcc_fc_run_device for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  It has no counterpart in the OpenVINO sources.  Same arguments, same
+ * kernels and bit-identical results, but the call allocates nothing: launches that split K take their partial
+ * tiles and arrival counters from a fixed scratch array in device memory (32 MiB of partial tiles, 16384
+ * counters, held by every GPU the library runs on until the process ends) instead of buffers of the request,
+ * and clear the counters they use with a small fill kernel first.  A launch that needs more than the array holds,
+ * and a node whose activations would be quantised to int8 (OVFCC_DYNQUANT_I8 taking effect), is
+ * OVFCC_EUNSUPPORTED.  All requests of a GPU share that GPU's array: calls of this entry point that overlap in time
+ * on one GPU race; serialise them (one stream, or events between streams). */
+int ovfcc_fc_run_device_static(ovfcc_request* req, const ovfcc_weights* w, const void* x_dev, void* y_dev, int64_t M);
+
 /* Several independent nodes of one shape and weight format in one launch: the experts of a
  * mixture-of-experts layer, each with its own gathered rows.  Stands in for the grouped forms of the op,
  * ov::op::internal::GatherMatmulCompressed (src/common/transformations/include/ov_ops/

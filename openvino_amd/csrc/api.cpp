@@ -106,6 +106,38 @@ int ensure_split_buffers(ovfcc_request* r, const ovfcc::LaunchPlan& plan) {
     return OVFCC_OK;
 }
 
+// Split-K workspace and arrival counters for one launch: the request's own buffers (grown on demand), or -- for
+// the entry point that allocates nothing -- the device's fixed scratch array, whose counters are cleared by a fill
+// kernel ahead of the launch (the array keeps whatever the last call left, on this or any other request).
+int split_buffers(ovfcc_request* r, const ovfcc::LaunchPlan& plan, bool static_scratch, ovfcc::FcDeviceArgs* a) {
+    if (!static_scratch) {
+        int rc = ensure_split_buffers(r, plan);
+        a->workspace = r->workspace;
+        a->counters = r->counters;
+        return rc;
+    }
+    a->workspace = nullptr;
+    a->counters = nullptr;
+    if (plan.workspace_bytes == 0 && plan.counter_count == 0)
+        return OVFCC_OK;
+    if (plan.workspace_bytes > ovfcc::kStaticWorkspaceBytes ||
+        plan.counter_count * sizeof(unsigned) > ovfcc::kStaticCounterBytes)
+        return fail(OVFCC_EUNSUPPORTED,
+                    "this launch splits K and needs " + std::to_string(plan.workspace_bytes) + " bytes of partial tiles and " +
+                        std::to_string(plan.counter_count) + " counters; the fixed scratch array holds " +
+                        std::to_string(ovfcc::kStaticWorkspaceBytes) + " bytes and " +
+                        std::to_string(ovfcc::kStaticCounterBytes / sizeof(unsigned)) + " counters");
+    unsigned char* base = static_cast<unsigned char*>(ovfcc::static_scratch_ptr(r->ctx->device));
+    if (!base)
+        return fail(OVFCC_EDEVICE, "the fixed scratch array was not set up on this device");
+    a->counters = reinterpret_cast<unsigned*>(base);
+    a->workspace = reinterpret_cast<float*>(base + ovfcc::kStaticCounterBytes);
+    int e = ovfcc::launch_zero_u32(a->counters, plan.counter_count, r->stream);
+    if (e)
+        return hip_fail((hipError_t)e, "counter fill launch");
+    return OVFCC_OK;
+}
+
 // row length of the node's output
 int64_t out_channels(const ovfcc_weights* w) {
     return w->layout.glu ? w->desc.N / 2 : w->desc.N;
@@ -223,11 +255,11 @@ void record(ovfcc_request* r, const ovfcc::LaunchPlan& p) {
     std::snprintf(i.name, sizeof(i.name), "%s", p.name);
 }
 
-int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M);
+int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch);
 
 // Enqueue one node.  The fast kernels address the activations with 32-bit byte offsets and the plain kernel puts
 // the rows on a 16-bit grid axis: a longer node runs as consecutive row blocks on the same stream.
-int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M) {
+int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch = false) {
     int64_t block = M;
     if (w->layout.tiled) {
         const int64_t lim = ((((int64_t)1 << 31) - 1) / (2 * w->desc.K)) & ~(int64_t)127;
@@ -240,7 +272,7 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
     for (int64_t m0 = 0; m0 < M; m0 += block) {
         const int64_t rows = M - m0 < block ? M - m0 : block;
         int rc = enqueue_rows(r, w, static_cast<const char*>(x) + (size_t)m0 * w->desc.K * 2,
-                              static_cast<char*>(y) + (size_t)m0 * out_row, rows);
+                              static_cast<char*>(y) + (size_t)m0 * out_row, rows, static_scratch);
         if (rc)
             return rc;
     }
@@ -249,7 +281,7 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
 
 // One block of rows.  A tiled node is cut into decode-family launches of at most 48 rows when M is small
 // enough that they beat one sparse prefill grid, or when N is not a multiple of the prefill tile.
-int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M) {
+int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch) {
     if (M == 0)
         return OVFCC_OK;
     ovfcc::FcDeviceArgs a;
@@ -265,6 +297,8 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
         // OVFCC_PREFILL_WIDE = 1 forces the 256-wide kernels onto small shapes, for tests)
         ((w->desc.N / 256) * ((M + 127) / 128) * 2 >= r->ctx->n_cus ||
          (std::getenv("OVFCC_PREFILL_WIDE") && std::atoi(std::getenv("OVFCC_PREFILL_WIDE")) == 1))) {
+        if (static_scratch)
+            return fail(OVFCC_EUNSUPPORTED, "a node with int8 activations needs a quantisation buffer of the request");
         const size_t q_bytes = ((size_t)M * w->desc.K + 255) & ~(size_t)255;
         const size_t need = q_bytes + (size_t)M * 8;
         if (need > r->quant_cap)
@@ -309,11 +343,9 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
             int rc = ovfcc::plan_launch(a, OVFCC_KERNEL_DECODE, r->force_split, r->ctx->n_cus, &p);
             if (rc)
                 return rc;
-            rc = ensure_split_buffers(r, p);
+            rc = split_buffers(r, p, static_scratch, &a);
             if (rc)
                 return rc;
-            a.workspace = r->workspace;
-            a.counters = r->counters;
             int e = ovfcc::launch_fc(a, p, r->stream);
             if (e)
                 return hip_fail((hipError_t)e, "kernel launch");
@@ -325,11 +357,9 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
     int rc = ovfcc::plan_launch(a, force, r->force_split, r->ctx->n_cus, &p);
     if (rc)
         return rc;
-    rc = ensure_split_buffers(r, p);
+    rc = split_buffers(r, p, static_scratch, &a);
     if (rc)
         return rc;
-    a.workspace = r->workspace;
-    a.counters = r->counters;
     int e = ovfcc::launch_fc(a, p, r->stream);
     if (e)
         return hip_fail((hipError_t)e, "kernel launch");
@@ -368,6 +398,9 @@ int ovfcc_init(int device, ovfcc_ctx** out) {
     std::string arch = prop.gcnArchName;
     if (arch.rfind("gfx950", 0) != 0)
         return fail(OVFCC_EDEVICE, "device is " + arch + "; the kernels are built for gfx950 only");
+    // the fixed scratch array of ovfcc_fc_run_device_static: its address on this device, looked up once
+    if (int se = ovfcc::static_scratch_setup(device))
+        return hip_fail((hipError_t)se, "hipGetSymbolAddress of the fixed scratch array");
     ovfcc_ctx* c = new ovfcc_ctx();
     c->device = device;
     c->n_cus = prop.multiProcessorCount;
@@ -844,6 +877,21 @@ int ovfcc_fc_run_device(ovfcc_request* r, const ovfcc_weights* w, const void* x_
         return fail(OVFCC_EUNSUPPORTED, "M is limited to 2^24");
     HIP_TRY(hipSetDevice(r->ctx->device));
     return enqueue(r, w, x_dev, y_dev, M);
+}
+
+int ovfcc_fc_run_device_static(ovfcc_request* r, const ovfcc_weights* w, const void* x_dev, void* y_dev, int64_t M) {
+    if (!r || !w)
+        return fail(OVFCC_EINVAL, "request or weights is null");
+    if (M < 0)
+        return fail(OVFCC_EINVAL, "M is negative");
+    if (M > 0 && (!x_dev || !y_dev))
+        return fail(OVFCC_EINVAL, "x or y is null");
+    if (w->ctx != r->ctx)
+        return fail(OVFCC_EINVAL, "weights and request belong to different contexts");
+    if (M > ((int64_t)1 << 24))
+        return fail(OVFCC_EUNSUPPORTED, "M is limited to 2^24");
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    return enqueue(r, w, x_dev, y_dev, M, true);
 }
 
 int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items, int n_items) {

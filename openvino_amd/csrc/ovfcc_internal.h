@@ -193,6 +193,13 @@ int launch_touch(const void* src, size_t bytes, void* stream);
 int launch_moe_combine(void* y, const void* d, const void* routing, const int* pos, int rows, int top_k, int H,
                        int d_f32, int out_f32, void* stream);
 
+// Scratch array of the entry point that allocates nothing: arrival counters, then split-K partial tiles
+constexpr size_t kStaticCounterBytes = (size_t)64 << 10;
+constexpr size_t kStaticWorkspaceBytes = (size_t)32 << 20;
+int static_scratch_setup(int device);
+void* static_scratch_ptr(int device);
+int launch_zero_u32(unsigned* p, size_t n, void* stream);
+
 constexpr int kDecodeMaxRows = 48;                       // rows one decode-family launch covers
 constexpr int kPrefillGroupRows = 128;                   // rows per slice of a grouped prefill launch (one tile)
 constexpr int kChunkedMinPrefillRows = 48;                // ... unless, above this, the async prefill kernel fills the chip

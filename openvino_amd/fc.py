@@ -228,6 +228,12 @@ class InferRequest:
         check(self.device.lib.ovfcc_fc_run_device(self.handle, weights.handle, ctypes.c_void_p(x_ptr),
                                                   ctypes.c_void_p(y_ptr), M))
 
+    def infer_device_static(self, weights: CompressedWeights, x_ptr: int, y_ptr: int, M: int) -> None:
+        """infer_device through the entry point that allocates nothing (fixed scratch array instead of buffers of
+        the request); calls that overlap on one GPU race."""
+        check(self.device.lib.ovfcc_fc_run_device_static(self.handle, weights.handle, ctypes.c_void_p(x_ptr),
+                                                         ctypes.c_void_p(y_ptr), M))
+
     def _group_items(self, items):
         arr = (_lib.GroupItem * len(items))()
         for a, (w, x_ptr, y_ptr, M) in zip(arr, items):
