@@ -910,7 +910,9 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
             return fail(OVFCC_EINVAL, "an item's weights are null or belong to another context");
         if (items[i].M < 0 || (items[i].M > 0 && (!items[i].x_dev || !items[i].y_dev)))
             return fail(OVFCC_EINVAL, "an item has a negative row count or a null buffer");
-        same = std::memcmp(&w->desc, &w0->desc, sizeof(ovfcc_fc_desc)) == 0 && (w->d_bias != nullptr) == (w0->d_bias != nullptr);
+        // (a scalar zero-point lives in the layout, not in the descriptor, and the grouped kernels take one for all)
+        same = std::memcmp(&w->desc, &w0->desc, sizeof(ovfcc_fc_desc)) == 0 &&
+               (w->d_bias != nullptr) == (w0->d_bias != nullptr) && w->layout.zp_const == w0->layout.zp_const;
     }
     // one launch needs a common shape and format, the tiled layout and no forced kernel; otherwise item by item
     bool grouped = same && w0->layout.tiled && r->force_kernel == OVFCC_KERNEL_AUTO;
@@ -938,6 +940,7 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
     }
     ovfcc::FcDeviceArgs a;
     std::vector<ovfcc::BatchGroupItem> work;
+    std::vector<const ovfcc_weights*> work_w;  // the node of every slice, for slices that end up running one by one
     if (grouped) {
         // cut every item into equal slices of at most rows_cap rows
         const size_t out_bytes = w0->desc.out_type == OVFCC_F32 ? 4 : 2;
@@ -957,6 +960,7 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
                 it.M = (int)std::min(M - m0, step);
                 rows_max = std::max<int64_t>(rows_max, it.M);
                 work.push_back(it);
+                work_w.push_back(w);
             }
         }
     }
@@ -990,9 +994,16 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
             grouped = !rc && p.async_dma && p.tiles_y == n;
         }
         if (!grouped) {
-            if (first != 0)
-                return fail(OVFCC_EUNSUPPORTED, "grouped launch plan changed between batches of slices");
-            break;
+            if (first == 0)
+                break;
+            // A later, smaller batch of slices for which no grouped kernel applies (a short tail of a long list):
+            // its slices run one by one, with the same results.
+            for (size_t j = first; j < work.size(); ++j) {
+                rc = enqueue(r, work_w[j], work[j].x, work[j].y, work[j].M);
+                if (rc)
+                    return rc;
+            }
+            return OVFCC_OK;
         }
         ovfcc::LaunchPlan all = p;  // split-K buffers for n slices
         if (decode) {

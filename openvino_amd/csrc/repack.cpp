@@ -86,8 +86,11 @@ Layout make_layout(const ovfcc_fc_desc& d) {
     L.glu = d.flags & OVFCC_GLU_TYPE_MASK;
     L.glu_gate_second = (d.flags & OVFCC_GLU_GATE_SECOND) != 0;
     const bool small_groups = L.bits == 4 && (d.group_size == 32 || d.group_size == 64);
+    // The tiled zero-point table holds zp + zp_offset in one byte: signed weights with 8-bit zero-points per group
+    // (up to 255 + 8 or 255 + 128) do not fit and keep OpenVINO's layout, which the plain kernel runs.
+    const bool zp_fits = !L.zp_table || L.zp_offset + (d.zp_type == OVFCC_U4 ? 15 : 255) <= 255;
     L.tiled = (d.N % (L.glu ? 2 * kTileRows : kTileRows) == 0) && (d.K % kBlockK == 0) &&
-              (d.group_size % kBlockK == 0 || small_groups) && (d.K / kBlockK < 65536);
+              (d.group_size % kBlockK == 0 || small_groups) && (d.K / kBlockK < 65536) && zp_fits;
     if (L.tiled) {
         L.n_tiles = d.N / kTileRows;
         L.k_blocks = d.K / kBlockK;

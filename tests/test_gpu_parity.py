@@ -714,3 +714,82 @@ def test_device_memory_helpers(dev):
         finally:
             dev.free(p)
             dev.free(q)
+
+
+@pytest.mark.parametrize("wt,zt,zp_top", [("i8", "u8", 255), ("i4", "u8", 255), ("i4", "u4", 15)])
+def test_signed_weights_with_zero_points(oracle, dev, req, wt, zt, zp_top):
+    """Signed weights with per-group zero-points, zero-points at the top of their range included: the stored form is
+    unsigned with the zero-point raised by 8 / 128, which fits the tiled table's byte only for 4-bit zero-points;
+    the other two keep OpenVINO's layout and run the plain kernel."""
+    say(f"signed weights with zero-points {wt}/{zt}")
+    c = datagen.make_case(3100, 20, 512, 64, wt, 128, zt, with_bias=True)
+    zp = c.zp.copy()
+    if zt == "u8":
+        zp.reshape(-1)[::3] = zp_top            # 255: beyond what one byte holds once the offset is added
+        zp.reshape(-1)[1::3] = 200
+    else:
+        zp[:] = 0xFF                            # every 4-bit zero-point 15
+    c = datagen.FcCase(c.M, c.K, c.N, c.group_size, c.w_type, c.zp_type, c.w, c.scale, zp, c.x, c.bias)
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        assert w.tiled == (zt == "u4")
+        ref = oracle_y(oracle, c)
+        for M in (1, 5, 20):
+            y = req.infer(w, c.x[:M])
+            check_parity(oracle, y, ref[:M], c.K, f"M={M} {req.last_kernel()}", output_rounding_slack=True)
+    finally:
+        w.close()
+
+
+def test_grouped_run_with_different_scalar_zero_points(oracle, dev, req):
+    """Experts whose scalar zero-points differ agree in every descriptor field (the scalar lives beside it): they
+    must not share a grouped launch, which carries one constant for all; each still gets its own result."""
+    say("grouped, scalar zero-points differ")
+    cases, ws = [], []
+    for i, zpv in enumerate((3, 11, 7)):
+        c = datagen.make_case(3200 + i, 24, 512, 256, "u4", 128, "u8", with_bias=False)
+        c = datagen.FcCase(c.M, c.K, c.N, c.group_size, c.w_type, "u8", c.w, c.scale, np.array([zpv], np.uint8), c.x,
+                           None, zp_scalar=True)
+        cases.append(c)
+        ws.append(fc.CompressedWeights.from_case(dev, c))
+    try:
+        ys = req.infer_grouped([(w, c.x) for w, c in zip(ws, cases)])
+        assert "grouped" not in req.last_kernel()["name"]
+        for y, c in zip(ys, cases):
+            check_parity(oracle, y, oracle_y(oracle, c), c.K, "scalar zp per expert", output_rounding_slack=True)
+        same = req.infer_grouped([(ws[1], cases[1].x), (ws[1], cases[1].x[:9])])   # equal constants: one launch
+        assert "grouped" in req.last_kernel()["name"]
+        check_parity(oracle, same[1], oracle_y(oracle, cases[1], x=cases[1].x[:9]), 512, "equal scalar zp",
+                     output_rounding_slack=True)
+    finally:
+        for w in ws:
+            w.close()
+
+
+def test_grouped_run_more_than_64_slices(oracle, dev, req):
+    """More slices than one grouped launch carries (64): the list runs in batches, and a short last batch for which
+    the planner picks no grouped kernel runs slice by slice -- every item still gets its result."""
+    say("grouped, 70 items")
+    c = datagen.make_case(3300, 12, 512, 128, "u4", 128, "u4", with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        rows = [1 + (i * 5) % 12 for i in range(70)]
+        ys = req.infer_grouped([(w, c.x[:m]) for m in rows])
+        ref = oracle_y(oracle, c)
+        for m, y in zip(rows, ys):
+            check_parity(oracle, y, ref[:m], c.K, f"M={m}", output_rounding_slack=True)
+    finally:
+        w.close()
+    # prefill row counts: 64 slices fill the chip with 256-wide tiles and share a launch, the remaining six do not
+    c = datagen.make_case(3301, 64, 1024, 512, "u4", 128, "u4", with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        rows = [50 + i % 15 for i in range(70)]
+        ys = req.infer_grouped([(w, c.x[:m]) for m in rows])
+        say(f"   last launch: {req.last_kernel()['name']}")
+        assert "grouped" not in req.last_kernel()["name"]       # the tail ran slice by slice
+        ref = oracle_y(oracle, c)
+        for m, y in zip(rows, ys):
+            check_parity(oracle, y, ref[:m], c.K, f"M={m}", output_rounding_slack=True)
+    finally:
+        w.close()

@@ -137,3 +137,21 @@ def test_input_major_nibble_transpose_known_answer():
     assert d.pack_nibbles(rows).tolist() == [0x21, 0x43, 0x65]
     assert d.pack_nibbles(rows.T).tolist() == [0x41, 0x52, 0x63]
     assert d.unpack_nibbles(d.pack_nibbles(rows.T), 6).reshape(3, 2).T.tolist() == rows.tolist()
+
+
+def test_signed_weights_with_byte_zero_points_stay_untiled():
+    """The tiled zero-point table stores zp + 8 (i4) or zp + 128 (i8) in one byte.  With 8-bit zero-points per group
+    that sum can pass 255, so such nodes keep OpenVINO's layout (the plain kernel subtracts the zero-point itself);
+    i4 with 4-bit zero-points (at most 15 + 8) is tiled and its table holds zp + 8 exactly."""
+    for wt_ in ("i8", "i4"):
+        desc = fc.make_desc(16, 128, 128, wt_, zp_type="u8")
+        assert fc.tiled_sizes(desc) == (0, 0, 0), wt_
+        with pytest.raises(fc.OvfccError):
+            fc.repack_host(desc, np.zeros(16 * 128, np.uint8), np.ones((16, 1), np.float16), np.full((16, 1), 200, np.uint8))
+    # a scalar zero-point travels as an integer, not in the byte table: tiled
+    assert fc.tiled_sizes(fc.make_desc(16, 128, 128, "i8", zp_type="u8", zp_scalar=True))[0] > 0
+    desc = fc.make_desc(16, 256, 128, "i4", zp_type="u4")
+    assert fc.tiled_sizes(desc)[2] == 16 * 2
+    zp = np.full(16, 0xFF, np.uint8)                      # every zero-point 15, two per byte
+    _, _, zt = fc.repack_host(desc, np.zeros(16 * 128, np.uint8), np.ones((16, 2), np.float16), zp)
+    assert np.all(zt == 23)
