@@ -1,0 +1,117 @@
+/*
+ * ovfcc_graph -- the graph-side half of the weight-compressed FullyConnected path, free of OpenVINO types.
+ *
+ * A host (the ov::IPlugin shim, a test) describes the relevant part of a model as an array of plain nodes;
+ * the functions here decide what OpenVINO's transformation passes decide on the real graph and return
+ * descriptors for ovfcc_weights_create / ovfcc_weights_concat / ovfcc_weights_glu:
+ *
+ *   ovfcc_fold_match   MatMul (or internal FullyConnected) over a weight-decompression subgraph
+ *                      -> one FullyConnectedCompressed node: the roles of pattern::op::CompressedWeightsBlock
+ *                      (src/common/transformations/src/transformations/pattern_blocks/compressed_weights_block.cpp:31-84),
+ *                      ConvertMatMulToFC (src/plugins/intel_cpu/src/transformations/cpu_opset/common/pass/
+ *                      convert_matmul_to_fc.cpp:47-270), ConvertFullyConnectedToFullyConnectedCompressed with its
+ *                      combine_groups shape algebra (src/common/transformations/src/transformations/op_conversions/
+ *                      convert_fc_to_compressed.cpp:32-225) and FullyConnectedBiasFusion
+ *                      (src/plugins/intel_cpu/src/transformations/cpu_opset/common/pass/fc_bias_fusion.cpp:32-93).
+ *   ovfcc_fold_model   all such nodes of a model, plus which of them share a launch: horizontal fusion of
+ *                      siblings that read the same activations (src/plugins/intel_gpu/src/plugin/transformations/
+ *                      fc_horizontal_fusion.cpp:30-140) and the gated linear unit act(gate(x)) * up(x)
+ *                      (src/common/transformations/include/ov_ops/glu.hpp:16-40; kernel-side fusion
+ *                      src/plugins/intel_gpu/src/kernel_selector/kernels/fully_connected/
+ *                      fully_connected_kernel_bf_tiled.cpp:223-236).
+ *
+ * Nothing here touches constant data or a device: shapes, element types and small integer attributes in,
+ * decisions out.  Return codes and ovfcc_last_error() as in ovfcc.h; "this subgraph is not a compressed
+ * FullyConnected" is OVFCC_EUNSUPPORTED with the reason in the error string.
+ */
+#ifndef OVFCC_GRAPH_H
+#define OVFCC_GRAPH_H
+
+#include "ovfcc.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* operations the matchers look at (openvino/op/*.hpp, ov_ops/fully_connected.hpp); everything else is OTHER */
+enum ovfcc_op {
+    OVFCC_OP_OTHER = 0,
+    OVFCC_OP_PARAMETER = 1,
+    OVFCC_OP_CONSTANT = 2,
+    OVFCC_OP_CONVERT = 3,
+    OVFCC_OP_SUBTRACT = 4,
+    OVFCC_OP_MULTIPLY = 5,
+    OVFCC_OP_RESHAPE = 6,
+    OVFCC_OP_TRANSPOSE = 7,
+    OVFCC_OP_MATMUL = 8,          /* v0::MatMul: inputs (A, B), attributes transpose_a / transpose_b */
+    OVFCC_OP_FULLY_CONNECTED = 9, /* internal::FullyConnected: inputs (A, W [N, K], bias or -1) */
+    OVFCC_OP_ADD = 10,
+    OVFCC_OP_SWISH = 11,          /* v4::Swish with beta = 1 (one input) */
+    OVFCC_OP_GELU = 12,           /* v7::Gelu; attr = 0 erf, 1 tanh */
+    OVFCC_OP_RESULT = 13
+};
+
+/* element types beyond enum ovfcc_type that a graph may carry (bf16, i32 shape constants, ...) */
+#define OVFCC_TYPE_OTHER 7
+#define OVFCC_MAX_RANK 6
+
+/* One node, described by its first output. */
+typedef struct ovfcc_gnode {
+    int32_t op;                    /* enum ovfcc_op */
+    int32_t type;                  /* enum ovfcc_type or OVFCC_TYPE_OTHER */
+    int32_t rank;                  /* rank of the output shape, -1 when dynamic */
+    int64_t dims[OVFCC_MAX_RANK];  /* -1 = dynamic dimension */
+    int32_t n_inputs;
+    int32_t inputs[4];             /* indices into the node array; -1 = absent (FullyConnected without bias) */
+    int32_t transpose_a, transpose_b; /* MatMul */
+    int32_t attr;                  /* Gelu: 1 = tanh approximation */
+    int32_t consumers;             /* how many node inputs read this output */
+    int32_t n_ints;                /* integer Constant of at most OVFCC_MAX_RANK elements: its values (a Transpose */
+    int64_t ints[OVFCC_MAX_RANK];  /* order, a Reshape pattern); n_ints = -1 when not supplied */
+} ovfcc_gnode;
+
+/* A matched FullyConnectedCompressed node. */
+typedef struct ovfcc_fold {
+    ovfcc_fc_desc desc;       /* for ovfcc_weights_create; flags carry OVFCC_W_INPUT_MAJOR where the constants are [K, N] */
+    int32_t root;             /* node whose output the fused node produces: the MatMul / FullyConnected, or the bias Add */
+    int32_t matmul;           /* the MatMul / FullyConnected itself */
+    int32_t activations;      /* producer of X */
+    int32_t weights, scales, zero_points, bias; /* Constant nodes; -1 = absent */
+    int32_t scale_broadcast;  /* the scale Constant holds one value for the whole node: replicate it N * K/G times */
+    int32_t zp_from_real;     /* the zero-point Constant is f16 / f32: its values must be integers in 0..255 and become u8 */
+    int32_t activations_f32;  /* X is f32: the host converts to f16 */
+    /* The constants re-viewed without touching bytes (combine_groups): W as [N, K] (input-major: [K, N]), scales
+     * and zero-point table as [N, K/G] (input-major: [K/G, N]); all zero for an absent or one-element constant. */
+    int64_t w_view[2], scale_view[2], zp_view[2];
+    int32_t n_chain;          /* nodes between the weights Constant and the root that the fused node absorbs */
+    int32_t chain[16];
+} ovfcc_fold;
+
+/* Matches the subgraph that ends in `root` (a MatMul, a FullyConnected, or an Add of one of them with a Constant). */
+int ovfcc_fold_match(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_fold* out);
+
+/* How matched nodes share launches. */
+enum ovfcc_fused_kind {
+    OVFCC_FUSED_SINGLE = 0, /* one node of its own */
+    OVFCC_FUSED_CONCAT = 1, /* siblings reading the same activations, concatenated along N (ovfcc_weights_concat);
+                               part i owns the next parts[i].N output columns */
+    OVFCC_FUSED_GLU = 2     /* parts[0] = gate, parts[1] = up, glu_type applied (ovfcc_weights_glu); root = the Multiply */
+};
+typedef struct ovfcc_fused {
+    int32_t kind;
+    int32_t n_parts;
+    int32_t parts[4];  /* indices into the folds array */
+    int32_t glu_type;  /* OVFCC_GLU_SWISH | OVFCC_GLU_GELU | OVFCC_GLU_GELU_TANH */
+    int32_t root;      /* GLU: the Multiply node that the fused node's output replaces; otherwise -1 */
+} ovfcc_fused;
+
+/* Every compressed FullyConnected of the node array (bias Adds folded in where the reference's rule allows) in
+ * folds[0 .. *n_folds), and their grouping into launches in fused[0 .. *n_fused).  Every fold appears in exactly one
+ * group.  OVFCC_EINVAL when an output array is too small. */
+int ovfcc_fold_model(const ovfcc_gnode* nodes, int n_nodes, ovfcc_fold* folds, int max_folds, int* n_folds,
+                     ovfcc_fused* fused, int max_fused, int* n_fused);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OVFCC_GRAPH_H */

@@ -24,7 +24,7 @@ SYMBOLS = [
     "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
     "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_memcpy_d2d", "ovfcc_bench_copy", "ovfcc_desc_validate", "ovfcc_tiled_sizes",
     "ovfcc_repack_host", "ovfcc_unrepack_host", "ovfcc_unpack_u4", "ovfcc_unpack_i4", "ovfcc_last_error",
-    "ovfcc_version",
+    "ovfcc_version", "ovfcc_fold_match", "ovfcc_fold_model",
 ]
 
 
@@ -41,6 +41,36 @@ class FcDesc(ctypes.Structure):
         ("zp_scalar", ctypes.c_int32), ("bias_type", ctypes.c_int32), ("act_type", ctypes.c_int32),
         ("out_type", ctypes.c_int32), ("flags", ctypes.c_int32),
     ]
+
+
+MAX_RANK = 6
+TYPE_OTHER = 7
+OP = {"other": 0, "parameter": 1, "constant": 2, "convert": 3, "subtract": 4, "multiply": 5, "reshape": 6,
+      "transpose": 7, "matmul": 8, "fully_connected": 9, "add": 10, "swish": 11, "gelu": 12, "result": 13}
+FUSED_SINGLE, FUSED_CONCAT, FUSED_GLU = 0, 1, 2
+
+
+class GNode(ctypes.Structure):
+    """struct ovfcc_gnode (include/ovfcc_graph.h)"""
+    _fields_ = [("op", ctypes.c_int32), ("type", ctypes.c_int32), ("rank", ctypes.c_int32),
+                ("dims", ctypes.c_int64 * MAX_RANK), ("n_inputs", ctypes.c_int32), ("inputs", ctypes.c_int32 * 4),
+                ("transpose_a", ctypes.c_int32), ("transpose_b", ctypes.c_int32), ("attr", ctypes.c_int32),
+                ("consumers", ctypes.c_int32), ("n_ints", ctypes.c_int32), ("ints", ctypes.c_int64 * MAX_RANK)]
+
+
+class Fold(ctypes.Structure):
+    """struct ovfcc_fold"""
+    _fields_ = [("desc", FcDesc), ("root", ctypes.c_int32), ("matmul", ctypes.c_int32), ("activations", ctypes.c_int32),
+                ("weights", ctypes.c_int32), ("scales", ctypes.c_int32), ("zero_points", ctypes.c_int32),
+                ("bias", ctypes.c_int32), ("scale_broadcast", ctypes.c_int32), ("zp_from_real", ctypes.c_int32),
+                ("activations_f32", ctypes.c_int32), ("w_view", ctypes.c_int64 * 2), ("scale_view", ctypes.c_int64 * 2),
+                ("zp_view", ctypes.c_int64 * 2), ("n_chain", ctypes.c_int32), ("chain", ctypes.c_int32 * 16)]
+
+
+class Fused(ctypes.Structure):
+    """struct ovfcc_fused"""
+    _fields_ = [("kind", ctypes.c_int32), ("n_parts", ctypes.c_int32), ("parts", ctypes.c_int32 * 4),
+                ("glu_type", ctypes.c_int32), ("root", ctypes.c_int32)]
 
 
 class KernelInfo(ctypes.Structure):
@@ -112,6 +142,9 @@ def load() -> ctypes.CDLL:
         "ovfcc_unpack_i4": (ci, [vp, sz, vp]),
         "ovfcc_last_error": (ctypes.c_char_p, []),
         "ovfcc_version": (ctypes.c_char_p, []),
+        "ovfcc_fold_match": (ci, [ctypes.POINTER(GNode), ci, ci, ctypes.POINTER(Fold)]),
+        "ovfcc_fold_model": (ci, [ctypes.POINTER(GNode), ci, ctypes.POINTER(Fold), ci, ctypes.POINTER(ci),
+                                  ctypes.POINTER(Fused), ci, ctypes.POINTER(ci)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)

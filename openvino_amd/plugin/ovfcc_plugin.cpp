@@ -5,25 +5,31 @@
 //   core.register_plugin("/abs/path/libovfcc_plugin.so", "MI355X");
 //   auto compiled = core.compile_model(model, "MI355X");      // unchanged ov::Model
 //
-// What the plugin accepts: models whose Results are MatMuls (transpose_a = false) of a Parameter with a
-// weight-decompression subgraph
+// What the plugin accepts: models whose Results are produced by weight-compressed FullyConnected nodes over a
+// Parameter, each a MatMul (transpose_a = false) or internal FullyConnected with a weight-decompression subgraph
 //     Constant(u4|i4|u8|i8) -> Convert -> [Subtract(zp)] -> Multiply(scale) -> [Reshape] -> [Convert] ->
-//     [Transpose] -> [Convert] -> MatMul
+//     [Transpose] -> [Convert] -> MatMul [-> Add(bias Constant)]
 // with the constants either output-major ([N, K]: transpose_b = true, or a Transpose node under transpose_b = false)
-// or input-major ([K, N]: transpose_b = false and no Transpose node),
-// i.e. exactly what ConvertMatMulToFC + ConvertFullyConnectedToFullyConnectedCompressed fold into
+// or input-major ([K, N]: transpose_b = false and no Transpose node) -- what ConvertMatMulToFC,
+// ConvertFullyConnectedToFullyConnectedCompressed and FullyConnectedBiasFusion fold into
 // ov::op::internal::FullyConnectedCompressed on the CPU plugin
 // (src/plugins/intel_cpu/src/transformations/cpu_opset/common/pass/convert_matmul_to_fc.cpp:47-270,
-//  src/common/transformations/src/transformations/op_conversions/convert_fc_to_compressed.cpp:170-225).
-// The pattern is matched on the untouched input model, before any folding pass, so the u4/u8 constants
-// are still there and no MarkDequantization pass is needed.  Everything else is reported as unsupported by
-// query_model (a HETERO device can place it elsewhere) and rejected by compile_model.
+//  src/common/transformations/src/transformations/op_conversions/convert_fc_to_compressed.cpp:170-225,
+//  src/plugins/intel_cpu/src/transformations/cpu_opset/common/pass/fc_bias_fusion.cpp:32-93).  Two or three such nodes
+// of one format over the same Parameter run as one launch (horizontal fusion,
+// src/plugins/intel_gpu/src/plugin/transformations/fc_horizontal_fusion.cpp), and Multiply(Swish | Gelu (gate(x)), up(x))
+// runs as one node with a gated-linear-unit epilogue.  The pattern is matched on the untouched input model, before
+// any folding pass, so the u4/u8 constants are still there and no MarkDequantization pass is needed.  Everything
+// else is reported as unsupported by query_model (a HETERO device can place it elsewhere) and rejected by
+// compile_model.
 //
 // The interfaces implemented are ov::IPlugin (src/inference/dev_api/openvino/runtime/iplugin.hpp:74-255),
 // ov::ICompiledModel (icompiled_model.hpp:36-190) and ov::ISyncInferRequest (isync_infer_request.hpp:30-175);
 // the template plugin (src/plugins/template/src) is the model for which properties to answer.
 //
 // This file needs OpenVINO's developer headers and libopenvino to build; it is not part of libovfcc.so.
+#include <atomic>
+#include <chrono>
 #include <cstring>
 #include <istream>
 #include <memory>
@@ -31,27 +37,35 @@
 #include <ostream>
 #include <sstream>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "openvino/core/model.hpp"
 #include "openvino/core/type/float16.hpp"
 #include "openvino/op/constant.hpp"
+#include "openvino/op/add.hpp"
 #include "openvino/op/convert.hpp"
+#include "openvino/op/gelu.hpp"
 #include "openvino/op/matmul.hpp"
 #include "openvino/op/multiply.hpp"
 #include "openvino/op/parameter.hpp"
 #include "openvino/op/reshape.hpp"
 #include "openvino/op/result.hpp"
 #include "openvino/op/subtract.hpp"
+#include "openvino/op/swish.hpp"
 #include "openvino/op/transpose.hpp"
 #include "openvino/pass/serialize.hpp"
+#include "openvino/runtime/exec_model_info.hpp"
 #include "openvino/runtime/icompiled_model.hpp"
 #include "openvino/runtime/internal_properties.hpp"
 #include "openvino/runtime/iplugin.hpp"
 #include "openvino/runtime/isync_infer_request.hpp"
 #include "openvino/runtime/make_tensor.hpp"
 #include "openvino/runtime/properties.hpp"
+#include "ov_ops/fully_connected.hpp"
+#include "ov_ops/fully_connected_compressed.hpp"
 #include "ovfcc.h"
+#include "ovfcc_graph.h"
 
 namespace ovfcc_plugin {
 
@@ -59,217 +73,149 @@ namespace ovfcc_plugin {
     OPENVINO_THROW("ovfcc: ", what, ": ", ovfcc_last_error());
 }
 
-// ---- the decompression pattern ------------------------------------------------------------------------
+// ---- the model as plain nodes, and what the graph-side entry points make of it --------------------------
+// The decisions -- which subgraph is one FullyConnectedCompressed node, how its constants are re-viewed, which bias
+// Add folds in, which nodes share a launch -- are taken by libovfcc on a plain description of the model
+// (include/ovfcc_graph.h), where they are unit-tested without OpenVINO.  This file only translates: ov::Node ->
+// ovfcc_gnode on the way in, constant bytes -> ovfcc_weights_create on the way out.
 
-struct CompressedFc {
-    std::shared_ptr<ov::op::v0::MatMul> matmul;
-    std::shared_ptr<ov::op::v0::Parameter> activations;
-    std::shared_ptr<ov::op::v0::Constant> weights, scales, zero_points;  // zero_points may be null
-    ovfcc_fc_desc desc{};
-    std::vector<ov::float16> scales_f16;  // [N, K/G] ([K/G, N] with OVFCC_W_INPUT_MAJOR)
-    std::vector<uint8_t> zp_bytes;        // packed u4 / u8 in OpenVINO order, or one element
-};
-
-static std::shared_ptr<ov::op::v0::Constant> constant_behind_convert(const ov::Output<ov::Node>& out) {
-    auto node = out.get_node_shared_ptr();
-    if (auto cvt = ov::as_type_ptr<ov::op::v0::Convert>(node))
-        node = cvt->input_value(0).get_node_shared_ptr();
-    return ov::as_type_ptr<ov::op::v0::Constant>(node);
-}
-
-static int weight_tag(const ov::element::Type& t) {
+static int type_tag(const ov::element::Type& t) {
     if (t == ov::element::u4) return OVFCC_U4;
     if (t == ov::element::i4) return OVFCC_I4;
     if (t == ov::element::u8) return OVFCC_U8;
     if (t == ov::element::i8) return OVFCC_I8;
-    return OVFCC_NONE;
+    if (t == ov::element::f16) return OVFCC_F16;
+    if (t == ov::element::f32) return OVFCC_F32;
+    return OVFCC_TYPE_OTHER;
 }
 
-// Matches MatMul(Parameter, decompression chain) and fills the C-ABI descriptor.  Mirrors the anchors of
-// pattern::op::CompressedWeightsBlock (src/common/transformations/src/transformations/pattern_blocks/
-// compressed_weights_block.cpp:31-84) and the shape algebra of combine_groups
-// (convert_fc_to_compressed.cpp:42-78): W [N, K] or [N, K/G, G]; scale and zero-point [N, 1], [N, K/G, 1],
-// [N], [1] or []; or all of them input-major ([K, N], [K/G, G, N], [K/G, 1, N], ...) under a MatMul with
-// transpose_b = false, the form of the reference's decompression tests without transpose_weights
-// (src/tests/test_utils/common_test_utils/src/subgraph_builders/weights_decompression_builders.cpp:60-204).
-static bool match_compressed_fc(const std::shared_ptr<ov::Node>& node, CompressedFc& fc, std::string& why) {
-    auto mm = ov::as_type_ptr<ov::op::v0::MatMul>(node);
-    if (!mm)
-        return false;
-    if (mm->get_transpose_a()) {
-        why = "MatMul must have transpose_a = false";
-        return false;
-    }
-    auto param = ov::as_type_ptr<ov::op::v0::Parameter>(mm->input_value(0).get_node_shared_ptr());
-    if (!param) {
-        why = "activations must come straight from a Parameter";
-        return false;
-    }
-    // walk up from the MatMul's weight input: [Convert] <- [Transpose of the last two axes] <- [Convert] <-
-    // [Reshape] <- Multiply
-    auto w = mm->input_value(1).get_node_shared_ptr();
-    if (auto cvt = ov::as_type_ptr<ov::op::v0::Convert>(w))
-        w = cvt->input_value(0).get_node_shared_ptr();
-    bool transposed_in_graph = false;
-    if (auto tr = ov::as_type_ptr<ov::op::v1::Transpose>(w)) {
-        auto order = ov::as_type_ptr<ov::op::v0::Constant>(tr->input_value(1).get_node_shared_ptr());
-        if (!order || order->cast_vector<int64_t>() != std::vector<int64_t>{1, 0}) {
-            why = "a Transpose on the weight path must swap the two axes of a 2-D constant";
-            return false;
-        }
-        transposed_in_graph = true;
-        w = tr->input_value(0).get_node_shared_ptr();
-        if (auto cvt = ov::as_type_ptr<ov::op::v0::Convert>(w))
-            w = cvt->input_value(0).get_node_shared_ptr();
-    }
-    // The constants are output-major ([N, K], what FullyConnected wants) when exactly one of transpose_b and the
-    // Transpose node turns them; otherwise they are input-major ([K, N]) and the library transposes them once,
-    // as the Transpose that ConvertMatMulToFC inserts does in the reference (convert_matmul_to_fc.cpp:47-270).
-    const bool input_major = mm->get_transpose_b() == transposed_in_graph;
-    if (auto rs = ov::as_type_ptr<ov::op::v1::Reshape>(w))
-        w = rs->input_value(0).get_node_shared_ptr();
-    auto mul = ov::as_type_ptr<ov::op::v1::Multiply>(w);
-    if (!mul) {
-        why = "no Multiply(scale) on the weight path";
-        return false;
-    }
-    // one Multiply input is the scale constant, the other Convert(W) or Subtract(Convert(W), zp)
-    std::shared_ptr<ov::op::v0::Constant> scale;
-    ov::Output<ov::Node> body;
-    for (int side = 0; side < 2 && !scale; ++side) {
-        auto c = constant_behind_convert(mul->input_value(side));
-        if (c && c->get_element_type().is_real()) {
-            scale = c;
-            body = mul->input_value(1 - side);
-        }
-    }
-    if (!scale) {
-        why = "scale is not a floating-point constant";
-        return false;
-    }
-    std::shared_ptr<ov::op::v0::Constant> zp;
-    auto body_node = body.get_node_shared_ptr();
-    if (auto sub = ov::as_type_ptr<ov::op::v1::Subtract>(body_node)) {
-        zp = constant_behind_convert(sub->input_value(1));
-        if (!zp) {
-            why = "zero-point is not a constant";
-            return false;
-        }
-        body_node = sub->input_value(0).get_node_shared_ptr();
-    }
-    auto wcvt = ov::as_type_ptr<ov::op::v0::Convert>(body_node);
-    auto wconst = wcvt ? ov::as_type_ptr<ov::op::v0::Constant>(wcvt->input_value(0).get_node_shared_ptr()) : nullptr;
-    if (!wconst || weight_tag(wconst->get_element_type()) == OVFCC_NONE) {
-        why = "weights are not a u4/i4/u8/i8 constant behind a Convert";
-        return false;
-    }
+struct ModelGraph {
+    std::vector<std::shared_ptr<ov::Node>> ops;  // topological order; index = node id
+    std::vector<ovfcc_gnode> nodes;
+    std::vector<ovfcc_fold> folds;
+    std::vector<ovfcc_fused> fused;
+};
 
-    const auto& ws = wconst->get_shape();
-    int64_t N, K, G;
-    if (ws.size() == 2) {
-        N = (int64_t)ws[input_major ? 1 : 0];
-        K = (int64_t)ws[input_major ? 0 : 1];
-        G = K;
-    } else if (ws.size() == 3 && !input_major) {
-        N = (int64_t)ws[0];
-        K = (int64_t)(ws[1] * ws[2]);
-        G = (int64_t)ws[2];
-    } else if (ws.size() == 3) {
-        N = (int64_t)ws[2];
-        K = (int64_t)(ws[0] * ws[1]);
-        G = (int64_t)ws[1];
-    } else {
-        why = "weights must be [N, K] or [N, K/G, G] (or [K, N], [K/G, G, N] for a MatMul that does not transpose them)";
-        return false;
-    }
-    const int64_t ng = K / G;
-    const size_t scale_count = ov::shape_size(scale->get_shape());
-    if (scale_count != (size_t)(N * ng)) {
-        if (scale_count == (size_t)N && ng == 1) {
-            // per-channel [N] / [N, 1]
-        } else {
-            why = "scale must hold one value per (channel, group)";
-            return false;
+static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
+    ModelGraph g;
+    g.ops = model->get_ordered_ops();
+    std::unordered_map<const ov::Node*, int> index;
+    for (size_t i = 0; i < g.ops.size(); ++i)
+        index[g.ops[i].get()] = (int)i;
+    g.nodes.resize(g.ops.size());
+    for (size_t i = 0; i < g.ops.size(); ++i) {
+        const auto& op = g.ops[i];
+        ovfcc_gnode& n = g.nodes[i];
+        std::memset(&n, 0, sizeof(n));
+        n.n_ints = -1;
+        if (ov::is_type<ov::op::v0::Parameter>(op)) n.op = OVFCC_OP_PARAMETER;
+        else if (ov::is_type<ov::op::v0::Constant>(op)) n.op = OVFCC_OP_CONSTANT;
+        else if (ov::is_type<ov::op::v0::Convert>(op)) n.op = OVFCC_OP_CONVERT;
+        else if (ov::is_type<ov::op::v1::Subtract>(op)) n.op = OVFCC_OP_SUBTRACT;
+        else if (ov::is_type<ov::op::v1::Multiply>(op)) n.op = OVFCC_OP_MULTIPLY;
+        else if (ov::is_type<ov::op::v1::Reshape>(op)) n.op = OVFCC_OP_RESHAPE;
+        else if (ov::is_type<ov::op::v1::Transpose>(op)) n.op = OVFCC_OP_TRANSPOSE;
+        else if (ov::is_type<ov::op::v0::MatMul>(op)) n.op = OVFCC_OP_MATMUL;
+        else if (ov::is_type<ov::op::internal::FullyConnected>(op)) n.op = OVFCC_OP_FULLY_CONNECTED;
+        else if (ov::is_type<ov::op::v1::Add>(op)) n.op = OVFCC_OP_ADD;
+        else if (ov::is_type<ov::op::v4::Swish>(op)) n.op = OVFCC_OP_SWISH;
+        else if (ov::is_type<ov::op::v7::Gelu>(op)) n.op = OVFCC_OP_GELU;
+        else if (ov::is_type<ov::op::v0::Result>(op)) n.op = OVFCC_OP_RESULT;
+        else n.op = OVFCC_OP_OTHER;
+        if (op->get_output_size() == 0 || op->get_input_size() > 4) {
+            n.op = OVFCC_OP_OTHER;
+            n.rank = -1;
+            continue;
         }
-    }
-    if (mm->get_input_partial_shape(0).rbegin()->is_dynamic() ||
-        mm->get_input_partial_shape(0).rbegin()->get_length() != K) {
-        why = "last activation dimension must equal K";
-        return false;
-    }
-    const auto act_type = param->get_element_type();
-    if (act_type != ov::element::f16 && act_type != ov::element::f32) {
-        why = "activations must be f16 (or f32, converted on the host)";
-        return false;
-    }
-
-    fc.matmul = mm;
-    fc.activations = param;
-    fc.weights = wconst;
-    fc.scales = scale;
-    fc.zero_points = zp;
-    fc.desc.N = N;
-    fc.desc.K = K;
-    fc.desc.group_size = G;
-    fc.desc.w_type = weight_tag(wconst->get_element_type());
-    fc.desc.scale_type = OVFCC_F16;
-    fc.desc.bias_type = OVFCC_NONE;
-    fc.desc.act_type = OVFCC_F16;
-    fc.desc.out_type = mm->get_output_element_type(0) == ov::element::f32 ? OVFCC_F32 : OVFCC_F16;
-    fc.desc.flags = input_major ? OVFCC_W_INPUT_MAJOR : 0;
-    // scales as f16 in the constant's own order: [N, K/G], or [K/G, N] for input-major constants
-    fc.scales_f16.resize((size_t)(N * ng));
-    {
-        const auto vals = scale->cast_vector<float>();
-        for (size_t i = 0; i < fc.scales_f16.size(); ++i)
-            fc.scales_f16[i] = ov::float16(vals[i]);
-    }
-    // zero-points: u4/u8 constants are passed through untouched; real-typed ones (NNCF sometimes stores
-    // them as f16) must be integers in 0..255 and become u8
-    fc.desc.zp_type = OVFCC_NONE;
-    fc.desc.zp_scalar = 0;
-    if (zp) {
-        const size_t zc = ov::shape_size(zp->get_shape());
-        if (zc != 1 && zc != (size_t)(N * ng)) {
-            why = "zero-point must be scalar or hold one value per (channel, group)";
-            return false;
-        }
-        fc.desc.zp_scalar = zc == 1 && N * ng != 1;
-        const auto zt = zp->get_element_type();
-        if (zt == ov::element::u4 || zt == ov::element::u8) {
-            fc.desc.zp_type = zt == ov::element::u4 ? OVFCC_U4 : OVFCC_U8;
-            fc.zp_bytes.assign(static_cast<const uint8_t*>(zp->get_data_ptr()),
-                               static_cast<const uint8_t*>(zp->get_data_ptr()) + zp->get_byte_size());
+        n.type = type_tag(op->get_output_element_type(0));
+        const auto& ps = op->get_output_partial_shape(0);
+        if (ps.rank().is_dynamic() || ps.size() > OVFCC_MAX_RANK) {
+            n.rank = -1;
         } else {
-            const auto vals = zp->cast_vector<float>();
-            fc.desc.zp_type = OVFCC_U8;
-            fc.zp_bytes.resize(vals.size());
-            for (size_t i = 0; i < vals.size(); ++i) {
-                if (vals[i] < 0 || vals[i] > 255 || vals[i] != (float)(int)vals[i]) {
-                    why = "zero-point values must be integers in 0..255";
-                    return false;
-                }
-                fc.zp_bytes[i] = (uint8_t)vals[i];
+            n.rank = (int32_t)ps.size();
+            for (size_t d = 0; d < ps.size(); ++d)
+                n.dims[d] = ps[d].is_static() ? ps[d].get_length() : -1;
+        }
+        n.n_inputs = (int32_t)op->get_input_size();
+        for (size_t k = 0; k < op->get_input_size(); ++k)
+            n.inputs[k] = index.at(op->get_input_node_ptr(k));
+        n.consumers = (int32_t)op->output(0).get_target_inputs().size();
+        if (auto mm = ov::as_type_ptr<ov::op::v0::MatMul>(op)) {
+            n.transpose_a = mm->get_transpose_a();
+            n.transpose_b = mm->get_transpose_b();
+        } else if (auto gelu = ov::as_type_ptr<ov::op::v7::Gelu>(op)) {
+            n.attr = gelu->get_approximation_mode() == ov::op::GeluApproximationMode::TANH;
+        } else if (auto sw = ov::as_type_ptr<ov::op::v4::Swish>(op)) {
+            if (sw->get_input_size() != 1)
+                n.op = OVFCC_OP_OTHER;  // a beta input: not the beta = 1 form the kernels compute
+        } else if (auto c = ov::as_type_ptr<ov::op::v0::Constant>(op)) {
+            // FullyConnected's "no bias" is Constant(dynamic, Shape{0}); small integer constants carry their values
+            if (c->get_element_type().is_integral_number() && c->get_element_type().bitwidth() >= 8 &&
+                ov::shape_size(c->get_shape()) <= OVFCC_MAX_RANK) {
+                const auto vals = c->cast_vector<int64_t>();
+                n.n_ints = (int32_t)vals.size();
+                for (size_t k = 0; k < vals.size(); ++k)
+                    n.ints[k] = vals[k];
             }
         }
     }
-    if (ovfcc_desc_validate(&fc.desc) != OVFCC_OK) {
-        why = ovfcc_last_error();
-        return false;
-    }
-    return true;
+    g.folds.resize(g.nodes.size() + 1);
+    g.fused.resize(g.nodes.size() + 1);
+    int n_folds = 0, n_fused = 0;
+    if (ovfcc_fold_model(g.nodes.data(), (int)g.nodes.size(), g.folds.data(), (int)g.folds.size(), &n_folds,
+                         g.fused.data(), (int)g.fused.size(), &n_fused) != OVFCC_OK)
+        throw_last("fold_model");
+    g.folds.resize(n_folds);
+    g.fused.resize(n_fused);
+    return g;
 }
 
-// Nodes of the decompression chain of a matched MatMul (for query_model)
-static void chain_nodes(const CompressedFc& fc, std::vector<std::shared_ptr<ov::Node>>& out) {
-    std::vector<std::shared_ptr<ov::Node>> stack{fc.matmul->input_value(1).get_node_shared_ptr()};
-    while (!stack.empty()) {
-        auto n = stack.back();
-        stack.pop_back();
-        out.push_back(n);
-        for (const auto& in : n->input_values())
-            stack.push_back(in.get_node_shared_ptr());
+// Host copies of one matched node's constants in the form ovfcc_weights_create takes them.
+struct NodeData {
+    ovfcc_fc_desc desc{};
+    const void* weights = nullptr;         // the Constant's own bytes, OpenVINO order
+    std::vector<ov::float16> scales;       // [N, K/G] ([K/G, N] with OVFCC_W_INPUT_MAJOR)
+    std::vector<uint8_t> zero_points;      // packed u4 / u8, or one element
+    std::vector<ov::float16> bias;         // [N]
+};
+
+static NodeData node_data(const ModelGraph& g, const ovfcc_fold& f) {
+    NodeData d;
+    d.desc = f.desc;
+    const auto constant = [&g](int id) { return ov::as_type_ptr<ov::op::v0::Constant>(g.ops[(size_t)id]); };
+    d.weights = constant(f.weights)->get_data_ptr();
+    const size_t groups = (size_t)(f.desc.N * (f.desc.K / f.desc.group_size));
+    {
+        const auto vals = constant(f.scales)->cast_vector<float>();
+        d.scales.resize(groups);
+        OPENVINO_ASSERT(f.scale_broadcast ? vals.size() == 1 : vals.size() == groups, "MI355X: scale constant of ",
+                        vals.size(), " elements for ", groups, " groups");
+        for (size_t i = 0; i < groups; ++i)
+            d.scales[i] = ov::float16(vals[f.scale_broadcast ? 0 : i]);
     }
+    if (f.zero_points >= 0) {
+        auto zp = constant(f.zero_points);
+        if (f.zp_from_real) {
+            // real-typed zero-points (NNCF stores some so) must be integers in 0..255 and become u8
+            const auto vals = zp->cast_vector<float>();
+            d.zero_points.resize(vals.size());
+            for (size_t i = 0; i < vals.size(); ++i) {
+                OPENVINO_ASSERT(vals[i] >= 0 && vals[i] <= 255 && vals[i] == (float)(int)vals[i],
+                                "MI355X: zero-point values must be integers in 0..255");
+                d.zero_points[i] = (uint8_t)vals[i];
+            }
+        } else {
+            const auto* bytes = static_cast<const uint8_t*>(zp->get_data_ptr());
+            d.zero_points.assign(bytes, bytes + zp->get_byte_size());
+        }
+    }
+    if (f.bias >= 0) {
+        const auto vals = constant(f.bias)->cast_vector<float>();
+        d.bias.resize(vals.size());
+        for (size_t i = 0; i < vals.size(); ++i)
+            d.bias[i] = ov::float16(vals[i]);
+    }
+    return d;
 }
 
 // ---- device-resident tensors -------------------------------------------------------------------------------
@@ -412,27 +358,39 @@ private:
 
 class Plugin;
 
+// One fused node of the compiled model = one kernel launch per inference.
+struct Launch {
+    struct Output {
+        size_t result_index;    // the model output that receives ...
+        int64_t column, width;  // ... these columns of the launch's [M, N_out] rows
+    };
+    ovfcc_weights* weights = nullptr;
+    int kind = OVFCC_FUSED_SINGLE;  // enum ovfcc_fused_kind
+    size_t input_index = 0;         // the Parameter that holds X
+    int64_t K = 0, N_out = 0;
+    int out_type = OVFCC_F16;
+    std::vector<Output> outputs;    // one (the whole row), or one per horizontally fused part
+    std::string name;               // friendly name of the node the launch stands for
+    std::vector<std::string> original_names;
+    std::string primitive;          // primitiveType of the executed graph
+    std::vector<int> folds;         // indices into ModelGraph::folds
+};
+
 class CompiledModel : public ov::ICompiledModel {
 public:
-    struct Node {
-        CompressedFc fc;
-        ovfcc_weights* weights = nullptr;
-        size_t input_index = 0, output_index = 0;
-    };
-
     // node_flags: OVFCC_* flags for every node's descriptor (OVFCC_DYNQUANT_I8 when the caller allows dynamic
-    // quantisation); blobs: the repacked nodes of an exported model, in result order, instead of a fresh repack
+    // quantisation); blobs: the repacked nodes of an exported model, in launch order, instead of a fresh repack
     CompiledModel(const std::shared_ptr<ov::Model>& model, const std::shared_ptr<const ov::IPlugin>& plugin,
                   ovfcc_ctx* ctx, bool profiling, int node_flags,
                   const std::vector<std::vector<uint8_t>>* blobs = nullptr);
     ~CompiledModel() override {
-        for (auto& n : m_nodes)
-            ovfcc_weights_destroy(n.weights);
+        for (auto& l : m_launches)
+            ovfcc_weights_destroy(l.weights);
     }
 
     // Stream layout: magic, node flags, the model as the template plugin stores it (xml and constants from
     // ov::pass::Serialize, each behind its size; src/plugins/template/src/compiled_model.cpp:173-192), then the
-    // number of nodes and every node's repacked device image (ovfcc_weights_export) behind its size.
+    // number of launches and every launch's repacked device image (ovfcc_weights_export) behind its size.
     void export_model(std::ostream& out) const override {
         std::stringstream xml, bin;
         ov::pass::Serialize(xml, bin).run_on_model(m_model);
@@ -446,21 +404,57 @@ public:
         out.write(reinterpret_cast<const char*>(&flags), sizeof(flags));
         put(x.data(), x.size());
         put(b.data(), b.size());
-        const uint64_t count = m_nodes.size();
+        const uint64_t count = m_launches.size();
         out.write(reinterpret_cast<const char*>(&count), sizeof(count));
-        for (const auto& n : m_nodes) {
+        for (const auto& l : m_launches) {
             size_t bytes = 0;
-            if (ovfcc_weights_export_size(n.weights, &bytes) != OVFCC_OK)
+            if (ovfcc_weights_export_size(l.weights, &bytes) != OVFCC_OK)
                 throw_last("weights_export_size");
             std::vector<uint8_t> blob(bytes);
-            if (ovfcc_weights_export(n.weights, blob.data(), bytes) != OVFCC_OK)
+            if (ovfcc_weights_export(l.weights, blob.data(), bytes) != OVFCC_OK)
                 throw_last("weights_export");
             put(blob.data(), blob.size());
         }
     }
-    static constexpr char kExportMagic[8] = {'O', 'V', 'F', 'C', 'C', 'M', '0', '1'};
+    static constexpr char kExportMagic[8] = {'O', 'V', 'F', 'C', 'C', 'M', '0', '2'};
+
+    // The executed graph (src/inference/dev_api/openvino/runtime/exec_model_info.hpp:31-110): one node per launch
+    // with the keys the CPU plugin's executed graph carries -- layerType "FullyConnected", primitiveType,
+    // originalLayersNames, outputPrecisions, outputLayouts, execOrder and execTimeMcs (the last measured time of the
+    // launch, or "not_executed").  A node that stands for one unfused FullyConnected whose constants are
+    // output-major is an ov::op::internal::FullyConnectedCompressed over the model's own constants, re-viewed as
+    // ConvertFullyConnectedToFullyConnectedCompressed re-views them; fused nodes are ExecutionNodes.
     std::shared_ptr<const ov::Model> get_runtime_model() const override {
-        return m_model;
+        ov::ParameterVector params;
+        for (const auto& p : m_model->get_parameters())
+            params.push_back(std::make_shared<ov::op::v0::Parameter>(p->get_element_type(), p->get_partial_shape()));
+        ov::ResultVector results(m_model->get_results().size());
+        for (size_t i = 0; i < m_launches.size(); ++i) {
+            const Launch& l = m_launches[i];
+            std::shared_ptr<ov::Node> node;
+            if (l.kind == OVFCC_FUSED_SINGLE && !(m_graph.folds[(size_t)l.folds[0]].desc.flags & OVFCC_W_INPUT_MAJOR))
+                node = compressed_node(m_graph.folds[(size_t)l.folds[0]], params[l.input_index]);
+            else
+                node = std::make_shared<ov::exec_model_info::ExecutionNode>(ov::OutputVector{params[l.input_index]}, 1);
+            node->set_friendly_name(l.name);
+            auto& rt = node->get_rt_info();
+            std::string names;
+            for (const auto& n : l.original_names)
+                names += (names.empty() ? "" : ",") + n;
+            rt[ov::exec_model_info::LAYER_TYPE] = std::string("FullyConnected");
+            rt[ov::exec_model_info::IMPL_TYPE] = l.primitive;
+            rt[ov::exec_model_info::ORIGINAL_NAMES] = names;
+            rt[ov::exec_model_info::OUTPUT_PRECISIONS] = std::string(l.out_type == OVFCC_F32 ? "f32" : "f16");
+            rt[ov::exec_model_info::OUTPUT_LAYOUTS] = std::string("ab");
+            rt[ov::exec_model_info::EXECUTION_ORDER] = std::to_string(i);
+            const double us = m_last_us[i].load();
+            rt[ov::exec_model_info::PERF_COUNTER] = us < 0 ? std::string("not_executed") : std::to_string((long long)us);
+            for (const auto& o : l.outputs) {
+                results[o.result_index] = std::make_shared<ov::op::v0::Result>(node);
+                results[o.result_index]->set_friendly_name(m_model->get_results()[o.result_index]->get_friendly_name());
+            }
+        }
+        return std::make_shared<ov::Model>(results, params, m_model->get_friendly_name() + "_executed");
     }
     void set_property(const ov::AnyMap&) override {
         OPENVINO_THROW_NOT_IMPLEMENTED("MI355X: compiled model has no mutable properties");
@@ -482,16 +476,40 @@ public:
     }
     std::shared_ptr<ov::ISyncInferRequest> create_sync_infer_request() const override;
 
-    const std::vector<Node>& nodes() const {
-        return m_nodes;
+    const std::vector<Launch>& launches() const {
+        return m_launches;
     }
     ovfcc_ctx* ctx() const {
         return m_ctx;
     }
+    void record_time(size_t launch, double us) const {
+        m_last_us[launch].store(us);
+    }
 
 private:
+    // FullyConnectedCompressed over the fold's own constants (output-major), for the executed graph
+    std::shared_ptr<ov::Node> compressed_node(const ovfcc_fold& f, const ov::Output<ov::Node>& x) const {
+        const auto constant = [this](int id) { return ov::as_type_ptr<ov::op::v0::Constant>(m_graph.ops[(size_t)id]); };
+        const auto view = [](const std::shared_ptr<ov::op::v0::Constant>& c, const int64_t v[2]) {
+            return v[0] == 0 ? c : std::make_shared<ov::op::v0::Constant>(*c, ov::Shape{(size_t)v[0], (size_t)v[1]});
+        };
+        std::shared_ptr<ov::Node> bias = f.bias >= 0
+                                             ? std::static_pointer_cast<ov::Node>(constant(f.bias))
+                                             : std::make_shared<ov::op::v0::Constant>(ov::element::dynamic, ov::Shape{0});
+        const auto out_type = f.desc.out_type == OVFCC_F32 ? ov::element::f32 : ov::element::f16;
+        auto w = view(constant(f.weights), f.w_view);
+        auto s = view(constant(f.scales), f.scale_view);
+        if (f.zero_points >= 0)
+            return std::make_shared<ov::op::internal::FullyConnectedCompressed>(x, w, bias, s,
+                                                                                 view(constant(f.zero_points), f.zp_view),
+                                                                                 out_type);
+        return std::make_shared<ov::op::internal::FullyConnectedCompressed>(x, w, bias, s, out_type);
+    }
+
     std::shared_ptr<ov::Model> m_model;
-    std::vector<Node> m_nodes;
+    ModelGraph m_graph;
+    std::vector<Launch> m_launches;
+    mutable std::vector<std::atomic<double>> m_last_us;  // per launch: last measured time, -1 before the first run
     ovfcc_ctx* m_ctx;
     int m_node_flags = 0;
     bool m_profiling;
@@ -525,51 +543,77 @@ public:
     void infer() override {
         check_tensors();
         m_kernels.clear();
-        for (const auto& node : m_compiled->nodes()) {
-            auto in = get_tensor(get_inputs()[node.input_index]);
-            auto out = get_tensor(get_outputs()[node.output_index]);
+        m_times_us.clear();
+        const auto& launches = m_compiled->launches();
+        for (size_t li = 0; li < launches.size(); ++li) {
+            const Launch& l = launches[li];
+            const auto t0 = std::chrono::steady_clock::now();
+            auto in = get_tensor(get_inputs()[l.input_index]);
             const ov::Shape in_shape = in->get_shape();
             int64_t M = 1;  // 3-D activations flatten to [B*S, K] like the CPU path does
             for (size_t d = 0; d + 1 < in_shape.size(); ++d)
                 M *= (int64_t)in_shape[d];
-            ov::Shape out_shape = in_shape;
-            out_shape.back() = (size_t)node.fc.desc.N;
-            out->set_shape(out_shape);  // dynamic M: the output follows the input
+            std::vector<ov::SoPtr<ov::ITensor>> outs;
+            for (const auto& o : l.outputs) {
+                auto out = get_tensor(get_outputs()[o.result_index]);
+                ov::Shape out_shape = in_shape;
+                out_shape.back() = (size_t)o.width;
+                out->set_shape(out_shape);  // dynamic M: the output follows the input
+                outs.push_back(out);
+            }
+            const size_t out_el = l.out_type == OVFCC_F32 ? 4 : 2;
             auto rin = std::dynamic_pointer_cast<RemoteTensor>(in._ptr);
-            auto rout = std::dynamic_pointer_cast<RemoteTensor>(out._ptr);
+            auto rout = l.outputs.size() == 1 ? std::dynamic_pointer_cast<RemoteTensor>(outs[0]._ptr) : nullptr;
+            for (const auto& out : outs)
+                OPENVINO_ASSERT(l.outputs.size() == 1 || !std::dynamic_pointer_cast<RemoteTensor>(out._ptr),
+                                "MI355X: the outputs of a horizontally fused node must be host tensors");
             if (rin || rout) {
                 // Device-resident tensors: no copy on their side.  A host tensor on the other side goes through a
                 // device buffer of the request.
                 OPENVINO_ASSERT(in->get_element_type() == ov::element::f16,
                                 "MI355X: a device-resident input must be f16, got ", in->get_element_type());
-                const size_t x_bytes = (size_t)M * node.fc.desc.K * sizeof(ov::float16);
-                const size_t y_bytes = out->get_byte_size();
+                const size_t x_bytes = (size_t)M * l.K * sizeof(ov::float16);
+                const size_t y_bytes = (size_t)M * l.N_out * out_el;
                 void* x_dev = rin ? rin->device_ptr() : device_staging(0, x_bytes);
                 void* y_dev = rout ? rout->device_ptr() : device_staging(1, y_bytes);
                 if (!rin && x_bytes && ovfcc_memcpy_h2d(m_compiled->ctx(), x_dev, in->data(), x_bytes) != OVFCC_OK)
                     throw_last("memcpy_h2d");
-                if (ovfcc_fc_run_device(m_request, node.weights, x_dev, y_dev, M) != OVFCC_OK)
+                if (ovfcc_fc_run_device(m_request, l.weights, x_dev, y_dev, M) != OVFCC_OK)
                     throw_last("fc_run_device");
                 if (ovfcc_request_sync(m_request) != OVFCC_OK)
                     throw_last("request_sync");
-                if (!rout && y_bytes && ovfcc_memcpy_d2h(m_compiled->ctx(), out->data(), y_dev, y_bytes) != OVFCC_OK)
-                    throw_last("memcpy_d2h");
+                if (!rout) {
+                    m_y_staging.resize(y_bytes);
+                    if (y_bytes && ovfcc_memcpy_d2h(m_compiled->ctx(), m_y_staging.data(), y_dev, y_bytes) != OVFCC_OK)
+                        throw_last("memcpy_d2h");
+                    scatter_columns(l, outs, M, out_el);
+                }
             } else {
                 const void* x = in->data();
                 if (in->get_element_type() == ov::element::f32) {
                     // the device path computes on f16 activations
                     const float* src = static_cast<const float*>(in->data());
-                    m_staging.resize((size_t)M * node.fc.desc.K);
+                    m_staging.resize((size_t)M * l.K);
                     for (size_t i = 0; i < m_staging.size(); ++i)
                         m_staging[i] = ov::float16(src[i]);
                     x = m_staging.data();
                 }
-                if (ovfcc_fc_run(m_request, node.weights, x, out->data(), M) != OVFCC_OK)
-                    throw_last("fc_run");
+                if (l.outputs.size() == 1) {
+                    if (ovfcc_fc_run(m_request, l.weights, x, outs[0]->data(), M) != OVFCC_OK)
+                        throw_last("fc_run");
+                } else {
+                    m_y_staging.resize((size_t)M * l.N_out * out_el);
+                    if (ovfcc_fc_run(m_request, l.weights, x, m_y_staging.data(), M) != OVFCC_OK)
+                        throw_last("fc_run");
+                    scatter_columns(l, outs, M, out_el);
+                }
             }
             ovfcc_kernel_info info;
             ovfcc_last_kernel_info(m_request, &info);
             m_kernels.push_back(info);
+            const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+            m_times_us.push_back(us);
+            m_compiled->record_time(li, us);
         }
     }
 
@@ -578,9 +622,10 @@ public:
         for (size_t i = 0; i < m_kernels.size(); ++i) {
             ov::ProfilingInfo p;
             p.status = ov::ProfilingInfo::Status::EXECUTED;
-            p.node_name = m_compiled->nodes()[i].fc.matmul->get_friendly_name();
+            p.node_name = m_compiled->launches()[i].name;
             p.node_type = "FullyConnected";
             p.exec_type = m_kernels[i].name;
+            p.real_time = p.cpu_time = std::chrono::microseconds((long long)m_times_us[i]);
             out.push_back(p);
         }
         return out;
@@ -596,6 +641,17 @@ private:
             tensor = ov::make_tensor(type, shape);
         else
             tensor->set_shape(shape);
+    }
+
+    // rows of m_y_staging ([M, N_out]) -> every output's columns (the VariadicSplit after a horizontally fused node)
+    void scatter_columns(const Launch& l, const std::vector<ov::SoPtr<ov::ITensor>>& outs, int64_t M, size_t el) {
+        for (size_t k = 0; k < l.outputs.size(); ++k) {
+            const auto& o = l.outputs[k];
+            auto* dst = static_cast<uint8_t*>(outs[k]->data());
+            for (int64_t m = 0; m < M; ++m)
+                std::memcpy(dst + (size_t)m * o.width * el,
+                            m_y_staging.data() + ((size_t)m * l.N_out + (size_t)o.column) * el, (size_t)o.width * el);
+        }
     }
 
     // device buffer `which` (0 = activations, 1 = outputs) of at least `bytes`, kept and grown across calls
@@ -620,7 +676,9 @@ private:
     ovfcc_request* m_request = nullptr;
     DeviceBuffer m_device_staging[2];
     std::vector<ov::float16> m_staging;
+    std::vector<uint8_t> m_y_staging;
     std::vector<ovfcc_kernel_info> m_kernels;
+    std::vector<double> m_times_us;
 };
 
 class Plugin : public ov::IPlugin {
@@ -782,23 +840,39 @@ public:
         return import_model(blob, properties);
     }
 
-    // Supported: each matched MatMul with its whole decompression chain, and the Parameter / Result around it.
+    // Supported: every matched node with its whole decompression chain (bias Add, gate activation and the Multiply
+    // of a gated linear unit included), and the Parameter / Results around it.
     ov::SupportedOpsMap query_model(const std::shared_ptr<const ov::Model>& model, const ov::AnyMap&) const override {
         ov::SupportedOpsMap res;
-        for (const auto& node : model->get_ordered_ops()) {
-            CompressedFc fc;
-            std::string why;
-            if (!match_compressed_fc(node, fc, why))
-                continue;
-            std::vector<std::shared_ptr<ov::Node>> nodes;
-            chain_nodes(fc, nodes);
-            nodes.push_back(fc.matmul);
-            nodes.push_back(fc.activations);
-            for (const auto& user : fc.matmul->output(0).get_target_inputs())
+        const ModelGraph g = describe(model);
+        auto mark = [&](int id) {
+            if (id >= 0)
+                res[g.ops[(size_t)id]->get_friendly_name()] = get_device_name();
+        };
+        auto mark_results_of = [&](int id) {
+            for (const auto& user : g.ops[(size_t)id]->output(0).get_target_inputs())
                 if (ov::is_type<ov::op::v0::Result>(user.get_node()))
-                    nodes.push_back(user.get_node()->shared_from_this());
-            for (const auto& n : nodes)
-                res[n->get_friendly_name()] = get_device_name();
+                    res[user.get_node()->get_friendly_name()] = get_device_name();
+        };
+        for (const auto& u : g.fused) {
+            for (int k = 0; k < u.n_parts; ++k) {
+                const ovfcc_fold& f = g.folds[(size_t)u.parts[k]];
+                for (int c = 0; c < f.n_chain; ++c)
+                    mark(f.chain[c]);
+                mark(f.matmul);
+                mark(f.root);
+                if (g.nodes[(size_t)f.activations].op == OVFCC_OP_PARAMETER)
+                    mark(f.activations);
+                if (u.kind != OVFCC_FUSED_GLU)
+                    mark_results_of(f.root);
+            }
+            if (u.kind == OVFCC_FUSED_GLU) {
+                mark(u.root);
+                for (const auto& in : g.ops[(size_t)u.root]->input_values())  // the gate's activation node
+                    if (ov::is_type<ov::op::v4::Swish>(in.get_node()) || ov::is_type<ov::op::v7::Gelu>(in.get_node()))
+                        res[in.get_node()->get_friendly_name()] = get_device_name();
+                mark_results_of(u.root);
+            }
         }
         return res;
     }
@@ -827,43 +901,137 @@ private:
 CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std::shared_ptr<const ov::IPlugin>& plugin,
                              ovfcc_ctx* ctx, bool profiling, int node_flags,
                              const std::vector<std::vector<uint8_t>>* blobs)
-    : ov::ICompiledModel(model, plugin), m_model(model), m_ctx(ctx), m_node_flags(node_flags), m_profiling(profiling) {
-    if (blobs && blobs->size() != model->get_results().size())
-        OPENVINO_THROW("MI355X: the imported blob holds ", blobs->size(), " nodes, the model ", model->get_results().size());
-    // every Result must be fed by a matched MatMul; every Parameter must feed one
+    : ov::ICompiledModel(model, plugin), m_model(model), m_graph(describe(model)), m_ctx(ctx), m_node_flags(node_flags),
+      m_profiling(profiling) {
+    const ModelGraph& g = m_graph;
     const auto& results = model->get_results();
     const auto& params = model->get_parameters();
-    for (size_t r = 0; r < results.size(); ++r) {
-        Node n;
-        std::string why = "not a MatMul";
-        auto producer = results[r]->input_value(0).get_node_shared_ptr();
-        if (!match_compressed_fc(producer, n.fc, why))
-            OPENVINO_THROW("MI355X: result ", results[r]->get_friendly_name(),
-                           " is not produced by a weight-compressed FullyConnected: ", why,
-                           " (use HETERO:MI355X,CPU for the rest of the graph)");
-        n.output_index = r;
+    std::vector<bool> fed(results.size(), false);
+    // the model outputs that read node `id`
+    auto results_of = [&](int id) {
+        std::vector<size_t> out;
+        for (size_t r = 0; r < results.size(); ++r)
+            if (results[r]->get_input_node_ptr(0) == g.ops[(size_t)id].get())
+                out.push_back(r);
+        return out;
+    };
+    auto create = [&](const ovfcc_fold& f) {
+        NodeData d = node_data(g, f);
+        d.desc.flags |= node_flags;
+        ovfcc_weights* w = nullptr;
+        if (ovfcc_weights_create(ctx, &d.desc, d.weights, d.scales.data(), d.zero_points.empty() ? nullptr : d.zero_points.data(),
+                                 d.bias.empty() ? nullptr : d.bias.data(), &w) != OVFCC_OK)
+            throw_last("weights_create");
+        return w;
+    };
+    auto primitive = [](const ovfcc_weights* w, const ovfcc_fc_desc& d, const char* suffix) {
+        return std::string(ovfcc_weights_is_tiled(w) ? "hip_tiled_w" : "hip_plain_w") +
+               (d.w_type == OVFCC_U8 || d.w_type == OVFCC_I8 ? "8" : "4") + suffix;
+    };
+    auto start_launch = [&](const ovfcc_fold& f, int kind) {
+        Launch l;
+        l.kind = kind;
+        l.K = f.desc.K;
+        l.out_type = f.desc.out_type;
+        OPENVINO_ASSERT(g.nodes[(size_t)f.activations].op == OVFCC_OP_PARAMETER, "MI355X: the activations of ",
+                        g.ops[(size_t)f.matmul]->get_friendly_name(),
+                        " do not come straight from a Parameter (use HETERO:MI355X,CPU for the rest of the graph)");
         for (size_t p = 0; p < params.size(); ++p)
-            if (params[p] == n.fc.activations)
-                n.input_index = p;
-        n.fc.desc.flags |= node_flags;
-        if (blobs) {
-            // the cached device image; the library checks it against its own descriptor
-            if (ovfcc_weights_import(ctx, (*blobs)[r].data(), (*blobs)[r].size(), &n.weights) != OVFCC_OK)
-                throw_last("weights_import");
-        } else {
-            const void* zp = n.fc.zp_bytes.empty() ? nullptr : n.fc.zp_bytes.data();
-            if (ovfcc_weights_create(ctx, &n.fc.desc, n.fc.weights->get_data_ptr(), n.fc.scales_f16.data(), zp,
-                                     nullptr, &n.weights) != OVFCC_OK)
-                throw_last("weights_create");
+            if (params[p].get() == g.ops[(size_t)f.activations].get())
+                l.input_index = p;
+        return l;
+    };
+    auto add_outputs = [&](Launch& l, int root, int64_t column, int64_t width) {
+        const auto rs = results_of(root);
+        OPENVINO_ASSERT(!rs.empty(), "MI355X: ", g.ops[(size_t)root]->get_friendly_name(),
+                        " feeds no model output (use HETERO:MI355X,CPU for the rest of the graph)");
+        for (size_t r : rs) {
+            l.outputs.push_back({r, column, width});
+            fed[r] = true;
         }
-        // the executed graph shows the same layer type the CPU plugin shows
-        // (src/inference/dev_api/openvino/runtime/exec_model_info.hpp:31-73)
-        n.fc.matmul->get_rt_info()["layerType"] = std::string("FullyConnected");
-        n.fc.matmul->get_rt_info()["primitiveType"] =
-            std::string(ovfcc_weights_is_tiled(n.weights) ? "hip_tiled_w" : "hip_plain_w") +
-            (n.fc.desc.w_type == OVFCC_U8 || n.fc.desc.w_type == OVFCC_I8 ? "8" : "4");
-        m_nodes.push_back(std::move(n));
+    };
+    for (const auto& u : g.fused) {
+        const ovfcc_fold& f0 = g.folds[(size_t)u.parts[0]];
+        if (u.kind == OVFCC_FUSED_GLU) {
+            Launch l = start_launch(f0, u.kind);
+            l.N_out = f0.desc.N;
+            l.name = g.ops[(size_t)u.root]->get_friendly_name();
+            l.folds = {u.parts[0], u.parts[1]};
+            add_outputs(l, u.root, 0, l.N_out);
+            if (!blobs) {
+                ovfcc_weights *gate = create(f0), *up = create(g.folds[(size_t)u.parts[1]]);
+                const int rc = ovfcc_weights_glu(gate, up, u.glu_type, &l.weights);
+                ovfcc_weights_destroy(gate);
+                ovfcc_weights_destroy(up);
+                if (rc != OVFCC_OK)
+                    throw_last("weights_glu");
+            }
+            for (int k = 0; k < 2; ++k)
+                l.original_names.push_back(g.ops[(size_t)g.folds[(size_t)u.parts[k]].matmul]->get_friendly_name());
+            l.original_names.push_back(l.name);
+            m_launches.push_back(std::move(l));
+            continue;
+        }
+        // horizontally fused siblings share a launch when the library can concatenate them (equal scalar
+        // zero-points included); otherwise, like single nodes, each gets its own
+        ovfcc_weights* fused_w = nullptr;
+        std::vector<ovfcc_weights*> parts;
+        if (!blobs)
+            for (int k = 0; k < u.n_parts; ++k)
+                parts.push_back(create(g.folds[(size_t)u.parts[k]]));
+        bool together = u.kind == OVFCC_FUSED_CONCAT;
+        if (together && !blobs)
+            together = ovfcc_weights_concat(parts.data(), (int)parts.size(), &fused_w) == OVFCC_OK;
+        if (together) {
+            Launch l = start_launch(f0, OVFCC_FUSED_CONCAT);
+            int64_t column = 0;
+            for (int k = 0; k < u.n_parts; ++k) {
+                const ovfcc_fold& f = g.folds[(size_t)u.parts[k]];
+                add_outputs(l, f.root, column, f.desc.N);
+                column += f.desc.N;
+                l.folds.push_back(u.parts[k]);
+                l.original_names.push_back(g.ops[(size_t)f.root]->get_friendly_name());
+                l.name += (k ? "+" : "") + g.ops[(size_t)f.root]->get_friendly_name();
+            }
+            l.N_out = column;
+            l.weights = fused_w;
+            for (auto* w : parts)
+                ovfcc_weights_destroy(w);
+            m_launches.push_back(std::move(l));
+        } else {
+            for (int k = 0; k < u.n_parts; ++k) {
+                const ovfcc_fold& f = g.folds[(size_t)u.parts[k]];
+                Launch l = start_launch(f, OVFCC_FUSED_SINGLE);
+                l.N_out = f.desc.N;
+                l.name = g.ops[(size_t)f.root]->get_friendly_name();
+                l.folds = {u.parts[k]};
+                l.original_names.push_back(g.ops[(size_t)f.matmul]->get_friendly_name());
+                if (f.root != f.matmul)
+                    l.original_names.push_back(l.name);
+                add_outputs(l, f.root, 0, l.N_out);
+                l.weights = blobs ? nullptr : parts[(size_t)k];
+                m_launches.push_back(std::move(l));
+            }
+        }
     }
+    for (size_t r = 0; r < results.size(); ++r)
+        OPENVINO_ASSERT(fed[r], "MI355X: result ", results[r]->get_friendly_name(),
+                        " is not produced by a weight-compressed FullyConnected (use HETERO:MI355X,CPU for the rest "
+                        "of the graph)");
+    if (blobs) {
+        // the cached device images, one per launch in this order; the library checks each against its own descriptor
+        OPENVINO_ASSERT(blobs->size() == m_launches.size(), "MI355X: the imported blob holds ", blobs->size(),
+                        " nodes, the model compiles to ", m_launches.size());
+        for (size_t i = 0; i < m_launches.size(); ++i)
+            if (ovfcc_weights_import(ctx, (*blobs)[i].data(), (*blobs)[i].size(), &m_launches[i].weights) != OVFCC_OK)
+                throw_last("weights_import");
+    }
+    for (auto& l : m_launches)
+        l.primitive = primitive(l.weights, g.folds[(size_t)l.folds[0]].desc,
+                                l.kind == OVFCC_FUSED_GLU ? "_glu" : (l.kind == OVFCC_FUSED_CONCAT ? "_fused" : ""));
+    m_last_us = std::vector<std::atomic<double>>(m_launches.size());
+    for (auto& t : m_last_us)
+        t.store(-1.0);
 }
 
 std::shared_ptr<ov::ISyncInferRequest> CompiledModel::create_sync_infer_request() const {

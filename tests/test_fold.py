@@ -1,0 +1,312 @@
+"""The graph-side half of the path on plain node arrays (include/ovfcc_graph.h): the MatMul -> FullyConnected ->
+FullyConnectedCompressed fold with its shape algebra, the bias fusion rule, horizontal fusion and the gated linear
+unit -- driven by the structural cases of the reference's own tests (tests/golden/fold_cases.json) and by negative
+cases for every rule.  No GPU, no OpenVINO."""
+import json
+import os
+
+import pytest
+
+from openvino_amd import _lib, fc
+from openvino_amd.graph import Graph, decompression_subgraph
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "fold_cases.json")) as fh:
+    CASES = json.load(fh)
+
+
+def ids(rows, keys):
+    return ["-".join(str(r[k]) for k in keys) for r in rows]
+
+
+@pytest.mark.parametrize("p", CASES["convert_fc_to_compressed"],
+                         ids=ids(CASES["convert_fc_to_compressed"], ("type", "with_zp", "grouped", "wei_shape")))
+@pytest.mark.parametrize("root_op", ["fully_connected", "matmul"])
+def test_reference_fold_cases(p, root_op):
+    """The twelve rows of ConvertFCToCompressed: a FullyConnected (or the MatMul with transpose_b = true it came
+    from) over Constant -> Convert -> [Subtract(Convert(zp))] -> Multiply(scale) -> [Reshape].  Expected, as in the
+    reference's model_ref: weights re-viewed as [OC, IC], scale / zero-point as the scale shape without its last
+    axis, zero-point present iff with_zp, no bias."""
+    g = Graph()
+    x = g.parameter("f32", p["in_shape"])
+    wshape, sshape = p["wei_shape"], p["scale_zp_shape"]
+    OC, IC = wshape[0], (wshape[1] * wshape[2] if p["grouped"] else wshape[1])
+    chain = decompression_subgraph(g, p["type"], wshape, sshape, sshape if p["with_zp"] else None, p["type"],
+                                   reshape_to=[OC, IC] if p["grouped"] else None)
+    root = g.fully_connected(x, chain) if root_op == "fully_connected" else g.matmul(x, chain, transpose_b=True)
+    f = g.fold_match(root)
+    d = f.desc
+    assert (d.N, d.K) == (OC, IC)
+    assert d.group_size == (wshape[2] if p["grouped"] else IC)
+    assert d.w_type == _lib.TYPE[p["type"]] and d.flags == 0 and d.bias_type == _lib.NONE and d.out_type == _lib.F32
+    assert d.zp_type == (_lib.TYPE[p["type"]] if p["with_zp"] else _lib.NONE) and d.zp_scalar == 0
+    assert list(f.w_view) == [OC, IC]
+    expect_view = sshape[:-1] if p["grouped"] else sshape          # the reference pops the trailing 1 of grouped shapes
+    assert list(f.scale_view) == expect_view + ([1] if len(expect_view) == 1 else [])
+    assert list(f.zp_view) == (list(f.scale_view) if p["with_zp"] else [0, 0])
+    assert f.root == root and f.matmul == root and f.activations == x and f.bias == -1
+    assert g.nodes[f.weights].op == _lib.OP["constant"] and g.shape(f.weights) == wshape
+    assert g.shape(f.scales) == sshape and f.scale_broadcast == 0 and f.activations_f32 == 1
+    assert (f.zero_points >= 0) == p["with_zp"]
+    # everything between the constants and the root is absorbed: Convert, [zp, Convert, Subtract], scale, Multiply,
+    # [Reshape + pattern], weights
+    assert f.n_chain == 4 + (3 if p["with_zp"] else 0) + (2 if p["grouped"] else 0)
+    assert _lib.load().ovfcc_desc_validate(d) == _lib.OK
+
+
+@pytest.mark.parametrize("p", CASES["transposed_constants"], ids=[p["name"] for p in CASES["transposed_constants"]])
+def test_reference_rank1_and_rank0_constants_under_a_transpose(p):
+    """[IC, OC] weights with rank-1 (per output channel) or rank-0 (per tensor) scale and zero-point and a
+    Transpose([1, 0]) above the Multiply.  The reference keeps the weights Constant in its [IC, OC] layout behind
+    the Transpose, promotes rank-1 constants to [OC, 1] and leaves rank-0 ones alone; here the node is marked
+    input-major (the library transposes once at creation) with the same per-channel meaning."""
+    g = Graph()
+    x = g.parameter("f32", p["in_shape"])
+    chain = decompression_subgraph(g, p["type"], p["wei_shape"], p["scale_zp_shape"], p["scale_zp_shape"], p["type"],
+                                   transpose=True)
+    root = g.fully_connected(x, chain)
+    f = g.fold_match(root)
+    e = p["expect"]
+    assert (f.desc.N, f.desc.K, f.desc.group_size) == (e["N"], e["K"], e["G"])
+    assert f.desc.flags == _lib.W_INPUT_MAJOR and list(f.w_view) == p["wei_shape"]
+    assert f.desc.zp_scalar == e["zp_scalar"] and f.scale_broadcast == e["scale_broadcast"]
+    assert list(f.scale_view) == ([1, e["N"]] if not e["scale_broadcast"] else [0, 0])
+    assert list(f.zp_view) == ([1, e["N"]] if not e["zp_scalar"] else [0, 0])
+    assert g.shape(f.scales) == p["scale_zp_shape"]
+
+
+@pytest.mark.parametrize("p", CASES["builders"], ids=ids(CASES["builders"], ("type", "weights_shape", "group", "transpose_weights", "zp")))
+def test_reference_builder_shapes(p):
+    """Subgraphs as initMatMulDecompressionSubgraph emits them: weights_shape = [IC, OC]; with transpose_weights the
+    constants are stored [OC, IC] ([OC, IC/G, G], scales [OC, IC/G, 1]) and a Transpose node follows, without it they
+    are [IC, OC] ([IC/G, G, OC], scales [IC/G, 1, OC]); the MatMul never transposes."""
+    IC, OC = p["weights_shape"]
+    G = p["group"] if p["group"] != -1 else IC
+    grouped = p["group"] != -1
+    tw = p["transpose_weights"]
+    if tw:
+        wshape = [OC, IC // G, G] if grouped else [OC, IC]
+        sshape = [OC, IC // G, 1] if grouped else [OC, 1]
+        reshape_to = [OC, IC] if grouped else None
+    else:
+        wshape = [IC // G, G, OC] if grouped else [IC, OC]
+        sshape = [IC // G, 1, OC] if grouped else [1, OC]
+        reshape_to = [IC, OC] if grouped else None
+    zp_shape = None if p["zp"] == "empty" else (sshape if p["zp"] == "full" else [])
+    squeezed = [d for d in sshape if d != 1] if p.get("reshape_on_decompression") else None
+    g = Graph()
+    x = g.parameter("f16", [-1, -1, IC])
+    chain = decompression_subgraph(g, p["type"], wshape, sshape, zp_shape, p["type"], scale_type="f16", compute_type="f16",
+                                   reshape_to=reshape_to, transpose=tw, scale_const_shape=squeezed)
+    root = g.matmul(x, chain)
+    f = g.fold_match(root)
+    d = f.desc
+    assert (d.N, d.K, d.group_size) == (OC, IC, G)
+    assert d.flags == (0 if tw else _lib.W_INPUT_MAJOR)
+    assert list(f.w_view) == ([OC, IC] if tw else [IC, OC])
+    assert list(f.scale_view) == ([OC, IC // G] if tw else [IC // G, OC])
+    assert d.zp_scalar == int(p["zp"] == "scalar" and OC * (IC // G) != 1)
+    assert d.zp_type == (_lib.NONE if p["zp"] == "empty" else _lib.TYPE[p["type"]])
+    assert d.out_type == _lib.F16 and f.activations_f32 == 0
+
+
+def _simple(g, x, N=64, K=256, G=128, w_type="u4", zp=True, major="output", scale_type="f16", out=None):
+    ng = K // G
+    if major == "output":
+        chain = decompression_subgraph(g, w_type, [N, ng, G], [N, ng, 1], [N, ng, 1] if zp else None, w_type,
+                                       scale_type=scale_type, compute_type="f16", reshape_to=[N, K])
+        return g.matmul(x, chain, transpose_b=True, type_=out)
+    chain = decompression_subgraph(g, w_type, [ng, G, N], [ng, 1, N], [ng, 1, N] if zp else None, w_type,
+                                   scale_type=scale_type, compute_type="f16", reshape_to=[K, N])
+    return g.matmul(x, chain, type_=out)
+
+
+def test_bias_add_folds_in_by_the_reference_rule():
+    """FullyConnectedBiasFusion: Add(FC, Constant) folds when the constant's last dimension is N, every other one is
+    1 and the FC has no other consumer."""
+    for shape, ok in (([64], True), ([1, 64], True), ([1, 1, 64], True), ([2, 64], False), ([64, 1], False), ([], False),
+                      ([1], False)):
+        g = Graph()
+        x = g.parameter("f16", [-1, 256])
+        mm = _simple(g, x)
+        add = g.add(mm, g.constant("f16", shape))
+        if ok:
+            f = g.fold_match(add)
+            assert f.root == add and f.matmul == mm and f.desc.bias_type == _lib.F16 and g.shape(f.bias) == shape
+        else:
+            with pytest.raises(fc.OvfccError):
+                g.fold_match(add)
+    # constant first, MatMul second: Add is commutative
+    g = Graph()
+    x = g.parameter("f16", [4, 256])
+    mm = _simple(g, x)
+    add = g.add(g.constant("f32", [64]), mm)
+    assert g.fold_match(add).bias >= 0
+    # a second consumer of the MatMul keeps the Add outside
+    g = Graph()
+    x = g.parameter("f16", [4, 256])
+    mm = _simple(g, x)
+    add = g.add(mm, g.constant("f16", [64]))
+    g.result(mm)
+    with pytest.raises(fc.OvfccError, match="only consumer"):
+        g.fold_match(add)
+    folds, fused = g.fold_model()
+    assert len(folds) == 1 and folds[0].root == mm and folds[0].bias == -1
+    # FullyConnected with its own bias input; an Add above it is then not folded
+    g = Graph()
+    x = g.parameter("f16", [4, 256])
+    chain = decompression_subgraph(g, "u8", [64, 256], [64, 1], scale_type="f16", compute_type="f16")
+    fcn = g.fully_connected(x, chain, g.constant("f16", [64]))
+    assert g.fold_match(fcn).desc.bias_type == _lib.F16
+    with pytest.raises(fc.OvfccError, match="already has a bias"):
+        g.fold_match(g.add(fcn, g.constant("f16", [64])))
+    # FullyConnected whose bias is the reference's "absent" constant, Constant(dynamic, Shape{0})
+    g = Graph()
+    x = g.parameter("f16", [4, 256])
+    chain = decompression_subgraph(g, "u8", [64, 256], [64, 1], scale_type="f16", compute_type="f16")
+    assert g.fold_match(g.fully_connected(x, chain, g.constant("other", [0]))).bias == -1
+
+
+def test_rejections_name_their_reason():
+    def build(mutate):
+        g = Graph()
+        x = g.parameter("f16", [4, 256])
+        return g, x, mutate(g, x)
+    cases = {
+        "transpose_a": lambda g, x: g.matmul(x, decompression_subgraph(g, "u4", [64, 256], [64, 1], compute_type="f16"),
+                                             transpose_a=True, transpose_b=True),
+        "no Multiply": lambda g, x: g.matmul(x, g.convert(g.constant("u4", [64, 256]), "f16"), transpose_b=True),
+        "scale is not": lambda g, x: g.matmul(x, g.multiply(g.convert(g.constant("u4", [64, 256]), "f16"),
+                                                           g.convert(g.constant("u8", [64, 1]), "f16")), transpose_b=True),
+        "through a Convert": lambda g, x: g.matmul(x, g.multiply(g.constant("f16", [64, 256]), g.constant("f16", [64, 1])),
+                                                   transpose_b=True),
+        "u4 / i4 / u8 / i8": lambda g, x: g.matmul(x, g.multiply(g.convert(g.constant("other", [64, 256]), "f16"),
+                                                                 g.constant("f16", [64, 1])), transpose_b=True),
+        # a rank-1 scale broadcasts along the LAST axis: against [N, K] weights that is K, not N
+        "one value per": lambda g, x: g.matmul(x, decompression_subgraph(g, "u8", [256, 256], [256], compute_type="f16"),
+                                               transpose_b=True),
+        "zero-point must be scalar": lambda g, x: g.matmul(
+            x, decompression_subgraph(g, "u8", [64, 256], [64, 1], [1, 256], "u8", compute_type="f16"), transpose_b=True),
+        "zero-point must be u4": lambda g, x: g.matmul(
+            x, decompression_subgraph(g, "u8", [64, 256], [64, 1], [64, 1], "i8", compute_type="f16"), transpose_b=True),
+        "swap the two axes": lambda g, x: g.matmul(x, g.transpose(decompression_subgraph(
+            g, "u8", [256, 64], [1, 64], compute_type="f16"), [0, 1])),
+        "Reshape to two": lambda g, x: g.matmul(x, decompression_subgraph(g, "u4", [64, 2, 128], [64, 2, 1],
+                                                                         compute_type="f16"), transpose_b=True),
+        "does not produce": lambda g, x: g.matmul(x, decompression_subgraph(g, "u4", [64, 2, 128], [64, 2, 1],
+                                                                           compute_type="f16", reshape_to=[128, 128]),
+                                                  transpose_b=True),
+        "last dimension equal to K": lambda g, x: g.matmul(g.parameter("f16", [4, 128]), decompression_subgraph(
+            g, "u4", [64, 256], [64, 1], compute_type="f16"), transpose_b=True),
+        "activations must be f16": lambda g, x: g.matmul(g.parameter("other", [4, 256]), decompression_subgraph(
+            g, "u4", [64, 256], [64, 1], compute_type="f16"), transpose_b=True),
+    }
+    for reason, mutate in cases.items():
+        g, x, root = build(mutate)
+        with pytest.raises(fc.OvfccError, match=reason):
+            g.fold_match(root)
+    # what the support gate of the library refuses is refused here too (N and K are limited to 2^24)
+    g = Graph()
+    big = 1 << 25
+    x = g.parameter("f16", [4, big])
+    with pytest.raises(fc.OvfccError, match="2\\^24"):
+        g.fold_match(g.matmul(x, decompression_subgraph(g, "u4", [64, big], [64, 1], compute_type="f16"), transpose_b=True))
+
+
+def test_zero_point_and_scale_variants():
+    # f16 zero-points (NNCF stores them so for some models): the host turns them into u8
+    g = Graph()
+    x = g.parameter("f16", [4, 256])
+    f = g.fold_match(g.matmul(x, decompression_subgraph(g, "u8", [64, 256], [64, 1], [64, 1], "f16", scale_type="f16",
+                                                        compute_type="f16"), transpose_b=True))
+    assert f.zp_from_real == 1 and f.desc.zp_type == _lib.U8
+    # u4 weights with u8 zero-points, scalar zero-point of shape [1]
+    g = Graph()
+    x = g.parameter("f16", [4, 256])
+    f = g.fold_match(g.matmul(x, decompression_subgraph(g, "u4", [64, 2, 128], [64, 2, 1], [1], "u8", compute_type="f16",
+                                                        reshape_to=[64, 256]), transpose_b=True))
+    assert f.desc.zp_scalar == 1 and f.desc.zp_type == _lib.U8 and list(f.zp_view) == [0, 0]
+    # Multiply(scale, body): the scale may be the first input; f32 output type follows the MatMul
+    g = Graph()
+    x = g.parameter("f16", [2, 3, 256])
+    body = g.convert(g.constant("i4", [64, 256]), "f16")
+    f = g.fold_match(g.matmul(x, g.multiply(g.constant("f16", [64, 1]), body), transpose_b=True, type_="f32"))
+    assert f.desc.w_type == _lib.I4 and f.desc.zp_type == _lib.NONE and f.desc.out_type == _lib.F32
+    # a Convert to the data precision after the decompression, before or after the Transpose
+    for convert_first in (True, False):
+        g = Graph()
+        x = g.parameter("f32", [4, 256])
+        chain = decompression_subgraph(g, "u8", [256, 64], [1, 64], compute_type="f16",
+                                       convert_to="f32" if convert_first else None, transpose=True)
+        if not convert_first:
+            chain = g.convert(chain, "f32")
+        f = g.fold_match(g.matmul(x, chain, transpose_b=True))
+        assert f.desc.flags == _lib.W_INPUT_MAJOR and f.activations_f32 == 1
+
+
+def test_model_level_grouping():
+    """An attention block's q / k / v over one activation tensor, o on its own, gate / up with SwiGLU, down: what
+    shares a launch."""
+    g = Graph()
+    h = g.parameter("f16", [-1, 256])
+    q = _simple(g, h, N=256)
+    k = _simple(g, h, N=64)
+    v = _simple(g, h, N=64)
+    attn = g.other([q, k, v], shape=[-1, 256])
+    o = _simple(g, attn, N=256)
+    o_b = g.add(o, g.constant("f16", [1, 256]))
+    gate = _simple(g, o_b, N=512, zp=False, w_type="i4")
+    up = _simple(g, o_b, N=512, zp=False, w_type="i4")
+    act = g.multiply(g.swish(gate), up)
+    down = _simple(g, act, N=256, K=512)
+    g.result(down)
+    folds, fused = g.fold_model()
+    assert len(folds) == 7
+    by_root = {f.root: i for i, f in enumerate(folds)}
+    kinds = {}
+    for u in fused:
+        kinds.setdefault(u.kind, []).append(u)
+    (qkv,) = kinds[_lib.FUSED_CONCAT]
+    assert [folds[qkv.parts[i]].root for i in range(qkv.n_parts)] == [q, k, v]
+    (glu,) = kinds[_lib.FUSED_GLU]
+    assert folds[glu.parts[0]].root == gate and folds[glu.parts[1]].root == up
+    assert glu.glu_type == _lib.GLU["swish"] and glu.root == act
+    singles = sorted(folds[u.parts[0]].root for u in kinds[_lib.FUSED_SINGLE])
+    assert singles == sorted([o_b, down]) and folds[by_root[o_b]].bias >= 0
+    assert sorted(p for u in fused for p in u.parts[:u.n_parts]) == list(range(7))   # every fold in exactly one group
+
+
+def test_grouping_rules():
+    def two(g, h, **kw):
+        a = _simple(g, h, **kw)
+        return a, _simple(g, h, **kw)
+    # Gelu with the tanh approximation; the activation may be the second Multiply input
+    g = Graph()
+    h = g.parameter("f16", [8, 256])
+    a, b = two(g, h)
+    m = g.multiply(b, g.gelu(a, tanh=True))
+    _, fused = g.fold_model()
+    assert fused[0].kind == _lib.FUSED_GLU and fused[0].glu_type == _lib.GLU["gelu_tanh"] and fused[0].root == m
+    # a gate that something else reads as well cannot disappear into a fused node
+    g = Graph()
+    h = g.parameter("f16", [8, 256])
+    a, b = two(g, h)
+    g.multiply(g.swish(a), b)
+    g.result(a)
+    _, fused = g.fold_model()
+    assert [u.kind for u in fused] == [_lib.FUSED_CONCAT]
+    # different formats, four siblings, different activations: no horizontal fusion
+    for build in (lambda g, h: (_simple(g, h), _simple(g, h, zp=False)),
+                  lambda g, h: tuple(_simple(g, h) for _ in range(4)),
+                  lambda g, h: (_simple(g, h), _simple(g, g.parameter("f16", [8, 256]))),
+                  lambda g, h: (_simple(g, h), _simple(g, h, major="input"))):
+        g = Graph()
+        build(g, g.parameter("f16", [8, 256]))
+        folds, fused = g.fold_model()
+        assert all(u.kind == _lib.FUSED_SINGLE for u in fused) and len(fused) == len(folds)
+    # output arrays that are too small are an error, not a truncation
+    g = Graph()
+    h = g.parameter("f16", [8, 256])
+    two(g, h)
+    with pytest.raises(fc.OvfccError):
+        g.fold_model(max_folds=1)
