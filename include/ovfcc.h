@@ -246,6 +246,18 @@ int ovfcc_gather_matmul_device(ovfcc_request* req, const ovfcc_weights* const* e
                                const void* a_dev, int a_batches, const int32_t* indices, int64_t M, int top_k,
                                void* y_dev);
 
+/* The same with the indices in device memory, where a router's TopK leaves them: the (row, selection) pairs are
+ * bucketed per expert by a kernel on the request's stream (one workgroup per expert; the reference's GPU plugin builds
+ * its expert masks on the device as well, src/plugins/intel_gpu/src/graph/impls/ocl_v2/moe_mask_gen.cl), the grouped
+ * launch reads its slice table from device memory, and the call neither waits for the stream nor depends on the row
+ * counts.  An index outside [0, n_experts) selects nothing: its row of Y is left untouched.  Needs tiled 4-bit
+ * experts with N % 256 == 0 and one scalar zero-point (what the grouped prefill kernel runs) and at most 64 experts;
+ * otherwise OVFCC_EUNSUPPORTED.  ovfcc_gather_matmul_device takes this path itself wherever it fits, after copying
+ * its indices to the device (OVFCC_MOE_HOST_ROUTING=1 in the environment keeps the bucketing on the host). */
+int ovfcc_gather_matmul_routed_device(ovfcc_request* req, const ovfcc_weights* const* experts, int n_experts,
+                                      const void* a_dev, int a_batches, const int32_t* indices_dev, int64_t M, int top_k,
+                                      void* y_dev);
+
 /* The expert block of a mixture-of-experts layer as one call: ov::op::internal::MOECompressed with
  * Expert_type::GEMM3_SWIGLU (src/common/transformations/include/ov_ops/moe_compressed.hpp:15-75,
  * src/core/dev_api/openvino/op/moe.hpp:17-45), the node that MoE op fusion folds three GatherMatmulCompressed, the
@@ -262,6 +274,13 @@ int ovfcc_gather_matmul_device(ovfcc_request* req, const ovfcc_weights* const* e
 int ovfcc_moe_device(ovfcc_request* req, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down,
                      int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices_host, int64_t M,
                      int top_k, void* y_dev);
+
+/* ovfcc_moe_device with indices_dev [M, top_k] int32 in device memory (see ovfcc_gather_matmul_routed_device): the
+ * routing kernel runs once per projection, nothing in the call waits for the stream.  A pair whose index lies outside
+ * [0, n_experts) contributes nothing to its row's sum. */
+int ovfcc_moe_routed_device(ovfcc_request* req, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down,
+                            int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices_dev,
+                            int64_t M, int top_k, void* y_dev);
 
 /* Benchmark twin of ovfcc_bench_layers for grouped runs: `iters` eager calls of ovfcc_fc_run_grouped_device on the
  * request's stream, bracketed by HIP events on that stream. */

@@ -367,6 +367,230 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
     return OVFCC_OK;
 }
 
+
+// ---- mixture-of-experts layers with the routing done on the device --------------------------------------------
+// The grouped launch whose slices the routing kernel cuts: tiled 4-bit experts that the all-asynchronous prefill
+// kernel runs, at most kMaxGroupItems of them (their pointers travel in the routing kernel's arguments).  The
+// slice height is fixed from the average bucket (the counts stay on the device): 64 rows up to an average of 56,
+// 128 above (OVFCC_PREFILL_ROWS overrides).  How many slices the buckets make is known on the device only, where
+// the routing kernel also chooses the cut along K for that count; grid, workspace and counters are sized for the
+// worst count up to ceil(R / cap) + n_experts, and workgroups beyond the header's grid return at once.
+struct RoutedLaunch {
+    int cap = 0, n_slices = 0;
+    ovfcc::LaunchPlan plan;
+    ovfcc::FcDeviceArgs args;
+};
+
+bool plan_routed(ovfcc_request* r, const ovfcc_weights* w0, int64_t R, int n_experts, RoutedLaunch* out) {
+    if (n_experts > ovfcc::kMaxGroupItems || !w0->layout.tiled || w0->layout.bits != 4 ||
+        r->force_kernel != OVFCC_KERNEL_AUTO || R <= 0)
+        return false;
+    int cap = R / n_experts > 56 ? ovfcc::kPrefillGroupRows : ovfcc::kPrefillGroupRows / 2;
+    if (const char* e = std::getenv("OVFCC_PREFILL_ROWS"))
+        cap = std::atoi(e) == 64 ? 64 : ovfcc::kPrefillGroupRows;
+    const int64_t n = (R + cap - 1) / cap + n_experts;
+    if (n * cap * w0->desc.K * 2 >= ((int64_t)1 << 31) || n > 65535)
+        return false;
+    fill_args(w0, nullptr, nullptr, n * cap, &out->args);
+    out->args.tile_rows = cap;
+    out->args.want_async = true;
+    if (ovfcc::plan_launch(out->args, OVFCC_KERNEL_PREFILL, r->force_split, r->ctx->n_cus, &out->plan) != OVFCC_OK ||
+        !out->plan.async_dma || out->plan.big || out->plan.tiles_y != (int)n)
+        return false;
+    ovfcc::LaunchPlan& p = out->plan;
+    int grid = 0;
+    bool split = false;
+    for (int t = 1; t <= (int)n; ++t) {
+        const ovfcc::RoutedHeader h = ovfcc::routed_header(p.tiles_x, t, (int)w0->layout.k_blocks, r->ctx->n_cus);
+        grid = std::max(grid, h.grid);
+        split = split || h.split_k > 1;
+    }
+    p.n_cus = r->ctx->n_cus;
+    p.grid[0] = (unsigned)grid, p.grid[1] = p.grid[2] = 1;
+    p.workspace_bytes = split ? (size_t)grid * p.tile_m * ovfcc::kPrefillWideN * sizeof(float) : 0;
+    p.counter_count = split ? (size_t)p.tiles_x * n : 0;
+    out->cap = cap;
+    out->n_slices = (int)n;
+    return true;
+}
+
+int run_routed(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, RoutedLaunch& L,
+               const int* indices_dev, int64_t M, int top_k, int a_batches, int inverse, const void* x_base,
+               size_t x_row_bytes, void* y_base, size_t y_row_bytes, int* d_maps, ovfcc::RoutedHeader* d_header) {
+    auto* d_table = reinterpret_cast<ovfcc::BatchGroupItem*>(d_header + 1);
+    ovfcc::ExpertPointers ptrs{};
+    for (int e = 0; e < n_experts; ++e)
+        ptrs.w[e] = experts[e]->d_w, ptrs.scale[e] = experts[e]->d_scale, ptrs.zp[e] = experts[e]->d_zp,
+        ptrs.bias[e] = experts[e]->d_bias;
+    const int64_t R = M * top_k;
+    int e1 = ovfcc::launch_moe_route(indices_dev, M, top_k, n_experts, a_batches, inverse, L.cap, ptrs, x_base,
+                                     x_row_bytes, y_base, y_row_bytes, d_maps, d_maps + R, d_table, L.n_slices, d_header,
+                                     L.plan.tiles_x, (int)experts[0]->layout.k_blocks, L.plan.n_cus, r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "routing kernel launch");
+    return OVFCC_OK;
+}
+
+int launch_routed(ovfcc_request* r, RoutedLaunch& L, const ovfcc::RoutedHeader* d_header) {
+    auto* d_table = reinterpret_cast<const ovfcc::BatchGroupItem*>(d_header + 1);
+    int rc = ensure_split_buffers(r, L.plan);
+    if (rc)
+        return rc;
+    L.args.workspace = r->workspace;
+    L.args.counters = r->counters;
+    const ovfcc::BatchGroupTable none{};
+    const int e = ovfcc::launch_prefill_async_grouped(none, L.n_slices, L.args, L.plan, r->stream, d_table, d_header);
+    if (e)
+        return hip_fail((hipError_t)e, "grouped kernel launch");
+    ovfcc::LaunchPlan shown = L.plan;
+    shown.name = "fcc_prefill_async_grouped_w4";
+    record(r, shown);
+    return OVFCC_OK;
+}
+
+// Same shape, format, bias presence and scalar zero-point for every expert (one grouped launch carries one of each).
+int experts_agree(const ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, bool* same_zp) {
+    const ovfcc_weights* w0 = experts[0];
+    *same_zp = true;
+    for (int e = 0; e < n_experts; ++e) {
+        const ovfcc_weights* w = experts[e];
+        if (!w || w->ctx != r->ctx)
+            return fail(OVFCC_EINVAL, "an expert's weights are null or belong to another context");
+        if (std::memcmp(&w->desc, &w0->desc, sizeof(ovfcc_fc_desc)) != 0 || (w->d_bias != nullptr) != (w0->d_bias != nullptr))
+            return fail(OVFCC_EUNSUPPORTED, "experts differ in shape, types, bias or output type");
+        if (w->layout.zp_const != w0->layout.zp_const)
+            *same_zp = false;
+    }
+    return OVFCC_OK;
+}
+
+// Indices given in host memory: checked there, then copied to the device through the request's pinned buffer.
+int upload_indices(ovfcc_request* r, const int32_t* indices, int64_t R, int n_experts, int* d_indices) {
+    for (int64_t j = 0; j < R; ++j)
+        if (indices[j] < 0 || indices[j] >= n_experts)
+            return fail(OVFCC_EINVAL, "an expert index is out of range");
+    const size_t bytes = (size_t)R * sizeof(int);
+    if (!r->maps_uploaded)
+        HIP_TRY(hipEventCreateWithFlags(&r->maps_uploaded, hipEventDisableTiming));
+    else
+        HIP_TRY(hipEventSynchronize(r->maps_uploaded));  // the previous call's copy has left the buffer
+    if (bytes > r->h_maps_cap) {
+        if (r->h_maps)
+            HIP_TRY(hipHostFree(r->h_maps));
+        r->h_maps = nullptr, r->h_maps_cap = 0;
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->h_maps), bytes, hipHostMallocDefault));
+        r->h_maps_cap = bytes;
+    }
+    std::memcpy(r->h_maps, indices, bytes);
+    HIP_TRY(hipMemcpyAsync(d_indices, r->h_maps, bytes, hipMemcpyHostToDevice, r->stream));
+    HIP_TRY(hipEventRecord(r->maps_uploaded, r->stream));
+    return OVFCC_OK;
+}
+
+// GatherMatmul with the routing on the device.  indices_dev is in device memory, or indices_host is given and
+// copied there.  Returns OVFCC_EUNSUPPORTED (without an error string of its own) when no routed launch fits.
+int gather_matmul_routed(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, const void* a_dev,
+                         int a_batches, const int32_t* indices_dev, const int32_t* indices_host, int64_t M, int top_k,
+                         void* y_dev, bool* ran) {
+    *ran = false;
+    const ovfcc_weights* w0 = experts[0];
+    const int64_t K = w0->desc.K, N_out = out_channels(w0), R = M * top_k;
+    const size_t out_bytes = w0->desc.out_type == OVFCC_F32 ? 4 : 2;
+    RoutedLaunch L;
+    if (!plan_routed(r, w0, R, n_experts, &L))
+        return OVFCC_OK;
+    auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t x_bytes = (size_t)R * K * 2, y_bytes = (size_t)R * N_out * out_bytes;
+    const size_t y_off = up256(x_bytes), m_off = up256(y_off + y_bytes), t_off = up256(m_off + (size_t)2 * R * sizeof(int));
+    const size_t i_off = up256(t_off + sizeof(ovfcc::RoutedHeader) + (size_t)L.n_slices * sizeof(ovfcc::BatchGroupItem));
+    const size_t need = i_off + (size_t)R * sizeof(int);
+    if (need > r->gather_cap)
+        HIP_TRY(hipStreamSynchronize(r->stream));
+    int rc = grow(&r->d_gather, &r->gather_cap, need);
+    if (rc)
+        return rc;
+    char* base = static_cast<char*>(r->d_gather);
+    int* d_maps = reinterpret_cast<int*>(base + m_off);
+    auto* d_table = reinterpret_cast<ovfcc::RoutedHeader*>(base + t_off);  // header, then the slices
+    if (!indices_dev) {
+        rc = upload_indices(r, indices_host, R, n_experts, reinterpret_cast<int*>(base + i_off));
+        if (rc)
+            return rc;
+        indices_dev = reinterpret_cast<const int32_t*>(base + i_off);
+    }
+    rc = run_routed(r, experts, n_experts, L, indices_dev, M, top_k, a_batches, 0, base, (size_t)K * 2, base + y_off,
+                    (size_t)N_out * out_bytes, d_maps, d_table);
+    if (rc)
+        return rc;
+    int e1 = ovfcc::launch_rows(base, a_dev, d_maps, nullptr, (int)R, (int)(K * 2), r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "row gather launch");
+    rc = launch_routed(r, L, d_table);
+    if (rc)
+        return rc;
+    e1 = ovfcc::launch_rows(y_dev, base + y_off, nullptr, d_maps + R, (int)R, (int)(N_out * out_bytes), r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "row scatter launch");
+    *ran = true;
+    return OVFCC_OK;
+}
+
+int moe_routed(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down, int n_experts,
+               const void* x_dev, const void* routing_dev, const int32_t* indices_dev, const int32_t* indices_host,
+               int64_t M, int top_k, void* y_dev, bool* ran) {
+    *ran = false;
+    const ovfcc_weights *g0 = gate_up[0], *d0 = down[0];
+    const int64_t H = g0->desc.K, I = out_channels(g0), R = M * top_k;
+    const int d_f32 = d0->desc.out_type == OVFCC_F32 ? 1 : 0;
+    RoutedLaunch Lg, Ld;
+    if (!plan_routed(r, g0, R, n_experts, &Lg) || !plan_routed(r, d0, R, n_experts, &Ld))
+        return OVFCC_OK;
+    auto up256 = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t x_bytes = (size_t)R * H * 2, h_bytes = (size_t)R * I * 2, d_bytes = (size_t)R * H * (d_f32 ? 4 : 2);
+    const size_t h_off = up256(x_bytes), d_off = up256(h_off + h_bytes), m_off = up256(d_off + d_bytes);
+    const size_t tg_off = up256(m_off + (size_t)2 * R * sizeof(int));
+    const size_t td_off = up256(tg_off + sizeof(ovfcc::RoutedHeader) + (size_t)Lg.n_slices * sizeof(ovfcc::BatchGroupItem));
+    const size_t i_off = up256(td_off + sizeof(ovfcc::RoutedHeader) + (size_t)Ld.n_slices * sizeof(ovfcc::BatchGroupItem));
+    const size_t need = i_off + (size_t)R * sizeof(int);
+    if (need > r->gather_cap)
+        HIP_TRY(hipStreamSynchronize(r->stream));
+    int rc = grow(&r->d_gather, &r->gather_cap, need);
+    if (rc)
+        return rc;
+    char* base = static_cast<char*>(r->d_gather);
+    int* d_maps = reinterpret_cast<int*>(base + m_off);
+    auto* tab_g = reinterpret_cast<ovfcc::RoutedHeader*>(base + tg_off);  // header, then the slices
+    auto* tab_d = reinterpret_cast<ovfcc::RoutedHeader*>(base + td_off);
+    if (!indices_dev) {
+        rc = upload_indices(r, indices_host, R, n_experts, reinterpret_cast<int*>(base + i_off));
+        if (rc)
+            return rc;
+        indices_dev = reinterpret_cast<const int32_t*>(base + i_off);
+    }
+    // the routing kernel runs once per projection: same buckets and maps, a slice table each
+    rc = run_routed(r, gate_up, n_experts, Lg, indices_dev, M, top_k, 1, 1, base, (size_t)H * 2, base + h_off,
+                    (size_t)I * 2, d_maps, tab_g);
+    if (!rc)
+        rc = run_routed(r, down, n_experts, Ld, indices_dev, M, top_k, 1, 1, base + h_off, (size_t)I * 2, base + d_off,
+                        (size_t)H * (d_f32 ? 4 : 2), d_maps, tab_d);
+    if (rc)
+        return rc;
+    int e1 = ovfcc::launch_rows(base, x_dev, d_maps, nullptr, (int)R, (int)(H * 2), r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "row gather launch");
+    rc = launch_routed(r, Lg, tab_g);
+    if (!rc)
+        rc = launch_routed(r, Ld, tab_d);
+    if (rc)
+        return rc;
+    e1 = ovfcc::launch_moe_combine(y_dev, base + d_off, routing_dev, d_maps + R, (int)M, top_k, (int)H, d_f32, d_f32,
+                                   r->stream);
+    if (e1)
+        return hip_fail((hipError_t)e1, "expert combine launch");
+    *ran = true;
+    return OVFCC_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1036,37 +1260,74 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
     return OVFCC_OK;
 }
 
-int ovfcc_gather_matmul_device(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, const void* a_dev,
-                               int a_batches, const int32_t* indices, int64_t M, int top_k, void* y_dev) {
+namespace {
+// argument checks shared by the two forms of the gather-matmul entry point; *same_zp: the experts' scalar
+// zero-points agree (a grouped launch carries one)
+int check_gather_matmul(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, const void* a_dev,
+                        int a_batches, const void* indices, int64_t M, int top_k, void* y_dev, bool* same_zp) {
     if (!r || !experts || n_experts <= 0 || !indices || M < 0 || top_k <= 0)
         return fail(OVFCC_EINVAL, "bad gather-matmul arguments");
     if (a_batches != 1 && a_batches != top_k)
         return fail(OVFCC_EINVAL, "A must have one batch or one batch per selected expert");
     if (top_k > n_experts)
         return fail(OVFCC_EINVAL, "more selected experts per row than experts");
-    if (M == 0)
-        return OVFCC_OK;
-    if (!a_dev || !y_dev)
+    if (M > 0 && (!a_dev || !y_dev))
         return fail(OVFCC_EINVAL, "A or Y is null");
     if (M * top_k > ((int64_t)1 << 24))
         return fail(OVFCC_EUNSUPPORTED, "M * top_k is limited to 2^24");
+    if (!experts[0])
+        return fail(OVFCC_EINVAL, "an expert's weights are null or belong to another context");
+    int rc = experts_agree(r, experts, n_experts, same_zp);
+    if (rc)
+        return rc;
     const ovfcc_weights* w0 = experts[0];
-    for (int e = 0; e < n_experts; ++e) {
-        const ovfcc_weights* w = experts[e];
-        if (!w || w->ctx != r->ctx)
-            return fail(OVFCC_EINVAL, "an expert's weights are null or belong to another context");
-        if (std::memcmp(&w->desc, &w0->desc, sizeof(ovfcc_fc_desc)) != 0 || (w->d_bias != nullptr) != (w0->d_bias != nullptr))
-            return fail(OVFCC_EUNSUPPORTED, "experts differ in shape, types, bias or output type");
-    }
+    const size_t out_bytes = w0->desc.out_type == OVFCC_F32 ? 4 : 2;
+    if ((w0->desc.K * 2) % 16 != 0 || (out_channels(w0) * out_bytes) % 16 != 0)
+        return fail(OVFCC_EUNSUPPORTED, "rows of A and Y must be multiples of 16 bytes");
+    return OVFCC_OK;
+}
+}  // namespace
+
+int ovfcc_gather_matmul_routed_device(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts,
+                                      const void* a_dev, int a_batches, const int32_t* indices_dev, int64_t M, int top_k,
+                                      void* y_dev) {
+    bool same_zp = true, ran = false;
+    int rc = check_gather_matmul(r, experts, n_experts, a_dev, a_batches, indices_dev, M, top_k, y_dev, &same_zp);
+    if (rc || M == 0)
+        return rc;
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    if (same_zp)
+        rc = gather_matmul_routed(r, experts, n_experts, a_dev, a_batches, indices_dev, nullptr, M, top_k, y_dev, &ran);
+    if (rc)
+        return rc;
+    if (!ran)
+        return fail(OVFCC_EUNSUPPORTED,
+                    "routing on the device needs tiled 4-bit experts of one scalar zero-point that the grouped prefill "
+                    "kernel runs (N % 256 == 0), at most 64 of them; pass the indices in host memory instead");
+    return OVFCC_OK;
+}
+
+int ovfcc_gather_matmul_device(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, const void* a_dev,
+                               int a_batches, const int32_t* indices, int64_t M, int top_k, void* y_dev) {
+    bool same_zp = true, ran = false;
+    int rc = check_gather_matmul(r, experts, n_experts, a_dev, a_batches, indices, M, top_k, y_dev, &same_zp);
+    if (rc || M == 0)
+        return rc;
+    const ovfcc_weights* w0 = experts[0];
     const int64_t K = w0->desc.K, N_out = out_channels(w0);
     const size_t out_bytes = w0->desc.out_type == OVFCC_F32 ? 4 : 2;
-    if ((K * 2) % 16 != 0 || (N_out * out_bytes) % 16 != 0)
-        return fail(OVFCC_EUNSUPPORTED, "rows of A and Y must be multiples of 16 bytes");
     HIP_TRY(hipSetDevice(r->ctx->device));
+    // the routed form wherever it fits: the indices are copied to the device and bucketed there, and the call does
+    // not depend on what the host threads were doing; otherwise the rows are bucketed here
+    if (same_zp && !std::getenv("OVFCC_MOE_HOST_ROUTING")) {
+        rc = gather_matmul_routed(r, experts, n_experts, a_dev, a_batches, nullptr, indices, M, top_k, y_dev, &ran);
+        if (rc || ran)
+            return rc;
+    }
 
     const int64_t R = M * top_k;
     std::vector<int> count, start;
-    int rc = bucket_rows(r, indices, M, top_k, n_experts, a_batches, false, &count, &start);
+    rc = bucket_rows(r, indices, M, top_k, n_experts, a_batches, false, &count, &start);
     if (rc)
         return rc;
     const size_t map_bytes = (size_t)2 * R * sizeof(int);
@@ -1100,43 +1361,79 @@ int ovfcc_gather_matmul_device(ovfcc_request* r, const ovfcc_weights* const* exp
     return OVFCC_OK;
 }
 
-int ovfcc_moe_device(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down,
-                     int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices, int64_t M,
-                     int top_k, void* y_dev) {
+namespace {
+int check_moe(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down, int n_experts,
+              const void* x_dev, const void* routing_dev, const void* indices, int64_t M, int top_k, void* y_dev,
+              bool* same_zp) {
     if (!r || !gate_up || !down || n_experts <= 0 || !indices || M < 0 || top_k <= 0)
         return fail(OVFCC_EINVAL, "bad mixture-of-experts arguments");
     if (top_k > n_experts)
         return fail(OVFCC_EINVAL, "more selected experts per row than experts");
-    if (M == 0)
-        return OVFCC_OK;
-    if (!x_dev || !routing_dev || !y_dev)
+    if (M > 0 && (!x_dev || !routing_dev || !y_dev))
         return fail(OVFCC_EINVAL, "hidden states, routing weights or output is null");
     if (M * top_k > ((int64_t)1 << 24))
         return fail(OVFCC_EUNSUPPORTED, "M * top_k is limited to 2^24");
+    if (!gate_up[0] || !down[0])
+        return fail(OVFCC_EINVAL, "an expert's weights are null or belong to another context");
+    bool zg = true, zd = true;
+    int rc = experts_agree(r, gate_up, n_experts, &zg);
+    if (!rc)
+        rc = experts_agree(r, down, n_experts, &zd);
+    if (rc)
+        return rc;
+    *same_zp = zg && zd;
     const ovfcc_weights *g0 = gate_up[0], *d0 = down[0];
-    for (int e = 0; e < n_experts; ++e) {
-        const ovfcc_weights *g = gate_up[e], *d = down[e];
-        if (!g || !d || g->ctx != r->ctx || d->ctx != r->ctx)
-            return fail(OVFCC_EINVAL, "an expert's weights are null or belong to another context");
-        if (std::memcmp(&g->desc, &g0->desc, sizeof(ovfcc_fc_desc)) != 0 ||
-            std::memcmp(&d->desc, &d0->desc, sizeof(ovfcc_fc_desc)) != 0 ||
-            (g->d_bias != nullptr) != (g0->d_bias != nullptr) || (d->d_bias != nullptr) != (d0->d_bias != nullptr))
-            return fail(OVFCC_EUNSUPPORTED, "experts differ in shape, types, bias or output type");
-    }
     // gate/up: [2 I, H] with a gated linear unit, f16 out (it feeds the down projection); down: [H, I], no unit
     const int64_t H = g0->desc.K, I = out_channels(g0);
     if (!g0->layout.glu || g0->desc.out_type != OVFCC_F16)
         return fail(OVFCC_EINVAL, "the gate/up nodes must carry a gated linear unit and write f16");
     if (d0->layout.glu || d0->desc.K != I || d0->desc.N != H)
         return fail(OVFCC_EINVAL, "the down nodes must map the gate/up output back to the hidden size, without a unit");
-    const int d_f32 = d0->desc.out_type == OVFCC_F32 ? 1 : 0;
     if ((H * 2) % 16 != 0 || (I * 2) % 16 != 0)
         return fail(OVFCC_EUNSUPPORTED, "hidden and intermediate rows must be multiples of 16 bytes");
+    return OVFCC_OK;
+}
+}  // namespace
+
+int ovfcc_moe_routed_device(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down,
+                            int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices_dev,
+                            int64_t M, int top_k, void* y_dev) {
+    bool same_zp = true, ran = false;
+    int rc = check_moe(r, gate_up, down, n_experts, x_dev, routing_dev, indices_dev, M, top_k, y_dev, &same_zp);
+    if (rc || M == 0)
+        return rc;
     HIP_TRY(hipSetDevice(r->ctx->device));
+    if (same_zp)
+        rc = moe_routed(r, gate_up, down, n_experts, x_dev, routing_dev, indices_dev, nullptr, M, top_k, y_dev, &ran);
+    if (rc)
+        return rc;
+    if (!ran)
+        return fail(OVFCC_EUNSUPPORTED,
+                    "routing on the device needs tiled 4-bit experts of one scalar zero-point that the grouped prefill "
+                    "kernel runs (N % 256 == 0), at most 64 of them; pass the indices in host memory instead");
+    return OVFCC_OK;
+}
+
+int ovfcc_moe_device(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down,
+                     int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices, int64_t M,
+                     int top_k, void* y_dev) {
+    bool same_zp = true, ran = false;
+    int rc = check_moe(r, gate_up, down, n_experts, x_dev, routing_dev, indices, M, top_k, y_dev, &same_zp);
+    if (rc || M == 0)
+        return rc;
+    const ovfcc_weights *g0 = gate_up[0], *d0 = down[0];
+    const int64_t H = g0->desc.K, I = out_channels(g0);
+    const int d_f32 = d0->desc.out_type == OVFCC_F32 ? 1 : 0;
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    if (same_zp && !std::getenv("OVFCC_MOE_HOST_ROUTING")) {
+        rc = moe_routed(r, gate_up, down, n_experts, x_dev, routing_dev, nullptr, indices, M, top_k, y_dev, &ran);
+        if (rc || ran)
+            return rc;
+    }
 
     const int64_t R = M * top_k;
     std::vector<int> count, start;
-    int rc = bucket_rows(r, indices, M, top_k, n_experts, 1, true, &count, &start);
+    rc = bucket_rows(r, indices, M, top_k, n_experts, 1, true, &count, &start);
     if (rc)
         return rc;
     const size_t map_bytes = (size_t)2 * R * sizeof(int);

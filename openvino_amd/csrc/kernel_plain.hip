@@ -101,14 +101,17 @@ __global__ __launch_bounds__(256) void fcc_touch_kernel(const uint4_t* __restric
 // ------------------------------------------------------------------------------------------------
 // Row gather / scatter for the mixture-of-experts entry point: dst row r = src row src_row[r] (gather, dst_row
 // null) or dst row dst_row[r] = src row r (scatter, src_row null); rows of row_bytes (a multiple of 16) bytes.
-// One workgroup per row.
+// A negative map entry skips the row.  One workgroup per row.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fcc_rows_kernel(uint4_t* __restrict__ dst, const uint4_t* __restrict__ src,
                                                        const int* __restrict__ src_row,
                                                        const int* __restrict__ dst_row, int row_bytes) {
     const int r = blockIdx.x;
-    const size_t from = (size_t)(src_row ? src_row[r] : r) * (row_bytes / 16);
-    const size_t to = (size_t)(dst_row ? dst_row[r] : r) * (row_bytes / 16);
+    const int named = src_row ? src_row[r] : dst_row[r];
+    if (named < 0)
+        return;  // a slot that the routing left empty
+    const size_t from = (size_t)(src_row ? named : r) * (row_bytes / 16);
+    const size_t to = (size_t)(dst_row ? named : r) * (row_bytes / 16);
     for (int i = threadIdx.x; i < row_bytes / 16; i += blockDim.x)
         dst[to + i] = src[from + i];
 }
@@ -140,8 +143,11 @@ __global__ __launch_bounds__(256) void fcc_moe_combine_kernel(void* __restrict__
     for (int c = 4 * threadIdx.x; c < H; c += 4 * blockDim.x) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
         for (int j = 0; j < top_k; ++j) {
+            const int slot = pos[(size_t)m * top_k + j];
+            if (slot < 0)
+                continue;  // an index outside the experts selects nothing
             const float wgt = (float)routing[(size_t)m * top_k + j];
-            const size_t row = (size_t)pos[(size_t)m * top_k + j] * H + c;
+            const size_t row = (size_t)slot * H + c;
             if constexpr (IN_F32) {
                 const float4_t v = *reinterpret_cast<const float4_t*>(static_cast<const float*>(d) + row);
                 acc[0] += wgt * v.x, acc[1] += wgt * v.y, acc[2] += wgt * v.z, acc[3] += wgt * v.w;
@@ -158,6 +164,121 @@ __global__ __launch_bounds__(256) void fcc_moe_combine_kernel(void* __restrict__
             *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + (size_t)m * H + c) =
                 half4_t{(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
     }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Mixture-of-experts routing on the device (the reference's GPU plugin builds its expert masks there too,
+// src/plugins/intel_gpu/src/graph/impls/ocl_v2/moe_mask_gen.cl; the bucket order is that of the CPU executor,
+// src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_gathermatmul_executor.cpp:492-509).  One workgroup per
+// expert, no communication between workgroups: every workgroup counts all experts' pairs (a histogram in LDS over
+// the R indices), derives its own bucket's first slot and first slice from the counts of the experts before it,
+// and then places its own pairs in ascending order with a block-wide prefix sum.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restrict__ indices, int R, int M, int top_k,
+                                                            int n_experts, int a_batches, int inverse, int cap,
+                                                            ExpertPointers experts, const char* x_base,
+                                                            size_t x_row_bytes, char* y_base, size_t y_row_bytes,
+                                                            int* __restrict__ first, int* __restrict__ second,
+                                                            BatchGroupItem* __restrict__ table, int n_slices_max,
+                                                            RoutedHeader* __restrict__ header, int tiles_x,
+                                                            int kb_total, int n_cus) {
+    __shared__ int hist[kMaxGroupItems];
+    __shared__ int wave_total[4];
+    __shared__ int start_s, slice_s, total_slices_s, total_pairs_s;
+    const int e = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid < kMaxGroupItems)
+        hist[tid] = 0;
+    __syncthreads();
+    for (int j = tid; j < R; j += 256) {
+        const int v = indices[j];
+        if (v >= 0 && v < n_experts)
+            atomicAdd(&hist[v], 1);
+        else if (e == 0 && inverse)
+            second[j] = -1;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int start = 0, slice = 0, total = 0, pairs = 0;
+        for (int k = 0; k < n_experts; ++k) {
+            const int slices = (hist[k] + cap - 1) / cap;
+            if (k < e)
+                start += hist[k], slice += slices;
+            total += slices;
+            pairs += hist[k];
+        }
+        start_s = start, slice_s = slice, total_slices_s = total, total_pairs_s = pairs;
+    }
+    __syncthreads();
+    const int start = start_s, count = hist[e];
+    // this expert's pairs, in ascending order of (row, selection)
+    int placed = 0;
+    for (int j0 = 0; j0 < R; j0 += 256) {
+        const int j = j0 + tid;
+        const bool mine = j < R && indices[j] == e;
+        const unsigned long long ballot = __ballot(mine);
+        const int before = __popcll(ballot & ((1ull << lane) - 1ull));
+        if (lane == 0)
+            wave_total[wave] = __popcll(ballot);
+        __syncthreads();
+        int base = placed;
+        for (int w = 0; w < wave; ++w)
+            base += wave_total[w];
+        if (mine) {
+            const int slot = start + base + before;
+            const int m = j / top_k, i = j - m * top_k;
+            first[slot] = a_batches == 1 ? m : i * M + m;
+            if (inverse)
+                second[j] = slot;
+            else
+                second[slot] = i * M + m;
+        }
+        placed += wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+        __syncthreads();
+    }
+    // the bucket cut into equal slices of at most cap rows
+    const int slices = (count + cap - 1) / cap;
+    const int step = slices ? (count + slices - 1) / slices : 0;
+    for (int t = tid; t < slices; t += 256) {
+        BatchGroupItem it;
+        it.w = experts.w[e], it.scale = experts.scale[e], it.zp = experts.zp[e], it.bias = experts.bias[e];
+        it.x = x_base + (size_t)(start + t * step) * x_row_bytes;
+        it.y = y_base + (size_t)(start + t * step) * y_row_bytes;
+        it.M = min(step, count - t * step);
+        it.reserved = 0;
+        table[slice_s + t] = it;
+    }
+    // the last workgroup closes what no bucket owns: the slices beyond the last one, and the slots beyond the
+    // last pair (there are some when an index named no expert)
+    if (e == n_experts - 1) {
+        if (tid == 0)
+            *header = routed_header(tiles_x, total_slices_s, kb_total, n_cus);
+        for (int t = total_slices_s + tid; t < n_slices_max; t += 256) {
+            BatchGroupItem it{};
+            table[t] = it;
+        }
+        for (int slot = total_pairs_s + tid; slot < R; slot += 256) {
+            first[slot] = -1;
+            if (!inverse)
+                second[slot] = -1;
+        }
+    }
+}
+
+int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts, int a_batches, int inverse, int cap,
+                     const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
+                     size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
+                     RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream) {
+    const int64_t R = M * top_k;
+    if (R <= 0 || R > ((int64_t)1 << 24) || n_experts < 1 || n_experts > kMaxGroupItems || cap < 1 ||
+        n_slices_max < (R + cap - 1) / cap + n_experts || (a_batches != 1 && a_batches != top_k) || !header ||
+        tiles_x < 1 || kb_total < 1 || n_cus < 1)
+        return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(fcc_moe_route_kernel, dim3((unsigned)n_experts), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       indices_dev, (int)R, (int)M, top_k, n_experts, a_batches, inverse, cap, experts,
+                       static_cast<const char*>(x_base), x_row_bytes, static_cast<char*>(y_base), y_row_bytes, first,
+                       second, table, n_slices_max, header, tiles_x, kb_total, n_cus);
+    return (int)hipGetLastError();
 }
 
 int launch_moe_combine(void* y, const void* d, const void* routing, const int* pos, int rows, int top_k, int H,

@@ -378,14 +378,25 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* _
 // item sit together in a super-tile and share its activations in L2.
 template <bool ZP_TABLE, bool PRESCALE, int NT, int GPB>
 __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const BatchGroupTable tab,
+                                                                        const BatchGroupItem* __restrict__ dev_tab,
+                                                                        const RoutedHeader* __restrict__ dev_hdr,
                                                                         float* __restrict__ ws,
                                                                         unsigned* __restrict__ counters, int N, int K,
                                                                         int kb_total, int kb_per_group, int ng,
                                                                         int zp_const, int out_f32, int glu,
                                                                         int tiles_x, int tiles_y, int full_tiles,
                                                                         int tail_split, int kb_per_split) {
+    // the table travels in the kernel arguments, or -- when the rows were bucketed on the device -- lies in memory,
+    // with the slice count and the cut along K that the routing kernel chose for it
+    if (dev_tab) {
+        const RoutedHeader h = *dev_hdr;
+        if ((int)blockIdx.x >= h.grid)
+            return;
+        tiles_y = h.tiles_y, tail_split = h.split_k, kb_per_split = h.kb_per_split;
+        full_tiles = h.split_k == 1 ? tiles_x * tiles_y : 0;
+    }
     TileWork wk = tile_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT, PA_BN / 2);
-    const BatchGroupItem& it = tab.item[wk.tile_y];
+    const BatchGroupItem it = dev_tab ? dev_tab[wk.tile_y] : tab.item[wk.tile_y];
     if (it.M <= 0)
         return;
     wk.m0 = 0;
@@ -443,30 +454,32 @@ static int launch_async_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStre
 }
 
 template <bool ZPT, bool PRE, int NT, int GPB>
-static int launch_async_grouped_gpb(const BatchGroupTable& tab, const FcDeviceArgs& a, const LaunchPlan& p,
+static int launch_async_grouped_gpb(const BatchGroupTable& tab, const BatchGroupItem* dev_tab,
+                                    const RoutedHeader* dev_hdr, const FcDeviceArgs& a, const LaunchPlan& p,
                                     hipStream_t s) {
     const Layout& L = a.layout;
     auto kern = fcc_prefill_async_grouped_kernel<ZPT, PRE, NT, GPB>;
     static bool attr_set = false;  // per instantiation
     if (int e = allow_lds(kern, &attr_set, pa_lds_bytes(GPB)))
         return e;
-    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(GPB), s, tab, a.workspace,
-                       a.counters, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(GPB), s, tab, dev_tab,
+                       dev_hdr, a.workspace, a.counters, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
                        L.zp_const, a.out_f32, L.glu, p.tiles_x, p.tiles_y, p.full_tiles, p.split_k,
                        p.kblocks_per_split);
     return (int)hipGetLastError();
 }
 
 template <bool ZPT, bool PRE, int NT>
-static int launch_async_grouped_impl(const BatchGroupTable& tab, const FcDeviceArgs& a, const LaunchPlan& p,
+static int launch_async_grouped_impl(const BatchGroupTable& tab, const BatchGroupItem* dev_tab,
+                                     const RoutedHeader* dev_hdr, const FcDeviceArgs& a, const LaunchPlan& p,
                                      hipStream_t s) {
     if constexpr (PRE) {
         if (a.layout.groups_per_kblock == 2)
-            return launch_async_grouped_gpb<ZPT, PRE, NT, 2>(tab, a, p, s);
+            return launch_async_grouped_gpb<ZPT, PRE, NT, 2>(tab, dev_tab, dev_hdr, a, p, s);
         if (a.layout.groups_per_kblock == 4)
-            return launch_async_grouped_gpb<ZPT, PRE, NT, 4>(tab, a, p, s);
+            return launch_async_grouped_gpb<ZPT, PRE, NT, 4>(tab, dev_tab, dev_hdr, a, p, s);
     }
-    return launch_async_grouped_gpb<ZPT, PRE, NT, 1>(tab, a, p, s);
+    return launch_async_grouped_gpb<ZPT, PRE, NT, 1>(tab, dev_tab, dev_hdr, a, p, s);
 }
 
 // dispatch on zero-point table, per-group scales and tile height
@@ -486,18 +499,38 @@ int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& p, void* strea
     return OVFCC_ASYNC_DISPATCH(launch_async_impl, a, p, s);
 }
 
-// p plans one node of n_items * tile_m rows: its tile rows are the items of the table.
+// p plans one node of n_items * tile_m rows: its tile rows are the items of the table.  dev_tab and dev_hdr
+// (optional, both or none): table and header in device memory, written by the routing kernel earlier on the same
+// stream -- at most n_items entries of at most tile_m rows each; how many are in use and how K is cut for them is
+// the header's word, and p only sizes the launch: a 1-D grid, workspace and counters that hold
+// routed_header(tiles_x, t, k_blocks, .).grid workgroups for every t <= n_items.  `tab` is then ignored and n_items
+// is not limited to kMaxGroupItems.
 int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& p,
-                                 void* stream) {
+                                 void* stream, const BatchGroupItem* dev_tab, const RoutedHeader* dev_hdr) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
-    if (L.bits != 4 || !async_plan_ok(a, p) || n_items < 1 || n_items > kMaxGroupItems || p.tiles_y != n_items)
+    if (L.bits != 4 || n_items < 1 || p.tiles_y != n_items || !dev_tab != !dev_hdr)
         return (int)hipErrorInvalidValue;
-    for (int i = 0; i < n_items; ++i)
-        if (tab.item[i].M < 1 || tab.item[i].M > p.tile_m)
+    if (!dev_tab) {
+        if (!async_plan_ok(a, p) || n_items > kMaxGroupItems)
             return (int)hipErrorInvalidValue;
+        for (int i = 0; i < n_items; ++i)
+            if (tab.item[i].M < 1 || tab.item[i].M > p.tile_m)
+                return (int)hipErrorInvalidValue;
+    } else {
+        if ((p.tile_m != PA_BM && p.tile_m != PA_BM / 2) || p.tiles_x != a.N / PA_BN || p.grid[1] != 1 || p.grid[2] != 1)
+            return (int)hipErrorInvalidValue;
+        for (int t = 1; t <= n_items; ++t) {
+            const RoutedHeader h = routed_header(p.tiles_x, t, (int)L.k_blocks, p.n_cus);
+            if ((unsigned)h.grid > p.grid[0] ||
+                (h.split_k > 1 && (!a.workspace || !a.counters ||
+                                   (size_t)h.grid * p.tile_m * PA_BN * sizeof(float) > p.workspace_bytes ||
+                                   (size_t)p.tiles_x * t > p.counter_count)))
+                return (int)hipErrorInvalidValue;
+        }
+    }
     const bool nt8 = p.tile_m == PA_BM;
-    return OVFCC_ASYNC_DISPATCH(launch_async_grouped_impl, tab, a, p, s);
+    return OVFCC_ASYNC_DISPATCH(launch_async_grouped_impl, tab, dev_tab, dev_hdr, a, p, s);
 }
 #undef OVFCC_ASYNC_DISPATCH
 

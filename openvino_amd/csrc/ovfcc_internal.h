@@ -111,6 +111,9 @@ struct FcDeviceArgs {
     int64_t N_out;       // row length of y: N, or N / 2 with a gated-linear-unit epilogue
     int gate_offset, up_offset;  // untiled layout with such an epilogue: first gate / up channel
     int tile_rows = 0;   // async prefill kernel: 64 or 128 forces the tile height, 0 leaves it to the planner
+    bool want_async = false;  // take the all-asynchronous prefill kernel wherever it can run the node, also where
+                              // smaller tiles would spread a small node further (a slice table in device memory
+                              // has no other reader)
     Layout layout;
 };
 
@@ -134,6 +137,7 @@ struct LaunchPlan {
     unsigned dynamic_lds = 0;   // bytes of dynamic LDS (decode kernel: the cross-wave reduction buffer)
     size_t workspace_bytes = 0;
     size_t counter_count = 0;
+    int n_cus = 0;  // routed grouped launches: the compute-unit count that the cut along K is chosen for on the device
     const char* name = "";
 };
 
@@ -171,8 +175,53 @@ struct BatchGroupTable {
 int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& plan,
                          void* stream);
 // Same table, items of at most 128 rows, 4-bit async prefill kernel; plan is that of one node of 128 * n_items rows.
+#ifdef __HIPCC__
+#define OVFCC_HOST_DEVICE __host__ __device__
+#else
+#define OVFCC_HOST_DEVICE
+#endif
+// What a grouped launch whose slice count is known only on the device reads there: the routing kernel counts the
+// slices and cuts K by the rule below, the host sizes grid, workspace and counters for the worst slice count.
+struct RoutedHeader {
+    int tiles_y;       // slices in use
+    int split_k;       // parts along K of every tile (1: whole tiles)
+    int kb_per_split;  // k-blocks per part
+    int grid;          // workgroups with work: tiles_x * tiles_y * split_k
+};
+// K is split while the tiles alone leave compute units idle and every part keeps at least eight k-blocks (the
+// planner's rule for the register-fed prefill kernels).
+OVFCC_HOST_DEVICE inline RoutedHeader routed_header(int tiles_x, int slices, int kb_total, int n_cus) {
+    const long long tiles = (long long)tiles_x * slices;
+    int split = 1;
+    while (split < 8 && tiles * split * 2 <= n_cus && kb_total / (split * 2) >= 8)
+        split *= 2;
+    const int per = (kb_total + split - 1) / split;
+    split = (kb_total + per - 1) / per;
+    RoutedHeader h;
+    h.tiles_y = slices, h.split_k = split, h.kb_per_split = per, h.grid = (int)(tiles * split);
+    return h;
+}
 int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& plan,
-                                 void* stream);
+                                 void* stream, const BatchGroupItem* dev_tab = nullptr,
+                                 const RoutedHeader* dev_hdr = nullptr);
+// Routing of a mixture-of-experts layer on the device: buckets the R = M * top_k (row, selection) pairs of
+// indices [M, top_k] (device memory) by expert, ascending inside a bucket, and writes the row maps and the slice
+// table that the gather kernel and the grouped launch read -- first[slot] = row of A that bucket slot `slot`
+// reads (m, or i * M + m with one batch of A per selection); second[slot] = i * M + m (inverse == 0) or
+// second[m * top_k + i] = slot, -1 for an index outside [0, n_experts) (inverse != 0); table[.] = the experts' rows
+// cut into equal slices of at most `cap` rows, n_slices_max = ceil(R / cap) + n_experts entries, unused ones with
+// M = 0; *header = routed_header(tiles_x, slices in use, kb_total, n_cus).  x_base / y_base: where bucket slot 0's
+// gathered row and result row lie.
+struct ExpertPointers {
+    const void* w[kMaxGroupItems];
+    const void* scale[kMaxGroupItems];
+    const void* zp[kMaxGroupItems];
+    const void* bias[kMaxGroupItems];
+};
+int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts, int a_batches, int inverse, int cap,
+                     const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
+                     size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
+                     RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream);
 int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);

@@ -232,7 +232,7 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             for (int split = 1; split < 8 && reach * 2 <= n_cus && L.k_blocks / (split * 2) >= 8; split *= 2)
                 reach *= 2;
         }
-        bool big = reach * 2 >= n_cus;
+        bool big = reach * 2 >= n_cus || (a.want_async && may_async);
         const int wide_env = env_int("OVFCC_PREFILL_WIDE", -1);
         if (wide_env >= 0)
             big = wide_env != 0;

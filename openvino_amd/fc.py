@@ -282,8 +282,19 @@ class InferRequest:
                                                          idx.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), M, top_k,
                                                          ctypes.c_void_p(y_ptr)))
 
-    def gather_matmul(self, experts: Sequence[CompressedWeights], A: np.ndarray, indices: np.ndarray) -> np.ndarray:
-        """Host convenience: A float16 [a_batches, M, K] (a_batches 1 or top_k), indices [M, top_k] -> Y [top_k, M, N_out]."""
+    def gather_matmul_routed_device(self, experts: Sequence[CompressedWeights], a_ptr: int, a_batches: int,
+                                    indices_ptr: int, M: int, top_k: int, y_ptr: int) -> None:
+        """The same with the indices int32 [M, top_k] in device memory at indices_ptr: bucketed on the device."""
+        arr = (ctypes.c_void_p * len(experts))(*[w.handle for w in experts])
+        check(self.device.lib.ovfcc_gather_matmul_routed_device(self.handle, arr, len(experts), ctypes.c_void_p(a_ptr),
+                                                                a_batches, ctypes.c_void_p(indices_ptr), M, top_k,
+                                                                ctypes.c_void_p(y_ptr)))
+
+    def gather_matmul(self, experts: Sequence[CompressedWeights], A: np.ndarray, indices: np.ndarray,
+                      device_indices: bool = False, y_fill: Optional[float] = None) -> np.ndarray:
+        """Host convenience: A float16 [a_batches, M, K] (a_batches 1 or top_k), indices [M, top_k] -> Y [top_k, M, N_out].
+        device_indices: the indices are uploaded and the device-routed entry point is called; y_fill: Y is
+        preset to this value (rows that no expert writes keep it)."""
         A = np.ascontiguousarray(A, dtype=np.float16)
         idx = np.ascontiguousarray(indices, dtype=np.int32)
         M, top_k = idx.shape
@@ -295,14 +306,23 @@ class InferRequest:
             return np.empty((top_k, 0, w.N_out), dt)
         dev = self.device
         a_ptr, y_ptr = dev.malloc(A.nbytes), dev.malloc(top_k * M * w.N_out * np.dtype(dt).itemsize)
+        i_ptr = dev.malloc(max(idx.nbytes, 16)) if device_indices else None
         try:
             dev.upload(a_ptr, A)
-            self.gather_matmul_device(experts, a_ptr, A.shape[0], idx, y_ptr)
+            if y_fill is not None:
+                dev.upload(y_ptr, np.full((top_k, M, w.N_out), y_fill, dt))
+            if device_indices:
+                dev.upload(i_ptr, idx)
+                self.gather_matmul_routed_device(experts, a_ptr, A.shape[0], i_ptr, M, top_k, y_ptr)
+            else:
+                self.gather_matmul_device(experts, a_ptr, A.shape[0], idx, y_ptr)
             self.sync()
             return dev.download(y_ptr, (top_k, M, w.N_out), dt)
         finally:
             dev.free(a_ptr)
             dev.free(y_ptr)
+            if i_ptr:
+                dev.free(i_ptr)
 
     def moe_device(self, gate_up: Sequence[CompressedWeights], down: Sequence[CompressedWeights], x_ptr: int,
                    routing_ptr: int, indices: np.ndarray, y_ptr: int) -> None:
@@ -318,9 +338,19 @@ class InferRequest:
                                                idx.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), M, top_k,
                                                ctypes.c_void_p(y_ptr)))
 
+    def moe_routed_device(self, gate_up: Sequence[CompressedWeights], down: Sequence[CompressedWeights], x_ptr: int,
+                          routing_ptr: int, indices_ptr: int, M: int, top_k: int, y_ptr: int) -> None:
+        """The same with the indices int32 [M, top_k] in device memory at indices_ptr: bucketed on the device."""
+        g = (ctypes.c_void_p * len(gate_up))(*[w.handle for w in gate_up])
+        d = (ctypes.c_void_p * len(down))(*[w.handle for w in down])
+        check(self.device.lib.ovfcc_moe_routed_device(self.handle, g, d, len(gate_up), ctypes.c_void_p(x_ptr),
+                                                      ctypes.c_void_p(routing_ptr), ctypes.c_void_p(indices_ptr), M,
+                                                      top_k, ctypes.c_void_p(y_ptr)))
+
     def moe(self, gate_up: Sequence[CompressedWeights], down: Sequence[CompressedWeights], x: np.ndarray,
-            routing: np.ndarray, indices: np.ndarray) -> np.ndarray:
-        """Host convenience: x float16 [M, H], routing float16 [M, top_k], indices [M, top_k] -> Y [M, H]."""
+            routing: np.ndarray, indices: np.ndarray, device_indices: bool = False) -> np.ndarray:
+        """Host convenience: x float16 [M, H], routing float16 [M, top_k], indices [M, top_k] -> Y [M, H].
+        device_indices: the indices are uploaded and the device-routed entry point is called."""
         x = np.ascontiguousarray(x, dtype=np.float16)
         routing = np.ascontiguousarray(routing, dtype=np.float16)
         idx = np.ascontiguousarray(indices, dtype=np.int32)
@@ -333,16 +363,23 @@ class InferRequest:
             return np.empty((0, H), dt)
         dev = self.device
         x_ptr, r_ptr, y_ptr = dev.malloc(x.nbytes), dev.malloc(max(routing.nbytes, 16)), dev.malloc(M * H * np.dtype(dt).itemsize)
+        i_ptr = dev.malloc(max(idx.nbytes, 16)) if device_indices else None
         try:
             dev.upload(x_ptr, x)
             dev.upload(r_ptr, routing)
-            self.moe_device(gate_up, down, x_ptr, r_ptr, idx, y_ptr)
+            if device_indices:
+                dev.upload(i_ptr, idx)
+                self.moe_routed_device(gate_up, down, x_ptr, r_ptr, i_ptr, M, top_k, y_ptr)
+            else:
+                self.moe_device(gate_up, down, x_ptr, r_ptr, idx, y_ptr)
             self.sync()
             return dev.download(y_ptr, (M, H), dt)
         finally:
             dev.free(x_ptr)
             dev.free(r_ptr)
             dev.free(y_ptr)
+            if i_ptr:
+                dev.free(i_ptr)
 
     def bench_grouped(self, items: Sequence[tuple], warmup: int, iters: int) -> float:
         """Milliseconds for `iters` grouped runs, HIP events on the launching stream."""

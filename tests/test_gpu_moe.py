@@ -98,3 +98,84 @@ def test_moe_rejects_what_it_cannot_run(oracle, dev, req):
     finally:
         for w in wg + wd + plain_gate:
             w.close()
+
+
+@pytest.mark.parametrize("M", [1, 7, 48, 300, 1100])
+@pytest.mark.parametrize("wt,zt,G,kind,out", [("u4", "u4", 128, "swish", "f16"), ("i4", "none", 128, "gelu_tanh", "f32")])
+def test_moe_block_routed_on_the_device(oracle, dev, req, monkeypatch, M, wt, zt, G, kind, out):
+    """The same block with the indices in device memory: the buckets are cut by the routing kernel.  Against the
+    oracle, and against the call that buckets on the host: bit for bit where that call also runs the grouped
+    prefill kernel (a row's result does not depend on the slice it sits in), otherwise -- few rows per expert run
+    node by node through the decode kernels -- within the rounding of the f16 results."""
+    E, top_k, H, I = 8, 2, 256, 512
+    say(f"moe routed {wt}/{zt} G={G} {kind} out={out} M={M}")
+    gu, dn = make_layer(930, E, H, I, wt=wt, zt=zt, G=G)
+    wg = [fc.CompressedWeights.from_case(dev, c, glu=kind) for c in gu]
+    wd = [fc.CompressedWeights.from_case(dev, c, output_type=out) for c in dn]
+    idx, routing = routed(931 + M, M, E, top_k)
+    x = np.random.default_rng(932).standard_normal((M, H)).astype(np.float16)
+    glu_type = {"swish": 1, "gelu": 2, "gelu_tanh": 3}[kind]
+    try:
+        y = req.moe(wg, wd, x, routing, idx, device_indices=True)
+        assert req.last_kernel()["name"] == "fcc_prefill_async_grouped_w4"
+        ref = oracle.moe_reference(x, routing, idx, [expert_args(c) for c in gu], [expert_args(c) for c in dn], glu_type)
+        check(oracle, y, ref, max(H, I), f"M={M} routed")
+        assert np.array_equal(req.moe(wg, wd, x, routing, idx, device_indices=True).view(np.uint8), y.view(np.uint8))
+        assert np.array_equal(req.moe(wg, wd, x, routing, idx).view(np.uint8), y.view(np.uint8))  # uploads, then routes
+        monkeypatch.setenv("OVFCC_MOE_HOST_ROUTING", "1")
+        monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+        y_host = req.moe(wg, wd, x, routing, idx)
+        if req.last_kernel()["name"] == "fcc_prefill_async_grouped_w4":
+            assert np.array_equal(y_host.view(np.uint8), y.view(np.uint8)), "host- and device-routed results differ"
+        else:
+            check(oracle, y_host, ref, max(H, I), f"M={M} host-routed")
+            assert M < 300
+    finally:
+        for w in wg + wd:
+            w.close()
+
+
+def test_moe_routed_index_outside_the_experts(oracle, dev, req):
+    """Device indices cannot be checked without waiting for them: a pair whose index names no expert adds nothing
+    to its row; every other row is what it is without that pair."""
+    E, top_k, H, I, M = 8, 2, 256, 512, 40
+    say("moe routed, bad index")
+    gu, dn = make_layer(950, E, H, I)
+    wg = [fc.CompressedWeights.from_case(dev, c, glu="swish") for c in gu]
+    wd = [fc.CompressedWeights.from_case(dev, c) for c in dn]
+    idx, routing = routed(951, M, E, top_k)
+    x = np.random.default_rng(952).standard_normal((M, H)).astype(np.float16)
+    try:
+        good = req.moe(wg, wd, x, routing, idx, device_indices=True)
+        bad = idx.copy()
+        bad[3, 1], bad[17, 0], bad[39, 1] = E, -1, 1 << 20
+        got = req.moe(wg, wd, x, routing, bad, device_indices=True)
+        zeroed = routing.copy()
+        zeroed[3, 1], zeroed[17, 0], zeroed[39, 1] = 0, 0, 0
+        want = req.moe(wg, wd, x, zeroed, idx, device_indices=True)
+        rows = [3, 17, 39]
+        keep = np.setdiff1d(np.arange(M), rows)
+        assert np.array_equal(got[keep].view(np.uint16), good[keep].view(np.uint16))
+        assert np.array_equal(got[rows].view(np.uint16), want[rows].view(np.uint16))
+    finally:
+        for w in wg + wd:
+            w.close()
+
+
+def test_moe_routed_refuses_what_only_the_host_route_runs(oracle, dev, req):
+    """8-bit experts have no grouped launch with a table in device memory: OVFCC_EUNSUPPORTED, while the
+    host-index call runs them."""
+    E, H, I = 4, 256, 512
+    gu, dn = make_layer(960, E, H, I, wt="u8", zt="u8", G=256)
+    wg = [fc.CompressedWeights.from_case(dev, c, glu="swish") for c in gu]
+    wd = [fc.CompressedWeights.from_case(dev, c) for c in dn]
+    idx, routing = routed(961, 6, E, 2)
+    x = np.random.default_rng(962).standard_normal((6, H)).astype(np.float16)
+    try:
+        with pytest.raises(fc.OvfccError) as err:
+            req.moe(wg, wd, x, routing, idx, device_indices=True)
+        assert err.value.code == -2            # OVFCC_EUNSUPPORTED
+        assert req.moe(wg, wd, x, routing, idx).shape == (6, H)
+    finally:
+        for w in wg + wd:
+            w.close()
