@@ -57,7 +57,7 @@ typedef struct ovfcc_fc_desc {
     int32_t bias_type;  /* OVFCC_NONE | OVFCC_F16, [N] */
     int32_t act_type;   /* OVFCC_F16 */
     int32_t out_type;   /* OVFCC_F16 | OVFCC_F32 (FullyConnected's output_type; default = activation type) */
-    int32_t flags;      /* 0, or OVFCC_GLU_* [| OVFCC_GLU_GATE_SECOND] | OVFCC_DYNQUANT_I8 | OVFCC_W_INPUT_MAJOR */
+    int32_t flags;      /* 0, or OVFCC_GLU_* [| OVFCC_GLU_GATE_SECOND] | OVFCC_DYNQUANT_I8 [| OVFCC_DYNQUANT_PER_GROUP] | OVFCC_W_INPUT_MAJOR */
 } ovfcc_fc_desc;
 
 /* Gated linear unit fused into the node (flags).  The reference fuses ov::op::internal::GLU
@@ -93,6 +93,19 @@ typedef struct ovfcc_fc_desc {
  * integers exact, which differs from the f16 result by the quantisation noise (about 1e-2 relative; the
  * reference tests such nodes with absolute tolerances of 0.1-0.2). */
 #define OVFCC_DYNQUANT_I8 8
+
+/* With OVFCC_DYNQUANT_I8, for 4-bit weights with one scale (and zero-point) per group of 128 inputs (W4A8): the
+ * reference quantises the source of such a node too -- the CPU plugin in groups of
+ * ov::hint::dynamic_quantization_group_size inputs (src/plugins/intel_cpu/src/nodes/executors/dnnl/
+ * dnnl_fullyconnected_primitive.cpp:161-241,284-298), the GPU plugin per token on matrix-engine hardware and per
+ * group elsewhere (src/plugins/intel_gpu/src/plugin/transformations/dynamic_quantize_fully_connected.cpp:24-140,
+ * src/plugins/intel_gpu/src/runtime/execution_config.cpp:348-354).  OVFCC_DYNQUANT_I8 alone quantises per token;
+ * with OVFCC_DYNQUANT_PER_GROUP every group of 128 inputs of a row has its own scale (group size = the weights'
+ * group).  Takes effect for u4 / i4 weights, G = 128, zero-points none, scalar or a u4 table, N % 256 == 0 and more
+ * than 48 rows:
+ *     y[m, n] = sum_g ( sum_{k in g} q[m, k] (W[n, k] - ZP[n, g]) ) * S[n, g] * inv_scale[m (, g)]  + bias[n],
+ * q and inv_scale as above over a row or a group, the integer sums exact, the sum over groups in f32. */
+#define OVFCC_DYNQUANT_PER_GROUP 32
 
 /* Input-major constants (flags): W is given as [K, N] (grouped: [K/G, G, N]) and scales / zero-points as
  * [K/G, N], each packed over its own flattened index -- the form in which a MatMul with transpose_b = false holds

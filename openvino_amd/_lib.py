@@ -14,7 +14,8 @@ KERNEL_AUTO, KERNEL_PLAIN, KERNEL_DECODE, KERNEL_PREFILL = range(4)
 GLU = {None: 0, "none": 0, "swish": 1, "gelu": 2, "gelu_tanh": 3}      # OVFCC_GLU_*
 GLU_GATE_SECOND = 4
 DYNQUANT_I8 = 8                                                        # OVFCC_DYNQUANT_I8
-W_INPUT_MAJOR = 16                                                     # OVFCC_W_INPUT_MAJOR
+W_INPUT_MAJOR = 16
+DYNQUANT_PER_GROUP = 32                                                # OVFCC_DYNQUANT_PER_GROUP                                                     # OVFCC_W_INPUT_MAJOR
 
 # every symbol include/ovfcc.h declares
 SYMBOLS = [

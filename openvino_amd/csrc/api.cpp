@@ -322,6 +322,38 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
         record(r, shown);
         return OVFCC_OK;
     }
+    // The same permission for 4-bit weights with groups of 128 inputs (W4A8): activations per token, or per row
+    // and group where the node asks for it.
+    if (L0.dynquant && ovfcc::prefill_i8w4_applies(L0, w->desc.N, w->desc.zp_type) && M > ovfcc::kDecodeMaxRows &&
+        (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL) && M * w->desc.K < ((int64_t)1 << 31) &&
+        (M + 127) / 128 <= 65535 &&
+        ((w->desc.N / 256) * ((M + 127) / 128) * 2 >= r->ctx->n_cus ||
+         (std::getenv("OVFCC_PREFILL_WIDE") && std::atoi(std::getenv("OVFCC_PREFILL_WIDE")) == 1))) {
+        if (static_scratch)
+            return fail(OVFCC_EUNSUPPORTED, "a node with int8 activations needs a quantisation buffer of the request");
+        const bool grouped = L0.dynquant_grouped;
+        const size_t q_bytes = ((size_t)M * w->desc.K + 255) & ~(size_t)255;
+        const size_t need = q_bytes + ovfcc::dynquant_w4_scale_floats(M, w->desc.K, grouped) * sizeof(float);
+        if (need > r->quant_cap)
+            HIP_TRY(hipStreamSynchronize(r->stream));
+        int rc = grow(&r->d_quant, &r->quant_cap, need);
+        if (rc)
+            return rc;
+        char* base = static_cast<char*>(r->d_quant);
+        float* inv_scale = reinterpret_cast<float*>(base + q_bytes);
+        int e = ovfcc::launch_dynquant_w4(x, base, inv_scale, M, w->desc.K, grouped, r->stream);
+        if (!e)
+            e = ovfcc::launch_prefill_i8w4(a, base, inv_scale, grouped, r->stream);
+        if (e)
+            return hip_fail((hipError_t)e, "integer kernel launch");
+        ovfcc::LaunchPlan shown;
+        shown.kernel = OVFCC_KERNEL_PREFILL;
+        shown.tile_m = 128, shown.tile_n = 256, shown.block = 512;
+        shown.grid[0] = (unsigned)(w->desc.N / 256), shown.grid[1] = (unsigned)((M + 127) / 128);
+        shown.name = grouped ? "fcc_prefill_i8_w4_grouped" : "fcc_prefill_i8_w4";
+        record(r, shown);
+        return OVFCC_OK;
+    }
     bool chunked = w->layout.tiled && M > ovfcc::kDecodeMaxRows &&
                    ((force == OVFCC_KERNEL_AUTO && M <= ovfcc::kChunkedMaxRows) ||
                     ((w->desc.N % 128) != 0 && (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL)));

@@ -51,7 +51,8 @@ struct Layout {
     bool glu_gate_second = false;
     int gemv_c = 0;         // k-blocks per wave of the matrix-vector kernel, fixed when the node's channel-major
                             // parameter tables are written (0: the node has none)
-    bool dynquant = false;  // the node allows per-token int8 activations (OVFCC_DYNQUANT_I8) where a kernel exists
+    bool dynquant = false;  // the node allows int8 activations (OVFCC_DYNQUANT_I8) where a kernel exists
+    bool dynquant_grouped = false;  // ... quantised per group of 128 inputs rather than per token (4-bit nodes)
     // element index of the scale / zero-point of channel r of tile nt for group g
     size_t param_index(int64_t nt, int64_t g, int r) const {
         if (groups_per_kblock == 1)
@@ -230,6 +231,13 @@ int launch_prefill_big(const FcDeviceArgs& a, const LaunchPlan& plan, void* stre
 // Per-row int8 quantisation of x [M, K] f16 (K % 128 == 0): xq [M, K] in the weight tiles' input order, one
 // inverse scale and one sum of quantised values per row.
 int launch_dynquant(const void* x, void* xq, float* inv_scale, int* qsum, int64_t M, int64_t K, void* stream);
+// The same for tiled 4-bit weights with one group per 128 inputs (W4A8): activations quantised per token
+// (inv [M]) or per row and k-block (grouped; inv holds dynquant_w4_scale_floats floats), the integer kernel over
+// them, and whether that kernel can run a node.
+size_t dynquant_w4_scale_floats(int64_t M, int64_t K, bool grouped);
+int launch_dynquant_w4(const void* x, void* xq, float* inv, int64_t M, int64_t K, bool grouped, void* stream);
+bool prefill_i8w4_applies(const Layout& L, int64_t N, int zp_type);
+int launch_prefill_i8w4(const FcDeviceArgs& a, const void* xq, const float* inv, bool grouped, void* stream);
 // Integer prefill kernel over launch_dynquant's outputs: tiled 8-bit weights, one group per channel, N % 256 == 0.
 int launch_prefill_i8(const FcDeviceArgs& a, const void* xq, const float* inv_scale, const int* qsum, void* stream);
 int launch_copy(void* dst, const void* src, size_t bytes, void* stream);

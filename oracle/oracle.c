@@ -383,6 +383,51 @@ int ovo_fc_dynquant_reference(const int8_t* q, const float* inv_scale, const int
     return 0;
 }
 
+/* The same quantisation over groups of G consecutive inputs of a row instead of whole rows (the reference's
+ * DynamicQuantize with group_sizes = {1, .., G}, src/plugins/intel_gpu/src/kernel_selector/cl_kernels/
+ * dynamic_quantize_gpu_ref.cl:100-250 with GROUP_SIZE_DIM3 = G; on the CPU the source group of
+ * src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_fullyconnected_primitive.cpp:161-241,284-298):
+ * q [M, K], inv_scale [M, K / G], qsum [M, K / G].  G = K is ovo_dynquant_rows. */
+int ovo_dynquant_groups(const uint16_t* x, int64_t M, int64_t K, int64_t G, int8_t* q, float* inv_scale,
+                        int32_t* qsum) {
+    if (!x || !q || !inv_scale || !qsum || M < 0 || K <= 0 || G <= 0 || K % G)
+        return -1;
+    /* a [M, K] matrix cut into groups of G along K is a [M K / G, G] matrix cut into rows */
+    return ovo_dynquant_rows(x, M * (K / G), G, q, inv_scale, qsum);
+}
+
+/* FullyConnected over activations quantised in groups of Ga inputs, 4- or 8-bit weights with scales (and
+ * zero-points) per group of Gw inputs; Ga and Gw divide K and one of them divides the other.  With
+ * g = min(Ga, Gw):
+ *     y[m, n] = sum_blocks-of-g ( sum_{k in block} q[m, k] (w[n, k] - zp[n, k / Gw]) ) * scale[n, k / Gw]
+ *               * inv_scale[m, k / Ga]  (+ bias[n]),
+ * the integer sums exact, the sum over blocks in double.  w holds one code per byte ([N, K], already unpacked;
+ * w_signed: two's complement), zp one value per (n, group) or null (0); scale [N, K / Gw] f32. */
+int ovo_fc_dynquant_grouped_reference(const int8_t* q, const float* inv_scale, int64_t M, int64_t K, int64_t Ga,
+                                      int64_t N, const uint8_t* w, int32_t w_signed, int64_t Gw, const float* scale,
+                                      const float* zp, const float* bias, float* y) {
+    if (!q || !inv_scale || !w || !scale || !y || M < 0 || K <= 0 || N <= 0 || Ga <= 0 || Gw <= 0 || K % Ga || K % Gw ||
+        (Ga % Gw && Gw % Ga))
+        return -1;
+    const int64_t g = Ga < Gw ? Ga : Gw, nga = K / Ga, ngw = K / Gw;
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t m = 0; m < M; ++m) {
+            double sum = 0.0;
+            for (int64_t k0 = 0; k0 < K; k0 += g) {
+                const int32_t z = zp ? (int32_t)zp[n * ngw + k0 / Gw] : 0;
+                int64_t acc = 0;
+                for (int64_t k = k0; k < k0 + g; ++k) {
+                    const int32_t wv = w_signed ? (int32_t)(int8_t)w[n * K + k] : (int32_t)w[n * K + k];
+                    acc += (int32_t)q[m * K + k] * (wv - z);
+                }
+                sum += (double)acc * ((double)scale[n * ngw + k0 / Gw] * (double)inv_scale[m * nga + k0 / Ga]);
+            }
+            y[m * N + n] = (float)(sum + (bias ? (double)bias[n] : 0.0));
+        }
+    return 0;
+}
+
 int ovo_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

@@ -276,6 +276,59 @@ def fc_dynquant_reference(x, w, w_type, scale, zp=None, bias=None, *, N, K) -> n
     return y
 
 
+def dynquant_groups(x, G):
+    """C oracle: symmetric int8 quantisation of x [M, K] float16 in groups of G inputs -> (q int8 [M, K],
+    inv_scale float32 [M, K / G], qsum int32 [M, K / G])."""
+    x = np.ascontiguousarray(x, dtype=np.float16)
+    M, K = x.shape
+    q, inv, qs = np.empty((M, K), np.int8), np.empty((M, K // G), np.float32), np.empty((M, K // G), np.int32)
+    f = lib().ovo_dynquant_groups
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p,
+                  ctypes.c_void_p]
+    if f(_ptr(x), M, K, G, _ptr(q), _ptr(inv), _ptr(qs)) != 0:
+        raise ValueError("ovo_dynquant_groups rejected its arguments")
+    return q, inv, qs
+
+
+def _codes(packed, type_, n):
+    """One code per byte (two's complement for the signed types) from n packed 4- or 8-bit elements."""
+    if type_ == U4:
+        return unpack_u4(packed, n)
+    if type_ == I4:
+        return unpack_i4(packed, n).view(np.uint8)
+    return np.ascontiguousarray(packed).view(np.uint8).ravel()[:n].copy()
+
+
+def fc_dynquant_grouped_reference(x, w, w_type, scale, zp=None, zp_type=NONE, bias=None, *, N, K, group_size,
+                                  act_group, zp_scalar=False) -> np.ndarray:
+    """C oracle of the FullyConnected with int8 activations quantised in groups of act_group inputs (K: per token)
+    over 4- or 8-bit weights with scales / zero-points per group of group_size inputs.  w, zp packed as for
+    fc_reference.  Returns float32 [M, N]."""
+    q, inv, _ = dynquant_groups(np.asarray(x).reshape(-1, K), act_group)
+    M = q.shape[0]
+    ng = K // group_size
+    codes = _codes(w, w_type, N * K)
+    scale = np.ascontiguousarray(np.asarray(scale, dtype=np.float32).reshape(N, ng))
+    if zp is None or zp_type == NONE:
+        zpf = None
+    else:
+        z = _codes(zp, zp_type, 1 if zp_scalar else N * ng).astype(np.float32)
+        zpf = np.ascontiguousarray(np.broadcast_to(z, (N, ng)) if zp_scalar else z.reshape(N, ng), dtype=np.float32)
+    bias = None if bias is None else np.ascontiguousarray(np.asarray(bias, dtype=np.float32).reshape(N))
+    y = np.empty((M, N), np.float32)
+    f = lib().ovo_fc_dynquant_grouped_reference
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                  ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                  ctypes.c_void_p]
+    signed = w_type in (I4, I8)
+    if f(_ptr(q), _ptr(inv), M, K, act_group, N, _ptr(codes), int(signed), group_size, _ptr(scale), _ptr(zpf),
+         _ptr(bias), _ptr(y)) != 0:
+        raise ValueError("ovo_fc_dynquant_grouped_reference rejected its arguments")
+    return y
+
+
 # ---- independent numpy restatement (bit operations and float64 matmul) ----
 
 def np_unpack_nibbles(packed: np.ndarray, n: int, signed: bool) -> np.ndarray:

@@ -46,7 +46,7 @@ def test_version_and_error_string():
     (dict(group_size=96), _lib.EINVAL), (dict(w_type=_lib.F16), _lib.EUNSUPPORTED),
     (dict(scale_type=_lib.F32), _lib.EUNSUPPORTED), (dict(zp_type=_lib.I4), _lib.EUNSUPPORTED),
     (dict(act_type=_lib.F32), _lib.EUNSUPPORTED), (dict(out_type=_lib.U8), _lib.EUNSUPPORTED),
-    (dict(bias_type=_lib.F32), _lib.EUNSUPPORTED), (dict(flags=32), _lib.EINVAL),
+    (dict(bias_type=_lib.F32), _lib.EUNSUPPORTED), (dict(flags=32), _lib.EINVAL), (dict(flags=64), _lib.EINVAL),
     (dict(flags=4), _lib.EINVAL), (dict(flags=1, N=63), _lib.EINVAL),
 ])
 def test_descriptor_gate(mutate, code):

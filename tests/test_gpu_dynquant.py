@@ -72,8 +72,9 @@ def test_dynquant_prefill_matches_integer_oracle(oracle, dev, req, monkeypatch, 
 
 
 def test_dynquant_flag_without_a_kernel_is_ignored(oracle, dev, req, monkeypatch):
-    """4-bit weights, grouped scales or a narrow node: the permission has no integer kernel to take effect in; nor
-    does it take effect where the integer kernel's grid would leave most of the chip idle."""
+    """4-bit weights with groups of 64, 8-bit weights with grouped scales or a narrow node: the permission has no
+    integer kernel to take effect in; nor does it take effect where the integer kernel's grid would leave most of the
+    chip idle."""
     say("dynquant ignored")
     c = datagen.make_case(1111, 200, 512, 256, "u8", 512, "u8")
     w = fc.CompressedWeights.from_case(dev, c, dynamic_quantization=True)
@@ -84,12 +85,13 @@ def test_dynquant_flag_without_a_kernel_is_ignored(oracle, dev, req, monkeypatch
     finally:
         w.close()
     monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
-    for wt, zt, N, K, G in (("u4", "u4", 256, 512, 128), ("u8", "u8", 256, 512, 128), ("u8", "u8", 128, 512, 512)):
+    for wt, zt, N, K, G in (("u4", "u4", 256, 512, 64), ("u4", "u8", 256, 512, 128), ("u8", "u8", 256, 512, 128),
+                            ("u8", "u8", 128, 512, 512)):
         c = datagen.make_case(1110, 200, K, N, wt, G, zt)
         w = fc.CompressedWeights.from_case(dev, c, dynamic_quantization=True)
         try:
             y = req.infer(w, c.x)
-            assert req.last_kernel()["name"] != "fcc_prefill_i8_w8"
+            assert not req.last_kernel()["name"].startswith("fcc_prefill_i8")
             check_parity(oracle, y, oracle_y(oracle, c), K, f"{wt} G={G} N={N}", output_rounding_slack=True)
         finally:
             w.close()
@@ -129,3 +131,88 @@ def test_dynquant_with_gated_linear_unit(oracle, dev, req, monkeypatch):
             assert oracle.rel_l2(y, ref) < 2e-6, oracle.rel_l2(y, ref)
         finally:
             w.close()
+
+
+# ---- 4-bit weights with groups of 128 inputs (W4A8) ----
+
+TN = {"none": 0, "u4": 1, "i4": 2, "u8": 3, "i8": 4}
+
+
+def dq4_reference(oracle, c, x, act_group):
+    return oracle.fc_dynquant_grouped_reference(x, c.w, TN[c.w_type], c.scale, c.zp, TN[c.zp_type], c.bias, N=c.N, K=c.K,
+                                                group_size=c.group_size, act_group=act_group, zp_scalar=c.zp_scalar)
+
+
+@pytest.mark.parametrize("mode", ["per_token", "per_group"])
+@pytest.mark.parametrize("wt,zt,N,K,bias,out", [("u4", "u4", 256, 512, True, "f32"), ("u4", "none", 512, 384, False, "f16"),
+                                                ("i4", "none", 256, 1024, True, "f32"), ("u4", "u4", 768, 128, False, "f32")])
+def test_w4a8_prefill_matches_integer_oracle(oracle, dev, req, monkeypatch, mode, wt, zt, N, K, bias, out):
+    """4-bit weights, scales and zero-points per 128 inputs, activations int8 per token or per row and group: the
+    integer sums are exact, so against the oracle of the same arithmetic only the f32 sum over the groups (in k-block
+    order on the GPU, in double in the oracle) and the output rounding differ."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")   # the policy keeps grids this small on the f16 kernels
+    say(f"w4a8 {mode} {wt}/{zt} N={N} K={K} bias={bias} out={out}")
+    c = datagen.make_case(1200, 300, K, N, wt, 128, zt, with_bias=bias)
+    c.x[5] = 0
+    c.x[6] *= 40
+    c.x[7, 130:] *= 25                            # groups of very different range in one row
+    w = fc.CompressedWeights.from_case(dev, c, output_type=out, dynamic_quantization=mode)
+    name = "fcc_prefill_i8_w4_grouped" if mode == "per_group" else "fcc_prefill_i8_w4"
+    try:
+        for M in (49, 128, 129, 300):
+            y = req.infer(w, c.x[:M])
+            assert req.last_kernel()["name"] == name, req.last_kernel()
+            ref = dq4_reference(oracle, c, c.x[:M], 128 if mode == "per_group" else K)
+            tol = 2e-6 if out == "f32" else 5e-4
+            assert oracle.rel_l2(y.astype(np.float32), ref) < tol, (M, oracle.rel_l2(y.astype(np.float32), ref))
+            if out == "f32":
+                assert np.all(np.abs(y - ref) <= 4e-6 * np.max(np.abs(ref)))
+            plain = oracle_y(oracle, c, x=c.x[:M])
+            assert oracle.rel_l2(y.astype(np.float32), plain) < 3e-2
+            assert np.array_equal(req.infer(w, c.x[:M]).view(np.uint8), y.view(np.uint8))
+        y = req.infer(w, c.x[:32])                # decode row counts compute in f16: the flag is a permission
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
+        check_parity(oracle, y, oracle_y(oracle, c, x=c.x[:32]), K, "decode rows", output_rounding_slack=True)
+    finally:
+        w.close()
+
+
+def test_w4a8_scalar_zero_point_and_gated_linear_unit(oracle, dev, req, monkeypatch):
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    say("w4a8 scalar zp + glu")
+    c = datagen.make_case(1210, 200, 512, 512, "u4", 128, "u4", with_bias=True)
+    c.zp, c.zp_scalar = np.array([7], np.uint8), True
+    for kind, second, mode in (("swish", False, "per_group"), ("gelu_tanh", True, "per_token")):
+        w = fc.CompressedWeights.from_case(dev, c, output_type="f32", glu=kind, glu_gate_second=second,
+                                           dynamic_quantization=mode)
+        try:
+            y = req.infer(w, c.x)
+            assert req.last_kernel()["name"].startswith("fcc_prefill_i8_w4") and y.shape == (200, 256)
+            full = dq4_reference(oracle, c, c.x, 128 if mode == "per_group" else c.K)
+            ref = oracle.glu(full, {"swish": 1, "gelu_tanh": 3}[kind], second)
+            assert oracle.rel_l2(y, ref) < 4e-6, oracle.rel_l2(y, ref)
+        finally:
+            w.close()
+
+
+@pytest.mark.parametrize("mode", ["per_token", "per_group"])
+def test_w4a8_llama8b_prefill_shape(oracle, dev, req, mode):
+    """Config 3's q/o projection (4096 -> 4096, i4 g128, outlier channels) at M = 2048 through the integer kernel,
+    sampled rows."""
+    say(f"w4a8 8B q/o {mode}")
+    c = datagen.config3("qo", 2048)
+    w = fc.CompressedWeights.from_case(dev, c, output_type="f32", dynamic_quantization=mode)
+    try:
+        y = req.infer(w, c.x)
+        assert req.last_kernel()["name"].startswith("fcc_prefill_i8_w4")
+        pick = np.array([0, 1, 500, 777, 2047])
+        ref = dq4_reference(oracle, c, c.x[pick], 128 if mode == "per_group" else c.K)
+        assert oracle.rel_l2(y[pick], ref) < 2e-6
+        plain = oracle_y(oracle, c, x=c.x[pick])
+        r = oracle.rel_l2(y[pick], plain)
+        say(f"   rel-L2 against the f16-activation oracle: {r:.2e}")
+        # the configuration's outlier channels (x 20) set a token's scale: per-token noise is several times the
+        # per-group noise, where an outlier only costs its own group of 128 inputs
+        assert r < (2e-2 if mode == "per_group" else 1e-1)
+    finally:
+        w.close()

@@ -63,3 +63,90 @@ def test_fc_dynquant_equals_float_oracle_on_dequantised_activations(oracle, wt, 
     plain = oracle.fc_reference(c.x, c.w, T[wt], c.scale, c.zp, oracle.U8 if zt == "u8" else oracle.NONE, c.bias,
                                 N=c.N, K=c.K, group_size=c.K)
     assert 1e-4 < oracle.rel_l2(y, plain) < 3e-2
+
+
+# ---- quantisation in groups and the integer FullyConnected over grouped weights ----
+
+def test_dynquant_groups_is_the_row_quantisation_of_the_regrouped_matrix(oracle):
+    """Groups of G inputs of a row are rows of the [M K / G, G] view: equality with the numpy restatement applied to
+    that view; G = K gives the per-token result; a group's scale ignores the other groups of its row."""
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((12, 512)) * rng.uniform(0.01, 30, (12, 1))).astype(np.float16)
+    for G in (32, 128, 512):
+        q, inv, qs = oracle.dynquant_groups(x, G)
+        q2, inv2, qs2 = np_dynquant(x.reshape(-1, G))
+        assert np.array_equal(q, q2.reshape(12, 512)) and np.array_equal(inv.ravel(), inv2)
+        assert np.array_equal(qs.ravel(), qs2)
+    qr, invr, qsr = oracle.dynquant_rows(x)
+    q, inv, qs = oracle.dynquant_groups(x, 512)
+    assert np.array_equal(q, qr) and np.array_equal(inv[:, 0], invr) and np.array_equal(qs[:, 0], qsr)
+    x2 = x.copy()
+    x2[:, 128:] *= np.float16(4)                  # other groups change ...
+    qa, inva, _ = oracle.dynquant_groups(x, 128)
+    qb, invb, _ = oracle.dynquant_groups(x2, 128)
+    assert np.array_equal(qa[:, :128], qb[:, :128]) and np.array_equal(inva[:, 0], invb[:, 0])  # ... group 0 does not
+    with pytest.raises(ValueError):
+        oracle.dynquant_groups(x, 100)
+
+
+def np_fc_grouped(q, inv, Ga, codes, Gw, scale, zp, bias):
+    """Independent restatement: dequantise both sides to float64 and multiply."""
+    M, K = q.shape
+    xd = q.astype(np.float64) * np.repeat(inv.astype(np.float64), Ga, axis=1)
+    wd = (codes.astype(np.float64) - (0 if zp is None else np.repeat(zp.astype(np.float64), Gw, axis=1)))
+    wd = wd * np.repeat(scale.astype(np.float64), Gw, axis=1)
+    return xd @ wd.T + (0 if bias is None else bias.astype(np.float64))
+
+
+@pytest.mark.parametrize("wt,zt,Gw,Ga", [("u4", "u4", 128, 128), ("u4", "u4", 128, 512), ("u4", "u4", 128, 32),
+                                         ("i4", "none", 128, 128), ("u8", "u8", 512, 128), ("u4", "u4", 64, 128),
+                                         ("i8", "none", 256, 512)])
+def test_fc_dynquant_grouped_equals_dequantised_product(oracle, wt, zt, Gw, Ga):
+    """The integer form (exact sums per block, scales applied per block) equals the float64 product of the
+    dequantised operands -- with weight groups, activation groups finer, equal or coarser than them, with and without
+    zero-points; and it equals the float oracle run on the dequantised activations where those are exact halves."""
+    c = datagen.make_case(41, 20, 512, 48, wt, Gw, zt, with_bias=True)
+    T = oracle.TYPE_NAMES
+    y = oracle.fc_dynquant_grouped_reference(c.x, c.w, T[wt], c.scale, c.zp, T[zt], c.bias, N=c.N, K=c.K,
+                                             group_size=Gw, act_group=Ga)
+    q, inv, _ = oracle.dynquant_groups(c.x, Ga)
+    ng = c.K // Gw
+    if wt == "u4":
+        codes = oracle.unpack_u4(c.w, c.N * c.K).astype(np.int32)
+    elif wt == "i4":
+        codes = oracle.unpack_i4(c.w, c.N * c.K).astype(np.int32)
+    else:
+        codes = c.w.view(np.int8 if wt == "i8" else np.uint8).astype(np.int32)
+    zp = None
+    if zt == "u4":
+        zp = oracle.unpack_u4(c.zp, c.N * ng).reshape(c.N, ng)
+    elif zt == "u8":
+        zp = c.zp.reshape(c.N, ng)
+    ref = np_fc_grouped(q, inv, Ga, codes.reshape(c.N, c.K), Gw, c.scale.reshape(c.N, ng).astype(np.float32), zp, c.bias)
+    assert oracle.rel_l2(y, ref.astype(np.float32)) < 2e-7
+    assert np.max(np.abs(y - ref)) <= 1e-6 * np.max(np.abs(ref))
+    plain = oracle.fc_reference(c.x, c.w, T[wt], c.scale, c.zp, T[zt], c.bias, N=c.N, K=c.K, group_size=Gw)
+    assert 1e-4 < oracle.rel_l2(y, plain) < 3e-2      # quantisation noise, nothing else
+
+
+def test_fc_dynquant_grouped_reduces_to_the_per_token_oracle(oracle):
+    """One weight group per channel and one activation group per row: the per-token, per-channel function."""
+    c = datagen.make_case(43, 9, 256, 32, "u8", 256, "u8", with_bias=True)
+    a = oracle.fc_dynquant_grouped_reference(c.x, c.w, oracle.U8, c.scale, c.zp, oracle.U8, c.bias, N=c.N, K=c.K,
+                                             group_size=c.K, act_group=c.K)
+    b = oracle.fc_dynquant_reference(c.x, c.w, oracle.U8, c.scale, c.zp.astype(np.float32), c.bias, N=c.N, K=c.K)
+    assert np.allclose(a, b, rtol=2e-6, atol=1e-6)
+
+
+def test_fc_dynquant_grouped_known_answer(oracle):
+    """Hand-computed: K = 4, weight groups of 2, activation groups of 2.  x = [127, -127 | 2, 1] quantises to
+    q = [127, -127 | 127, 64] (2 * 63.5 = 127, 1 * 63.5 = 63.5 -> 64) with inv = [1, 1 / 63.5 in half]."""
+    x = np.array([[127, -127, 2, 1]], np.float16)
+    w = np.array([[3, 1, 2, 5]], np.uint8)
+    scale = np.array([[0.5, 2.0]], np.float16)
+    zp = np.array([[1, 2]], np.uint8)
+    y = oracle.fc_dynquant_grouped_reference(x, w, oracle.U8, scale, zp, oracle.U8, None, N=1, K=4, group_size=2,
+                                             act_group=2)
+    inv1 = float(np.float16(1.0 / float(np.float16(63.5))))
+    want = (127 * 2 - 127 * 0) * 0.5 * 1.0 + (127 * 0 + 64 * 3) * 2.0 * inv1
+    assert abs(float(y[0, 0]) - want) < 1e-4
