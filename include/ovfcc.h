@@ -295,11 +295,6 @@ int ovfcc_moe_routed_device(ovfcc_request* req, const ovfcc_weights* const* gate
                             int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices_dev,
                             int64_t M, int top_k, void* y_dev);
 
-/* Benchmark twin of ovfcc_bench_layers for grouped runs: `iters` eager calls of ovfcc_fc_run_grouped_device on the
- * request's stream, bracketed by HIP events on that stream. */
-int ovfcc_bench_grouped(ovfcc_request* req, const ovfcc_group_item* items, int n_items, int warmup, int iters,
-                        float* elapsed_ms);
-
 /* Wait for everything enqueued on the request (IAsyncInferRequest::wait). */
 int ovfcc_request_sync(ovfcc_request* req);
 
@@ -312,22 +307,20 @@ int ovfcc_request_force_kernel(ovfcc_request* req, int kernel, int split_k);
  * (src/inference/dev_api/openvino/runtime/exec_model_info.hpp:31-73). */
 int ovfcc_last_kernel_info(const ovfcc_request* req, ovfcc_kernel_info* info);
 
-/* Timed back-to-back launches for the benchmark: runs `iters` passes over the `n_layers` nodes
- * in order (layer i reads x_dev, writes y_dev; buffers must fit the largest layer), all on the
- * request's stream, bracketed by HIP events on that stream.  Returns elapsed milliseconds of the
- * whole timed region.  use_graph != 0 captures one pass into a HIP graph and replays it. */
-int ovfcc_bench_layers(ovfcc_request* req, const ovfcc_weights* const* layers, int n_layers, const void* x_dev,
-                       void* y_dev, int64_t M, int warmup, int iters, int use_graph, float* elapsed_ms);
-
 /* ---- device memory helpers (plain pointers; for hosts that do not link HIP themselves) ------ */
 int ovfcc_device_malloc(ovfcc_ctx* ctx, size_t bytes, void** out);
 int ovfcc_device_free(ovfcc_ctx* ctx, void* ptr);
 int ovfcc_memcpy_h2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
 int ovfcc_memcpy_d2h(ovfcc_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
 int ovfcc_memcpy_d2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes);
-/* Plain device-to-device copy kernel of `bytes` (multiple of 16) repeated `iters` times, timed with
- * HIP events: the yardstick the HBM counters and the achieved-bandwidth figures are scaled by. */
-int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, int iters, float* elapsed_ms);
+
+/* The OVFCC_* variables of the process environment (tuning overrides for experiments, and OVFCC_VERBOSE = 1: one
+ * line per launch and per created node on stderr -- kernel, grid, tile, split-K; layout, bytes, repack and upload
+ * time; = 2: every ovfcc_fc_run_device call is also timed with events and waited for, and its time, GB/s and
+ * TFLOP/s are printed; the counterpart of OV_CPU_VERBOSE / the oneDNN verbose mode) are read once, at the first
+ * ovfcc_init.  A process that changes them afterwards calls this to have them read again; launch plans cached
+ * under the old values are dropped. */
+void ovfcc_env_reload(void);
 
 /* ---- host-only pieces (no device needed) ----------------------------------------------------- */
 

@@ -1,0 +1,35 @@
+/*
+ * ovfcc_bench -- timing helpers of the benchmark driver.  Not part of the drop-in boundary: nothing in the
+ * OpenVINO sources corresponds to them and an integration does not bind them.  They live in the library because
+ * the timed region has to be bracketed by HIP events on the very stream the kernels are launched on, which a
+ * host without HIP (the Python benchmark) cannot do itself.
+ */
+#ifndef OVFCC_BENCH_H
+#define OVFCC_BENCH_H
+
+#include "ovfcc.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Timed back-to-back launches: runs `iters` passes over the `n_layers` nodes in order (layer i reads x_dev,
+ * writes y_dev; buffers must fit the largest layer), all on the request's stream, bracketed by HIP events on
+ * that stream.  Returns elapsed milliseconds of the whole timed region.  use_graph != 0 captures one pass into
+ * a HIP graph and replays it. */
+int ovfcc_bench_layers(ovfcc_request* req, const ovfcc_weights* const* layers, int n_layers, const void* x_dev,
+                       void* y_dev, int64_t M, int warmup, int iters, int use_graph, float* elapsed_ms);
+
+/* The same for grouped runs: `iters` eager calls of ovfcc_fc_run_grouped_device on the request's stream,
+ * bracketed by HIP events on that stream. */
+int ovfcc_bench_grouped(ovfcc_request* req, const ovfcc_group_item* items, int n_items, int warmup, int iters,
+                        float* elapsed_ms);
+
+/* Plain device-to-device copy kernel of `bytes` (multiple of 16) repeated `iters` times, timed with HIP
+ * events: the yardstick the HBM counters and the achieved-bandwidth figures are scaled by. */
+int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, int iters, float* elapsed_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OVFCC_BENCH_H */

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -10,6 +11,7 @@
 #include <string>
 #include <vector>
 
+#include "ovfcc_bench.h"
 #include "ovfcc_internal.h"
 
 struct ovfcc_ctx {
@@ -29,6 +31,17 @@ struct ovfcc_weights {
     void* d_scale_cm = nullptr;  // channel-major copies of the group parameters for the matrix-vector kernel
     void* d_zp_cm = nullptr;
     size_t bytes = 0;
+    // Launch plans of recent calls, keyed by what a plan depends on besides the node itself.  Shared by every
+    // request that runs the node, hence the lock; eight entries, replaced in turn.
+    struct PlanEntry {
+        int64_t M = -1;
+        int force_kernel = 0, force_split = 0, n_cus = 0;
+        unsigned env_generation = 0;
+        ovfcc::LaunchPlan plan;
+    };
+    mutable std::mutex plan_mu;
+    mutable PlanEntry plans[8];
+    mutable unsigned plan_next = 0;
 };
 
 struct ovfcc_request {
@@ -253,7 +266,45 @@ void record(ovfcc_request* r, const ovfcc::LaunchPlan& p) {
     i.tile_m = p.tile_m;
     i.tile_n = p.tile_n;
     std::snprintf(i.name, sizeof(i.name), "%s", p.name);
+    if (ovfcc::env_int("OVFCC_VERBOSE", 0) >= 1)
+        std::fprintf(stderr, "ovfcc: launch %s grid=(%u,%u,%u) block=%u tile=%dx%d split_k=%d\n", p.name, p.grid[0],
+                     p.grid[1], p.grid[2], p.block, p.tile_m, p.tile_n, p.split_k);
 }
+
+// OVFCC_VERBOSE >= 2: the call is bracketed by events and waited for, and its time and algorithmic bandwidth
+// (weights, scales, zero-points, activations and results once each) are printed.  Serialises the stream.
+struct VerboseTimer {
+    ovfcc_request* r;
+    const ovfcc_weights* w;
+    int64_t M;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    VerboseTimer(ovfcc_request* req, const ovfcc_weights* wt, int64_t rows) : r(req), w(wt), M(rows) {
+        if (ovfcc::env_int("OVFCC_VERBOSE", 0) < 2 || M == 0)
+            return;
+        if (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess) {
+            (void)hipGetLastError();
+            t0 = t1 = nullptr;
+            return;
+        }
+        (void)hipEventRecord(t0, r->stream);
+    }
+    ~VerboseTimer() {
+        if (!t0 || !t1)
+            return;
+        float ms = 0.f;
+        if (hipEventRecord(t1, r->stream) == hipSuccess && hipEventSynchronize(t1) == hipSuccess &&
+            hipEventElapsedTime(&ms, t0, t1) == hipSuccess && ms > 0.f) {
+            const ovfcc_fc_desc& d = w->desc;
+            const double out_n = (double)((d.flags & OVFCC_GLU_TYPE_MASK) ? d.N / 2 : d.N);
+            const double bytes = (double)w->bytes + (double)M * d.K * 2 + (double)M * out_n * (d.out_type == OVFCC_F32 ? 4 : 2);
+            std::fprintf(stderr, "ovfcc: run M=%lld N=%lld K=%lld %s: %.2f us, %.0f GB/s, %.1f TFLOP/s\n", (long long)M,
+                         (long long)d.N, (long long)d.K, r->last.name, ms * 1e3, bytes / ms / 1e6,
+                         2.0 * M * d.N * d.K / ms / 1e9);
+        }
+        (void)hipEventDestroy(t0);
+        (void)hipEventDestroy(t1);
+    }
+};
 
 int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch);
 
@@ -279,6 +330,30 @@ int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, in
     return OVFCC_OK;
 }
 
+// plan_launch for a call of the node on its own (fill_args's arguments, nothing set by a grouped run), through the
+// node's cache: the plan depends on the node, M, the request's overrides, the chip and the environment overrides.
+int cached_plan(const ovfcc_request* r, const ovfcc_weights* w, const ovfcc::FcDeviceArgs& a, int force,
+                ovfcc::LaunchPlan* p) {
+    const unsigned gen = ovfcc::env_generation();
+    {
+        std::lock_guard<std::mutex> lock(w->plan_mu);
+        for (const auto& e : w->plans)
+            if (e.M == a.M && e.force_kernel == force && e.force_split == r->force_split && e.n_cus == r->ctx->n_cus &&
+                e.env_generation == gen) {
+                *p = e.plan;
+                return OVFCC_OK;
+            }
+    }
+    int rc = ovfcc::plan_launch(a, force, r->force_split, r->ctx->n_cus, p);
+    if (rc)
+        return rc;
+    std::lock_guard<std::mutex> lock(w->plan_mu);
+    auto& e = w->plans[w->plan_next++ % 8];
+    e.M = a.M, e.force_kernel = force, e.force_split = r->force_split, e.n_cus = r->ctx->n_cus, e.env_generation = gen;
+    e.plan = *p;
+    return OVFCC_OK;
+}
+
 // One block of rows.  A tiled node is cut into decode-family launches of at most 48 rows when M is small
 // enough that they beat one sparse prefill grid, or when N is not a multiple of the prefill tile.
 int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch) {
@@ -296,7 +371,7 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
         // (it has no split-K: a grid that leaves half the chip idle stays with the f16 kernels, which have;
         // OVFCC_PREFILL_WIDE = 1 forces the 256-wide kernels onto small shapes, for tests)
         ((w->desc.N / 256) * ((M + 127) / 128) * 2 >= r->ctx->n_cus ||
-         (std::getenv("OVFCC_PREFILL_WIDE") && std::atoi(std::getenv("OVFCC_PREFILL_WIDE")) == 1))) {
+         ovfcc::env_int("OVFCC_PREFILL_WIDE", -1) == 1)) {
         if (static_scratch)
             return fail(OVFCC_EUNSUPPORTED, "a node with int8 activations needs a quantisation buffer of the request");
         const size_t q_bytes = ((size_t)M * w->desc.K + 255) & ~(size_t)255;
@@ -328,7 +403,7 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
         (force == OVFCC_KERNEL_AUTO || force == OVFCC_KERNEL_PREFILL) && M * w->desc.K < ((int64_t)1 << 31) &&
         (M + 127) / 128 <= 65535 &&
         ((w->desc.N / 256) * ((M + 127) / 128) * 2 >= r->ctx->n_cus ||
-         (std::getenv("OVFCC_PREFILL_WIDE") && std::atoi(std::getenv("OVFCC_PREFILL_WIDE")) == 1))) {
+         ovfcc::env_int("OVFCC_PREFILL_WIDE", -1) == 1)) {
         if (static_scratch)
             return fail(OVFCC_EUNSUPPORTED, "a node with int8 activations needs a quantisation buffer of the request");
         const bool grouped = L0.dynquant_grouped;
@@ -386,7 +461,7 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
         return OVFCC_OK;
     }
     ovfcc::LaunchPlan p;
-    int rc = ovfcc::plan_launch(a, force, r->force_split, r->ctx->n_cus, &p);
+    int rc = cached_plan(r, w, a, force, &p);
     if (rc)
         return rc;
     rc = split_buffers(r, p, static_scratch, &a);
@@ -418,8 +493,8 @@ bool plan_routed(ovfcc_request* r, const ovfcc_weights* w0, int64_t R, int n_exp
         r->force_kernel != OVFCC_KERNEL_AUTO || R <= 0)
         return false;
     int cap = R / n_experts > 56 ? ovfcc::kPrefillGroupRows : ovfcc::kPrefillGroupRows / 2;
-    if (const char* e = std::getenv("OVFCC_PREFILL_ROWS"))
-        cap = std::atoi(e) == 64 ? 64 : ovfcc::kPrefillGroupRows;
+    if (const int rows = ovfcc::env_int("OVFCC_PREFILL_ROWS", 0))
+        cap = rows == 64 ? 64 : ovfcc::kPrefillGroupRows;
     const int64_t n = (R + cap - 1) / cap + n_experts;
     if (n * cap * w0->desc.K * 2 >= ((int64_t)1 << 31) || n > 65535)
         return false;
@@ -636,6 +711,10 @@ int ovfcc_device_count(void) {
     return n;
 }
 
+void ovfcc_env_reload(void) {
+    ovfcc::env_reload();
+}
+
 int ovfcc_init(int device, ovfcc_ctx** out) {
     if (!out)
         return fail(OVFCC_EINVAL, "out is null");
@@ -648,6 +727,7 @@ int ovfcc_init(int device, ovfcc_ctx** out) {
     }
     if (device < 0 || device >= n)
         return fail(OVFCC_EINVAL, "device index out of range");
+    (void)ovfcc::env_generation();  // the OVFCC_* overrides are read here, once
     HIP_TRY(hipSetDevice(device));
     hipDeviceProp_t prop;
     HIP_TRY(hipGetDeviceProperties(&prop, device));
@@ -713,10 +793,13 @@ int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* 
     };
 
     const int64_t N = desc->N, K = desc->K, ng = L.groups;
+    const auto t_start = std::chrono::steady_clock::now();
+    auto t_repacked = t_start;
     if (L.tiled) {
         std::vector<uint8_t> wt(L.w_bytes), st(L.scale_bytes), zt(L.zp_bytes);
         ovfcc::repack_weights(*desc, L, w, wt.data());
         ovfcc::repack_params(*desc, L, scales, zp, st.data(), zt.data());
+        t_repacked = std::chrono::steady_clock::now();
         rc = upload(&W->d_w, wt.data(), wt.size());
         if (!rc)
             rc = upload(&W->d_scale, st.data(), st.size());
@@ -750,6 +833,14 @@ int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* 
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;
+    }
+    if (ovfcc::env_int("OVFCC_VERBOSE", 0) >= 1) {
+        using ms = std::chrono::duration<double, std::milli>;
+        const auto t_end = std::chrono::steady_clock::now();
+        std::fprintf(stderr, "ovfcc: weights N=%lld K=%lld group=%lld w_type=%d zp_type=%d%s: %s layout, %zu bytes on the "
+                     "device, repack %.2f ms, upload %.2f ms\n", (long long)N, (long long)K, (long long)desc->group_size,
+                     desc->w_type, desc->zp_type, desc->zp_scalar ? " (scalar)" : "", L.tiled ? "tiled" : "OpenVINO",
+                     W->bytes, ms(t_repacked - t_start).count(), ms(t_end - t_repacked).count());
     }
     *out = W;
     return OVFCC_OK;
@@ -1132,6 +1223,7 @@ int ovfcc_fc_run_device(ovfcc_request* r, const ovfcc_weights* w, const void* x_
     if (M > ((int64_t)1 << 24))
         return fail(OVFCC_EUNSUPPORTED, "M is limited to 2^24");
     HIP_TRY(hipSetDevice(r->ctx->device));
+    VerboseTimer timer(r, w, M);
     return enqueue(r, w, x_dev, y_dev, M);
 }
 
@@ -1191,8 +1283,8 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
             }
         const int64_t tiles128 = padded[0] / ovfcc::kPrefillGroupRows, tiles64 = padded[1] / (ovfcc::kPrefillGroupRows / 2);
         rows_cap = tiles64 * 7 < tiles128 * 10 ? ovfcc::kPrefillGroupRows / 2 : ovfcc::kPrefillGroupRows;
-        if (const char* e = std::getenv("OVFCC_PREFILL_ROWS"))
-            rows_cap = std::atoi(e) == 64 ? 64 : ovfcc::kPrefillGroupRows;
+        if (const int rows = ovfcc::env_int("OVFCC_PREFILL_ROWS", 0))
+            rows_cap = rows == 64 ? 64 : ovfcc::kPrefillGroupRows;
     }
     ovfcc::FcDeviceArgs a;
     std::vector<ovfcc::BatchGroupItem> work;
@@ -1351,7 +1443,7 @@ int ovfcc_gather_matmul_device(ovfcc_request* r, const ovfcc_weights* const* exp
     HIP_TRY(hipSetDevice(r->ctx->device));
     // the routed form wherever it fits: the indices are copied to the device and bucketed there, and the call does
     // not depend on what the host threads were doing; otherwise the rows are bucketed here
-    if (same_zp && !std::getenv("OVFCC_MOE_HOST_ROUTING")) {
+    if (same_zp && ovfcc::env_int("OVFCC_MOE_HOST_ROUTING", 0) == 0) {
         rc = gather_matmul_routed(r, experts, n_experts, a_dev, a_batches, nullptr, indices, M, top_k, y_dev, &ran);
         if (rc || ran)
             return rc;
@@ -1457,7 +1549,7 @@ int ovfcc_moe_device(ovfcc_request* r, const ovfcc_weights* const* gate_up, cons
     const int64_t H = g0->desc.K, I = out_channels(g0);
     const int d_f32 = d0->desc.out_type == OVFCC_F32 ? 1 : 0;
     HIP_TRY(hipSetDevice(r->ctx->device));
-    if (same_zp && !std::getenv("OVFCC_MOE_HOST_ROUTING")) {
+    if (same_zp && ovfcc::env_int("OVFCC_MOE_HOST_ROUTING", 0) == 0) {
         rc = moe_routed(r, gate_up, down, n_experts, x_dev, routing_dev, nullptr, indices, M, top_k, y_dev, &ran);
         if (rc || ran)
             return rc;

@@ -144,6 +144,11 @@ struct LaunchPlan {
 
 // Chooses kernel family and decomposition (force_kernel / force_split 0 = policy).
 int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_cus, LaunchPlan* plan);
+// OVFCC_* overrides of the process environment: cached at the first use, re-read by env_reload only.
+// env_generation changes with every (re)read; plans cached under an older generation are stale.
+int env_int(const char* name, int fallback);
+void env_reload();
+unsigned env_generation();
 // Enqueues on `stream` (a hipStream_t passed as void*); returns a HIP error code (0 = success).
 int launch_fc(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_plain(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);

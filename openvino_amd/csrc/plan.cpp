@@ -4,18 +4,65 @@
 // M <= 48 (the streaming kernel for a few rows, the small-batch kernel above) and the prefill kernel for more
 // (the roofline ridge of int4 g128 sits near M = 83).  The caller cuts 48 < M <= 128 into decode launches:
 // a single 128-row prefill tile per column block leaves most of the chip idle.
+#include <atomic>
 #include <cstdlib>
+#include <cstring>
+#include <mutex>
 
 #include "ovfcc_internal.h"
 
 namespace ovfcc {
 
-// Tuning overrides for experiments: OVFCC_DECODE_WAVES = 4 | 8 | 16 (workgroup size),
-// OVFCC_DECODE_RT = 1 | 2 | 4 (channel tiles per workgroup or wave), OVFCC_DECODE_XLDS = 0 | 1 (activations
-// via LDS), OVFCC_DECODE_BATCH = 0 | 1 (small-batch kernel instead of the streaming kernel).
-static int env_int(const char* name, int fallback) {
-    const char* e = std::getenv(name);
-    return e ? std::atoi(e) : fallback;
+// Overrides from the process environment, read once -- at the first use, which ovfcc_init forces -- and again only
+// by env_reload (tests and experiments that change the environment of a running process).
+//   tuning:  OVFCC_DECODE_WAVES = 4 | 8 | 16 (workgroup size), OVFCC_DECODE_RT = 1 | 2 | 4 (channel tiles per
+//            workgroup or wave), OVFCC_DECODE_XLDS = 0 | 1 (activations via LDS), OVFCC_DECODE_BATCH = 0 | 1
+//            (small-batch kernel instead of the streaming kernel), OVFCC_GEMV = 0 | 1, OVFCC_GEMV_C = 2 | 4 | 8,
+//            OVFCC_PREFILL_{DIRECT, ASYNC, WIDE, BIG, TAIL} = 0 | 1, OVFCC_PREFILL_ROWS = 64 | 128,
+//            OVFCC_MOE_HOST_ROUTING = 1;
+//   logging: OVFCC_VERBOSE = 1 (one line per launch on stderr), 2 (also weights and requests as they come and go).
+namespace {
+struct EnvEntry {
+    const char* name;
+    std::atomic<int> set{0};
+    std::atomic<int> value{0};
+    explicit EnvEntry(const char* n) : name(n) {}
+};
+EnvEntry g_env[] = {EnvEntry("OVFCC_DECODE_WAVES"),   EnvEntry("OVFCC_DECODE_RT"),      EnvEntry("OVFCC_DECODE_XLDS"),
+                    EnvEntry("OVFCC_DECODE_BATCH"),   EnvEntry("OVFCC_GEMV"),           EnvEntry("OVFCC_GEMV_C"),
+                    EnvEntry("OVFCC_PREFILL_DIRECT"), EnvEntry("OVFCC_PREFILL_ASYNC"),  EnvEntry("OVFCC_PREFILL_WIDE"),
+                    EnvEntry("OVFCC_PREFILL_BIG"),    EnvEntry("OVFCC_PREFILL_TAIL"),   EnvEntry("OVFCC_PREFILL_ROWS"),
+                    EnvEntry("OVFCC_MOE_HOST_ROUTING"), EnvEntry("OVFCC_VERBOSE")};
+std::atomic<unsigned> g_env_generation{0};
+std::once_flag g_env_once;
+
+void env_read_all() {
+    for (EnvEntry& e : g_env) {
+        const char* v = std::getenv(e.name);
+        e.value.store(v ? std::atoi(v) : 0, std::memory_order_relaxed);
+        e.set.store(v ? 1 : 0, std::memory_order_release);
+    }
+    g_env_generation.fetch_add(1, std::memory_order_acq_rel);
+}
+}  // namespace
+
+void env_reload() {
+    std::call_once(g_env_once, [] {});  // a later first use must not read again on top of this
+    env_read_all();
+}
+
+unsigned env_generation() {
+    std::call_once(g_env_once, env_read_all);
+    return g_env_generation.load(std::memory_order_acquire);
+}
+
+int env_int(const char* name, int fallback) {
+    std::call_once(g_env_once, env_read_all);
+    for (EnvEntry& e : g_env)
+        if (std::strcmp(e.name, name) == 0)
+            return e.set.load(std::memory_order_acquire) ? e.value.load(std::memory_order_relaxed) : fallback;
+    const char* v = std::getenv(name);  // a name the table does not know
+    return v ? std::atoi(v) : fallback;
 }
 
 // k-blocks per wave of the matrix-vector kernel for this node (0: the kernel does not fit it).  The waves of one

@@ -43,10 +43,16 @@ class Device:
     """One MI355X and its library context (the plugin object's device half)."""
 
     def __init__(self, index: int = 0):
-        self.lib = _lib.load()
+        self._lib = _lib.load()
         h = ctypes.c_void_p()
         check(self.lib.ovfcc_init(index, ctypes.byref(h)))
         self.handle = h
+
+    @property
+    def lib(self):
+        """The loaded library, with environment overrides changed since the last call taken over first."""
+        _lib.sync_env()
+        return self._lib
 
     def close(self):
         if self.handle:

@@ -147,7 +147,24 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     }
 }
 
+// The environment overrides are read once and again only on request.
+static void check_env_cache() {
+    unsetenv("OVFCC_PREFILL_ROWS");
+    ovfcc::env_reload();
+    const unsigned g0 = ovfcc::env_generation();
+    CHECK(ovfcc::env_int("OVFCC_PREFILL_ROWS", 7) == 7, "unset variable gives the fallback");
+    setenv("OVFCC_PREFILL_ROWS", "64", 1);
+    CHECK(ovfcc::env_int("OVFCC_PREFILL_ROWS", 7) == 7, "a change of the environment is not seen before a reload");
+    CHECK(ovfcc::env_generation() == g0, "generation unchanged without a reload");
+    ovfcc::env_reload();
+    CHECK(ovfcc::env_int("OVFCC_PREFILL_ROWS", 7) == 64 && ovfcc::env_generation() != g0, "reload takes the change over");
+    unsetenv("OVFCC_PREFILL_ROWS");
+    ovfcc::env_reload();
+    CHECK(ovfcc::env_int("OVFCC_PREFILL_ROWS", 7) == 7, "and its removal");
+}
+
 int main() {
+    check_env_cache();
     std::mt19937 rng(12345);
     const int64_t Ns[] = {16, 32, 48, 96, 128, 256, 272, 1024, 4096, 14336};
     const int64_t Ks[] = {128, 256, 384, 1024, 4096, 14336};
