@@ -69,6 +69,8 @@ def lib() -> ctypes.CDLL:
             getattr(L, name).restype = None
         L.ovo_fc_reference.argtypes = [ctypes.POINTER(_FcArgs), ctypes.c_void_p]
         L.ovo_fc_reference.restype = ctypes.c_int
+        L.ovo_fc_blocked.argtypes = [ctypes.POINTER(_FcArgs), ctypes.c_void_p]
+        L.ovo_fc_blocked.restype = ctypes.c_int
         L.ovo_num_threads.restype = ctypes.c_int
         L.ovo_set_num_threads.argtypes = [ctypes.c_int]
         _lib = L
@@ -157,8 +159,10 @@ def _as_real(a, name):
 
 
 def fc_reference(x, w, w_type, scale, zp=None, zp_type=NONE, bias=None, *, N, K, group_size,
-                 zp_scalar=False, acc_f64=False, n_index=None) -> np.ndarray:
-    """C oracle.  ``w`` and u4 ``zp`` are the raw packed bytes in OpenVINO order.
+                 zp_scalar=False, acc_f64=False, n_index=None, blocked=False) -> np.ndarray:
+    """C oracle.  ``w`` and u4 ``zp`` are the raw packed bytes in OpenVINO order.  blocked: the blocked,
+    vectorised port of the same formula (oracle_fast.c, the benchmark's CPU baseline) instead of the exact
+    restatement; it agrees with it up to the order of the f32 sum.
 
     x: [M, K] float16/float32; scale: [N, K/G] float16/float32; zp: packed u4 bytes, u8 or
     float32 [N, K/G] (or one element with ``zp_scalar``); bias: [N].  Returns float32 [M, N]
@@ -190,9 +194,10 @@ def fc_reference(x, w, w_type, scale, zp=None, zp_type=NONE, bias=None, *, N, K,
         a.n_index, a.n_count = _ptr(idx), idx.size
         ncols = idx.size
     y = np.empty((M, ncols), dtype=np.float32)
-    rc = lib().ovo_fc_reference(ctypes.byref(a), _ptr(y))
+    fn = lib().ovo_fc_blocked if blocked else lib().ovo_fc_reference
+    rc = fn(ctypes.byref(a), _ptr(y))
     if rc != 0:
-        raise ValueError(f"ovo_fc_reference rejected its arguments (code {rc})")
+        raise ValueError(f"{'ovo_fc_blocked' if blocked else 'ovo_fc_reference'} rejected its arguments (code {rc})")
     return y
 
 
