@@ -28,7 +28,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/ (counters cannot be
 # read from inside this process): FETCH_SIZE x 2.000 (its reading for a copy kernel of known size) + WRITE_SIZE.
-TRAFFIC_DECODE_M1 = {"qo": 8869888, "kv": 2375680, "gate_up": 30526464, "down": 30669824}
+TRAFFIC_DECODE_M1 = {"qo": 8794112, "kv": 2283520, "gate_up": 30461952, "down": 30605312}
 TRAFFIC_PREFILL_M2048 = {"qo": 85494784, "kv": 72139776, "gate_up": 264916992, "down": 255920128}
 
 
@@ -290,7 +290,7 @@ def main() -> int:
     ap.add_argument("--table", action="store_true",
                     help="time and parity-check every benchmark configuration (1-5) and print a markdown table on "
                          "stdout instead of the JSON line")
-    ap.add_argument("--profile", choices=["decode", "prefill", "w8a8"], default=None,
+    ap.add_argument("--profile", choices=["decode", "batch", "prefill", "w8a8", "w4a8"], default=None,
                     help="short run for rocprofv3: one copy-kernel launch of known size (the counter yardstick), "
                          "then a few eager passes of the chosen kernel family; prints no JSON")
     args = ap.parse_args()
@@ -350,10 +350,26 @@ def main() -> int:
                 w.close()
                 dev.free(xq_dev)
                 dev.free(yq_dev)
-        elif args.profile == "decode":
+        elif args.profile == "w4a8":
+            # Llama-3-8B i4 g128 projections at the prefill row count with int8 activations allowed: per token, then
+            # per row and group of 128 inputs (config 3's nodes through the integer kernel)
+            for mode in ("per_token", "per_group"):
+                for shape in ("qo", "gate_up", "down"):
+                    c = datagen.config3(shape, args.prefill_m)
+                    w = fc.CompressedWeights.from_case(dev, c, dynamic_quantization=mode)
+                    xq_dev, yq_dev = dev.malloc(c.x.nbytes), dev.malloc(c.M * c.N * 2)
+                    dev.upload(xq_dev, c.x)
+                    for _ in range(3):
+                        req.infer_device(w, xq_dev, yq_dev, c.M)
+                    req.sync()
+                    w.close()
+                    dev.free(xq_dev)
+                    dev.free(yq_dev)
+        elif args.profile in ("decode", "batch"):
+            rows = 1 if args.profile == "decode" else 32     # small-batch decode: config 2's largest row count
             for _ in range(3):
                 for _, w in layers:
-                    req.infer_device(w, x_dev, y_dev, 1)
+                    req.infer_device(w, x_dev, y_dev, rows)
         else:
             for _ in range(3):
                 for name in datagen.LLAMA3_8B_BLOCK:
@@ -445,7 +461,7 @@ def main() -> int:
             "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
             "traffic": (sum(TRAFFIC_DECODE_M1[name] for name, _ in layers) // launches
                         if set(n for n, _ in layers) <= set(TRAFFIC_DECODE_M1) else None),
-            "traffic_source": "profiles/fcc_decode_w4_llama3_8b_m1.md",
+            "traffic_source": "profiles/fcc_gemv_w4_llama3_8b_m1.md",
             "algorithmic_bytes_per_launch": pass_bytes // launches,
             "avg_launch_us": round(ms_per_step * 1e3 / launches, 3),
         },
