@@ -116,6 +116,39 @@ def results_table(dev, req, args) -> int:
         w.close()
         dev.free(x_dev)
         dev.free(y_dev)
+    # Config 3's nodes at M = 2048 with int8 activations allowed (W4A8): per token, and per row and group of 128
+    # inputs; checked against the oracle of that arithmetic and, for reference, against the f16 oracle.
+    for mode, act_group in (("per_token", None), ("per_group", 128)):
+        for shape in datagen.LLAMA3_8B_SHAPES:
+            c = datagen.config3(shape, 2048)
+            w = fc.CompressedWeights.from_case(dev, c, dynamic_quantization=mode)
+            x_dev, y_dev = dev.malloc(c.x.nbytes), dev.malloc(c.M * c.N * 2)
+            dev.upload(x_dev, c.x)
+            y = req.infer(w, c.x).astype(np.float32)
+            info = req.last_kernel()
+            quantised = info["name"].startswith("fcc_prefill_i8_w4")
+            pick = np.sort(np.random.default_rng(99).choice(c.M, size=8, replace=False))
+            ref_f = oracle.fc_reference(c.x[pick], c.w, type_tag[c.w_type], c.scale, c.zp, type_tag[c.zp_type], None,
+                                        N=c.N, K=c.K, group_size=c.group_size)
+            ref_q = oracle.fc_dynquant_grouped_reference(c.x[pick], c.w, type_tag[c.w_type], c.scale, c.zp,
+                                                         type_tag[c.zp_type], None, N=c.N, K=c.K,
+                                                         group_size=c.group_size, act_group=act_group or c.K) \
+                if quantised else ref_f
+            us = min(req.bench_layers([w], x_dev, y_dev, c.M, 3, 10, use_graph=True) for _ in range(2)) / 10 * 1e3
+            nbytes = algorithmic_bytes(c.K, c.N, c.M, 4, c.group_size, 0.0)
+            gbs, tfs = nbytes / us / 1e3, 2.0 * c.M * c.N * c.K / us / 1e6
+            rows.append(f"| 3 | {shape} {c.K}->{c.N}, int8 activations allowed ({mode.replace('_', ' ')}) | {c.M} | i4 g128 sym"
+                        f"{' x i8 ' + mode.replace('_', ' ') if quantised else ''} | "
+                        f"{'fcc_dynquant_w4 + ' if quantised else ''}{info['name']} | {us:.1f} | "
+                        f"{gbs:.0f} ({100 * gbs / HBM_PEAK_GBS:.1f} %) | {tfs:.1f} ({100 * tfs / 1000 / 2.5:.1f} % of f16 peak) | "
+                        f"{oracle.rel_l2(y[pick], ref_q):.1e} vs its own oracle, {oracle.rel_l2(y[pick], ref_f):.1e} vs f16 | "
+                        f"{oracle.max_abs(y[pick], ref_q):.1e} |")
+            log(rows[-1])
+            w.close()
+            dev.free(x_dev)
+            dev.free(y_dev)
+
+
     routes = datagen.moe_routing()
     t_total, flops_total = 0.0, 0.0
     for e, tokens in enumerate(routes):
@@ -258,6 +291,28 @@ def results_table(dev, req, args) -> int:
     log(rows[-1])
     moe_line = (f"config 5 as one mixture-of-experts call (wall time; SwiGLU fused into gate/up, weighted sum over the "
                 f"two experts of a token included): {best:.1f} us, {tfs:.1f} TFLOP/s")
+    # the same call with the indices already in device memory (where a router's TopK leaves them)
+    i_ptr = dev.malloc(indices.nbytes)
+    dev.upload(i_ptr, np.ascontiguousarray(indices, dtype=np.int32))
+    req.moe_routed_device(wg, wd, x_ptr, r_ptr, i_ptr, tokens, 2, y_ptr)
+    req.sync()
+    yd = dev.download(y_ptr, (tokens, 4096), np.float16).astype(np.float32)
+    rl2d, mabd = oracle.rel_l2(yd[pick], ref), oracle.max_abs(yd[pick], ref)
+    bestd = 1e30
+    for _ in range(6):
+        t0 = time.perf_counter()
+        for _ in range(20):
+            req.moe_routed_device(wg, wd, x_ptr, r_ptr, i_ptr, tokens, 2, y_ptr)
+        req.sync()
+        bestd = min(bestd, (time.perf_counter() - t0) / 20 * 1e6)
+    gbsd, tfsd = nbytes / bestd / 1e3, flops_total / bestd / 1e6
+    rows.append(f"| 5 | mixture-of-experts block, indices in device memory (routing kernel, no wait on the stream) | {tokens} tokens | "
+                f"u4 g128 asym | 2 x fcc_moe_route + rows gather + 2 x fcc_prefill_async_grouped_w4 + weighted sum | {bestd:.1f} | "
+                f"{gbsd:.0f} ({100 * gbsd / HBM_PEAK_GBS:.1f} %) | {tfsd:.1f} ({100 * tfsd / 1000 / 2.5:.1f} %) | "
+                f"{rl2d:.1e} | {mabd:.1e} |")
+    log(rows[-1])
+    dev.free(i_ptr)
+    moe_line += f"; with the indices in device memory: {bestd:.1f} us"
     for w in wg + wd:
         w.close()
     for ptr in (x_ptr, r_ptr, y_ptr):
@@ -271,6 +326,56 @@ def results_table(dev, req, args) -> int:
     print(grouped_line)
     print(op_line)
     print(moe_line)
+    req.close()
+    dev.close()
+    return 0
+
+
+def floors_table(dev, req, args) -> int:
+    """Per Llama-3-8B shape at M = 1: the time of an empty graph node, of the best loads-only streaming kernel over the
+    node's weight bytes (a sweep of workgroup shapes), and of the node itself -- all as nodes of replayed graphs over
+    rotating buffers larger than the caches."""
+    from openvino_amd import datagen, fc
+
+    arena_bytes = 768 << 20
+    arena = dev.malloc(arena_bytes)
+    dev.copy_bandwidth(256 << 20, 1)
+    empty = min(dev.floor_us(arena, arena_bytes, 0) for _ in range(3))
+    x_dev, y_dev = dev.malloc(14336 * 2 * 4), dev.malloc(2 * 14336 * 2 * 4)
+    print("| node | weight bytes | empty graph node us | loads-only streaming kernel us (GB/s) | fcc_gemv_w4 us (GB/s) | "
+          "kernel / streaming |")
+    print("|---|---|---|---|---|---|")
+    total_probe = total_kernel = 0.0
+    for name, (K, N) in datagen.LLAMA3_8B_SHAPES.items():
+        wbytes = N * K // 2
+        best = 1e30
+        for waves in (4, 8, 16):
+            for kpw in (8, 16, 32):
+                if (wbytes >> 10) % (waves * kpw) or (wbytes >> 10) // (waves * kpw) < 64:
+                    continue
+                best = min(best, min(dev.floor_us(arena, arena_bytes, wbytes, 96, waves, kpw) for _ in range(2)))
+        c = datagen.weights_only(2001, K, N, "i4", 128, "none")
+        w = fc.CompressedWeights.from_case(dev, c)
+        copies = [w]
+        while sum(h.device_bytes for h in copies) < (600 << 20) and len(copies) < 48:
+            copies.append(w.clone())
+        t = min(req.bench_layers(copies, x_dev, y_dev, 1, 3, 20, use_graph=True) for _ in range(3)) / 20 / len(copies) * 1e3
+        nbytes = algorithmic_bytes(K, N, 1)
+        per_block = 2 if name in ("qo", "kv", "gate_up") else 1
+        total_probe += per_block * best
+        total_kernel += per_block * t
+        print(f"| {name} {K}->{N} | {wbytes} | {empty:.2f} | {best:.2f} ({wbytes / best / 1e3:.0f}) | {t:.2f} "
+              f"({nbytes / t / 1e3:.0f}) | {t / best:.2f} |")
+        log(f"{name}: empty {empty:.2f} probe {best:.2f} kernel {t:.2f}")
+        for h in copies:
+            h.close()
+    block_bytes = sum(algorithmic_bytes(*datagen.LLAMA3_8B_SHAPES[n], 1) for n in datagen.LLAMA3_8B_BLOCK)
+    print(f"\none block (q, k, v, o, gate, up, down): streaming kernels {total_probe:.1f} us = "
+          f"{block_bytes / total_probe / 1e3:.0f} GB/s ({100 * block_bytes / total_probe / 1e3 / HBM_PEAK_GBS:.1f} % of 8 TB/s); "
+          f"fcc_gemv_w4 {total_kernel:.1f} us = {block_bytes / total_kernel / 1e3:.0f} GB/s "
+          f"({100 * block_bytes / total_kernel / 1e3 / HBM_PEAK_GBS:.1f} %)")
+    for ptr in (arena, x_dev, y_dev):
+        dev.free(ptr)
     req.close()
     dev.close()
     return 0
@@ -290,6 +395,9 @@ def main() -> int:
     ap.add_argument("--table", action="store_true",
                     help="time and parity-check every benchmark configuration (1-5) and print a markdown table on "
                          "stdout instead of the JSON line")
+    ap.add_argument("--floors", action="store_true",
+                    help="measure what bounds a decode node from below -- an empty graph node, a loads-only streaming "
+                         "kernel over the node's weight bytes -- beside the node's own time, and print a markdown table")
     ap.add_argument("--profile", choices=["decode", "batch", "prefill", "w8a8", "w4a8"], default=None,
                     help="short run for rocprofv3: one copy-kernel launch of known size (the counter yardstick), "
                          "then a few eager passes of the chosen kernel family; prints no JSON")
@@ -308,6 +416,8 @@ def main() -> int:
     req = fc.InferRequest(dev)
     if args.table:
         return results_table(dev, req, args)
+    if args.floors:
+        return floors_table(dev, req, args)
 
     # ---- weights: one host tensor set per shape, one device copy per use ----
     t0 = time.perf_counter()

@@ -29,6 +29,15 @@ int ovfcc_bench_grouped(ovfcc_request* req, const ovfcc_group_item* items, int n
  * events: the yardstick the HBM counters and the achieved-bandwidth figures are scaled by. */
 int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, int iters, float* elapsed_ms);
 
+/* Launch floors under graph replay: a graph of n_nodes launches of a probe kernel is replayed `iters` times and
+ * timed with events.  node_bytes = 0: empty kernels (what a graph node costs with nothing in it).  Otherwise a
+ * loads-only streaming kernel over node_bytes (a multiple of waves * kib_per_wave KiB; workgroups of `waves` waves,
+ * kib_per_wave >= 8 KiB per wave, eight 1 KiB loads in flight per wave), node i reading slice i mod
+ * (arena_bytes / node_bytes) of arena_dev so that the caches do not serve it: how fast a kernel that only reads can
+ * move that many bytes. */
+int ovfcc_bench_floor(ovfcc_ctx* ctx, const void* arena_dev, size_t arena_bytes, size_t node_bytes, int n_nodes, int waves,
+                      int kib_per_wave, int iters, float* elapsed_ms);
+
 #ifdef __cplusplus
 }
 #endif

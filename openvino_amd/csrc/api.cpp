@@ -1809,4 +1809,52 @@ int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t 
     return OVFCC_OK;
 }
 
+// One graph of n_nodes probe launches, replayed `iters` times after three warm-up replays.
+int ovfcc_bench_floor(ovfcc_ctx* ctx, const void* arena_dev, size_t arena_bytes, size_t node_bytes, int n_nodes, int waves,
+                      int kib_per_wave, int iters, float* elapsed_ms) {
+    if (!ctx || !elapsed_ms || n_nodes <= 0 || iters <= 0 || (node_bytes && (!arena_dev || arena_bytes < node_bytes)))
+        return fail(OVFCC_EINVAL, "bad floor benchmark arguments");
+    HIP_TRY(hipSetDevice(ctx->device));
+    hipStream_t s = nullptr;
+    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    unsigned* out = nullptr;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&out), 256));
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int e = 0;
+    HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    const size_t slices = node_bytes ? arena_bytes / node_bytes : 1;
+    for (int i = 0; i < n_nodes && !e; ++i)
+        e = node_bytes ? ovfcc::launch_stream_probe(static_cast<const char*>(arena_dev) + (size_t)(i % slices) * node_bytes,
+                                                    node_bytes, waves, kib_per_wave, out, s)
+                       : ovfcc::launch_empty(out, s);
+    hipError_t ce = hipStreamEndCapture(s, &graph);
+    if (e || ce != hipSuccess) {
+        if (graph) (void)hipGraphDestroy(graph);
+        (void)hipFree(out);
+        (void)hipStreamDestroy(s);
+        return e ? hip_fail((hipError_t)e, "probe launch") : hip_fail(ce, "graph capture");
+    }
+    HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    hipEvent_t t0, t1;
+    HIP_TRY(hipEventCreate(&t0));
+    HIP_TRY(hipEventCreate(&t1));
+    for (int i = 0; i < 3; ++i)
+        HIP_TRY(hipGraphLaunch(exec, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    HIP_TRY(hipEventRecord(t0, s));
+    for (int i = 0; i < iters; ++i)
+        HIP_TRY(hipGraphLaunch(exec, s));
+    HIP_TRY(hipEventRecord(t1, s));
+    HIP_TRY(hipEventSynchronize(t1));
+    HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    (void)hipGraphExecDestroy(exec);
+    (void)hipGraphDestroy(graph);
+    (void)hipFree(out);
+    (void)hipStreamDestroy(s);
+    return OVFCC_OK;
+}
+
 }  // extern "C"

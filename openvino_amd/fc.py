@@ -81,6 +81,15 @@ class Device:
         """Device-to-device copy (blocking)."""
         check(self.lib.ovfcc_memcpy_d2d(self.handle, ctypes.c_void_p(dst_ptr), ctypes.c_void_p(src_ptr), nbytes))
 
+    def floor_us(self, arena_ptr: int, arena_bytes: int, node_bytes: int, n_nodes: int = 96, waves: int = 8,
+                 kib_per_wave: int = 8, iters: int = 20) -> float:
+        """Microseconds per node of a replayed graph of probe launches: empty kernels (node_bytes = 0) or loads-only
+        streaming kernels over node_bytes each (ovfcc_bench_floor)."""
+        ms = ctypes.c_float()
+        check(self.lib.ovfcc_bench_floor(self.handle, ctypes.c_void_p(arena_ptr), arena_bytes, node_bytes, n_nodes, waves,
+                                         kib_per_wave, iters, ctypes.byref(ms)))
+        return ms.value * 1e3 / iters / n_nodes
+
     def copy_bandwidth(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
         """GB/s (read + write) of the plain copy kernel."""
         src, dst = self.malloc(nbytes), self.malloc(nbytes)
