@@ -48,12 +48,18 @@ enum ovfcc_op {
     OVFCC_OP_ADD = 10,
     OVFCC_OP_SWISH = 11,          /* v4::Swish with beta = 1 (one input) */
     OVFCC_OP_GELU = 12,           /* v7::Gelu; attr = 0 erf, 1 tanh */
-    OVFCC_OP_RESULT = 13
+    OVFCC_OP_RESULT = 13,
+    OVFCC_OP_GATHER_MATMUL = 14,            /* internal::GatherMatmul: inputs (A, B, indices, bias) */
+    OVFCC_OP_GATHER_MATMUL_COMPRESSED = 15, /* internal::GatherMatmulCompressed: (A, B, indices, bias, scale, zp) */
+    OVFCC_OP_UNSQUEEZE = 16,
+    OVFCC_OP_SLICE = 17,
+    OVFCC_OP_REDUCE_SUM = 18                /* v1::ReduceSum; attr = keep_dims */
 };
 
 /* element types beyond enum ovfcc_type that a graph may carry (bf16, i32 shape constants, ...) */
 #define OVFCC_TYPE_OTHER 7
 #define OVFCC_MAX_RANK 6
+#define OVFCC_MAX_INPUTS 6
 
 /* One node, described by its first output. */
 typedef struct ovfcc_gnode {
@@ -62,9 +68,9 @@ typedef struct ovfcc_gnode {
     int32_t rank;                  /* rank of the output shape, -1 when dynamic */
     int64_t dims[OVFCC_MAX_RANK];  /* -1 = dynamic dimension */
     int32_t n_inputs;
-    int32_t inputs[4];             /* indices into the node array; -1 = absent (FullyConnected without bias) */
+    int32_t inputs[OVFCC_MAX_INPUTS]; /* indices into the node array; -1 = absent (FullyConnected without bias) */
     int32_t transpose_a, transpose_b; /* MatMul */
-    int32_t attr;                  /* Gelu: 1 = tanh approximation */
+    int32_t attr;                  /* Gelu: 1 = tanh approximation; ReduceSum: keep_dims */
     int32_t consumers;             /* how many node inputs read this output */
     int32_t n_ints;                /* integer Constant of at most OVFCC_MAX_RANK elements: its values (a Transpose */
     int64_t ints[OVFCC_MAX_RANK];  /* order, a Reshape pattern); n_ints = -1 when not supplied */
@@ -110,6 +116,61 @@ typedef struct ovfcc_fused {
  * group.  OVFCC_EINVAL when an output array is too small. */
 int ovfcc_fold_model(const ovfcc_gnode* nodes, int n_nodes, ovfcc_fold* folds, int max_folds, int* n_folds,
                      ovfcc_fused* fused, int max_fused, int* n_fused);
+
+/* ---- mixture-of-experts layers ---------------------------------------------------------------------------- */
+
+/* A matched GatherMatmulCompressed node: the expert matrices of a mixture-of-experts layer applied to routed rows
+ * (src/common/transformations/include/ov_ops/gather_matmul.hpp:17-41, gather_matmul_compressed.hpp:17-33; shapes
+ * src/common/transformations/src/ov_ops/gather_matmul.cpp:38-130).  Either an internal::GatherMatmul whose B input is
+ * the weight-decompression subgraph over a batched Constant -- [E, N, K], or grouped [E, N, K/G, G] behind a Reshape to
+ * three dimensions -- the role of ConvertGatherMatmulToGatherMatmulCompressed
+ * (src/common/transformations/src/transformations/op_conversions/convert_gather_matmul_to_compressed.cpp:27-92), or an
+ * internal::GatherMatmulCompressed as that pass leaves it.  desc describes ONE expert: expert e's node is created
+ * with ovfcc_weights_create from slice e of every constant (the views are [E, N, K] and [E, N, K/G]: slice e
+ * starts at element e N K, resp. e N K/G, of the flattened constant -- for 4-bit types with an odd element count per
+ * expert that is in the middle of a byte and the host re-packs the slice), and the E nodes go to
+ * ovfcc_gather_matmul_device / ovfcc_gather_matmul_routed_device. */
+typedef struct ovfcc_gather_fold {
+    ovfcc_fc_desc desc;
+    int32_t n_experts;
+    int32_t root;         /* the GatherMatmul / GatherMatmulCompressed node */
+    int32_t activations;  /* A [1 or top_k, M, K] */
+    int32_t indices;      /* [M, top_k] */
+    int32_t top_k;        /* -1 when dynamic */
+    int32_t weights, scales, zero_points, bias; /* Constant nodes; -1 = absent */
+    int32_t scale_broadcast;  /* one scale value for the whole layer */
+    int32_t zp_from_real;     /* as in ovfcc_fold */
+    int32_t bias_per_expert;  /* the bias Constant holds E x N values (else N, shared by the experts) */
+    int32_t activations_f32;
+    int64_t w_view[3], scale_view[3], zp_view[3];
+    int32_t n_chain;
+    int32_t chain[16];
+} ovfcc_gather_fold;
+
+int ovfcc_fold_gather_matmul(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_gather_fold* out);
+
+/* A matched expert block: three GatherMatmul[Compressed] nodes, the gate activation, the Multiply by the routing
+ * weights and the ReduceSum over the selected experts -- what Convert3GatherMatmulMoeBlockToMoeOp
+ * (src/common/transformations/src/transformations/common_optimizations/moe_op_fusion.cpp:55-232) folds into
+ * MOE / MOECompressed with Expert_type::GEMM3_SWIGLU (src/common/transformations/include/ov_ops/moe_compressed.hpp:15-75):
+ *     Reshape( ReduceSum( down(act(gate(u)) * up(u)) * Unsqueeze(Transpose([Slice](routing))) ) ),
+ *     u = Unsqueeze([Reshape](hidden_states)), all three over the same indices.
+ * gate[e] and up[e] become one node with a gated linear unit (ovfcc_weights_glu, glu_type), down[e] another, and the
+ * block is one ovfcc_moe_device / ovfcc_moe_routed_device call with x = hidden_states as [M, H], routing = the
+ * tensor that enters the Transpose ([M, top_k]) and the indices. */
+typedef struct ovfcc_moe_fold {
+    ovfcc_gather_fold gate, up, down;
+    int32_t glu_type;       /* OVFCC_GLU_SWISH | OVFCC_GLU_GELU | OVFCC_GLU_GELU_TANH */
+    int32_t root;           /* the closing Reshape: the node whose output the block produces */
+    int32_t hidden_states;
+    int32_t routing;        /* producer of the [M, top_k] routing weights (the Slice, where there is one) */
+    int32_t indices;
+    int32_t n_chain;        /* nodes between the inputs and the root that the block absorbs, the three folds' own aside */
+    int32_t chain[16];
+} ovfcc_moe_fold;
+
+/* root: the closing Reshape (or the ReduceSum under it). */
+int ovfcc_fold_moe(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_moe_fold* out);
 
 #ifdef __cplusplus
 }

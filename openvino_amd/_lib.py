@@ -25,7 +25,7 @@ SYMBOLS = [
     "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
     "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_memcpy_d2d", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_desc_validate", "ovfcc_env_reload", "ovfcc_tiled_sizes",
     "ovfcc_repack_host", "ovfcc_unrepack_host", "ovfcc_unpack_u4", "ovfcc_unpack_i4", "ovfcc_last_error",
-    "ovfcc_version", "ovfcc_fold_match", "ovfcc_fold_model",
+    "ovfcc_version", "ovfcc_fold_match", "ovfcc_fold_model", "ovfcc_fold_gather_matmul", "ovfcc_fold_moe",
 ]
 
 
@@ -47,14 +47,16 @@ class FcDesc(ctypes.Structure):
 MAX_RANK = 6
 TYPE_OTHER = 7
 OP = {"other": 0, "parameter": 1, "constant": 2, "convert": 3, "subtract": 4, "multiply": 5, "reshape": 6,
-      "transpose": 7, "matmul": 8, "fully_connected": 9, "add": 10, "swish": 11, "gelu": 12, "result": 13}
+      "transpose": 7, "matmul": 8, "fully_connected": 9, "add": 10, "swish": 11, "gelu": 12, "result": 13,
+      "gather_matmul": 14, "gather_matmul_compressed": 15, "unsqueeze": 16, "slice": 17, "reduce_sum": 18}
+MAX_INPUTS = 6
 FUSED_SINGLE, FUSED_CONCAT, FUSED_GLU = 0, 1, 2
 
 
 class GNode(ctypes.Structure):
     """struct ovfcc_gnode (include/ovfcc_graph.h)"""
     _fields_ = [("op", ctypes.c_int32), ("type", ctypes.c_int32), ("rank", ctypes.c_int32),
-                ("dims", ctypes.c_int64 * MAX_RANK), ("n_inputs", ctypes.c_int32), ("inputs", ctypes.c_int32 * 4),
+                ("dims", ctypes.c_int64 * MAX_RANK), ("n_inputs", ctypes.c_int32), ("inputs", ctypes.c_int32 * MAX_INPUTS),
                 ("transpose_a", ctypes.c_int32), ("transpose_b", ctypes.c_int32), ("attr", ctypes.c_int32),
                 ("consumers", ctypes.c_int32), ("n_ints", ctypes.c_int32), ("ints", ctypes.c_int64 * MAX_RANK)]
 
@@ -66,6 +68,24 @@ class Fold(ctypes.Structure):
                 ("bias", ctypes.c_int32), ("scale_broadcast", ctypes.c_int32), ("zp_from_real", ctypes.c_int32),
                 ("activations_f32", ctypes.c_int32), ("w_view", ctypes.c_int64 * 2), ("scale_view", ctypes.c_int64 * 2),
                 ("zp_view", ctypes.c_int64 * 2), ("n_chain", ctypes.c_int32), ("chain", ctypes.c_int32 * 16)]
+
+
+class GatherFold(ctypes.Structure):
+    """struct ovfcc_gather_fold"""
+    _fields_ = [("desc", FcDesc), ("n_experts", ctypes.c_int32), ("root", ctypes.c_int32),
+                ("activations", ctypes.c_int32), ("indices", ctypes.c_int32), ("top_k", ctypes.c_int32),
+                ("weights", ctypes.c_int32), ("scales", ctypes.c_int32), ("zero_points", ctypes.c_int32),
+                ("bias", ctypes.c_int32), ("scale_broadcast", ctypes.c_int32), ("zp_from_real", ctypes.c_int32),
+                ("bias_per_expert", ctypes.c_int32), ("activations_f32", ctypes.c_int32),
+                ("w_view", ctypes.c_int64 * 3), ("scale_view", ctypes.c_int64 * 3), ("zp_view", ctypes.c_int64 * 3),
+                ("n_chain", ctypes.c_int32), ("chain", ctypes.c_int32 * 16)]
+
+
+class MoeFold(ctypes.Structure):
+    """struct ovfcc_moe_fold"""
+    _fields_ = [("gate", GatherFold), ("up", GatherFold), ("down", GatherFold), ("glu_type", ctypes.c_int32),
+                ("root", ctypes.c_int32), ("hidden_states", ctypes.c_int32), ("routing", ctypes.c_int32),
+                ("indices", ctypes.c_int32), ("n_chain", ctypes.c_int32), ("chain", ctypes.c_int32 * 16)]
 
 
 class Fused(ctypes.Structure):
@@ -150,6 +170,8 @@ def load() -> ctypes.CDLL:
         "ovfcc_fold_match": (ci, [ctypes.POINTER(GNode), ci, ci, ctypes.POINTER(Fold)]),
         "ovfcc_fold_model": (ci, [ctypes.POINTER(GNode), ci, ctypes.POINTER(Fold), ci, ctypes.POINTER(ci),
                                   ctypes.POINTER(Fused), ci, ctypes.POINTER(ci)]),
+        "ovfcc_fold_gather_matmul": (ci, [ctypes.POINTER(GNode), ci, ci, ctypes.POINTER(GatherFold)]),
+        "ovfcc_fold_moe": (ci, [ctypes.POINTER(GNode), ci, ci, ctypes.POINTER(MoeFold)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)

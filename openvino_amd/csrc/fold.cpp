@@ -24,7 +24,7 @@ struct Graph {
     }
     int input(int node, int k) const {
         const ovfcc_gnode& n = nodes[node];
-        return k < n.n_inputs && k < 4 && has(n.inputs[k]) ? n.inputs[k] : -1;
+        return k < n.n_inputs && k < OVFCC_MAX_INPUTS && has(n.inputs[k]) ? n.inputs[k] : -1;
     }
 };
 
@@ -354,6 +354,352 @@ bool same_format(const ovfcc_fc_desc& a, const ovfcc_fc_desc& b) {
            a.zp_scalar == b.zp_scalar && a.bias_type == b.bias_type && a.out_type == b.out_type && a.flags == b.flags;
 }
 
+
+// ---- mixture-of-experts layers --------------------------------------------------------------------------------
+
+struct GatherChain {
+    ovfcc_gather_fold* f;
+    void add(int node) {
+        if (node < 0)
+            return;
+        for (int i = 0; i < f->n_chain; ++i)
+            if (f->chain[i] == node)
+                return;
+        if (f->n_chain < 16)
+            f->chain[f->n_chain++] = node;
+    }
+};
+
+// a Constant, directly or behind one Convert
+int expert_constant(const Graph& g, int node, GatherChain& chain) {
+    if (!g.has(node))
+        return -1;
+    int c = node;
+    if (g.at(c).op == OVFCC_OP_CONVERT) {
+        c = g.input(c, 0);
+        if (c < 0)
+            return -1;
+        chain.add(node);
+    }
+    if (g.at(c).op != OVFCC_OP_CONSTANT)
+        return -1;
+    chain.add(c);
+    return c;
+}
+
+// scale / zero-point of batched weights: one value per (expert, channel, group) in the weights' own axis order
+// ([E, N, 1], or [E, N, K/G, 1] for grouped weights, leading ones allowed to be missing), or one value in all
+bool per_expert_group(const ovfcc_gnode& c, int64_t E, int64_t N, int64_t ng, bool grouped) {
+    const int64_t want3[3] = {E, N, 1}, want4[4] = {E, N, ng, 1};
+    return grouped ? broadcasts_per_group(c, want4, 4) : (broadcasts_per_group(c, want3, 3) && ng == 1);
+}
+
+int gather_impl(const Graph& g, int root, ovfcc_gather_fold* out) {
+    ovfcc_gather_fold f;
+    std::memset(&f, 0, sizeof(f));
+    f.root = root;
+    f.activations = f.indices = f.weights = f.scales = f.zero_points = f.bias = -1;
+    f.top_k = -1;
+    GatherChain chain{&f};
+    if (!g.has(root))
+        return fail(OVFCC_EINVAL, "root is not a node of the graph");
+    const ovfcc_gnode& m = g.at(root);
+    const bool compressed = m.op == OVFCC_OP_GATHER_MATMUL_COMPRESSED;
+    if (m.op != OVFCC_OP_GATHER_MATMUL && !compressed)
+        return fail(OVFCC_EUNSUPPORTED, "root is neither a GatherMatmul nor a GatherMatmulCompressed");
+    if (m.n_inputs < (compressed ? 6 : 3))
+        return fail(OVFCC_EINVAL, "GatherMatmul with too few inputs");
+    f.activations = g.input(root, 0);
+    f.indices = g.input(root, 2);
+    if (f.activations < 0 || f.indices < 0)
+        return fail(OVFCC_EINVAL, "GatherMatmul without activations or indices");
+
+    int wc = -1, scale = -1, zp = -1, reshape = -1;
+    if (compressed) {
+        // the node as ConvertGatherMatmulToGatherMatmulCompressed leaves it: B, scale and zero-point are Constants
+        // of three dimensions (a zero-point of no elements stands for "none")
+        wc = g.input(root, 1), scale = g.input(root, 4), zp = g.input(root, 5);
+        if (wc < 0 || g.at(wc).op != OVFCC_OP_CONSTANT || scale < 0 || g.at(scale).op != OVFCC_OP_CONSTANT)
+            return fail(OVFCC_EUNSUPPORTED, "GatherMatmulCompressed needs Constant weights and scales");
+        if (zp >= 0 && (g.at(zp).op != OVFCC_OP_CONSTANT || element_count(g.at(zp)) == 0))
+            zp = -1;
+        chain.add(wc), chain.add(scale), chain.add(zp);
+    } else {
+        // B = [Convert] <- [Reshape] <- Multiply(Subtract(Convert(W), zp) | Convert(W), scale)
+        int w = g.input(root, 1);
+        if (w >= 0 && g.at(w).op == OVFCC_OP_CONVERT) {
+            chain.add(w);
+            w = g.input(w, 0);
+        }
+        if (w >= 0 && g.at(w).op == OVFCC_OP_TRANSPOSE)
+            return fail(OVFCC_EUNSUPPORTED, "expert weights behind a Transpose ([E, K, N]) are not supported");
+        if (w >= 0 && g.at(w).op == OVFCC_OP_RESHAPE) {
+            reshape = w;
+            chain.add(w);
+            chain.add(g.input(w, 1));
+            w = g.input(w, 0);
+        }
+        if (w < 0 || g.at(w).op != OVFCC_OP_MULTIPLY)
+            return fail(OVFCC_EUNSUPPORTED, "no Multiply(scale) on the weight path");
+        chain.add(w);
+        int body = -1;
+        for (int side = 0; side < 2 && scale < 0; ++side) {
+            ovfcc_gather_fold probe = f;
+            GatherChain pc{&probe};
+            const int c = expert_constant(g, g.input(w, side), pc);
+            if (c >= 0 && is_real(g.at(c).type)) {
+                scale = c;
+                body = g.input(w, 1 - side);
+                f = probe;
+            }
+        }
+        if (scale < 0)
+            return fail(OVFCC_EUNSUPPORTED, "scale is not an f16 / f32 Constant");
+        if (body >= 0 && g.at(body).op == OVFCC_OP_SUBTRACT) {
+            chain.add(body);
+            zp = expert_constant(g, g.input(body, 1), chain);
+            if (zp < 0)
+                return fail(OVFCC_EUNSUPPORTED, "zero-point is not a Constant");
+            body = g.input(body, 0);
+        }
+        if (body < 0 || g.at(body).op != OVFCC_OP_CONVERT)
+            return fail(OVFCC_EUNSUPPORTED, "weights do not enter through a Convert");
+        chain.add(body);
+        wc = g.input(body, 0);
+        if (wc < 0 || g.at(wc).op != OVFCC_OP_CONSTANT)
+            return fail(OVFCC_EUNSUPPORTED, "weights are not a Constant");
+        chain.add(wc);
+    }
+    const ovfcc_gnode& W = g.at(wc);
+    if (!is_weight_type(W.type))
+        return fail(OVFCC_EUNSUPPORTED, "weights are not a u4 / i4 / u8 / i8 Constant");
+    if (element_count(W) <= 0)
+        return fail(OVFCC_EUNSUPPORTED, "weights need a static, non-empty shape");
+    int64_t E, N, K, G;
+    bool grouped = false;
+    if (W.rank == 3) {
+        if (reshape >= 0)
+            return fail(OVFCC_EUNSUPPORTED, "a Reshape on the weight path must merge [E, N, K/G, G] into [E, N, K]");
+        E = W.dims[0], N = W.dims[1], K = W.dims[2], G = K;
+        // GatherMatmulCompressed carries grouped scales as [E, N, K/G] beside [E, N, K] weights
+        if (compressed && g.at(scale).rank == 3 && g.at(scale).dims[2] > 1) {
+            if (K % g.at(scale).dims[2])
+                return fail(OVFCC_EUNSUPPORTED, "the scales' group count does not divide K");
+            G = K / g.at(scale).dims[2];
+            grouped = true;
+        }
+    } else if (W.rank == 4) {
+        E = W.dims[0], N = W.dims[1], K = W.dims[2] * W.dims[3], G = W.dims[3];
+        grouped = true;
+        if (!compressed) {
+            if (reshape < 0 || g.at(reshape).rank != 3 || g.at(reshape).dims[0] != E || g.at(reshape).dims[1] != N ||
+                g.at(reshape).dims[2] != K)
+                return fail(OVFCC_EUNSUPPORTED, "grouped expert weights [E, N, K/G, G] need a Reshape to [E, N, K]");
+        }
+    } else {
+        return fail(OVFCC_EUNSUPPORTED, "expert weights must be [E, N, K] or [E, N, K/G, G]");
+    }
+    const int64_t ng = K / G;
+    auto shaped_ok = [&](const ovfcc_gnode& c) {
+        if (compressed && W.rank == 3) {  // [E, N, K/G]
+            const int64_t want[3] = {E, N, ng};
+            return broadcasts_per_group(c, want, 3);
+        }
+        return per_expert_group(c, E, N, ng, grouped);
+    };
+    const int64_t sc = element_count(g.at(scale));
+    if (sc == 1 && E * N * ng != 1)
+        f.scale_broadcast = 1;
+    else if (!shaped_ok(g.at(scale)))
+        return fail(OVFCC_EUNSUPPORTED, "scale must hold one value, or one per (expert, output channel, group)");
+    f.desc.zp_type = OVFCC_NONE;
+    if (zp >= 0) {
+        const int64_t zc = element_count(g.at(zp));
+        if (zc == 1 && E * N * ng != 1)
+            f.desc.zp_scalar = 1;
+        else if (!shaped_ok(g.at(zp)))
+            return fail(OVFCC_EUNSUPPORTED, "zero-point must be scalar or hold one value per (expert, output channel, group)");
+        const int zt = g.at(zp).type;
+        if (zt == OVFCC_U4 || zt == OVFCC_U8) {
+            f.desc.zp_type = zt;
+        } else if (is_real(zt)) {
+            f.desc.zp_type = OVFCC_U8;
+            f.zp_from_real = 1;
+        } else {
+            return fail(OVFCC_EUNSUPPORTED, "zero-point must be u4, u8 or a real type holding integers");
+        }
+    }
+
+    // ---- activations [1 or top_k, M, K], indices [M, top_k] ----
+    const ovfcc_gnode& A = g.at(f.activations);
+    if (A.type == OVFCC_F32)
+        f.activations_f32 = 1;
+    else if (A.type != OVFCC_F16)
+        return fail(OVFCC_EUNSUPPORTED, "activations must be f16 (or f32, converted by the host)");
+    if (A.rank != 3 || A.dims[2] != K)
+        return fail(OVFCC_EUNSUPPORTED, "activations must be [1 or top_k, M, K]");
+    const ovfcc_gnode& I = g.at(f.indices);
+    if (I.rank != 2)
+        return fail(OVFCC_EUNSUPPORTED, "indices must be [M, top_k]");
+    f.top_k = I.dims[1] >= 0 ? (int32_t)I.dims[1] : -1;
+    if (f.top_k > 0 && A.dims[0] >= 0 && A.dims[0] != 1 && A.dims[0] != f.top_k)
+        return fail(OVFCC_EUNSUPPORTED, "the first dimension of the activations must be 1 or top_k");
+    if (f.top_k > E)
+        return fail(OVFCC_EUNSUPPORTED, "more selections per row than experts");
+
+    // ---- bias: Constant(dynamic, Shape{0}) = none; N values shared, or E x N ----
+    const int bias = g.input(root, 3);
+    if (bias >= 0 && element_count(g.at(bias)) != 0) {
+        const ovfcc_gnode& B = g.at(bias);
+        const int64_t bc = element_count(B);
+        if (B.op != OVFCC_OP_CONSTANT || !is_real(B.type) || (bc != N && bc != E * N) || B.rank < 1 ||
+            B.dims[B.rank - 1] != N)
+            return fail(OVFCC_EUNSUPPORTED, "bias must be an f16 / f32 Constant of N or E x N values with N innermost");
+        f.bias = bias;
+        f.bias_per_expert = bc == E * N && E > 1;
+        f.desc.bias_type = OVFCC_F16;
+        chain.add(bias);
+    }
+    f.n_experts = (int32_t)E;
+    f.weights = wc, f.scales = scale, f.zero_points = zp;
+    f.desc.N = N, f.desc.K = K, f.desc.group_size = G;
+    f.desc.w_type = W.type;
+    f.desc.scale_type = OVFCC_F16;
+    f.desc.act_type = OVFCC_F16;
+    f.desc.out_type = m.type == OVFCC_F32 ? OVFCC_F32 : OVFCC_F16;
+    f.w_view[0] = E, f.w_view[1] = N, f.w_view[2] = K;
+    if (!f.scale_broadcast)
+        f.scale_view[0] = E, f.scale_view[1] = N, f.scale_view[2] = ng;
+    if (zp >= 0 && !f.desc.zp_scalar)
+        f.zp_view[0] = E, f.zp_view[1] = N, f.zp_view[2] = ng;
+    if (E > ((int64_t)1 << 16))
+        return fail(OVFCC_EUNSUPPORTED, "more than 65536 experts");
+    int rc = ovfcc::validate_desc(&f.desc);
+    if (rc != OVFCC_OK)
+        return rc;
+    *out = f;
+    return OVFCC_OK;
+}
+
+bool is_gather(const ovfcc_gnode& n) {
+    return n.op == OVFCC_OP_GATHER_MATMUL || n.op == OVFCC_OP_GATHER_MATMUL_COMPRESSED;
+}
+
+int moe_impl(const Graph& g, int root, ovfcc_moe_fold* out) {
+    ovfcc_moe_fold f;
+    std::memset(&f, 0, sizeof(f));
+    f.root = root;
+    f.hidden_states = f.routing = f.indices = -1;
+    auto absorb = [&](int node) {
+        if (node >= 0 && f.n_chain < 16)
+            f.chain[f.n_chain++] = node;
+    };
+    if (!g.has(root))
+        return fail(OVFCC_EINVAL, "root is not a node of the graph");
+    int sum = root;
+    if (g.at(root).op == OVFCC_OP_RESHAPE) {
+        absorb(root);
+        absorb(g.input(root, 1));
+        sum = g.input(root, 0);
+    }
+    if (sum < 0 || g.at(sum).op != OVFCC_OP_REDUCE_SUM || g.at(sum).attr != 0)
+        return fail(OVFCC_EUNSUPPORTED, "the block does not end in ReduceSum(keep_dims = false) [-> Reshape]");
+    absorb(sum);
+    absorb(g.input(sum, 1));
+    const int mul = g.input(sum, 0);
+    if (mul < 0 || g.at(mul).op != OVFCC_OP_MULTIPLY || g.at(mul).consumers != 1)
+        return fail(OVFCC_EUNSUPPORTED, "ReduceSum must read a Multiply that nothing else reads");
+    absorb(mul);
+    // Multiply(down(..), Unsqueeze(Transpose([Slice](routing))))
+    int down = -1, unsq = -1;
+    for (int side = 0; side < 2; ++side) {
+        const int a = g.input(mul, side), b = g.input(mul, 1 - side);
+        if (a >= 0 && b >= 0 && is_gather(g.at(a)) && g.at(b).op == OVFCC_OP_UNSQUEEZE)
+            down = a, unsq = b;
+    }
+    if (down < 0)
+        return fail(OVFCC_EUNSUPPORTED, "no GatherMatmul multiplied by the unsqueezed routing weights");
+    absorb(unsq);
+    absorb(g.input(unsq, 1));
+    const int tr = g.input(unsq, 0);
+    if (tr < 0 || g.at(tr).op != OVFCC_OP_TRANSPOSE)
+        return fail(OVFCC_EUNSUPPORTED, "the routing weights must pass a Transpose ([M, top_k] -> [top_k, M])");
+    absorb(tr);
+    absorb(g.input(tr, 1));
+    f.routing = g.input(tr, 0);
+    if (f.routing < 0)
+        return fail(OVFCC_EINVAL, "Transpose without an input");
+    // the expert projections
+    const int glu_mul = g.input(down, 0);
+    if (glu_mul < 0 || g.at(glu_mul).op != OVFCC_OP_MULTIPLY)
+        return fail(OVFCC_EUNSUPPORTED, "the down projection must read Multiply(act(gate), up)");
+    absorb(glu_mul);
+    int gate = -1, up = -1, act = -1;
+    for (int side = 0; side < 2; ++side) {
+        const int a = g.input(glu_mul, side), b = g.input(glu_mul, 1 - side);
+        if (a >= 0 && b >= 0 && (g.at(a).op == OVFCC_OP_SWISH || g.at(a).op == OVFCC_OP_GELU) && is_gather(g.at(b))) {
+            const int gt = g.input(a, 0);
+            if (gt >= 0 && is_gather(g.at(gt)))
+                act = a, gate = gt, up = b;
+        }
+    }
+    if (gate < 0)
+        return fail(OVFCC_EUNSUPPORTED, "no Swish / Gelu of a GatherMatmul beside a second GatherMatmul");
+    if (g.at(act).op == OVFCC_OP_SWISH && g.at(act).n_inputs != 1)
+        return fail(OVFCC_EUNSUPPORTED, "Swish with a beta input");
+    absorb(act);
+    f.glu_type = g.at(act).op == OVFCC_OP_SWISH ? OVFCC_GLU_SWISH : (g.at(act).attr ? OVFCC_GLU_GELU_TANH : OVFCC_GLU_GELU);
+    // the three nodes are all plain or all compressed (the reference bails out on a mix)
+    if (g.at(gate).op != g.at(up).op || g.at(gate).op != g.at(down).op)
+        return fail(OVFCC_EUNSUPPORTED, "the three projections mix GatherMatmul and GatherMatmulCompressed");
+    int rc = gather_impl(g, gate, &f.gate);
+    if (!rc)
+        rc = gather_impl(g, up, &f.up);
+    if (!rc)
+        rc = gather_impl(g, down, &f.down);
+    if (rc)
+        return rc;
+    if (f.gate.bias >= 0 || f.up.bias >= 0 || f.down.bias >= 0)
+        return fail(OVFCC_EUNSUPPORTED, "the expert block has no place for biases");
+    if (f.gate.indices != f.up.indices || f.gate.indices != f.down.indices)
+        return fail(OVFCC_EUNSUPPORTED, "the three projections read different indices");
+    f.indices = f.gate.indices;
+    if (f.gate.activations != f.up.activations)
+        return fail(OVFCC_EUNSUPPORTED, "gate and up read different activations");
+    if (f.gate.n_experts != f.up.n_experts || f.gate.n_experts != f.down.n_experts)
+        return fail(OVFCC_EUNSUPPORTED, "the projections differ in their number of experts");
+    if (f.gate.desc.N != f.up.desc.N || f.gate.desc.K != f.up.desc.K || f.down.desc.K != f.gate.desc.N ||
+        f.down.desc.N != f.gate.desc.K)
+        return fail(OVFCC_EUNSUPPORTED, "the projections' shapes do not chain (gate, up: H -> I; down: I -> H)");
+    if (!same_format(f.gate.desc, f.up.desc))
+        return fail(OVFCC_EUNSUPPORTED, "gate and up differ in format");
+    if (f.gate.desc.out_type != OVFCC_F16)
+        return fail(OVFCC_EUNSUPPORTED, "the activations between the projections are f16");
+    // u = Unsqueeze([Reshape](hidden_states))
+    const int u = f.gate.activations;
+    if (g.at(u).op != OVFCC_OP_UNSQUEEZE)
+        return fail(OVFCC_EUNSUPPORTED, "gate and up must read Unsqueeze([Reshape](hidden states))");
+    absorb(u);
+    absorb(g.input(u, 1));
+    int h = g.input(u, 0);
+    if (h >= 0 && g.at(h).op == OVFCC_OP_RESHAPE) {
+        absorb(h);
+        absorb(g.input(h, 1));
+        h = g.input(h, 0);
+    }
+    if (h < 0)
+        return fail(OVFCC_EINVAL, "Unsqueeze without an input");
+    f.hidden_states = h;
+    const ovfcc_gnode& H = g.at(h);
+    if (H.rank < 2 || H.dims[H.rank - 1] != f.gate.desc.K)
+        return fail(OVFCC_EUNSUPPORTED, "the hidden states' last dimension is not the projections' input size");
+    const ovfcc_gnode& R = g.at(f.routing);
+    if (R.rank != 2 || (f.gate.top_k > 0 && R.dims[1] >= 0 && R.dims[1] != f.gate.top_k))
+        return fail(OVFCC_EUNSUPPORTED, "the routing weights that enter the Transpose must be [M, top_k]");
+    *out = f;
+    return OVFCC_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -362,8 +708,8 @@ int ovfcc_fold_match(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_fold
     if (!nodes || n_nodes <= 0 || !out)
         return fail(OVFCC_EINVAL, "null graph or output");
     for (int i = 0; i < n_nodes; ++i)
-        if (nodes[i].n_inputs < 0 || nodes[i].n_inputs > 4 || nodes[i].rank > OVFCC_MAX_RANK)
-            return fail(OVFCC_EINVAL, "a node has more than four inputs or a rank above OVFCC_MAX_RANK");
+        if (nodes[i].n_inputs < 0 || nodes[i].n_inputs > OVFCC_MAX_INPUTS || nodes[i].rank > OVFCC_MAX_RANK)
+            return fail(OVFCC_EINVAL, "a node has more than OVFCC_MAX_INPUTS inputs or a rank above OVFCC_MAX_RANK");
     return match_impl(Graph{nodes, n_nodes}, root, out);
 }
 
@@ -376,8 +722,8 @@ int ovfcc_fold_model(const ovfcc_gnode* nodes, int n_nodes, ovfcc_fold* folds, i
     // consumers of every node
     std::vector<std::vector<int>> users((size_t)n_nodes);
     for (int i = 0; i < n_nodes; ++i) {
-        if (nodes[i].n_inputs < 0 || nodes[i].n_inputs > 4 || nodes[i].rank > OVFCC_MAX_RANK)
-            return fail(OVFCC_EINVAL, "a node has more than four inputs or a rank above OVFCC_MAX_RANK");
+        if (nodes[i].n_inputs < 0 || nodes[i].n_inputs > OVFCC_MAX_INPUTS || nodes[i].rank > OVFCC_MAX_RANK)
+            return fail(OVFCC_EINVAL, "a node has more than OVFCC_MAX_INPUTS inputs or a rank above OVFCC_MAX_RANK");
         for (int k = 0; k < nodes[i].n_inputs; ++k)
             if (g.has(nodes[i].inputs[k]))
                 users[(size_t)nodes[i].inputs[k]].push_back(i);
@@ -473,6 +819,24 @@ int ovfcc_fold_model(const ovfcc_gnode* nodes, int n_nodes, ovfcc_fold* folds, i
     *n_folds = (int)found.size();
     *n_fused = (int)groups.size();
     return OVFCC_OK;
+}
+
+int ovfcc_fold_gather_matmul(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_gather_fold* out) {
+    if (!nodes || n_nodes <= 0 || !out)
+        return fail(OVFCC_EINVAL, "null graph or output");
+    for (int i = 0; i < n_nodes; ++i)
+        if (nodes[i].n_inputs < 0 || nodes[i].n_inputs > OVFCC_MAX_INPUTS || nodes[i].rank > OVFCC_MAX_RANK)
+            return fail(OVFCC_EINVAL, "a node has more than OVFCC_MAX_INPUTS inputs or a rank above OVFCC_MAX_RANK");
+    return gather_impl(Graph{nodes, n_nodes}, root, out);
+}
+
+int ovfcc_fold_moe(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_moe_fold* out) {
+    if (!nodes || n_nodes <= 0 || !out)
+        return fail(OVFCC_EINVAL, "null graph or output");
+    for (int i = 0; i < n_nodes; ++i)
+        if (nodes[i].n_inputs < 0 || nodes[i].n_inputs > OVFCC_MAX_INPUTS || nodes[i].rank > OVFCC_MAX_RANK)
+            return fail(OVFCC_EINVAL, "a node has more than OVFCC_MAX_INPUTS inputs or a rank above OVFCC_MAX_RANK");
+    return moe_impl(Graph{nodes, n_nodes}, root, out);
 }
 
 }  // extern "C"

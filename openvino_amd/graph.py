@@ -98,6 +98,41 @@ class Graph:
     def gelu(self, x, tanh=False):
         return self._add("gelu", self.type(x), self.shape(x), [x], attr=int(tanh))
 
+    def unsqueeze(self, x, axis):
+        s = self.shape(x)
+        axis = axis if axis >= 0 else axis + len(s) + 1
+        c = self.constant("i32", [1], ints=[axis])
+        return self._add("unsqueeze", self.type(x), s[:axis] + [1] + s[axis:], [x, c])
+
+    def slice(self, x, shape):
+        """v8::Slice with constant begin / end / step / axes; shape: the resolved output shape"""
+        cs = [self.constant("i32", [1]) for _ in range(4)]
+        return self._add("slice", self.type(x), shape, [x] + cs)
+
+    def reduce_sum(self, x, axis, keep_dims=False):
+        s = self.shape(x)
+        c = self.constant("i32", [1], ints=[axis])
+        out = [d for i, d in enumerate(s) if i != axis] if not keep_dims else [1 if i == axis else d for i, d in enumerate(s)]
+        return self._add("reduce_sum", self.type(x), out, [x, c], attr=int(keep_dims))
+
+    def no_bias(self):
+        """Constant(element::dynamic, Shape{0}): the reference's "no bias" input"""
+        return self.constant("other", [0])
+
+    def gather_matmul(self, a, b, indices, bias=None, type_=None):
+        """ov::op::internal::GatherMatmul: A [1 or top_k, M, K], B [E, N, K], indices [M, top_k] -> [top_k, M, N]"""
+        bias = self.no_bias() if bias is None else bias
+        sa, sb, si = self.shape(a), self.shape(b), self.shape(indices)
+        return self._add("gather_matmul", type_ or self.type(a), [si[1], sa[1], sb[1]], [a, b, indices, bias])
+
+    def gather_matmul_compressed(self, a, b, indices, scale, zp=None, bias=None, type_=None):
+        """ov::op::internal::GatherMatmulCompressed: B, scale, zp Constants of three dimensions"""
+        bias = self.no_bias() if bias is None else bias
+        zp = self.constant("other", [0]) if zp is None else zp
+        sa, sb, si = self.shape(a), self.shape(b), self.shape(indices)
+        return self._add("gather_matmul_compressed", type_ or self.type(a), [si[1], sa[1], sb[1]],
+                         [a, b, indices, bias, scale, zp])
+
     def other(self, inputs, type_="f16", shape=None):
         return self._add("other", type_, shape, list(inputs))
 
@@ -114,6 +149,16 @@ class Graph:
     def fold_match(self, root: int) -> _lib.Fold:
         out = _lib.Fold()
         check(_lib.load().ovfcc_fold_match(self._array(), len(self.nodes), root, ctypes.byref(out)))
+        return out
+
+    def fold_gather_matmul(self, root: int) -> _lib.GatherFold:
+        out = _lib.GatherFold()
+        check(_lib.load().ovfcc_fold_gather_matmul(self._array(), len(self.nodes), root, ctypes.byref(out)))
+        return out
+
+    def fold_moe(self, root: int) -> _lib.MoeFold:
+        out = _lib.MoeFold()
+        check(_lib.load().ovfcc_fold_moe(self._array(), len(self.nodes), root, ctypes.byref(out)))
         return out
 
     def fold_model(self, max_folds: int = 64):

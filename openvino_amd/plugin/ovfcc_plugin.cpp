@@ -18,7 +18,12 @@
 //  src/plugins/intel_cpu/src/transformations/cpu_opset/common/pass/fc_bias_fusion.cpp:32-93).  Two or three such nodes
 // of one format over the same Parameter run as one launch (horizontal fusion,
 // src/plugins/intel_gpu/src/plugin/transformations/fc_horizontal_fusion.cpp), and Multiply(Swish | Gelu (gate(x)), up(x))
-// runs as one node with a gated-linear-unit epilogue.  The pattern is matched on the untouched input model, before
+// runs as one node with a gated-linear-unit epilogue.  A mixture-of-experts block in the form the reference's
+// Convert3GatherMatmulMoeBlockToMoeOp matches (three GatherMatmul / GatherMatmulCompressed nodes over batched
+// compressed constants [E, N, K] or [E, N, K/G, G], the gate activation, the Multiply by the transposed routing
+// weights, ReduceSum and Reshape; src/common/transformations/src/transformations/common_optimizations/
+// moe_op_fusion.cpp:55-232) whose hidden states, routing weights and expert indices are Parameters runs as one
+// ovfcc_moe_device call -- MOECompressed in the executed graph.  The pattern is matched on the untouched input model, before
 // any folding pass, so the u4/u8 constants are still there and no MarkDequantization pass is needed.  Everything
 // else is reported as unsupported by query_model (a HETERO device can place it elsewhere) and rejected by
 // compile_model.
@@ -49,11 +54,14 @@
 #include "openvino/op/matmul.hpp"
 #include "openvino/op/multiply.hpp"
 #include "openvino/op/parameter.hpp"
+#include "openvino/op/reduce_sum.hpp"
 #include "openvino/op/reshape.hpp"
 #include "openvino/op/result.hpp"
+#include "openvino/op/slice.hpp"
 #include "openvino/op/subtract.hpp"
 #include "openvino/op/swish.hpp"
 #include "openvino/op/transpose.hpp"
+#include "openvino/op/unsqueeze.hpp"
 #include "openvino/pass/serialize.hpp"
 #include "openvino/runtime/exec_model_info.hpp"
 #include "openvino/runtime/icompiled_model.hpp"
@@ -64,6 +72,8 @@
 #include "openvino/runtime/properties.hpp"
 #include "ov_ops/fully_connected.hpp"
 #include "ov_ops/fully_connected_compressed.hpp"
+#include "ov_ops/gather_matmul.hpp"
+#include "ov_ops/gather_matmul_compressed.hpp"
 #include "ovfcc.h"
 #include "ovfcc_graph.h"
 
@@ -94,6 +104,7 @@ struct ModelGraph {
     std::vector<ovfcc_gnode> nodes;
     std::vector<ovfcc_fold> folds;
     std::vector<ovfcc_fused> fused;
+    std::vector<ovfcc_moe_fold> moes;  // expert blocks (three GatherMatmul nodes and what joins them)
 };
 
 static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
@@ -121,8 +132,13 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
         else if (ov::is_type<ov::op::v4::Swish>(op)) n.op = OVFCC_OP_SWISH;
         else if (ov::is_type<ov::op::v7::Gelu>(op)) n.op = OVFCC_OP_GELU;
         else if (ov::is_type<ov::op::v0::Result>(op)) n.op = OVFCC_OP_RESULT;
+        else if (ov::is_type<ov::op::internal::GatherMatmulCompressed>(op)) n.op = OVFCC_OP_GATHER_MATMUL_COMPRESSED;
+        else if (ov::is_type<ov::op::internal::GatherMatmul>(op)) n.op = OVFCC_OP_GATHER_MATMUL;
+        else if (ov::is_type<ov::op::v0::Unsqueeze>(op)) n.op = OVFCC_OP_UNSQUEEZE;
+        else if (ov::is_type<ov::op::v8::Slice>(op)) n.op = OVFCC_OP_SLICE;
+        else if (ov::is_type<ov::op::v1::ReduceSum>(op)) n.op = OVFCC_OP_REDUCE_SUM;
         else n.op = OVFCC_OP_OTHER;
-        if (op->get_output_size() == 0 || op->get_input_size() > 4) {
+        if (op->get_output_size() == 0 || op->get_input_size() > OVFCC_MAX_INPUTS) {
             n.op = OVFCC_OP_OTHER;
             n.rank = -1;
             continue;
@@ -145,6 +161,8 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
             n.transpose_b = mm->get_transpose_b();
         } else if (auto gelu = ov::as_type_ptr<ov::op::v7::Gelu>(op)) {
             n.attr = gelu->get_approximation_mode() == ov::op::GeluApproximationMode::TANH;
+        } else if (auto rs = ov::as_type_ptr<ov::op::v1::ReduceSum>(op)) {
+            n.attr = rs->get_keep_dims();
         } else if (auto sw = ov::as_type_ptr<ov::op::v4::Swish>(op)) {
             if (sw->get_input_size() != 1)
                 n.op = OVFCC_OP_OTHER;  // a beta input: not the beta = 1 form the kernels compute
@@ -167,6 +185,14 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
         throw_last("fold_model");
     g.folds.resize(n_folds);
     g.fused.resize(n_fused);
+    // expert blocks: every node that feeds a Result is tried as the block's root
+    for (size_t i = 0; i < g.nodes.size(); ++i) {
+        if (g.nodes[i].op != OVFCC_OP_RESULT)
+            continue;
+        ovfcc_moe_fold m;
+        if (ovfcc_fold_moe(g.nodes.data(), (int)g.nodes.size(), g.nodes[i].inputs[0], &m) == OVFCC_OK)
+            g.moes.push_back(m);
+    }
     return g;
 }
 
@@ -216,6 +242,70 @@ static NodeData node_data(const ModelGraph& g, const ovfcc_fold& f) {
             d.bias[i] = ov::float16(vals[i]);
     }
     return d;
+}
+
+// Expert e's node of a GatherMatmul fold: slice e of every constant, unpacked and re-packed where a 4-bit slice
+// starts in the middle of a byte.
+static ovfcc_weights* create_expert(ovfcc_ctx* ctx, const ModelGraph& g, const ovfcc_gather_fold& f, int e, int flags) {
+    const auto constant = [&g](int id) { return ov::as_type_ptr<ov::op::v0::Constant>(g.ops[(size_t)id]); };
+    const auto four = [](int t) { return t == OVFCC_U4 || t == OVFCC_I4; };
+    // `count` elements starting at element `first` of a packed constant, as a packed buffer of their own
+    const auto slice = [&](const std::shared_ptr<ov::op::v0::Constant>& c, bool nibbles, size_t first, size_t count) {
+        const auto* bytes = static_cast<const uint8_t*>(c->get_data_ptr());
+        std::vector<uint8_t> out(nibbles ? (count + 1) / 2 : count, 0);
+        if (!nibbles) {
+            std::memcpy(out.data(), bytes + first, count);
+        } else if ((first & 1) == 0) {
+            std::memcpy(out.data(), bytes + first / 2, (count + 1) / 2);
+        } else {
+            for (size_t i = 0; i < count; ++i) {
+                const size_t at = first + i;
+                const uint8_t v = (at & 1) ? (bytes[at >> 1] >> 4) : (bytes[at >> 1] & 15);
+                out[i >> 1] |= (uint8_t)((i & 1) ? v << 4 : v);
+            }
+        }
+        return out;
+    };
+    ovfcc_fc_desc d = f.desc;
+    d.flags |= flags;
+    const size_t N = (size_t)d.N, K = (size_t)d.K, ng = K / (size_t)d.group_size;
+    const auto w = slice(constant(f.weights), four(d.w_type), (size_t)e * N * K, N * K);
+    std::vector<ov::float16> scales(N * ng);
+    {
+        const auto vals = constant(f.scales)->cast_vector<float>();
+        for (size_t i = 0; i < N * ng; ++i)
+            scales[i] = ov::float16(vals[f.scale_broadcast ? 0 : (size_t)e * N * ng + i]);
+    }
+    std::vector<uint8_t> zp;
+    if (f.zero_points >= 0) {
+        auto z = constant(f.zero_points);
+        if (f.zp_from_real) {
+            const auto vals = z->cast_vector<float>();
+            const size_t count = d.zp_scalar ? 1 : N * ng, first = d.zp_scalar ? 0 : (size_t)e * N * ng;
+            zp.resize(count);
+            for (size_t i = 0; i < count; ++i) {
+                const float v = vals[first + i];
+                OPENVINO_ASSERT(v >= 0 && v <= 255 && v == (float)(int)v, "MI355X: zero-point values must be integers in 0..255");
+                zp[i] = (uint8_t)v;
+            }
+        } else if (d.zp_scalar) {
+            zp = slice(z, d.zp_type == OVFCC_U4, 0, 1);
+        } else {
+            zp = slice(z, d.zp_type == OVFCC_U4, (size_t)e * N * ng, N * ng);
+        }
+    }
+    std::vector<ov::float16> bias;
+    if (f.bias >= 0) {
+        const auto vals = constant(f.bias)->cast_vector<float>();
+        bias.resize(N);
+        for (size_t i = 0; i < N; ++i)
+            bias[i] = ov::float16(vals[(f.bias_per_expert ? (size_t)e * N : 0) + i]);
+    }
+    ovfcc_weights* out = nullptr;
+    if (ovfcc_weights_create(ctx, &d, w.data(), scales.data(), zp.empty() ? nullptr : zp.data(),
+                             bias.empty() ? nullptr : bias.data(), &out) != OVFCC_OK)
+        throw_last("weights_create (expert)");
+    return out;
 }
 
 // ---- device-resident tensors -------------------------------------------------------------------------------
@@ -376,6 +466,17 @@ struct Launch {
     std::vector<int> folds;         // indices into ModelGraph::folds
 };
 
+// One expert block of the compiled model = one ovfcc_moe_device call per inference.
+struct MoeLaunch {
+    std::vector<ovfcc_weights*> gate_up, down;  // per expert: gate and up with the gated linear unit, down
+    size_t hidden_index = 0, routing_index = 0, indices_index = 0;  // the Parameters
+    size_t result_index = 0;
+    int64_t H = 0;
+    int top_k = 0, out_type = OVFCC_F16;
+    std::string name;
+    std::vector<std::string> original_names;
+};
+
 class CompiledModel : public ov::ICompiledModel {
 public:
     // node_flags: OVFCC_* flags for every node's descriptor (OVFCC_DYNQUANT_I8 when the caller allows dynamic
@@ -386,12 +487,20 @@ public:
     ~CompiledModel() override {
         for (auto& l : m_launches)
             ovfcc_weights_destroy(l.weights);
+        for (auto& m : m_moes) {
+            for (auto* w : m.gate_up)
+                ovfcc_weights_destroy(w);
+            for (auto* w : m.down)
+                ovfcc_weights_destroy(w);
+        }
     }
 
     // Stream layout: magic, node flags, the model as the template plugin stores it (xml and constants from
     // ov::pass::Serialize, each behind its size; src/plugins/template/src/compiled_model.cpp:173-192), then the
     // number of launches and every launch's repacked device image (ovfcc_weights_export) behind its size.
     void export_model(std::ostream& out) const override {
+        OPENVINO_ASSERT(m_moes.empty(), "MI355X: a model with expert blocks is compiled from its constants each time "
+                                         "(no blob form of an expert block)");
         std::stringstream xml, bin;
         ov::pass::Serialize(xml, bin).run_on_model(m_model);
         const std::string x = xml.str(), b = bin.str();
@@ -454,6 +563,26 @@ public:
                 results[o.result_index]->set_friendly_name(m_model->get_results()[o.result_index]->get_friendly_name());
             }
         }
+        for (size_t i = 0; i < m_moes.size(); ++i) {
+            const MoeLaunch& m = m_moes[i];
+            auto node = std::make_shared<ov::exec_model_info::ExecutionNode>(
+                ov::OutputVector{params[m.hidden_index], params[m.routing_index], params[m.indices_index]}, 1);
+            node->set_friendly_name(m.name);
+            auto& rt = node->get_rt_info();
+            std::string names;
+            for (const auto& n : m.original_names)
+                names += (names.empty() ? "" : ",") + n;
+            rt[ov::exec_model_info::LAYER_TYPE] = std::string("MOECompressed");
+            rt[ov::exec_model_info::IMPL_TYPE] = std::string("hip_moe_grouped_w4");
+            rt[ov::exec_model_info::ORIGINAL_NAMES] = names;
+            rt[ov::exec_model_info::OUTPUT_PRECISIONS] = std::string(m.out_type == OVFCC_F32 ? "f32" : "f16");
+            rt[ov::exec_model_info::OUTPUT_LAYOUTS] = std::string("ab");
+            rt[ov::exec_model_info::EXECUTION_ORDER] = std::to_string(m_launches.size() + i);
+            const double us = m_last_us[m_launches.size() + i].load();
+            rt[ov::exec_model_info::PERF_COUNTER] = us < 0 ? std::string("not_executed") : std::to_string((long long)us);
+            results[m.result_index] = std::make_shared<ov::op::v0::Result>(node);
+            results[m.result_index]->set_friendly_name(m_model->get_results()[m.result_index]->get_friendly_name());
+        }
         return std::make_shared<ov::Model>(results, params, m_model->get_friendly_name() + "_executed");
     }
     void set_property(const ov::AnyMap&) override {
@@ -478,6 +607,9 @@ public:
 
     const std::vector<Launch>& launches() const {
         return m_launches;
+    }
+    const std::vector<MoeLaunch>& moes() const {
+        return m_moes;
     }
     ovfcc_ctx* ctx() const {
         return m_ctx;
@@ -509,6 +641,7 @@ private:
     std::shared_ptr<ov::Model> m_model;
     ModelGraph m_graph;
     std::vector<Launch> m_launches;
+    std::vector<MoeLaunch> m_moes;
     mutable std::vector<std::atomic<double>> m_last_us;  // per launch: last measured time, -1 before the first run
     ovfcc_ctx* m_ctx;
     int m_node_flags = 0;
@@ -615,6 +748,7 @@ public:
             m_times_us.push_back(us);
             m_compiled->record_time(li, us);
         }
+        run_expert_blocks();
     }
 
     std::vector<ov::ProfilingInfo> get_profiling_info() const override {
@@ -622,8 +756,9 @@ public:
         for (size_t i = 0; i < m_kernels.size(); ++i) {
             ov::ProfilingInfo p;
             p.status = ov::ProfilingInfo::Status::EXECUTED;
-            p.node_name = m_compiled->launches()[i].name;
-            p.node_type = "FullyConnected";
+            const size_t n_fc = m_compiled->launches().size();
+            p.node_name = i < n_fc ? m_compiled->launches()[i].name : m_compiled->moes()[i - n_fc].name;
+            p.node_type = i < n_fc ? "FullyConnected" : "MOECompressed";
             p.exec_type = m_kernels[i].name;
             p.real_time = p.cpu_time = std::chrono::microseconds((long long)m_times_us[i]);
             out.push_back(p);
@@ -641,6 +776,79 @@ private:
             tensor = ov::make_tensor(type, shape);
         else
             tensor->set_shape(shape);
+    }
+
+    // Expert blocks: hidden states [.., H], routing weights [M, top_k] and indices [M, top_k] in host tensors;
+    // staged to the device (f16, f16, int32), one ovfcc_moe_device call, result copied back.
+    void run_expert_blocks() {
+        const auto& moes = m_compiled->moes();
+        for (size_t mi = 0; mi < moes.size(); ++mi) {
+            const MoeLaunch& m = moes[mi];
+            const auto t0 = std::chrono::steady_clock::now();
+            auto hidden = get_tensor(get_inputs()[m.hidden_index]);
+            auto routing = get_tensor(get_inputs()[m.routing_index]);
+            auto indices = get_tensor(get_inputs()[m.indices_index]);
+            auto out = get_tensor(get_outputs()[m.result_index]);
+            const ov::Shape in_shape = hidden->get_shape();
+            int64_t M = 1;
+            for (size_t d = 0; d + 1 < in_shape.size(); ++d)
+                M *= (int64_t)in_shape[d];
+            out->set_shape(in_shape);
+            const size_t pairs = (size_t)M * (size_t)m.top_k;
+            OPENVINO_ASSERT(routing->get_size() == pairs && indices->get_size() == pairs,
+                            "MI355X: routing weights and indices must hold M x top_k values");
+            auto to_half = [this](const ov::SoPtr<ov::ITensor>& t, size_t count) -> const void* {
+                if (t->get_element_type() == ov::element::f16)
+                    return t->data();
+                OPENVINO_ASSERT(t->get_element_type() == ov::element::f32, "MI355X: expected an f16 or f32 tensor");
+                const float* src = static_cast<const float*>(t->data());
+                m_staging.resize(count);
+                for (size_t i = 0; i < count; ++i)
+                    m_staging[i] = ov::float16(src[i]);
+                return m_staging.data();
+            };
+            const size_t x_bytes = (size_t)M * m.H * 2, r_bytes = pairs * 2, y_bytes = (size_t)M * m.H * (m.out_type == OVFCC_F32 ? 4 : 2);
+            void* x_dev = device_staging(0, x_bytes);
+            void* y_dev = device_staging(1, y_bytes);
+            void* r_dev = device_staging(2, r_bytes);
+            if (x_bytes && ovfcc_memcpy_h2d(m_compiled->ctx(), x_dev, to_half(hidden, (size_t)M * m.H), x_bytes) != OVFCC_OK)
+                throw_last("memcpy_h2d");
+            if (r_bytes && ovfcc_memcpy_h2d(m_compiled->ctx(), r_dev, to_half(routing, pairs), r_bytes) != OVFCC_OK)
+                throw_last("memcpy_h2d");
+            std::vector<int32_t> idx(pairs);
+            if (indices->get_element_type() == ov::element::i32) {
+                std::memcpy(idx.data(), indices->data(), pairs * sizeof(int32_t));
+            } else {
+                OPENVINO_ASSERT(indices->get_element_type() == ov::element::i64, "MI355X: indices must be i32 or i64");
+                const int64_t* src = static_cast<const int64_t*>(indices->data());
+                for (size_t i = 0; i < pairs; ++i)
+                    idx[i] = (int32_t)src[i];
+            }
+            if (ovfcc_moe_device(m_request, m.gate_up.data(), m.down.data(), (int)m.gate_up.size(), x_dev, r_dev, idx.data(), M,
+                                 m.top_k, y_dev) != OVFCC_OK)
+                throw_last("moe_device");
+            if (ovfcc_request_sync(m_request) != OVFCC_OK)
+                throw_last("request_sync");
+            if (y_bytes) {
+                if (out->get_element_type() == ov::element::f32 && m.out_type != OVFCC_F32) {
+                    m_y_staging.resize(y_bytes);
+                    if (ovfcc_memcpy_d2h(m_compiled->ctx(), m_y_staging.data(), y_dev, y_bytes) != OVFCC_OK)
+                        throw_last("memcpy_d2h");
+                    const auto* h = reinterpret_cast<const ov::float16*>(m_y_staging.data());
+                    float* dst = static_cast<float*>(out->data());
+                    for (size_t i = 0; i < (size_t)M * m.H; ++i)
+                        dst[i] = (float)h[i];
+                } else if (ovfcc_memcpy_d2h(m_compiled->ctx(), out->data(), y_dev, y_bytes) != OVFCC_OK) {
+                    throw_last("memcpy_d2h");
+                }
+            }
+            ovfcc_kernel_info info;
+            ovfcc_last_kernel_info(m_request, &info);
+            m_kernels.push_back(info);
+            const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+            m_times_us.push_back(us);
+            m_compiled->record_time(m_compiled->launches().size() + mi, us);
+        }
     }
 
     // rows of m_y_staging ([M, N_out]) -> every output's columns (the VariadicSplit after a horizontally fused node)
@@ -674,7 +882,7 @@ private:
     };
     std::shared_ptr<const CompiledModel> m_compiled;
     ovfcc_request* m_request = nullptr;
-    DeviceBuffer m_device_staging[2];
+    DeviceBuffer m_device_staging[3];
     std::vector<ov::float16> m_staging;
     std::vector<uint8_t> m_y_staging;
     std::vector<ovfcc_kernel_info> m_kernels;
@@ -874,6 +1082,21 @@ public:
                 mark_results_of(u.root);
             }
         }
+        for (const auto& m : g.moes) {
+            for (int c = 0; c < m.n_chain; ++c)
+                mark(m.chain[c]);
+            for (const ovfcc_gather_fold* f : {&m.gate, &m.up, &m.down}) {
+                for (int c = 0; c < f->n_chain; ++c)
+                    mark(f->chain[c]);
+                mark(f->root);
+                if (g.ops[(size_t)f->root]->get_input_size() > 3)
+                    mark(g.nodes[(size_t)f->root].inputs[3]);  // the empty bias constant
+            }
+            for (int id : {m.hidden_states, m.routing, m.indices})
+                if (g.nodes[(size_t)id].op == OVFCC_OP_PARAMETER)
+                    mark(id);
+            mark_results_of(m.root);
+        }
         return res;
     }
 
@@ -1014,6 +1237,46 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
             }
         }
     }
+    for (const auto& m : g.moes) {
+        OPENVINO_ASSERT(!blobs, "MI355X: a model with expert blocks has no blob form");
+        MoeLaunch l;
+        auto param_index = [&](int id, const char* what) {
+            OPENVINO_ASSERT(g.nodes[(size_t)id].op == OVFCC_OP_PARAMETER, "MI355X: the ", what, " of ",
+                            g.ops[(size_t)m.root]->get_friendly_name(),
+                            " do not come straight from a Parameter (use HETERO:MI355X,CPU for the rest of the graph)");
+            for (size_t p = 0; p < params.size(); ++p)
+                if (params[p].get() == g.ops[(size_t)id].get())
+                    return p;
+            return (size_t)0;
+        };
+        l.hidden_index = param_index(m.hidden_states, "hidden states");
+        l.routing_index = param_index(m.routing, "routing weights");
+        l.indices_index = param_index(m.indices, "expert indices");
+        const auto rs = results_of(m.root);
+        OPENVINO_ASSERT(rs.size() == 1, "MI355X: an expert block must feed exactly one model output");
+        l.result_index = rs[0];
+        fed[rs[0]] = true;
+        l.H = m.gate.desc.K;
+        l.top_k = m.gate.top_k;
+        OPENVINO_ASSERT(l.top_k > 0, "MI355X: the number of experts per token must be static");
+        l.out_type = m.down.desc.out_type;
+        l.name = g.ops[(size_t)m.root]->get_friendly_name();
+        for (const ovfcc_gather_fold* f : {&m.gate, &m.up, &m.down})
+            l.original_names.push_back(g.ops[(size_t)f->root]->get_friendly_name());
+        l.original_names.push_back(l.name);
+        for (int e = 0; e < m.gate.n_experts; ++e) {
+            ovfcc_weights *gate = create_expert(ctx, g, m.gate, e, node_flags), *up = create_expert(ctx, g, m.up, e, node_flags);
+            ovfcc_weights* gu = nullptr;
+            const int rc = ovfcc_weights_glu(gate, up, m.glu_type, &gu);
+            ovfcc_weights_destroy(gate);
+            ovfcc_weights_destroy(up);
+            if (rc != OVFCC_OK)
+                throw_last("weights_glu (expert)");
+            l.gate_up.push_back(gu);
+            l.down.push_back(create_expert(ctx, g, m.down, e, node_flags));
+        }
+        m_moes.push_back(std::move(l));
+    }
     for (size_t r = 0; r < results.size(); ++r)
         OPENVINO_ASSERT(fed[r], "MI355X: result ", results[r]->get_friendly_name(),
                         " is not produced by a weight-compressed FullyConnected (use HETERO:MI355X,CPU for the rest "
@@ -1029,7 +1292,7 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
     for (auto& l : m_launches)
         l.primitive = primitive(l.weights, g.folds[(size_t)l.folds[0]].desc,
                                 l.kind == OVFCC_FUSED_GLU ? "_glu" : (l.kind == OVFCC_FUSED_CONCAT ? "_fused" : ""));
-    m_last_us = std::vector<std::atomic<double>>(m_launches.size());
+    m_last_us = std::vector<std::atomic<double>>(m_launches.size() + m_moes.size());
     for (auto& t : m_last_us)
         t.store(-1.0);
 }

@@ -8,6 +8,7 @@ import os
 import pytest
 
 from openvino_amd import _lib, fc
+from openvino_amd._lib import OvfccError
 from openvino_amd.graph import Graph, decompression_subgraph
 
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -310,3 +311,155 @@ def test_grouping_rules():
     two(g, h)
     with pytest.raises(fc.OvfccError):
         g.fold_model(max_folds=1)
+
+
+# ---- mixture-of-experts layers: GatherMatmul over batched compressed weights, and the three-projection block ----
+
+def expert_weights(g, type_, wei_shape, scale_zp_shape, grouped, with_zp=True, compute="f32"):
+    """Constant -> Convert -> [Subtract] -> Multiply -> [Reshape to three dimensions], as the reference's test builds it."""
+    w = g.convert(g.constant(type_, wei_shape), compute)
+    if with_zp:
+        w = g.subtract(w, g.convert(g.constant(type_, scale_zp_shape), compute))
+    w = g.multiply(w, g.constant(compute, scale_zp_shape))
+    if grouped:
+        w = g.reshape(w, list(wei_shape[:-2]) + [wei_shape[-2] * wei_shape[-1]])
+    return w
+
+
+@pytest.mark.parametrize("case", CASES["convert_gather_matmul_to_compressed"],
+                         ids=lambda c: f"{c['type']}-{'grouped' if c['grouped'] else 'plain'}-{c['wei_shape']}")
+def test_gather_matmul_over_compressed_experts(case):
+    """ConvertGatherMatmulToGatherMatmulCompressed's own cases: the node it would produce, as a per-expert descriptor
+    and views [E, N, K], [E, N, K/G] of the constants."""
+    g = Graph()
+    a = g.parameter("f32", case["in_shape"])
+    b = expert_weights(g, case["type"], case["wei_shape"], case["scale_zp_shape"], case["grouped"])
+    idx = g.constant("i32", case["index_shape"])
+    root = g.gather_matmul(a, b, idx)
+    f = g.fold_gather_matmul(root)
+    E, N = case["wei_shape"][0], case["wei_shape"][1]
+    K = case["wei_shape"][2] * (case["wei_shape"][3] if case["grouped"] else 1)
+    G = case["wei_shape"][3] if case["grouped"] else K
+    assert (f.n_experts, f.desc.N, f.desc.K, f.desc.group_size) == (E, N, K, G)
+    assert f.desc.w_type == _lib.TYPE[case["type"]] and f.desc.zp_type == _lib.TYPE[case["type"]]
+    assert f.desc.zp_scalar == 0 and f.scale_broadcast == 0 and f.bias == -1 and f.activations_f32 == 1
+    assert list(f.w_view) == [E, N, K] and list(f.scale_view) == [E, N, K // G] and list(f.zp_view) == [E, N, K // G]
+    assert f.activations == a and f.indices == idx and f.top_k == case["index_shape"][1] and f.root == root
+    assert g.nodes[f.weights].op == _lib.OP["constant"] and g.shape(f.weights) == case["wei_shape"]
+    # the same node as the pass leaves it: GatherMatmulCompressed over three-dimensional constants
+    g2 = Graph()
+    a2 = g2.parameter("f32", case["in_shape"])
+    sz = case["scale_zp_shape"][:-1] if case["grouped"] else case["scale_zp_shape"]
+    root2 = g2.gather_matmul_compressed(a2, g2.constant(case["type"], [E, N, K]), g2.constant("i32", case["index_shape"]),
+                                        g2.constant("f32", sz), g2.constant(case["type"], sz))
+    f2 = g2.fold_gather_matmul(root2)
+    assert (f2.n_experts, f2.desc.N, f2.desc.K, f2.desc.group_size) == (E, N, K, G)
+    assert f2.desc.zp_type == f.desc.zp_type and list(f2.scale_view) == list(f.scale_view)
+
+
+def test_gather_matmul_fold_variants_and_refusals():
+    g = Graph()
+    a = g.parameter("f16", [1, 40, 256])
+    idx = g.parameter("i32", [40, 2])
+    # symmetric i4 (no Subtract), f16 compute, scalar zero-point elsewhere, shared and per-expert bias
+    sym = g.gather_matmul(a, expert_weights(g, "i4", [8, 64, 2, 128], [8, 64, 2, 1], True, with_zp=False, compute="f16"), idx)
+    f = g.fold_gather_matmul(sym)
+    assert f.desc.zp_type == _lib.TYPE["none"] and f.desc.w_type == _lib.TYPE["i4"] and f.activations_f32 == 0
+    w = g.convert(g.constant("u4", [8, 64, 256]), "f16")
+    w = g.multiply(g.subtract(w, g.convert(g.constant("u4", []), "f16")), g.constant("f16", [8, 64, 1]))
+    f = g.fold_gather_matmul(g.gather_matmul(a, w, idx, bias=g.constant("f16", [8, 1, 64])))
+    assert f.desc.zp_scalar == 1 and f.bias_per_expert == 1 and f.desc.bias_type == _lib.TYPE["f16"]
+    f = g.fold_gather_matmul(g.gather_matmul(a, w, idx, bias=g.constant("f16", [64])))
+    assert f.bias_per_expert == 0 and f.bias >= 0
+    for bad, why in [
+        (lambda: g.gather_matmul(a, g.constant("f16", [8, 64, 256]), idx), "no decompression subgraph"),
+        (lambda: g.gather_matmul(g.parameter("f16", [1, 40, 128]), w, idx), "K mismatch"),
+        (lambda: g.gather_matmul(g.parameter("f16", [3, 40, 256]), w, idx), "A batches neither 1 nor top_k"),
+        (lambda: g.gather_matmul(a, w, g.parameter("i32", [40, 9])), "more selections than experts"),
+        (lambda: g.gather_matmul(a, g.transpose(w, [0, 2, 1]), idx), "transposed expert weights"),
+        (lambda: g.gather_matmul(a, w, idx, bias=g.constant("f16", [8, 1, 32])), "bias of the wrong width"),
+    ]:
+        with pytest.raises(OvfccError) as e:
+            g.fold_gather_matmul(bad())
+        assert e.value.code == _lib.EUNSUPPORTED, why
+
+
+def moe_block(g, act, compressed, E, H, I, top_k, hidden_shape, wtype="u4", G=128, routing_slice=False):
+    """build_3gemm_bgm_model with compressed experts: returns (root, hidden, routing producer, indices, nodes)."""
+    hidden = g.parameter("f16", hidden_shape)
+    flat = g.reshape(hidden, [-1, H]) if len(hidden_shape) != 2 else hidden
+    u = g.unsqueeze(flat, 0)
+    idx = g.parameter("i32", [-1, top_k])
+    routing = g.parameter("f16", [-1, E if routing_slice else top_k])
+
+    def bgm(x, N, K):
+        if compressed:
+            return g.gather_matmul_compressed(x, g.constant(wtype, [E, N, K]), idx, g.constant("f16", [E, N, K // G]),
+                                              g.constant(wtype, [E, N, K // G]))
+        return g.gather_matmul(x, expert_weights(g, wtype, [E, N, K // G, G], [E, N, K // G, 1], True, compute="f16"), idx)
+    gate = bgm(u, I, H)
+    a = g.swish(gate) if act == "swish" else g.gelu(gate, tanh=(act == "gelu_tanh"))
+    up = bgm(u, I, H)
+    down = bgm(g.multiply(a, up), H, I)
+    r = g.slice(routing, [-1, top_k]) if routing_slice else routing
+    final = g.multiply(down, g.unsqueeze(g.transpose(r, [1, 0]), -1))
+    out = g.reshape(g.reduce_sum(final, 0), hidden_shape)
+    return out, hidden, r, idx, (gate, up, down)
+
+
+@pytest.mark.parametrize("act", CASES["moe_block"]["activations"])
+@pytest.mark.parametrize("compressed", [False, True])
+def test_moe_block_of_three_gather_matmuls(act, compressed):
+    """The shapes of the reference's build_3gemm_bgm_model: one MOECompressed block with its inputs named."""
+    c = CASES["moe_block"]
+    E, H, I, top_k = c["number_of_experts"], c["hidden_size"], c["intermediate_size"], c["topk"]
+    g = Graph()
+    root, hidden, routing, idx, (gate, up, down) = moe_block(g, act, compressed, E, H, I, top_k, [c["batch"], -1, H])
+    m = g.fold_moe(root)
+    assert m.glu_type == {"swish": 1, "gelu_erf": 2, "gelu_tanh": 3}[act]
+    assert (m.root, m.hidden_states, m.routing, m.indices) == (root, hidden, routing, idx)
+    assert (m.gate.root, m.up.root, m.down.root) == (gate, up, down)
+    for f, (N, K) in ((m.gate, (I, H)), (m.up, (I, H)), (m.down, (H, I))):
+        assert (f.n_experts, f.desc.N, f.desc.K, f.desc.group_size, f.top_k) == (E, N, K, 128, top_k)
+        assert f.desc.w_type == _lib.TYPE["u4"] and f.desc.zp_type == _lib.TYPE["u4"]
+    # the ReduceSum is accepted as root too
+    assert g.fold_moe(g.nodes[root].inputs[0]).hidden_states == hidden
+
+
+def test_moe_block_refusals():
+    E, H, I, top_k = 4, 256, 512, 2
+    g = Graph()
+    root, *_ = moe_block(g, "swish", True, E, H, I, top_k, [6, H], routing_slice=True)
+    m = g.fold_moe(root)
+    assert g.nodes[m.routing].op == _lib.OP["slice"]          # the Slice stays outside and feeds the block
+    # ReduceSum that keeps the dimension, a second reader of the final Multiply, mixed plain / compressed nodes
+    g = Graph()
+    root, hidden, r, idx, (gate, up, down) = moe_block(g, "swish", True, E, H, I, top_k, [6, H])
+    final = g.nodes[g.nodes[root].inputs[0]].inputs[0]
+    g.result(final)
+    with pytest.raises(OvfccError):
+        g.fold_moe(root)
+    g = Graph()
+    hidden = g.parameter("f16", [6, H])
+    u = g.unsqueeze(hidden, 0)
+    idx = g.parameter("i32", [6, top_k])
+    gate = g.gather_matmul_compressed(u, g.constant("u4", [E, I, H]), idx, g.constant("f16", [E, I, 2]), g.constant("u4", [E, I, 2]))
+    up = g.gather_matmul(u, expert_weights(g, "u4", [E, I, 2, 128], [E, I, 2, 1], True, compute="f16"), idx)
+    down = g.gather_matmul_compressed(g.multiply(g.swish(gate), up), g.constant("u4", [E, H, I]), idx,
+                                      g.constant("f16", [E, H, 4]), g.constant("u4", [E, H, 4]))
+    out = g.reduce_sum(g.multiply(down, g.unsqueeze(g.transpose(g.parameter("f16", [6, top_k]), [1, 0]), -1)), 0)
+    with pytest.raises(OvfccError) as e:
+        g.fold_moe(out)
+    assert "mix" in e.value.message
+    # shapes that do not chain
+    g = Graph()
+    hidden = g.parameter("f16", [6, H])
+    u = g.unsqueeze(hidden, 0)
+    idx = g.parameter("i32", [6, top_k])
+    mk = lambda x, N, K: g.gather_matmul_compressed(x, g.constant("u4", [E, N, K]), idx, g.constant("f16", [E, N, K // 128]),
+                                                    g.constant("u4", [E, N, K // 128]))
+    down = mk(g.multiply(g.swish(mk(u, I, H)), mk(u, I, H)), H + 128, I)
+    out = g.reduce_sum(g.multiply(down, g.unsqueeze(g.transpose(g.parameter("f16", [6, top_k]), [1, 0]), -1)), 0)
+    with pytest.raises(OvfccError) as e:
+        g.fold_moe(out)
+    assert "chain" in e.value.message
