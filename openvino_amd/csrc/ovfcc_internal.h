@@ -131,6 +131,7 @@ struct LaunchPlan {
     bool batch = false;         // decode family: the small-batch kernel (waves own channel tiles)
     bool gemv = false;          // decode family: the matrix-vector kernel for M <= 4 (4-bit weights, G = 128)
     int gemv_c = 0;             // ... and its k-blocks per wave (2, 4 or 8)
+    bool gemv16 = false;        // decode family: its 16-row sibling with stationary activations (5 <= M <= 32)
     int tiles_x = 0, tiles_y = 0;  // async prefill kernel: the tile grid; its launch is 1-D
     int full_tiles = 0;         // ... of which this many run unsplit (the rest in split_k parts each)
     unsigned grid[3] = {1, 1, 1};
@@ -155,6 +156,9 @@ int launch_plain(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_decode(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_batch(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_gemv(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+// dynamic LDS of the 16-row kernel: c k-blocks per wave, `waves` waves, one or two buffers of partial sums
+size_t gemv16_lds_bytes(int c, int waves, int red_bufs);
 // dynamic LDS of the matrix-vector kernel: c k-blocks per wave, m rows, `waves` waves per workgroup
 size_t gemv_lds_bytes(int c, int m, int waves);
 // [N/16][groups][16] scales f16 (and zero-points u8, or null) -> channel-major [N/16][16][groups]

@@ -4,6 +4,7 @@
 // M <= 48 (the streaming kernel for a few rows, the small-batch kernel above) and the prefill kernel for more
 // (the roofline ridge of int4 g128 sits near M = 83).  The caller cuts 48 < M <= 128 into decode launches:
 // a single 128-row prefill tile per column block leaves most of the chip idle.
+#include <algorithm>
 #include <atomic>
 #include <cstdlib>
 #include <cstring>
@@ -18,6 +19,8 @@ namespace ovfcc {
 //   tuning:  OVFCC_DECODE_WAVES = 4 | 8 | 16 (workgroup size), OVFCC_DECODE_RT = 1 | 2 | 4 (channel tiles per
 //            workgroup or wave), OVFCC_DECODE_XLDS = 0 | 1 (activations via LDS), OVFCC_DECODE_BATCH = 0 | 1
 //            (small-batch kernel instead of the streaming kernel), OVFCC_GEMV = 0 | 1, OVFCC_GEMV_C = 2 | 4 | 8,
+//            OVFCC_GEMV16 = 0 | 1 (the 16-row kernel with stationary activations for 5-32 rows),
+//            OVFCC_GEMV16_GRID = n (its workgroups per row tile),
 //            OVFCC_PREFILL_{DIRECT, ASYNC, WIDE, BIG, TAIL} = 0 | 1, OVFCC_PREFILL_ROWS = 64 | 128,
 //            OVFCC_MOE_HOST_ROUTING = 1;
 //   logging: OVFCC_VERBOSE = 1 (one line per launch on stderr), 2 (also weights and requests as they come and go).
@@ -30,6 +33,7 @@ struct EnvEntry {
 };
 EnvEntry g_env[] = {EnvEntry("OVFCC_DECODE_WAVES"),   EnvEntry("OVFCC_DECODE_RT"),      EnvEntry("OVFCC_DECODE_XLDS"),
                     EnvEntry("OVFCC_DECODE_BATCH"),   EnvEntry("OVFCC_GEMV"),           EnvEntry("OVFCC_GEMV_C"),
+                    EnvEntry("OVFCC_GEMV16"),         EnvEntry("OVFCC_GEMV16_GRID"),
                     EnvEntry("OVFCC_PREFILL_DIRECT"), EnvEntry("OVFCC_PREFILL_ASYNC"),  EnvEntry("OVFCC_PREFILL_WIDE"),
                     EnvEntry("OVFCC_PREFILL_BIG"),    EnvEntry("OVFCC_PREFILL_TAIL"),   EnvEntry("OVFCC_PREFILL_ROWS"),
                     EnvEntry("OVFCC_MOE_HOST_ROUTING"), EnvEntry("OVFCC_VERBOSE")};
@@ -67,7 +71,8 @@ int env_int(const char* name, int fallback) {
 
 // k-blocks per wave of the matrix-vector kernel for this node (0: the kernel does not fit it).  The waves of one
 // channel tile (of a gate / up tile pair) share a workgroup of at most 16 waves and each takes 2, 4 or 8 whole
-// k-blocks; of the divisions that fit, the coarsest one that still gives every SIMD of the chip about two waves.
+// k-blocks; of the divisions that fit, the coarsest one that still gives every SIMD of the chip about two waves,
+// but no coarser than a workgroup of eight waves needs.
 // OVFCC_GEMV_C overrides for experiments.
 int gemv_kblocks_per_wave(const Layout& L, int n_cus) {
     const int tiles_per_wg = L.glu ? 2 : 1;
@@ -81,6 +86,11 @@ int gemv_kblocks_per_wave(const Layout& L, int n_cus) {
     for (int c : {2, 4, 8})
         if (fits(c) && (best == 0 || L.n_tiles * (L.k_blocks / c) >= (int64_t)8 * n_cus))
             best = c;
+    // Eight k-blocks per wave leave a plain node of K = 4096 with four waves per workgroup; eight waves of four
+    // k-blocks stream the same bytes faster (gate / up at one row: 7.0 against 7.3 us) and give the 16-row kernel
+    // two waves per SIMD (16 rows: 10.7 against 12.8 us).
+    if (best == 8 && !L.glu && fits(4) && L.k_blocks / 4 <= 8)
+        best = 4;
     return best;
 }
 
@@ -154,6 +164,49 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.name = L.bits == 4 ? "fcc_batch_w4" : "fcc_batch_w8";
         return OVFCC_OK;
     };
+    // Five to 32 rows of a 4-bit node with groups of 128 inputs whose 16 rows x K of activations fit in LDS (and,
+    // divided among the waves, in registers): the 16-row sibling of the matrix-vector kernel.  Every workgroup
+    // keeps its row tile of the activations and walks channel tiles; the grid is as many workgroups as the chip
+    // holds at once, rounded so that all of them visit the same number of tiles.
+    auto plan_gemv16 = [&]() -> bool {
+        if (a.M <= 4 || a.M > 32 || !a.scale_cm || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 ||
+            L.glu || force_split > 0 || L.gemv_c == 0 || env_int("OVFCC_GEMV16", 1) == 0 ||
+            env_int("OVFCC_DECODE_BATCH", -1) >= 0)
+            return false;
+        const int c = L.gemv_c, waves = (int)(L.k_blocks / c);
+        // the kernel's registers allow 4, 8 and 16 waves per compute unit with 8, 4 and 2 k-blocks per wave
+        const int cu_waves = c == 8 ? 4 : c == 4 ? 8 : 16;
+        if (waves > cu_waves || L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 30))
+            return false;
+        const size_t lds_limit = 160 * 1024 - 64;
+        const size_t lds2 = gemv16_lds_bytes(c, waves, 2);
+        const int64_t rows = (a.M + 15) / 16;
+        const int64_t per_cu = std::max<int64_t>(1, std::min<int64_t>((int64_t)(160 * 1024 / lds2), cu_waves / waves));
+        const int64_t at_once = std::max<int64_t>(1, (int64_t)n_cus * per_cu / rows);
+        int64_t visits = (L.n_tiles + at_once - 1) / at_once;
+        int64_t grid = (L.n_tiles + visits - 1) / visits;
+        const int grid_env = env_int("OVFCC_GEMV16_GRID", 0);
+        if (grid_env > 0) {
+            grid = std::min<int64_t>(grid_env, L.n_tiles);
+            visits = (L.n_tiles + grid - 1) / grid;
+        }
+        const size_t lds = gemv16_lds_bytes(c, waves, grid < L.n_tiles ? 2 : 1);
+        if (lds > lds_limit)
+            return false;
+        p.gemv16 = true;
+        p.gemv_c = c;
+        p.split_k = 1;
+        p.kblocks_per_split = (int)L.k_blocks;
+        p.tiles_per_group = (int)visits;
+        p.grid[0] = (unsigned)grid;
+        p.grid[1] = (unsigned)rows;
+        p.block = 64u * waves;
+        p.tile_m = 16;
+        p.tile_n = 16;
+        p.dynamic_lds = (unsigned)lds;
+        p.name = "fcc_gemv16_w4";
+        return true;
+    };
     if (kernel == OVFCC_KERNEL_PLAIN) {
         if (a.M > 65535)
             return fail(OVFCC_EUNSUPPORTED, "the plain kernel handles at most 65535 rows");
@@ -161,6 +214,8 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.grid[1] = (unsigned)a.M;
         p.block = 64;
         p.name = "fcc_plain";
+    } else if (kernel == OVFCC_KERNEL_DECODE && plan_gemv16()) {
+        // planned
     } else if (kernel == OVFCC_KERNEL_DECODE && want_batch) {
         if (int rc = plan_batch())
             return rc;
@@ -383,7 +438,10 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     case OVFCC_KERNEL_PLAIN:
         return launch_plain(a, p, stream);
     case OVFCC_KERNEL_DECODE:
-        return p.gemv ? launch_gemv(a, p, stream) : p.batch ? launch_batch(a, p, stream) : launch_decode(a, p, stream);
+        return p.gemv     ? launch_gemv(a, p, stream)
+               : p.gemv16 ? launch_gemv16(a, p, stream)
+               : p.batch  ? launch_batch(a, p, stream)
+                          : launch_decode(a, p, stream);
     default:
         if (p.big)
             return launch_prefill_big(a, p, stream);

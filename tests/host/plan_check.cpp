@@ -15,6 +15,8 @@ int launch_plain(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_decode(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_batch(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_gemv(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int launch_gemv16(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+size_t gemv16_lds_bytes(int c, int waves, int red_bufs) { return (size_t)waves * c * 4096 + (size_t)red_bufs * waves * 1024; }
 int launch_prefill(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_wide(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_direct(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
@@ -107,6 +109,15 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
             CHECK((c == 2 || c == 4 || c == 8) && kb % c == 0 && nw == (kb / c) * per_wg && nw <= 16, "%s c=%d nw=%d", what, c, nw);
             CHECK((int64_t)p.grid[0] * per_wg == L.n_tiles && p.grid[1] == 1 && p.split_k == 1, "%s", what);
             CHECK(p.dynamic_lds == ovfcc::gemv_lds_bytes(c, (int)M, nw) && p.dynamic_lds <= 150 * 1024, "%s lds=%u", what, p.dynamic_lds);
+        } else if (p.gemv16) {
+            const int c = p.gemv_c;
+            CHECK(M > 4 && M <= 32 && L.bits == 4 && L.groups_per_kblock == 1 && L.kblocks_per_group == 1 && !L.glu && c == L.gemv_c, "%s", what);
+            CHECK((c == 2 || c == 4 || c == 8) && kb % c == 0 && nw == kb / c && nw <= (c == 8 ? 4 : c == 4 ? 8 : 16), "%s c=%d nw=%d", what, c, nw);
+            CHECK((int64_t)p.grid[0] <= L.n_tiles && (int64_t)p.grid[0] * rt >= L.n_tiles && (int64_t)p.grid[0] * (rt - 1) < L.n_tiles &&
+                      p.grid[1] == (unsigned)((M + 15) / 16) && p.split_k == 1,
+                  "%s grid=%u visits=%d", what, p.grid[0], rt);
+            CHECK(p.dynamic_lds == ovfcc::gemv16_lds_bytes(c, nw, (int64_t)p.grid[0] < L.n_tiles ? 2 : 1) && p.dynamic_lds <= 160 * 1024 - 64,
+                  "%s lds=%u", what, p.dynamic_lds);
         } else if (p.batch) {
             const int mt = (int)(M + 15) / 16;
             CHECK(p.tile_m == 16 * mt && (rt == 1 || rt == 2), "%s", what);

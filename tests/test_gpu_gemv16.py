@@ -1,0 +1,150 @@
+"""GPU parity of the 16-row decode kernel with stationary activations (five to 32 rows, 4-bit weights, groups of 128
+inputs) against the CPU oracle: every division of K over the waves of a workgroup (2, 4 or 8 k-blocks per wave),
+every row count class (part of a row tile, a whole one, part of the second, both), workgroups that visit one, two
+and many channel tiles, zero-point table / constant / none, bias, both output types, the same bits on every
+repetition, and the node shapes of the benchmark."""
+import sys
+
+import numpy as np
+import pytest
+
+from openvino_amd import datagen, fc
+from parity import check_parity, oracle_y
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = fc.Device(0)
+    yield d
+    d.close()
+
+
+@pytest.fixture()
+def req(dev):
+    r = fc.InferRequest(dev)
+    yield r
+    r.close()
+
+
+# (w_type, zp_type, N, K, k-blocks per wave forced at creation, workgroups per row tile forced (0: policy), bias)
+SHAPES = [
+    ("u4", "u4", 272, 1024, 2, 0, True),     # 4 waves, 17 channel tiles, one visit each
+    ("u4", "u4", 272, 1024, 2, 5, False),    # ... 5 workgroups: four visits for two of them, three for the rest
+    ("u4", "u4", 64, 1024, 4, 2, True),      # 2 waves, two visits each
+    ("i4", "none", 48, 1024, 8, 1, True),    # 1 wave walks all three tiles; symmetric weights (zero-point 8)
+    ("i4", "none", 256, 4096, 4, 0, False),  # 8 waves, 128 KiB of activations through LDS
+    ("u4", "u8", 128, 4096, 2, 0, True),     # 16 waves, 8-bit zero-point table
+    ("u4", "u8", 128, 4096, 2, 3, True),     # ... three workgroups: two buffers of partial sums would be needed
+    ("u4", "none", 64, 2048, 4, 0, True),    # no zero-point at all: the second MFMA chain is skipped
+    ("u4", "u4", 80, 3072, 4, 2, True),      # 6 waves
+    ("u4", "u4", 96, 4096, 8, 4, False),     # 4 waves of 8 k-blocks
+]
+
+
+@pytest.mark.parametrize("wt,zt,N,K,C,grid,bias", SHAPES)
+@pytest.mark.parametrize("out", ["f16", "f32"])
+def test_gemv16_rows_five_to_thirty_two(oracle, dev, req, monkeypatch, wt, zt, N, K, C, grid, bias, out):
+    monkeypatch.setenv("OVFCC_GEMV_C", str(C))
+    if grid:
+        monkeypatch.setenv("OVFCC_GEMV16_GRID", str(grid))
+    c = datagen.make_case(7500 + N + K, 32, K, N, wt, 128, zt, with_bias=bias)
+    w = fc.CompressedWeights.from_case(dev, c, output_type=out)
+    ref = oracle_y(oracle, c)
+    try:
+        for M in (5, 8, 15, 16, 17, 31, 32):
+            say(f"gemv16 {wt}/{zt} N={N} K={K} C={C} grid={grid} out={out} M={M}")
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            if K == 4096 and C == 2 and grid:
+                # 16 waves x 8 KiB of activations leave no room for a second buffer of partial sums
+                assert info["name"] != "fcc_gemv16_w4", info
+                continue
+            assert info["name"] == "fcc_gemv16_w4" and info["block"] == 64 * (K // 128 // C), info
+            assert info["grid"][0] == (grid or N // 16) and info["grid"][1] == (M + 15) // 16, info
+            assert y.dtype == (np.float32 if out == "f32" else np.float16)
+            check_parity(oracle, y, ref[:M], K, f"M={M} {info}", output_rounding_slack=True)
+            for _ in range(3):    # partial sums are added in wave order
+                assert np.array_equal(req.infer(w, c.x[:M]).view(np.uint8), y.view(np.uint8))
+    finally:
+        w.close()
+
+
+def test_gemv16_scalar_zero_point(oracle, dev, req):
+    """One zero-point for the whole node (Shape{}): it travels as a constant, not as a table."""
+    c = datagen.make_case(7601, 12, 2048, 96, "u4", 128, "u8", with_bias=True)
+    zp = np.array([11], dtype=np.uint8)
+    c = datagen.FcCase(c.M, c.K, c.N, c.group_size, c.w_type, "u8", c.w, c.scale, zp, c.x, c.bias, zp_scalar=1)
+    w = fc.CompressedWeights.from_case(dev, c)
+    try:
+        y = req.infer(w, c.x)
+        assert req.last_kernel()["name"] == "fcc_gemv16_w4"
+        check_parity(oracle, y, oracle_y(oracle, c), c.K, "scalar zp", output_rounding_slack=True)
+    finally:
+        w.close()
+
+
+def test_gemv16_tiny_and_huge_activations(oracle, dev, req):
+    """Half of the activations are multiplied by 2^-4 in their registers: values below 2^-10 lose bits there (at most
+    2^-21 absolute each); subnormal activations, activations near the top of the half range and a row of zeros
+    between rows of ordinary values must come out right."""
+    c = datagen.make_case(7700, 8, 1024, 64, "u4", 128, "u4")
+    x = c.x.astype(np.float32)
+    x[0] *= 2.0 ** -12
+    x[1] = np.where(np.arange(c.K) % 3 == 0, 6.0e-8, 0.0)   # the smallest subnormal half
+    x[2] = np.where(np.arange(c.K) % 128 == 5, 60000.0, x[2])  # near the largest half
+    x[3] = 0.0
+    xh = x.astype(np.float16)
+    w = fc.CompressedWeights.from_case(dev, c, output_type="f32")
+    try:
+        y = req.infer(w, xh)
+        assert req.last_kernel()["name"] == "fcc_gemv16_w4"
+        ref = oracle_y(oracle, c, x=xh)
+        assert np.all(y[3] == 0.0)
+        for m in range(8):
+            scale = float(np.max(np.abs(ref[m]))) or 1.0
+            err = float(np.max(np.abs(y[m] - ref[m])))
+            say(f"   row {m}: max |y| {scale:.3e}, max-abs error {err:.3e}")
+            # 1e-3 of the row's own magnitude, plus what 2^-21 per input can add: K/2 inputs * 15 * max scale 0.02
+            assert err <= 1e-3 * scale + 2.0 ** -21 * (c.K / 2) * 15 * 0.02, (m, err, scale)
+    finally:
+        w.close()
+
+
+@pytest.mark.parametrize("name,N,K", [("q/o", 4096, 4096), ("k/v", 1024, 4096), ("gate/up", 14336, 4096)])
+def test_gemv16_benchmark_nodes(oracle, dev, req, name, N, K):
+    """The Llama-3-8B projections whose activations fit in LDS, at the benchmark's row counts, against the oracle on
+    a sample of channels; the down projection (K = 14336) stays with the small-batch kernel."""
+    c = datagen.make_case(7800 + N, 32, K, N, "i4", 128, "none")
+    w = fc.CompressedWeights.from_case(dev, c)
+    rng = np.random.default_rng(5)
+    cols = np.sort(rng.choice(N, size=256, replace=False))
+    ref = oracle_y(oracle, c, n_index=cols)
+    try:
+        for M in (8, 16, 32):
+            say(f"gemv16 {name} M={M}")
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            assert info["name"] == "fcc_gemv16_w4", info
+            check_parity(oracle, y[:, cols], ref[:M], K, f"{name} M={M} {info}")
+    finally:
+        w.close()
+
+
+def test_gemv16_leaves_what_does_not_fit(dev, req):
+    """Activations beyond LDS (K = 14336), groups of 64 inputs, 8-bit weights, a gated linear unit: other kernels."""
+    for wt, zt, N, K, G, glu in (("u4", "none", 64, 14336, 128, None), ("u4", "u4", 64, 1024, 64, None),
+                                 ("u8", "u8", 64, 1024, 128, None), ("u4", "u4", 64, 1024, 128, "swish")):
+        c = datagen.make_case(7900, 8, K, N, wt, G, zt)
+        w = fc.CompressedWeights.from_case(dev, c, glu=glu) if glu else fc.CompressedWeights.from_case(dev, c)
+        try:
+            req.infer(w, c.x)
+            assert req.last_kernel()["name"] != "fcc_gemv16_w4", (wt, zt, N, K, G, glu)
+        finally:
+            w.close()

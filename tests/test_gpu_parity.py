@@ -162,7 +162,7 @@ def test_decode_split_k_is_deterministic(oracle, dev, req, split, M):
         w.close()
 
 
-def test_kernel_policy(dev, req):
+def test_kernel_policy(dev, req, monkeypatch):
     say("policy")
     c = datagen.make_case(3, 130, 256, 128, "u4", 128, "u4")
     w = fc.CompressedWeights.from_case(dev, c)
@@ -171,9 +171,15 @@ def test_kernel_policy(dev, req):
         req.infer(w, c.x[:1])
         assert req.last_kernel()["name"] == "fcc_gemv_w4"    # one to four rows, 4-bit weights, groups of 128
         req.infer(w, c.x[:5])
+        assert req.last_kernel()["name"] == "fcc_gemv16_w4"  # five to 32 rows of such a node, activations fit in LDS
+        req.infer(w, c.x[:32])
+        assert req.last_kernel()["name"] == "fcc_gemv16_w4"
+        monkeypatch.setenv("OVFCC_GEMV16", "0")
+        req.infer(w, c.x[:5])
         assert req.last_kernel()["name"] == "fcc_decode_w4"
         req.infer(w, c.x[:32])
         assert req.last_kernel()["name"] == "fcc_batch_w4"
+        monkeypatch.delenv("OVFCC_GEMV16")
         req.infer(w, c.x[:48])
         assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
         req.infer(w, c.x[:128])          # three launches of the small-batch kernel
