@@ -9,8 +9,8 @@
 // workgroup walks the channel tiles blockIdx.x, blockIdx.x + gridDim.x, ... streaming only weights: three register
 // sets in turn hold the weight tiles and group parameters of this visit and the next two, so two visits' loads
 // travel while one is multiplied, and a visit reads nothing but registers.  The waves' partial sums of a tile meet
-// in LDS behind one barrier per visit and one wave (a different one every visit) adds them in wave order, applies
-// the bias and stores.  Nothing is split along K through memory -- which is what the small-batch kernel
+// in LDS behind one barrier per visit, where four waves add them in wave order (four rows each), apply the bias
+// and store.  Nothing is split along K through memory -- which is what the small-batch kernel
 // (kernel_batch.hip) pays five dependent round trips for -- and the activations travel from L2 once per workgroup,
 // not once per channel tile.  Rows 16-31 are the second workgroup row (blockIdx.y = 1).  The price: 16 rows x K x 2
 // bytes of LDS for the hand-over, so K <= 4096 or so, and registers (16 C for the activations, 4 C for their group
@@ -24,6 +24,8 @@
 // their registers; group scales multiply the f32 sums per k-block.  Zero-points leave through the activations'
 // group sums c = sum_k x_k per row and k-block, which one MFMA chain per k-block against a constant operand
 // leaves in exactly the registers that hold the products' rows:  y = 2^24 sum_kb s_kb (P_kb - zp_kb 2^-24 c_kb).
+#include <type_traits>
+
 #include "device_common.h"
 
 namespace ovfcc {
@@ -54,14 +56,14 @@ struct TileRegs {
 };
 }  // namespace
 
-// C: k-blocks per wave; ZP_TABLE: zero-points per (channel, group)
-template <int C, bool ZP_TABLE>
+// C: k-blocks per wave; ZP_TABLE: zero-points per (channel, group); MULTI: workgroups visit more than one channel tile
+template <int C, bool ZP_TABLE, bool MULTI>
 __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16_kernel(
     const uint4_t* __restrict__ wt, const half_t* __restrict__ scale_cm, const uint8_t* __restrict__ zp_cm,
     const half_t* __restrict__ x, const half_t* __restrict__ bias, void* __restrict__ y, int M, int N, int K,
     int kb_total, int nwt, int n_tiles, int zp_const, int out_f32, int red_bufs) {
     constexpr int kWaveBytes = C * 4096;  // 16 rows x C k-blocks x 256 bytes
-    constexpr int kDepth = 3;             // visits whose weights are in registers or on their way
+    constexpr int kDepth = MULTI ? 3 : 1;  // visits whose weights are in registers or on their way
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [waves] slices | partial sums
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
     typedef __attribute__((address_space(3))) const uint4_t* lds_u4_ptr;
@@ -90,9 +92,11 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
     const __amdgpu_buffer_rsrc_t rb =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(bias), 0, bias ? n_tiles * 32 : 0, kRsrcFlags);
 
-    // ---- one channel tile's parameters and weights; a tile past the end is sent out of range ----
+    // ---- one channel tile's parameters and weights ----
     auto load_tile = [&](int t, TileRegs<C>& r) {
-        const unsigned oob = (unsigned)((n_tiles - 1 - t) >> 31) & kOob;  // no branch
+        // no branch (the compiler counts the loads in flight only along straight code); a load sent out of range
+        // still costs its issue cycles, which is why workgroups with one visit run the kernel without prefetches
+        const unsigned oob = (unsigned)((n_tiles - 1 - t) >> 31) & kOob;
         const unsigned pofs = (unsigned)((t * 16 + col) * kb_total + wave * C);
         if constexpr (C == 8)
             r.sv = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, (pofs * 2u) | oob, 0, 0));
@@ -120,12 +124,12 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
     };
 
     // ---- loads: the first two visits' weights, then the activations: load q of the wave fills units 64 q ..
-    // 64 q + 63 of its slice; rows >= M arrive as zeros.  The wait below is for everything in flight -- the
+    // 64 q + 63 of its slice.  The wait below is for everything in flight -- the
     // compiler cannot see that the LDS reads depend on these loads -- so that it holds wherever the loads whose
     // results the compiler tracks itself end up. ----
     TileRegs<C> ring[kDepth];
 #pragma unroll
-    for (int u = 0; u + 1 < kDepth; ++u)
+    for (int u = 0; u < (MULTI ? kDepth - 1 : 1); ++u)
         load_tile(tile + u * step, ring[u]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -134,9 +138,12 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
         const int row = unit / (16 * C), in_row = unit % (16 * C);
         const int slot = in_row >> 4, chunk = (in_row & 15) ^ row;
         const unsigned ofs = ((unsigned)((m0 + row) * K + (wave + nwt * slot) * 128 + chunk * 8) * 2u) |
-                             ((unsigned)((M - 1 - m0 - row) >> 31) & kOob);  // no branch
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void_ptr)(lds3 + wave * kWaveBytes + q * 1024), 16, ofs, 0, 0,
-                                                 0);
+                             ((unsigned)((M - 1 - m0 - row) >> 31) & kOob);
+        // a load whose rows all lie beyond M is left out (it would cost its issue cycles all the same): those rows
+        // of the slice keep what LDS held, and what is computed from them is never stored
+        if (m0 + (64 * q) / (16 * C) < M)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void_ptr)(lds3 + wave * kWaveBytes + q * 1024), 16, ofs,
+                                                     0, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));
@@ -180,7 +187,7 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
     }
 
     const uint32_t mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u;
-    int reducer = 0, buf = 0;
+    int buf = 0;
 
     // ---- one visit: multiply the channel tile held in `cur`, meet the other waves, store ----
     auto visit = [&](const TileRegs<C>& cur, int t) {
@@ -219,38 +226,41 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
                     acc[q] += scale * (pr[q] + cz[i][q]);
             }
         }
-        // Partial sums of the workgroup's waves meet in LDS; one wave adds them in wave order.  With two buffers in
-        // turn, the barrier of the next visit stands between a buffer's readers and its next writers.
-        const lds_f32_ptr red = (lds_f32_ptr)(lds3 + waves * kWaveBytes + buf * (waves * 1024));  // [wave][16 rows][16]
+        // Partial sums of the workgroup's waves meet in LDS, 16 rows x 16 channels per wave with the 16-float
+        // pieces of a row group rotated by the group (no two lanes of a write or a read share a bank); waves 0-3
+        // add one group of four rows each, in wave order, apply the bias and store.  With two buffers in turn, the
+        // barrier of the next visit stands between a buffer's readers and its next writers.
+        const lds_f32_ptr red = (lds_f32_ptr)(lds3 + waves * kWaveBytes + buf * (waves * 1024));
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-            red[(wave * 16 + 4 * kq + q) * 16 + col] = acc[q];
+            red[wave * 256 + (((4 * kq + q) * 16 + col) ^ (kq << 4))] = acc[q];
         __syncthreads();
-        if (wave == reducer) {
-            const int n = t * 16 + col;
-            const float b = (float)__builtin_bit_cast(half_t, (uint16_t)cur.bias);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int row = m0 + 4 * kq + q;
-                float s = 0.f;
-                for (int w = 0; w < waves; ++w)
-                    s += red[(w * 16 + 4 * kq + q) * 16 + col];
-                if (row < M)
-                    store_out(y, (size_t)row * N + n, s * 0x1p24f + b, out_f32);
-            }
+        for (int g = wave; g < 4; g += waves) {
+            const int at = ((4 * g + kq) * 16 + col) ^ (g << 4);  // this lane: row 4 g + kq of the tile, channel col
+            float s = 0.f;
+#pragma unroll 4
+            for (int w = 0; w < waves; ++w)
+                s += red[w * 256 + at];
+            const int row = m0 + 4 * g + kq;
+            if (row < M)
+                store_out(y, (size_t)row * N + t * 16 + col, s * 0x1p24f + (float)__builtin_bit_cast(half_t, (uint16_t)cur.bias),
+                          out_f32);
         }
-        reducer = reducer + 1 == waves ? 0 : reducer + 1;
         buf = buf + 1 == red_bufs ? 0 : buf + 1;
     };
 
-    // ---- kDepth register sets in turn: the set multiplied last is refilled for the visit kDepth - 1 from now ----
-    while (true) {
+    if constexpr (!MULTI) {
+        visit(ring[0], tile);
+    } else {
+        // kDepth register sets in turn: the set multiplied last is refilled for the visit kDepth - 1 from now
+        while (true) {
 #pragma unroll
-        for (int u = 0; u < kDepth; ++u) {
-            load_tile(tile + (kDepth - 1) * step, ring[(u + kDepth - 1) % kDepth]);
-            visit(ring[u], tile);
-            if ((tile += step) >= n_tiles)
-                return;
+            for (int u = 0; u < kDepth; ++u) {
+                load_tile(tile + (kDepth - 1) * step, ring[(u + kDepth - 1) % kDepth]);
+                visit(ring[u], tile);
+                if ((tile += step) >= n_tiles)
+                    return;
+            }
         }
     }
 }
@@ -260,10 +270,10 @@ size_t gemv16_lds_bytes(int c, int waves, int red_bufs) {
     return (size_t)waves * c * 4096 + (size_t)red_bufs * waves * 1024;
 }
 
-template <int C, bool ZPT>
+template <int C, bool ZPT, bool MULTI>
 static int launch_gemv16_impl(const FcDeviceArgs& a, const LaunchPlan& p, int red_bufs, hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_gemv16_kernel<C, ZPT>;
+    auto kern = fcc_gemv16_kernel<C, ZPT, MULTI>;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -298,13 +308,16 @@ int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
         a.M * a.K * 2 >= ((int64_t)1 << 31) || (L.n_tiles + p.grid[0]) * L.k_blocks * kTileBytes >= ((int64_t)1 << 32) ||
         L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 31))
         return (int)hipErrorInvalidValue;
+    const bool multi = red_bufs == 2;
+    auto go = [&](auto zpt, auto mul) {
+        constexpr bool Z = decltype(zpt)::value, U = decltype(mul)::value;
+        return c == 8   ? launch_gemv16_impl<8, Z, U>(a, p, red_bufs, s)
+               : c == 4 ? launch_gemv16_impl<4, Z, U>(a, p, red_bufs, s)
+                        : launch_gemv16_impl<2, Z, U>(a, p, red_bufs, s);
+    };
     if (L.zp_table)
-        return c == 8   ? launch_gemv16_impl<8, true>(a, p, red_bufs, s)
-               : c == 4 ? launch_gemv16_impl<4, true>(a, p, red_bufs, s)
-                        : launch_gemv16_impl<2, true>(a, p, red_bufs, s);
-    return c == 8   ? launch_gemv16_impl<8, false>(a, p, red_bufs, s)
-           : c == 4 ? launch_gemv16_impl<4, false>(a, p, red_bufs, s)
-                    : launch_gemv16_impl<2, false>(a, p, red_bufs, s);
+        return multi ? go(std::true_type{}, std::true_type{}) : go(std::true_type{}, std::false_type{});
+    return multi ? go(std::false_type{}, std::true_type{}) : go(std::false_type{}, std::false_type{});
 }
 
 }  // namespace ovfcc
