@@ -14,7 +14,10 @@
 // (kernel_batch.hip) pays five dependent round trips for -- and the activations travel from L2 once per workgroup,
 // not once per channel tile.  Rows 16-31 are the second workgroup row (blockIdx.y = 1).  The price: 16 rows x K x 2
 // bytes of LDS for the hand-over, so K <= 4096 or so, and registers (16 C for the activations, 4 C for their group
-// sums, 3 (4 C + 4) for the weights), which bound the workgroup at 4, 8 and 16 waves for C = 8, 4 and 2.
+// sums, 3 (4 C + 4) for the weights), which bound the workgroup at 8 and 16 waves for C = 4 and 2.  A node whose
+// channel-major tables were laid out for eight k-blocks per wave runs with two waves per table row, four k-blocks
+// each.  With a gated linear unit a workgroup visits the gate tile and the up tile of 16 channels in turn; the
+// waves that add the sums keep the gate values in a register for the visit between.
 //
 // LDS slice of a wave, in 16-byte units: row r, slot s (k-block w + NWT s), chunk c of the k-block's 16 sits at
 // r (16 C) + 16 s + (c ^ r): the sixteen rows that one operand read touches lie in sixteen different bank groups.
@@ -41,28 +44,28 @@ template <>
 struct Vec16Of<4> {
     typedef uint2_t type;
 };
-template <>
-struct Vec16Of<8> {
-    typedef uint4_t type;
-};
 
 // group parameters and weight tiles of one channel tile, as one wave holds them
 template <int C>
 struct TileRegs {
     typename Vec16Of<C>::type sv;  // C scales (f16) of channel col
-    uint32_t zv[2];                // C zero-points (u8) of channel col
+    uint32_t zv;                   // C zero-points (u8) of channel col
     uint32_t bias;                 // bias (f16) of channel col; 0 without one
     uint4_t wv[C];                 // the wave's C weight tiles
 };
 }  // namespace
 
-// C: k-blocks per wave; ZP_TABLE: zero-points per (channel, group); MULTI: workgroups visit more than one channel tile
-template <int C, bool ZP_TABLE, bool MULTI>
-__global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16_kernel(
+// C: k-blocks per wave (the node's channel-major tables may be laid out for 2 C: then two waves share a table
+// row, `parts` = k_blocks / c_table of them side by side, and a wave takes half of its slots); ZP_TABLE: zero-points
+// per (channel, group); MULTI: workgroups visit more than one channel tile; GLU: tiles 2 j and 2 j + 1 hold the gate
+// and up channels 16 j .. of a gated linear unit and a workgroup visits them one after the other
+template <int C, bool ZP_TABLE, bool MULTI, bool GLU>
+__global__ __launch_bounds__(C == 4 ? 512 : 1024) void fcc_gemv16_kernel(
     const uint4_t* __restrict__ wt, const half_t* __restrict__ scale_cm, const uint8_t* __restrict__ zp_cm,
     const half_t* __restrict__ x, const half_t* __restrict__ bias, void* __restrict__ y, int M, int N, int K,
-    int kb_total, int nwt, int n_tiles, int zp_const, int out_f32, int red_bufs) {
-    constexpr int kWaveBytes = C * 4096;  // 16 rows x C k-blocks x 256 bytes
+    int kb_total, int parts, int c_table, int n_tiles, int zp_const, int out_f32, int red_bufs, int glu) {
+    static_assert(!GLU || MULTI, "a gated linear unit takes two visits");
+    constexpr int kWaveBytes = C * 4096;   // 16 rows x C k-blocks x 256 bytes
     constexpr int kDepth = MULTI ? 3 : 1;  // visits whose weights are in registers or on their way
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [waves] slices | partial sums
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
@@ -71,12 +74,16 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int waves = blockDim.x >> 6;  // = nwt
+    const int waves = blockDim.x >> 6;  // parts * c_table / C
+    const int part = wave % parts;      // the table row this wave reads: k-blocks part, part + parts, ...
+    const int slot0 = wave / parts * C; // ... of which it takes slots slot0 .. slot0 + C - 1
     const int col = lane & 15;
     const int kq = lane >> 4;
     const int m0 = 16 * blockIdx.y;
-    const int step = gridDim.x;
-    int tile = blockIdx.x;
+    // visit v of this workgroup
+    auto tile_of = [&](int v) {
+        return GLU ? 2 * ((int)blockIdx.x + (v >> 1) * (int)gridDim.x) + (v & 1) : (int)blockIdx.x + v * (int)gridDim.x;
+    };
 
     constexpr unsigned kOob = 0x80000000u;
     constexpr int kRsrcFlags = 0x00020000;
@@ -88,7 +95,7 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
                                                                         n_tiles * 16 * kb_total * 2, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rz = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint8_t*>(zp_cm), 0, ZP_TABLE ? n_tiles * 16 * kb_total : 0, kRsrcFlags);
-    // fetched with the weights, so that the wave that stores never waits for a load younger than its prefetches
+    // fetched with the weights, so that the waves that store never wait for a load younger than their prefetches
     const __amdgpu_buffer_rsrc_t rb =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(bias), 0, bias ? n_tiles * 32 : 0, kRsrcFlags);
 
@@ -97,47 +104,41 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
         // no branch (the compiler counts the loads in flight only along straight code); a load sent out of range
         // still costs its issue cycles, which is why workgroups with one visit run the kernel without prefetches
         const unsigned oob = (unsigned)((n_tiles - 1 - t) >> 31) & kOob;
-        const unsigned pofs = (unsigned)((t * 16 + col) * kb_total + wave * C);
-        if constexpr (C == 8)
-            r.sv = __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rs, (pofs * 2u) | oob, 0, 0));
-        else if constexpr (C == 4)
+        const unsigned pofs = (unsigned)((t * 16 + col) * kb_total + part * c_table + slot0);
+        if constexpr (C == 4)
             r.sv = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(rs, (pofs * 2u) | oob, 0, 0));
         else
             r.sv = __builtin_amdgcn_raw_buffer_load_b32(rs, (pofs * 2u) | oob, 0, 0);
         r.bias = __builtin_amdgcn_raw_buffer_load_b16(rb, (unsigned)((t * 16 + col) * 2) | oob, 0, 0);
-        r.zv[0] = r.zv[1] = 0u;
+        r.zv = 0u;
         if constexpr (ZP_TABLE) {
-            if constexpr (C == 8) {
-                const uint2_t v = __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(rz, pofs | oob, 0, 0));
-                r.zv[0] = v.x, r.zv[1] = v.y;
-            } else if constexpr (C == 4) {
-                r.zv[0] = __builtin_amdgcn_raw_buffer_load_b32(rz, pofs | oob, 0, 0);
-            } else {
-                r.zv[0] = __builtin_amdgcn_raw_buffer_load_b16(rz, pofs | oob, 0, 0);
-            }
+            if constexpr (C == 4)
+                r.zv = __builtin_amdgcn_raw_buffer_load_b32(rz, pofs | oob, 0, 0);
+            else
+                r.zv = __builtin_amdgcn_raw_buffer_load_b16(rz, pofs | oob, 0, 0);
         }
-        const unsigned wofs = (unsigned)(t * kb_total + wave) * kTileBytes + lane * 16;
+        const unsigned wofs = (unsigned)(t * kb_total + part + parts * slot0) * kTileBytes + lane * 16;
 #pragma unroll
         for (int i = 0; i < C; ++i)
             r.wv[i] = __builtin_bit_cast(
-                uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rw, (wofs + (unsigned)(i * nwt) * kTileBytes) | oob, 0, 2));
+                uint4_t, __builtin_amdgcn_raw_buffer_load_b128(rw, (wofs + (unsigned)(i * parts) * kTileBytes) | oob, 0, 2));
     };
 
     // ---- loads: the first two visits' weights, then the activations: load q of the wave fills units 64 q ..
-    // 64 q + 63 of its slice.  The wait below is for everything in flight -- the
-    // compiler cannot see that the LDS reads depend on these loads -- so that it holds wherever the loads whose
-    // results the compiler tracks itself end up. ----
+    // 64 q + 63 of its slice.  The wait below is for everything in flight -- the compiler cannot see that the LDS
+    // reads depend on these loads -- so that it holds wherever the loads whose results the compiler tracks itself
+    // end up. ----
     TileRegs<C> ring[kDepth];
 #pragma unroll
     for (int u = 0; u < (MULTI ? kDepth - 1 : 1); ++u)
-        load_tile(tile + u * step, ring[u]);
+        load_tile(tile_of(u), ring[u]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int q = 0; q < 4 * C; ++q) {
         const int unit = 64 * q + lane;
         const int row = unit / (16 * C), in_row = unit % (16 * C);
         const int slot = in_row >> 4, chunk = (in_row & 15) ^ row;
-        const unsigned ofs = ((unsigned)((m0 + row) * K + (wave + nwt * slot) * 128 + chunk * 8) * 2u) |
+        const unsigned ofs = ((unsigned)((m0 + row) * K + (part + parts * (slot0 + slot)) * 128 + chunk * 8) * 2u) |
                              ((unsigned)((M - 1 - m0 - row) >> 31) & kOob);
         // a load whose rows all lie beyond M is left out (it would cost its issue cycles all the same): those rows
         // of the slice keep what LDS held, and what is computed from them is never stored
@@ -188,6 +189,7 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
 
     const uint32_t mask_lo = 0x000F000Fu, mask_hi = 0x00F000F0u;
     int buf = 0;
+    float gate[4] = {0.f, 0.f, 0.f, 0.f};  // gated linear unit: what the gate tile's visit left for the up tile's
 
     // ---- one visit: multiply the channel tile held in `cur`, meet the other waves, store ----
     auto visit = [&](const TileRegs<C>& cur, int t) {
@@ -207,16 +209,14 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
                 p = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[i][j].v, b.v, p, 0, 0, 0);
             }
             uint32_t sbits;
-            if constexpr (C == 8)
-                sbits = (i < 2 ? cur.sv.x : i < 4 ? cur.sv.y : i < 6 ? cur.sv.z : cur.sv.w) >> (16 * (i & 1));
-            else if constexpr (C == 4)
+            if constexpr (C == 4)
                 sbits = (i < 2 ? cur.sv.x : cur.sv.y) >> (16 * (i & 1));
             else
                 sbits = cur.sv >> (16 * (i & 1));
             const float scale = (float)__builtin_bit_cast(half_t, (uint16_t)sbits);
             const float pr[4] = {p.x, p.y, p.z, p.w};
             if constexpr (ZP_TABLE) {
-                const float zpf = (float)((cur.zv[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+                const float zpf = (float)((cur.zv >> (8 * i)) & 0xFFu);
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
                     acc[q] += scale * (pr[q] - zpf * cz[i][q]);
@@ -235,30 +235,43 @@ __global__ __launch_bounds__(C == 8 ? 256 : C == 4 ? 512 : 1024) void fcc_gemv16
         for (int q = 0; q < 4; ++q)
             red[wave * 256 + (((4 * kq + q) * 16 + col) ^ (kq << 4))] = acc[q];
         __syncthreads();
-        for (int g = wave; g < 4; g += waves) {
-            const int at = ((4 * g + kq) * 16 + col) ^ (g << 4);  // this lane: row 4 g + kq of the tile, channel col
-            float s = 0.f;
+#pragma unroll
+        for (int gi = 0; gi < 4; ++gi) {
+            const int g = wave + gi * waves;  // wave-uniform
+            if (g < 4) {
+                const int at = ((4 * g + kq) * 16 + col) ^ (g << 4);  // this lane: row 4 g + kq of the tile, channel col
+                float s = 0.f;
 #pragma unroll 4
-            for (int w = 0; w < waves; ++w)
-                s += red[w * 256 + at];
-            const int row = m0 + 4 * g + kq;
-            if (row < M)
-                store_out(y, (size_t)row * N + t * 16 + col, s * 0x1p24f + (float)__builtin_bit_cast(half_t, (uint16_t)cur.bias),
-                          out_f32);
+                for (int w = 0; w < waves; ++w)
+                    s += red[w * 256 + at];
+                s = s * 0x1p24f + (float)__builtin_bit_cast(half_t, (uint16_t)cur.bias);
+                const int row = m0 + 4 * g + kq;
+                if constexpr (GLU) {
+                    if (t & 1) {
+                        if (row < M)
+                            store_out(y, (size_t)row * (N / 2) + (t >> 1) * 16 + col, glu_value(glu, gate[gi], s), out_f32);
+                    } else {
+                        gate[gi] = s;
+                    }
+                } else {
+                    if (row < M)
+                        store_out(y, (size_t)row * N + t * 16 + col, s, out_f32);
+                }
+            }
         }
         buf = buf + 1 == red_bufs ? 0 : buf + 1;
     };
 
     if constexpr (!MULTI) {
-        visit(ring[0], tile);
+        visit(ring[0], tile_of(0));
     } else {
         // kDepth register sets in turn: the set multiplied last is refilled for the visit kDepth - 1 from now
-        while (true) {
+        for (int v = 0;; v += kDepth) {
 #pragma unroll
             for (int u = 0; u < kDepth; ++u) {
-                load_tile(tile + (kDepth - 1) * step, ring[(u + kDepth - 1) % kDepth]);
-                visit(ring[u], tile);
-                if ((tile += step) >= n_tiles)
+                load_tile(tile_of(v + u + kDepth - 1), ring[(u + kDepth - 1) % kDepth]);
+                visit(ring[u], tile_of(v + u));
+                if (tile_of(v + u + 1) >= n_tiles)
                     return;
             }
         }
@@ -270,10 +283,15 @@ size_t gemv16_lds_bytes(int c, int waves, int red_bufs) {
     return (size_t)waves * c * 4096 + (size_t)red_bufs * waves * 1024;
 }
 
-template <int C, bool ZPT, bool MULTI>
+// k-blocks per wave that the kernel runs a node with: tables laid out for eight are read by two waves per row
+int gemv16_kblocks_per_wave(int c_table) {
+    return c_table == 2 ? 2 : 4;
+}
+
+template <int C, bool ZPT, bool MULTI, bool GLU>
 static int launch_gemv16_impl(const FcDeviceArgs& a, const LaunchPlan& p, int red_bufs, hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_gemv16_kernel<C, ZPT, MULTI>;
+    auto kern = fcc_gemv16_kernel<C, ZPT, MULTI, GLU>;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -284,40 +302,43 @@ static int launch_gemv16_impl(const FcDeviceArgs& a, const LaunchPlan& p, int re
     }
     hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], 1), dim3(p.block), p.dynamic_lds, s, (const uint4_t*)a.w,
                        (const half_t*)a.scale_cm, (const uint8_t*)a.zp_cm, (const half_t*)a.x, (const half_t*)a.bias,
-                       a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)(L.k_blocks / C), (int)L.n_tiles,
-                       L.zp_const, a.out_f32, red_bufs);
+                       a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)(L.k_blocks / L.gemv_c), L.gemv_c,
+                       (int)L.n_tiles, L.zp_const, a.out_f32, red_bufs, L.glu);
     return (int)hipGetLastError();
 }
 
 int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
-    const int c = L.gemv_c;
+    const int ct = L.gemv_c;
     // what the kernel and its grid assume, checked against the operands before anything is launched
-    if (!L.tiled || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 || L.glu || !a.scale_cm ||
-        (L.zp_table && !a.zp_cm) || a.M < 1 || a.M > 32 || (c != 2 && c != 4 && c != 8) || L.k_blocks % c != 0 ||
-        p.gemv_c != c || (!L.zp_table && (L.zp_const < 0 || L.zp_const > 255)))
+    if (!L.tiled || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 || !a.scale_cm ||
+        (L.zp_table && !a.zp_cm) || a.M < 1 || a.M > 32 || (ct != 2 && ct != 4 && ct != 8) || L.k_blocks % ct != 0 ||
+        p.gemv_c != ct || (!L.zp_table && (L.zp_const < 0 || L.zp_const > 255)) || (L.glu && (L.n_tiles & 1)))
         return (int)hipErrorInvalidValue;
-    const int nwt = (int)(L.k_blocks / c);
-    const int max_waves = c == 8 ? 4 : c == 4 ? 8 : 16;
-    if (nwt < 1 || nwt > max_waves || p.block != 64u * nwt || p.grid[0] < 1 || (int64_t)p.grid[0] > L.n_tiles ||
+    const int c = gemv16_kblocks_per_wave(ct);
+    const int waves = (int)(L.k_blocks / c);
+    const int64_t units = L.glu ? L.n_tiles / 2 : L.n_tiles;  // what a workgroup visits in one go: tiles or tile pairs
+    if (waves < 1 || waves > (c == 4 ? 8 : 16) || p.block != 64u * waves || p.grid[0] < 1 || (int64_t)p.grid[0] > units ||
         p.grid[1] != (unsigned)((a.M + 15) / 16) || p.grid[2] != 1)
         return (int)hipErrorInvalidValue;
-    const int red_bufs = (int64_t)p.grid[0] < L.n_tiles ? 2 : 1;
-    if (p.dynamic_lds != gemv16_lds_bytes(c, nwt, red_bufs) || p.dynamic_lds > 160 * 1024 - 64 ||
-        a.M * a.K * 2 >= ((int64_t)1 << 31) || (L.n_tiles + p.grid[0]) * L.k_blocks * kTileBytes >= ((int64_t)1 << 32) ||
+    const int red_bufs = (L.glu || (int64_t)p.grid[0] < units) ? 2 : 1;
+    if (p.dynamic_lds != gemv16_lds_bytes(c, waves, red_bufs) || p.dynamic_lds > 160 * 1024 - 64 ||
+        a.M * a.K * 2 >= ((int64_t)1 << 31) || (L.n_tiles + 2 * (int64_t)p.grid[0]) * L.k_blocks * kTileBytes >= ((int64_t)1 << 32) ||
         L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 31))
         return (int)hipErrorInvalidValue;
     const bool multi = red_bufs == 2;
-    auto go = [&](auto zpt, auto mul) {
-        constexpr bool Z = decltype(zpt)::value, U = decltype(mul)::value;
-        return c == 8   ? launch_gemv16_impl<8, Z, U>(a, p, red_bufs, s)
-               : c == 4 ? launch_gemv16_impl<4, Z, U>(a, p, red_bufs, s)
-                        : launch_gemv16_impl<2, Z, U>(a, p, red_bufs, s);
+    auto go = [&](auto zpt, auto mul, auto gl) {
+        constexpr bool Z = decltype(zpt)::value, U = decltype(mul)::value, G = decltype(gl)::value;
+        return c == 4 ? launch_gemv16_impl<4, Z, U, G>(a, p, red_bufs, s) : launch_gemv16_impl<2, Z, U, G>(a, p, red_bufs, s);
     };
+    const std::true_type yes{};
+    const std::false_type no{};
+    if (L.glu)
+        return L.zp_table ? go(yes, yes, yes) : go(no, yes, yes);
     if (L.zp_table)
-        return multi ? go(std::true_type{}, std::true_type{}) : go(std::true_type{}, std::false_type{});
-    return multi ? go(std::false_type{}, std::true_type{}) : go(std::false_type{}, std::false_type{});
+        return multi ? go(yes, yes, no) : go(yes, no, no);
+    return multi ? go(no, yes, no) : go(no, no, no);
 }
 
 }  // namespace ovfcc

@@ -170,34 +170,35 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
     // holds at once, rounded so that all of them visit the same number of tiles.
     auto plan_gemv16 = [&]() -> bool {
         if (a.M <= 4 || a.M > 32 || !a.scale_cm || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 ||
-            L.glu || force_split > 0 || L.gemv_c == 0 || env_int("OVFCC_GEMV16", 1) == 0 ||
+            force_split > 0 || L.gemv_c == 0 || (L.glu && (L.n_tiles & 1)) || env_int("OVFCC_GEMV16", 1) == 0 ||
             env_int("OVFCC_DECODE_BATCH", -1) >= 0)
             return false;
-        const int c = L.gemv_c, waves = (int)(L.k_blocks / c);
-        // the kernel's registers allow 4, 8 and 16 waves per compute unit with 8, 4 and 2 k-blocks per wave
-        const int cu_waves = c == 8 ? 4 : c == 4 ? 8 : 16;
+        // the kernel's registers allow 8 and 16 waves per compute unit with 4 and 2 k-blocks per wave
+        const int c = gemv16_kblocks_per_wave(L.gemv_c), waves = (int)(L.k_blocks / c);
+        const int cu_waves = c == 4 ? 8 : 16;
         if (waves > cu_waves || L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 30))
             return false;
         const size_t lds_limit = 160 * 1024 - 64;
         const size_t lds2 = gemv16_lds_bytes(c, waves, 2);
         const int64_t rows = (a.M + 15) / 16;
+        const int64_t units = L.glu ? L.n_tiles / 2 : L.n_tiles;  // visited in one go: tiles, or pairs of gate and up tile
         const int64_t per_cu = std::max<int64_t>(1, std::min<int64_t>((int64_t)(160 * 1024 / lds2), cu_waves / waves));
         const int64_t at_once = std::max<int64_t>(1, (int64_t)n_cus * per_cu / rows);
-        int64_t visits = (L.n_tiles + at_once - 1) / at_once;
-        int64_t grid = (L.n_tiles + visits - 1) / visits;
+        int64_t visits = (units + at_once - 1) / at_once;
+        int64_t grid = (units + visits - 1) / visits;
         const int grid_env = env_int("OVFCC_GEMV16_GRID", 0);
         if (grid_env > 0) {
-            grid = std::min<int64_t>(grid_env, L.n_tiles);
-            visits = (L.n_tiles + grid - 1) / grid;
+            grid = std::min<int64_t>(grid_env, units);
+            visits = (units + grid - 1) / grid;
         }
-        const size_t lds = gemv16_lds_bytes(c, waves, grid < L.n_tiles ? 2 : 1);
+        const size_t lds = gemv16_lds_bytes(c, waves, (L.glu || grid < units) ? 2 : 1);
         if (lds > lds_limit)
             return false;
         p.gemv16 = true;
-        p.gemv_c = c;
+        p.gemv_c = L.gemv_c;
         p.split_k = 1;
         p.kblocks_per_split = (int)L.k_blocks;
-        p.tiles_per_group = (int)visits;
+        p.tiles_per_group = (int)(visits * (L.glu ? 2 : 1));
         p.grid[0] = (unsigned)grid;
         p.grid[1] = (unsigned)rows;
         p.block = 64u * waves;

@@ -16,6 +16,7 @@ int launch_decode(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_batch(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_gemv(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_gemv16(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
+int gemv16_kblocks_per_wave(int c_table) { return c_table == 2 ? 2 : 4; }
 size_t gemv16_lds_bytes(int c, int waves, int red_bufs) { return (size_t)waves * c * 4096 + (size_t)red_bufs * waves * 1024; }
 int launch_prefill(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_wide(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
@@ -110,13 +111,18 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
             CHECK((int64_t)p.grid[0] * per_wg == L.n_tiles && p.grid[1] == 1 && p.split_k == 1, "%s", what);
             CHECK(p.dynamic_lds == ovfcc::gemv_lds_bytes(c, (int)M, nw) && p.dynamic_lds <= 150 * 1024, "%s lds=%u", what, p.dynamic_lds);
         } else if (p.gemv16) {
-            const int c = p.gemv_c;
-            CHECK(M > 4 && M <= 32 && L.bits == 4 && L.groups_per_kblock == 1 && L.kblocks_per_group == 1 && !L.glu && c == L.gemv_c, "%s", what);
-            CHECK((c == 2 || c == 4 || c == 8) && kb % c == 0 && nw == kb / c && nw <= (c == 8 ? 4 : c == 4 ? 8 : 16), "%s c=%d nw=%d", what, c, nw);
-            CHECK((int64_t)p.grid[0] <= L.n_tiles && (int64_t)p.grid[0] * rt >= L.n_tiles && (int64_t)p.grid[0] * (rt - 1) < L.n_tiles &&
-                      p.grid[1] == (unsigned)((M + 15) / 16) && p.split_k == 1,
+            const int c = ovfcc::gemv16_kblocks_per_wave(p.gemv_c);
+            const int64_t units = L.glu ? L.n_tiles / 2 : L.n_tiles;
+            const int per_unit = L.glu ? 2 : 1;
+            CHECK(M > 4 && M <= 32 && L.bits == 4 && L.groups_per_kblock == 1 && L.kblocks_per_group == 1 && p.gemv_c == L.gemv_c &&
+                      (!L.glu || L.n_tiles % 2 == 0),
+                  "%s", what);
+            CHECK(kb % c == 0 && nw == kb / c && nw <= (c == 4 ? 8 : 16), "%s c=%d nw=%d", what, c, nw);
+            CHECK(rt % per_unit == 0 && (int64_t)p.grid[0] <= units && (int64_t)p.grid[0] * (rt / per_unit) >= units &&
+                      (int64_t)p.grid[0] * (rt / per_unit - 1) < units && p.grid[1] == (unsigned)((M + 15) / 16) && p.split_k == 1,
                   "%s grid=%u visits=%d", what, p.grid[0], rt);
-            CHECK(p.dynamic_lds == ovfcc::gemv16_lds_bytes(c, nw, (int64_t)p.grid[0] < L.n_tiles ? 2 : 1) && p.dynamic_lds <= 160 * 1024 - 64,
+            CHECK(p.dynamic_lds == ovfcc::gemv16_lds_bytes(c, nw, (L.glu || (int64_t)p.grid[0] < units) ? 2 : 1) &&
+                      p.dynamic_lds <= 160 * 1024 - 64,
                   "%s lds=%u", what, p.dynamic_lds);
         } else if (p.batch) {
             const int mt = (int)(M + 15) / 16;

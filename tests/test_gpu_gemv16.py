@@ -2,14 +2,14 @@
 inputs) against the CPU oracle: every division of K over the waves of a workgroup (2, 4 or 8 k-blocks per wave),
 every row count class (part of a row tile, a whole one, part of the second, both), workgroups that visit one, two
 and many channel tiles, zero-point table / constant / none, bias, both output types, the same bits on every
-repetition, and the node shapes of the benchmark."""
+repetition, the gated linear unit, and the node shapes of the benchmark."""
 import sys
 
 import numpy as np
 import pytest
 
 from openvino_amd import datagen, fc
-from parity import check_parity, oracle_y
+from parity import check_parity, glu_reference, oracle_y
 
 pytestmark = pytest.mark.gpu
 
@@ -38,13 +38,14 @@ SHAPES = [
     ("u4", "u4", 272, 1024, 2, 0, True),     # 4 waves, 17 channel tiles, one visit each
     ("u4", "u4", 272, 1024, 2, 5, False),    # ... 5 workgroups: four visits for two of them, three for the rest
     ("u4", "u4", 64, 1024, 4, 2, True),      # 2 waves, two visits each
-    ("i4", "none", 48, 1024, 8, 1, True),    # 1 wave walks all three tiles; symmetric weights (zero-point 8)
+    ("i4", "none", 48, 1024, 8, 1, True),    # 2 waves walk all three tiles; symmetric weights (zero-point 8)
     ("i4", "none", 256, 4096, 4, 0, False),  # 8 waves, 128 KiB of activations through LDS
     ("u4", "u8", 128, 4096, 2, 0, True),     # 16 waves, 8-bit zero-point table
     ("u4", "u8", 128, 4096, 2, 3, True),     # ... three workgroups: two buffers of partial sums would be needed
     ("u4", "none", 64, 2048, 4, 0, True),    # no zero-point at all: the second MFMA chain is skipped
     ("u4", "u4", 80, 3072, 4, 2, True),      # 6 waves
-    ("u4", "u4", 96, 4096, 8, 4, False),     # 4 waves of 8 k-blocks
+    ("u4", "u4", 96, 4096, 8, 4, False),     # tables for 4 waves of 8 k-blocks: 8 waves of 4
+    ("u4", "none", 32, 256, 2, 0, True),     # 1 wave adds all four row groups itself
 ]
 
 
@@ -66,7 +67,8 @@ def test_gemv16_rows_five_to_thirty_two(oracle, dev, req, monkeypatch, wt, zt, N
                 # 16 waves x 8 KiB of activations leave no room for a second buffer of partial sums
                 assert info["name"] != "fcc_gemv16_w4", info
                 continue
-            assert info["name"] == "fcc_gemv16_w4" and info["block"] == 64 * (K // 128 // C), info
+            # tables laid out for eight k-blocks per wave are read by two waves per row, four k-blocks each
+            assert info["name"] == "fcc_gemv16_w4" and info["block"] == 64 * (K // 128 // min(C, 4)), info
             assert info["grid"][0] == (grid or N // 16) and info["grid"][1] == (M + 15) // 16, info
             assert y.dtype == (np.float32 if out == "f32" else np.float16)
             check_parity(oracle, y, ref[:M], K, f"M={M} {info}", output_rounding_slack=True)
@@ -137,14 +139,39 @@ def test_gemv16_benchmark_nodes(oracle, dev, req, name, N, K):
         w.close()
 
 
+@pytest.mark.parametrize("wt,zt,N,K,C,grid,kind,second", [("u4", "u4", 512, 1024, 2, 0, "swish", False),
+                                                         ("i4", "none", 256, 2048, 4, 3, "gelu", True),
+                                                         ("i4", "none", 128, 4096, 8, 0, "gelu_tanh", False),
+                                                         ("u4", "u4", 64, 4096, 4, 1, "swish", True)])
+def test_gemv16_gated_linear_unit(oracle, dev, req, monkeypatch, wt, zt, N, K, C, grid, kind, second):
+    """Gate and up tile of 16 channels are two visits of one workgroup; the gate values wait in registers."""
+    monkeypatch.setenv("OVFCC_GEMV_C", str(C))
+    if grid:
+        monkeypatch.setenv("OVFCC_GEMV16_GRID", str(grid))
+    c = datagen.make_case(7950 + N, 32, K, N, wt, 128, zt, with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c, glu=kind, glu_gate_second=second)
+    try:
+        for M in (5, 16, 17, 32):
+            say(f"gemv16 glu {kind} {wt}/{zt} N={N} K={K} C={C} grid={grid} M={M}")
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            assert info["name"] == "fcc_gemv16_w4" and info["block"] == 64 * (K // 128 // min(C, 4)), info
+            assert info["grid"][0] == (grid or N // 32) and info["grid"][1] == (M + 15) // 16, info
+            assert y.shape == (M, N // 2)
+            ref, amp = glu_reference(oracle, c, kind, second, x=c.x[:M])
+            check_parity(oracle, y, ref, K, f"M={M} {info}", output_rounding_slack=True, limit_scale=amp)
+            assert np.array_equal(req.infer(w, c.x[:M]).view(np.uint8), y.view(np.uint8))
+    finally:
+        w.close()
+
+
 def test_gemv16_leaves_what_does_not_fit(dev, req):
-    """Activations beyond LDS (K = 14336), groups of 64 inputs, 8-bit weights, a gated linear unit: other kernels."""
-    for wt, zt, N, K, G, glu in (("u4", "none", 64, 14336, 128, None), ("u4", "u4", 64, 1024, 64, None),
-                                 ("u8", "u8", 64, 1024, 128, None), ("u4", "u4", 64, 1024, 128, "swish")):
+    """Activations beyond LDS (K = 14336), groups of 64 inputs, 8-bit weights: other kernels."""
+    for wt, zt, N, K, G in (("u4", "none", 64, 14336, 128), ("u4", "u4", 64, 1024, 64), ("u8", "u8", 64, 1024, 128)):
         c = datagen.make_case(7900, 8, K, N, wt, G, zt)
-        w = fc.CompressedWeights.from_case(dev, c, glu=glu) if glu else fc.CompressedWeights.from_case(dev, c)
+        w = fc.CompressedWeights.from_case(dev, c)
         try:
             req.infer(w, c.x)
-            assert req.last_kernel()["name"] != "fcc_gemv16_w4", (wt, zt, N, K, G, glu)
+            assert req.last_kernel()["name"] != "fcc_gemv16_w4", (wt, zt, N, K, G)
         finally:
             w.close()
