@@ -401,6 +401,8 @@ def main() -> int:
     ap.add_argument("--profile", choices=["decode", "batch", "prefill", "w8a8", "w4a8"], default=None,
                     help="short run for rocprofv3: one copy-kernel launch of known size (the counter yardstick), "
                          "then a few eager passes of the chosen kernel family; prints no JSON")
+    ap.add_argument("--profile-rows", type=int, default=32,
+                    help="row count of --profile batch (2..32; default: config 2's largest)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build measures one GPU only (the path has no collectives); run with --gpus 1")
@@ -476,7 +478,7 @@ def main() -> int:
                     dev.free(xq_dev)
                     dev.free(yq_dev)
         elif args.profile in ("decode", "batch"):
-            rows = 1 if args.profile == "decode" else 32     # small-batch decode: config 2's largest row count
+            rows = 1 if args.profile == "decode" else min(32, max(2, args.profile_rows))
             for _ in range(3):
                 for _, w in layers:
                     req.infer_device(w, x_dev, y_dev, rows)
