@@ -1,4 +1,4 @@
-// Decode kernel for five to thirty-two rows over 4-bit tiles with one group per k-block (G = 128): the matrix-vector
+// Decode kernel for five to forty-eight rows over 4-bit tiles with one group per k-block (G = 128): the matrix-vector
 // kernel's structure (kernel_gemv.hip) carried to whole 16-row MFMA tiles, with the activations stationary.
 //
 // A workgroup has K / (128 C) waves; wave w owns the k-blocks w, w + NWT, ... (C of them) of every channel tile the
@@ -12,7 +12,7 @@
 // in LDS behind one barrier per visit, where four waves add them in wave order (four rows each), apply the bias
 // and store.  Nothing is split along K through memory -- which is what the small-batch kernel
 // (kernel_batch.hip) pays five dependent round trips for -- and the activations travel from L2 once per workgroup,
-// not once per channel tile.  Rows 16-31 are the second workgroup row (blockIdx.y = 1).  The price: 16 rows x K x 2
+// not once per channel tile.  Rows 16-31 and 32-47 are further workgroup rows (blockIdx.y).  The price: 16 rows x K x 2
 // bytes of LDS for the hand-over, so K <= 4096 or so, and registers (16 C for the activations, 4 C for their group
 // sums, 3 (4 C + 4) for the weights), which bound the workgroup at 8 and 16 waves for C = 4 and 2.  A node whose
 // channel-major tables were laid out for eight k-blocks per wave runs with two waves per table row, four k-blocks
@@ -313,7 +313,7 @@ int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     const int ct = L.gemv_c;
     // what the kernel and its grid assume, checked against the operands before anything is launched
     if (!L.tiled || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 || !a.scale_cm ||
-        (L.zp_table && !a.zp_cm) || a.M < 1 || a.M > 32 || (ct != 2 && ct != 4 && ct != 8) || L.k_blocks % ct != 0 ||
+        (L.zp_table && !a.zp_cm) || a.M < 1 || a.M > kDecodeMaxRows || (ct != 2 && ct != 4 && ct != 8) || L.k_blocks % ct != 0 ||
         p.gemv_c != ct || (!L.zp_table && (L.zp_const < 0 || L.zp_const > 255)) || (L.glu && (L.n_tiles & 1)))
         return (int)hipErrorInvalidValue;
     const int c = gemv16_kblocks_per_wave(ct);

@@ -131,7 +131,7 @@ struct LaunchPlan {
     bool batch = false;         // decode family: the small-batch kernel (waves own channel tiles)
     bool gemv = false;          // decode family: the matrix-vector kernel for M <= 4 (4-bit weights, G = 128)
     int gemv_c = 0;             // ... and its k-blocks per wave (2, 4 or 8)
-    bool gemv16 = false;        // decode family: its 16-row sibling with stationary activations (5 <= M <= 32)
+    bool gemv16 = false;        // decode family: its 16-row sibling with stationary activations (5 <= M <= 48)
     int tiles_x = 0, tiles_y = 0;  // async prefill kernel: the tile grid; its launch is 1-D
     int full_tiles = 0;         // ... of which this many run unsplit (the rest in split_k parts each)
     unsigned grid[3] = {1, 1, 1};

@@ -19,7 +19,7 @@ namespace ovfcc {
 //   tuning:  OVFCC_DECODE_WAVES = 4 | 8 | 16 (workgroup size), OVFCC_DECODE_RT = 1 | 2 | 4 (channel tiles per
 //            workgroup or wave), OVFCC_DECODE_XLDS = 0 | 1 (activations via LDS), OVFCC_DECODE_BATCH = 0 | 1
 //            (small-batch kernel instead of the streaming kernel), OVFCC_GEMV = 0 | 1, OVFCC_GEMV_C = 2 | 4 | 8,
-//            OVFCC_GEMV16 = 0 | 1 (the 16-row kernel with stationary activations for 5-32 rows),
+//            OVFCC_GEMV16 = 0 | 1 (the 16-row kernel with stationary activations for 5-48 rows),
 //            OVFCC_GEMV16_GRID = n (its workgroups per row tile),
 //            OVFCC_PREFILL_{DIRECT, ASYNC, WIDE, BIG, TAIL} = 0 | 1, OVFCC_PREFILL_ROWS = 64 | 128,
 //            OVFCC_MOE_HOST_ROUTING = 1;
@@ -164,12 +164,12 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.name = L.bits == 4 ? "fcc_batch_w4" : "fcc_batch_w8";
         return OVFCC_OK;
     };
-    // Five to 32 rows of a 4-bit node with groups of 128 inputs whose 16 rows x K of activations fit in LDS (and,
+    // Five to 48 rows of a 4-bit node with groups of 128 inputs whose 16 rows x K of activations fit in LDS (and,
     // divided among the waves, in registers): the 16-row sibling of the matrix-vector kernel.  Every workgroup
     // keeps its row tile of the activations and walks channel tiles; the grid is as many workgroups as the chip
     // holds at once, rounded so that all of them visit the same number of tiles.
     auto plan_gemv16 = [&]() -> bool {
-        if (a.M <= 4 || a.M > 32 || !a.scale_cm || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 ||
+        if (a.M <= 4 || a.M > kDecodeMaxRows || !a.scale_cm || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 ||
             force_split > 0 || L.gemv_c == 0 || (L.glu && (L.n_tiles & 1)) || env_int("OVFCC_GEMV16", 1) == 0 ||
             env_int("OVFCC_DECODE_BATCH", -1) >= 0)
             return false;

@@ -114,7 +114,7 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
             const int c = ovfcc::gemv16_kblocks_per_wave(p.gemv_c);
             const int64_t units = L.glu ? L.n_tiles / 2 : L.n_tiles;
             const int per_unit = L.glu ? 2 : 1;
-            CHECK(M > 4 && M <= 32 && L.bits == 4 && L.groups_per_kblock == 1 && L.kblocks_per_group == 1 && p.gemv_c == L.gemv_c &&
+            CHECK(M > 4 && M <= 48 && L.bits == 4 && L.groups_per_kblock == 1 && L.kblocks_per_group == 1 && p.gemv_c == L.gemv_c &&
                       (!L.glu || L.n_tiles % 2 == 0),
                   "%s", what);
             CHECK(kb % c == 0 && nw == kb / c && nw <= (c == 4 ? 8 : 16), "%s c=%d nw=%d", what, c, nw);

@@ -1,6 +1,6 @@
-"""GPU parity of the 16-row decode kernel with stationary activations (five to 32 rows, 4-bit weights, groups of 128
+"""GPU parity of the 16-row decode kernel with stationary activations (five to 48 rows, 4-bit weights, groups of 128
 inputs) against the CPU oracle: every division of K over the waves of a workgroup (2, 4 or 8 k-blocks per wave),
-every row count class (part of a row tile, a whole one, part of the second, both), workgroups that visit one, two
+every row count class (part of a row tile, a whole one, part of the second, two, part of the third, three), workgroups that visit one, two
 and many channel tiles, zero-point table / constant / none, bias, both output types, the same bits on every
 repetition, the gated linear unit, and the node shapes of the benchmark."""
 import sys
@@ -51,15 +51,15 @@ SHAPES = [
 
 @pytest.mark.parametrize("wt,zt,N,K,C,grid,bias", SHAPES)
 @pytest.mark.parametrize("out", ["f16", "f32"])
-def test_gemv16_rows_five_to_thirty_two(oracle, dev, req, monkeypatch, wt, zt, N, K, C, grid, bias, out):
+def test_gemv16_rows_five_to_forty_eight(oracle, dev, req, monkeypatch, wt, zt, N, K, C, grid, bias, out):
     monkeypatch.setenv("OVFCC_GEMV_C", str(C))
     if grid:
         monkeypatch.setenv("OVFCC_GEMV16_GRID", str(grid))
-    c = datagen.make_case(7500 + N + K, 32, K, N, wt, 128, zt, with_bias=bias)
+    c = datagen.make_case(7500 + N + K, 48, K, N, wt, 128, zt, with_bias=bias)
     w = fc.CompressedWeights.from_case(dev, c, output_type=out)
     ref = oracle_y(oracle, c)
     try:
-        for M in (5, 8, 15, 16, 17, 31, 32):
+        for M in (5, 8, 15, 16, 17, 31, 32, 33, 48):
             say(f"gemv16 {wt}/{zt} N={N} K={K} C={C} grid={grid} out={out} M={M}")
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
@@ -123,13 +123,13 @@ def test_gemv16_tiny_and_huge_activations(oracle, dev, req):
 def test_gemv16_benchmark_nodes(oracle, dev, req, name, N, K):
     """The Llama-3-8B projections whose activations fit in LDS, at the benchmark's row counts, against the oracle on
     a sample of channels; the down projection (K = 14336) stays with the small-batch kernel."""
-    c = datagen.make_case(7800 + N, 32, K, N, "i4", 128, "none")
+    c = datagen.make_case(7800 + N, 48, K, N, "i4", 128, "none")
     w = fc.CompressedWeights.from_case(dev, c)
     rng = np.random.default_rng(5)
     cols = np.sort(rng.choice(N, size=256, replace=False))
     ref = oracle_y(oracle, c, n_index=cols)
     try:
-        for M in (8, 16, 32):
+        for M in (8, 16, 32, 48):
             say(f"gemv16 {name} M={M}")
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
@@ -148,10 +148,10 @@ def test_gemv16_gated_linear_unit(oracle, dev, req, monkeypatch, wt, zt, N, K, C
     monkeypatch.setenv("OVFCC_GEMV_C", str(C))
     if grid:
         monkeypatch.setenv("OVFCC_GEMV16_GRID", str(grid))
-    c = datagen.make_case(7950 + N, 32, K, N, wt, 128, zt, with_bias=True)
+    c = datagen.make_case(7950 + N, 48, K, N, wt, 128, zt, with_bias=True)
     w = fc.CompressedWeights.from_case(dev, c, glu=kind, glu_gate_second=second)
     try:
-        for M in (5, 16, 17, 32):
+        for M in (5, 16, 17, 32, 40):
             say(f"gemv16 glu {kind} {wt}/{zt} N={N} K={K} C={C} grid={grid} M={M}")
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()

@@ -181,9 +181,13 @@ def test_kernel_policy(dev, req, monkeypatch):
         assert req.last_kernel()["name"] == "fcc_batch_w4"
         monkeypatch.delenv("OVFCC_GEMV16")
         req.infer(w, c.x[:48])
-        assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
-        req.infer(w, c.x[:128])          # three launches of the small-batch kernel
+        assert req.last_kernel()["name"] == "fcc_gemv16_w4" and req.last_kernel()["grid"][1] == 3
+        req.infer(w, c.x[:128])          # three launches of 43, 43 and 42 rows
+        assert req.last_kernel()["name"] == "fcc_gemv16_w4" and req.last_kernel()["grid"][1] == 3
+        monkeypatch.setenv("OVFCC_GEMV16", "0")
+        req.infer(w, c.x[:128])          # ... of the small-batch kernel
         assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE and req.last_kernel()["tile_m"] == 48
+        monkeypatch.delenv("OVFCC_GEMV16")
         req.infer(w, c.x[:129])
         assert req.last_kernel()["kernel"] == _lib.KERNEL_PREFILL
         req.force_kernel(_lib.KERNEL_PLAIN)
