@@ -244,6 +244,19 @@ typedef struct ovfcc_group_item {
 } ovfcc_group_item;
 int ovfcc_fc_run_grouped_device(ovfcc_request* req, const ovfcc_group_item* items, int n_items);
 
+/* GroupedMatMulCompressed (src/common/transformations/include/ov_ops/grouped_matmul_compressed.hpp:17-66, the
+ * compressed form of ov::op::v17::GroupedMatMul, src/core/include/openvino/op/grouped_matmul.hpp:26-50; arithmetic
+ * src/core/reference/include/openvino/reference/grouped_matmul.hpp:36-88): groups[g] is group g's node (B[g] of the
+ * op's [G, N, K] constant, all of one shape and format).
+ *   2-D x 3-D form (offsets != NULL): a_dev is A [rows, K] f16, offsets [n_groups] int32 in host memory are the
+ *   cumulative row ends -- group g multiplies rows [offsets[g-1], offsets[g]) (offsets[-1] = 0; a group may be
+ *   empty) -- and y_dev receives [rows, N_out]; rows from offsets[n_groups-1] on come out as zeros, as in the
+ *   reference.  Offsets that decrease or exceed `rows` are OVFCC_EINVAL.
+ *   3-D x 3-D form (offsets == NULL): a_dev is A [n_groups, rows, K], y_dev receives [n_groups, rows, N_out].
+ * One grouped launch (ovfcc_fc_run_grouped_device) on the request's stream; no copies, no waiting. */
+int ovfcc_grouped_matmul_device(ovfcc_request* req, const ovfcc_weights* const* groups, int n_groups, const void* a_dev,
+                                const int32_t* offsets, int64_t rows, void* y_dev);
+
 /* GatherMatmulCompressed (src/common/transformations/include/ov_ops/gather_matmul.hpp:17-41,
  * gather_matmul_compressed.hpp:17-33; shapes src/common/transformations/src/ov_ops/gather_matmul.cpp:38-130; CPU
  * executor src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_gathermatmul_executor.cpp:470-600): the expert

@@ -53,7 +53,9 @@ enum ovfcc_op {
     OVFCC_OP_GATHER_MATMUL_COMPRESSED = 15, /* internal::GatherMatmulCompressed: (A, B, indices, bias, scale, zp) */
     OVFCC_OP_UNSQUEEZE = 16,
     OVFCC_OP_SLICE = 17,
-    OVFCC_OP_REDUCE_SUM = 18                /* v1::ReduceSum; attr = keep_dims */
+    OVFCC_OP_REDUCE_SUM = 18,               /* v1::ReduceSum; attr = keep_dims */
+    OVFCC_OP_GROUPED_MATMUL = 19,           /* v17::GroupedMatMul: inputs (A, B) or (A, B, offsets) */
+    OVFCC_OP_GROUPED_MATMUL_COMPRESSED = 20 /* internal::GroupedMatMulCompressed: (A, B, [offsets,] scale[, zp]) */
 };
 
 /* element types beyond enum ovfcc_type that a graph may carry (bf16, i32 shape constants, ...) */
@@ -148,6 +150,18 @@ typedef struct ovfcc_gather_fold {
 } ovfcc_gather_fold;
 
 int ovfcc_fold_gather_matmul(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_gather_fold* out);
+
+/* A matched GroupedMatMulCompressed node (src/common/transformations/include/ov_ops/grouped_matmul_compressed.hpp:
+ * 17-66): either a v17::GroupedMatMul (src/core/include/openvino/op/grouped_matmul.hpp:26-50) whose B input is the
+ * weight-decompression subgraph over a batched Constant [G, N, K] (or [G, N, K/g, g] behind a Reshape) -- the role
+ * of ConvertGroupedMatMulToGroupedMatMulCompressed (src/common/transformations/src/transformations/op_conversions/
+ * convert_grouped_matmul_to_compressed.cpp:25-118) -- or an internal::GroupedMatMulCompressed as that pass leaves
+ * it.  The result uses ovfcc_gather_fold with this reading: n_experts = the number of groups G, activations = A
+ * ([rows, K] with offsets, [G, M, K] without), indices = the offsets node ([G], int32 or int64 cumulative row ends)
+ * or -1 for the 3-D x 3-D form, top_k = -1, bias = -1 (the op has none).  Group g's node is created from slice g of
+ * every constant, as for ovfcc_fold_gather_matmul, and the G nodes go to ovfcc_grouped_matmul_device.  Weights
+ * behind a Transpose ([G, K, N] constants) are OVFCC_EUNSUPPORTED. */
+int ovfcc_fold_grouped_matmul(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_gather_fold* out);
 
 /* A matched expert block: three GatherMatmul[Compressed] nodes, the gate activation, the Multiply by the routing
  * weights and the ReduceSum over the selected experts -- what Convert3GatherMatmulMoeBlockToMoeOp

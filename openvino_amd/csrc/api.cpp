@@ -1485,6 +1485,59 @@ int ovfcc_gather_matmul_device(ovfcc_request* r, const ovfcc_weights* const* exp
     return OVFCC_OK;
 }
 
+int ovfcc_grouped_matmul_device(ovfcc_request* r, const ovfcc_weights* const* groups, int n_groups, const void* a_dev,
+                                const int32_t* offsets, int64_t rows, void* y_dev) {
+    if (!r || !groups || n_groups <= 0 || rows < 0)
+        return fail(OVFCC_EINVAL, "bad grouped-matmul arguments");
+    if (!groups[0])
+        return fail(OVFCC_EINVAL, "a group's weights are null or belong to another context");
+    bool same_zp = true;
+    int rc = experts_agree(r, groups, n_groups, &same_zp);
+    if (rc)
+        return rc;
+    const ovfcc_weights* w0 = groups[0];
+    const int64_t K = w0->desc.K, N_out = out_channels(w0);
+    const size_t out_bytes = w0->desc.out_type == OVFCC_F32 ? 4 : 2;
+    if (offsets) {
+        int64_t before = 0;
+        for (int g = 0; g < n_groups; ++g) {
+            if (offsets[g] < before || offsets[g] > rows)
+                return fail(OVFCC_EINVAL, "offsets must not decrease and must not exceed the rows of A");
+            before = offsets[g];
+        }
+    }
+    if (rows == 0)
+        return OVFCC_OK;
+    if (!a_dev || !y_dev)
+        return fail(OVFCC_EINVAL, "A or Y is null");
+    if ((N_out * out_bytes) % 4 != 0)
+        return fail(OVFCC_EUNSUPPORTED, "rows of Y must be multiples of 4 bytes");
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    const char* a = static_cast<const char*>(a_dev);
+    char* y = static_cast<char*>(y_dev);
+    std::vector<ovfcc_group_item> items;
+    items.reserve((size_t)n_groups);
+    if (offsets) {
+        int64_t start = 0;
+        for (int g = 0; g < n_groups; ++g) {
+            const int64_t end = offsets[g];
+            if (end > start)
+                items.push_back({groups[g], a + (size_t)start * K * 2, y + (size_t)start * N_out * out_bytes, end - start});
+            start = end;
+        }
+        if (start < rows) {  // rows that belong to no group: zeros
+            int e = ovfcc::launch_zero_u32(reinterpret_cast<unsigned*>(y + (size_t)start * N_out * out_bytes),
+                                           (size_t)(rows - start) * N_out * out_bytes / 4, r->stream);
+            if (e)
+                return hip_fail((hipError_t)e, "zero fill launch");
+        }
+    } else {
+        for (int g = 0; g < n_groups; ++g)
+            items.push_back({groups[g], a + (size_t)g * rows * K * 2, y + (size_t)g * rows * N_out * out_bytes, rows});
+    }
+    return ovfcc_fc_run_grouped_device(r, items.data(), (int)items.size());
+}
+
 namespace {
 int check_moe(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down, int n_experts,
               const void* x_dev, const void* routing_dev, const void* indices, int64_t M, int top_k, void* y_dev,

@@ -394,7 +394,9 @@ bool per_expert_group(const ovfcc_gnode& c, int64_t E, int64_t N, int64_t ng, bo
     return grouped ? broadcasts_per_group(c, want4, 4) : (broadcasts_per_group(c, want3, 3) && ng == 1);
 }
 
-int gather_impl(const Graph& g, int root, ovfcc_gather_fold* out) {
+// grouped_op: the root is a GroupedMatMul[Compressed] (groups of consecutive rows, cut by offsets or by the first
+// dimension of A) instead of a GatherMatmul[Compressed] (rows routed by indices); the weight side is the same
+int gather_impl(const Graph& g, int root, ovfcc_gather_fold* out, bool grouped_op = false) {
     ovfcc_gather_fold f;
     std::memset(&f, 0, sizeof(f));
     f.root = root;
@@ -404,23 +406,40 @@ int gather_impl(const Graph& g, int root, ovfcc_gather_fold* out) {
     if (!g.has(root))
         return fail(OVFCC_EINVAL, "root is not a node of the graph");
     const ovfcc_gnode& m = g.at(root);
-    const bool compressed = m.op == OVFCC_OP_GATHER_MATMUL_COMPRESSED;
-    if (m.op != OVFCC_OP_GATHER_MATMUL && !compressed)
-        return fail(OVFCC_EUNSUPPORTED, "root is neither a GatherMatmul nor a GatherMatmulCompressed");
-    if (m.n_inputs < (compressed ? 6 : 3))
-        return fail(OVFCC_EINVAL, "GatherMatmul with too few inputs");
+    const bool compressed =
+        m.op == (grouped_op ? OVFCC_OP_GROUPED_MATMUL_COMPRESSED : OVFCC_OP_GATHER_MATMUL_COMPRESSED);
+    if (m.op != (grouped_op ? OVFCC_OP_GROUPED_MATMUL : OVFCC_OP_GATHER_MATMUL) && !compressed)
+        return fail(OVFCC_EUNSUPPORTED, grouped_op ? "root is neither a GroupedMatMul nor a GroupedMatMulCompressed"
+                                                    : "root is neither a GatherMatmul nor a GatherMatmulCompressed");
     f.activations = g.input(root, 0);
-    f.indices = g.input(root, 2);
-    if (f.activations < 0 || f.indices < 0)
-        return fail(OVFCC_EINVAL, "GatherMatmul without activations or indices");
+    if (f.activations < 0)
+        return fail(OVFCC_EINVAL, "no activations");
+    // input slots: GatherMatmul (A, B, indices, bias[, scale, zp]); GroupedMatMul (A, B[, offsets]) and its
+    // compressed form (A, B, [offsets,] scale[, zp]), where the rank of A tells whether there are offsets
+    int scale_slot = 4, zp_slot = 5;
+    if (grouped_op) {
+        const bool with_offsets = g.at(f.activations).rank == 2;
+        if (m.n_inputs < (compressed ? 3 : 2) + (with_offsets ? 1 : 0))
+            return fail(OVFCC_EINVAL, "GroupedMatMul with too few inputs");
+        f.indices = with_offsets ? g.input(root, 2) : -1;
+        if (with_offsets && f.indices < 0)
+            return fail(OVFCC_EINVAL, "GroupedMatMul over two-dimensional activations without offsets");
+        scale_slot = with_offsets ? 3 : 2, zp_slot = scale_slot + 1;
+    } else {
+        if (m.n_inputs < (compressed ? 6 : 3))
+            return fail(OVFCC_EINVAL, "GatherMatmul with too few inputs");
+        f.indices = g.input(root, 2);
+        if (f.indices < 0)
+            return fail(OVFCC_EINVAL, "GatherMatmul without indices");
+    }
 
     int wc = -1, scale = -1, zp = -1, reshape = -1;
     if (compressed) {
-        // the node as ConvertGatherMatmulToGatherMatmulCompressed leaves it: B, scale and zero-point are Constants
-        // of three dimensions (a zero-point of no elements stands for "none")
-        wc = g.input(root, 1), scale = g.input(root, 4), zp = g.input(root, 5);
+        // the node as the conversion pass leaves it: B, scale and zero-point are Constants of three dimensions (a
+        // zero-point of no elements, or a missing one, stands for "none")
+        wc = g.input(root, 1), scale = g.input(root, scale_slot), zp = zp_slot < m.n_inputs ? g.input(root, zp_slot) : -1;
         if (wc < 0 || g.at(wc).op != OVFCC_OP_CONSTANT || scale < 0 || g.at(scale).op != OVFCC_OP_CONSTANT)
-            return fail(OVFCC_EUNSUPPORTED, "GatherMatmulCompressed needs Constant weights and scales");
+            return fail(OVFCC_EUNSUPPORTED, "the compressed node needs Constant weights and scales");
         if (zp >= 0 && (g.at(zp).op != OVFCC_OP_CONSTANT || element_count(g.at(zp)) == 0))
             zp = -1;
         chain.add(wc), chain.add(scale), chain.add(zp);
@@ -530,25 +549,38 @@ int gather_impl(const Graph& g, int root, ovfcc_gather_fold* out) {
         }
     }
 
-    // ---- activations [1 or top_k, M, K], indices [M, top_k] ----
     const ovfcc_gnode& A = g.at(f.activations);
     if (A.type == OVFCC_F32)
         f.activations_f32 = 1;
     else if (A.type != OVFCC_F16)
         return fail(OVFCC_EUNSUPPORTED, "activations must be f16 (or f32, converted by the host)");
-    if (A.rank != 3 || A.dims[2] != K)
-        return fail(OVFCC_EUNSUPPORTED, "activations must be [1 or top_k, M, K]");
-    const ovfcc_gnode& I = g.at(f.indices);
-    if (I.rank != 2)
-        return fail(OVFCC_EUNSUPPORTED, "indices must be [M, top_k]");
-    f.top_k = I.dims[1] >= 0 ? (int32_t)I.dims[1] : -1;
-    if (f.top_k > 0 && A.dims[0] >= 0 && A.dims[0] != 1 && A.dims[0] != f.top_k)
-        return fail(OVFCC_EUNSUPPORTED, "the first dimension of the activations must be 1 or top_k");
-    if (f.top_k > E)
-        return fail(OVFCC_EUNSUPPORTED, "more selections per row than experts");
+    if (grouped_op) {
+        // ---- activations [rows, K] with offsets [G], or [G, M, K] ----
+        if (f.indices >= 0) {
+            const ovfcc_gnode& O = g.at(f.indices);
+            if (A.rank != 2 || A.dims[1] != K)
+                return fail(OVFCC_EUNSUPPORTED, "activations must be [rows, K]");
+            if (O.rank != 1 || (O.dims[0] >= 0 && O.dims[0] != E))
+                return fail(OVFCC_EUNSUPPORTED, "offsets must hold one cumulative row end per group");
+        } else if (A.rank != 3 || A.dims[2] != K || (A.dims[0] >= 0 && A.dims[0] != E)) {
+            return fail(OVFCC_EUNSUPPORTED, "activations must be [G, M, K]");
+        }
+    } else {
+        // ---- activations [1 or top_k, M, K], indices [M, top_k] ----
+        if (A.rank != 3 || A.dims[2] != K)
+            return fail(OVFCC_EUNSUPPORTED, "activations must be [1 or top_k, M, K]");
+        const ovfcc_gnode& I = g.at(f.indices);
+        if (I.rank != 2)
+            return fail(OVFCC_EUNSUPPORTED, "indices must be [M, top_k]");
+        f.top_k = I.dims[1] >= 0 ? (int32_t)I.dims[1] : -1;
+        if (f.top_k > 0 && A.dims[0] >= 0 && A.dims[0] != 1 && A.dims[0] != f.top_k)
+            return fail(OVFCC_EUNSUPPORTED, "the first dimension of the activations must be 1 or top_k");
+        if (f.top_k > E)
+            return fail(OVFCC_EUNSUPPORTED, "more selections per row than experts");
+    }
 
-    // ---- bias: Constant(dynamic, Shape{0}) = none; N values shared, or E x N ----
-    const int bias = g.input(root, 3);
+    // ---- bias (GatherMatmul only): Constant(dynamic, Shape{0}) = none; N values shared, or E x N ----
+    const int bias = grouped_op ? -1 : g.input(root, 3);
     if (bias >= 0 && element_count(g.at(bias)) != 0) {
         const ovfcc_gnode& B = g.at(bias);
         const int64_t bc = element_count(B);
@@ -819,6 +851,12 @@ int ovfcc_fold_model(const ovfcc_gnode* nodes, int n_nodes, ovfcc_fold* folds, i
     *n_folds = (int)found.size();
     *n_fused = (int)groups.size();
     return OVFCC_OK;
+}
+
+int ovfcc_fold_grouped_matmul(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_gather_fold* out) {
+    if (!nodes || n_nodes <= 0 || !out)
+        return fail(OVFCC_EINVAL, "null argument");
+    return gather_impl(Graph{nodes, n_nodes}, root, out, true);
 }
 
 int ovfcc_fold_gather_matmul(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_gather_fold* out) {

@@ -287,6 +287,48 @@ class InferRequest:
                 dev.free(xp)
                 dev.free(yp)
 
+    def grouped_matmul_device(self, groups: Sequence[CompressedWeights], a_ptr: int, offsets: Optional[np.ndarray],
+                              rows: int, y_ptr: int) -> None:
+        """GroupedMatMulCompressed on device buffers.  offsets int32 [G] on the host (cumulative row ends): A
+        [rows, K] at a_ptr, Y [rows, N_out] at y_ptr; offsets None: A [G, rows, K], Y [G, rows, N_out]."""
+        arr = (ctypes.c_void_p * len(groups))(*[w.handle for w in groups])
+        off = None
+        if offsets is not None:
+            off_arr = np.ascontiguousarray(offsets, dtype=np.int32)
+            if off_arr.shape != (len(groups),):
+                raise OvfccError(_lib.EINVAL, f"offsets have shape {off_arr.shape}, expected ({len(groups)},)")
+            off = off_arr.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+        check(self.device.lib.ovfcc_grouped_matmul_device(self.handle, arr, len(groups), ctypes.c_void_p(a_ptr), off,
+                                                          rows, ctypes.c_void_p(y_ptr)))
+
+    def grouped_matmul(self, groups: Sequence[CompressedWeights], A: np.ndarray,
+                       offsets: Optional[np.ndarray] = None, y_fill: Optional[float] = None) -> np.ndarray:
+        """Host convenience: with offsets A float16 [rows, K] -> Y [rows, N_out]; without, A [G, M, K] -> Y [G, M, N_out].
+        y_fill: Y is preset to this value (the call must overwrite all of it)."""
+        A = np.ascontiguousarray(A, dtype=np.float16)
+        w = groups[0]
+        want = 2 if offsets is not None else 3
+        if A.ndim != want or A.shape[-1] != w.K or (offsets is None and A.shape[0] != len(groups)):
+            raise OvfccError(_lib.EINVAL, f"A has shape {A.shape}")
+        rows = A.shape[0] if offsets is not None else A.shape[1]
+        out_shape = (rows, w.N_out) if offsets is not None else (len(groups), rows, w.N_out)
+        dt = np.float32 if w.desc.out_type == _lib.F32 else np.float16
+        if rows == 0:
+            self.grouped_matmul_device(groups, 0, offsets, 0, 0)
+            return np.empty(out_shape, dt)
+        dev = self.device
+        a_ptr, y_ptr = dev.malloc(A.nbytes), dev.malloc(int(np.prod(out_shape)) * np.dtype(dt).itemsize)
+        try:
+            dev.upload(a_ptr, A)
+            if y_fill is not None:
+                dev.upload(y_ptr, np.full(out_shape, y_fill, dt))
+            self.grouped_matmul_device(groups, a_ptr, offsets, rows, y_ptr)
+            self.sync()
+            return dev.download(y_ptr, out_shape, dt)
+        finally:
+            dev.free(a_ptr)
+            dev.free(y_ptr)
+
     def gather_matmul_device(self, experts: Sequence[CompressedWeights], a_ptr: int, a_batches: int,
                              indices: np.ndarray, y_ptr: int) -> None:
         """GatherMatmulCompressed on device buffers: A [a_batches, M, K] at a_ptr, indices int32 [M, top_k] on the

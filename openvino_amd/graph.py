@@ -133,6 +133,18 @@ class Graph:
         return self._add("gather_matmul_compressed", type_ or self.type(a), [si[1], sa[1], sb[1]],
                          [a, b, indices, bias, scale, zp])
 
+    def grouped_matmul(self, a, b, offsets=None, type_=None):
+        """ov::op::v17::GroupedMatMul: A [rows, K] with offsets [G], or A [G, M, K]; B [G, N, K]"""
+        sa, sb = self.shape(a), self.shape(b)
+        return self._add("grouped_matmul", type_ or self.type(a), list(sa[:-1]) + [sb[1]],
+                         [a, b] + ([offsets] if offsets is not None else []))
+
+    def grouped_matmul_compressed(self, a, b, scale, zp=None, offsets=None, type_=None):
+        """ov::op::internal::GroupedMatMulCompressed: (A, B, [offsets,] scale[, zp]), B, scale, zp Constants"""
+        sa, sb = self.shape(a), self.shape(b)
+        ins = [a, b] + ([offsets] if offsets is not None else []) + [scale] + ([zp] if zp is not None else [])
+        return self._add("grouped_matmul_compressed", type_ or self.type(a), list(sa[:-1]) + [sb[1]], ins)
+
     def other(self, inputs, type_="f16", shape=None):
         return self._add("other", type_, shape, list(inputs))
 
@@ -154,6 +166,11 @@ class Graph:
     def fold_gather_matmul(self, root: int) -> _lib.GatherFold:
         out = _lib.GatherFold()
         check(_lib.load().ovfcc_fold_gather_matmul(self._array(), len(self.nodes), root, ctypes.byref(out)))
+        return out
+
+    def fold_grouped_matmul(self, root: int) -> _lib.GatherFold:
+        out = _lib.GatherFold()
+        check(_lib.load().ovfcc_fold_grouped_matmul(self._array(), len(self.nodes), root, ctypes.byref(out)))
         return out
 
     def fold_moe(self, root: int) -> _lib.MoeFold:

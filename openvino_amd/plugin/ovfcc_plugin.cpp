@@ -23,7 +23,10 @@
 // compressed constants [E, N, K] or [E, N, K/G, G], the gate activation, the Multiply by the transposed routing
 // weights, ReduceSum and Reshape; src/common/transformations/src/transformations/common_optimizations/
 // moe_op_fusion.cpp:55-232) whose hidden states, routing weights and expert indices are Parameters runs as one
-// ovfcc_moe_device call -- MOECompressed in the executed graph.  The pattern is matched on the untouched input model, before
+// ovfcc_moe_device call -- MOECompressed in the executed graph.  A v17::GroupedMatMul over batched compressed constants
+// (or the GroupedMatMulCompressed that ConvertGroupedMatMulToGroupedMatMulCompressed makes of it,
+// src/common/transformations/src/transformations/op_conversions/convert_grouped_matmul_to_compressed.cpp:25-118) whose
+// activations and offsets are Parameters runs as one ovfcc_grouped_matmul_device call.  The pattern is matched on the untouched input model, before
 // any folding pass, so the u4/u8 constants are still there and no MarkDequantization pass is needed.  Everything
 // else is reported as unsupported by query_model (a HETERO device can place it elsewhere) and rejected by
 // compile_model.
@@ -74,6 +77,7 @@
 #include "ov_ops/fully_connected_compressed.hpp"
 #include "ov_ops/gather_matmul.hpp"
 #include "ov_ops/gather_matmul_compressed.hpp"
+#include "ov_ops/grouped_matmul_compressed.hpp"
 #include "ovfcc.h"
 #include "ovfcc_graph.h"
 
@@ -105,6 +109,7 @@ struct ModelGraph {
     std::vector<ovfcc_fold> folds;
     std::vector<ovfcc_fused> fused;
     std::vector<ovfcc_moe_fold> moes;  // expert blocks (three GatherMatmul nodes and what joins them)
+    std::vector<ovfcc_gather_fold> grouped;  // GroupedMatMul[Compressed] nodes over batched compressed constants
 };
 
 static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
@@ -134,6 +139,8 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
         else if (ov::is_type<ov::op::v0::Result>(op)) n.op = OVFCC_OP_RESULT;
         else if (ov::is_type<ov::op::internal::GatherMatmulCompressed>(op)) n.op = OVFCC_OP_GATHER_MATMUL_COMPRESSED;
         else if (ov::is_type<ov::op::internal::GatherMatmul>(op)) n.op = OVFCC_OP_GATHER_MATMUL;
+        else if (ov::is_type<ov::op::internal::GroupedMatMulCompressed>(op)) n.op = OVFCC_OP_GROUPED_MATMUL_COMPRESSED;
+        else if (ov::is_type<ov::op::v17::GroupedMatMul>(op)) n.op = OVFCC_OP_GROUPED_MATMUL;
         else if (ov::is_type<ov::op::v0::Unsqueeze>(op)) n.op = OVFCC_OP_UNSQUEEZE;
         else if (ov::is_type<ov::op::v8::Slice>(op)) n.op = OVFCC_OP_SLICE;
         else if (ov::is_type<ov::op::v1::ReduceSum>(op)) n.op = OVFCC_OP_REDUCE_SUM;
@@ -192,6 +199,14 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
         ovfcc_moe_fold m;
         if (ovfcc_fold_moe(g.nodes.data(), (int)g.nodes.size(), g.nodes[i].inputs[0], &m) == OVFCC_OK)
             g.moes.push_back(m);
+    }
+    // grouped matrix products over batched compressed constants
+    for (size_t i = 0; i < g.nodes.size(); ++i) {
+        if (g.nodes[i].op != OVFCC_OP_GROUPED_MATMUL && g.nodes[i].op != OVFCC_OP_GROUPED_MATMUL_COMPRESSED)
+            continue;
+        ovfcc_gather_fold f;
+        if (ovfcc_fold_grouped_matmul(g.nodes.data(), (int)g.nodes.size(), (int)i, &f) == OVFCC_OK)
+            g.grouped.push_back(f);
     }
     return g;
 }
@@ -477,6 +492,17 @@ struct MoeLaunch {
     std::vector<std::string> original_names;
 };
 
+// One GroupedMatMulCompressed node: a node per group, activations and (in the 2-D x 3-D form) offsets from Parameters
+struct GroupedLaunch {
+    std::vector<ovfcc_weights*> groups;
+    size_t a_index = 0, offsets_index = 0, result_index = 0;
+    bool with_offsets = false;
+    int64_t K = 0, N = 0;
+    int out_type = OVFCC_F16;
+    std::string name;
+    std::vector<std::string> original_names;
+};
+
 class CompiledModel : public ov::ICompiledModel {
 public:
     // node_flags: OVFCC_* flags for every node's descriptor (OVFCC_DYNQUANT_I8 when the caller allows dynamic
@@ -493,14 +519,18 @@ public:
             for (auto* w : m.down)
                 ovfcc_weights_destroy(w);
         }
+        for (auto& gm : m_grouped)
+            for (auto* w : gm.groups)
+                ovfcc_weights_destroy(w);
     }
 
     // Stream layout: magic, node flags, the model as the template plugin stores it (xml and constants from
     // ov::pass::Serialize, each behind its size; src/plugins/template/src/compiled_model.cpp:173-192), then the
     // number of launches and every launch's repacked device image (ovfcc_weights_export) behind its size.
     void export_model(std::ostream& out) const override {
-        OPENVINO_ASSERT(m_moes.empty(), "MI355X: a model with expert blocks is compiled from its constants each time "
-                                         "(no blob form of an expert block)");
+        OPENVINO_ASSERT(m_moes.empty() && m_grouped.empty(),
+                        "MI355X: a model with expert blocks or grouped matrix products is compiled from its constants "
+                        "each time (no blob form of batched weights)");
         std::stringstream xml, bin;
         ov::pass::Serialize(xml, bin).run_on_model(m_model);
         const std::string x = xml.str(), b = bin.str();
@@ -583,6 +613,29 @@ public:
             results[m.result_index] = std::make_shared<ov::op::v0::Result>(node);
             results[m.result_index]->set_friendly_name(m_model->get_results()[m.result_index]->get_friendly_name());
         }
+        for (size_t i = 0; i < m_grouped.size(); ++i) {
+            const GroupedLaunch& gm = m_grouped[i];
+            ov::OutputVector ins{params[gm.a_index]};
+            if (gm.with_offsets)
+                ins.push_back(params[gm.offsets_index]);
+            auto node = std::make_shared<ov::exec_model_info::ExecutionNode>(ins, 1);
+            node->set_friendly_name(gm.name);
+            auto& rt = node->get_rt_info();
+            std::string names;
+            for (const auto& n : gm.original_names)
+                names += (names.empty() ? "" : ",") + n;
+            rt[ov::exec_model_info::LAYER_TYPE] = std::string("GroupedMatMulCompressed");
+            rt[ov::exec_model_info::IMPL_TYPE] = std::string("hip_grouped");
+            rt[ov::exec_model_info::ORIGINAL_NAMES] = names;
+            rt[ov::exec_model_info::OUTPUT_PRECISIONS] = std::string(gm.out_type == OVFCC_F32 ? "f32" : "f16");
+            rt[ov::exec_model_info::OUTPUT_LAYOUTS] = std::string(gm.with_offsets ? "ab" : "abc");
+            const size_t order = m_launches.size() + m_moes.size() + i;
+            rt[ov::exec_model_info::EXECUTION_ORDER] = std::to_string(order);
+            const double us = m_last_us[order].load();
+            rt[ov::exec_model_info::PERF_COUNTER] = us < 0 ? std::string("not_executed") : std::to_string((long long)us);
+            results[gm.result_index] = std::make_shared<ov::op::v0::Result>(node);
+            results[gm.result_index]->set_friendly_name(m_model->get_results()[gm.result_index]->get_friendly_name());
+        }
         return std::make_shared<ov::Model>(results, params, m_model->get_friendly_name() + "_executed");
     }
     void set_property(const ov::AnyMap&) override {
@@ -610,6 +663,9 @@ public:
     }
     const std::vector<MoeLaunch>& moes() const {
         return m_moes;
+    }
+    const std::vector<GroupedLaunch>& grouped() const {
+        return m_grouped;
     }
     ovfcc_ctx* ctx() const {
         return m_ctx;
@@ -642,6 +698,7 @@ private:
     ModelGraph m_graph;
     std::vector<Launch> m_launches;
     std::vector<MoeLaunch> m_moes;
+    std::vector<GroupedLaunch> m_grouped;
     mutable std::vector<std::atomic<double>> m_last_us;  // per launch: last measured time, -1 before the first run
     ovfcc_ctx* m_ctx;
     int m_node_flags = 0;
@@ -749,6 +806,7 @@ public:
             m_compiled->record_time(li, us);
         }
         run_expert_blocks();
+        run_grouped_products();
     }
 
     std::vector<ov::ProfilingInfo> get_profiling_info() const override {
@@ -756,9 +814,11 @@ public:
         for (size_t i = 0; i < m_kernels.size(); ++i) {
             ov::ProfilingInfo p;
             p.status = ov::ProfilingInfo::Status::EXECUTED;
-            const size_t n_fc = m_compiled->launches().size();
-            p.node_name = i < n_fc ? m_compiled->launches()[i].name : m_compiled->moes()[i - n_fc].name;
-            p.node_type = i < n_fc ? "FullyConnected" : "MOECompressed";
+            const size_t n_fc = m_compiled->launches().size(), n_moe = m_compiled->moes().size();
+            p.node_name = i < n_fc           ? m_compiled->launches()[i].name
+                          : i < n_fc + n_moe ? m_compiled->moes()[i - n_fc].name
+                                             : m_compiled->grouped()[i - n_fc - n_moe].name;
+            p.node_type = i < n_fc ? "FullyConnected" : i < n_fc + n_moe ? "MOECompressed" : "GroupedMatMulCompressed";
             p.exec_type = m_kernels[i].name;
             p.real_time = p.cpu_time = std::chrono::microseconds((long long)m_times_us[i]);
             out.push_back(p);
@@ -848,6 +908,80 @@ private:
             const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
             m_times_us.push_back(us);
             m_compiled->record_time(m_compiled->launches().size() + mi, us);
+        }
+    }
+
+    // GroupedMatMulCompressed: activations [rows, K] with offsets [G] (cumulative row ends, i32 or i64), or
+    // [G, M, K], in host tensors; staged to the device as f16, one ovfcc_grouped_matmul_device call, result copied back.
+    void run_grouped_products() {
+        const auto& all = m_compiled->grouped();
+        for (size_t gi = 0; gi < all.size(); ++gi) {
+            const GroupedLaunch& gm = all[gi];
+            const auto t0 = std::chrono::steady_clock::now();
+            auto a = get_tensor(get_inputs()[gm.a_index]);
+            auto out = get_tensor(get_outputs()[gm.result_index]);
+            const ov::Shape as = a->get_shape();
+            OPENVINO_ASSERT(as.size() == (gm.with_offsets ? 2u : 3u) && (int64_t)as.back() == gm.K,
+                            "MI355X: activations of ", gm.name, " have an unexpected shape");
+            const int n_groups = (int)gm.groups.size();
+            OPENVINO_ASSERT(gm.with_offsets || (int)as[0] == n_groups, "MI355X: one batch of activations per group");
+            const int64_t rows = gm.with_offsets ? (int64_t)as[0] : (int64_t)as[1];
+            ov::Shape os = as;
+            os.back() = (size_t)gm.N;
+            out->set_shape(os);
+            std::vector<int32_t> offsets;
+            if (gm.with_offsets) {
+                auto off = get_tensor(get_inputs()[gm.offsets_index]);
+                OPENVINO_ASSERT(off->get_size() == (size_t)n_groups, "MI355X: one offset per group");
+                offsets.resize((size_t)n_groups);
+                if (off->get_element_type() == ov::element::i32) {
+                    std::memcpy(offsets.data(), off->data(), offsets.size() * sizeof(int32_t));
+                } else {
+                    OPENVINO_ASSERT(off->get_element_type() == ov::element::i64, "MI355X: offsets must be i32 or i64");
+                    const int64_t* src = static_cast<const int64_t*>(off->data());
+                    for (size_t i = 0; i < offsets.size(); ++i)
+                        offsets[i] = (int32_t)src[i];
+                }
+            }
+            const size_t count = a->get_size(), out_count = out->get_size();
+            const size_t x_bytes = count * 2, y_bytes = out_count * (gm.out_type == OVFCC_F32 ? 4 : 2);
+            void* x_dev = device_staging(0, x_bytes);
+            void* y_dev = device_staging(1, y_bytes);
+            const void* x = a->data();
+            if (a->get_element_type() != ov::element::f16) {
+                OPENVINO_ASSERT(a->get_element_type() == ov::element::f32, "MI355X: expected f16 or f32 activations");
+                const float* src = static_cast<const float*>(a->data());
+                m_staging.resize(count);
+                for (size_t i = 0; i < count; ++i)
+                    m_staging[i] = ov::float16(src[i]);
+                x = m_staging.data();
+            }
+            if (x_bytes && ovfcc_memcpy_h2d(m_compiled->ctx(), x_dev, x, x_bytes) != OVFCC_OK)
+                throw_last("memcpy_h2d");
+            if (ovfcc_grouped_matmul_device(m_request, gm.groups.data(), n_groups, x_dev,
+                                            gm.with_offsets ? offsets.data() : nullptr, rows, y_dev) != OVFCC_OK)
+                throw_last("grouped_matmul_device");
+            if (ovfcc_request_sync(m_request) != OVFCC_OK)
+                throw_last("request_sync");
+            if (y_bytes) {
+                if (out->get_element_type() == ov::element::f32 && gm.out_type != OVFCC_F32) {
+                    m_y_staging.resize(y_bytes);
+                    if (ovfcc_memcpy_d2h(m_compiled->ctx(), m_y_staging.data(), y_dev, y_bytes) != OVFCC_OK)
+                        throw_last("memcpy_d2h");
+                    const auto* h = reinterpret_cast<const ov::float16*>(m_y_staging.data());
+                    float* dst = static_cast<float*>(out->data());
+                    for (size_t i = 0; i < out_count; ++i)
+                        dst[i] = (float)h[i];
+                } else if (ovfcc_memcpy_d2h(m_compiled->ctx(), out->data(), y_dev, y_bytes) != OVFCC_OK) {
+                    throw_last("memcpy_d2h");
+                }
+            }
+            ovfcc_kernel_info info;
+            ovfcc_last_kernel_info(m_request, &info);
+            m_kernels.push_back(info);
+            const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+            m_times_us.push_back(us);
+            m_compiled->record_time(m_compiled->launches().size() + m_compiled->moes().size() + gi, us);
         }
     }
 
@@ -1097,6 +1231,15 @@ public:
                     mark(id);
             mark_results_of(m.root);
         }
+        for (const auto& f : g.grouped) {
+            for (int c = 0; c < f.n_chain; ++c)
+                mark(f.chain[c]);
+            mark(f.root);
+            for (int id : {f.activations, f.indices})
+                if (id >= 0 && g.nodes[(size_t)id].op == OVFCC_OP_PARAMETER)
+                    mark(id);
+            mark_results_of(f.root);
+        }
         return res;
     }
 
@@ -1277,6 +1420,34 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
         }
         m_moes.push_back(std::move(l));
     }
+    for (const auto& f : g.grouped) {
+        OPENVINO_ASSERT(!blobs, "MI355X: a model with grouped matrix products has no blob form");
+        GroupedLaunch l;
+        l.name = g.ops[(size_t)f.root]->get_friendly_name();
+        auto param_index = [&](int id, const char* what) {
+            OPENVINO_ASSERT(g.nodes[(size_t)id].op == OVFCC_OP_PARAMETER, "MI355X: the ", what, " of ", l.name,
+                            " do not come straight from a Parameter (use HETERO:MI355X,CPU for the rest of the graph)");
+            for (size_t p = 0; p < params.size(); ++p)
+                if (params[p].get() == g.ops[(size_t)id].get())
+                    return p;
+            return (size_t)0;
+        };
+        l.a_index = param_index(f.activations, "activations");
+        l.with_offsets = f.indices >= 0;
+        if (l.with_offsets)
+            l.offsets_index = param_index(f.indices, "offsets");
+        const auto rs = results_of(f.root);
+        OPENVINO_ASSERT(rs.size() == 1, "MI355X: a grouped matrix product must feed exactly one model output");
+        l.result_index = rs[0];
+        fed[rs[0]] = true;
+        l.K = f.desc.K;
+        l.N = f.desc.N;
+        l.out_type = f.desc.out_type;
+        l.original_names.push_back(l.name);
+        for (int e = 0; e < f.n_experts; ++e)
+            l.groups.push_back(create_expert(ctx, g, f, e, node_flags));
+        m_grouped.push_back(std::move(l));
+    }
     for (size_t r = 0; r < results.size(); ++r)
         OPENVINO_ASSERT(fed[r], "MI355X: result ", results[r]->get_friendly_name(),
                         " is not produced by a weight-compressed FullyConnected (use HETERO:MI355X,CPU for the rest "
@@ -1292,7 +1463,7 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
     for (auto& l : m_launches)
         l.primitive = primitive(l.weights, g.folds[(size_t)l.folds[0]].desc,
                                 l.kind == OVFCC_FUSED_GLU ? "_glu" : (l.kind == OVFCC_FUSED_CONCAT ? "_fused" : ""));
-    m_last_us = std::vector<std::atomic<double>>(m_launches.size() + m_moes.size());
+    m_last_us = std::vector<std::atomic<double>>(m_launches.size() + m_moes.size() + m_grouped.size());
     for (auto& t : m_last_us)
         t.store(-1.0);
 }

@@ -246,6 +246,27 @@ def moe_reference(x, routing, indices, gate_up, down, glu_type) -> np.ndarray:
     return y.astype(np.float32)
 
 
+def grouped_matmul_reference(a, groups, offsets=None) -> np.ndarray:
+    """GroupedMatMul over decompressed weights (ov::op::v17::GroupedMatMul; arithmetic of
+    src/core/reference/include/openvino/reference/grouped_matmul.hpp:36-88 with B[g] = the decompressed weights of
+    group g): groups[g] holds the keyword arguments of fc_reference for group g.
+
+    offsets given (2-D x 3-D form, :61-88): a is [rows, K]; the output [rows, N] starts as zeros and group g fills
+    rows [offsets[g-1], offsets[g]) -- offsets are cumulative row ends, a group may be empty, rows beyond the last
+    offset stay zero.  offsets None (3-D x 3-D form, :36-58): a is [G, M, K], output [G, M, N].  float32."""
+    a = np.asarray(a)
+    N = groups[0]["N"]
+    if offsets is None:
+        return np.stack([fc_reference(a[g], **groups[g]) for g in range(len(groups))]).astype(np.float32)
+    out = np.zeros((a.shape[0], N), np.float32)
+    start = 0
+    for g, end in enumerate(np.asarray(offsets).tolist()):
+        if end > start:
+            out[start:end] = fc_reference(a[start:end], **groups[g])
+        start = end
+    return out
+
+
 def dynquant_rows(x):
     """C oracle: per-token symmetric int8 quantisation of x [M, K] float16 -> (q int8 [M, K], inv_scale float32 [M],
     qsum int32 [M])."""
