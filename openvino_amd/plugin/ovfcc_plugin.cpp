@@ -26,7 +26,8 @@
 // ovfcc_moe_device call -- MOECompressed in the executed graph.  A v17::GroupedMatMul over batched compressed constants
 // (or the GroupedMatMulCompressed that ConvertGroupedMatMulToGroupedMatMulCompressed makes of it,
 // src/common/transformations/src/transformations/op_conversions/convert_grouped_matmul_to_compressed.cpp:25-118) whose
-// activations and offsets are Parameters runs as one ovfcc_grouped_matmul_device call.  The pattern is matched on the untouched input model, before
+// activations and offsets are Parameters runs as one ovfcc_grouped_matmul_device call, and a GatherMatmul[Compressed]
+// outside such a block, over Parameters for activations and indices, as one ovfcc_gather_matmul_device call.  The pattern is matched on the untouched input model, before
 // any folding pass, so the u4/u8 constants are still there and no MarkDequantization pass is needed.  Everything
 // else is reported as unsupported by query_model (a HETERO device can place it elsewhere) and rejected by
 // compile_model.
@@ -109,7 +110,13 @@ struct ModelGraph {
     std::vector<ovfcc_fold> folds;
     std::vector<ovfcc_fused> fused;
     std::vector<ovfcc_moe_fold> moes;  // expert blocks (three GatherMatmul nodes and what joins them)
-    std::vector<ovfcc_gather_fold> grouped;  // GroupedMatMul[Compressed] nodes over batched compressed constants
+    // GroupedMatMul[Compressed] nodes over batched compressed constants, and GatherMatmul[Compressed] nodes that
+    // are no part of an expert block
+    struct Batched {
+        ovfcc_gather_fold fold;
+        bool gather;
+    };
+    std::vector<Batched> grouped;
 };
 
 static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
@@ -200,13 +207,20 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
         if (ovfcc_fold_moe(g.nodes.data(), (int)g.nodes.size(), g.nodes[i].inputs[0], &m) == OVFCC_OK)
             g.moes.push_back(m);
     }
-    // grouped matrix products over batched compressed constants
+    // grouped matrix products over batched compressed constants, and routed ones outside expert blocks
     for (size_t i = 0; i < g.nodes.size(); ++i) {
-        if (g.nodes[i].op != OVFCC_OP_GROUPED_MATMUL && g.nodes[i].op != OVFCC_OP_GROUPED_MATMUL_COMPRESSED)
-            continue;
+        const int op = g.nodes[i].op;
         ovfcc_gather_fold f;
-        if (ovfcc_fold_grouped_matmul(g.nodes.data(), (int)g.nodes.size(), (int)i, &f) == OVFCC_OK)
-            g.grouped.push_back(f);
+        if (op == OVFCC_OP_GROUPED_MATMUL || op == OVFCC_OP_GROUPED_MATMUL_COMPRESSED) {
+            if (ovfcc_fold_grouped_matmul(g.nodes.data(), (int)g.nodes.size(), (int)i, &f) == OVFCC_OK)
+                g.grouped.push_back({f, false});
+        } else if (op == OVFCC_OP_GATHER_MATMUL || op == OVFCC_OP_GATHER_MATMUL_COMPRESSED) {
+            bool in_block = false;
+            for (const auto& m : g.moes)
+                in_block = in_block || m.gate.root == (int)i || m.up.root == (int)i || m.down.root == (int)i;
+            if (!in_block && ovfcc_fold_gather_matmul(g.nodes.data(), (int)g.nodes.size(), (int)i, &f) == OVFCC_OK)
+                g.grouped.push_back({f, true});
+        }
     }
     return g;
 }
@@ -492,11 +506,14 @@ struct MoeLaunch {
     std::vector<std::string> original_names;
 };
 
-// One GroupedMatMulCompressed node: a node per group, activations and (in the 2-D x 3-D form) offsets from Parameters
+// One GroupedMatMulCompressed node -- a node per group, activations and (in the 2-D x 3-D form) offsets from
+// Parameters -- or one GatherMatmulCompressed node outside an expert block: a node per expert, activations
+// [1 or top_k, M, K] and indices [M, top_k] from Parameters (offsets_index names the indices then)
 struct GroupedLaunch {
     std::vector<ovfcc_weights*> groups;
     size_t a_index = 0, offsets_index = 0, result_index = 0;
     bool with_offsets = false;
+    bool gather = false;
     int64_t K = 0, N = 0;
     int out_type = OVFCC_F16;
     std::string name;
@@ -624,11 +641,11 @@ public:
             std::string names;
             for (const auto& n : gm.original_names)
                 names += (names.empty() ? "" : ",") + n;
-            rt[ov::exec_model_info::LAYER_TYPE] = std::string("GroupedMatMulCompressed");
+            rt[ov::exec_model_info::LAYER_TYPE] = std::string(gm.gather ? "GatherMatmulCompressed" : "GroupedMatMulCompressed");
             rt[ov::exec_model_info::IMPL_TYPE] = std::string("hip_grouped");
             rt[ov::exec_model_info::ORIGINAL_NAMES] = names;
             rt[ov::exec_model_info::OUTPUT_PRECISIONS] = std::string(gm.out_type == OVFCC_F32 ? "f32" : "f16");
-            rt[ov::exec_model_info::OUTPUT_LAYOUTS] = std::string(gm.with_offsets ? "ab" : "abc");
+            rt[ov::exec_model_info::OUTPUT_LAYOUTS] = std::string(gm.with_offsets && !gm.gather ? "ab" : "abc");
             const size_t order = m_launches.size() + m_moes.size() + i;
             rt[ov::exec_model_info::EXECUTION_ORDER] = std::to_string(order);
             const double us = m_last_us[order].load();
@@ -818,7 +835,10 @@ public:
             p.node_name = i < n_fc           ? m_compiled->launches()[i].name
                           : i < n_fc + n_moe ? m_compiled->moes()[i - n_fc].name
                                              : m_compiled->grouped()[i - n_fc - n_moe].name;
-            p.node_type = i < n_fc ? "FullyConnected" : i < n_fc + n_moe ? "MOECompressed" : "GroupedMatMulCompressed";
+            p.node_type = i < n_fc           ? "FullyConnected"
+                          : i < n_fc + n_moe ? "MOECompressed"
+                          : m_compiled->grouped()[i - n_fc - n_moe].gather ? "GatherMatmulCompressed"
+                                                                           : "GroupedMatMulCompressed";
             p.exec_type = m_kernels[i].name;
             p.real_time = p.cpu_time = std::chrono::microseconds((long long)m_times_us[i]);
             out.push_back(p);
@@ -921,19 +941,29 @@ private:
             auto a = get_tensor(get_inputs()[gm.a_index]);
             auto out = get_tensor(get_outputs()[gm.result_index]);
             const ov::Shape as = a->get_shape();
-            OPENVINO_ASSERT(as.size() == (gm.with_offsets ? 2u : 3u) && (int64_t)as.back() == gm.K,
+            OPENVINO_ASSERT(as.size() == (gm.with_offsets && !gm.gather ? 2u : 3u) && (int64_t)as.back() == gm.K,
                             "MI355X: activations of ", gm.name, " have an unexpected shape");
             const int n_groups = (int)gm.groups.size();
-            OPENVINO_ASSERT(gm.with_offsets || (int)as[0] == n_groups, "MI355X: one batch of activations per group");
-            const int64_t rows = gm.with_offsets ? (int64_t)as[0] : (int64_t)as[1];
+            OPENVINO_ASSERT(gm.gather || gm.with_offsets || (int)as[0] == n_groups,
+                            "MI355X: one batch of activations per group");
+            const int64_t rows = gm.with_offsets && !gm.gather ? (int64_t)as[0] : (int64_t)as[1];
+            int top_k = 0;
             ov::Shape os = as;
             os.back() = (size_t)gm.N;
-            out->set_shape(os);
             std::vector<int32_t> offsets;
             if (gm.with_offsets) {
                 auto off = get_tensor(get_inputs()[gm.offsets_index]);
-                OPENVINO_ASSERT(off->get_size() == (size_t)n_groups, "MI355X: one offset per group");
-                offsets.resize((size_t)n_groups);
+                if (gm.gather) {
+                    // indices [M, top_k]; the output is [top_k, M, N]
+                    const ov::Shape is = off->get_shape();
+                    OPENVINO_ASSERT(is.size() == 2 && (int64_t)is[0] == rows, "MI355X: indices must be [M, top_k]");
+                    top_k = (int)is[1];
+                    OPENVINO_ASSERT(as[0] == 1 || (int)as[0] == top_k, "MI355X: one batch of activations, or one per selection");
+                    os[0] = (size_t)top_k;
+                } else {
+                    OPENVINO_ASSERT(off->get_size() == (size_t)n_groups, "MI355X: one offset per group");
+                }
+                offsets.resize(off->get_size());
                 if (off->get_element_type() == ov::element::i32) {
                     std::memcpy(offsets.data(), off->data(), offsets.size() * sizeof(int32_t));
                 } else {
@@ -943,6 +973,7 @@ private:
                         offsets[i] = (int32_t)src[i];
                 }
             }
+            out->set_shape(os);
             const size_t count = a->get_size(), out_count = out->get_size();
             const size_t x_bytes = count * 2, y_bytes = out_count * (gm.out_type == OVFCC_F32 ? 4 : 2);
             void* x_dev = device_staging(0, x_bytes);
@@ -958,9 +989,14 @@ private:
             }
             if (x_bytes && ovfcc_memcpy_h2d(m_compiled->ctx(), x_dev, x, x_bytes) != OVFCC_OK)
                 throw_last("memcpy_h2d");
-            if (ovfcc_grouped_matmul_device(m_request, gm.groups.data(), n_groups, x_dev,
-                                            gm.with_offsets ? offsets.data() : nullptr, rows, y_dev) != OVFCC_OK)
+            if (gm.gather) {
+                if (ovfcc_gather_matmul_device(m_request, gm.groups.data(), n_groups, x_dev, (int)as[0], offsets.data(), rows,
+                                               top_k, y_dev) != OVFCC_OK)
+                    throw_last("gather_matmul_device");
+            } else if (ovfcc_grouped_matmul_device(m_request, gm.groups.data(), n_groups, x_dev,
+                                                   gm.with_offsets ? offsets.data() : nullptr, rows, y_dev) != OVFCC_OK) {
                 throw_last("grouped_matmul_device");
+            }
             if (ovfcc_request_sync(m_request) != OVFCC_OK)
                 throw_last("request_sync");
             if (y_bytes) {
@@ -1231,10 +1267,13 @@ public:
                     mark(id);
             mark_results_of(m.root);
         }
-        for (const auto& f : g.grouped) {
+        for (const auto& b : g.grouped) {
+            const ovfcc_gather_fold& f = b.fold;
             for (int c = 0; c < f.n_chain; ++c)
                 mark(f.chain[c]);
             mark(f.root);
+            if (b.gather && g.ops[(size_t)f.root]->get_input_size() > 3)
+                mark(g.nodes[(size_t)f.root].inputs[3]);  // the bias constant, empty or not
             for (int id : {f.activations, f.indices})
                 if (id >= 0 && g.nodes[(size_t)id].op == OVFCC_OP_PARAMETER)
                     mark(id);
@@ -1420,9 +1459,11 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
         }
         m_moes.push_back(std::move(l));
     }
-    for (const auto& f : g.grouped) {
+    for (const auto& b : g.grouped) {
+        const ovfcc_gather_fold& f = b.fold;
         OPENVINO_ASSERT(!blobs, "MI355X: a model with grouped matrix products has no blob form");
         GroupedLaunch l;
+        l.gather = b.gather;
         l.name = g.ops[(size_t)f.root]->get_friendly_name();
         auto param_index = [&](int id, const char* what) {
             OPENVINO_ASSERT(g.nodes[(size_t)id].op == OVFCC_OP_PARAMETER, "MI355X: the ", what, " of ", l.name,
@@ -1435,9 +1476,9 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
         l.a_index = param_index(f.activations, "activations");
         l.with_offsets = f.indices >= 0;
         if (l.with_offsets)
-            l.offsets_index = param_index(f.indices, "offsets");
+            l.offsets_index = param_index(f.indices, b.gather ? "expert indices" : "offsets");
         const auto rs = results_of(f.root);
-        OPENVINO_ASSERT(rs.size() == 1, "MI355X: a grouped matrix product must feed exactly one model output");
+        OPENVINO_ASSERT(rs.size() == 1, "MI355X: a grouped or routed matrix product must feed exactly one model output");
         l.result_index = rs[0];
         fed[rs[0]] = true;
         l.K = f.desc.K;
