@@ -257,6 +257,15 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* req, const ovfcc_group_item* item
 int ovfcc_grouped_matmul_device(ovfcc_request* req, const ovfcc_weights* const* groups, int n_groups, const void* a_dev,
                                 const int32_t* offsets, int64_t rows, void* y_dev);
 
+/* The 2-D x 3-D form with the offsets in device memory, where the kernel that sorted the rows by group leaves them:
+ * the slices of the grouped launch are cut by a kernel on the request's stream and the call never waits for it.
+ * Needs tiled 4-bit groups of one scalar zero-point that the grouped prefill kernel runs (N % 256 == 0), at most 64
+ * of them; otherwise OVFCC_EUNSUPPORTED (pass the offsets in host memory).  The host cannot check what it does not
+ * read: an offset below its predecessor or above `rows` is taken as that bound (the group loses rows, nothing is
+ * read or written outside A and Y). */
+int ovfcc_grouped_matmul_offsets_device(ovfcc_request* req, const ovfcc_weights* const* groups, int n_groups,
+                                        const void* a_dev, const int32_t* offsets_dev, int64_t rows, void* y_dev);
+
 /* GatherMatmulCompressed (src/common/transformations/include/ov_ops/gather_matmul.hpp:17-41,
  * gather_matmul_compressed.hpp:17-33; shapes src/common/transformations/src/ov_ops/gather_matmul.cpp:38-130; CPU
  * executor src/plugins/intel_cpu/src/nodes/executors/dnnl/dnnl_gathermatmul_executor.cpp:470-600): the expert

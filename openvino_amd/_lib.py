@@ -21,7 +21,7 @@ DYNQUANT_PER_GROUP = 32                                                # OVFCC_D
 SYMBOLS = [
     "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_glu", "ovfcc_weights_export_size", "ovfcc_weights_export", "ovfcc_weights_import", "ovfcc_weights_destroy",
     "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
-    "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_device_static", "ovfcc_fc_run_grouped_device", "ovfcc_grouped_matmul_device", "ovfcc_gather_matmul_device", "ovfcc_gather_matmul_routed_device", "ovfcc_moe_device", "ovfcc_moe_routed_device", "ovfcc_bench_grouped", "ovfcc_request_sync", "ovfcc_request_force_kernel",
+    "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_device_static", "ovfcc_fc_run_grouped_device", "ovfcc_grouped_matmul_device", "ovfcc_grouped_matmul_offsets_device", "ovfcc_gather_matmul_device", "ovfcc_gather_matmul_routed_device", "ovfcc_moe_device", "ovfcc_moe_routed_device", "ovfcc_bench_grouped", "ovfcc_request_sync", "ovfcc_request_force_kernel",
     "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
     "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_memcpy_d2d", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_desc_validate", "ovfcc_env_reload", "ovfcc_tiled_sizes",
     "ovfcc_repack_host", "ovfcc_unrepack_host", "ovfcc_unpack_u4", "ovfcc_unpack_i4", "ovfcc_last_error",
@@ -144,6 +144,7 @@ def load() -> ctypes.CDLL:
         "ovfcc_fc_run_device_static": (ci, [vp, vp, vp, vp, i64]),
         "ovfcc_fc_run_grouped_device": (ci, [vp, ctypes.POINTER(GroupItem), ci]),
         "ovfcc_grouped_matmul_device": (ci, [vp, pp, ci, vp, ctypes.POINTER(ctypes.c_int32), i64, vp]),
+        "ovfcc_grouped_matmul_offsets_device": (ci, [vp, pp, ci, vp, vp, i64, vp]),
         "ovfcc_gather_matmul_device": (ci, [vp, pp, ci, vp, ci, ctypes.POINTER(ctypes.c_int32), i64, ci, vp]),
         "ovfcc_moe_device": (ci, [vp, pp, pp, ci, vp, vp, ctypes.POINTER(ctypes.c_int32), i64, ci, vp]),
         "ovfcc_gather_matmul_routed_device": (ci, [vp, pp, ci, vp, ci, vp, i64, ci, vp]),

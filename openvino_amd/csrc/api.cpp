@@ -1538,6 +1538,49 @@ int ovfcc_grouped_matmul_device(ovfcc_request* r, const ovfcc_weights* const* gr
     return ovfcc_fc_run_grouped_device(r, items.data(), (int)items.size());
 }
 
+int ovfcc_grouped_matmul_offsets_device(ovfcc_request* r, const ovfcc_weights* const* groups, int n_groups,
+                                        const void* a_dev, const int32_t* offsets_dev, int64_t rows, void* y_dev) {
+    if (!r || !groups || n_groups <= 0 || rows < 0 || !offsets_dev)
+        return fail(OVFCC_EINVAL, "bad grouped-matmul arguments");
+    if (!groups[0])
+        return fail(OVFCC_EINVAL, "a group's weights are null or belong to another context");
+    bool same_zp = true;
+    int rc = experts_agree(r, groups, n_groups, &same_zp);
+    if (rc || rows == 0)
+        return rc;
+    if (!a_dev || !y_dev)
+        return fail(OVFCC_EINVAL, "A or Y is null");
+    const ovfcc_weights* w0 = groups[0];
+    const int64_t K = w0->desc.K, N_out = out_channels(w0);
+    const size_t out_bytes = w0->desc.out_type == OVFCC_F32 ? 4 : 2;
+    HIP_TRY(hipSetDevice(r->ctx->device));
+    RoutedLaunch L;
+    if (!same_zp || (K * 2) % 16 != 0 || (N_out * out_bytes) % 16 != 0 || !plan_routed(r, w0, rows, n_groups, &L))
+        return fail(OVFCC_EUNSUPPORTED,
+                    "offsets in device memory need tiled 4-bit groups of one scalar zero-point that the grouped prefill "
+                    "kernel runs (N % 256 == 0), at most 64 of them; pass the offsets in host memory instead");
+    const size_t need = sizeof(ovfcc::RoutedHeader) + (size_t)L.n_slices * sizeof(ovfcc::BatchGroupItem) + 256;
+    if (need > r->gather_cap)
+        HIP_TRY(hipStreamSynchronize(r->stream));
+    rc = grow(&r->d_gather, &r->gather_cap, need);
+    if (rc)
+        return rc;
+    char* base = static_cast<char*>(r->d_gather);
+    int* d_tail = reinterpret_cast<int*>(base);  // the header starts 256 bytes in
+    auto* d_header = reinterpret_cast<ovfcc::RoutedHeader*>(base + 256);
+    ovfcc::ExpertPointers ptrs{};
+    for (int g = 0; g < n_groups; ++g)
+        ptrs.w[g] = groups[g]->d_w, ptrs.scale[g] = groups[g]->d_scale, ptrs.zp[g] = groups[g]->d_zp,
+        ptrs.bias[g] = groups[g]->d_bias;
+    const int e = ovfcc::launch_offsets_table(offsets_dev, n_groups, rows, L.cap, ptrs, a_dev, (size_t)K * 2, y_dev,
+                                              (size_t)N_out * out_bytes,
+                                              reinterpret_cast<ovfcc::BatchGroupItem*>(d_header + 1), L.n_slices, d_header,
+                                              d_tail, L.plan.tiles_x, (int)w0->layout.k_blocks, L.plan.n_cus, r->stream);
+    if (e)
+        return hip_fail((hipError_t)e, "offsets kernel launch");
+    return launch_routed(r, L, d_header);
+}
+
 namespace {
 int check_moe(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down, int n_experts,
               const void* x_dev, const void* routing_dev, const void* indices, int64_t M, int top_k, void* y_dev,

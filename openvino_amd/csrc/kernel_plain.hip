@@ -281,6 +281,82 @@ int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts
     return (int)hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------------
+// GroupedMatMul with its offsets in device memory: the slice table of the grouped prefill launch from the
+// cumulative row ends offsets[0 .. n_groups) of rows that are already contiguous per group (group g owns rows
+// [offsets[g-1], offsets[g]) of x and y).  One workgroup.  Offsets are read as the reference's loop reads them
+// (start = previous end), clamped to [previous end, rows], so that a bad value can empty a group but never reach
+// outside the buffers.  tail[0] receives the first row that belongs to no group.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fcc_offsets_table_kernel(const int* __restrict__ offsets, int n_groups, int rows,
+                                                                int cap, ExpertPointers groups, const char* x_base,
+                                                                size_t x_row_bytes, char* y_base, size_t y_row_bytes,
+                                                                BatchGroupItem* __restrict__ table, int n_slices_max,
+                                                                RoutedHeader* __restrict__ header, int* __restrict__ tail,
+                                                                int tiles_x, int kb_total, int n_cus) {
+    __shared__ int start_s[kMaxGroupItems], count_s[kMaxGroupItems], slice_s[kMaxGroupItems];
+    __shared__ int total_s;
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        int start = 0, slice = 0;
+        for (int g = 0; g < n_groups; ++g) {
+            const int end = min(max(offsets[g], start), rows);
+            start_s[g] = start, count_s[g] = end - start, slice_s[g] = slice;
+            slice += (end - start + cap - 1) / cap;
+            start = end;
+        }
+        total_s = slice;
+        *tail = start;
+        *header = routed_header(tiles_x, slice, kb_total, n_cus);
+    }
+    __syncthreads();
+    for (int g = 0; g < n_groups; ++g) {
+        const int count = count_s[g], slices = (count + cap - 1) / cap;
+        const int step = slices ? (count + slices - 1) / slices : 0;  // equal slices of at most cap rows
+        for (int t = tid; t < slices; t += 256) {
+            BatchGroupItem it;
+            it.w = groups.w[g], it.scale = groups.scale[g], it.zp = groups.zp[g], it.bias = groups.bias[g];
+            it.x = x_base + (size_t)(start_s[g] + t * step) * x_row_bytes;
+            it.y = y_base + (size_t)(start_s[g] + t * step) * y_row_bytes;
+            it.M = min(step, count - t * step);
+            it.reserved = 0;
+            table[slice_s[g] + t] = it;
+        }
+    }
+    for (int t = total_s + tid; t < n_slices_max; t += 256) {
+        BatchGroupItem it{};
+        table[t] = it;
+    }
+}
+
+// rows [tail[0], rows) of y, row_bytes each (a multiple of 4): zeros.  One workgroup per row.
+__global__ __launch_bounds__(256) void fcc_zero_tail_kernel(unsigned* __restrict__ y, const int* __restrict__ tail,
+                                                            int row_words) {
+    const int row = blockIdx.x;
+    if (row < tail[0])
+        return;
+    unsigned* p = y + (size_t)row * row_words;
+    for (int i = threadIdx.x; i < row_words; i += 256)
+        p[i] = 0u;
+}
+
+int launch_offsets_table(const int* offsets_dev, int n_groups, int64_t rows, int cap, const ExpertPointers& groups,
+                         const void* x_base, size_t x_row_bytes, void* y_base, size_t y_row_bytes,
+                         BatchGroupItem* table, int n_slices_max, RoutedHeader* header, int* tail, int tiles_x,
+                         int kb_total, int n_cus, void* stream) {
+    if (!offsets_dev || rows <= 0 || rows > ((int64_t)1 << 24) || n_groups < 1 || n_groups > kMaxGroupItems || cap < 1 ||
+        n_slices_max < (rows + cap - 1) / cap + n_groups || !header || !tail || tiles_x < 1 || kb_total < 1 ||
+        n_cus < 1 || (y_row_bytes & 3))
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(fcc_offsets_table_kernel, dim3(1), dim3(256), 0, s, offsets_dev, n_groups, (int)rows, cap, groups,
+                       static_cast<const char*>(x_base), x_row_bytes, static_cast<char*>(y_base), y_row_bytes, table,
+                       n_slices_max, header, tail, tiles_x, kb_total, n_cus);
+    hipLaunchKernelGGL(fcc_zero_tail_kernel, dim3((unsigned)rows), dim3(256), 0, s, static_cast<unsigned*>(y_base), tail,
+                       (int)(y_row_bytes / 4));
+    return (int)hipGetLastError();
+}
+
 int launch_moe_combine(void* y, const void* d, const void* routing, const int* pos, int rows, int top_k, int H,
                        int d_f32, int out_f32, void* stream) {
     if (rows <= 0)

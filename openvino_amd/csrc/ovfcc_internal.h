@@ -234,6 +234,13 @@ int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts
                      const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
                      size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
                      RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream);
+// GroupedMatMul with offsets in device memory: table[0 .. n_slices_max) and *header as for launch_moe_route, from
+// cumulative row ends over rows that are already contiguous per group; rows of y from the last offset on are
+// zeroed; tail: one int of scratch.
+int launch_offsets_table(const int* offsets_dev, int n_groups, int64_t rows, int cap, const ExpertPointers& groups,
+                         const void* x_base, size_t x_row_bytes, void* y_base, size_t y_row_bytes,
+                         BatchGroupItem* table, int n_slices_max, RoutedHeader* header, int* tail, int tiles_x,
+                         int kb_total, int n_cus, void* stream);
 int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);

@@ -301,10 +301,19 @@ class InferRequest:
         check(self.device.lib.ovfcc_grouped_matmul_device(self.handle, arr, len(groups), ctypes.c_void_p(a_ptr), off,
                                                           rows, ctypes.c_void_p(y_ptr)))
 
+    def grouped_matmul_offsets_device(self, groups: Sequence[CompressedWeights], a_ptr: int, offsets_ptr: int,
+                                      rows: int, y_ptr: int) -> None:
+        """The 2-D x 3-D form with the offsets int32 [G] in device memory at offsets_ptr."""
+        arr = (ctypes.c_void_p * len(groups))(*[w.handle for w in groups])
+        check(self.device.lib.ovfcc_grouped_matmul_offsets_device(self.handle, arr, len(groups), ctypes.c_void_p(a_ptr),
+                                                                  ctypes.c_void_p(offsets_ptr), rows, ctypes.c_void_p(y_ptr)))
+
     def grouped_matmul(self, groups: Sequence[CompressedWeights], A: np.ndarray,
-                       offsets: Optional[np.ndarray] = None, y_fill: Optional[float] = None) -> np.ndarray:
+                       offsets: Optional[np.ndarray] = None, y_fill: Optional[float] = None,
+                       device_offsets: bool = False) -> np.ndarray:
         """Host convenience: with offsets A float16 [rows, K] -> Y [rows, N_out]; without, A [G, M, K] -> Y [G, M, N_out].
-        y_fill: Y is preset to this value (the call must overwrite all of it)."""
+        y_fill: Y is preset to this value (the call must overwrite all of it); device_offsets: the offsets are uploaded
+        and the entry point that reads them on the device is called."""
         A = np.ascontiguousarray(A, dtype=np.float16)
         w = groups[0]
         want = 2 if offsets is not None else 3
@@ -322,8 +331,18 @@ class InferRequest:
             dev.upload(a_ptr, A)
             if y_fill is not None:
                 dev.upload(y_ptr, np.full(out_shape, y_fill, dt))
-            self.grouped_matmul_device(groups, a_ptr, offsets, rows, y_ptr)
-            self.sync()
+            if device_offsets:
+                off = np.ascontiguousarray(offsets, dtype=np.int32)
+                o_ptr = dev.malloc(max(off.nbytes, 16))
+                try:
+                    dev.upload(o_ptr, off)
+                    self.grouped_matmul_offsets_device(groups, a_ptr, o_ptr, rows, y_ptr)
+                    self.sync()
+                finally:
+                    dev.free(o_ptr)
+            else:
+                self.grouped_matmul_device(groups, a_ptr, offsets, rows, y_ptr)
+                self.sync()
             return dev.download(y_ptr, out_shape, dt)
         finally:
             dev.free(a_ptr)

@@ -161,3 +161,54 @@ def test_expert_layer_of_the_benchmarks_proportions(oracle, dev, req):
     finally:
         for w in ws:
             w.close()
+
+
+@pytest.mark.parametrize("tpe,tail", [([65, 64, 54, 71, 70, 70, 56, 62], 0), ([0, 200, 0, 0, 3, 0, 129, 0], 9),
+                                      ([1, 1, 1, 1, 1, 1, 1, 1], 0), ([0, 0, 0, 0, 0, 0, 0, 0], 5)])
+def test_offsets_in_device_memory(oracle, dev, req, tpe, tail):
+    """The same op with the offsets read on the device: against the oracle, and against the host-offset call; rows
+    beyond the last offset are zeros; nothing waits for the stream in between."""
+    G, N, K = 8, 1024, 512
+    cases, ws = make_groups(dev, 8500, G, N, K, "u4", "scalar", 128)
+    groups = [args_of(c) for c in cases]
+    offsets = np.cumsum(tpe).astype(np.int32)
+    rows = int(offsets[-1]) + tail
+    a = np.random.default_rng(8501).standard_normal((rows, K)).astype(np.float16)
+    try:
+        y = req.grouped_matmul(ws, a, offsets, y_fill=3.0, device_offsets=True)
+        say(f"   tokens {tpe} tail {tail}: {req.last_kernel()['name']}")
+        assert req.last_kernel()["name"] == "fcc_prefill_async_grouped_w4"
+        assert np.all(y[int(offsets[-1]):] == 0)
+        check_parity(oracle, y, oracle.grouped_matmul_reference(a, groups, offsets), K, f"device offsets {tpe}",
+                     output_rounding_slack=True)
+        host = req.grouped_matmul(ws, a, offsets, y_fill=3.0)
+        assert oracle.rel_l2(y.astype(np.float32), host.astype(np.float32)) < 2e-3 if rows else True
+        assert np.array_equal(req.grouped_matmul(ws, a, offsets, device_offsets=True).view(np.uint8), y.view(np.uint8))
+    finally:
+        for w in ws:
+            w.close()
+
+
+def test_device_offsets_out_of_order_lose_rows_but_stay_inside(oracle, dev, req):
+    """What the host form refuses cannot be checked without reading the offsets: a value below its predecessor or
+    above the row count is taken as that bound."""
+    G, N, K = 4, 512, 256
+    cases, ws = make_groups(dev, 8600, G, N, K, "i4", "empty", 128)
+    groups = [args_of(c) for c in cases]
+    a = np.random.default_rng(8601).standard_normal((40, K)).astype(np.float16)
+    try:
+        y = req.grouped_matmul(ws, a, np.array([10, 5, 30, 99], np.int32), y_fill=2.0, device_offsets=True)
+        clamped = np.array([10, 10, 30, 40], np.int32)
+        check_parity(oracle, y, oracle.grouped_matmul_reference(a, groups, clamped), K, "clamped", output_rounding_slack=True)
+        # 8-bit groups have no launch that reads its slices from memory
+        c8, w8 = make_groups(dev, 8610, G, N, K, "u8", "full", K)
+        try:
+            with pytest.raises(fc.OvfccError) as e:
+                req.grouped_matmul(w8, a, clamped, device_offsets=True)
+            assert e.value.code == _lib.EUNSUPPORTED
+        finally:
+            for w in w8:
+                w.close()
+    finally:
+        for w in ws:
+            w.close()
