@@ -17,7 +17,10 @@
 // sums, 3 (4 C + 4) for the weights), which bound the workgroup at 8 and 16 waves for C = 4 and 2.  A node whose
 // channel-major tables were laid out for eight k-blocks per wave runs with two waves per table row, four k-blocks
 // each.  With a gated linear unit a workgroup visits the gate tile and the up tile of 16 channels in turn; the
-// waves that add the sums keep the gate values in a register for the visit between.
+// waves that add the sums keep the gate values in a register for the visit between.  Where 16 rows x K do not fit
+// (K = 14336), K is cut in parts across blockIdx.z -- every workgroup then takes a share of each table row's slots --
+// the parts leave f32 partial sums in a workspace and a second, small launch adds them: two launches and plain
+// stores instead of the tickets and fences of a split-K epilogue inside one.
 //
 // LDS slice of a wave, in 16-byte units: row r, slot s (k-block w + NWT s), chunk c of the k-block's 16 sits at
 // r (16 C) + 16 s + (c ^ r): the sixteen rows that one operand read touches lie in sixteen different bank groups.
@@ -58,13 +61,17 @@ struct TileRegs {
 // C: k-blocks per wave (the node's channel-major tables may be laid out for 2 C: then two waves share a table
 // row, `parts` = k_blocks / c_table of them side by side, and a wave takes half of its slots); ZP_TABLE: zero-points
 // per (channel, group); MULTI: workgroups visit more than one channel tile; GLU: tiles 2 j and 2 j + 1 hold the gate
-// and up channels 16 j .. of a gated linear unit and a workgroup visits them one after the other
-template <int C, bool ZP_TABLE, bool MULTI, bool GLU>
+// and up channels 16 j .. of a gated linear unit and a workgroup visits them one after the other; KSPLIT: the
+// workgroups of one blockIdx.z take the same share of every table row's slots (K cut in gridDim.z parts, so that a
+// part's 16 rows of activations fit in LDS) and leave f32 partial sums [gridDim.z][16 gridDim.y][N] without bias
+// in `y`, which fcc_gemv16_sum_kernel adds up
+template <int C, bool ZP_TABLE, bool MULTI, bool GLU, bool KSPLIT>
 __global__ __launch_bounds__(C == 4 ? 512 : 1024) void fcc_gemv16_kernel(
     const uint4_t* __restrict__ wt, const half_t* __restrict__ scale_cm, const uint8_t* __restrict__ zp_cm,
     const half_t* __restrict__ x, const half_t* __restrict__ bias, void* __restrict__ y, int M, int N, int K,
     int kb_total, int parts, int c_table, int n_tiles, int zp_const, int out_f32, int red_bufs, int glu) {
     static_assert(!GLU || MULTI, "a gated linear unit takes two visits");
+    static_assert(!GLU || !KSPLIT, "partial sums cannot pass through a gated linear unit");
     constexpr int kWaveBytes = C * 4096;   // 16 rows x C k-blocks x 256 bytes
     constexpr int kDepth = MULTI ? 3 : 1;  // visits whose weights are in registers or on their way
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];  // [waves] slices | partial sums
@@ -74,9 +81,10 @@ __global__ __launch_bounds__(C == 4 ? 512 : 1024) void fcc_gemv16_kernel(
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int waves = blockDim.x >> 6;  // parts * c_table / C
+    const int waves = blockDim.x >> 6;  // parts * c_table / C (/ gridDim.z with KSPLIT)
     const int part = wave % parts;      // the table row this wave reads: k-blocks part, part + parts, ...
-    const int slot0 = wave / parts * C; // ... of which it takes slots slot0 .. slot0 + C - 1
+    // ... of which it takes slots slot0 .. slot0 + C - 1
+    const int slot0 = (wave / parts + (KSPLIT ? (int)blockIdx.z * ((int)(blockDim.x >> 6) / parts) : 0)) * C;
     const int col = lane & 15;
     const int kq = lane >> 4;
     const int m0 = 16 * blockIdx.y;
@@ -244,8 +252,13 @@ __global__ __launch_bounds__(C == 4 ? 512 : 1024) void fcc_gemv16_kernel(
 #pragma unroll 4
                 for (int w = 0; w < waves; ++w)
                     s += red[w * 256 + at];
-                s = s * 0x1p24f + (float)__builtin_bit_cast(half_t, (uint16_t)cur.bias);
                 const int row = m0 + 4 * g + kq;
+                if constexpr (KSPLIT) {
+                    // rows >= M of the last row tile are stored too: the partial buffer has whole row tiles
+                    static_cast<float*>(y)[((size_t)blockIdx.z * (16 * gridDim.y) + row) * N + t * 16 + col] = s * 0x1p24f;
+                    continue;
+                }
+                s = s * 0x1p24f + (float)__builtin_bit_cast(half_t, (uint16_t)cur.bias);
                 if constexpr (GLU) {
                     if (t & 1) {
                         if (row < M)
@@ -278,20 +291,41 @@ __global__ __launch_bounds__(C == 4 ? 512 : 1024) void fcc_gemv16_kernel(
     }
 }
 
+// y[m][n] = sum over z of partial[z][m][n] + bias[n], in the order of z; partial has rows_pad rows per part
+__global__ __launch_bounds__(256) void fcc_gemv16_sum_kernel(const float* __restrict__ partial, const half_t* __restrict__ bias,
+                                                             void* __restrict__ y, int M, int N, int rows_pad, int parts,
+                                                             int out_f32) {
+    const int i = blockIdx.x * 256 + threadIdx.x;  // four neighbouring channels of one row
+    const int per_row = N / 4;
+    if (i >= M * per_row)
+        return;
+    const int m = i / per_row, n = (i - m * per_row) * 4;
+    float4_t s = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < parts; ++z)
+        s += *reinterpret_cast<const float4_t*>(partial + ((size_t)z * rows_pad + m) * N + n);
+    const float v[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        store_out(y, (size_t)m * N + n + j, v[j] + (bias ? (float)bias[n + j] : 0.f), out_f32);
+}
+
 // Dynamic LDS: every wave hands over 16 rows of its c k-blocks and leaves 16 x 16 partial sums per buffer.
 size_t gemv16_lds_bytes(int c, int waves, int red_bufs) {
     return (size_t)waves * c * 4096 + (size_t)red_bufs * waves * 1024;
 }
 
-// k-blocks per wave that the kernel runs a node with: tables laid out for eight are read by two waves per row
-int gemv16_kblocks_per_wave(int c_table) {
+// k-blocks per wave that the kernel runs a node with: tables laid out for eight are read by two waves per row; with
+// K cut in split_k parts a wave takes its share of the row's slots
+int gemv16_kblocks_per_wave(int c_table, int split_k) {
+    if (split_k > 1)
+        return c_table / split_k;
     return c_table == 2 ? 2 : 4;
 }
 
-template <int C, bool ZPT, bool MULTI, bool GLU>
+template <int C, bool ZPT, bool MULTI, bool GLU, bool KSPLIT>
 static int launch_gemv16_impl(const FcDeviceArgs& a, const LaunchPlan& p, int red_bufs, hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_gemv16_kernel<C, ZPT, MULTI, GLU>;
+    auto kern = fcc_gemv16_kernel<C, ZPT, MULTI, GLU, KSPLIT>;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -300,10 +334,16 @@ static int launch_gemv16_impl(const FcDeviceArgs& a, const LaunchPlan& p, int re
             return (int)e;
         attr_set = true;
     }
-    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], 1), dim3(p.block), p.dynamic_lds, s, (const uint4_t*)a.w,
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(p.block), p.dynamic_lds, s, (const uint4_t*)a.w,
                        (const half_t*)a.scale_cm, (const uint8_t*)a.zp_cm, (const half_t*)a.x, (const half_t*)a.bias,
-                       a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)(L.k_blocks / L.gemv_c), L.gemv_c,
-                       (int)L.n_tiles, L.zp_const, a.out_f32, red_bufs, L.glu);
+                       KSPLIT ? (void*)a.workspace : a.y, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
+                       (int)(L.k_blocks / L.gemv_c), L.gemv_c, (int)L.n_tiles, L.zp_const, a.out_f32, red_bufs, L.glu);
+    if constexpr (KSPLIT) {
+        const int64_t quads = a.M * (a.N / 4);
+        hipLaunchKernelGGL(fcc_gemv16_sum_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
+                           (const float*)a.workspace, (const half_t*)a.bias, a.y, (int)a.M, (int)a.N, (int)(16 * p.grid[1]),
+                           (int)p.grid[2], a.out_f32);
+    }
     return (int)hipGetLastError();
 }
 
@@ -316,11 +356,17 @@ int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
         (L.zp_table && !a.zp_cm) || a.M < 1 || a.M > kDecodeMaxRows || (ct != 2 && ct != 4 && ct != 8) || L.k_blocks % ct != 0 ||
         p.gemv_c != ct || (!L.zp_table && (L.zp_const < 0 || L.zp_const > 255)) || (L.glu && (L.n_tiles & 1)))
         return (int)hipErrorInvalidValue;
-    const int c = gemv16_kblocks_per_wave(ct);
-    const int waves = (int)(L.k_blocks / c);
+    const int split = p.split_k;
+    if (split < 1 || (split > 1 && (L.glu || ct % split != 0 || !a.workspace || (a.N & 3) ||
+                                    p.workspace_bytes != (size_t)split * 16 * p.grid[1] * a.N * sizeof(float))))
+        return (int)hipErrorInvalidValue;
+    const int c = gemv16_kblocks_per_wave(ct, split);
+    if (c != 2 && c != 4)
+        return (int)hipErrorInvalidValue;
+    const int waves = (int)(L.k_blocks / c / split);
     const int64_t units = L.glu ? L.n_tiles / 2 : L.n_tiles;  // what a workgroup visits in one go: tiles or tile pairs
     if (waves < 1 || waves > (c == 4 ? 8 : 16) || p.block != 64u * waves || p.grid[0] < 1 || (int64_t)p.grid[0] > units ||
-        p.grid[1] != (unsigned)((a.M + 15) / 16) || p.grid[2] != 1)
+        p.grid[1] != (unsigned)((a.M + 15) / 16) || p.grid[2] != (unsigned)split)
         return (int)hipErrorInvalidValue;
     const int red_bufs = (L.glu || (int64_t)p.grid[0] < units) ? 2 : 1;
     if (p.dynamic_lds != gemv16_lds_bytes(c, waves, red_bufs) || p.dynamic_lds > 160 * 1024 - 64 ||
@@ -330,7 +376,13 @@ int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     const bool multi = red_bufs == 2;
     auto go = [&](auto zpt, auto mul, auto gl) {
         constexpr bool Z = decltype(zpt)::value, U = decltype(mul)::value, G = decltype(gl)::value;
-        return c == 4 ? launch_gemv16_impl<4, Z, U, G>(a, p, red_bufs, s) : launch_gemv16_impl<2, Z, U, G>(a, p, red_bufs, s);
+        if constexpr (!G) {
+            if (split > 1)
+                return c == 4 ? launch_gemv16_impl<4, Z, U, false, true>(a, p, red_bufs, s)
+                              : launch_gemv16_impl<2, Z, U, false, true>(a, p, red_bufs, s);
+        }
+        return c == 4 ? launch_gemv16_impl<4, Z, U, G, false>(a, p, red_bufs, s)
+                      : launch_gemv16_impl<2, Z, U, G, false>(a, p, red_bufs, s);
     };
     const std::true_type yes{};
     const std::false_type no{};

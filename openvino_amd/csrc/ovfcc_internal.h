@@ -159,8 +159,9 @@ int launch_gemv(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 // dynamic LDS of the 16-row kernel: c k-blocks per wave, `waves` waves, one or two buffers of partial sums
 size_t gemv16_lds_bytes(int c, int waves, int red_bufs);
-// k-blocks per wave that the 16-row kernel runs a node with, given those of the node's channel-major tables
-int gemv16_kblocks_per_wave(int c_table);
+// k-blocks per wave that the 16-row kernel runs a node with, given those of the node's channel-major tables and the
+// number of parts K is cut in
+int gemv16_kblocks_per_wave(int c_table, int split_k = 1);
 // dynamic LDS of the matrix-vector kernel: c k-blocks per wave, m rows, `waves` waves per workgroup
 size_t gemv_lds_bytes(int c, int m, int waves);
 // [N/16][groups][16] scales f16 (and zero-points u8, or null) -> channel-major [N/16][16][groups]

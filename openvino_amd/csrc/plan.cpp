@@ -20,7 +20,7 @@ namespace ovfcc {
 //            workgroup or wave), OVFCC_DECODE_XLDS = 0 | 1 (activations via LDS), OVFCC_DECODE_BATCH = 0 | 1
 //            (small-batch kernel instead of the streaming kernel), OVFCC_GEMV = 0 | 1, OVFCC_GEMV_C = 2 | 4 | 8,
 //            OVFCC_GEMV16 = 0 | 1 (the 16-row kernel with stationary activations for 5-48 rows),
-//            OVFCC_GEMV16_GRID = n (its workgroups per row tile),
+//            OVFCC_GEMV16_GRID = n (its workgroups per row tile), OVFCC_GEMV16_SPLIT = 1 | 2 | 4 | 8 (parts it cuts K in),
 //            OVFCC_PREFILL_{DIRECT, ASYNC, WIDE, BIG, TAIL} = 0 | 1, OVFCC_PREFILL_ROWS = 64 | 128,
 //            OVFCC_MOE_HOST_ROUTING = 1;
 //   logging: OVFCC_VERBOSE = 1 (one line per launch on stderr), 2 (also weights and requests as they come and go).
@@ -33,7 +33,7 @@ struct EnvEntry {
 };
 EnvEntry g_env[] = {EnvEntry("OVFCC_DECODE_WAVES"),   EnvEntry("OVFCC_DECODE_RT"),      EnvEntry("OVFCC_DECODE_XLDS"),
                     EnvEntry("OVFCC_DECODE_BATCH"),   EnvEntry("OVFCC_GEMV"),           EnvEntry("OVFCC_GEMV_C"),
-                    EnvEntry("OVFCC_GEMV16"),         EnvEntry("OVFCC_GEMV16_GRID"),
+                    EnvEntry("OVFCC_GEMV16"),         EnvEntry("OVFCC_GEMV16_GRID"),    EnvEntry("OVFCC_GEMV16_SPLIT"),
                     EnvEntry("OVFCC_PREFILL_DIRECT"), EnvEntry("OVFCC_PREFILL_ASYNC"),  EnvEntry("OVFCC_PREFILL_WIDE"),
                     EnvEntry("OVFCC_PREFILL_BIG"),    EnvEntry("OVFCC_PREFILL_TAIL"),   EnvEntry("OVFCC_PREFILL_ROWS"),
                     EnvEntry("OVFCC_MOE_HOST_ROUTING"), EnvEntry("OVFCC_VERBOSE")};
@@ -169,44 +169,62 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
     // keeps its row tile of the activations and walks channel tiles; the grid is as many workgroups as the chip
     // holds at once, rounded so that all of them visit the same number of tiles.
     auto plan_gemv16 = [&]() -> bool {
-        if (a.M <= 4 || a.M > kDecodeMaxRows || !a.scale_cm || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 ||
-            force_split > 0 || L.gemv_c == 0 || (L.glu && (L.n_tiles & 1)) || env_int("OVFCC_GEMV16", 1) == 0 ||
-            env_int("OVFCC_DECODE_BATCH", -1) >= 0)
-            return false;
-        // the kernel's registers allow 8 and 16 waves per compute unit with 4 and 2 k-blocks per wave
-        const int c = gemv16_kblocks_per_wave(L.gemv_c), waves = (int)(L.k_blocks / c);
-        const int cu_waves = c == 4 ? 8 : 16;
-        if (waves > cu_waves || L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 30))
+        if (a.M <= 4 || a.M > kDecodeMaxRows || !a.scale_cm || L.bits != 4 || L.groups_per_kblock != 1 ||
+            L.kblocks_per_group != 1 || force_split > 0 || L.gemv_c == 0 || (L.glu && (L.n_tiles & 1)) ||
+            env_int("OVFCC_GEMV16", 1) == 0 ||
+            env_int("OVFCC_DECODE_BATCH", -1) >= 0 || L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 30))
             return false;
         const size_t lds_limit = 160 * 1024 - 64;
-        const size_t lds2 = gemv16_lds_bytes(c, waves, 2);
         const int64_t rows = (a.M + 15) / 16;
         const int64_t units = L.glu ? L.n_tiles / 2 : L.n_tiles;  // visited in one go: tiles, or pairs of gate and up tile
-        const int64_t per_cu = std::max<int64_t>(1, std::min<int64_t>((int64_t)(160 * 1024 / lds2), cu_waves / waves));
-        const int64_t at_once = std::max<int64_t>(1, (int64_t)n_cus * per_cu / rows);
-        int64_t visits = (units + at_once - 1) / at_once;
-        int64_t grid = (units + visits - 1) / visits;
-        const int grid_env = env_int("OVFCC_GEMV16_GRID", 0);
-        if (grid_env > 0) {
-            grid = std::min<int64_t>(grid_env, units);
-            visits = (units + grid - 1) / grid;
+        // K whole where 16 rows x K fit in LDS and the waves in the register file; else cut in 2, 4 or 8 parts whose
+        // partial sums a second launch adds (OVFCC_GEMV16_SPLIT picks the number of parts)
+        const int split_env = env_int("OVFCC_GEMV16_SPLIT", 0);
+        for (int split : {1, 2, 4, 8}) {
+            if (split_env > 0 && split != split_env)
+                continue;
+            // (up to 16 rows the parts and their second launch only tie with the small-batch kernel: down projection
+            // 12.8 against 12.7 us; from 17 rows on they are ahead, 16.2 against 21.5 us at 32 rows)
+            if (split > 1 && (L.glu || L.gemv_c % split != 0 || (a.N & 3) || (a.M <= 16 && split_env <= 0)))
+                continue;
+            // the kernel's registers allow 8 and 16 waves per compute unit with 4 and 2 k-blocks per wave
+            const int c = gemv16_kblocks_per_wave(L.gemv_c, split);
+            if (c != 2 && c != 4)
+                continue;
+            const int waves = (int)(L.k_blocks / c / split);
+            const int cu_waves = c == 4 ? 8 : 16;
+            if (waves < 1 || waves > cu_waves)
+                continue;
+            const size_t lds2 = gemv16_lds_bytes(c, waves, 2);
+            const int64_t per_cu = std::max<int64_t>(1, std::min<int64_t>((int64_t)(160 * 1024 / lds2), cu_waves / waves));
+            const int64_t at_once = std::max<int64_t>(1, (int64_t)n_cus * per_cu / (rows * split));
+            int64_t visits = (units + at_once - 1) / at_once;
+            int64_t grid = (units + visits - 1) / visits;
+            const int grid_env = env_int("OVFCC_GEMV16_GRID", 0);
+            if (grid_env > 0) {
+                grid = std::min<int64_t>(grid_env, units);
+                visits = (units + grid - 1) / grid;
+            }
+            const size_t lds = gemv16_lds_bytes(c, waves, (L.glu || grid < units) ? 2 : 1);
+            if (lds > lds_limit)
+                continue;
+            p.gemv16 = true;
+            p.gemv_c = L.gemv_c;
+            p.split_k = split;
+            p.kblocks_per_split = (int)(L.k_blocks / split);
+            p.tiles_per_group = (int)(visits * (L.glu ? 2 : 1));
+            p.grid[0] = (unsigned)grid;
+            p.grid[1] = (unsigned)rows;
+            p.grid[2] = (unsigned)split;
+            p.block = 64u * waves;
+            p.tile_m = 16;
+            p.tile_n = 16;
+            p.dynamic_lds = (unsigned)lds;
+            p.workspace_bytes = split > 1 ? (size_t)split * 16 * rows * a.N * sizeof(float) : 0;
+            p.name = "fcc_gemv16_w4";
+            return true;
         }
-        const size_t lds = gemv16_lds_bytes(c, waves, (L.glu || grid < units) ? 2 : 1);
-        if (lds > lds_limit)
-            return false;
-        p.gemv16 = true;
-        p.gemv_c = L.gemv_c;
-        p.split_k = 1;
-        p.kblocks_per_split = (int)L.k_blocks;
-        p.tiles_per_group = (int)(visits * (L.glu ? 2 : 1));
-        p.grid[0] = (unsigned)grid;
-        p.grid[1] = (unsigned)rows;
-        p.block = 64u * waves;
-        p.tile_m = 16;
-        p.tile_n = 16;
-        p.dynamic_lds = (unsigned)lds;
-        p.name = "fcc_gemv16_w4";
-        return true;
+        return false;
     };
     if (kernel == OVFCC_KERNEL_PLAIN) {
         if (a.M > 65535)

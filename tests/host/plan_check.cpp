@@ -16,7 +16,7 @@ int launch_decode(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_batch(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_gemv(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_gemv16(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int gemv16_kblocks_per_wave(int c_table) { return c_table == 2 ? 2 : 4; }
+int gemv16_kblocks_per_wave(int c_table, int split_k) { return split_k > 1 ? c_table / split_k : (c_table == 2 ? 2 : 4); }
 size_t gemv16_lds_bytes(int c, int waves, int red_bufs) { return (size_t)waves * c * 4096 + (size_t)red_bufs * waves * 1024; }
 int launch_prefill(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
 int launch_prefill_wide(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
@@ -88,8 +88,9 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
     CHECK(p.block >= 64 && p.block <= 1024 && p.block % 64 == 0, "%s block=%u", what, p.block);
     CHECK(p.dynamic_lds <= 160 * 1024, "%s lds=%u", what, p.dynamic_lds);
     CHECK(p.split_k >= 1, "%s", what);
-    CHECK((p.split_k > 1) == (p.workspace_bytes > 0) && (p.split_k > 1) == (p.counter_count > 0), "%s ws=%zu counters=%zu split=%d",
-          what, p.workspace_bytes, p.counter_count, p.split_k);
+    // (the 16-row kernel's parts meet in a second launch: a workspace, no counters)
+    CHECK((p.split_k > 1) == (p.workspace_bytes > 0) && (p.gemv16 ? p.counter_count == 0 : (p.split_k > 1) == (p.counter_count > 0)),
+          "%s ws=%zu counters=%zu split=%d", what, p.workspace_bytes, p.counter_count, p.split_k);
     if (p.kernel == OVFCC_KERNEL_PLAIN) {
         CHECK(!L.tiled && p.grid[0] == (unsigned)a.N_out && p.grid[1] == (unsigned)M, "%s", what);
         return;
@@ -111,19 +112,23 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
             CHECK((int64_t)p.grid[0] * per_wg == L.n_tiles && p.grid[1] == 1 && p.split_k == 1, "%s", what);
             CHECK(p.dynamic_lds == ovfcc::gemv_lds_bytes(c, (int)M, nw) && p.dynamic_lds <= 150 * 1024, "%s lds=%u", what, p.dynamic_lds);
         } else if (p.gemv16) {
-            const int c = ovfcc::gemv16_kblocks_per_wave(p.gemv_c);
+            const int c = ovfcc::gemv16_kblocks_per_wave(p.gemv_c, p.split_k);
             const int64_t units = L.glu ? L.n_tiles / 2 : L.n_tiles;
             const int per_unit = L.glu ? 2 : 1;
             CHECK(M > 4 && M <= 48 && L.bits == 4 && L.groups_per_kblock == 1 && L.kblocks_per_group == 1 && p.gemv_c == L.gemv_c &&
-                      (!L.glu || L.n_tiles % 2 == 0),
+                      (!L.glu || (L.n_tiles % 2 == 0 && p.split_k == 1)),
                   "%s", what);
-            CHECK(kb % c == 0 && nw == kb / c && nw <= (c == 4 ? 8 : 16), "%s c=%d nw=%d", what, c, nw);
+            CHECK((c == 2 || c == 4) && kb % (c * p.split_k) == 0 && nw == kb / c / p.split_k && nw <= (c == 4 ? 8 : 16) &&
+                      p.gemv_c % p.split_k == 0,
+                  "%s c=%d nw=%d", what, c, nw);
             CHECK(rt % per_unit == 0 && (int64_t)p.grid[0] <= units && (int64_t)p.grid[0] * (rt / per_unit) >= units &&
-                      (int64_t)p.grid[0] * (rt / per_unit - 1) < units && p.grid[1] == (unsigned)((M + 15) / 16) && p.split_k == 1,
+                      (int64_t)p.grid[0] * (rt / per_unit - 1) < units && p.grid[1] == (unsigned)((M + 15) / 16) &&
+                      p.grid[2] == (unsigned)p.split_k,
                   "%s grid=%u visits=%d", what, p.grid[0], rt);
             CHECK(p.dynamic_lds == ovfcc::gemv16_lds_bytes(c, nw, (L.glu || (int64_t)p.grid[0] < units) ? 2 : 1) &&
                       p.dynamic_lds <= 160 * 1024 - 64,
                   "%s lds=%u", what, p.dynamic_lds);
+            CHECK(p.workspace_bytes == (p.split_k > 1 ? (size_t)p.split_k * 16 * p.grid[1] * d.N * sizeof(float) : 0), "%s", what);
         } else if (p.batch) {
             const int mt = (int)(M + 15) / 16;
             CHECK(p.tile_m == 16 * mt && (rt == 1 || rt == 2), "%s", what);

@@ -122,7 +122,7 @@ def test_gemv16_tiny_and_huge_activations(oracle, dev, req):
 @pytest.mark.parametrize("name,N,K", [("q/o", 4096, 4096), ("k/v", 1024, 4096), ("gate/up", 14336, 4096)])
 def test_gemv16_benchmark_nodes(oracle, dev, req, name, N, K):
     """The Llama-3-8B projections whose activations fit in LDS, at the benchmark's row counts, against the oracle on
-    a sample of channels; the down projection (K = 14336) stays with the small-batch kernel."""
+    a sample of channels."""
     c = datagen.make_case(7800 + N, 48, K, N, "i4", 128, "none")
     w = fc.CompressedWeights.from_case(dev, c)
     rng = np.random.default_rng(5)
@@ -165,9 +165,66 @@ def test_gemv16_gated_linear_unit(oracle, dev, req, monkeypatch, wt, zt, N, K, C
         w.close()
 
 
+# (w_type, zp_type, N, K, k-blocks per wave of the tables, parts, workgroups per row tile forced, bias, output)
+SPLIT_SHAPES = [
+    ("u4", "u4", 64, 1024, 8, 4, 0, True, "f16"),     # tables for 1 wave of 8: four parts of one wave with 2 k-blocks
+    ("u4", "u4", 272, 1024, 8, 2, 5, True, "f32"),    # two parts of one wave with 4; several visits
+    ("i4", "none", 48, 2048, 4, 2, 0, False, "f16"),  # tables for 4 waves of 4: two parts of 4 waves with 2
+    ("u4", "u8", 96, 4096, 8, 4, 2, True, "f16"),     # 4 waves, zero-point table, three visits
+    ("i4", "none", 64, 14336, 8, 4, 0, True, "f16"),  # the down projection's K: 14 waves per part
+    ("u4", "u4", 80, 14336, 8, 4, 3, False, "f32"),   # ... with a zero-point table and two visits
+]
+
+
+@pytest.mark.parametrize("wt,zt,N,K,C,parts,grid,bias,out", SPLIT_SHAPES)
+def test_gemv16_k_in_parts(oracle, dev, req, monkeypatch, wt, zt, N, K, C, parts, grid, bias, out):
+    """K cut in parts across workgroups, partial sums added by a second launch: every row count class, the same bits
+    on every repetition (the parts are added in a fixed order)."""
+    monkeypatch.setenv("OVFCC_GEMV_C", str(C))
+    monkeypatch.setenv("OVFCC_GEMV16_SPLIT", str(parts))
+    if grid:
+        monkeypatch.setenv("OVFCC_GEMV16_GRID", str(grid))
+    c = datagen.make_case(7650 + N + K, 48, K, N, wt, 128, zt, with_bias=bias)
+    w = fc.CompressedWeights.from_case(dev, c, output_type=out)
+    ref = oracle_y(oracle, c)
+    try:
+        for M in (5, 16, 17, 33, 48):
+            say(f"gemv16 parts {wt}/{zt} N={N} K={K} C={C} parts={parts} grid={grid} out={out} M={M}")
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            assert info["name"] == "fcc_gemv16_w4" and info["split_k"] == parts, info
+            assert info["grid"] == (grid or N // 16, (M + 15) // 16, parts), info
+            assert info["block"] == 64 * (K // 128 // (C // parts) // parts), info
+            check_parity(oracle, y, ref[:M], K, f"M={M} {info}", output_rounding_slack=True)
+            assert np.array_equal(req.infer(w, c.x[:M]).view(np.uint8), y.view(np.uint8))
+    finally:
+        w.close()
+
+
+def test_gemv16_down_projection(oracle, dev, req):
+    """The benchmark's down projection (14336 -> 4096) takes the kernel with K in four parts from 17 rows on."""
+    K, N = 14336, 4096
+    c = datagen.make_case(7860, 48, K, N, "i4", 128, "none")
+    w = fc.CompressedWeights.from_case(dev, c)
+    cols = np.sort(np.random.default_rng(6).choice(N, size=256, replace=False))
+    ref = oracle_y(oracle, c, n_index=cols)
+    try:
+        for M in (8, 16, 17, 32, 48):
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            say(f"gemv16 down M={M} {info}")
+            if M <= 16:    # one row tile: the small-batch kernel is as fast and needs one launch
+                assert info["name"] == "fcc_batch_w4", info
+            else:
+                assert info["name"] == "fcc_gemv16_w4" and info["split_k"] == 4 and info["block"] == 64 * 14, info
+            check_parity(oracle, y[:, cols], ref[:M], K, f"down M={M} {info}")
+    finally:
+        w.close()
+
+
 def test_gemv16_leaves_what_does_not_fit(dev, req):
-    """Activations beyond LDS (K = 14336), groups of 64 inputs, 8-bit weights: other kernels."""
-    for wt, zt, N, K, G in (("u4", "none", 64, 14336, 128), ("u4", "u4", 64, 1024, 64), ("u8", "u8", 64, 1024, 128)):
+    """Groups of 64 inputs, 8-bit weights, K whose k-blocks the waves cannot share out (K = 128 x 9): other kernels."""
+    for wt, zt, N, K, G in (("u4", "none", 64, 128 * 9, 128), ("u4", "u4", 64, 1024, 64), ("u8", "u8", 64, 1024, 128)):
         c = datagen.make_case(7900, 8, K, N, wt, G, zt)
         w = fc.CompressedWeights.from_case(dev, c)
         try:
