@@ -518,13 +518,20 @@ def main() -> int:
     per_shape = {}
     for name, (K, N) in datagen.LLAMA3_8B_SHAPES.items():
         hs = [w for n_, w in layers if n_ == name]
-        for Mx in (1, 4, 16, 32):
+        for Mx in (1, 4, 8, 16, 32):
             t = req.bench_layers(hs, x_dev, y_dev, Mx, 2, max(5, args.steps // 5), use_graph=not args.no_graph)
             per = t / max(5, args.steps // 5) / len(hs)
             b = algorithmic_bytes(K, N, Mx)
             per_shape[f"{name}_M{Mx}"] = {"us": per * 1e3, "GBps": b / (per * 1e-3) / 1e9}
         log(f"  {name}: " + ", ".join(f"M={m}: {per_shape[f'{name}_M{m}']['us']:.2f} us "
-                                      f"{per_shape[f'{name}_M{m}']['GBps']:.0f} GB/s" for m in (1, 4, 16, 32)))
+                                      f"{per_shape[f'{name}_M{m}']['GBps']:.0f} GB/s" for m in (1, 4, 8, 16, 32)))
+    # small batches: one block of seven nodes (q, k, v, o, gate, up, down) against its time at one row
+    block_us = {m: sum(per_shape[f"{n_}_M{m}"]["us"] * reps for n_, reps in (("qo", 2), ("kv", 2), ("gate_up", 2), ("down", 1)))
+                for m in (1, 4, 8, 16, 32)}
+    small_batch = {f"M{m}": {"block_us": round(block_us[m], 2), "vs_M1": round(block_us[m] / block_us[1], 3)}
+                   for m in (1, 4, 8, 16, 32)}
+    log("  block of seven nodes: " + ", ".join(f"M={m}: {block_us[m]:.1f} us ({block_us[m] / block_us[1]:.2f} x)"
+                                               for m in (1, 4, 8, 16, 32)))
 
     # horizontal fusion (q,k,v -> one node; gate,up -> one node): 4 launches per block instead of 7
     fused_base = {
@@ -582,6 +589,7 @@ def main() -> int:
                                  "(ovfcc_weights_concat), 4 launches per block",
                          "launches": args.layers * 4, "ms_per_pass": round(fms / args.steps, 5),
                          "GBps": round(fused_gbs, 1), "pct_of_hbm_peak": round(100 * fused_gbs / HBM_PEAK_GBS, 2)},
+        "decode_small_batch": small_batch,
         "decode_per_shape": {k: {"us": round(v["us"], 3), "GBps": round(v["GBps"], 1)} for k, v in per_shape.items()},
         "parity": {k: {a: float(f"{b:.3e}") for a, b in v.items()} for k, v in parity.items()},
     }
