@@ -183,9 +183,10 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         for (int split : {1, 2, 4, 8}) {
             if (split_env > 0 && split != split_env)
                 continue;
-            // (up to 16 rows the parts and their second launch only tie with the small-batch kernel: down projection
-            // 12.8 against 12.7 us; from 17 rows on they are ahead, 16.2 against 21.5 us at 32 rows)
-            if (split > 1 && (L.glu || L.gemv_c % split != 0 || (a.N & 3) || (a.M <= 16 && split_env <= 0)))
+            // (up to 16 rows, four parts and their second launch only tie with the small-batch kernel -- 14336 -> 4096:
+            // 12.8 against 12.7 us; from 17 rows on they are ahead, 16.2 against 21.5 us at 32 rows -- while two
+            // parts are ahead from the start: 8192 -> 8192 at 16 rows 12.5 against 14.7 us)
+            if (split > 1 && (L.glu || L.gemv_c % split != 0 || (a.N & 3) || (a.M <= 16 && split > 2 && split_env <= 0)))
                 continue;
             // the kernel's registers allow 8 and 16 waves per compute unit with 4 and 2 k-blocks per wave
             const int c = gemv16_kblocks_per_wave(L.gemv_c, split);

@@ -201,6 +201,23 @@ def test_gemv16_k_in_parts(oracle, dev, req, monkeypatch, wt, zt, N, K, C, parts
         w.close()
 
 
+def test_gemv16_two_parts_by_policy(oracle, dev, req):
+    """K = 8192 (the q / o class of Llama-3-70B): 16 rows of activations are 256 KiB, so the planner cuts K in two
+    parts, at any row count from five on."""
+    c = datagen.make_case(7870, 48, 8192, 256, "u4", 128, "u4", with_bias=True)
+    w = fc.CompressedWeights.from_case(dev, c)
+    ref = oracle_y(oracle, c)
+    try:
+        for M in (5, 16, 32):
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            say(f"gemv16 K=8192 M={M} {info}")
+            assert info["name"] == "fcc_gemv16_w4" and info["split_k"] == 2, info
+            check_parity(oracle, y, ref[:M], c.K, f"K=8192 M={M} {info}", output_rounding_slack=True)
+    finally:
+        w.close()
+
+
 def test_gemv16_down_projection(oracle, dev, req):
     """The benchmark's down projection (14336 -> 4096) takes the kernel with K in four parts from 17 rows on."""
     K, N = 14336, 4096
