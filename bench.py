@@ -28,7 +28,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs recorded under profiles/ (counters cannot be
 # read from inside this process): FETCH_SIZE x 2.000 (its reading for a copy kernel of known size) + WRITE_SIZE.
-TRAFFIC_DECODE_M1 = {"qo": 8794112, "kv": 2283520, "gate_up": 30461952, "down": 30605312}
+TRAFFIC_DECODE_M1 = {"qo": 8794112, "kv": 2283520, "gate_up": 30441472, "down": 30605312}
 TRAFFIC_PREFILL_M2048 = {"qo": 85494784, "kv": 72139776, "gate_up": 264916992, "down": 255920128}
 
 
