@@ -86,6 +86,13 @@ __device__ __forceinline__ void unpack8_biased(uint32_t w0, uint32_t w1, Frag8& 
     f.u[3] = __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u);
 }
 
+// A pointer that is the same in every lane, told to the compiler (both halves through readfirstlane).
+__device__ __forceinline__ const void* uniform_ptr(const void* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
+}
+
 // Tile coordinates of this workgroup for a 2-D tile grid, arranged for the chip's eight XCDs.  The dispatcher
 // hands consecutive workgroups to consecutive XCDs (workgroup L runs on XCD L % 8), every XCD has its own L2,
 // and one XCD runs 32 workgroups of a one-per-CU kernel at a time.  Workgroups that run together on an XCD

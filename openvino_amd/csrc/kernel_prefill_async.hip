@@ -1,6 +1,8 @@
 // Prefill kernel for 4-bit weights with register-fed matrix-core operands and fully asynchronous data
 // movement: 128 x 256 output tile per workgroup (NT = 8 row tiles of 16), 8 waves; also built with 64 x 256
-// tiles (NT = 4) for grids that 128-row tiles would underfill.  The text below describes NT = 8.
+// tiles (NT = 4) for grids that 128-row tiles would underfill and, for grouped runs whose slices have between 64
+// and 128 rows (the experts of a mixture-of-experts layer), with 80 and 96 rows (NT = 5, 6; four stages of
+// weights).  The text below describes NT = 8.
 //
 // 1-D grid, block = 512: workgroup -> (tile, part of K) by tile_work (device_common.h); the first full_tiles
 // workgroups own whole tiles in XCD-aware order, the others one of split_k parts of a tile (deterministic
@@ -48,14 +50,16 @@ namespace ovfcc {
 constexpr int PA_BM = 128, PA_BN = 256, PA_BK = 128;  // PA_BM: rows of the full tile (NT = 8 row tiles of 16)
 constexpr int PA_STAGES = 3;
 constexpr int PA_XQ = 3;  // activation operands in registers: the one in use and PA_XQ - 1 on their way from LDS
-constexpr int PA_A_BYTES = PA_BM * PA_BK * 2;  // 32 KiB per stage
 constexpr int PA_W_BYTES = 16 * kTileBytes;    // 16 KiB per stage
 constexpr int PA_P_BYTES = 1024;               // per group of a k-block: scales (512) + zero-points (256)
-constexpr int PA_W_OFF = PA_STAGES * PA_A_BYTES;
-constexpr int PA_P_OFF = PA_W_OFF + PA_STAGES * PA_W_BYTES;
-// 147 KiB with one group per k-block, 150 and 156 KiB with two and four
-constexpr unsigned pa_lds_bytes(int gpb) {
-    return (unsigned)(PA_P_OFF + PA_STAGES * PA_P_BYTES * gpb);
+// Tiles of 80 and 96 rows stage 96 rows of activations (24 KiB instead of 32) and spend the room on more stages of
+// weights and parameters: their weights come from memory rather than from L2 (every slice of a grouped run has its
+// own) and need the longer lead.
+constexpr int pa_a_bytes(int nt) { return nt == 5 || nt == 6 ? 96 * PA_BK * 2 : PA_BM * PA_BK * 2; }
+constexpr int pa_w_stages(int nt) { return nt == 5 || nt == 6 ? 4 : PA_STAGES; }
+// 128- and 64-row tiles: 147 KiB with one group per k-block, 150 and 156 KiB with two and four
+constexpr unsigned pa_lds_bytes(int nt, int gpb) {
+    return (unsigned)(PA_STAGES * pa_a_bytes(nt) + pa_w_stages(nt) * (PA_W_BYTES + PA_P_BYTES * gpb));
 }
 
 // The whole kernel for one workgroup's share of one node.  The two kernels below differ only in where the node's
@@ -70,12 +74,14 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                                                    float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N,
                                                    int K, int kb_total, int kb_per_group, int ng, int zp_const,
                                                    int out_f32, int glu, const TileWork wk) {
-    static_assert(NT == 8 || NT == 4, "tiles of 128 or 64 rows");
+    static_assert(NT == 8 || NT == 6 || NT == 5 || NT == 4, "tiles of 128, 96, 80 or 64 rows");
     static_assert(GPB == 1 || ((GPB == 2 || GPB == 4) && PRESCALE), "several groups per k-block: scales go into the weights");
     constexpr int PB = PA_P_BYTES * GPB;  // parameter bytes per stage
+    constexpr int WS = pa_w_stages(NT);   // stages of weights and parameters
+    constexpr int PA_A_BYTES = pa_a_bytes(NT), PA_W_OFF = PA_STAGES * PA_A_BYTES, PA_P_OFF = PA_W_OFF + WS * PA_W_BYTES;
     constexpr int ZOFF = 512 * GPB;       // zero-points follow the scales
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
-    constexpr int AL = NT / 2;                          // activation loads per wave and k-block
+    constexpr int AL = (NT + 1) / 2;                    // activation loads per wave and k-block (32 AL rows staged)
     constexpr int S = 4 * NT;                           // MFMA slots per step (a wave's two steps make a k-block)
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     const lds_byte_ptr lds3 = (lds_byte_ptr)lds_raw;
@@ -106,13 +112,16 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     // row 4 i + (lane >> 4) of those, LDS slot lane & 15 of that row, which holds global chunk
     // (lane & 15) ^ (row & 15).  Rows >= M lie beyond the descriptor's range and arrive as zeros.
     // (row & 15 = 4 i + (lane >> 4) = 4 i ^ (lane >> 4), so the chunk of load i is c0 ^ 4 i.) ----
-    // (64-row tiles: two loads per wave, rows 8 wave + 4 i + (lane >> 4); row & 15 = 8 (wave & 1) ^ 4 i ^ (lane >> 4).)
+    // (Other tile heights: AL loads per wave, rows 4 AL wave + 4 i + (lane >> 4); 4 AL wave + 4 i is a multiple of
+    // four, so row & 15 = ((4 AL wave + 4 i) & 15) ^ (lane >> 4).  80-row tiles stage 96 rows; the loads of rows
+    // past the tile go out of range.)
     const unsigned a_row0 = (unsigned)((m0 + 4 * AL * wave + (lane >> 4)) * K) * 2u;
-    const unsigned a_c0 = (unsigned)((lane & 15) ^ (lane >> 4) ^ (NT == 4 ? 8 * (wave & 1) : 0));
+    const unsigned a_c0 = (unsigned)((lane & 15) ^ (lane >> 4));
     auto dma_a = [&](int kb, int stage, int i) {
-        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
+        const int r0 = 4 * AL * wave + 4 * i;  // first of the load's four rows, uniform
+        const unsigned oob = (unsigned)(((kb_hi - 1 - kb) | (16 * NT - 1 - r0)) >> 31) & kOob;
         const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(4 * i * K + kb * PA_BK) * 2u);
-        const unsigned voff = a_row0 + sterm + ((a_c0 ^ (unsigned)(4 * i)) << 4);
+        const unsigned voff = a_row0 + sterm + ((a_c0 ^ (unsigned)(r0 & 15)) << 4);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void_ptr)(lds3 + stage * PA_A_BYTES + (AL * wave + i) * 1024), 16,
                                                  voff | oob, 0, 0, 0);
     };
@@ -168,11 +177,12 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             }
         }
     };
-    // Per k-block a wave issues, in this order: AL (4 or 2) activation loads (for k-block + 2), then 2 weight
-    // loads and at most one parameter load (for k-block + 3).  The wait at the top of a k-block needs the
+    // Per k-block a wave issues, in this order: AL activation loads (for k-block + 2), then 2 weight
+    // loads and at most one parameter load (for k-block + WS).  The wait at the top of a k-block needs the
     // activations of this k-block and the weights and parameters of the next; the instructions issued after those
-    // are one k-block's worth, at least AL + 2.
-    constexpr int kWaitTop = AL + 2;
+    // are one k-block's worth, at least AL + 2; with more than three stages the weights of the next k-block were
+    // requested before the activations of this one, and the two weight loads that followed those may be in flight too.
+    constexpr int kWaitTop = WS == 3 ? AL + 2 : AL + 4;
 
     // ---- the wave's share of a staged k-block of weights: 8 bytes per tile, plus scale and zero-point ----
     typedef __attribute__((address_space(3))) const uint2_t* lds_u2_ptr;
@@ -226,8 +236,11 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
             const int k = op - 5;
             half2_t off;
             if constexpr (ZP_TABLE) {
-                const float zpv = GPB == 4 ? (float)((wzp[par][r] >> (8 * js)) & 0xFFu) : (float)wzp[par][r];
-                off = (k & 1) ? splat(64.f + zpv) : splat(1024.f + zpv);
+                // 1024 + zp in both halves with one integer operation (f16 1024 .. 2047 are 0x6400 + n), and
+                // 64 + zp = (1024 + zp) - 960 with one packed subtraction; both exact for zp <= 255
+                const uint32_t zpv = GPB == 4 ? (wzp[par][r] >> (8 * js)) & 0xFFu : wzp[par][r];
+                const half2_t lo = as_half2(zpv * 0x00010001u + 0x64006400u);
+                off = (k & 1) ? lo - half2_t{(half_t)960.f, (half_t)960.f} : lo;
             } else {
                 off = (k & 1) ? off_hi_c : off_lo_c;
             }
@@ -294,7 +307,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
         for (int i = 0; i < AL; ++i)
             dma_a(kb_lo + j, j, i);
 #pragma unroll
-    for (int j = 0; j < 3; ++j) {
+    for (int j = 0; j < WS; ++j) {
         dma_w(kb_lo + j, j, 0);
         dma_w(kb_lo + j, j, 1);
         if (has_p)
@@ -318,13 +331,15 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
 
     // ---- main loop: two k-blocks per trip so that the parity of the weight registers is static.  k-blocks
     // past the end are loaded out of range (zeros) and add nothing. ----
-    int s0 = 0;  // stage of k-block kb (activations, weights and parameters cycle alike): kb % 3
+    int s0 = 0;  // stage of k-block kb's activations: kb % 3
+    int w0 = 0;  // stage of its weights and parameters: kb % WS
     for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += 2) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int kb = kb0 + u;
             const int s1 = s0 == 2 ? 0 : s0 + 1;  // stage of k-block kb + 1 and kb - 2
             const int s2 = s1 == 2 ? 0 : s1 + 1;  // stage of k-block kb + 2 and kb - 1
+            const int w1 = w0 == WS - 1 ? 0 : w0 + 1;
             // own loads landed: activations of kb, weights and parameters of kb + 1
             __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(kWaitTop));
             asm volatile("" ::: "memory");
@@ -338,17 +353,18 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                 if (i < S && (i & 7) == 2)
                     dma_a(kb + 2, s2, i >> 3);
                 if (i >= S - 8 && i < S - 4)
-                    read_p(u ^ 1, s1, i - (S - 8));
+                    read_p(u ^ 1, w1, i - (S - 8));
                 if (i >= S - 4 && i < S)
-                    read_w(u ^ 1, s1, i - (S - 4));
+                    read_w(u ^ 1, w1, i - (S - 4));
                 if (i == S + 4)
-                    dma_w(kb + 3, s0, 0);
+                    dma_w(kb + WS, w0, 0);
                 if (i == S + 4 + S / 2)
-                    dma_w(kb + 3, s0, 1);
+                    dma_w(kb + WS, w0, 1);
                 if (i == S + 4 + S / 4 && has_p)
-                    dma_p(kb + 3, s0);
+                    dma_p(kb + WS, w0);
             });
             s0 = s1;
+            w0 = w1;
         }
     }
 
@@ -396,7 +412,12 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const Ba
         full_tiles = h.split_k == 1 ? tiles_x * tiles_y : 0;
     }
     TileWork wk = tile_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT, PA_BN / 2);
-    const BatchGroupItem it = dev_tab ? dev_tab[wk.tile_y] : tab.item[wk.tile_y];
+    BatchGroupItem it = dev_tab ? dev_tab[wk.tile_y] : tab.item[wk.tile_y];
+    // The item is the same for every lane, but the compiler cannot tell: without this, every buffer load of the body
+    // sits in a loop that looks for lanes with equal descriptors (six vector instructions and a branch per load).
+    it.w = uniform_ptr(it.w), it.scale = uniform_ptr(it.scale), it.zp = uniform_ptr(it.zp);
+    it.bias = uniform_ptr(it.bias), it.x = uniform_ptr(it.x), it.y = const_cast<void*>(uniform_ptr(it.y));
+    it.M = __builtin_amdgcn_readfirstlane(it.M);
     if (it.M <= 0)
         return;
     wk.m0 = 0;
@@ -421,7 +442,7 @@ static int allow_lds(Kern kern, bool* done, unsigned bytes) {
 // remaining tile, parts that cover K.
 static bool async_plan_ok(const FcDeviceArgs& a, const LaunchPlan& p) {
     const int64_t tiles = (int64_t)p.tiles_x * p.tiles_y;
-    return (p.tile_m == PA_BM || p.tile_m == PA_BM / 2) && p.tiles_x == a.N / PA_BN && p.tiles_y >= 1 && p.full_tiles >= 0 && p.full_tiles <= tiles && p.split_k >= 1 &&
+    return (p.tile_m == 128 || p.tile_m == 96 || p.tile_m == 80 || p.tile_m == 64) && p.tiles_x == a.N / PA_BN && p.tiles_y >= 1 && p.full_tiles >= 0 && p.full_tiles <= tiles && p.split_k >= 1 &&
            (int64_t)p.kblocks_per_split * p.split_k >= a.layout.k_blocks && (p.full_tiles == tiles || p.kblocks_per_split >= 1) &&
            p.grid[0] == (unsigned)(p.full_tiles + (tiles - p.full_tiles) * p.split_k) && p.grid[1] == 1 && p.grid[2] == 1 &&
            (p.split_k == 1 || (a.workspace && a.counters));
@@ -432,9 +453,9 @@ static int launch_async_gpb(const FcDeviceArgs& a, const LaunchPlan& p, hipStrea
     const Layout& L = a.layout;
     auto kern = fcc_prefill_async_kernel<ZPT, PRE, NT, GPB>;
     static bool attr_set = false;  // per instantiation
-    if (int e = allow_lds(kern, &attr_set, pa_lds_bytes(GPB)))
+    if (int e = allow_lds(kern, &attr_set, pa_lds_bytes(NT, GPB)))
         return e;
-    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(GPB), s, (const uint4_t*)a.w,
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(NT, GPB), s, (const uint4_t*)a.w,
                        (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.x, (const half_t*)a.bias, a.y,
                        a.workspace, a.counters, (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks,
                        (int)L.kblocks_per_group, (int)L.groups, L.zp_const, a.out_f32, L.glu, p.tiles_x,
@@ -460,9 +481,9 @@ static int launch_async_grouped_gpb(const BatchGroupTable& tab, const BatchGroup
     const Layout& L = a.layout;
     auto kern = fcc_prefill_async_grouped_kernel<ZPT, PRE, NT, GPB>;
     static bool attr_set = false;  // per instantiation
-    if (int e = allow_lds(kern, &attr_set, pa_lds_bytes(GPB)))
+    if (int e = allow_lds(kern, &attr_set, pa_lds_bytes(NT, GPB)))
         return e;
-    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(GPB), s, tab, dev_tab,
+    hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(NT, GPB), s, tab, dev_tab,
                        dev_hdr, a.workspace, a.counters, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
                        L.zp_const, a.out_f32, L.glu, p.tiles_x, p.tiles_y, p.full_tiles, p.split_k,
                        p.kblocks_per_split);
@@ -493,7 +514,7 @@ int launch_prefill_async(const FcDeviceArgs& a, const LaunchPlan& p, void* strea
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
     // (the planner sends 8-bit nodes to the register-ring kernel)
-    if (L.bits != 4 || !async_plan_ok(a, p) || (int64_t)p.tiles_y * p.tile_m < a.M)
+    if (L.bits != 4 || !async_plan_ok(a, p) || (int64_t)p.tiles_y * p.tile_m < a.M || (p.tile_m != PA_BM && p.tile_m != PA_BM / 2))
         return (int)hipErrorInvalidValue;
     const bool nt8 = p.tile_m == PA_BM;
     return OVFCC_ASYNC_DISPATCH(launch_async_impl, a, p, s);
@@ -518,7 +539,7 @@ int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const 
             if (tab.item[i].M < 1 || tab.item[i].M > p.tile_m)
                 return (int)hipErrorInvalidValue;
     } else {
-        if ((p.tile_m != PA_BM && p.tile_m != PA_BM / 2) || p.tiles_x != a.N / PA_BN || p.grid[1] != 1 || p.grid[2] != 1)
+        if ((p.tile_m != 128 && p.tile_m != 96 && p.tile_m != 80 && p.tile_m != 64) || p.tiles_x != a.N / PA_BN || p.grid[1] != 1 || p.grid[2] != 1)
             return (int)hipErrorInvalidValue;
         for (int t = 1; t <= n_items; ++t) {
             const RoutedHeader h = routed_header(p.tiles_x, t, (int)L.k_blocks, p.n_cus);
@@ -528,6 +549,18 @@ int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const 
                                    (size_t)p.tiles_x * t > p.counter_count)))
                 return (int)hipErrorInvalidValue;
         }
+    }
+    if (p.tile_m == 80 || p.tile_m == 96) {
+        // slices of 80 and 96 rows: one group per k-block only
+        if (L.groups_per_kblock != 1)
+            return (int)hipErrorInvalidValue;
+        const bool nt5 = p.tile_m == 80;
+#define OVFCC_ASYNC_MID(ZPT, PRE)                                                                          \
+    (nt5 ? launch_async_grouped_gpb<ZPT, PRE, 5, 1>(tab, dev_tab, dev_hdr, a, p, s)                         \
+         : launch_async_grouped_gpb<ZPT, PRE, 6, 1>(tab, dev_tab, dev_hdr, a, p, s))
+        return L.groups == 1 ? (L.zp_table ? OVFCC_ASYNC_MID(true, false) : OVFCC_ASYNC_MID(false, false))
+                             : (L.zp_table ? OVFCC_ASYNC_MID(true, true) : OVFCC_ASYNC_MID(false, true));
+#undef OVFCC_ASYNC_MID
     }
     const bool nt8 = p.tile_m == PA_BM;
     return OVFCC_ASYNC_DISPATCH(launch_async_grouped_impl, tab, dev_tab, dev_hdr, a, p, s);

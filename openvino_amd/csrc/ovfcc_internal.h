@@ -111,7 +111,7 @@ struct FcDeviceArgs {
     int out_f32;         // output_type f32 instead of f16
     int64_t N_out;       // row length of y: N, or N / 2 with a gated-linear-unit epilogue
     int gate_offset, up_offset;  // untiled layout with such an epilogue: first gate / up channel
-    int tile_rows = 0;   // async prefill kernel: 64 or 128 forces the tile height, 0 leaves it to the planner
+    int tile_rows = 0;   // async prefill kernel: 64 or 128 (grouped runs: also 80, 96) forces the tile height, 0 leaves it to the planner
     bool want_async = false;  // take the all-asynchronous prefill kernel wherever it can run the node, also where
                               // smaller tiles would spread a small node further (a slice table in device memory
                               // has no other reader)
@@ -187,7 +187,7 @@ struct BatchGroupTable {
 };
 int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& plan,
                          void* stream);
-// Same table, items of at most 128 rows, 4-bit async prefill kernel; plan is that of one node of 128 * n_items rows.
+// Same table, items of at most tile_m rows, 4-bit async prefill kernel; plan is that of one node of tile_m * n_items rows.
 #ifdef __HIPCC__
 #define OVFCC_HOST_DEVICE __host__ __device__
 #else

@@ -374,12 +374,17 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             // the time of a 128-row tile (same weight traffic and unpack work, half the MFMAs), so it pays only
             // where 128-row tiles would leave half the chip idle.  (OVFCC_PREFILL_ROWS = 64 | 128 overrides;
             // a.tile_rows, set by the grouped run, wins over both.)
-            int rows = env_int("OVFCC_PREFILL_ROWS", (int64_t)p.grid[0] * ((a.M + 63) / 64) <= n_cus ? 64 : 128);
+            int rows = (int64_t)p.grid[0] * ((a.M + 63) / 64) <= n_cus ? 64 : 128;
+            if (const int env_rows = env_int("OVFCC_PREFILL_ROWS", 0); env_rows == 64 || env_rows == 128)
+                rows = env_rows;
             if (a.tile_rows == 64 || a.tile_rows == 128)
                 rows = a.tile_rows;
-            if (rows == 64) {
-                p.tile_m = 64;
-                p.grid[1] = (unsigned)((a.M + 63) / 64);
+            // (80 and 96 rows: grouped runs only, one group per k-block)
+            if ((a.tile_rows == 80 || a.tile_rows == 96) && L.groups_per_kblock == 1)
+                rows = a.tile_rows;
+            if (rows != 128) {
+                p.tile_m = rows == 80 || rows == 96 ? rows : 64;
+                p.grid[1] = (unsigned)((a.M + p.tile_m - 1) / p.tile_m);
             }
         }
         p.kblocks_per_split = (int)L.k_blocks;
