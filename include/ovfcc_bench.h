@@ -38,6 +38,13 @@ int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t 
 int ovfcc_bench_floor(ovfcc_ctx* ctx, const void* arena_dev, size_t arena_bytes, size_t node_bytes, int n_nodes, int waves,
                       int kib_per_wave, int iters, float* elapsed_ms);
 
+/* Matrix-core ceiling: one workgroup per compute unit with `waves` waves (4 or 8: one or two per SIMD), every
+ * wave `rounds` times eight independent v_mfma_f32_16x16x32_f16 on registers, each followed by `valu` (0..4)
+ * packed-f16 vector multiplications on other registers; no memory traffic.  Timed with HIP events; *flops is the
+ * matrix-core work of the timed launch (2 * 16 * 16 * 32 per instruction).  What the chip sustains under that load
+ * (it lowers its clock) is the ceiling the prefill kernels are measured against beside the nominal peak. */
+int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int rounds, float* elapsed_ms, double* flops);
+
 #ifdef __cplusplus
 }
 #endif

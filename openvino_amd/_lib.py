@@ -23,7 +23,7 @@ SYMBOLS = [
     "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
     "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_device_static", "ovfcc_fc_run_grouped_device", "ovfcc_grouped_matmul_device", "ovfcc_grouped_matmul_offsets_device", "ovfcc_gather_matmul_device", "ovfcc_gather_matmul_routed_device", "ovfcc_moe_device", "ovfcc_moe_routed_device", "ovfcc_bench_grouped", "ovfcc_request_sync", "ovfcc_request_force_kernel",
     "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
-    "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_memcpy_d2d", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_desc_validate", "ovfcc_env_reload", "ovfcc_tiled_sizes",
+    "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_memcpy_d2d", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_bench_mfma", "ovfcc_desc_validate", "ovfcc_env_reload", "ovfcc_tiled_sizes",
     "ovfcc_repack_host", "ovfcc_unrepack_host", "ovfcc_unpack_u4", "ovfcc_unpack_i4", "ovfcc_last_error",
     "ovfcc_version", "ovfcc_fold_match", "ovfcc_fold_model", "ovfcc_fold_gather_matmul", "ovfcc_fold_grouped_matmul", "ovfcc_fold_moe",
 ]
@@ -161,6 +161,7 @@ def load() -> ctypes.CDLL:
         "ovfcc_memcpy_d2d": (ci, [vp, vp, vp, sz]),
         "ovfcc_bench_copy": (ci, [vp, vp, vp, sz, ci, ctypes.POINTER(ctypes.c_float)]),
         "ovfcc_bench_floor": (ci, [vp, vp, sz, sz, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_float)]),
+        "ovfcc_bench_mfma": (ci, [vp, ci, ci, ci, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]),
         "ovfcc_desc_validate": (ci, [ctypes.POINTER(FcDesc)]),
         "ovfcc_env_reload": (None, []),
         "ovfcc_tiled_sizes": (ci, [ctypes.POINTER(FcDesc), ctypes.POINTER(sz), ctypes.POINTER(sz), ctypes.POINTER(sz)]),

@@ -1924,6 +1924,36 @@ int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t 
     return OVFCC_OK;
 }
 
+int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int rounds, float* elapsed_ms, double* flops) {
+    if (!ctx || !elapsed_ms || !flops || rounds <= 0 || (waves != 4 && waves != 8) || valu < 0 || valu > 4)
+        return fail(OVFCC_EINVAL, "bad matrix-core benchmark arguments");
+    HIP_TRY(hipSetDevice(ctx->device));
+    hipStream_t s = nullptr;
+    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    const int workgroups = ctx->n_cus;
+    float* sink = nullptr;
+    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&sink), (size_t)workgroups * 64 * waves * sizeof(float)));
+    hipEvent_t t0, t1;
+    HIP_TRY(hipEventCreate(&t0));
+    HIP_TRY(hipEventCreate(&t1));
+    int e = ovfcc::launch_mfma_probe(sink, workgroups, waves, valu, 16, s);  // warm-up
+    HIP_TRY(hipStreamSynchronize(s));
+    HIP_TRY(hipEventRecord(t0, s));
+    if (!e)
+        e = ovfcc::launch_mfma_probe(sink, workgroups, waves, valu, rounds, s);
+    HIP_TRY(hipEventRecord(t1, s));
+    HIP_TRY(hipEventSynchronize(t1));
+    HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    (void)hipFree(sink);
+    (void)hipStreamDestroy(s);
+    if (e)
+        return hip_fail((hipError_t)e, "matrix-core probe launch");
+    *flops = 2.0 * 16 * 16 * 32 * 8.0 * rounds * waves * workgroups;
+    return OVFCC_OK;
+}
+
 // One graph of n_nodes probe launches, replayed `iters` times after three warm-up replays.
 int ovfcc_bench_floor(ovfcc_ctx* ctx, const void* arena_dev, size_t arena_bytes, size_t node_bytes, int n_nodes, int waves,
                       int kib_per_wave, int iters, float* elapsed_ms) {

@@ -1,4 +1,6 @@
-// Benchmark probes (no part of the FullyConnected path): what a graph node costs with nothing in it, and how
+// Benchmark probes (no part of the FullyConnected path): what a graph node costs with nothing in it, how fast the
+// matrix cores run a loop of nothing but v_mfma_f32_16x16x32_f16 (the chip lowers its clock under that load, so
+// the figure lies below the nominal peak), and how
 // fast a bare streaming kernel -- loads only, the access pattern of the decode kernels, no arithmetic, no
 // reduction, no store -- reads a buffer of a given size under graph replay.  The decode kernels are measured
 // against these: a node cannot finish sooner than an empty one starts and stops, nor move its weights faster
@@ -42,6 +44,52 @@ __global__ __launch_bounds__(1024) void fcc_stream_probe_kernel(const uint4_t* _
     const unsigned v = acc.x ^ acc.y ^ acc.z ^ acc.w;
     if (v == 0x12345678u)  // keeps the loads alive; the buffers never hold this pattern
         out[0] = v;
+}
+
+// Every wave runs `iters` rounds of eight independent MFMAs (eight accumulators, operands in registers, no
+// memory traffic), each followed by VALU packed-f16 multiplications on registers the MFMAs do not touch.
+template <int VALU>
+__global__ __launch_bounds__(512) void fcc_mfma_probe_kernel(float* __restrict__ sink, int iters) {
+    half8_t a, b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        a[i] = (half_t)(0.001f * (float)(threadIdx.x & 63) + (float)i), b[i] = (half_t)(0.5f * (float)i);
+    float4_t acc[8];
+    uint32_t r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        acc[i] = float4_t{0.f, 0.f, 0.f, 0.f}, r[i] = 0x3c003c00u + (uint32_t)i;
+    const uint32_t c = 0x3c003c00u;  // 1.0 in both halves
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a), "v"(b));
+#pragma unroll
+            for (int v = 0; v < VALU; ++v)
+                asm volatile("v_pk_mul_f16 %0, %0, %1" : "+v"(r[(j + v) & 7]) : "v"(c));
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        s += acc[i].x + acc[i].y + acc[i].z + acc[i].w + (float)r[i];
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+// sink: 4 * workgroups * 64 * waves bytes.  valu: 0 to 4 multiplications after every MFMA.
+int launch_mfma_probe(float* sink, int workgroups, int waves, int valu, int iters, void* stream) {
+    if (!sink || workgroups < 1 || (waves != 4 && waves != 8) || valu < 0 || valu > 4 || iters < 1)
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 g((unsigned)workgroups), b(64u * waves);
+    switch (valu) {
+    case 0: hipLaunchKernelGGL(fcc_mfma_probe_kernel<0>, g, b, 0, s, sink, iters); break;
+    case 1: hipLaunchKernelGGL(fcc_mfma_probe_kernel<1>, g, b, 0, s, sink, iters); break;
+    case 2: hipLaunchKernelGGL(fcc_mfma_probe_kernel<2>, g, b, 0, s, sink, iters); break;
+    case 3: hipLaunchKernelGGL(fcc_mfma_probe_kernel<3>, g, b, 0, s, sink, iters); break;
+    default: hipLaunchKernelGGL(fcc_mfma_probe_kernel<4>, g, b, 0, s, sink, iters); break;
+    }
+    return (int)hipGetLastError();
 }
 
 int launch_empty(unsigned* out, void* stream) {

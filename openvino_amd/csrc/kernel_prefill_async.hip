@@ -78,7 +78,9 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     static_assert(GPB == 1 || ((GPB == 2 || GPB == 4) && PRESCALE), "several groups per k-block: scales go into the weights");
     constexpr int PB = PA_P_BYTES * GPB;  // parameter bytes per stage
     constexpr int WS = pa_w_stages(NT);   // stages of weights and parameters
-    constexpr int PA_A_BYTES = pa_a_bytes(NT), PA_W_OFF = PA_STAGES * PA_A_BYTES, PA_P_OFF = PA_W_OFF + WS * PA_W_BYTES;
+    // LDS: parameters first, then weights, then activations -- the small, scattered reads of scales and zero-points
+    // keep their offsets within the 16 bits of an LDS instruction's immediate
+    constexpr int PA_A_BYTES = pa_a_bytes(NT), PA_W_OFF = WS * PB, PA_A_OFF = PA_W_OFF + WS * PA_W_BYTES;
     constexpr int ZOFF = 512 * GPB;       // zero-points follow the scales
     constexpr int NOPS = 5 + 4 + (PRESCALE ? 4 : 0);  // unpack micro-operations per dword
     constexpr int AL = (NT + 1) / 2;                    // activation loads per wave and k-block (32 AL rows staged)
@@ -97,41 +99,48 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
 
     constexpr unsigned kOob = 0x80000000u;
     constexpr int kRsrcFlags = 0x00020000;
-    // Every offset goes through the vector operand: the scalar offset of a buffer load is not range-checked.
-    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, M * K * 2, kRsrcFlags);
+    // Buffer loads: the per-lane part of an offset (row, chunk, lane) is computed once and travels in the vector
+    // operand, which the hardware checks against the descriptor's range (rows >= M read zeros); the part that
+    // advances with the k-block is uniform and travels in the scalar operand, which is not checked -- a load for a
+    // k-block past kb_hi uses a descriptor of length zero instead.  That keeps the loop free of vector address
+    // arithmetic.
     const int nt0 = n0 / 16;  // the workgroup's 16 channel tiles
-    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint4_t*>(wt + (size_t)nt0 * kb_total * 64), 0, 16 * kb_total * kTileBytes, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t rs =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(st + (size_t)nt0 * ng * 16), 0, 16 * ng * 32, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t rz = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(ZP_TABLE ? zt + (size_t)nt0 * ng * 16 : zt), 0, ZP_TABLE ? 16 * ng * 16 : 0, kRsrcFlags);
+    auto live = [&](int kb, int bytes) { return kb < kb_hi ? bytes : 0; };
+#define PA_DESC_X(kb) \
+    __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, live(kb, M * K * 2), kRsrcFlags)
+#define PA_DESC_W(kb)                                                                                  \
+    __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4_t*>(wt + (size_t)nt0 * kb_total * 64), 0,        \
+                                      live(kb, 16 * kb_total * kTileBytes), kRsrcFlags)
+#define PA_DESC_S(kb) \
+    __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(st + (size_t)nt0 * ng * 16), 0, live(kb, 16 * ng * 32), kRsrcFlags)
+#define PA_DESC_Z(kb)                                                                                       \
+    __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ZP_TABLE ? zt + (size_t)nt0 * ng * 16 : zt), 0, \
+                                      ZP_TABLE ? live(kb, 16 * ng * 16) : 0, kRsrcFlags)
     const unsigned g_mul = kb_per_group == 1 ? 0u : (unsigned)((0x100000000ull + kb_per_group - 1) / kb_per_group);
 
-    // ---- activations: direct-to-LDS load i of the wave covers rows 16 wave + 4 i .. +3 of the tile; lane ->
-    // row 4 i + (lane >> 4) of those, LDS slot lane & 15 of that row, which holds global chunk
-    // (lane & 15) ^ (row & 15).  Rows >= M lie beyond the descriptor's range and arrive as zeros.
-    // (row & 15 = 4 i + (lane >> 4) = 4 i ^ (lane >> 4), so the chunk of load i is c0 ^ 4 i.) ----
-    // (Other tile heights: AL loads per wave, rows 4 AL wave + 4 i + (lane >> 4); 4 AL wave + 4 i is a multiple of
-    // four, so row & 15 = ((4 AL wave + 4 i) & 15) ^ (lane >> 4).  80-row tiles stage 96 rows; the loads of rows
-    // past the tile go out of range.)
-    const unsigned a_row0 = (unsigned)((m0 + 4 * AL * wave + (lane >> 4)) * K) * 2u;
-    const unsigned a_c0 = (unsigned)((lane & 15) ^ (lane >> 4));
-    auto dma_a = [&](int kb, int stage, int i) {
+    // ---- activations: direct-to-LDS load i of the wave covers rows 4 AL wave + 4 i .. +3 of the tile (AL loads per
+    // wave; 16 wave + 4 i with 128-row tiles); lane -> row (lane >> 4) of those, LDS slot lane & 15 of that row,
+    // which holds global chunk (lane & 15) ^ (row & 15).  4 AL wave + 4 i is a multiple of four, so
+    // row & 15 = ((4 AL wave + 4 i) & 15) ^ (lane >> 4).  80-row tiles stage 96 rows; the loads of rows past the
+    // tile go out of range. ----
+    unsigned a_voff[4];  // AL entries in use (a bound that depends on NT does not pass the host pass)
+#pragma unroll
+    for (int i = 0; i < AL; ++i) {
         const int r0 = 4 * AL * wave + 4 * i;  // first of the load's four rows, uniform
-        const unsigned oob = (unsigned)(((kb_hi - 1 - kb) | (16 * NT - 1 - r0)) >> 31) & kOob;
-        const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(4 * i * K + kb * PA_BK) * 2u);
-        const unsigned voff = a_row0 + sterm + ((a_c0 ^ (unsigned)(r0 & 15)) << 4);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void_ptr)(lds3 + stage * PA_A_BYTES + (AL * wave + i) * 1024), 16,
-                                                 voff | oob, 0, 0, 0);
+        a_voff[i] = ((unsigned)((m0 + r0 + (lane >> 4)) * K) * 2u + ((unsigned)((lane & 15) ^ (lane >> 4) ^ (r0 & 15)) << 4)) |
+                    (r0 >= 16 * NT ? kOob : 0u);
+    }
+    auto dma_a = [&](int kb, int stage, int i) {
+        { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_X(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_,
+                                                 (lds_void_ptr)(lds3 + PA_A_OFF + stage * PA_A_BYTES + (AL * wave + i) * 1024),
+                                                 16, a_voff[i], kb * (PA_BK * 2), 0, 0); }
     };
     // ---- weights: the wave copies tiles 2 wave, 2 wave + 1 of the workgroup's 16 ----
+    const unsigned w_voff = lane * 16u;
     auto dma_w = [&](int kb, int stage, int i) {
-        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
         const int t = 2 * wave + i;
-        const unsigned sterm = __builtin_amdgcn_readfirstlane((unsigned)(t * kb_total + kb) * kTileBytes);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (lds_void_ptr)(lds3 + PA_W_OFF + stage * PA_W_BYTES + t * kTileBytes),
-                                                 16, (sterm + lane * 16u) | oob, 0, 0, 0);
+        { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_W(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_, (lds_void_ptr)(lds3 + PA_W_OFF + stage * PA_W_BYTES + t * kTileBytes),
+                                                 16, w_voff, (t * kb_total + kb) * kTileBytes, 0, 0); }
     };
     // ---- parameters: waves 0 and 1 fetch the scales of eight channel tiles each (32 bytes per tile, 4 per
     // lane), wave 2 the zero-points of all sixteen (16 bytes per tile, 4 per lane); other waves fetch nothing ----
@@ -141,40 +150,43 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     const bool has_p = GPB == 1   ? (PRESCALE && wave < 2) || (ZP_TABLE && wave == 2)
                        : GPB == 2 ? wave == 0 || (ZP_TABLE && (wave == 2 || wave == 3))
                                   : wave < 2 || (ZP_TABLE && wave == 2);
+    // the lane's part of its parameter load's offset (the tile's row of the table and the lane's bytes in it)
+    unsigned p_voff = 0;
+    if constexpr (GPB == 1) {
+        if (PRESCALE && wave < 2)
+            p_voff = (8u * wave + (lane >> 3)) * ng * 32u + (lane & 7) * 4u;
+        else if (ZP_TABLE && wave == 2)
+            p_voff = (lane >> 2) * ng * 16u + (lane & 3) * 4u;
+    } else if constexpr (GPB == 2) {
+        if (wave == 0)
+            p_voff = (lane >> 2) * kb_total * 64u + (lane & 3) * 16u;
+        else if (ZP_TABLE && (wave == 2 || wave == 3))
+            p_voff = (8u * (wave - 2) + (lane >> 3)) * kb_total * 32u + (lane & 7) * 4u;
+    } else {
+        if (wave < 2)
+            p_voff = (8u * wave + (lane >> 3)) * kb_total * 128u + (lane & 7) * 16u;
+        else if (ZP_TABLE && wave == 2)
+            p_voff = (lane >> 2) * kb_total * 64u + (lane & 3) * 16u;
+    }
     auto dma_p = [&](int kb, int stage) {
-        const unsigned oob = (unsigned)((kb_hi - 1 - kb) >> 31) & kOob;
-        const lds_byte_ptr pbase = lds3 + PA_P_OFF + stage * PB;
+        const lds_byte_ptr pbase = lds3 + stage * PB;
         if constexpr (GPB == 1) {
-            const unsigned g = kb_per_group == 1 ? (unsigned)kb : __umulhi((unsigned)kb, g_mul);
-            if (PRESCALE && wave < 2) {
-                const unsigned tile = 8u * wave + (lane >> 3);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_ptr)(pbase + 256 * wave), 4,
-                                                         ((tile * ng + g) * 32u + (lane & 7) * 4u) | oob, 0, 0, 0);
-            } else if (ZP_TABLE && wave == 2) {
-                const unsigned tile = lane >> 2;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(pbase + ZOFF), 4,
-                                                         ((tile * ng + g) * 16u + (lane & 3) * 4u) | oob, 0, 0, 0);
-            }
+            const int g = kb_per_group == 1 ? kb : (int)__umulhi((unsigned)kb, g_mul);
+            if (PRESCALE && wave < 2)
+                { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_S(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_, (lds_void_ptr)(pbase + 256 * wave), 4, p_voff, g * 32, 0, 0); }
+            else if (ZP_TABLE && wave == 2)
+                { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_Z(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_, (lds_void_ptr)(pbase + ZOFF), 4, p_voff, g * 16, 0, 0); }
         } else if constexpr (GPB == 2) {
-            if (wave == 0) {
-                const unsigned tile = lane >> 2;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_ptr)pbase, 16,
-                                                         ((tile * kb_total + kb) * 64u + (lane & 3) * 16u) | oob, 0, 0, 0);
-            } else if (ZP_TABLE && (wave == 2 || wave == 3)) {
-                const unsigned tile = 8u * (wave - 2) + (lane >> 3);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(pbase + ZOFF + 256 * (wave - 2)), 4,
-                                                         ((tile * kb_total + kb) * 32u + (lane & 7) * 4u) | oob, 0, 0, 0);
-            }
+            if (wave == 0)
+                { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_S(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_, (lds_void_ptr)pbase, 16, p_voff, kb * 64, 0, 0); }
+            else if (ZP_TABLE && (wave == 2 || wave == 3))
+                { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_Z(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_, (lds_void_ptr)(pbase + ZOFF + 256 * (wave - 2)), 4,
+                                                         p_voff, kb * 32, 0, 0); }
         } else {
-            if (wave < 2) {
-                const unsigned tile = 8u * wave + (lane >> 3);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_ptr)(pbase + 1024 * wave), 16,
-                                                         ((tile * kb_total + kb) * 128u + (lane & 7) * 16u) | oob, 0, 0, 0);
-            } else if (ZP_TABLE && wave == 2) {
-                const unsigned tile = lane >> 2;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(pbase + ZOFF), 16,
-                                                         ((tile * kb_total + kb) * 64u + (lane & 3) * 16u) | oob, 0, 0, 0);
-            }
+            if (wave < 2)
+                { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_S(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_, (lds_void_ptr)(pbase + 1024 * wave), 16, p_voff, kb * 128, 0, 0); }
+            else if (ZP_TABLE && wave == 2)
+                { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_Z(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_, (lds_void_ptr)(pbase + ZOFF), 16, p_voff, kb * 64, 0, 0); }
         }
     };
     // Per k-block a wave issues, in this order: AL activation loads (for k-block + 2), then 2 weight
@@ -197,7 +209,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
         wraw[par][r][0] = v.x, wraw[par][r][1] = v.y;
     };
     auto read_p = [&](int par, int stage, int r) {
-        const lds_byte_ptr pbase = lds3 + PA_P_OFF + stage * PB;
+        const lds_byte_ptr pbase = lds3 + stage * PB;
         if constexpr (GPB == 4) {
             // groups 2 kg (step 0) and 2 kg + 1 (step 1) of the lane's channel
             const uint32_t v = *(lds_u32_ptr)(pbase + (4 * wn + r) * 128 + col * 8 + kg * 4);
@@ -265,8 +277,8 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     auto block = [&](int stage, Frag8 (&wf0)[4], Frag8 (&wf1)[4], int par_a, int par_b, auto&& mem) {
         typedef __attribute__((address_space(3))) const half8_t* lds_frag_ptr;
         // operand of row tile t and step js: row 16 t + col, chunk (4 (2 kg + js) + kq) ^ col
-        const lds_byte_ptr xa0 = lds3 + stage * PA_A_BYTES + col * 256 + (((8 * kg + kq) ^ col) << 4);
-        const lds_byte_ptr xa1 = lds3 + stage * PA_A_BYTES + col * 256 + (((8 * kg + 4 + kq) ^ col) << 4);
+        const lds_byte_ptr xa0 = lds3 + PA_A_OFF + stage * PA_A_BYTES + col * 256 + (((8 * kg + kq) ^ col) << 4);
+        const lds_byte_ptr xa1 = lds3 + PA_A_OFF + stage * PA_A_BYTES + col * 256 + (((8 * kg + 4 + kq) ^ col) << 4);
         auto x_at = [&](int tt) { return *(lds_frag_ptr)((tt < NT ? xa0 : xa1) + (tt % NT) * 16 * 256); };
         half8_t xq[PA_XQ];
 #pragma unroll
@@ -372,6 +384,10 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));  // the out-of-range loads of the last trips still target LDS
     tile_epilogue<PRESCALE, NT>(acc, lds_raw, st, bias, y, ws, counters, M, N, n0, m0, split_k, wk.z, tile_id, out_f32, glu);
 }
+#undef PA_DESC_X
+#undef PA_DESC_W
+#undef PA_DESC_S
+#undef PA_DESC_Z
 
 template <bool ZP_TABLE, bool PRESCALE, int NT, int GPB>
 __global__ __launch_bounds__(512) void fcc_prefill_async_kernel(const uint4_t* __restrict__ wt,

@@ -268,6 +268,7 @@ int launch_touch(const void* src, size_t bytes, void* stream);
 // benchmark probes: an empty kernel, and a loads-only streaming kernel (workgroups of `waves` waves, kib_per_wave
 // KiB per wave, eight loads in flight per wave) over `bytes`
 int launch_empty(unsigned* out, void* stream);
+int launch_mfma_probe(float* sink, int workgroups, int waves, int valu, int iters, void* stream);
 int launch_stream_probe(const void* src, size_t bytes, int waves, int kib_per_wave, unsigned* out, void* stream);
 // y[m, :] = sum_j routing[m, j] * d[pos[m * top_k + j], :], rows of H (a multiple of 4) channels; d f16 or f32
 int launch_moe_combine(void* y, const void* d, const void* routing, const int* pos, int rows, int top_k, int H,

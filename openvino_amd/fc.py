@@ -90,6 +90,13 @@ class Device:
                                          kib_per_wave, iters, ctypes.byref(ms)))
         return ms.value * 1e3 / iters / n_nodes
 
+    def mfma_ceiling(self, waves: int = 8, valu: int = 0, rounds: int = 20000) -> float:
+        """TFLOP/s of a loop of nothing but v_mfma_f32_16x16x32_f16 on every compute unit, `waves` waves each (4 or
+        8), with `valu` packed-f16 vector multiplications after every MFMA (ovfcc_bench_mfma)."""
+        ms, flops = ctypes.c_float(), ctypes.c_double()
+        check(self.lib.ovfcc_bench_mfma(self.handle, waves, valu, rounds, ctypes.byref(ms), ctypes.byref(flops)))
+        return flops.value / (ms.value * 1e-3) / 1e12
+
     def copy_bandwidth(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
         """GB/s (read + write) of the plain copy kernel."""
         src, dst = self.malloc(nbytes), self.malloc(nbytes)
