@@ -331,6 +331,47 @@ def results_table(dev, req, args) -> int:
     return 0
 
 
+def profile_moe(dev, req) -> int:
+    """Short run for rocprofv3: the copy-kernel yardstick, then config 5's expert block (Mixtral-8x7B shapes, 8 experts,
+    top-2, 256 tokens) a few times as one MOECompressed call with the routing indices in device memory."""
+    from openvino_amd import datagen, fc
+
+    dev.copy_bandwidth(256 << 20, 1)
+    routes = datagen.moe_routing()
+    tokens = 256
+    indices = np.full((tokens, 2), -1, np.int32)
+    for e, rows_e in enumerate(routes):
+        for t in rows_e:
+            indices[t, 0 if indices[t, 0] < 0 else 1] = e
+    wg, wd = [], []
+    for e in range(len(routes)):
+        g, u = datagen.config5_expert(e, "gate", 1), datagen.config5_expert(e, "up", 1)
+        gu = datagen.FcCase(1, g.K, 2 * g.N, 128, "u4", "u4", np.concatenate([g.w, u.w]),
+                            np.concatenate([g.scale, u.scale]), np.concatenate([g.zp, u.zp]), g.x)
+        wg.append(fc.CompressedWeights.from_case(dev, gu, glu="swish"))
+        wd.append(fc.CompressedWeights.from_case(dev, datagen.config5_expert(e, "down", 1)))
+    rng5 = np.random.default_rng(55)
+    xh = rng5.standard_normal((tokens, 4096)).astype(np.float16)
+    rw = rng5.uniform(0.2, 0.8, size=(tokens, 1))
+    routing = np.concatenate([rw, 1.0 - rw], axis=1).astype(np.float16)
+    x_ptr, r_ptr, y_ptr, i_ptr = (dev.malloc(xh.nbytes), dev.malloc(routing.nbytes), dev.malloc(tokens * 4096 * 2),
+                                  dev.malloc(indices.nbytes))
+    dev.upload(x_ptr, xh)
+    dev.upload(r_ptr, routing)
+    dev.upload(i_ptr, indices)
+    for _ in range(5):
+        req.moe_routed_device(wg, wd, x_ptr, r_ptr, i_ptr, tokens, 2, y_ptr)
+    req.sync()
+    log(f"rows per expert {[len(r) for r in routes]}; last launch {req.last_kernel()}")
+    for w in wg + wd:
+        w.close()
+    for ptr in (x_ptr, r_ptr, y_ptr, i_ptr):
+        dev.free(ptr)
+    req.close()
+    dev.close()
+    return 0
+
+
 def floors_table(dev, req, args) -> int:
     """Per Llama-3-8B shape at M = 1: the time of an empty graph node, of the best loads-only streaming kernel over the
     node's weight bytes (a sweep of workgroup shapes), and of the node itself -- all as nodes of replayed graphs over
@@ -405,7 +446,7 @@ def main() -> int:
     ap.add_argument("--floors", action="store_true",
                     help="measure what bounds a decode node from below -- an empty graph node, a loads-only streaming "
                          "kernel over the node's weight bytes -- beside the node's own time, and print a markdown table")
-    ap.add_argument("--profile", choices=["decode", "batch", "prefill", "w8a8", "w4a8"], default=None,
+    ap.add_argument("--profile", choices=["decode", "batch", "prefill", "w8a8", "w4a8", "moe"], default=None,
                     help="short run for rocprofv3: one copy-kernel launch of known size (the counter yardstick), "
                          "then a few eager passes of the chosen kernel family; prints no JSON")
     ap.add_argument("--profile-rows", type=int, default=32,
@@ -427,6 +468,8 @@ def main() -> int:
         return results_table(dev, req, args)
     if args.floors:
         return floors_table(dev, req, args)
+    if args.profile == "moe":
+        return profile_moe(dev, req)
 
     # ---- weights: one host tensor set per shape, one device copy per use ----
     t0 = time.perf_counter()
