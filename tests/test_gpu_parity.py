@@ -434,6 +434,44 @@ def test_grouped_run_matches_oracle_and_separate_runs(oracle, dev, req, monkeypa
             w.close()
 
 
+@pytest.mark.parametrize("wt,zt,G,bias", [("u4", "u4", 128, True), ("i4", "none", 1024, False), ("u4", "u8", 128, False)])
+def test_grouped_run_slice_heights(oracle, dev, req, monkeypatch, wt, zt, G, bias):
+    """The grouped prefill kernel's four tile heights (64, 80, 96, 128 rows; OVFCC_PREFILL_ROWS) over items whose row
+    counts straddle them, K cut in parts or not: every item within the oracle bounds at every height, the same bits
+    at every height that does not change the cut along K, and the height the policy picks for these counts."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    rows = [79, 80, 81, 96, 97, 54, 71, 65, 1, 128]
+    N, K = 512, 1024
+    say(f"grouped slice heights {wt}/{zt} G={G}")
+    cases = [datagen.make_case(760 + i, max(rows), K, N, wt, G, zt, with_bias=bias) for i in range(4)]
+    ws = [fc.CompressedWeights.from_case(dev, c) for c in cases]
+    try:
+        items = [(ws[i % 4], cases[i % 4].x[:m]) for i, m in enumerate(rows)]
+        seen = {}
+        for height in (128, 96, 80, 64):
+            monkeypatch.setenv("OVFCC_PREFILL_ROWS", str(height))
+            ys = req.infer_grouped(items)
+            info = req.last_kernel()
+            assert info["name"] == "fcc_prefill_async_grouped_w4" and info["tile_m"] == height, info
+            for i, (m, y) in enumerate(zip(rows, ys)):
+                c = cases[i % 4]
+                check_parity(oracle, y, oracle_y(oracle, c, x=c.x[:m]), K, f"height {height} item {i} M={m} {info}",
+                             output_rounding_slack=True)
+            seen[height] = (info["split_k"], ys)
+        for height in (96, 80, 64):
+            if seen[height][0] == seen[128][0]:
+                for y, z in zip(seen[height][1], seen[128][1]):
+                    assert np.array_equal(y.view(np.uint16), z.view(np.uint16)), height
+        monkeypatch.delenv("OVFCC_PREFILL_ROWS")
+        req.infer_grouped([(ws[0], cases[0].x[:70]), (ws[1], cases[1].x[:66]), (ws[2], cases[2].x[:75])])
+        assert req.last_kernel()["tile_m"] == 80, req.last_kernel()
+        req.infer_grouped([(ws[0], cases[0].x[:90]), (ws[1], cases[1].x[:66])])
+        assert req.last_kernel()["tile_m"] == 96, req.last_kernel()
+    finally:
+        for w in ws:
+            w.close()
+
+
 def test_grouped_run_falls_back_item_by_item(oracle, dev, req):
     """Items of different shapes, an untiled node, or a forced kernel cannot share a launch: the run still gives
     every item's result (through the ordinary per-node path)."""
