@@ -232,6 +232,14 @@ int main() {
         a.tile_rows = 128;
         CHECK(ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, 0, 256, &p) == 0 && !p.big && p.async_dma && p.tiles_y == 16,
               "grouped: 128-row tiles");
+        // the slice heights of a grouped run: one tile row per slice, whatever the height
+        for (int rows : {64, 80, 96}) {
+            a.tile_rows = rows;
+            a.M = 15 * rows;
+            CHECK(ovfcc::plan_launch(a, OVFCC_KERNEL_PREFILL, 0, 256, &p) == 0 && !p.big && p.async_dma && p.tile_m == rows &&
+                      p.tiles_y == 15 && (int64_t)p.tiles_x * p.tiles_y * p.split_k >= (int64_t)p.grid[0] - p.full_tiles,
+                  "grouped: 64-, 80- and 96-row tiles");
+        }
     }
     // the gate refuses what the kernels cannot index
     ovfcc_fc_desc bad = desc(64, 256, 96, OVFCC_U4, OVFCC_NONE, 0);
