@@ -476,29 +476,6 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
 }
 
 
-// Slice height of a grouped prefill launch over items of these row counts: every item is cut into equal slices of
-// at most that many rows and every slice is one tile.  Measured on a mixture-of-experts layer, a tile of 64 / 80 /
-// 96 rows costs 0.78 / 0.84 / 0.89 of a 128-row tile (the unpack work and the data movement of a tile do not
-// depend on its height), so the height that needs the fewest tiles wins unless a lower one needs no more.
-// mid_ok: tiles of 80 and 96 rows exist (one group per k-block).  OVFCC_PREFILL_ROWS = 64 | 80 | 96 | 128 overrides.
-int rows_cap_for(const int64_t* rows, int n, bool mid_ok) {
-    static const int caps[4] = {64, 80, 96, 128}, cost[4] = {780, 836, 890, 1000};
-    if (const int forced = ovfcc::env_int("OVFCC_PREFILL_ROWS", 0))
-        return forced == 64 ? 64 : ((forced == 80 || forced == 96) && mid_ok) ? forced : ovfcc::kPrefillGroupRows;
-    int best = ovfcc::kPrefillGroupRows;
-    int64_t best_cost = -1;
-    for (int c = 0; c < 4; ++c) {
-        if (!mid_ok && (caps[c] == 80 || caps[c] == 96))
-            continue;
-        int64_t total = 0;
-        for (int i = 0; i < n; ++i)
-            total += (rows[i] + caps[c] - 1) / caps[c] * cost[c];
-        if (best_cost < 0 || total < best_cost)
-            best_cost = total, best = caps[c];
-    }
-    return best;
-}
-
 // ---- mixture-of-experts layers with the routing done on the device --------------------------------------------
 // The grouped launch whose slices the routing kernel cuts: tiled 4-bit experts that the all-asynchronous prefill
 // kernel runs, at most kMaxGroupItems of them (their pointers travel in the routing kernel's arguments).  The
@@ -519,7 +496,7 @@ bool plan_routed(ovfcc_request* r, const ovfcc_weights* w0, int64_t R, int n_exp
     // routing stays under)
     const double avg = (double)R / n_experts;
     const int64_t likely = (int64_t)std::ceil(avg + 2.0 * std::sqrt(avg));
-    int cap = rows_cap_for(&likely, 1, w0->layout.groups_per_kblock == 1);
+    int cap = ovfcc::rows_cap_for(&likely, 1, w0->layout.groups_per_kblock == 1);
     const int64_t n = (R + cap - 1) / cap + n_experts;
     if (n * cap * w0->desc.K * 2 >= ((int64_t)1 << 31) || n > 65535)
         return false;
@@ -1303,7 +1280,7 @@ int ovfcc_fc_run_grouped_device(ovfcc_request* r, const ovfcc_group_item* items,
         std::vector<int64_t> rows(n_items);
         for (int i = 0; i < n_items; ++i)
             rows[i] = items[i].M;
-        rows_cap = rows_cap_for(rows.data(), n_items, w0->layout.groups_per_kblock == 1);
+        rows_cap = ovfcc::rows_cap_for(rows.data(), n_items, w0->layout.groups_per_kblock == 1);
     }
     ovfcc::FcDeviceArgs a;
     std::vector<ovfcc::BatchGroupItem> work;

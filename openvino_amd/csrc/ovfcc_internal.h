@@ -214,6 +214,8 @@ OVFCC_HOST_DEVICE inline RoutedHeader routed_header(int tiles_x, int slices, int
     h.tiles_y = slices, h.split_k = split, h.kb_per_split = per, h.grid = (int)(tiles * split);
     return h;
 }
+// Slice height (64, 80, 96 or 128 rows) of a grouped prefill launch over items of these row counts (plan.cpp).
+int rows_cap_for(const int64_t* rows, int n, bool mid_ok);
 int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const FcDeviceArgs& a, const LaunchPlan& plan,
                                  void* stream, const BatchGroupItem* dev_tab = nullptr,
                                  const RoutedHeader* dev_hdr = nullptr);

@@ -241,6 +241,19 @@ int main() {
                   "grouped: 64-, 80- and 96-row tiles");
         }
     }
+    // slice heights of grouped runs by cost
+    {
+        const int64_t mixtral[8] = {65, 64, 54, 71, 70, 70, 56, 62}, two[2] = {90, 66}, full[4] = {128, 128, 128, 128},
+                      small[2] = {50, 60}, tall[3] = {200, 130, 129}, one[1] = {81};
+        CHECK(ovfcc::rows_cap_for(mixtral, 8, true) == 80, "54-71 rows: 80-row slices");
+        CHECK(ovfcc::rows_cap_for(mixtral, 8, false) == 128, "54-71 rows without the middle heights: 128");
+        CHECK(ovfcc::rows_cap_for(two, 2, true) == 96, "66 and 90 rows: 96");
+        CHECK(ovfcc::rows_cap_for(full, 4, true) == 128, "full tiles: 128");
+        CHECK(ovfcc::rows_cap_for(small, 2, true) == 64, "up to 64 rows: 64");
+        CHECK(ovfcc::rows_cap_for(tall, 3, true) == 80 || ovfcc::rows_cap_for(tall, 3, true) == 128, "tall items: fewest tiles");
+        CHECK(ovfcc::rows_cap_for(one, 1, true) == 96, "81 rows: 96");
+        ++plans;
+    }
     // the gate refuses what the kernels cannot index
     ovfcc_fc_desc bad = desc(64, 256, 96, OVFCC_U4, OVFCC_NONE, 0);
     CHECK(ovfcc::validate_desc(&bad) != 0, "group size must divide K");
