@@ -20,8 +20,12 @@
 //     eight consecutive inputs per dword at 8 (lane >> 4)): a wave reads its 8 bytes per tile back with one
 //     LDS read and unpacks them in registers -- dequantised weights never exist in memory;
 //   - the group scales (and zero-points) of the k-block, 512 (+256) bytes, with the weights.
+// LDS holds the parameter stages first, then the weight stages, then the activation stages.
 // That is 6 to 7 vector-memory instructions per wave and k-block; each one costs the compute unit some
 // 15 cycles that nothing overlaps, which is why weights do not come as four 8-byte register loads per wave.
+// None of them needs vector address arithmetic in the loop: a lane's part of the offset is fixed, the part that
+// advances with the k-block goes in the instruction's scalar offset, and a load past the end of K is switched off
+// by a descriptor of length zero.
 // A wave waits for its own loads (the vector-memory counter is in order); one bare barrier per k-block
 // publishes the activations of this k-block and the weights of the next, and frees the oldest stages (a fence
 // would also wait for the loads meant to stay in flight).
