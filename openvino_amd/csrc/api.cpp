@@ -524,7 +524,7 @@ bool plan_routed(ovfcc_request* r, const ovfcc_weights* w0, int64_t R, int n_exp
 }
 
 int run_routed(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, RoutedLaunch& L,
-               const int* indices_dev, int64_t M, int top_k, int a_batches, int inverse, const void* x_base,
+               const int* indices_dev, int64_t M, int top_k, int a_batches, int inverse, int x_mapped, const void* x_base,
                size_t x_row_bytes, void* y_base, size_t y_row_bytes, int* d_maps, ovfcc::RoutedHeader* d_header) {
     auto* d_table = reinterpret_cast<ovfcc::BatchGroupItem*>(d_header + 1);
     ovfcc::ExpertPointers ptrs{};
@@ -532,7 +532,9 @@ int run_routed(ovfcc_request* r, const ovfcc_weights* const* experts, int n_expe
         ptrs.w[e] = experts[e]->d_w, ptrs.scale[e] = experts[e]->d_scale, ptrs.zp[e] = experts[e]->d_zp,
         ptrs.bias[e] = experts[e]->d_bias;
     const int64_t R = M * top_k;
-    int e1 = ovfcc::launch_moe_route(indices_dev, M, top_k, n_experts, a_batches, inverse, L.cap, ptrs, x_base,
+    L.args.row_map = x_mapped ? d_maps : nullptr;
+    L.args.x_rows = x_mapped ? (int64_t)a_batches * M : 0;
+    int e1 = ovfcc::launch_moe_route(indices_dev, M, top_k, n_experts, a_batches, inverse, L.cap, x_mapped, ptrs, x_base,
                                      x_row_bytes, y_base, y_row_bytes, d_maps, d_maps + R, d_table, L.n_slices, d_header,
                                      L.plan.tiles_x, (int)experts[0]->layout.k_blocks, L.plan.n_cus, r->stream);
     if (e1)
@@ -627,17 +629,15 @@ int gather_matmul_routed(ovfcc_request* r, const ovfcc_weights* const* experts, 
             return rc;
         indices_dev = reinterpret_cast<const int32_t*>(base + i_off);
     }
-    rc = run_routed(r, experts, n_experts, L, indices_dev, M, top_k, a_batches, 0, base, (size_t)K * 2, base + y_off,
+    // (the grouped launch reads the rows of A through the map: no gathered copy)
+    rc = run_routed(r, experts, n_experts, L, indices_dev, M, top_k, a_batches, 0, 1, a_dev, (size_t)K * 2, base + y_off,
                     (size_t)N_out * out_bytes, d_maps, d_table);
     if (rc)
         return rc;
-    int e1 = ovfcc::launch_rows(base, a_dev, d_maps, nullptr, (int)R, (int)(K * 2), r->stream);
-    if (e1)
-        return hip_fail((hipError_t)e1, "row gather launch");
     rc = launch_routed(r, L, d_table);
     if (rc)
         return rc;
-    e1 = ovfcc::launch_rows(y_dev, base + y_off, nullptr, d_maps + R, (int)R, (int)(N_out * out_bytes), r->stream);
+    int e1 = ovfcc::launch_rows(y_dev, base + y_off, nullptr, d_maps + R, (int)R, (int)(N_out * out_bytes), r->stream);
     if (e1)
         return hip_fail((hipError_t)e1, "row scatter launch");
     *ran = true;
@@ -677,22 +677,20 @@ int moe_routed(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfc
         indices_dev = reinterpret_cast<const int32_t*>(base + i_off);
     }
     // the routing kernel runs once per projection: same buckets and maps, a slice table each
-    rc = run_routed(r, gate_up, n_experts, Lg, indices_dev, M, top_k, 1, 1, base, (size_t)H * 2, base + h_off,
+    // (gate/up read the hidden states through the map: no gathered copy of them)
+    rc = run_routed(r, gate_up, n_experts, Lg, indices_dev, M, top_k, 1, 1, 1, x_dev, (size_t)H * 2, base + h_off,
                     (size_t)I * 2, d_maps, tab_g);
     if (!rc)
-        rc = run_routed(r, down, n_experts, Ld, indices_dev, M, top_k, 1, 1, base + h_off, (size_t)I * 2, base + d_off,
+        rc = run_routed(r, down, n_experts, Ld, indices_dev, M, top_k, 1, 1, 0, base + h_off, (size_t)I * 2, base + d_off,
                         (size_t)H * (d_f32 ? 4 : 2), d_maps, tab_d);
     if (rc)
         return rc;
-    int e1 = ovfcc::launch_rows(base, x_dev, d_maps, nullptr, (int)R, (int)(H * 2), r->stream);
-    if (e1)
-        return hip_fail((hipError_t)e1, "row gather launch");
     rc = launch_routed(r, Lg, tab_g);
     if (!rc)
         rc = launch_routed(r, Ld, tab_d);
     if (rc)
         return rc;
-    e1 = ovfcc::launch_moe_combine(y_dev, base + d_off, routing_dev, d_maps + R, (int)M, top_k, (int)H, d_f32, d_f32,
+    const int e1 = ovfcc::launch_moe_combine(y_dev, base + d_off, routing_dev, d_maps + R, (int)M, top_k, (int)H, d_f32, d_f32,
                                    r->stream);
     if (e1)
         return hip_fail((hipError_t)e1, "expert combine launch");

@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void fcc_moe_combine_kernel(void* __restrict__
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restrict__ indices, int R, int M, int top_k,
                                                             int n_experts, int a_batches, int inverse, int cap,
-                                                            ExpertPointers experts, const char* x_base,
+                                                            int x_mapped, ExpertPointers experts, const char* x_base,
                                                             size_t x_row_bytes, char* y_base, size_t y_row_bytes,
                                                             int* __restrict__ first, int* __restrict__ second,
                                                             BatchGroupItem* __restrict__ table, int n_slices_max,
@@ -242,10 +242,10 @@ __global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restric
     for (int t = tid; t < slices; t += 256) {
         BatchGroupItem it;
         it.w = experts.w[e], it.scale = experts.scale[e], it.zp = experts.zp[e], it.bias = experts.bias[e];
-        it.x = x_base + (size_t)(start + t * step) * x_row_bytes;
+        it.x = x_mapped ? x_base : x_base + (size_t)(start + t * step) * x_row_bytes;
         it.y = y_base + (size_t)(start + t * step) * y_row_bytes;
         it.M = min(step, count - t * step);
-        it.reserved = 0;
+        it.reserved = x_mapped ? start + t * step : 0;
         table[slice_s + t] = it;
     }
     // the last workgroup closes what no bucket owns: the slices beyond the last one, and the slots beyond the
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restric
 }
 
 int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts, int a_batches, int inverse, int cap,
-                     const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
+                     int x_mapped, const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
                      size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
                      RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream) {
     const int64_t R = M * top_k;
@@ -275,7 +275,7 @@ int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts
         tiles_x < 1 || kb_total < 1 || n_cus < 1)
         return (int)hipErrorInvalidValue;
     hipLaunchKernelGGL(fcc_moe_route_kernel, dim3((unsigned)n_experts), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       indices_dev, (int)R, (int)M, top_k, n_experts, a_batches, inverse, cap, experts,
+                       indices_dev, (int)R, (int)M, top_k, n_experts, a_batches, inverse, cap, x_mapped, experts,
                        static_cast<const char*>(x_base), x_row_bytes, static_cast<char*>(y_base), y_row_bytes, first,
                        second, table, n_slices_max, header, tiles_x, kb_total, n_cus);
     return (int)hipGetLastError();

@@ -77,7 +77,8 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
                                                    const half_t* __restrict__ bias, void* __restrict__ y,
                                                    float* __restrict__ ws, unsigned* __restrict__ counters, int M, int N,
                                                    int K, int kb_total, int kb_per_group, int ng, int zp_const,
-                                                   int out_f32, int glu, const TileWork wk) {
+                                                   int out_f32, int glu, const TileWork wk,
+                                                   const int* __restrict__ row_map = nullptr, int x_rows = 0) {
     static_assert(NT == 8 || NT == 6 || NT == 5 || NT == 4, "tiles of 128, 96, 80 or 64 rows");
     static_assert(GPB == 1 || ((GPB == 2 || GPB == 4) && PRESCALE), "several groups per k-block: scales go into the weights");
     constexpr int PB = PA_P_BYTES * GPB;  // parameter bytes per stage
@@ -111,7 +112,7 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
     const int nt0 = n0 / 16;  // the workgroup's 16 channel tiles
     auto live = [&](int kb, int bytes) { return kb < kb_hi ? bytes : 0; };
 #define PA_DESC_X(kb) \
-    __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, live(kb, M * K * 2), kRsrcFlags)
+    __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x), 0, live(kb, (row_map ? x_rows : M) * K * 2), kRsrcFlags)
 #define PA_DESC_W(kb)                                                                                  \
     __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4_t*>(wt + (size_t)nt0 * kb_total * 64), 0,        \
                                       live(kb, 16 * kb_total * kTileBytes), kRsrcFlags)
@@ -131,8 +132,16 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
 #pragma unroll
     for (int i = 0; i < AL; ++i) {
         const int r0 = 4 * AL * wave + 4 * i;  // first of the load's four rows, uniform
-        a_voff[i] = ((unsigned)((m0 + r0 + (lane >> 4)) * K) * 2u + ((unsigned)((lane & 15) ^ (lane >> 4) ^ (r0 & 15)) << 4)) |
-                    (r0 >= 16 * NT ? kOob : 0u);
+        int row = m0 + r0 + (lane >> 4);
+        unsigned dead = r0 >= 16 * NT ? kOob : 0u;
+        if (row_map) {
+            // the slice gathers its rows itself: row_map[.] names the row of x; rows past the slice and entries that
+            // name no row are switched off here (the descriptor spans the whole of x)
+            const int src = row < M ? row_map[row] : -1;
+            dead |= src < 0 ? kOob : 0u;
+            row = src < 0 ? 0 : src;
+        }
+        a_voff[i] = ((unsigned)(row * K) * 2u + ((unsigned)((lane & 15) ^ (lane >> 4) ^ (r0 & 15)) << 4)) | dead;
     }
     auto dma_a = [&](int kb, int stage, int i) {
         { const __amdgpu_buffer_rsrc_t d_ = PA_DESC_X(kb); __builtin_amdgcn_raw_ptr_buffer_load_lds(d_,
@@ -421,7 +430,8 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const Ba
                                                                         int kb_total, int kb_per_group, int ng,
                                                                         int zp_const, int out_f32, int glu,
                                                                         int tiles_x, int tiles_y, int full_tiles,
-                                                                        int tail_split, int kb_per_split) {
+                                                                        int tail_split, int kb_per_split,
+                                                                        const int* __restrict__ row_map, int x_rows) {
     // the table travels in the kernel arguments, or -- when the rows were bucketed on the device -- lies in memory,
     // with the slice count and the cut along K that the routing kernel chose for it
     if (dev_tab) {
@@ -444,7 +454,9 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const Ba
     prefill_async_body<ZP_TABLE, PRESCALE, NT, GPB>((const uint4_t*)it.w, (const half_t*)it.scale,
                                                     (const uint8_t*)it.zp, (const half_t*)it.x, (const half_t*)it.bias,
                                                     it.y, ws, counters, it.M, N, K, kb_total, kb_per_group, ng, zp_const,
-                                                    out_f32, glu, wk);
+                                                    out_f32, glu, wk,
+                                                    row_map ? row_map + __builtin_amdgcn_readfirstlane(it.reserved) : nullptr,
+                                                    x_rows);
 }
 
 template <typename Kern>
@@ -506,7 +518,7 @@ static int launch_async_grouped_gpb(const BatchGroupTable& tab, const BatchGroup
     hipLaunchKernelGGL(kern, dim3(p.grid[0], p.grid[1], p.grid[2]), dim3(512), pa_lds_bytes(NT, GPB), s, tab, dev_tab,
                        dev_hdr, a.workspace, a.counters, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.kblocks_per_group, (int)L.groups,
                        L.zp_const, a.out_f32, L.glu, p.tiles_x, p.tiles_y, p.full_tiles, p.split_k,
-                       p.kblocks_per_split);
+                       p.kblocks_per_split, a.row_map, (int)a.x_rows);
     return (int)hipGetLastError();
 }
 
@@ -550,7 +562,8 @@ int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const 
                                  void* stream, const BatchGroupItem* dev_tab, const RoutedHeader* dev_hdr) {
     hipStream_t s = static_cast<hipStream_t>(stream);
     const Layout& L = a.layout;
-    if (L.bits != 4 || n_items < 1 || p.tiles_y != n_items || !dev_tab != !dev_hdr)
+    if (L.bits != 4 || n_items < 1 || p.tiles_y != n_items || !dev_tab != !dev_hdr ||
+        (a.row_map && (!dev_tab || a.x_rows < 1 || a.x_rows * a.K * 2 >= ((int64_t)1 << 31))))
         return (int)hipErrorInvalidValue;
     if (!dev_tab) {
         if (!async_plan_ok(a, p) || n_items > kMaxGroupItems)

@@ -112,6 +112,10 @@ struct FcDeviceArgs {
     int64_t N_out;       // row length of y: N, or N / 2 with a gated-linear-unit epilogue
     int gate_offset, up_offset;  // untiled layout with such an epilogue: first gate / up channel
     int tile_rows = 0;   // async prefill kernel: 64 or 128 (grouped runs: also 80, 96) forces the tile height, 0 leaves it to the planner
+    // grouped prefill launch whose slices gather their rows themselves: row_map[item.reserved + r] is the row of item.x
+    // that slice row r reads (negative: none); x_rows = rows of that matrix.  Null: slices read contiguous rows.
+    const int* row_map = nullptr;
+    int64_t x_rows = 0;
     bool want_async = false;  // take the all-asynchronous prefill kernel wherever it can run the node, also where
                               // smaller tiles would spread a small node further (a slice table in device memory
                               // has no other reader)
@@ -180,7 +184,7 @@ struct BatchGroupItem {
     const void* x;
     void* y;
     int M;  // rows of this problem (0 = skip), at most kDecodeMaxRows (decode) or kPrefillGroupRows (prefill)
-    int reserved;
+    int reserved;  // with a row map (FcDeviceArgs::row_map): the map entry of the slice's first row; else 0
 };
 struct BatchGroupTable {
     BatchGroupItem item[kMaxGroupItems];
@@ -233,8 +237,10 @@ struct ExpertPointers {
     const void* zp[kMaxGroupItems];
     const void* bias[kMaxGroupItems];
 };
+// x_mapped != 0: the slices leave the gather to the grouped launch -- every entry gets x = x_base and reserved = its
+// first bucket slot, and the launch reads its rows through `first`.
 int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts, int a_batches, int inverse, int cap,
-                     const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
+                     int x_mapped, const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
                      size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
                      RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream);
 // GroupedMatMul with offsets in device memory: table[0 .. n_slices_max) and *header as for launch_moe_route, from
