@@ -525,7 +525,8 @@ bool plan_routed(ovfcc_request* r, const ovfcc_weights* w0, int64_t R, int n_exp
 
 int run_routed(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, RoutedLaunch& L,
                const int* indices_dev, int64_t M, int top_k, int a_batches, int inverse, int x_mapped, const void* x_base,
-               size_t x_row_bytes, void* y_base, size_t y_row_bytes, int* d_maps, ovfcc::RoutedHeader* d_header) {
+               size_t x_row_bytes, void* y_base, size_t y_row_bytes, int* d_maps, ovfcc::RoutedHeader* d_header,
+               const ovfcc::SecondTable* second_table = nullptr) {
     auto* d_table = reinterpret_cast<ovfcc::BatchGroupItem*>(d_header + 1);
     ovfcc::ExpertPointers ptrs{};
     for (int e = 0; e < n_experts; ++e)
@@ -536,7 +537,8 @@ int run_routed(ovfcc_request* r, const ovfcc_weights* const* experts, int n_expe
     L.args.x_rows = x_mapped ? (int64_t)a_batches * M : 0;
     int e1 = ovfcc::launch_moe_route(indices_dev, M, top_k, n_experts, a_batches, inverse, L.cap, x_mapped, ptrs, x_base,
                                      x_row_bytes, y_base, y_row_bytes, d_maps, d_maps + R, d_table, L.n_slices, d_header,
-                                     L.plan.tiles_x, (int)experts[0]->layout.k_blocks, L.plan.n_cus, r->stream);
+                                     L.plan.tiles_x, (int)experts[0]->layout.k_blocks, L.plan.n_cus, r->stream,
+                                     second_table);
     if (e1)
         return hip_fail((hipError_t)e1, "routing kernel launch");
     return OVFCC_OK;
@@ -678,11 +680,25 @@ int moe_routed(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfc
     }
     // the routing kernel runs once per projection: same buckets and maps, a slice table each
     // (gate/up read the hidden states through the map: no gathered copy of them)
-    rc = run_routed(r, gate_up, n_experts, Lg, indices_dev, M, top_k, 1, 1, 1, x_dev, (size_t)H * 2, base + h_off,
-                    (size_t)I * 2, d_maps, tab_g);
-    if (!rc)
-        rc = run_routed(r, down, n_experts, Ld, indices_dev, M, top_k, 1, 1, 0, base + h_off, (size_t)I * 2, base + d_off,
-                        (size_t)H * (d_f32 ? 4 : 2), d_maps, tab_d);
+    if (n_experts <= ovfcc::kMaxSecondTableItems && Lg.cap == Ld.cap && Lg.n_slices == Ld.n_slices) {
+        // one routing launch writes both slice tables: the buckets are the same, the down projection reads the
+        // bucket slots of the gate/up results in place
+        ovfcc::SecondTable t2{};
+        for (int e = 0; e < n_experts; ++e)
+            t2.w[e] = down[e]->d_w, t2.scale[e] = down[e]->d_scale, t2.zp[e] = down[e]->d_zp, t2.bias[e] = down[e]->d_bias;
+        t2.x_base = base + h_off, t2.x_row_bytes = (size_t)I * 2;
+        t2.y_base = base + d_off, t2.y_row_bytes = (size_t)H * (d_f32 ? 4 : 2);
+        t2.table = reinterpret_cast<ovfcc::BatchGroupItem*>(tab_d + 1), t2.header = tab_d;
+        t2.tiles_x = Ld.plan.tiles_x, t2.kb_total = (int)d0->layout.k_blocks;
+        rc = run_routed(r, gate_up, n_experts, Lg, indices_dev, M, top_k, 1, 1, 1, x_dev, (size_t)H * 2, base + h_off,
+                        (size_t)I * 2, d_maps, tab_g, &t2);
+    } else {
+        rc = run_routed(r, gate_up, n_experts, Lg, indices_dev, M, top_k, 1, 1, 1, x_dev, (size_t)H * 2, base + h_off,
+                        (size_t)I * 2, d_maps, tab_g);
+        if (!rc)
+            rc = run_routed(r, down, n_experts, Ld, indices_dev, M, top_k, 1, 1, 0, base + h_off, (size_t)I * 2,
+                            base + d_off, (size_t)H * (d_f32 ? 4 : 2), d_maps, tab_d);
+    }
     if (rc)
         return rc;
     rc = launch_routed(r, Lg, tab_g);

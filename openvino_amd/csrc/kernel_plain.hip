@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restric
                                                             int* __restrict__ first, int* __restrict__ second,
                                                             BatchGroupItem* __restrict__ table, int n_slices_max,
                                                             RoutedHeader* __restrict__ header, int tiles_x,
-                                                            int kb_total, int n_cus) {
+                                                            int kb_total, int n_cus, SecondTable t2) {
     __shared__ int hist[kMaxGroupItems];
     __shared__ int wave_total[4];
     __shared__ int start_s, slice_s, total_slices_s, total_pairs_s;
@@ -247,15 +247,27 @@ __global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restric
         it.M = min(step, count - t * step);
         it.reserved = x_mapped ? start + t * step : 0;
         table[slice_s + t] = it;
+        if (t2.table) {
+            it.w = t2.w[e], it.scale = t2.scale[e], it.zp = t2.zp[e], it.bias = t2.bias[e];
+            it.x = static_cast<const char*>(t2.x_base) + (size_t)(start + t * step) * t2.x_row_bytes;
+            it.y = static_cast<char*>(t2.y_base) + (size_t)(start + t * step) * t2.y_row_bytes;
+            it.reserved = 0;
+            t2.table[slice_s + t] = it;
+        }
     }
     // the last workgroup closes what no bucket owns: the slices beyond the last one, and the slots beyond the
     // last pair (there are some when an index named no expert)
     if (e == n_experts - 1) {
-        if (tid == 0)
+        if (tid == 0) {
             *header = routed_header(tiles_x, total_slices_s, kb_total, n_cus);
+            if (t2.table)
+                *t2.header = routed_header(t2.tiles_x, total_slices_s, t2.kb_total, n_cus);
+        }
         for (int t = total_slices_s + tid; t < n_slices_max; t += 256) {
             BatchGroupItem it{};
             table[t] = it;
+            if (t2.table)
+                t2.table[t] = it;
         }
         for (int slot = total_pairs_s + tid; slot < R; slot += 256) {
             first[slot] = -1;
@@ -268,8 +280,15 @@ __global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restric
 int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts, int a_batches, int inverse, int cap,
                      int x_mapped, const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
                      size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
-                     RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream) {
+                     RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream,
+                     const SecondTable* second_table) {
     const int64_t R = M * top_k;
+    SecondTable t2{};
+    if (second_table) {
+        t2 = *second_table;
+        if (n_experts > kMaxSecondTableItems || !t2.table || !t2.header || t2.tiles_x < 1 || t2.kb_total < 1)
+            return (int)hipErrorInvalidValue;
+    }
     if (R <= 0 || R > ((int64_t)1 << 24) || n_experts < 1 || n_experts > kMaxGroupItems || cap < 1 ||
         n_slices_max < (R + cap - 1) / cap + n_experts || (a_batches != 1 && a_batches != top_k) || !header ||
         tiles_x < 1 || kb_total < 1 || n_cus < 1)
@@ -277,7 +296,7 @@ int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts
     hipLaunchKernelGGL(fcc_moe_route_kernel, dim3((unsigned)n_experts), dim3(256), 0, static_cast<hipStream_t>(stream),
                        indices_dev, (int)R, (int)M, top_k, n_experts, a_batches, inverse, cap, x_mapped, experts,
                        static_cast<const char*>(x_base), x_row_bytes, static_cast<char*>(y_base), y_row_bytes, first,
-                       second, table, n_slices_max, header, tiles_x, kb_total, n_cus);
+                       second, table, n_slices_max, header, tiles_x, kb_total, n_cus, t2);
     return (int)hipGetLastError();
 }
 

@@ -237,12 +237,30 @@ struct ExpertPointers {
     const void* zp[kMaxGroupItems];
     const void* bias[kMaxGroupItems];
 };
+// A second slice table from the same buckets, written by the same launch (the down projection of an expert block,
+// whose rows are the bucket slots themselves): its own expert pointers, buffers, strides and header.  table == null:
+// none.  At most kMaxSecondTableItems experts, so that both pointer sets fit the kernel arguments.
+constexpr int kMaxSecondTableItems = 32;
+struct SecondTable {
+    const void* w[kMaxSecondTableItems];
+    const void* scale[kMaxSecondTableItems];
+    const void* zp[kMaxSecondTableItems];
+    const void* bias[kMaxSecondTableItems];
+    const void* x_base;
+    size_t x_row_bytes;
+    void* y_base;
+    size_t y_row_bytes;
+    BatchGroupItem* table;
+    RoutedHeader* header;
+    int tiles_x, kb_total;
+};
 // x_mapped != 0: the slices leave the gather to the grouped launch -- every entry gets x = x_base and reserved = its
 // first bucket slot, and the launch reads its rows through `first`.
 int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts, int a_batches, int inverse, int cap,
                      int x_mapped, const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
                      size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
-                     RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream);
+                     RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream,
+                     const SecondTable* second_table = nullptr);
 // GroupedMatMul with offsets in device memory: table[0 .. n_slices_max) and *header as for launch_moe_route, from
 // cumulative row ends over rows that are already contiguous per group; rows of y from the last offset on are
 // zeroed; tail: one int of scratch.
