@@ -416,12 +416,13 @@ def floors_table(dev, req, args) -> int:
           f"fcc_gemv_w4 {total_kernel:.1f} us = {block_bytes / total_kernel / 1e3:.0f} GB/s "
           f"({100 * block_bytes / total_kernel / 1e3 / HBM_PEAK_GBS:.1f} %)")
     # what the matrix cores sustain with nothing else to do (the chip lowers its clock under this load)
-    print("\n| matrix-core loop (v_mfma_f32_16x16x32_f16 on registers, all compute units) | TFLOP/s | of 2.5 PFLOP/s |")
+    print("\n| matrix-core loop on registers, all compute units | TFLOP/s | of 2.5 PFLOP/s |")
     print("|---|---|---|")
-    for waves, valu in ((4, 0), (8, 0), (8, 2), (8, 3), (8, 4)):
-        tf = max(dev.mfma_ceiling(waves, valu) for _ in range(2))
-        print(f"| {waves // 4} wave(s) per SIMD, {valu} packed-f16 multiplications after every MFMA | {tf:.0f} | "
-              f"{100 * tf / 2500:.1f} % |")
+    for shape, name in ((0, "v_mfma_f32_16x16x32_f16"), (1, "v_mfma_f32_32x32x16_f16")):
+        for waves, valu in ((4, 0), (8, 0), (8, 2), (8, 3), (8, 4)):
+            tf = max(dev.mfma_ceiling(waves, valu, shape=shape) for _ in range(2))
+            print(f"| {name}, {waves // 4} wave(s) per SIMD, {valu} packed-f16 multiplications per 16 x 16 x 32 of "
+                  f"matrix work | {tf:.0f} | {100 * tf / 2500:.1f} % |")
     for ptr in (arena, x_dev, y_dev):
         dev.free(ptr)
     req.close()

@@ -1,8 +1,9 @@
 /*
- * ovfcc_bench -- timing helpers of the benchmark driver.  Not part of the drop-in boundary: nothing in the
- * OpenVINO sources corresponds to them and an integration does not bind them.  They live in the library because
- * the timed region has to be bracketed by HIP events on the very stream the kernels are launched on, which a
- * host without HIP (the Python benchmark) cannot do itself.
+ * ovfcc_bench -- timing helpers of the benchmark driver, exported by libovfcc_bench.so (built beside libovfcc.so,
+ * which it links; the product library carries none of them and none of their probe kernels).  Not part of the
+ * drop-in boundary: nothing in the OpenVINO sources corresponds to them and an integration does not bind them.
+ * They are native code because the timed region has to be bracketed by HIP events on the very stream the kernels
+ * are launched on, which a host without HIP (the Python benchmark) cannot do itself.
  */
 #ifndef OVFCC_BENCH_H
 #define OVFCC_BENCH_H
@@ -39,11 +40,12 @@ int ovfcc_bench_floor(ovfcc_ctx* ctx, const void* arena_dev, size_t arena_bytes,
                       int kib_per_wave, int iters, float* elapsed_ms);
 
 /* Matrix-core ceiling: one workgroup per compute unit with `waves` waves (4 or 8: one or two per SIMD), every
- * wave `rounds` times eight independent v_mfma_f32_16x16x32_f16 on registers, each followed by `valu` (0..4)
- * packed-f16 vector multiplications on other registers; no memory traffic.  Timed with HIP events; *flops is the
- * matrix-core work of the timed launch (2 * 16 * 16 * 32 per instruction).  What the chip sustains under that load
- * (it lowers its clock) is the ceiling the prefill kernels are measured against beside the nominal peak. */
-int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int rounds, float* elapsed_ms, double* flops);
+ * wave `rounds` times eight independent v_mfma_f32_16x16x32_f16 (shape 0) or four independent
+ * v_mfma_f32_32x32x16_f16 (shape 1; the same matrix-core work) on registers, each followed by `valu` (0..4; twice
+ * that for shape 1) packed-f16 vector multiplications on other registers; no memory traffic.  Timed with HIP
+ * events; *flops is the matrix-core work of the timed launch.  What the chip sustains under that load (it lowers
+ * its clock) is the ceiling the prefill kernels are measured against beside the nominal peak. */
+int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int shape, int rounds, float* elapsed_ms, double* flops);
 
 #ifdef __cplusplus
 }

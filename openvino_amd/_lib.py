@@ -1,4 +1,5 @@
-"""ctypes binding of the C ABI declared in include/ovfcc.h."""
+"""ctypes binding of the C ABI declared in include/ovfcc.h and include/ovfcc_graph.h (libovfcc.so) and of the
+benchmark helpers declared in include/ovfcc_bench.h (libovfcc_bench.so)."""
 from __future__ import annotations
 
 import ctypes
@@ -6,6 +7,7 @@ import os
 
 PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG, "libovfcc.so")
+BENCH_LIB_PATH = os.path.join(PKG, "libovfcc_bench.so")
 
 OK, EINVAL, EUNSUPPORTED, EDEVICE, ENOMEM = 0, -1, -2, -3, -4
 NONE, U4, I4, U8, I8, F16, F32 = range(7)
@@ -17,13 +19,16 @@ DYNQUANT_I8 = 8                                                        # OVFCC_D
 W_INPUT_MAJOR = 16
 DYNQUANT_PER_GROUP = 32                                                # OVFCC_DYNQUANT_PER_GROUP                                                     # OVFCC_W_INPUT_MAJOR
 
-# every symbol include/ovfcc.h declares
+# every symbol include/ovfcc_bench.h declares (libovfcc_bench.so)
+BENCH_SYMBOLS = ["ovfcc_bench_layers", "ovfcc_bench_grouped", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_bench_mfma"]
+
+# every symbol include/ovfcc.h and include/ovfcc_graph.h declare (libovfcc.so)
 SYMBOLS = [
     "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_glu", "ovfcc_weights_export_size", "ovfcc_weights_export", "ovfcc_weights_import", "ovfcc_weights_destroy",
     "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
-    "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_device_static", "ovfcc_fc_run_grouped_device", "ovfcc_grouped_matmul_device", "ovfcc_grouped_matmul_offsets_device", "ovfcc_gather_matmul_device", "ovfcc_gather_matmul_routed_device", "ovfcc_moe_device", "ovfcc_moe_routed_device", "ovfcc_bench_grouped", "ovfcc_request_sync", "ovfcc_request_force_kernel",
-    "ovfcc_last_kernel_info", "ovfcc_bench_layers", "ovfcc_device_malloc", "ovfcc_device_free",
-    "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_memcpy_d2d", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_bench_mfma", "ovfcc_desc_validate", "ovfcc_env_reload", "ovfcc_tiled_sizes",
+    "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_device_static", "ovfcc_fc_run_grouped_device", "ovfcc_grouped_matmul_device", "ovfcc_grouped_matmul_offsets_device", "ovfcc_gather_matmul_device", "ovfcc_gather_matmul_routed_device", "ovfcc_moe_device", "ovfcc_moe_routed_device", "ovfcc_request_sync", "ovfcc_request_force_kernel",
+    "ovfcc_last_kernel_info", "ovfcc_device_malloc", "ovfcc_device_free",
+    "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_memcpy_d2d", "ovfcc_desc_validate", "ovfcc_env_reload", "ovfcc_tiled_sizes",
     "ovfcc_repack_host", "ovfcc_unrepack_host", "ovfcc_unpack_u4", "ovfcc_unpack_i4", "ovfcc_last_error",
     "ovfcc_version", "ovfcc_fold_match", "ovfcc_fold_model", "ovfcc_fold_gather_matmul", "ovfcc_fold_grouped_matmul", "ovfcc_fold_moe",
 ]
@@ -120,7 +125,12 @@ def load() -> ctypes.CDLL:
         return _lib
     if not os.path.exists(LIB_PATH):
         raise OvfccError(EDEVICE, f"{LIB_PATH} is not built; run python -m openvino_amd.build")
-    L = ctypes.CDLL(LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    # the benchmark helpers live in their own library; they are reached through the same object
+    if os.path.exists(BENCH_LIB_PATH):
+        B = ctypes.CDLL(BENCH_LIB_PATH)
+        for name in BENCH_SYMBOLS:
+            setattr(L, name, getattr(B, name))
     vp, i64, sz, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_size_t, ctypes.c_int
     pp = ctypes.POINTER(ctypes.c_void_p)
     sig = {
@@ -161,7 +171,7 @@ def load() -> ctypes.CDLL:
         "ovfcc_memcpy_d2d": (ci, [vp, vp, vp, sz]),
         "ovfcc_bench_copy": (ci, [vp, vp, vp, sz, ci, ctypes.POINTER(ctypes.c_float)]),
         "ovfcc_bench_floor": (ci, [vp, vp, sz, sz, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_float)]),
-        "ovfcc_bench_mfma": (ci, [vp, ci, ci, ci, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]),
+        "ovfcc_bench_mfma": (ci, [vp, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]),
         "ovfcc_desc_validate": (ci, [ctypes.POINTER(FcDesc)]),
         "ovfcc_env_reload": (None, []),
         "ovfcc_tiled_sizes": (ci, [ctypes.POINTER(FcDesc), ctypes.POINTER(sz), ctypes.POINTER(sz), ctypes.POINTER(sz)]),
@@ -179,6 +189,8 @@ def load() -> ctypes.CDLL:
         "ovfcc_fold_moe": (ci, [ctypes.POINTER(GNode), ci, ci, ctypes.POINTER(MoeFold)]),
     }
     for name, (res, args) in sig.items():
+        if name in BENCH_SYMBOLS and not hasattr(L, name):
+            continue
         fn = getattr(L, name)
         fn.restype = res
         fn.argtypes = args

@@ -12,62 +12,8 @@
 #include <string>
 #include <vector>
 
-#include "ovfcc_bench.h"
+#include "api_types.h"
 #include "ovfcc_internal.h"
-
-struct ovfcc_ctx {
-    int device = 0;
-    int n_cus = 256;
-    std::string arch;
-};
-
-struct ovfcc_weights {
-    ovfcc_ctx* ctx = nullptr;
-    ovfcc_fc_desc desc{};
-    ovfcc::Layout layout;
-    void* d_w = nullptr;
-    void* d_scale = nullptr;
-    void* d_zp = nullptr;
-    void* d_bias = nullptr;
-    void* d_scale_cm = nullptr;  // channel-major copies of the group parameters for the matrix-vector kernel
-    void* d_zp_cm = nullptr;
-    size_t bytes = 0;
-    // Launch plans of recent calls, keyed by what a plan depends on besides the node itself.  Shared by every
-    // request that runs the node, hence the lock; eight entries, replaced in turn.
-    struct PlanEntry {
-        int64_t M = -1;
-        int force_kernel = 0, force_split = 0, n_cus = 0;
-        unsigned env_generation = 0;
-        ovfcc::LaunchPlan plan;
-    };
-    mutable std::mutex plan_mu;
-    mutable PlanEntry plans[8];
-    mutable unsigned plan_next = 0;
-};
-
-struct ovfcc_request {
-    ovfcc_ctx* ctx = nullptr;
-    hipStream_t stream = nullptr;
-    void* d_x = nullptr;
-    void* d_y = nullptr;
-    size_t x_cap = 0, y_cap = 0;
-    void* h_stage = nullptr;   // pinned host memory that small host transfers of ovfcc_fc_run go through: x | y
-    size_t h_stage_cap = 0;
-    float* workspace = nullptr;
-    size_t ws_cap = 0;
-    unsigned* counters = nullptr;
-    size_t counter_cap = 0;
-    void* d_gather = nullptr;  // gather-matmul: gathered rows, results before the scatter, row maps
-    size_t gather_cap = 0;
-    void* d_quant = nullptr;   // dynamic quantisation: int8 activations, inverse scales, sums
-    size_t quant_cap = 0;
-    int* h_maps = nullptr;     // ... and the pinned host copy of the row maps, reused once its upload has finished
-    size_t h_maps_cap = 0;
-    hipEvent_t maps_uploaded = nullptr;
-    int force_kernel = OVFCC_KERNEL_AUTO;
-    int force_split = 0;
-    ovfcc_kernel_info last{};
-};
 
 namespace {
 
@@ -1764,92 +1710,6 @@ int ovfcc_fc_run(ovfcc_request* r, const ovfcc_weights* w, const void* x_host, v
     return OVFCC_OK;
 }
 
-int ovfcc_bench_layers(ovfcc_request* r, const ovfcc_weights* const* layers, int n_layers, const void* x_dev,
-                       void* y_dev, int64_t M, int warmup, int iters, int use_graph, float* elapsed_ms) {
-    if (!r || !layers || n_layers <= 0 || !elapsed_ms || iters <= 0 || warmup < 0)
-        return fail(OVFCC_EINVAL, "bad benchmark arguments");
-    HIP_TRY(hipSetDevice(r->ctx->device));
-    // one eager pass first: sizes the split-K buffers so that nothing allocates inside a capture
-    for (int i = 0; i < n_layers; ++i) {
-        int rc = ovfcc_fc_run_device(r, layers[i], x_dev, y_dev, M);
-        if (rc)
-            return rc;
-    }
-    HIP_TRY(hipStreamSynchronize(r->stream));
-
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t exec = nullptr;
-    if (use_graph) {
-        HIP_TRY(hipStreamBeginCapture(r->stream, hipStreamCaptureModeThreadLocal));
-        int rc = OVFCC_OK;
-        for (int i = 0; i < n_layers && !rc; ++i)
-            rc = ovfcc_fc_run_device(r, layers[i], x_dev, y_dev, M);
-        hipError_t e = hipStreamEndCapture(r->stream, &graph);
-        if (rc)
-            return rc;
-        if (e != hipSuccess)
-            return hip_fail(e, "hipStreamEndCapture");
-        HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
-    }
-    auto one_pass = [&]() -> int {
-        if (use_graph) {
-            HIP_TRY(hipGraphLaunch(exec, r->stream));
-            return OVFCC_OK;
-        }
-        for (int i = 0; i < n_layers; ++i) {
-            int rc = ovfcc_fc_run_device(r, layers[i], x_dev, y_dev, M);
-            if (rc)
-                return rc;
-        }
-        return OVFCC_OK;
-    };
-    int rc = OVFCC_OK;
-    for (int i = 0; i < warmup && !rc; ++i)
-        rc = one_pass();
-    hipEvent_t t0 = nullptr, t1 = nullptr;
-    if (!rc) {
-        HIP_TRY(hipEventCreate(&t0));
-        HIP_TRY(hipEventCreate(&t1));
-        HIP_TRY(hipStreamSynchronize(r->stream));
-        HIP_TRY(hipEventRecord(t0, r->stream));
-        for (int i = 0; i < iters && !rc; ++i)
-            rc = one_pass();
-        HIP_TRY(hipEventRecord(t1, r->stream));
-        HIP_TRY(hipEventSynchronize(t1));
-        HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
-    }
-    if (t0) (void)hipEventDestroy(t0);
-    if (t1) (void)hipEventDestroy(t1);
-    if (exec) (void)hipGraphExecDestroy(exec);
-    if (graph) (void)hipGraphDestroy(graph);
-    return rc;
-}
-
-int ovfcc_bench_grouped(ovfcc_request* r, const ovfcc_group_item* items, int n_items, int warmup, int iters,
-                        float* elapsed_ms) {
-    if (!r || !items || n_items <= 0 || !elapsed_ms || iters <= 0 || warmup < 0)
-        return fail(OVFCC_EINVAL, "bad benchmark arguments");
-    HIP_TRY(hipSetDevice(r->ctx->device));
-    int rc = OVFCC_OK;
-    for (int i = 0; i < warmup + 1 && !rc; ++i)
-        rc = ovfcc_fc_run_grouped_device(r, items, n_items);
-    if (rc)
-        return rc;
-    hipEvent_t t0 = nullptr, t1 = nullptr;
-    HIP_TRY(hipEventCreate(&t0));
-    HIP_TRY(hipEventCreate(&t1));
-    HIP_TRY(hipStreamSynchronize(r->stream));
-    HIP_TRY(hipEventRecord(t0, r->stream));
-    for (int i = 0; i < iters && !rc; ++i)
-        rc = ovfcc_fc_run_grouped_device(r, items, n_items);
-    HIP_TRY(hipEventRecord(t1, r->stream));
-    HIP_TRY(hipEventSynchronize(t1));
-    HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    return rc;
-}
-
 int ovfcc_device_malloc(ovfcc_ctx* ctx, size_t bytes, void** out) {
     if (!ctx || !out)
         return fail(OVFCC_EINVAL, "null argument");
@@ -1887,109 +1747,6 @@ int ovfcc_memcpy_d2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t 
         return fail(OVFCC_EINVAL, "null argument");
     if (bytes)
         HIP_TRY(hipMemcpy(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice));
-    return OVFCC_OK;
-}
-
-int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes, int iters, float* elapsed_ms) {
-    if (!ctx || !dst_dev || !src_dev || !elapsed_ms || iters <= 0 || bytes % 16)
-        return fail(OVFCC_EINVAL, "bad copy benchmark arguments");
-    HIP_TRY(hipSetDevice(ctx->device));
-    hipStream_t s = nullptr;
-    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-    hipEvent_t t0, t1;
-    HIP_TRY(hipEventCreate(&t0));
-    HIP_TRY(hipEventCreate(&t1));
-    int e = ovfcc::launch_copy(dst_dev, src_dev, bytes, s);  // warm-up
-    HIP_TRY(hipStreamSynchronize(s));
-    HIP_TRY(hipEventRecord(t0, s));
-    for (int i = 0; i < iters && !e; ++i)
-        e = ovfcc::launch_copy(dst_dev, src_dev, bytes, s);
-    HIP_TRY(hipEventRecord(t1, s));
-    HIP_TRY(hipEventSynchronize(t1));
-    HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    (void)hipStreamDestroy(s);
-    if (e)
-        return hip_fail((hipError_t)e, "copy kernel launch");
-    return OVFCC_OK;
-}
-
-int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int rounds, float* elapsed_ms, double* flops) {
-    if (!ctx || !elapsed_ms || !flops || rounds <= 0 || (waves != 4 && waves != 8) || valu < 0 || valu > 4)
-        return fail(OVFCC_EINVAL, "bad matrix-core benchmark arguments");
-    HIP_TRY(hipSetDevice(ctx->device));
-    hipStream_t s = nullptr;
-    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-    const int workgroups = ctx->n_cus;
-    float* sink = nullptr;
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&sink), (size_t)workgroups * 64 * waves * sizeof(float)));
-    hipEvent_t t0, t1;
-    HIP_TRY(hipEventCreate(&t0));
-    HIP_TRY(hipEventCreate(&t1));
-    int e = ovfcc::launch_mfma_probe(sink, workgroups, waves, valu, 16, s);  // warm-up
-    HIP_TRY(hipStreamSynchronize(s));
-    HIP_TRY(hipEventRecord(t0, s));
-    if (!e)
-        e = ovfcc::launch_mfma_probe(sink, workgroups, waves, valu, rounds, s);
-    HIP_TRY(hipEventRecord(t1, s));
-    HIP_TRY(hipEventSynchronize(t1));
-    HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    (void)hipFree(sink);
-    (void)hipStreamDestroy(s);
-    if (e)
-        return hip_fail((hipError_t)e, "matrix-core probe launch");
-    *flops = 2.0 * 16 * 16 * 32 * 8.0 * rounds * waves * workgroups;
-    return OVFCC_OK;
-}
-
-// One graph of n_nodes probe launches, replayed `iters` times after three warm-up replays.
-int ovfcc_bench_floor(ovfcc_ctx* ctx, const void* arena_dev, size_t arena_bytes, size_t node_bytes, int n_nodes, int waves,
-                      int kib_per_wave, int iters, float* elapsed_ms) {
-    if (!ctx || !elapsed_ms || n_nodes <= 0 || iters <= 0 || (node_bytes && (!arena_dev || arena_bytes < node_bytes)))
-        return fail(OVFCC_EINVAL, "bad floor benchmark arguments");
-    HIP_TRY(hipSetDevice(ctx->device));
-    hipStream_t s = nullptr;
-    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-    unsigned* out = nullptr;
-    HIP_TRY(hipMalloc(reinterpret_cast<void**>(&out), 256));
-    hipGraph_t graph = nullptr;
-    hipGraphExec_t exec = nullptr;
-    int e = 0;
-    HIP_TRY(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
-    const size_t slices = node_bytes ? arena_bytes / node_bytes : 1;
-    for (int i = 0; i < n_nodes && !e; ++i)
-        e = node_bytes ? ovfcc::launch_stream_probe(static_cast<const char*>(arena_dev) + (size_t)(i % slices) * node_bytes,
-                                                    node_bytes, waves, kib_per_wave, out, s)
-                       : ovfcc::launch_empty(out, s);
-    hipError_t ce = hipStreamEndCapture(s, &graph);
-    if (e || ce != hipSuccess) {
-        if (graph) (void)hipGraphDestroy(graph);
-        (void)hipFree(out);
-        (void)hipStreamDestroy(s);
-        return e ? hip_fail((hipError_t)e, "probe launch") : hip_fail(ce, "graph capture");
-    }
-    HIP_TRY(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
-    hipEvent_t t0, t1;
-    HIP_TRY(hipEventCreate(&t0));
-    HIP_TRY(hipEventCreate(&t1));
-    for (int i = 0; i < 3; ++i)
-        HIP_TRY(hipGraphLaunch(exec, s));
-    HIP_TRY(hipStreamSynchronize(s));
-    HIP_TRY(hipEventRecord(t0, s));
-    for (int i = 0; i < iters; ++i)
-        HIP_TRY(hipGraphLaunch(exec, s));
-    HIP_TRY(hipEventRecord(t1, s));
-    HIP_TRY(hipEventSynchronize(t1));
-    HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
-    (void)hipGraphExecDestroy(exec);
-    (void)hipGraphDestroy(graph);
-    (void)hipFree(out);
-    (void)hipStreamDestroy(s);
     return OVFCC_OK;
 }
 

@@ -1,0 +1,65 @@
+// The objects behind the C ABI's opaque handles.  Private to the library and to the benchmark library that is
+// built from the same tree (it brackets launches with events on a request's own stream).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+#include <string>
+
+#include "ovfcc.h"
+#include "ovfcc_internal.h"
+
+struct ovfcc_ctx {
+    int device = 0;
+    int n_cus = 256;
+    std::string arch;
+};
+
+struct ovfcc_weights {
+    ovfcc_ctx* ctx = nullptr;
+    ovfcc_fc_desc desc{};
+    ovfcc::Layout layout;
+    void* d_w = nullptr;
+    void* d_scale = nullptr;
+    void* d_zp = nullptr;
+    void* d_bias = nullptr;
+    void* d_scale_cm = nullptr;  // channel-major copies of the group parameters for the matrix-vector kernel
+    void* d_zp_cm = nullptr;
+    size_t bytes = 0;
+    // Launch plans of recent calls, keyed by what a plan depends on besides the node itself.  Shared by every
+    // request that runs the node, hence the lock; eight entries, replaced in turn.
+    struct PlanEntry {
+        int64_t M = -1;
+        int force_kernel = 0, force_split = 0, n_cus = 0;
+        unsigned env_generation = 0;
+        ovfcc::LaunchPlan plan;
+    };
+    mutable std::mutex plan_mu;
+    mutable PlanEntry plans[8];
+    mutable unsigned plan_next = 0;
+};
+
+struct ovfcc_request {
+    ovfcc_ctx* ctx = nullptr;
+    hipStream_t stream = nullptr;
+    void* d_x = nullptr;
+    void* d_y = nullptr;
+    size_t x_cap = 0, y_cap = 0;
+    void* h_stage = nullptr;   // pinned host memory that small host transfers of ovfcc_fc_run go through: x | y
+    size_t h_stage_cap = 0;
+    float* workspace = nullptr;
+    size_t ws_cap = 0;
+    unsigned* counters = nullptr;
+    size_t counter_cap = 0;
+    void* d_gather = nullptr;  // gather-matmul: gathered rows, results before the scatter, row maps
+    size_t gather_cap = 0;
+    void* d_quant = nullptr;   // dynamic quantisation: int8 activations, inverse scales, sums
+    size_t quant_cap = 0;
+    int* h_maps = nullptr;     // ... and the pinned host copy of the row maps, reused once its upload has finished
+    size_t h_maps_cap = 0;
+    hipEvent_t maps_uploaded = nullptr;
+    int force_kernel = OVFCC_KERNEL_AUTO;
+    int force_split = 0;
+    ovfcc_kernel_info last{};
+};

@@ -5,9 +5,26 @@
 // reduction, no store -- reads a buffer of a given size under graph replay.  The decode kernels are measured
 // against these: a node cannot finish sooner than an empty one starts and stops, nor move its weights faster
 // than a kernel that does nothing else.
+#include "bench_probe.h"
 #include "device_common.h"
 
 namespace ovfcc {
+
+// Plain 128-bit copy: the yardstick for bandwidth figures and for the scaling of the HBM traffic counters.
+__global__ __launch_bounds__(256) void fcc_copy_kernel(uint4_t* __restrict__ dst, const uint4_t* __restrict__ src,
+                                                       size_t n16) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n16; i += stride)
+        dst[i] = __builtin_nontemporal_load(src + i);
+}
+
+int launch_copy(void* dst, const void* src, size_t bytes, void* stream) {
+    const size_t n16 = bytes / 16;
+    hipLaunchKernelGGL(fcc_copy_kernel, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream), (uint4_t*)dst,
+                       (const uint4_t*)src, n16);
+    return (int)hipGetLastError();
+}
 
 __global__ void fcc_empty_kernel(unsigned* out) {
     if (out && threadIdx.x == 9999)
@@ -46,14 +63,31 @@ __global__ __launch_bounds__(1024) void fcc_stream_probe_kernel(const uint4_t* _
         out[0] = v;
 }
 
+// Operands of the matrix-core loops: four A and four B registers sets per lane, filled from a hash of lane and index
+// with halves of random sign and mantissa and magnitudes between 1/4 and 4 -- on constant operands nothing toggles
+// between consecutive instructions and the chip holds a clock that no real kernel sees.
+__device__ __forceinline__ half8_t probe_operand(unsigned seed) {
+    Frag8 f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        unsigned h = (seed * 4u + i) * 2654435761u;
+        h ^= h >> 15, h *= 2246822519u, h ^= h >> 13;
+        // per half: sign, exponent 13..16 (2^-2 .. 2^1), ten random mantissa bits
+        const unsigned lo = (h & 0x83FFu) | ((13u + ((h >> 10) & 3u)) << 10);
+        const unsigned hi = ((h >> 16) & 0x83FFu) | ((13u + ((h >> 26) & 3u)) << 10);
+        f.u[i] = lo | (hi << 16);
+    }
+    return f.v;
+}
+
 // Every wave runs `iters` rounds of eight independent MFMAs (eight accumulators, operands in registers, no
 // memory traffic), each followed by VALU packed-f16 multiplications on registers the MFMAs do not touch.
 template <int VALU>
 __global__ __launch_bounds__(512) void fcc_mfma_probe_kernel(float* __restrict__ sink, int iters) {
-    half8_t a, b;
+    half8_t a[4], b[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        a[i] = (half_t)(0.001f * (float)(threadIdx.x & 63) + (float)i), b[i] = (half_t)(0.5f * (float)i);
+    for (int i = 0; i < 4; ++i)
+        a[i] = probe_operand(threadIdx.x * 8u + i), b[i] = probe_operand(threadIdx.x * 8u + 4u + i);
     float4_t acc[8];
     uint32_t r[8];
 #pragma unroll
@@ -63,7 +97,7 @@ __global__ __launch_bounds__(512) void fcc_mfma_probe_kernel(float* __restrict__
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a), "v"(b));
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a[j & 3]), "v"(b[(j >> 1) & 3]));
 #pragma unroll
             for (int v = 0; v < VALU; ++v)
                 asm volatile("v_pk_mul_f16 %0, %0, %1" : "+v"(r[(j + v) & 7]) : "v"(c));
@@ -76,12 +110,64 @@ __global__ __launch_bounds__(512) void fcc_mfma_probe_kernel(float* __restrict__
     sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
-// sink: 4 * workgroups * 64 * waves bytes.  valu: 0 to 4 multiplications after every MFMA.
-int launch_mfma_probe(float* sink, int workgroups, int waves, int valu, int iters, void* stream) {
-    if (!sink || workgroups < 1 || (waves != 4 && waves != 8) || valu < 0 || valu > 4 || iters < 1)
+// The same loop with v_mfma_f32_32x32x16_f16: four independent accumulators of sixteen registers, so that one round
+// is the same matrix-core work as the eight 16 x 16 x 32 instructions above (VALU multiplications after each: twice
+// as many, to keep the ratio of vector work to matrix work).
+template <int VALU>
+__global__ __launch_bounds__(512) void fcc_mfma32_probe_kernel(float* __restrict__ sink, int iters) {
+    half8_t a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        a[i] = probe_operand(threadIdx.x * 8u + i), b[i] = probe_operand(threadIdx.x * 8u + 4u + i);
+    float16_t acc[4];
+    uint32_t r[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            acc[i][e] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        r[i] = 0x3c003c00u + (uint32_t)i;
+    const uint32_t c = 0x3c003c00u;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a[j]), "v"(b[(j + 1) & 3]));
+#pragma unroll
+            for (int v = 0; v < 2 * VALU; ++v)
+                asm volatile("v_pk_mul_f16 %0, %0, %1" : "+v"(r[(2 * j + v) & 7]) : "v"(c));
+        }
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            s += acc[i][e];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        s += (float)r[i];
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+// sink: 4 * workgroups * 64 * waves bytes.  valu: 0 to 4 multiplications after every MFMA.  shape 0: 16 x 16 x 32
+// instructions, shape 1: 32 x 32 x 16.
+int launch_mfma_probe(float* sink, int workgroups, int waves, int valu, int shape, int iters, void* stream) {
+    if (!sink || workgroups < 1 || (waves != 4 && waves != 8) || valu < 0 || valu > 4 || iters < 1 || shape < 0 || shape > 1)
         return (int)hipErrorInvalidValue;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 g((unsigned)workgroups), b(64u * waves);
+    if (shape == 1) {
+        switch (valu) {
+        case 0: hipLaunchKernelGGL(fcc_mfma32_probe_kernel<0>, g, b, 0, s, sink, iters); break;
+        case 1: hipLaunchKernelGGL(fcc_mfma32_probe_kernel<1>, g, b, 0, s, sink, iters); break;
+        case 2: hipLaunchKernelGGL(fcc_mfma32_probe_kernel<2>, g, b, 0, s, sink, iters); break;
+        case 3: hipLaunchKernelGGL(fcc_mfma32_probe_kernel<3>, g, b, 0, s, sink, iters); break;
+        default: hipLaunchKernelGGL(fcc_mfma32_probe_kernel<4>, g, b, 0, s, sink, iters); break;
+        }
+        return (int)hipGetLastError();
+    }
     switch (valu) {
     case 0: hipLaunchKernelGGL(fcc_mfma_probe_kernel<0>, g, b, 0, s, sink, iters); break;
     case 1: hipLaunchKernelGGL(fcc_mfma_probe_kernel<1>, g, b, 0, s, sink, iters); break;

@@ -1,4 +1,4 @@
-// Fallback kernel for shapes that keep OpenVINO's constant layout, and the copy yardstick.
+// Fallback kernel for shapes that keep OpenVINO's constant layout, and the small helper kernels of the routed calls.
 // Semantics: the scalar reference kernel of the OpenVINO Intel-GPU plugin
 // (src/plugins/intel_gpu/src/kernel_selector/cl_kernels/fully_connected_gpu_bfyx_ref.cl:88-160).
 #include "device_common.h"
@@ -69,33 +69,6 @@ __global__ __launch_bounds__(64) void fcc_plain_kernel(const uint8_t* __restrict
     }
     if (threadIdx.x == 0)
         store_out(y, (size_t)m * N_out + f, acc, out_f32);
-}
-
-// ------------------------------------------------------------------------------------------------
-// Plain 128-bit copy, the yardstick for bandwidth figures and counter scaling.
-// ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void fcc_copy_kernel(uint4_t* __restrict__ dst, const uint4_t* __restrict__ src,
-                                                       size_t n16) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < n16; i += stride)
-        dst[i] = __builtin_nontemporal_load(src + i);
-}
-
-
-// ------------------------------------------------------------------------------------------------
-// Read-only sweep over a weight buffer: pulls it through L2 into the memory-side Infinity Cache ahead of
-// the kernel that will consume it.
-// ------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void fcc_touch_kernel(const uint4_t* __restrict__ src, size_t n16) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    uint4_t acc = {0, 0, 0, 0};
-    for (; i < n16; i += stride) {
-        const uint4_t v = src[i];
-        acc.x ^= v.x, acc.y ^= v.y, acc.z ^= v.z, acc.w ^= v.w;
-    }
-    asm volatile("" ::"v"(acc.x), "v"(acc.y), "v"(acc.z), "v"(acc.w));  // keeps the loads alive
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -392,26 +365,11 @@ int launch_moe_combine(void* y, const void* d, const void* routing, const int* p
     return (int)hipGetLastError();
 }
 
-int launch_touch(const void* src, size_t bytes, void* stream) {
-    const size_t n16 = bytes / 16;
-    const unsigned blocks = (unsigned)((n16 + 256 * 4 - 1) / (256 * 4));  // four loads per thread
-    hipLaunchKernelGGL(fcc_touch_kernel, dim3(blocks ? blocks : 1), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       (const uint4_t*)src, n16);
-    return (int)hipGetLastError();
-}
-
 int launch_plain(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     hipLaunchKernelGGL(fcc_plain_kernel, dim3(p.grid[0], p.grid[1], 1), dim3(64), 0, static_cast<hipStream_t>(stream),
                        (const uint8_t*)a.w, (const half_t*)a.scale, (const uint8_t*)a.zp, (const half_t*)a.bias,
                        (const half_t*)a.x, a.y, (int)a.M, (int)a.N_out, (int)a.K, (int)a.group_size, a.w_type,
                        a.zp_type, a.zp_scalar, a.out_f32, a.layout.glu, a.gate_offset, a.up_offset);
-    return (int)hipGetLastError();
-}
-
-int launch_copy(void* dst, const void* src, size_t bytes, void* stream) {
-    const size_t n16 = bytes / 16;
-    hipLaunchKernelGGL(fcc_copy_kernel, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream), (uint4_t*)dst,
-                       (const uint4_t*)src, n16);
     return (int)hipGetLastError();
 }
 

@@ -285,17 +285,10 @@ bool prefill_i8w4_applies(const Layout& L, int64_t N, int zp_type);
 int launch_prefill_i8w4(const FcDeviceArgs& a, const void* xq, const float* inv, bool grouped, void* stream);
 // Integer prefill kernel over launch_dynquant's outputs: tiled 8-bit weights, one group per channel, N % 256 == 0.
 int launch_prefill_i8(const FcDeviceArgs& a, const void* xq, const float* inv_scale, const int* qsum, void* stream);
-int launch_copy(void* dst, const void* src, size_t bytes, void* stream);
 // dst[r] = src[src_row[r]] (dst_row null) or dst[dst_row[r]] = src[r] (src_row null), rows of row_bytes % 16 == 0 bytes;
 // the caller guarantees that every index is a row of the buffer it addresses
 int launch_rows(void* dst, const void* src, const int* src_row, const int* dst_row, int rows, int row_bytes,
                 void* stream);
-int launch_touch(const void* src, size_t bytes, void* stream);
-// benchmark probes: an empty kernel, and a loads-only streaming kernel (workgroups of `waves` waves, kib_per_wave
-// KiB per wave, eight loads in flight per wave) over `bytes`
-int launch_empty(unsigned* out, void* stream);
-int launch_mfma_probe(float* sink, int workgroups, int waves, int valu, int iters, void* stream);
-int launch_stream_probe(const void* src, size_t bytes, int waves, int kib_per_wave, unsigned* out, void* stream);
 // y[m, :] = sum_j routing[m, j] * d[pos[m * top_k + j], :], rows of H (a multiple of 4) channels; d f16 or f32
 int launch_moe_combine(void* y, const void* d, const void* routing, const int* pos, int rows, int top_k, int H,
                        int d_f32, int out_f32, void* stream);

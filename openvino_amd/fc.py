@@ -90,11 +90,12 @@ class Device:
                                          kib_per_wave, iters, ctypes.byref(ms)))
         return ms.value * 1e3 / iters / n_nodes
 
-    def mfma_ceiling(self, waves: int = 8, valu: int = 0, rounds: int = 20000) -> float:
-        """TFLOP/s of a loop of nothing but v_mfma_f32_16x16x32_f16 on every compute unit, `waves` waves each (4 or
-        8), with `valu` packed-f16 vector multiplications after every MFMA (ovfcc_bench_mfma)."""
+    def mfma_ceiling(self, waves: int = 8, valu: int = 0, rounds: int = 20000, shape: int = 0) -> float:
+        """TFLOP/s of a loop of nothing but v_mfma_f32_16x16x32_f16 (shape 0) or v_mfma_f32_32x32x16_f16 (shape 1) on
+        every compute unit, `waves` waves each (4 or 8), with `valu` packed-f16 vector multiplications after every
+        16 x 16 x 32 MFMA's worth of work (ovfcc_bench_mfma)."""
         ms, flops = ctypes.c_float(), ctypes.c_double()
-        check(self.lib.ovfcc_bench_mfma(self.handle, waves, valu, rounds, ctypes.byref(ms), ctypes.byref(flops)))
+        check(self.lib.ovfcc_bench_mfma(self.handle, waves, valu, shape, rounds, ctypes.byref(ms), ctypes.byref(flops)))
         return flops.value / (ms.value * 1e-3) / 1e12
 
     def copy_bandwidth(self, nbytes: int = 1 << 30, iters: int = 10) -> float:

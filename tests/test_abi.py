@@ -12,11 +12,11 @@ from openvino_amd import _lib, fc
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    """Every function that include/*.h declares."""
+def declared_symbols(bench: bool):
+    """Every function that include/*.h declares: the benchmark header's, or all the others'."""
     names = set()
     for header in sorted(os.listdir(os.path.join(ROOT, "include"))):
-        if not header.endswith(".h"):
+        if not header.endswith(".h") or (header == "ovfcc_bench.h") != bench:
             continue
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
@@ -25,12 +25,23 @@ def declared_symbols():
 
 
 def test_every_declared_symbol_is_exported():
-    L = _lib.load()
-    names = declared_symbols()
+    _lib.load()
+    product = ctypes.CDLL(_lib.LIB_PATH)
+    names = declared_symbols(bench=False)
     assert len(names) >= 25
     for name in names:
-        assert hasattr(L, name), f"{name} is declared in include/ovfcc.h but not exported"
+        assert hasattr(product, name), f"{name} is declared under include/ but libovfcc.so does not export it"
     assert sorted(_lib.SYMBOLS) == names
+
+
+def test_benchmark_helpers_live_in_their_own_library():
+    _lib.load()
+    product, bench = ctypes.CDLL(_lib.LIB_PATH), ctypes.CDLL(_lib.BENCH_LIB_PATH)
+    names = declared_symbols(bench=True)
+    assert sorted(_lib.BENCH_SYMBOLS) == names
+    for name in names:
+        assert hasattr(bench, name), f"{name} is declared in include/ovfcc_bench.h but libovfcc_bench.so does not export it"
+        assert not hasattr(product, name), f"{name} belongs to the benchmark library, not to libovfcc.so"
 
 
 def test_version_and_error_string():
