@@ -6,8 +6,10 @@ import ctypes
 import os
 
 PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG, "libovfcc.so")
-BENCH_LIB_PATH = os.path.join(PKG, "libovfcc_bench.so")
+# OVFCC_LIB_DIR: a directory with another build of the two libraries (experiments); default: beside this file
+LIB_DIR = os.environ.get("OVFCC_LIB_DIR") or PKG
+LIB_PATH = os.path.join(LIB_DIR, "libovfcc.so")
+BENCH_LIB_PATH = os.path.join(LIB_DIR, "libovfcc_bench.so")
 
 OK, EINVAL, EUNSUPPORTED, EDEVICE, ENOMEM = 0, -1, -2, -3, -4
 NONE, U4, I4, U8, I8, F16, F32 = range(7)

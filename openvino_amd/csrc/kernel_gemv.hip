@@ -27,12 +27,18 @@
 // fetch all C of them with one load; the table is stored in the order the waves use it, [tile][channel][wave][slot]
 // with k-block = wave + NWT slot, which fixes C per node when the node is created.
 //
-// Reduction.  Each wave leaves its M x 16 partial sums in LDS; one wave adds them in wave order (the result does
-// not depend on arrival order), applies bias, gated linear unit and output type, and stores.  Which wave: with
-// TICKET the one that draws the last ticket from an LDS counter (the counter is zeroed behind a barrier that
-// sits right after the loads have been issued, where it waits for no memory) -- best for small workgroups, whose
-// waves then retire one by one; without TICKET wave 0 after a closing barrier -- best for workgroups of eight
-// and more waves, which an early barrier would march in step (down projection: 6.5 against 5.7 us).
+// Reduction.  Each wave leaves its M x 16 partial sums in LDS; one wave adds them -- its four rows of sixteen lanes
+// take every fourth wave's sums each and two register exchanges add the rows, a fixed order that does not depend on
+// arrival -- applies bias, gated linear unit and output type, and stores.  Which wave: with TICKET the one that
+// draws the last ticket from an LDS counter (the counter is zeroed behind a barrier that sits right after the loads
+// have been issued, where it waits for no memory) -- best for small workgroups, whose waves then retire one by one;
+// without TICKET wave 0 after a closing barrier -- best for workgroups of eight and more waves, which an early
+// barrier would march in step (down projection: 6.5 against 5.7 us).
+//
+// What the compiler must not do to the ends of a wave's life (both seen in its output): sink the loads of the group
+// parameters to their only use, the final sums, where they are one more trip to memory behind the last weight
+// tile; and start on the activations after the first two of eight weight loads, so that six leave a round trip
+// late.  Scheduling fences around the load block and an empty asm statement at the point of need prevent both.
 #include "device_common.h"
 
 namespace ovfcc {
@@ -66,6 +72,22 @@ __device__ __forceinline__ float row_sum16(float v) {
     t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xF, 0xF, true);  // row_shr:8
     v += __builtin_bit_cast(float, t);
     return v;
+}
+
+// The value is needed here: keeps the compiler from sinking the load that produced it to a later, conditional use
+// (where it would be one more round trip to memory at the end of a wave's life).
+__device__ __forceinline__ void needed_here(uint32_t& v) {
+    asm volatile("" : "+v"(v));
+}
+__device__ __forceinline__ void needed_here(uint2_t& v) {
+    uint32_t a = v.x, b = v.y;
+    asm volatile("" : "+v"(a), "+v"(b));
+    v = uint2_t{a, b};
+}
+__device__ __forceinline__ void needed_here(uint4_t& v) {
+    uint32_t a = v.x, b = v.y, c = v.z, d = v.w;
+    asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    v = uint4_t{a, b, c, d};
 }
 
 }  // namespace
@@ -143,14 +165,32 @@ __global__ __launch_bounds__(1024) void fcc_gemv_kernel(const uint4_t* __restric
             zv[0] = __builtin_amdgcn_raw_buffer_load_b16(rz, pofs, 0, 0);
         }
     }
+    // (activations and group parameters are requested before the weights: loads return in order)
+    __builtin_amdgcn_sched_barrier(0);
     uint4_t wv[C];
 #pragma unroll
     for (int i = 0; i < C; ++i)
         wv[i] = __builtin_bit_cast(uint4_t,
                                    __builtin_amdgcn_raw_buffer_load_b128(rw, (unsigned)(i * nwt * kTileBytes + lane * 16), 0, 2));
+    // The output and bias pointers are wanted by one wave at the very end; fetched there, the kernel arguments would
+    // be one more wait in the tail.
+    uint64_t bias_bits = reinterpret_cast<uint64_t>(bias), y_bits = reinterpret_cast<uint64_t>(y);
+    asm volatile("" : "+s"(bias_bits), "+s"(y_bits));
+    typedef __attribute__((address_space(1))) const half_t* global_half_ptr;
+    typedef __attribute__((address_space(1))) void* global_void_ptr;
+    const global_half_ptr bias_k = reinterpret_cast<global_half_ptr>(bias_bits);
+    const global_void_ptr y_k = reinterpret_cast<global_void_ptr>(y_bits);
+    auto put = [&](size_t i, float v) {
+        if (out_f32)
+            static_cast<__attribute__((address_space(1))) float*>(y_k)[i] = v;
+        else
+            static_cast<__attribute__((address_space(1))) half_t*>(y_k)[i] = (half_t)v;
+    };
+    // Every load is on its way before anything waits for one: without the fence the compiler starts on the
+    // activations after the first two weight loads and the others leave one memory round trip late.
+    __builtin_amdgcn_sched_barrier(0);
     if constexpr (TICKET) {
         // publishes the zeroed ticket counter; pinned here so that the barrier waits for nothing that has left the chip
-        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -183,6 +223,15 @@ __global__ __launch_bounds__(1024) void fcc_gemv_kernel(const uint4_t* __restric
             if (4 * i + kq < C)
                 *reinterpret_cast<uint4_t*>(xs + m * kRowBytes + (i * 64 + lane) * 16) = p;
         }
+
+    // The group parameters arrived with the activations.  Their only use is the lanes' final sums; left alone, the
+    // compiler moves the loads down to that use, behind the last weight tile.
+    needed_here(sv);
+    if constexpr (ZP_TABLE) {
+        needed_here(zv[0]);
+        if constexpr (C == 8)
+            needed_here(zv[1]);
+    }
 
     // operand address of this lane: row col (rows >= MR repeat row 0, their results are never stored), quarter kq
     const unsigned char* xs_lane = xs + (col < MR ? col : 0) * kRowBytes + kq * 16;
@@ -241,40 +290,61 @@ __global__ __launch_bounds__(1024) void fcc_gemv_kernel(const uint4_t* __restric
         if (lane == 0)
             ticket = __hip_atomic_fetch_add(&arrived, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
         ticket = __builtin_amdgcn_readfirstlane(ticket);
-        if (ticket != (unsigned)(waves - 1) || kq != 0)
+        if (ticket != (unsigned)(waves - 1))
             return;
     } else {
         __syncthreads();
-        if (wave != 0 || kq != 0)
+        if (wave != 0)
             return;
     }
 
+    // The reducing wave's four rows of sixteen lanes each add a quarter of the partial sums (waves g, g + 4, ...:
+    // at most four reads per lane and row, all in flight together), then the rows are added across the wave with two
+    // register exchanges: (g0 + g2) + (g1 + g3), the same order every time.
+    // (The second result of an exchange passes through an empty asm statement: converted straight to a float, this
+    // compiler reads the first result in its place.)
+    auto across_rows = [](float v) {
+        const uint32_t a = __builtin_bit_cast(uint32_t, v);
+        const uint2_t h = __builtin_amdgcn_permlane32_swap(a, a, false, false);  // .x: lanes l & 31, .y: those + 32
+        uint32_t hy = h.y;
+        asm volatile("" : "+v"(hy));
+        const float t = __builtin_bit_cast(float, h.x) + __builtin_bit_cast(float, hy);
+        const uint32_t b = __builtin_bit_cast(uint32_t, t);
+        const uint2_t q = __builtin_amdgcn_permlane16_swap(b, b, false, false);  // .x: even rows, .y: odd rows
+        uint32_t qy = q.y;
+        asm volatile("" : "+v"(qy));
+        return __builtin_bit_cast(float, q.x) + __builtin_bit_cast(float, qy);
+    };
+    // sum over waves first, first + 1, ... first + count - 1 of row r, channel col
+    auto tile_sum = [&](int first, int count, int r) {
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int w = kq + 4 * j;
+            const float v = red[((first + (w < count ? w : 0)) * MR + r) * 16 + col];
+            s += w < count ? v : 0.f;
+        }
+        return across_rows(s);
+    };
     if (glu) {
         // waves 0 .. nwt-1 hold the gate tile, nwt .. 2 nwt-1 the up tile of channels 16 blockIdx.x ..
         const int n = blockIdx.x * 32 + col;  // position of the gate channel in the tiled bias order
-        const float bg = bias ? (float)bias[n] : 0.f, bu = bias ? (float)bias[n + 16] : 0.f;
+        const float bg = bias_k ? (float)bias_k[n] : 0.f, bu = bias_k ? (float)bias_k[n + 16] : 0.f;
 #pragma unroll
         for (int r = 0; r < MR; ++r) {
-            float g = 0.f, u = 0.f;
-            for (int w = 0; w < nwt; ++w) {
-                g += red[(w * MR + r) * 16 + col];
-                u += red[((w + nwt) * MR + r) * 16 + col];
-            }
-            if (r < M)
-                store_out(y, (size_t)r * (N / 2) + blockIdx.x * 16 + col,
-                          glu_value(glu, g * 0x1p24f + bg, u * 0x1p24f + bu), out_f32);
+            const float g = tile_sum(0, nwt, r), u = tile_sum(nwt, nwt, r);
+            if (r < M && kq == 0)
+                put((size_t)r * (N / 2) + blockIdx.x * 16 + col, glu_value(glu, g * 0x1p24f + bg, u * 0x1p24f + bu));
         }
         return;
     }
     const int n = tile * 16 + col;
-    const float b = bias ? (float)bias[n] : 0.f;
+    const float b = bias_k ? (float)bias_k[n] : 0.f;
 #pragma unroll
     for (int r = 0; r < MR; ++r) {
-        float s = 0.f;
-        for (int w = 0; w < waves; ++w)
-            s += red[(w * MR + r) * 16 + col];
-        if (r < M)
-            store_out(y, (size_t)r * N + n, s * 0x1p24f + b, out_f32);
+        const float s = tile_sum(0, waves, r);
+        if (r < M && kq == 0)
+            put((size_t)r * N + n, s * 0x1p24f + b);
     }
 }
 
