@@ -603,6 +603,33 @@ def main() -> int:
     for w in fused_layers:
         w.close()
 
+    # the same block with the gated MLP as one node (gate / up with SwiGLU, then down: the CPU plugin's LLMMLP): q/k/v, o,
+    # mlp.  The node runs as two launches (4 per block); OVFCC_MLP_FUSED=1 selects its one-launch kernel (3 per block).
+    mlp_base = {"qkv": fused_base["qkv"], "o": base["qo"]}
+    glu_node = fc.CompressedWeights.glu(base["gate_up"], base["gate_up"], "swish")
+    mlp_base["mlp"] = fc.CompressedWeights.mlp(glu_node, base["down"])
+    glu_node.close()
+    mlp_layers = [mlp_base[name].clone() for _ in range(args.layers) for name in ("qkv", "o", "mlp")]
+    mlp_modes = {}
+    saved = os.environ.get("OVFCC_MLP_FUSED")
+    for mode, flag in (("two_launches", "0"), ("one_launch", "1")):
+        os.environ["OVFCC_MLP_FUSED"] = flag
+        _lib.sync_env()
+        t = req.bench_layers(mlp_layers, x_dev, y_dev, 1, args.warmup, args.steps, use_graph=not args.no_graph)
+        g = fused_bytes / (t / args.steps * 1e-3) / 1e9
+        mlp_modes[mode] = {"ms_per_pass": round(t / args.steps, 5), "GBps": round(g, 1),
+                           "pct_of_hbm_peak": round(100 * g / HBM_PEAK_GBS, 2), "kernel": req.last_kernel()["name"]}
+        log(f"decode M=1 with q/k/v fused and the MLP as one node ({mode.replace('_', ' ')}): {t / args.steps:.4f} ms/pass -> "
+            f"{g:.1f} GB/s ({100 * g / HBM_PEAK_GBS:.1f} % of 8 TB/s)")
+    if saved is None:
+        os.environ.pop("OVFCC_MLP_FUSED", None)
+    else:
+        os.environ["OVFCC_MLP_FUSED"] = saved
+    _lib.sync_env()
+    for w in mlp_layers:
+        w.close()
+    mlp_base["mlp"].close()
+
     copy_gbs = dev.copy_bandwidth(1 << 30, 10)
     log(f"plain copy kernel: {copy_gbs:.0f} GB/s (read + write)")
 
@@ -640,6 +667,9 @@ def main() -> int:
                                  "(ovfcc_weights_concat), 4 launches per block",
                          "launches": args.layers * 4, "ms_per_pass": round(fms / args.steps, 5),
                          "GBps": round(fused_gbs, 1), "pct_of_hbm_peak": round(100 * fused_gbs / HBM_PEAK_GBS, 2)},
+        "decode_mlp_node": {"note": "same pass with q/k/v concatenated and gate/up (SwiGLU) + down as one MLP node "
+                                    "(ovfcc_weights_mlp): as the two launches it runs by default, and as its one-launch "
+                                    "kernel (OVFCC_MLP_FUSED=1); algorithmic bytes as in decode_fused", **mlp_modes},
         "decode_small_batch": small_batch,
         "decode_per_shape": {k: {"us": round(v["us"], 3), "GBps": round(v["GBps"], 1)} for k, v in per_shape.items()},
         "parity": {k: {a: float(f"{b:.3e}") for a, b in v.items()} for k, v in parity.items()},

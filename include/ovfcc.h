@@ -179,6 +179,18 @@ int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_w
  * with desc.flags = glu_type: both parts must be tiled nodes equal in shape, types, bias presence and output type;
  * they stay valid.  The result reports N = 2 * N_part and produces [M, N_part]. */
 int ovfcc_weights_glu(const ovfcc_weights* gate, const ovfcc_weights* up, int glu_type, ovfcc_weights** out);
+
+/* The gated MLP of a decoder block as one node: gate / up projection with its gated linear unit (a node created
+ * with OVFCC_GLU_* flags or by ovfcc_weights_glu, f16 output), then the down projection, whose K is the first
+ * node's output width.  The counterpart of the CPU plugin's LLMMLP node (src/plugins/intel_cpu/src/nodes/llm_mlp.cpp:
+ * 495-526; the pattern: cpu_opset/x64/pass/mlp_fusion.cpp:48-120).  ovfcc_fc_run[_device] on it takes X [M, K of
+ * the first node] and writes Y [M, N of the down projection] in the down projection's output_type; the
+ * intermediate activations live in a buffer of the request, rounded to f16 as between two separate nodes.  The
+ * node runs as two launches on the request's stream.  With OVFCC_MLP_FUSED=1 in the environment, one to four rows
+ * of 4-bit nodes with groups of 128 run as one kernel launch whose workgroups wait for each other in the middle (a
+ * bounded wait: if it runs out, ovfcc_request_sync / ovfcc_fc_run return OVFCC_EDEVICE); it gives the same bits and,
+ * as measured, is the slower of the two.  The new node owns copies of both; the arguments stay the caller's. */
+int ovfcc_weights_mlp(const ovfcc_weights* gate_up, const ovfcc_weights* down, ovfcc_weights** out);
 /* device bytes held by the repacked node */
 int64_t ovfcc_weights_device_bytes(const ovfcc_weights* w);
 /* 1 when the node uses the tiled layout (fast kernels), 0 for the OpenVINO-layout fallback */

@@ -103,6 +103,11 @@ int64_t out_channels(const ovfcc_weights* w) {
     return w->layout.glu ? w->desc.N / 2 : w->desc.N;
 }
 
+// the node whose output leaves the object: the down projection of an MLP node, else the node itself
+const ovfcc_weights* output_node(const ovfcc_weights* w) {
+    return w->mlp_down ? w->mlp_down : w;
+}
+
 void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc::FcDeviceArgs* a) {
     a->w = w->d_w;
     a->scale = w->d_scale;
@@ -257,7 +262,12 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
 
 // Enqueue one node.  The fast kernels address the activations with 32-bit byte offsets and the plain kernel puts
 // the rows on a 16-bit grid axis: a longer node runs as consecutive row blocks on the same stream.
-int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch = false) {
+int enqueue_mlp(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch);
+
+int enqueue(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch = false,
+            bool first_node_only = false) {
+    if (w->mlp_down && !first_node_only)
+        return enqueue_mlp(r, w, x, y, M, static_scratch);
     int64_t block = M;
     if (w->layout.tiled) {
         const int64_t lim = ((((int64_t)1 << 31) - 1) / (2 * w->desc.K)) & ~(int64_t)127;
@@ -660,6 +670,86 @@ int moe_routed(ovfcc_request* r, const ovfcc_weights* const* gate_up, const ovfc
     return OVFCC_OK;
 }
 
+// An MLP node: the gate / up node into the request's intermediate buffer and the down node out of it, as two
+// launches; with OVFCC_MLP_FUSED = 1 the one-launch kernel for one to four rows of nodes it can run.  (Measured on
+// the Llama-3-8B block at one row: one launch 21.7 us, two launches 18.9 us -- publishing the intermediate row,
+// raising the flags and reading the row back are three trips through a memory system whose queues hold the down
+// projection's weights, and cost more than the second launch they replace.  The kernel stays an option.)
+int enqueue_mlp(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* y, int64_t M, bool static_scratch) {
+    if (M == 0)
+        return OVFCC_OK;
+    if (static_scratch)
+        return fail(OVFCC_EUNSUPPORTED, "an MLP node needs the request's intermediate buffer");
+    const ovfcc_weights* d = w->mlp_down;
+    const int64_t I = out_channels(w);
+    const size_t mid_bytes = (size_t)M * I * 2;
+    if (mid_bytes > r->mid_cap) {
+        HIP_TRY(hipStreamSynchronize(r->stream));
+        int rc = grow(&r->d_mid, &r->mid_cap, mid_bytes);
+        if (rc)
+            return rc;
+    }
+    // One workgroup per compute unit (OVFCC_MLP_GRID overrides).  Fewer workgroups that share the tile pairs evenly
+    // were measured and lose: a compute unit's throughput is what its sixteen waves keep in flight, so the weight
+    // stream slows with the number of workgroups (Llama-3-8B block: 256 workgroups 21.6 us, 224 23.9, 128 26.4).
+    int grid = r->ctx->n_cus;
+    if (const int forced = ovfcc::env_int("OVFCC_MLP_GRID", 0); forced > 0 && forced <= r->ctx->n_cus)
+        grid = forced;
+    const bool fused = M <= 4 && r->force_kernel == OVFCC_KERNEL_AUTO && r->force_split == 0 &&
+                       ovfcc::env_int("OVFCC_MLP_FUSED", 0) != 0 && w->d_scale_cm && d->d_scale_cm &&
+                       ovfcc::mlp_fused_applies(w->layout, d->layout, M, grid);
+    if (!fused) {
+        int rc = enqueue(r, w, x, r->d_mid, M, false, true);
+        if (rc)
+            return rc;
+        return enqueue(r, d, r->d_mid, y, M);
+    }
+    const size_t sync_bytes = ovfcc::mlp_sync_bytes(r->ctx->n_cus);
+    if (!r->d_sync) {
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&r->d_sync), sync_bytes));
+        HIP_TRY(hipMemset(r->d_sync, 0, sync_bytes));
+        HIP_TRY(hipHostMalloc(reinterpret_cast<void**>(&r->h_error), 64, hipHostMallocDefault));
+        *r->h_error = 0;
+    }
+    if (*r->h_error) {
+        // an earlier launch gave up its wait: its counters may be anywhere; start from zero again
+        HIP_TRY(hipStreamSynchronize(r->stream));
+        HIP_TRY(hipMemset(r->d_sync, 0, sync_bytes));
+        *r->h_error = 0;
+        return fail(OVFCC_EDEVICE, "an earlier MLP launch on this request gave up waiting for its workgroups");
+    }
+    ovfcc::FcDeviceArgs ga, da;
+    fill_args(w, x, r->d_mid, M, &ga);
+    fill_args(d, r->d_mid, y, M, &da);
+    const int spin_env = ovfcc::env_int("OVFCC_MLP_SPIN_LIMIT", 0);
+    const unsigned spin_limit = spin_env > 0 ? (unsigned)spin_env : (1u << 20);
+    // One launch of this kind on the device at a time: its workgroups wait for each other, and two such grids that
+    // each hold half the compute units would wait for good.  The launch waits for the one before it on any stream.
+    // (A capturing stream cannot wait for an event from outside its capture; a caller that captures keeps such
+    // launches of different requests apart itself.)
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    HIP_TRY(hipStreamIsCapturing(r->stream, &cap));
+    std::lock_guard<std::mutex> lock(r->ctx->coop_mu);
+    if (cap == hipStreamCaptureStatusNone) {
+        if (!r->ctx->coop_done)
+            HIP_TRY(hipEventCreateWithFlags(&r->ctx->coop_done, hipEventDisableTiming));
+        else
+            HIP_TRY(hipStreamWaitEvent(r->stream, r->ctx->coop_done, 0));
+    }
+    int e = ovfcc::launch_mlp(ga, da, r->d_mid, r->d_sync, r->h_error, grid, r->ctx->n_cus, spin_limit, r->stream);
+    if (e)
+        return hip_fail((hipError_t)e, "MLP kernel launch");
+    if (cap == hipStreamCaptureStatusNone)
+        HIP_TRY(hipEventRecord(r->ctx->coop_done, r->stream));
+    ovfcc::LaunchPlan shown;
+    shown.kernel = OVFCC_KERNEL_DECODE;
+    shown.tile_m = 16, shown.tile_n = 16, shown.block = 1024;
+    shown.grid[0] = (unsigned)grid;
+    shown.name = "fcc_mlp_gemv_w4";
+    record(r, shown);
+    return OVFCC_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -708,6 +798,8 @@ int ovfcc_init(int device, ovfcc_ctx** out) {
 }
 
 void ovfcc_destroy(ovfcc_ctx* ctx) {
+    if (ctx && ctx->coop_done)
+        (void)hipEventDestroy(ctx->coop_done);
     delete ctx;
 }
 
@@ -811,6 +903,7 @@ int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* 
 void ovfcc_weights_destroy(ovfcc_weights* w) {
     if (!w)
         return;
+    ovfcc_weights_destroy(w->mlp_down);
     if (w->d_w) (void)hipFree(w->d_w);
     if (w->d_scale) (void)hipFree(w->d_scale);
     if (w->d_zp) (void)hipFree(w->d_zp);
@@ -859,6 +952,39 @@ int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out) {
     if (!rc) rc = dup(&W->d_bias, src->d_bias, (size_t)N * 2);
     if (!rc)
         rc = finish_weights(W);
+    if (!rc && src->mlp_down)
+        rc = ovfcc_weights_clone(src->mlp_down, &W->mlp_down);
+    if (rc) {
+        ovfcc_weights_destroy(W);
+        return rc;
+    }
+    *out = W;
+    return OVFCC_OK;
+}
+
+int ovfcc_weights_mlp(const ovfcc_weights* gate_up, const ovfcc_weights* down, ovfcc_weights** out) {
+    if (!gate_up || !down || !out)
+        return fail(OVFCC_EINVAL, "null argument");
+    *out = nullptr;
+    if (gate_up->ctx != down->ctx)
+        return fail(OVFCC_EINVAL, "the two nodes belong to different contexts");
+    if (gate_up->mlp_down || down->mlp_down)
+        return fail(OVFCC_EINVAL, "an MLP node cannot be part of another");
+    if (!gate_up->layout.glu)
+        return fail(OVFCC_EINVAL, "the first node must carry a gated linear unit (ovfcc_weights_glu or OVFCC_GLU_* flags)");
+    if (down->layout.glu)
+        return fail(OVFCC_EINVAL, "the down projection must not carry a gated linear unit");
+    if (gate_up->desc.out_type != OVFCC_F16)
+        return fail(OVFCC_EUNSUPPORTED, "the intermediate activations are f16: the first node's output_type must be f16");
+    if (out_channels(gate_up) != down->desc.K)
+        return fail(OVFCC_EINVAL, "the down projection's K (" + std::to_string(down->desc.K) +
+                                      ") is not the first node's output width (" +
+                                      std::to_string(out_channels(gate_up)) + ")");
+    ovfcc_weights* W = nullptr;
+    int rc = ovfcc_weights_clone(gate_up, &W);
+    if (rc)
+        return rc;
+    rc = ovfcc_weights_clone(down, &W->mlp_down);
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;
@@ -868,6 +994,9 @@ int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out) {
 }
 
 int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_weights** out) {
+    for (int i = 0; parts && i < n_parts; ++i)
+        if (parts[i] && parts[i]->mlp_down)
+            return fail(OVFCC_EINVAL, "an MLP node cannot be concatenated");
     if (!parts || n_parts <= 0 || !out)
         return fail(OVFCC_EINVAL, "null or empty part list");
     *out = nullptr;
@@ -934,6 +1063,8 @@ int ovfcc_weights_concat(const ovfcc_weights* const* parts, int n_parts, ovfcc_w
 }
 
 int ovfcc_weights_glu(const ovfcc_weights* gate, const ovfcc_weights* up, int glu_type, ovfcc_weights** out) {
+    if ((gate && gate->mlp_down) || (up && up->mlp_down))
+        return fail(OVFCC_EINVAL, "an MLP node cannot be one half of a gated linear unit");
     if (!gate || !up || !out)
         return fail(OVFCC_EINVAL, "null argument");
     *out = nullptr;
@@ -985,7 +1116,7 @@ int ovfcc_weights_glu(const ovfcc_weights* gate, const ovfcc_weights* up, int gl
 }
 
 int64_t ovfcc_weights_device_bytes(const ovfcc_weights* w) {
-    return w ? (int64_t)w->bytes : 0;
+    return w ? (int64_t)w->bytes + ovfcc_weights_device_bytes(w->mlp_down) : 0;
 }
 
 int ovfcc_weights_is_tiled(const ovfcc_weights* w) {
@@ -1031,6 +1162,8 @@ void device_sizes(const ovfcc_fc_desc& d, const ovfcc::Layout& L, uint64_t out[4
 }  // namespace
 
 int ovfcc_weights_export_size(const ovfcc_weights* w, size_t* bytes) {
+    if (w && w->mlp_down)
+        return fail(OVFCC_EUNSUPPORTED, "an MLP node is exported as its two nodes; export them before ovfcc_weights_mlp");
     if (!w || !bytes)
         return fail(OVFCC_EINVAL, "null argument");
     uint64_t sz[4];
@@ -1040,6 +1173,8 @@ int ovfcc_weights_export_size(const ovfcc_weights* w, size_t* bytes) {
 }
 
 int ovfcc_weights_export(const ovfcc_weights* w, void* blob, size_t bytes) {
+    if (w && w->mlp_down)
+        return fail(OVFCC_EUNSUPPORTED, "an MLP node is exported as its two nodes; export them before ovfcc_weights_mlp");
     size_t need = 0;
     int rc = ovfcc_weights_export_size(w, &need);
     if (rc)
@@ -1150,6 +1285,9 @@ void ovfcc_request_destroy(ovfcc_request* r) {
     if (r->counters) (void)hipFree(r->counters);
     if (r->d_gather) (void)hipFree(r->d_gather);
     if (r->d_quant) (void)hipFree(r->d_quant);
+    if (r->d_mid) (void)hipFree(r->d_mid);
+    if (r->d_sync) (void)hipFree(r->d_sync);
+    if (r->h_error) (void)hipHostFree(r->h_error);
     if (r->h_maps) (void)hipHostFree(r->h_maps);
     if (r->h_stage) (void)hipHostFree(r->h_stage);
     if (r->maps_uploaded) (void)hipEventDestroy(r->maps_uploaded);
@@ -1657,6 +1795,12 @@ int ovfcc_request_sync(ovfcc_request* r) {
     if (!r)
         return fail(OVFCC_EINVAL, "request is null");
     HIP_TRY(hipStreamSynchronize(r->stream));
+    if (r->h_error && *r->h_error) {
+        // a one-launch MLP kernel gave up waiting for its workgroups: its output is not valid
+        HIP_TRY(hipMemset(r->d_sync, 0, ovfcc::mlp_sync_bytes(r->ctx->n_cus)));
+        *r->h_error = 0;
+        return fail(OVFCC_EDEVICE, "an MLP launch on this request gave up waiting for its workgroups; its output is invalid");
+    }
     return OVFCC_OK;
 }
 
@@ -1671,7 +1815,8 @@ int ovfcc_fc_run(ovfcc_request* r, const ovfcc_weights* w, const void* x_host, v
         return fail(OVFCC_EINVAL, "x or y is null");
     HIP_TRY(hipSetDevice(r->ctx->device));
     const size_t xb = (size_t)M * w->desc.K * 2;
-    const size_t yb = (size_t)M * out_channels(w) * (w->desc.out_type == OVFCC_F32 ? 4 : 2);
+    const ovfcc_weights* last = output_node(w);
+    const size_t yb = (size_t)M * out_channels(last) * (last->desc.out_type == OVFCC_F32 ? 4 : 2);
     if (xb > r->x_cap || yb > r->y_cap)
         HIP_TRY(hipStreamSynchronize(r->stream));
     int rc = grow(&r->d_x, &r->x_cap, xb);
@@ -1704,7 +1849,9 @@ int ovfcc_fc_run(ovfcc_request* r, const ovfcc_weights* w, const void* x_host, v
         return rc;
     if (!staged)
         HIP_TRY(hipMemcpyAsync(y_host, r->d_y, yb, hipMemcpyDeviceToHost, r->stream));
-    HIP_TRY(hipStreamSynchronize(r->stream));
+    rc = ovfcc_request_sync(r);  // (also reports an MLP launch that gave up its wait)
+    if (rc)
+        return rc;
     if (staged)
         std::memcpy(y_host, hs + y_off, yb);
     return OVFCC_OK;

@@ -14,6 +14,10 @@ struct ovfcc_ctx {
     int device = 0;
     int n_cus = 256;
     std::string arch;
+    // Launches whose workgroups wait for each other (the one-launch MLP) must not share the chip with another of
+    // their kind: each waits, on its stream, for the event recorded behind the one before it.
+    std::mutex coop_mu;
+    hipEvent_t coop_done = nullptr;
 };
 
 struct ovfcc_weights {
@@ -24,6 +28,7 @@ struct ovfcc_weights {
     void* d_scale = nullptr;
     void* d_zp = nullptr;
     void* d_bias = nullptr;
+    ovfcc_weights* mlp_down = nullptr;  // ovfcc_weights_mlp: this node is gate / up, that one (owned) the down projection
     void* d_scale_cm = nullptr;  // channel-major copies of the group parameters for the matrix-vector kernel
     void* d_zp_cm = nullptr;
     size_t bytes = 0;
@@ -56,6 +61,10 @@ struct ovfcc_request {
     size_t gather_cap = 0;
     void* d_quant = nullptr;   // dynamic quantisation: int8 activations, inverse scales, sums
     size_t quant_cap = 0;
+    void* d_mid = nullptr;     // MLP node: the intermediate row block [M, I] f16
+    size_t mid_cap = 0;
+    unsigned* d_sync = nullptr;   // ... the two counters of its one-launch kernel (zero between launches)
+    unsigned* h_error = nullptr;  // ... and the pinned word that kernel sets when its wait ran out
     int* h_maps = nullptr;     // ... and the pinned host copy of the row maps, reused once its upload has finished
     size_t h_maps_cap = 0;
     hipEvent_t maps_uploaded = nullptr;

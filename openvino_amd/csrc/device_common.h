@@ -182,19 +182,33 @@ __device__ __forceinline__ TileWork tile_work(int tiles_x, int tiles_y, int full
 // formulas of the OpenVINO Intel-GPU plugin (cl_kernels/swiglu_gpu_ref.cl:74-85, swish beta = 1).  Exponential
 // and reciprocal are the hardware's (about 1e-6 relative, far inside the f16 result): the epilogue of a prefill
 // tile runs with the matrix cores idle, so its length is paid in full.  Both saturate correctly:
-// exp -> inf gives 1 / inf = 0, exp -> 0 gives 1.
+// exp -> inf gives 1 / inf = 0, exp -> 0 gives 1.  No multiply and add is contracted here: which ones the compiler
+// fuses depends on the code around the call, and kernels that promise each other's bits must not differ in that.
 __device__ __forceinline__ float glu_value(int type, float gate, float up) {
+#pragma clang fp contract(off)
+    // exp(t) as the hardware's 2^(t log2 e), one instruction: the library routine's range fix-ups are another place
+    // where two kernels can come to differ
+    constexpr float kLog2e = 1.44269504088896340736f;
     float a;
     if (type == 1) {
-        a = gate * __builtin_amdgcn_rcpf(1.f + __expf(-gate));
+        a = gate * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-gate * kLog2e));
     } else if (type == 2) {
         a = 0.5f * gate * (1.f + erff(gate * 0.70710678118654752440f));
     } else {
         // tanh z = 1 - 2 / (1 + exp 2 z)
-        const float z = 0.79788456080286535588f * gate * (1.f + 0.044715f * gate * gate);
-        a = gate * (1.f - __builtin_amdgcn_rcpf(1.f + __expf(2.f * z)));
+        const float z = 0.79788456080286535588f * gate * __builtin_fmaf(0.044715f * gate, gate, 1.f);
+        a = gate * (1.f - __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(z * (2.f * kLog2e))));
     }
     return a * up;
+}
+
+// f32 -> f16, round to nearest even, of a value that exists in f32 first.  The empty asm statement keeps the compiler
+// from folding the conversion into the multiply or fused multiply-add that produced the value (one rounding from the
+// exact product instead of two): it does so in some kernels and not in others, and a result that sits on a rounding
+// tie then differs by one f16 step between kernels that promise each other's bits.
+__device__ __forceinline__ half_t to_half_rne(float v) {
+    asm volatile("" : "+v"(v));
+    return (half_t)v;
 }
 
 // Output cast: FullyConnected's output_type is f16 (default, the activation type) or f32.
@@ -202,7 +216,7 @@ __device__ __forceinline__ void store_out(void* y, size_t i, float v, int out_f3
     if (out_f32)
         static_cast<float*>(y)[i] = v;
     else
-        static_cast<half_t*>(y)[i] = (half_t)v;
+        static_cast<half_t*>(y)[i] = to_half_rne(v);
 }
 
 __device__ __forceinline__ half2_t splat(float v) {

@@ -19,6 +19,10 @@
 // c = sum_k x_k, one f32 per row and k-block, which a wave computes from its own activations while its weights
 // travel:  y = 2^24 sum_kb s_kb (P_kb - zp_kb 2^-24 c_kb),  two vector operations per row and k-block.
 //
+// The f32 arithmetic behind a partial sum is spelled out with explicit fused multiply-adds (left to the compiler,
+// which products it fuses depends on the code around them, and the one-launch MLP kernel, kernel_mlp.hip, promises
+// this kernel's bits).
+//
 // Activations.  A wave loads X[0:M, its k-range] itself (M x C x 256 bytes, before the weights, because loads
 // retire in order), forms the group sums (four dot products and a 16-lane DPP reduction per load, read back into
 // scalar registers), and parks the rows in its own slice of LDS in operand order; no workgroup barrier sits
@@ -184,7 +188,7 @@ __global__ __launch_bounds__(1024) void fcc_gemv_kernel(const uint4_t* __restric
         if (out_f32)
             static_cast<__attribute__((address_space(1))) float*>(y_k)[i] = v;
         else
-            static_cast<__attribute__((address_space(1))) half_t*>(y_k)[i] = (half_t)v;
+            static_cast<__attribute__((address_space(1))) half_t*>(y_k)[i] = to_half_rne(v);
     };
     // Every load is on its way before anything waits for one: without the fence the compiler starts on the
     // activations after the first two weight loads and the others leave one memory round trip late.
@@ -268,11 +272,11 @@ __global__ __launch_bounds__(1024) void fcc_gemv_kernel(const uint4_t* __restric
             const float zpf = (float)((zv[i >> 2] >> (8 * (i & 3))) & 0xFFu);
 #pragma unroll
             for (int r = 0; r < MR; ++r)
-                acc[r] += scale * (pr[r] - zpf * csum[r][i]);
+                acc[r] = __builtin_fmaf(scale, __builtin_fmaf(-zpf, csum[r][i], pr[r]), acc[r]);
         } else {
 #pragma unroll
             for (int r = 0; r < MR; ++r)
-                acc[r] += scale * (pr[r] + csum[r][i]);
+                acc[r] = __builtin_fmaf(scale, pr[r] + csum[r][i], acc[r]);
         }
     }
 
@@ -334,7 +338,7 @@ __global__ __launch_bounds__(1024) void fcc_gemv_kernel(const uint4_t* __restric
         for (int r = 0; r < MR; ++r) {
             const float g = tile_sum(0, nwt, r), u = tile_sum(nwt, nwt, r);
             if (r < M && kq == 0)
-                put((size_t)r * (N / 2) + blockIdx.x * 16 + col, glu_value(glu, g * 0x1p24f + bg, u * 0x1p24f + bu));
+                put((size_t)r * (N / 2) + blockIdx.x * 16 + col, glu_value(glu, __builtin_fmaf(g, 0x1p24f, bg), __builtin_fmaf(u, 0x1p24f, bu)));
         }
         return;
     }
@@ -344,7 +348,7 @@ __global__ __launch_bounds__(1024) void fcc_gemv_kernel(const uint4_t* __restric
     for (int r = 0; r < MR; ++r) {
         const float s = tile_sum(0, waves, r);
         if (r < M && kq == 0)
-            put((size_t)r * N + n, s * 0x1p24f + b);
+            put((size_t)r * N + n, __builtin_fmaf(s, 0x1p24f, b));
     }
 }
 

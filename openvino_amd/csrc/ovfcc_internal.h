@@ -268,6 +268,13 @@ int launch_offsets_table(const int* offsets_dev, int n_groups, int64_t rows, int
                          const void* x_base, size_t x_row_bytes, void* y_base, size_t y_row_bytes,
                          BatchGroupItem* table, int n_slices_max, RoutedHeader* header, int* tail, int tiles_x,
                          int kb_total, int n_cus, void* stream);
+// The gated MLP as one launch (kernel_mlp.hip): gate / up node g with its gated linear unit, down node d, M <= 4.
+// mid: [M, d.K] f16 scratch; sync: mlp_sync_bytes(grid) bytes that are zero between launches; error: a host-visible
+// word the kernel sets when its wait for the other workgroups ran out after spin_limit polls.
+size_t mlp_sync_bytes(int grid);
+bool mlp_fused_applies(const Layout& g, const Layout& d, int64_t M, int grid);
+int launch_mlp(const FcDeviceArgs& g, const FcDeviceArgs& d, void* mid, unsigned* sync, unsigned* error, int grid,
+               int n_cus, unsigned spin_limit, void* stream);
 int launch_prefill(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_wide(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_prefill_direct(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);

@@ -22,7 +22,8 @@ namespace ovfcc {
 //            OVFCC_GEMV16 = 0 | 1 (the 16-row kernel with stationary activations for 5-48 rows),
 //            OVFCC_GEMV16_GRID = n (its workgroups per row tile), OVFCC_GEMV16_SPLIT = 1 | 2 | 4 | 8 (parts it cuts K in),
 //            OVFCC_PREFILL_{DIRECT, ASYNC, WIDE, BIG, TAIL} = 0 | 1, OVFCC_PREFILL_ROWS = 64 | 128,
-//            OVFCC_MOE_HOST_ROUTING = 1;
+//            OVFCC_MOE_HOST_ROUTING = 1, OVFCC_MLP_FUSED = 1 (an MLP node of up to four rows as one launch instead of two),
+//            OVFCC_MLP_GRID = n (its workgroups), OVFCC_MLP_SPIN_LIMIT = n (polls after which that launch's wait for its workgroups gives up; tests);
 //   logging: OVFCC_VERBOSE = 1 (one line per launch on stderr), 2 (also weights and requests as they come and go).
 namespace {
 struct EnvEntry {
@@ -36,7 +37,9 @@ EnvEntry g_env[] = {EnvEntry("OVFCC_DECODE_WAVES"),   EnvEntry("OVFCC_DECODE_RT"
                     EnvEntry("OVFCC_GEMV16"),         EnvEntry("OVFCC_GEMV16_GRID"),    EnvEntry("OVFCC_GEMV16_SPLIT"),
                     EnvEntry("OVFCC_PREFILL_DIRECT"), EnvEntry("OVFCC_PREFILL_ASYNC"),  EnvEntry("OVFCC_PREFILL_WIDE"),
                     EnvEntry("OVFCC_PREFILL_BIG"),    EnvEntry("OVFCC_PREFILL_TAIL"),   EnvEntry("OVFCC_PREFILL_ROWS"),
-                    EnvEntry("OVFCC_MOE_HOST_ROUTING"), EnvEntry("OVFCC_VERBOSE")};
+                    EnvEntry("OVFCC_MOE_HOST_ROUTING"), EnvEntry("OVFCC_MLP_FUSED"),      EnvEntry("OVFCC_MLP_SPIN_LIMIT"),
+                    EnvEntry("OVFCC_MLP_GRID"),
+                    EnvEntry("OVFCC_VERBOSE")};
 std::atomic<unsigned> g_env_generation{0};
 std::once_flag g_env_once;
 

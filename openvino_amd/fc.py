@@ -144,8 +144,30 @@ class CompressedWeights:
 
     @property
     def N_out(self) -> int:
-        """Row length of the node's output: N, or N / 2 with a gated-linear-unit epilogue."""
+        """Row length of the node's output: N, or N / 2 with a gated-linear-unit epilogue; an MLP node's is its down
+        projection's."""
+        down = getattr(self, "down", None)
+        if down is not None:
+            return down.N_out
         return self.N // 2 if self.desc.flags & 3 else self.N
+
+    @property
+    def out_f32(self) -> bool:
+        down = getattr(self, "down", None)
+        return (down.desc if down is not None else self.desc).out_type == _lib.F32
+
+    @classmethod
+    def mlp(cls, gate_up: "CompressedWeights", down: "CompressedWeights") -> "CompressedWeights":
+        """Gate / up node (with its gated linear unit) and down projection as one node: X [M, K] -> Y [M, N of down]
+        (the CPU plugin's LLMMLP node).  The new node owns device copies of both."""
+        h = ctypes.c_void_p()
+        check(gate_up.device.lib.ovfcc_weights_mlp(gate_up.handle, down.handle, ctypes.byref(h)))
+        other = object.__new__(CompressedWeights)
+        other.device, other.N, other.K, other.group_size = gate_up.device, gate_up.N, gate_up.K, gate_up.group_size
+        other.desc = FcDesc.from_buffer_copy(gate_up.desc)
+        other.down = down          # shapes and types of the output side (the handle inside the node is its own copy)
+        other.handle = h
+        return other
 
     @classmethod
     def glu(cls, gate: "CompressedWeights", up: "CompressedWeights", kind: str = "swish") -> "CompressedWeights":
@@ -166,6 +188,8 @@ class CompressedWeights:
         other = object.__new__(CompressedWeights)
         other.device, other.N, other.K, other.group_size, other.desc = (self.device, self.N, self.K,
                                                                         self.group_size, self.desc)
+        if getattr(self, "down", None) is not None:
+            other.down = self.down
         h = ctypes.c_void_p()
         check(self.device.lib.ovfcc_weights_clone(self.handle, ctypes.byref(h)))
         other.handle = h
@@ -243,8 +267,7 @@ class InferRequest:
         if X.shape[-1] != weights.K:
             raise OvfccError(_lib.EINVAL, f"last dimension of X is {X.shape[-1]}, expected K = {weights.K}")
         M = int(np.prod(X.shape[:-1], dtype=np.int64))
-        Y = np.empty(X.shape[:-1] + (weights.N_out,),
-                     dtype=np.float32 if weights.desc.out_type == _lib.F32 else np.float16)
+        Y = np.empty(X.shape[:-1] + (weights.N_out,), dtype=np.float32 if weights.out_f32 else np.float16)
         check(self.device.lib.ovfcc_fc_run(self.handle, weights.handle, _vp(X), _vp(Y), M))
         return Y
 
