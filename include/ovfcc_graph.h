@@ -20,9 +20,13 @@
  *                      src/plugins/intel_gpu/src/kernel_selector/kernels/fully_connected/
  *                      fully_connected_kernel_bf_tiled.cpp:223-236).
  *
- * Nothing here touches constant data or a device: shapes, element types and small integer attributes in,
+ * The matchers touch neither constant data nor a device: shapes, element types and small integer attributes in,
  * decisions out.  Return codes and ovfcc_last_error() as in ovfcc.h; "this subgraph is not a compressed
  * FullyConnected" is OVFCC_EUNSUPPORTED with the reason in the error string.
+ *
+ *   ovfcc_fold_weights_create / ovfcc_fold_expert_weights_create
+ *                      the data half of the same passes: from a matched node and the bytes of its Constants to an
+ *                      ovfcc_weights, so that a host's compile step is a loop over library calls.
  */
 #ifndef OVFCC_GRAPH_H
 #define OVFCC_GRAPH_H
@@ -98,6 +102,19 @@ typedef struct ovfcc_fold {
 /* Matches the subgraph that ends in `root` (a MatMul, a FullyConnected, or an Add of one of them with a Constant). */
 int ovfcc_fold_match(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_fold* out);
 
+/* Creates the node a fold describes from the bytes of its Constants -- what
+ * ConvertFullyConnectedToFullyConnectedCompressed does with the Constants it re-views and converts
+ * (src/common/transformations/src/transformations/op_conversions/convert_fc_to_compressed.cpp:127-225).
+ * constant_data has n_nodes entries; entry i points at the data of node i in OpenVINO's packing (4-bit types two per
+ * byte, low nibble first) where node i is one of fold->weights / scales / zero_points / bias, and is not read
+ * otherwise (null is fine).  Weights and integer zero-points are taken as they are; f32 scales and bias are rounded
+ * to f16 (nearest even), a scale Constant of one element is replicated (scale_broadcast), a real-typed zero-point
+ * (zp_from_real) must hold integers in 0..255 and becomes u8 -- OVFCC_EUNSUPPORTED otherwise.  Every Constant's
+ * element type and count are checked against the fold's descriptor (OVFCC_EINVAL).  extra_flags is or-ed into
+ * desc.flags (OVFCC_W_DYN_QUANT, ...). */
+int ovfcc_fold_weights_create(ovfcc_ctx* ctx, const ovfcc_gnode* nodes, int n_nodes, const ovfcc_fold* fold,
+                              const void* const* constant_data, int extra_flags, ovfcc_weights** out);
+
 /* How matched nodes share launches. */
 enum ovfcc_fused_kind {
     OVFCC_FUSED_SINGLE = 0, /* one node of its own */
@@ -150,6 +167,14 @@ typedef struct ovfcc_gather_fold {
 } ovfcc_gather_fold;
 
 int ovfcc_fold_gather_matmul(const ovfcc_gnode* nodes, int n_nodes, int root, ovfcc_gather_fold* out);
+
+/* Expert (or group) `expert` of a gather / grouped fold as a node of its own: slice `expert` of every batched
+ * Constant (convert_gather_matmul_to_compressed.cpp:27-92 re-views the same Constants as [E, N, K], [E, N, K/G]).  A
+ * 4-bit slice that begins or ends in the middle of a byte is re-packed; a one-element scale or zero-point serves
+ * every expert; the bias Constant holds N values shared by the experts or E x N (bias_per_expert).  Otherwise as
+ * ovfcc_fold_weights_create. */
+int ovfcc_fold_expert_weights_create(ovfcc_ctx* ctx, const ovfcc_gnode* nodes, int n_nodes, const ovfcc_gather_fold* fold,
+                                     int expert, const void* const* constant_data, int extra_flags, ovfcc_weights** out);
 
 /* A matched GroupedMatMulCompressed node (src/common/transformations/include/ov_ops/grouped_matmul_compressed.hpp:
  * 17-66): either a v17::GroupedMatMul (src/core/include/openvino/op/grouped_matmul.hpp:26-50) whose B input is the

@@ -32,7 +32,7 @@ SYMBOLS = [
     "ovfcc_last_kernel_info", "ovfcc_device_malloc", "ovfcc_device_free",
     "ovfcc_memcpy_h2d", "ovfcc_memcpy_d2h", "ovfcc_memcpy_d2d", "ovfcc_desc_validate", "ovfcc_env_reload", "ovfcc_tiled_sizes",
     "ovfcc_repack_host", "ovfcc_unrepack_host", "ovfcc_unpack_u4", "ovfcc_unpack_i4", "ovfcc_last_error",
-    "ovfcc_version", "ovfcc_fold_match", "ovfcc_fold_model", "ovfcc_fold_gather_matmul", "ovfcc_fold_grouped_matmul", "ovfcc_fold_moe",
+    "ovfcc_version", "ovfcc_fold_match", "ovfcc_fold_model", "ovfcc_fold_gather_matmul", "ovfcc_fold_grouped_matmul", "ovfcc_fold_moe", "ovfcc_fold_weights_create", "ovfcc_fold_expert_weights_create",
 ]
 
 
@@ -190,6 +190,9 @@ def load() -> ctypes.CDLL:
         "ovfcc_fold_gather_matmul": (ci, [ctypes.POINTER(GNode), ci, ci, ctypes.POINTER(GatherFold)]),
         "ovfcc_fold_grouped_matmul": (ci, [ctypes.POINTER(GNode), ci, ci, ctypes.POINTER(GatherFold)]),
         "ovfcc_fold_moe": (ci, [ctypes.POINTER(GNode), ci, ci, ctypes.POINTER(MoeFold)]),
+        "ovfcc_fold_weights_create": (ci, [vp, ctypes.POINTER(GNode), ci, ctypes.POINTER(Fold), ctypes.POINTER(vp), ci, pp]),
+        "ovfcc_fold_expert_weights_create": (ci, [vp, ctypes.POINTER(GNode), ci, ctypes.POINTER(GatherFold), ci,
+                                                  ctypes.POINTER(vp), ci, pp]),
     }
     for name, (res, args) in sig.items():
         if name in BENCH_SYMBOLS and not hasattr(L, name):

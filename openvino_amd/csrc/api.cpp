@@ -13,6 +13,7 @@
 #include <vector>
 
 #include "api_types.h"
+#include "ovfcc_graph.h"
 #include "ovfcc_internal.h"
 
 namespace {
@@ -960,6 +961,34 @@ int ovfcc_weights_clone(const ovfcc_weights* src, ovfcc_weights** out) {
     }
     *out = W;
     return OVFCC_OK;
+}
+
+static int create_from(ovfcc_ctx* ctx, ovfcc::FoldConstants& c, int extra_flags, ovfcc_weights** out) {
+    c.desc.flags |= extra_flags;
+    return ovfcc_weights_create(ctx, &c.desc, c.weights, c.scales.data(), c.zero_points.empty() ? nullptr : c.zero_points.data(),
+                                c.bias.empty() ? nullptr : c.bias.data(), out);
+}
+
+int ovfcc_fold_weights_create(ovfcc_ctx* ctx, const ovfcc_gnode* nodes, int n_nodes, const ovfcc_fold* fold,
+                              const void* const* constant_data, int extra_flags, ovfcc_weights** out) {
+    if (!ctx || !fold || !out)
+        return fail(OVFCC_EINVAL, "null argument");
+    *out = nullptr;
+    ovfcc::FoldConstants c;
+    if (int rc = ovfcc::fold_constants(nodes, n_nodes, *fold, constant_data, c))
+        return rc;
+    return create_from(ctx, c, extra_flags, out);
+}
+
+int ovfcc_fold_expert_weights_create(ovfcc_ctx* ctx, const ovfcc_gnode* nodes, int n_nodes, const ovfcc_gather_fold* fold,
+                                     int expert, const void* const* constant_data, int extra_flags, ovfcc_weights** out) {
+    if (!ctx || !fold || !out)
+        return fail(OVFCC_EINVAL, "null argument");
+    *out = nullptr;
+    ovfcc::FoldConstants c;
+    if (int rc = ovfcc::fold_expert_constants(nodes, n_nodes, *fold, expert, constant_data, c))
+        return rc;
+    return create_from(ctx, c, extra_flags, out);
 }
 
 int ovfcc_weights_mlp(const ovfcc_weights* gate_up, const ovfcc_weights* down, ovfcc_weights** out) {

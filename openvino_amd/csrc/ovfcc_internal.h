@@ -8,6 +8,10 @@
 
 #include "ovfcc.h"
 
+struct ovfcc_gnode;
+struct ovfcc_fold;
+struct ovfcc_gather_fold;
+
 namespace ovfcc {
 
 // ---- tiled layout ------------------------------------------------------------------------
@@ -68,6 +72,22 @@ struct Layout {
         return (is_gate != glu_gate_second ? 0 : n_tiles / 2) + (nt >> 1);
     }
 };
+
+// The constants of one matched node (include/ovfcc_graph.h) in the form ovfcc_weights_create takes them.
+struct FoldConstants {
+    ovfcc_fc_desc desc{};
+    const void* weights = nullptr;       // the Constant's own bytes, or `packed`
+    std::vector<uint8_t> packed;         // a 4-bit expert slice that does not start and end on byte boundaries
+    std::vector<uint16_t> scales;        // f16 bits, [N, K/G] ([K/G, N] for input-major constants)
+    std::vector<uint8_t> zero_points;    // packed u4 / u8, or one element
+    std::vector<uint16_t> bias;          // f16 bits, [N]
+};
+// data[i]: the bytes of node i where it is a Constant the fold names.  Element counts and types are checked
+// against the descriptor; real-typed zero-points must hold integers in 0..255 (OVFCC_EUNSUPPORTED otherwise).
+int fold_constants(const struct ::ovfcc_gnode* nodes, int n_nodes, const struct ::ovfcc_fold& f, const void* const* data,
+                   FoldConstants& out);
+int fold_expert_constants(const struct ::ovfcc_gnode* nodes, int n_nodes, const struct ::ovfcc_gather_fold& f, int expert,
+                          const void* const* data, FoldConstants& out);
 
 void set_error(const std::string& msg);
 int fail(int code, const std::string& msg);

@@ -142,6 +142,17 @@ class CompressedWeights:
                    zp_type=c.zp_type, zp_scalar=c.zp_scalar, output_type=output_type, glu=glu,
                    glu_gate_second=glu_gate_second, dynamic_quantization=dynamic_quantization)
 
+    @classmethod
+    def adopt(cls, device: Device, handle, desc, extra_flags: int = 0) -> "CompressedWeights":
+        """Wraps a node the library created by another route (graph.Graph.create_weights)."""
+        other = object.__new__(CompressedWeights)
+        other.device = device
+        other.desc = FcDesc.from_buffer_copy(desc)
+        other.desc.flags |= extra_flags
+        other.N, other.K, other.group_size = other.desc.N, other.desc.K, other.desc.group_size
+        other.handle = handle
+        return other
+
     @property
     def N_out(self) -> int:
         """Row length of the node's output: N, or N / 2 with a gated-linear-unit epilogue; an MLP node's is its down

@@ -16,6 +16,7 @@ class Graph:
 
     def __init__(self):
         self.nodes = []
+        self.data = {}   # node index -> the Constant's bytes (numpy uint8, OpenVINO packing), where supplied
 
     def _add(self, op, type_, shape, inputs=(), transpose_a=False, transpose_b=False, attr=0, ints=None):
         n = _lib.GNode()
@@ -52,8 +53,23 @@ class Graph:
     def parameter(self, type_, shape):
         return self._add("parameter", type_, shape)
 
-    def constant(self, type_, shape, ints=None):
-        return self._add("constant", type_, shape, ints=ints)
+    def constant(self, type_, shape, ints=None, data=None):
+        """data: the Constant's bytes in OpenVINO's packing (any contiguous numpy array; 4-bit types two per byte,
+        low nibble first), needed only by create_weights / create_expert_weights."""
+        i = self._add("constant", type_, shape, ints=ints)
+        if data is not None:
+            self.set_data(i, data)
+        return i
+
+    def set_data(self, i, data):
+        import numpy as np
+        self.data[i] = np.ascontiguousarray(data).reshape(-1).view(np.uint8)
+
+    def _data_table(self):
+        table = (ctypes.c_void_p * len(self.nodes))()
+        for i, a in self.data.items():
+            table[i] = a.ctypes.data
+        return table
 
     def convert(self, x, type_):
         return self._add("convert", type_, self.shape(x), [x])
@@ -177,6 +193,22 @@ class Graph:
         out = _lib.MoeFold()
         check(_lib.load().ovfcc_fold_moe(self._array(), len(self.nodes), root, ctypes.byref(out)))
         return out
+
+    def create_weights(self, device, fold: _lib.Fold, extra_flags: int = 0):
+        """The node a fold describes, created from the data of its Constants (ovfcc_fold_weights_create)."""
+        from .fc import CompressedWeights
+        h = ctypes.c_void_p()
+        check(device.lib.ovfcc_fold_weights_create(device.handle, self._array(), len(self.nodes), ctypes.byref(fold),
+                                                   self._data_table(), extra_flags, ctypes.byref(h)))
+        return CompressedWeights.adopt(device, h, fold.desc, extra_flags)
+
+    def create_expert_weights(self, device, fold: _lib.GatherFold, expert: int, extra_flags: int = 0):
+        """Expert (or group) `expert` of a gather / grouped fold as a node of its own."""
+        from .fc import CompressedWeights
+        h = ctypes.c_void_p()
+        check(device.lib.ovfcc_fold_expert_weights_create(device.handle, self._array(), len(self.nodes), ctypes.byref(fold),
+                                                          expert, self._data_table(), extra_flags, ctypes.byref(h)))
+        return CompressedWeights.adopt(device, h, fold.desc, extra_flags)
 
     def fold_model(self, max_folds: int = 64):
         folds = (_lib.Fold * max_folds)()

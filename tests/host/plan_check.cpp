@@ -1,6 +1,6 @@
 // Host-logic check, built with AddressSanitizer and UBSan by tests/test_host_logic.py: descriptor gate, layout,
 // repack round trips on exactly sized buffers, and the invariants every launch plan must satisfy before a kernel
-// may be launched with it.  No GPU: the kernel launchers are stubbed out below and never called.
+// may be launched with it.  No GPU: the kernel launchers are stubbed out (launch_stubs.h) and never called.
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -10,20 +10,7 @@
 
 #include "ovfcc_internal.h"
 
-namespace ovfcc {
-int launch_plain(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int launch_decode(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int launch_batch(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int launch_gemv(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int launch_gemv16(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int gemv16_kblocks_per_wave(int c_table, int split_k) { return split_k > 1 ? c_table / split_k : (c_table == 2 ? 2 : 4); }
-size_t gemv16_lds_bytes(int c, int waves, int red_bufs) { return (size_t)waves * c * 4096 + (size_t)red_bufs * waves * 1024; }
-int launch_prefill(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int launch_prefill_wide(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int launch_prefill_direct(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int launch_prefill_async(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-int launch_prefill_big(const FcDeviceArgs&, const LaunchPlan&, void*) { return -1; }
-}  // namespace ovfcc
+#include "launch_stubs.h"
 
 static int g_failures = 0;
 #define CHECK(cond, ...)                                   \

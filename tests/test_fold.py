@@ -2,18 +2,14 @@
 FullyConnectedCompressed fold with its shape algebra, the bias fusion rule, horizontal fusion and the gated linear
 unit -- driven by the structural cases of the reference's own tests (tests/golden/fold_cases.json) and by negative
 cases for every rule.  No GPU, no OpenVINO."""
-import json
-import os
-
 import pytest
 
 from openvino_amd import _lib, fc
 from openvino_amd._lib import OvfccError
 from openvino_amd.graph import Graph, decompression_subgraph
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-with open(os.path.join(HERE, "golden", "fold_cases.json")) as fh:
-    CASES = json.load(fh)
+from fold_graphs import CASES, expert_weights, moe_block
+from fold_graphs import simple_matmul as _simple
 
 
 def ids(rows, keys):
@@ -109,17 +105,6 @@ def test_reference_builder_shapes(p):
     assert d.zp_scalar == int(p["zp"] == "scalar" and OC * (IC // G) != 1)
     assert d.zp_type == (_lib.NONE if p["zp"] == "empty" else _lib.TYPE[p["type"]])
     assert d.out_type == _lib.F16 and f.activations_f32 == 0
-
-
-def _simple(g, x, N=64, K=256, G=128, w_type="u4", zp=True, major="output", scale_type="f16", out=None):
-    ng = K // G
-    if major == "output":
-        chain = decompression_subgraph(g, w_type, [N, ng, G], [N, ng, 1], [N, ng, 1] if zp else None, w_type,
-                                       scale_type=scale_type, compute_type="f16", reshape_to=[N, K])
-        return g.matmul(x, chain, transpose_b=True, type_=out)
-    chain = decompression_subgraph(g, w_type, [ng, G, N], [ng, 1, N], [ng, 1, N] if zp else None, w_type,
-                                   scale_type=scale_type, compute_type="f16", reshape_to=[K, N])
-    return g.matmul(x, chain, type_=out)
 
 
 def test_bias_add_folds_in_by_the_reference_rule():
@@ -315,17 +300,6 @@ def test_grouping_rules():
 
 # ---- mixture-of-experts layers: GatherMatmul over batched compressed weights, and the three-projection block ----
 
-def expert_weights(g, type_, wei_shape, scale_zp_shape, grouped, with_zp=True, compute="f32"):
-    """Constant -> Convert -> [Subtract] -> Multiply -> [Reshape to three dimensions], as the reference's test builds it."""
-    w = g.convert(g.constant(type_, wei_shape), compute)
-    if with_zp:
-        w = g.subtract(w, g.convert(g.constant(type_, scale_zp_shape), compute))
-    w = g.multiply(w, g.constant(compute, scale_zp_shape))
-    if grouped:
-        w = g.reshape(w, list(wei_shape[:-2]) + [wei_shape[-2] * wei_shape[-1]])
-    return w
-
-
 @pytest.mark.parametrize("case", CASES["convert_gather_matmul_to_compressed"],
                          ids=lambda c: f"{c['type']}-{'grouped' if c['grouped'] else 'plain'}-{c['wei_shape']}")
 def test_gather_matmul_over_compressed_experts(case):
@@ -462,29 +436,6 @@ def test_grouped_matmul_fold_refusals():
     with pytest.raises(OvfccError) as e:
         g.fold_grouped_matmul(g._add("grouped_matmul", "f16", [-1, 64], [a2, w]))   # two-dimensional A, no offsets
     assert e.value.code == _lib.EINVAL
-
-
-def moe_block(g, act, compressed, E, H, I, top_k, hidden_shape, wtype="u4", G=128, routing_slice=False):
-    """build_3gemm_bgm_model with compressed experts: returns (root, hidden, routing producer, indices, nodes)."""
-    hidden = g.parameter("f16", hidden_shape)
-    flat = g.reshape(hidden, [-1, H]) if len(hidden_shape) != 2 else hidden
-    u = g.unsqueeze(flat, 0)
-    idx = g.parameter("i32", [-1, top_k])
-    routing = g.parameter("f16", [-1, E if routing_slice else top_k])
-
-    def bgm(x, N, K):
-        if compressed:
-            return g.gather_matmul_compressed(x, g.constant(wtype, [E, N, K]), idx, g.constant("f16", [E, N, K // G]),
-                                              g.constant(wtype, [E, N, K // G]))
-        return g.gather_matmul(x, expert_weights(g, wtype, [E, N, K // G, G], [E, N, K // G, 1], True, compute="f16"), idx)
-    gate = bgm(u, I, H)
-    a = g.swish(gate) if act == "swish" else g.gelu(gate, tanh=(act == "gelu_tanh"))
-    up = bgm(u, I, H)
-    down = bgm(g.multiply(a, up), H, I)
-    r = g.slice(routing, [-1, top_k]) if routing_slice else routing
-    final = g.multiply(down, g.unsqueeze(g.transpose(r, [1, 0]), -1))
-    out = g.reshape(g.reduce_sum(final, 0), hidden_shape)
-    return out, hidden, r, idx, (gate, up, down)
 
 
 @pytest.mark.parametrize("act", CASES["moe_block"]["activations"])
