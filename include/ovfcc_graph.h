@@ -120,14 +120,20 @@ enum ovfcc_fused_kind {
     OVFCC_FUSED_SINGLE = 0, /* one node of its own */
     OVFCC_FUSED_CONCAT = 1, /* siblings reading the same activations, concatenated along N (ovfcc_weights_concat);
                                part i owns the next parts[i].N output columns */
-    OVFCC_FUSED_GLU = 2     /* parts[0] = gate, parts[1] = up, glu_type applied (ovfcc_weights_glu); root = the Multiply */
+    OVFCC_FUSED_GLU = 2,    /* parts[0] = gate, parts[1] = up, glu_type applied (ovfcc_weights_glu); root = the Multiply */
+    OVFCC_FUSED_MLP = 3     /* a gated unit read by nothing but one more compressed MatMul: parts[0] = gate, parts[1] = up,
+                               parts[2] = down (ovfcc_weights_glu, then ovfcc_weights_mlp with the down node); root = the
+                               down projection's root.  The subgraph MLPFusionPass folds into LLMMLP
+                               (src/plugins/intel_cpu/src/transformations/cpu_opset/x64/pass/mlp_fusion.cpp:48-120),
+                               here over compressed weights of any supported type; the gated unit's output must be f16 */
 };
 typedef struct ovfcc_fused {
     int32_t kind;
     int32_t n_parts;
     int32_t parts[4];  /* indices into the folds array */
     int32_t glu_type;  /* OVFCC_GLU_SWISH | OVFCC_GLU_GELU | OVFCC_GLU_GELU_TANH */
-    int32_t root;      /* GLU: the Multiply node that the fused node's output replaces; otherwise -1 */
+    int32_t root;      /* GLU: the Multiply node that the fused node's output replaces; MLP: the down projection's
+                          root; otherwise -1 */
 } ovfcc_fused;
 
 /* Every compressed FullyConnected of the node array (bias Adds folded in where the reference's rule allows) in

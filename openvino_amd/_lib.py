@@ -58,7 +58,7 @@ OP = {"other": 0, "parameter": 1, "constant": 2, "convert": 3, "subtract": 4, "m
       "gather_matmul": 14, "gather_matmul_compressed": 15, "unsqueeze": 16, "slice": 17, "reduce_sum": 18,
       "grouped_matmul": 19, "grouped_matmul_compressed": 20}
 MAX_INPUTS = 6
-FUSED_SINGLE, FUSED_CONCAT, FUSED_GLU = 0, 1, 2
+FUSED_SINGLE, FUSED_CONCAT, FUSED_GLU, FUSED_MLP = 0, 1, 2, 3
 
 
 class GNode(ctypes.Structure):

@@ -1161,10 +1161,11 @@ struct BlobHeader {
     uint32_t header_bytes;
     ovfcc_fc_desc desc;
     int32_t zp_const;
-    int32_t tiled;
+    int32_t tiled;        // kBlobTiled | kBlobHasDown
     uint64_t w_bytes, scale_bytes, zp_bytes, bias_bytes;
 };
 constexpr uint32_t kBlobVersion = 2;
+constexpr int32_t kBlobTiled = 1, kBlobHasDown = 2;  // bits of BlobHeader::tiled; HasDown: another node's blob follows
 const char kBlobMagic[8] = {'O', 'V', 'F', 'C', 'C', 'W', 0, 0};
 
 size_t pad16(size_t n) {
@@ -1190,26 +1191,33 @@ void device_sizes(const ovfcc_fc_desc& d, const ovfcc::Layout& L, uint64_t out[4
 
 }  // namespace
 
-int ovfcc_weights_export_size(const ovfcc_weights* w, size_t* bytes) {
-    if (w && w->mlp_down)
-        return fail(OVFCC_EUNSUPPORTED, "an MLP node is exported as its two nodes; export them before ovfcc_weights_mlp");
-    if (!w || !bytes)
-        return fail(OVFCC_EINVAL, "null argument");
+// one node's own part of a blob (an MLP node's blob is its first node's part followed by its down projection's)
+static size_t own_blob_bytes(const ovfcc_weights* w) {
     uint64_t sz[4];
     device_sizes(w->desc, w->layout, sz);
-    *bytes = pad16(sizeof(BlobHeader)) + pad16(sz[0]) + pad16(sz[1]) + pad16(sz[2]) + pad16(sz[3]);
+    return pad16(sizeof(BlobHeader)) + pad16(sz[0]) + pad16(sz[1]) + pad16(sz[2]) + pad16(sz[3]);
+}
+
+int ovfcc_weights_export_size(const ovfcc_weights* w, size_t* bytes) {
+    if (!w || !bytes)
+        return fail(OVFCC_EINVAL, "null argument");
+    *bytes = own_blob_bytes(w) + (w->mlp_down ? own_blob_bytes(w->mlp_down) : 0);
     return OVFCC_OK;
 }
 
 int ovfcc_weights_export(const ovfcc_weights* w, void* blob, size_t bytes) {
-    if (w && w->mlp_down)
-        return fail(OVFCC_EUNSUPPORTED, "an MLP node is exported as its two nodes; export them before ovfcc_weights_mlp");
-    size_t need = 0;
-    int rc = ovfcc_weights_export_size(w, &need);
+    size_t total = 0;
+    int rc = ovfcc_weights_export_size(w, &total);
     if (rc)
         return rc;
-    if (!blob || bytes < need)
+    if (!blob || bytes < total)
         return fail(OVFCC_EINVAL, "blob buffer is null or too small");
+    const size_t need = own_blob_bytes(w);
+    if (w->mlp_down) {
+        rc = ovfcc_weights_export(w->mlp_down, static_cast<char*>(blob) + need, bytes - need);
+        if (rc)
+            return rc;
+    }
     HIP_TRY(hipSetDevice(w->ctx->device));
     uint64_t sz[4];
     device_sizes(w->desc, w->layout, sz);
@@ -1219,7 +1227,7 @@ int ovfcc_weights_export(const ovfcc_weights* w, void* blob, size_t bytes) {
     h.header_bytes = (uint32_t)sizeof(BlobHeader);
     h.desc = w->desc;
     h.zp_const = w->layout.zp_const;
-    h.tiled = w->layout.tiled ? 1 : 0;
+    h.tiled = (w->layout.tiled ? kBlobTiled : 0) | (w->mlp_down ? kBlobHasDown : 0);
     h.w_bytes = sz[0], h.scale_bytes = sz[1], h.zp_bytes = sz[2], h.bias_bytes = sz[3];
     char* at = static_cast<char*>(blob);
     std::memset(at, 0, need);
@@ -1252,9 +1260,10 @@ int ovfcc_weights_import(ovfcc_ctx* ctx, const void* blob, size_t bytes, ovfcc_w
     device_sizes(h.desc, L, sz);
     // a scalar zero-point lives in zp_const; everything else must be exactly what the descriptor implies
     const int zp_lo = L.zp_offset, zp_hi = L.zp_offset + 255;
-    if ((h.tiled != 0) != L.tiled || h.w_bytes != sz[0] || h.scale_bytes != sz[1] || h.zp_bytes != sz[2] ||
+    const size_t need = pad16(sizeof(BlobHeader)) + pad16(sz[0]) + pad16(sz[1]) + pad16(sz[2]) + pad16(sz[3]);
+    if ((h.tiled & ~(kBlobTiled | kBlobHasDown)) != 0 || ((h.tiled & kBlobTiled) != 0) != L.tiled || h.w_bytes != sz[0] || h.scale_bytes != sz[1] || h.zp_bytes != sz[2] ||
         h.bias_bytes != sz[3] || h.zp_const < zp_lo || h.zp_const > zp_hi ||
-        bytes < pad16(sizeof(BlobHeader)) + pad16(sz[0]) + pad16(sz[1]) + pad16(sz[2]) + pad16(sz[3]))
+        bytes < need)
         return fail(OVFCC_EINVAL, "blob sizes do not match its descriptor");
     L.zp_const = h.zp_const;
     HIP_TRY(hipSetDevice(ctx->device));
@@ -1277,6 +1286,18 @@ int ovfcc_weights_import(ovfcc_ctx* ctx, const void* blob, size_t bytes, ovfcc_w
     }
     if (!rc)
         rc = finish_weights(W);
+    if (!rc && (h.tiled & kBlobHasDown)) {
+        // an MLP node: the down projection's blob follows; the pair must fit as ovfcc_weights_mlp demands
+        ovfcc_weights* down = nullptr;
+        rc = ovfcc_weights_import(ctx, static_cast<const char*>(blob) + need, bytes - need, &down);
+        if (!rc && (down->mlp_down || !W->layout.glu || down->layout.glu || W->desc.out_type != OVFCC_F16 ||
+                    out_channels(W) != down->desc.K))
+            rc = fail(OVFCC_EINVAL, "the two nodes of an MLP blob do not fit each other");
+        if (rc)
+            ovfcc_weights_destroy(down);
+        else
+            W->mlp_down = down;
+    }
     if (rc) {
         ovfcc_weights_destroy(W);
         return rc;

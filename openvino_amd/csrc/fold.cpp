@@ -813,6 +813,27 @@ int ovfcc_fold_model(const ovfcc_gnode* nodes, int n_nodes, ovfcc_fold* folds, i
             break;
         }
     }
+    // MLP: a gated unit whose only reader is one more compressed MatMul (the down projection) becomes one node with
+    // it, where the intermediate activations are f16 as between two nodes
+    for (ovfcc_fused& u : groups) {
+        const int mul = u.root;
+        if (users[(size_t)mul].size() != 1)
+            continue;
+        const ovfcc_fold& gate = found[(size_t)u.parts[0]];
+        for (size_t d = 0; d < found.size(); ++d) {
+            const ovfcc_fold& down = found[d];
+            if (taken[d] || down.activations != mul || down.matmul != users[(size_t)mul][0])
+                continue;
+            if (gate.desc.out_type != OVFCC_F16 || down.desc.K != gate.desc.N || down.activations_f32)
+                continue;
+            u.kind = OVFCC_FUSED_MLP;
+            u.n_parts = 3;
+            u.parts[2] = (int)d;
+            u.root = down.root;
+            taken[d] = 1;
+            break;
+        }
+    }
     // horizontal fusion: two or three siblings of one format over the same activations share a launch
     for (size_t a = 0; a < found.size(); ++a) {
         if (taken[a])

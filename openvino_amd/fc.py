@@ -111,6 +111,12 @@ class Device:
         return 2.0 * nbytes * iters / (ms.value * 1e-3) / 1e9
 
 
+class _BlobHeader(ctypes.Structure):
+    """Head of an exported node (ovfcc_weights_export): the device arrays follow, each padded to 16 bytes."""
+    _fields_ = [("magic", ctypes.c_char * 8), ("version", ctypes.c_uint32), ("header_bytes", ctypes.c_uint32),
+                ("desc", FcDesc), ("zp_const", ctypes.c_int32), ("tiled", ctypes.c_int32), ("sizes", ctypes.c_uint64 * 4)]
+
+
 class CompressedWeights:
     """Repacked, device-resident constants of one FullyConnectedCompressed node."""
 
@@ -234,10 +240,21 @@ class CompressedWeights:
         blob = np.ascontiguousarray(blob, dtype=np.uint8)
         h = ctypes.c_void_p()
         check(device.lib.ovfcc_weights_import(device.handle, _vp(blob), blob.nbytes, ctypes.byref(h)))
-        other = object.__new__(CompressedWeights)
-        other.device = device
-        other.desc = FcDesc.from_buffer_copy(blob[16:16 + ctypes.sizeof(FcDesc)].tobytes())
-        other.N, other.K, other.group_size = other.desc.N, other.desc.K, other.desc.group_size
+        def described(at):
+            """(stand-in carrying the descriptor of the node whose blob starts at byte `at`, where that blob ends,
+            whether another node's blob follows)"""
+            head = _BlobHeader.from_buffer_copy(blob[at:at + ctypes.sizeof(_BlobHeader)].tobytes())
+            node = object.__new__(CompressedWeights)
+            node.device, node.handle = device, None
+            node.desc = FcDesc.from_buffer_copy(head.desc)
+            node.N, node.K, node.group_size = node.desc.N, node.desc.K, node.desc.group_size
+            pad = lambda n: (n + 15) & ~15
+            end = at + pad(ctypes.sizeof(_BlobHeader)) + sum(pad(int(n)) for n in head.sizes)
+            return node, end, bool(head.tiled & 2)
+
+        other, end, has_down = described(0)
+        if has_down:     # an MLP node: shapes and types of the output side come from the second blob
+            other.down = described(end)[0]
         other.handle = h
         return other
 

@@ -92,7 +92,7 @@ namespace ovfcc_plugin {
 // The decisions -- which subgraph is one FullyConnectedCompressed node, how its constants are re-viewed, which bias
 // Add folds in, which nodes share a launch -- are taken by libovfcc on a plain description of the model
 // (include/ovfcc_graph.h), where they are unit-tested without OpenVINO.  This file only translates: ov::Node ->
-// ovfcc_gnode on the way in, constant bytes -> ovfcc_weights_create on the way out.
+// ovfcc_gnode on the way in, the Constants' bytes -> ovfcc_fold_weights_create on the way out.
 
 static int type_tag(const ov::element::Type& t) {
     if (t == ov::element::u4) return OVFCC_U4;
@@ -107,6 +107,7 @@ static int type_tag(const ov::element::Type& t) {
 struct ModelGraph {
     std::vector<std::shared_ptr<ov::Node>> ops;  // topological order; index = node id
     std::vector<ovfcc_gnode> nodes;
+    std::vector<const void*> constant_data;      // per node: a Constant's bytes (the model keeps them alive), else null
     std::vector<ovfcc_fold> folds;
     std::vector<ovfcc_fused> fused;
     std::vector<ovfcc_moe_fold> moes;  // expert blocks (three GatherMatmul nodes and what joins them)
@@ -126,6 +127,7 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
     for (size_t i = 0; i < g.ops.size(); ++i)
         index[g.ops[i].get()] = (int)i;
     g.nodes.resize(g.ops.size());
+    g.constant_data.assign(g.ops.size(), nullptr);
     for (size_t i = 0; i < g.ops.size(); ++i) {
         const auto& op = g.ops[i];
         ovfcc_gnode& n = g.nodes[i];
@@ -181,6 +183,7 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
             if (sw->get_input_size() != 1)
                 n.op = OVFCC_OP_OTHER;  // a beta input: not the beta = 1 form the kernels compute
         } else if (auto c = ov::as_type_ptr<ov::op::v0::Constant>(op)) {
+            g.constant_data[i] = c->get_data_ptr();
             // FullyConnected's "no bias" is Constant(dynamic, Shape{0}); small integer constants carry their values
             if (c->get_element_type().is_integral_number() && c->get_element_type().bitwidth() >= 8 &&
                 ov::shape_size(c->get_shape()) <= OVFCC_MAX_RANK) {
@@ -225,115 +228,19 @@ static ModelGraph describe(const std::shared_ptr<const ov::Model>& model) {
     return g;
 }
 
-// Host copies of one matched node's constants in the form ovfcc_weights_create takes them.
-struct NodeData {
-    ovfcc_fc_desc desc{};
-    const void* weights = nullptr;         // the Constant's own bytes, OpenVINO order
-    std::vector<ov::float16> scales;       // [N, K/G] ([K/G, N] with OVFCC_W_INPUT_MAJOR)
-    std::vector<uint8_t> zero_points;      // packed u4 / u8, or one element
-    std::vector<ov::float16> bias;         // [N]
-};
-
-static NodeData node_data(const ModelGraph& g, const ovfcc_fold& f) {
-    NodeData d;
-    d.desc = f.desc;
-    const auto constant = [&g](int id) { return ov::as_type_ptr<ov::op::v0::Constant>(g.ops[(size_t)id]); };
-    d.weights = constant(f.weights)->get_data_ptr();
-    const size_t groups = (size_t)(f.desc.N * (f.desc.K / f.desc.group_size));
-    {
-        const auto vals = constant(f.scales)->cast_vector<float>();
-        d.scales.resize(groups);
-        OPENVINO_ASSERT(f.scale_broadcast ? vals.size() == 1 : vals.size() == groups, "MI355X: scale constant of ",
-                        vals.size(), " elements for ", groups, " groups");
-        for (size_t i = 0; i < groups; ++i)
-            d.scales[i] = ov::float16(vals[f.scale_broadcast ? 0 : i]);
-    }
-    if (f.zero_points >= 0) {
-        auto zp = constant(f.zero_points);
-        if (f.zp_from_real) {
-            // real-typed zero-points (NNCF stores some so) must be integers in 0..255 and become u8
-            const auto vals = zp->cast_vector<float>();
-            d.zero_points.resize(vals.size());
-            for (size_t i = 0; i < vals.size(); ++i) {
-                OPENVINO_ASSERT(vals[i] >= 0 && vals[i] <= 255 && vals[i] == (float)(int)vals[i],
-                                "MI355X: zero-point values must be integers in 0..255");
-                d.zero_points[i] = (uint8_t)vals[i];
-            }
-        } else {
-            const auto* bytes = static_cast<const uint8_t*>(zp->get_data_ptr());
-            d.zero_points.assign(bytes, bytes + zp->get_byte_size());
-        }
-    }
-    if (f.bias >= 0) {
-        const auto vals = constant(f.bias)->cast_vector<float>();
-        d.bias.resize(vals.size());
-        for (size_t i = 0; i < vals.size(); ++i)
-            d.bias[i] = ov::float16(vals[i]);
-    }
-    return d;
+// A matched node, or expert e of a routed / grouped one, created by the library from the Constants' own bytes.
+static ovfcc_weights* create_node(ovfcc_ctx* ctx, const ModelGraph& g, const ovfcc_fold& f, int flags) {
+    ovfcc_weights* out = nullptr;
+    if (ovfcc_fold_weights_create(ctx, g.nodes.data(), (int)g.nodes.size(), &f, g.constant_data.data(), flags, &out) != OVFCC_OK)
+        throw_last("fold_weights_create");
+    return out;
 }
 
-// Expert e's node of a GatherMatmul fold: slice e of every constant, unpacked and re-packed where a 4-bit slice
-// starts in the middle of a byte.
 static ovfcc_weights* create_expert(ovfcc_ctx* ctx, const ModelGraph& g, const ovfcc_gather_fold& f, int e, int flags) {
-    const auto constant = [&g](int id) { return ov::as_type_ptr<ov::op::v0::Constant>(g.ops[(size_t)id]); };
-    const auto four = [](int t) { return t == OVFCC_U4 || t == OVFCC_I4; };
-    // `count` elements starting at element `first` of a packed constant, as a packed buffer of their own
-    const auto slice = [&](const std::shared_ptr<ov::op::v0::Constant>& c, bool nibbles, size_t first, size_t count) {
-        const auto* bytes = static_cast<const uint8_t*>(c->get_data_ptr());
-        std::vector<uint8_t> out(nibbles ? (count + 1) / 2 : count, 0);
-        if (!nibbles) {
-            std::memcpy(out.data(), bytes + first, count);
-        } else if ((first & 1) == 0) {
-            std::memcpy(out.data(), bytes + first / 2, (count + 1) / 2);
-        } else {
-            for (size_t i = 0; i < count; ++i) {
-                const size_t at = first + i;
-                const uint8_t v = (at & 1) ? (bytes[at >> 1] >> 4) : (bytes[at >> 1] & 15);
-                out[i >> 1] |= (uint8_t)((i & 1) ? v << 4 : v);
-            }
-        }
-        return out;
-    };
-    ovfcc_fc_desc d = f.desc;
-    d.flags |= flags;
-    const size_t N = (size_t)d.N, K = (size_t)d.K, ng = K / (size_t)d.group_size;
-    const auto w = slice(constant(f.weights), four(d.w_type), (size_t)e * N * K, N * K);
-    std::vector<ov::float16> scales(N * ng);
-    {
-        const auto vals = constant(f.scales)->cast_vector<float>();
-        for (size_t i = 0; i < N * ng; ++i)
-            scales[i] = ov::float16(vals[f.scale_broadcast ? 0 : (size_t)e * N * ng + i]);
-    }
-    std::vector<uint8_t> zp;
-    if (f.zero_points >= 0) {
-        auto z = constant(f.zero_points);
-        if (f.zp_from_real) {
-            const auto vals = z->cast_vector<float>();
-            const size_t count = d.zp_scalar ? 1 : N * ng, first = d.zp_scalar ? 0 : (size_t)e * N * ng;
-            zp.resize(count);
-            for (size_t i = 0; i < count; ++i) {
-                const float v = vals[first + i];
-                OPENVINO_ASSERT(v >= 0 && v <= 255 && v == (float)(int)v, "MI355X: zero-point values must be integers in 0..255");
-                zp[i] = (uint8_t)v;
-            }
-        } else if (d.zp_scalar) {
-            zp = slice(z, d.zp_type == OVFCC_U4, 0, 1);
-        } else {
-            zp = slice(z, d.zp_type == OVFCC_U4, (size_t)e * N * ng, N * ng);
-        }
-    }
-    std::vector<ov::float16> bias;
-    if (f.bias >= 0) {
-        const auto vals = constant(f.bias)->cast_vector<float>();
-        bias.resize(N);
-        for (size_t i = 0; i < N; ++i)
-            bias[i] = ov::float16(vals[(f.bias_per_expert ? (size_t)e * N : 0) + i]);
-    }
     ovfcc_weights* out = nullptr;
-    if (ovfcc_weights_create(ctx, &d, w.data(), scales.data(), zp.empty() ? nullptr : zp.data(),
-                             bias.empty() ? nullptr : bias.data(), &out) != OVFCC_OK)
-        throw_last("weights_create (expert)");
+    if (ovfcc_fold_expert_weights_create(ctx, g.nodes.data(), (int)g.nodes.size(), &f, e, g.constant_data.data(), flags,
+                                         &out) != OVFCC_OK)
+        throw_last("fold_expert_weights_create");
     return out;
 }
 
@@ -1241,15 +1148,19 @@ public:
                 mark(f.root);
                 if (g.nodes[(size_t)f.activations].op == OVFCC_OP_PARAMETER)
                     mark(f.activations);
-                if (u.kind != OVFCC_FUSED_GLU)
+                // gate and up of a gated unit feed its Multiply, not a model output
+                if (u.kind == OVFCC_FUSED_SINGLE || u.kind == OVFCC_FUSED_CONCAT || (u.kind == OVFCC_FUSED_MLP && k == 2))
                     mark_results_of(f.root);
             }
-            if (u.kind == OVFCC_FUSED_GLU) {
-                mark(u.root);
-                for (const auto& in : g.ops[(size_t)u.root]->input_values())  // the gate's activation node
+            if (u.kind == OVFCC_FUSED_GLU || u.kind == OVFCC_FUSED_MLP) {
+                // the unit's Multiply: the group's root, or what the down projection of an MLP group reads
+                const int mul = u.kind == OVFCC_FUSED_GLU ? u.root : g.folds[(size_t)u.parts[2]].activations;
+                mark(mul);
+                for (const auto& in : g.ops[(size_t)mul]->input_values())  // the gate's activation node
                     if (ov::is_type<ov::op::v4::Swish>(in.get_node()) || ov::is_type<ov::op::v7::Gelu>(in.get_node()))
                         res[in.get_node()->get_friendly_name()] = get_device_name();
-                mark_results_of(u.root);
+                if (u.kind == OVFCC_FUSED_GLU)
+                    mark_results_of(u.root);
             }
         }
         for (const auto& m : g.moes) {
@@ -1320,15 +1231,7 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
                 out.push_back(r);
         return out;
     };
-    auto create = [&](const ovfcc_fold& f) {
-        NodeData d = node_data(g, f);
-        d.desc.flags |= node_flags;
-        ovfcc_weights* w = nullptr;
-        if (ovfcc_weights_create(ctx, &d.desc, d.weights, d.scales.data(), d.zero_points.empty() ? nullptr : d.zero_points.data(),
-                                 d.bias.empty() ? nullptr : d.bias.data(), &w) != OVFCC_OK)
-            throw_last("weights_create");
-        return w;
-    };
+    auto create = [&](const ovfcc_fold& f) { return create_node(ctx, g, f, node_flags); };
     auto primitive = [](const ovfcc_weights* w, const ovfcc_fc_desc& d, const char* suffix) {
         return std::string(ovfcc_weights_is_tiled(w) ? "hip_tiled_w" : "hip_plain_w") +
                (d.w_type == OVFCC_U8 || d.w_type == OVFCC_I8 ? "8" : "4") + suffix;
@@ -1357,23 +1260,37 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
     };
     for (const auto& u : g.fused) {
         const ovfcc_fold& f0 = g.folds[(size_t)u.parts[0]];
-        if (u.kind == OVFCC_FUSED_GLU) {
+        if (u.kind == OVFCC_FUSED_GLU || u.kind == OVFCC_FUSED_MLP) {
+            // gate and up with their gated linear unit as one node; with the down projection behind it, one MLP node
+            const bool mlp = u.kind == OVFCC_FUSED_MLP;
+            const ovfcc_fold& last = g.folds[(size_t)u.parts[mlp ? 2 : 0]];
             Launch l = start_launch(f0, u.kind);
-            l.N_out = f0.desc.N;
+            l.N_out = last.desc.N;
+            l.out_type = last.desc.out_type;
             l.name = g.ops[(size_t)u.root]->get_friendly_name();
-            l.folds = {u.parts[0], u.parts[1]};
+            l.folds.assign(u.parts, u.parts + u.n_parts);
             add_outputs(l, u.root, 0, l.N_out);
             if (!blobs) {
                 ovfcc_weights *gate = create(f0), *up = create(g.folds[(size_t)u.parts[1]]);
-                const int rc = ovfcc_weights_glu(gate, up, u.glu_type, &l.weights);
+                int rc = ovfcc_weights_glu(gate, up, u.glu_type, &l.weights);
                 ovfcc_weights_destroy(gate);
                 ovfcc_weights_destroy(up);
                 if (rc != OVFCC_OK)
                     throw_last("weights_glu");
+                if (mlp) {
+                    ovfcc_weights *unit = l.weights, *down = create(last);
+                    l.weights = nullptr;
+                    rc = ovfcc_weights_mlp(unit, down, &l.weights);
+                    ovfcc_weights_destroy(unit);
+                    ovfcc_weights_destroy(down);
+                    if (rc != OVFCC_OK)
+                        throw_last("weights_mlp");
+                }
             }
-            for (int k = 0; k < 2; ++k)
+            for (int k = 0; k < u.n_parts; ++k)
                 l.original_names.push_back(g.ops[(size_t)g.folds[(size_t)u.parts[k]].matmul]->get_friendly_name());
-            l.original_names.push_back(l.name);
+            if (!mlp || last.root != last.matmul)
+                l.original_names.push_back(l.name);
             m_launches.push_back(std::move(l));
             continue;
         }
@@ -1503,7 +1420,9 @@ CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std:
     }
     for (auto& l : m_launches)
         l.primitive = primitive(l.weights, g.folds[(size_t)l.folds[0]].desc,
-                                l.kind == OVFCC_FUSED_GLU ? "_glu" : (l.kind == OVFCC_FUSED_CONCAT ? "_fused" : ""));
+                                l.kind == OVFCC_FUSED_MLP   ? "_mlp"
+                                : l.kind == OVFCC_FUSED_GLU ? "_glu"
+                                                            : (l.kind == OVFCC_FUSED_CONCAT ? "_fused" : ""));
     m_last_us = std::vector<std::atomic<double>>(m_launches.size() + m_moes.size() + m_grouped.size());
     for (auto& t : m_last_us)
         t.store(-1.0);

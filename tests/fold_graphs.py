@@ -183,6 +183,20 @@ def block_model(H=512, I=1024):
     return g, dict(x=x, x2=x2, x3=x3, q=q, k=k, v=v, gate=gate, up=up, act=act, down=down)
 
 
+def mlp_model(H=512, I=1024, w_type="i4", zp=False, down_bias=True):
+    """gate and up over one Parameter, Swish(gate) * up, and the down projection that alone reads it (with a bias
+    Add): the subgraph the reference's MLPFusionPass matches.  Returns (g, x, root)."""
+    g = Graph()
+    x = g.parameter("f16", [-1, H])
+    gate = simple_matmul(g, x, N=I, K=H, w_type=w_type, zp=zp)
+    up = simple_matmul(g, x, N=I, K=H, w_type=w_type, zp=zp)
+    down = simple_matmul(g, g.multiply(g.swish(gate), up), N=H, K=I, w_type=w_type, zp=zp)
+    if down_bias:
+        down = g.add(down, g.constant("f16", [H]))
+    g.result(down)
+    return g, x, down
+
+
 def gather_graph(case, compressed=False, bias=None):
     """The reference's GatherMatmul test graph with the indices as a Parameter; bias: None, "shared" ([N]) or
     "per_expert" ([E, N]).  Returns (g, a, idx, root)."""

@@ -254,12 +254,47 @@ def test_model_level_grouping():
         kinds.setdefault(u.kind, []).append(u)
     (qkv,) = kinds[_lib.FUSED_CONCAT]
     assert [folds[qkv.parts[i]].root for i in range(qkv.n_parts)] == [q, k, v]
-    (glu,) = kinds[_lib.FUSED_GLU]
-    assert folds[glu.parts[0]].root == gate and folds[glu.parts[1]].root == up
-    assert glu.glu_type == _lib.GLU["swish"] and glu.root == act
+    # gate / up with their unit and the down projection that alone reads it: one MLP group, rooted at down
+    (mlp,) = kinds[_lib.FUSED_MLP]
+    assert [folds[mlp.parts[i]].root for i in range(3)] == [gate, up, down] and mlp.n_parts == 3
+    assert mlp.glu_type == _lib.GLU["swish"] and mlp.root == down and folds[mlp.parts[2]].activations == act
+    assert _lib.FUSED_GLU not in kinds
     singles = sorted(folds[u.parts[0]].root for u in kinds[_lib.FUSED_SINGLE])
-    assert singles == sorted([o_b, down]) and folds[by_root[o_b]].bias >= 0
+    assert singles == [o_b] and folds[by_root[o_b]].bias >= 0
     assert sorted(p for u in fused for p in u.parts[:u.n_parts]) == list(range(7))   # every fold in exactly one group
+
+
+def test_mlp_group_rules():
+    """The gated unit stays a group of its own (root = the Multiply) unless exactly one compressed MatMul reads it,
+    with f16 between the two: a second reader, a model output on the Multiply, f32 intermediate activations or a
+    node in between keep the down projection apart."""
+    def block(second_reader=False, f32=False, between=False, down_bias=False):
+        g = Graph()
+        t = "f32" if f32 else "f16"
+        h = g.parameter(t, [-1, 256])
+        gate = _simple(g, h, N=512, zp=False, w_type="i4")
+        up = _simple(g, h, N=512, zp=False, w_type="i4")
+        act = g.multiply(g.swish(gate), up)
+        src = g.other([act], type_=t, shape=[-1, 512]) if between else act
+        down = _simple(g, src, N=256, K=512)
+        if down_bias:
+            down = g.add(down, g.constant("f16", [256]))
+        g.result(down)
+        if second_reader:
+            g.result(act)
+        folds, fused = g.fold_model()
+        assert len(folds) == 3
+        return sorted(u.kind for u in fused), fused, folds, act, down
+
+    kinds, fused, folds, act, down = block()
+    assert kinds == [_lib.FUSED_MLP]
+    kinds, fused, folds, act, down = block(down_bias=True)     # the down projection's bias Add is its root
+    assert kinds == [_lib.FUSED_MLP] and fused[0].root == down and folds[fused[0].parts[2]].bias >= 0
+    for kw in (dict(second_reader=True), dict(f32=True), dict(between=True)):
+        kinds, fused, folds, act, down = block(**kw)
+        assert kinds == [_lib.FUSED_SINGLE, _lib.FUSED_GLU], kw
+        (glu,) = [u for u in fused if u.kind == _lib.FUSED_GLU]
+        assert glu.root == act and glu.n_parts == 2
 
 
 def test_grouping_rules():

@@ -16,7 +16,7 @@ import numpy as np
 import pytest
 
 from fold_graphs import (CASES, GATHER_FORMS, VARIANTS, block_model, builder_graph, convert_fc_graph, fill_fold,
-                         gather_graph, grouped_matmul_graph, moe_block, simple_matmul, transposed_graph, variant_graph)
+                         gather_graph, grouped_matmul_graph, mlp_model, moe_block, simple_matmul, transposed_graph, variant_graph)
 from graph_eval import Evaluator, decode_constant
 from openvino_amd import _lib
 from openvino_amd.graph import Graph
@@ -92,6 +92,8 @@ def all_cases():
         out.append((f"moe compressed={compressed}", MOE, g, root))
     g, _ = block_model()
     out.append(("block model", MODEL, g, -1))
+    g, _, _ = mlp_model()
+    out.append(("mlp model", MODEL, g, -1))
     return out
 
 
