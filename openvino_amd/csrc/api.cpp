@@ -465,16 +465,16 @@ bool plan_routed(ovfcc_request* r, const ovfcc_weights* w0, int64_t R, int n_exp
         return false;
     ovfcc::LaunchPlan& p = out->plan;
     int grid = 0;
-    bool split = false;
+    long long parked = 0;
     for (int t = 1; t <= (int)n; ++t) {
         const ovfcc::RoutedHeader h = ovfcc::routed_header(p.tiles_x, t, (int)w0->layout.k_blocks, r->ctx->n_cus);
         grid = std::max(grid, h.grid);
-        split = split || h.split_k > 1;
+        parked = std::max(parked, ovfcc::routed_parked_tiles(h, p.tiles_x));
     }
     p.n_cus = r->ctx->n_cus;
     p.grid[0] = (unsigned)grid, p.grid[1] = p.grid[2] = 1;
-    p.workspace_bytes = split ? (size_t)grid * p.tile_m * ovfcc::kPrefillWideN * sizeof(float) : 0;
-    p.counter_count = split ? (size_t)p.tiles_x * n : 0;
+    p.workspace_bytes = (size_t)parked * p.tile_m * ovfcc::kPrefillWideN * sizeof(float);
+    p.counter_count = parked ? (size_t)p.tiles_x * n : 0;
     out->cap = cap;
     out->n_slices = (int)n;
     return true;

@@ -438,8 +438,7 @@ __global__ __launch_bounds__(512) void fcc_prefill_async_grouped_kernel(const Ba
         const RoutedHeader h = *dev_hdr;
         if ((int)blockIdx.x >= h.grid)
             return;
-        tiles_y = h.tiles_y, tail_split = h.split_k, kb_per_split = h.kb_per_split;
-        full_tiles = h.split_k == 1 ? tiles_x * tiles_y : 0;
+        tiles_y = h.tiles_y, tail_split = h.split_k, kb_per_split = h.kb_per_split, full_tiles = h.full_tiles;
     }
     TileWork wk = tile_work(tiles_x, tiles_y, full_tiles, tail_split, kb_per_split, kb_total, 16 * NT, PA_BN / 2);
     BatchGroupItem it = dev_tab ? dev_tab[wk.tile_y] : tab.item[wk.tile_y];
@@ -578,7 +577,7 @@ int launch_prefill_async_grouped(const BatchGroupTable& tab, int n_items, const 
             const RoutedHeader h = routed_header(p.tiles_x, t, (int)L.k_blocks, p.n_cus);
             if ((unsigned)h.grid > p.grid[0] ||
                 (h.split_k > 1 && (!a.workspace || !a.counters ||
-                                   (size_t)h.grid * p.tile_m * PA_BN * sizeof(float) > p.workspace_bytes ||
+                                   (size_t)routed_parked_tiles(h, p.tiles_x) * p.tile_m * PA_BN * sizeof(float) > p.workspace_bytes ||
                                    (size_t)p.tiles_x * t > p.counter_count)))
                 return (int)hipErrorInvalidValue;
         }

@@ -221,22 +221,40 @@ int launch_batch_grouped(const BatchGroupTable& tab, int n_items, const FcDevice
 // slices and cuts K by the rule below, the host sizes grid, workspace and counters for the worst slice count.
 struct RoutedHeader {
     int tiles_y;       // slices in use
-    int split_k;       // parts along K of every tile (1: whole tiles)
+    int split_k;       // parts along K of the tiles that are split (1: whole tiles only)
     int kb_per_split;  // k-blocks per part
-    int grid;          // workgroups with work: tiles_x * tiles_y * split_k
+    int grid;          // workgroups with work: full_tiles + (tiles_x * tiles_y - full_tiles) * split_k
+    int full_tiles;    // tiles that one workgroup each computes whole; the rest are split
+    int pad[3];        // the slice table follows the header: keeps it 8-byte aligned
 };
 // K is split while the tiles alone leave compute units idle and every part keeps at least eight k-blocks (the
-// planner's rule for the register-fed prefill kernels).
+// planner's rule for the register-fed prefill kernels).  With more tiles than compute units, the tiles of a last
+// round that would fill at most half of them are split instead, so that the launch ends with a full round of shorter
+// workgroups rather than a half-empty round of whole tiles (tile_work, device_common.h).
 OVFCC_HOST_DEVICE inline RoutedHeader routed_header(int tiles_x, int slices, int kb_total, int n_cus) {
     const long long tiles = (long long)tiles_x * slices;
     int split = 1;
     while (split < 8 && tiles * split * 2 <= n_cus && kb_total / (split * 2) >= 8)
         split *= 2;
+    long long full = split == 1 ? tiles : 0;
+    const long long rest = tiles % n_cus;
+    if (split == 1 && tiles > n_cus && rest != 0) {
+        while (split < 8 && rest * split * 2 <= n_cus && kb_total / (split * 2) >= 8)
+            split *= 2;
+        if (split > 1)
+            full = tiles - rest;
+    }
     const int per = (kb_total + split - 1) / split;
     split = (kb_total + per - 1) / per;
     RoutedHeader h;
-    h.tiles_y = slices, h.split_k = split, h.kb_per_split = per, h.grid = (int)(tiles * split);
+    h.tiles_y = slices, h.split_k = split, h.kb_per_split = per, h.full_tiles = (int)full;
+    h.grid = (int)(full + (tiles - full) * split);
+    h.pad[0] = h.pad[1] = h.pad[2] = 0;
     return h;
+}
+// f32 tiles that the split parts of such a launch park in the workspace
+OVFCC_HOST_DEVICE inline long long routed_parked_tiles(const RoutedHeader& h, int tiles_x) {
+    return h.split_k > 1 ? ((long long)tiles_x * h.tiles_y - h.full_tiles) * h.split_k : 0;
 }
 // Slice height (64, 80, 96 or 128 rows) of a grouped prefill launch over items of these row counts (plan.cpp).
 int rows_cap_for(const int64_t* rows, int n, bool mid_ok);

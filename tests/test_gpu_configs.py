@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 from openvino_amd import _lib, datagen, fc
-from parity import check_parity, oracle_y
+from parity import REL_L2_MAX, T, ZT, check_parity, max_abs_limit, oracle_y
 
 pytestmark = pytest.mark.gpu
 
@@ -145,3 +145,56 @@ def test_config5_moe_experts(oracle, dev, req):
                 say(f"   expert {e} {which} M={M}: {info['name']} rel-L2={r[0]:.2e} max-abs={r[1]:.2e}")
             finally:
                 w.close()
+
+
+def test_config5_moe_block_real_shape(oracle, dev, req):
+    """Config 5 as one call at its real shape: 8 experts 4096 -> 14336 -> 4096 (u4 asymmetric, groups of 128, SwiGLU
+    fused into the gate / up node), 256 tokens, top-2 routing from datagen.moe_routing().  Sixteen sampled tokens are
+    compared with oracle.moe_reference; the device-routed entry point (indices in device memory) must give the same
+    bits as the host-routed one."""
+    say("config 5 block")
+    routes = datagen.moe_routing()
+    tokens = 256
+    indices = np.full((tokens, 2), -1, np.int32)
+    for e, rows in enumerate(routes):
+        for t in rows:
+            indices[t, 0 if indices[t, 0] < 0 else 1] = e
+    assert (indices >= 0).all()
+    gu_cases, dn_cases, wg, wd = [], [], [], []
+    try:
+        for e in range(len(routes)):
+            g, u = datagen.config5_expert(e, "gate", 1), datagen.config5_expert(e, "up", 1)
+            gu_cases.append(datagen.FcCase(1, g.K, 2 * g.N, 128, "u4", "u4", np.concatenate([g.w, u.w]),
+                                           np.concatenate([g.scale, u.scale]), np.concatenate([g.zp, u.zp]), g.x))
+            dn_cases.append(datagen.config5_expert(e, "down", 1))
+            wg.append(fc.CompressedWeights.from_case(dev, gu_cases[-1], glu="swish"))
+            wd.append(fc.CompressedWeights.from_case(dev, dn_cases[-1]))
+        rng = np.random.default_rng(55)
+        x = rng.standard_normal((tokens, 4096)).astype(np.float16)
+        rw = rng.uniform(0.2, 0.8, size=(tokens, 1))
+        routing = np.concatenate([rw, 1.0 - rw], axis=1).astype(np.float16)
+        say("   host-routed call")
+        y_host = req.moe(wg, wd, x, routing, indices)
+        info = req.last_kernel()
+        say(f"   device-routed call ({info['name']})")
+        y_dev = req.moe(wg, wd, x, routing, indices, device_indices=True)
+        assert y_host.shape == (tokens, 4096) and y_host.dtype == np.float16
+        assert np.array_equal(y_host.view(np.uint16), y_dev.view(np.uint16)), "host- and device-routed results differ"
+        pick = np.sort(np.random.default_rng(56).choice(tokens, size=16, replace=False))
+
+        def eargs(c):
+            return dict(w=c.w, w_type=T[c.w_type], scale=c.scale, zp=c.zp, zp_type=ZT[c.zp_type], bias=None,
+                        N=c.N, K=c.K, group_size=c.group_size)
+        ref = oracle.moe_reference(x[pick], routing[pick], indices[pick], [eargs(c) for c in gu_cases],
+                                   [eargs(c) for c in dn_cases], 1)
+        y = y_host[pick].astype(np.float32)
+        rl2, mab = oracle.rel_l2(y, ref), oracle.max_abs(y, ref)
+        # two projections in a row: the down projection's bound counts twice (its own arithmetic and the error its
+        # input carries), plus half an f16 ulp of the largest output
+        limit = 2 * max_abs_limit(14336) + float(np.max(np.abs(ref))) * 2.0 ** -11
+        say(f"   16 sampled tokens: rel-L2={rl2:.2e} max-abs={mab:.2e} (limit {limit:.2e})")
+        assert rl2 <= 2 * REL_L2_MAX and mab <= limit
+        assert np.all(np.isfinite(y_host.astype(np.float32)))
+    finally:
+        for w in wg + wd:
+            w.close()
