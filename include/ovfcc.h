@@ -235,8 +235,12 @@ int ovfcc_fc_run_device(ovfcc_request* req, const ovfcc_weights* w, const void* 
  * counters, held by every GPU the library runs on until the process ends) instead of buffers of the request,
  * and clear the counters they use with a small fill kernel first.  A launch that needs more than the array holds,
  * and a node whose activations would be quantised to int8 (OVFCC_DYNQUANT_I8 taking effect), is
- * OVFCC_EUNSUPPORTED.  All requests of a GPU share that GPU's array: calls of this entry point that overlap in time
- * on one GPU race; serialise them (one stream, or events between streams). */
+ * OVFCC_EUNSUPPORTED.  All requests of a GPU share that GPU's array.  The library orders the launches that use it:
+ * each waits, on its own stream, for an event recorded behind the one before it (the event is created by
+ * ovfcc_init, not here), so calls from different requests and host threads are safe and simply do not overlap.  The
+ * exception is a stream under graph capture, which cannot wait for an event from outside its capture: replays of
+ * graphs that hold such launches, and anything else that uses the array at the same time, are the caller's to keep
+ * apart. */
 int ovfcc_fc_run_device_static(ovfcc_request* req, const ovfcc_weights* w, const void* x_dev, void* y_dev, int64_t M);
 
 /* Several independent nodes of one shape and weight format in one launch: the experts of a
@@ -297,7 +301,9 @@ int ovfcc_gather_matmul_device(ovfcc_request* req, const ovfcc_weights* const* e
  * bucketed per expert by a kernel on the request's stream (one workgroup per expert; the reference's GPU plugin builds
  * its expert masks on the device as well, src/plugins/intel_gpu/src/graph/impls/ocl_v2/moe_mask_gen.cl), the grouped
  * launch reads its slice table from device memory, and the call neither waits for the stream nor depends on the row
- * counts.  An index outside [0, n_experts) selects nothing: its row of Y is left untouched.  Needs tiled 4-bit
+ * counts.  Indices in device memory cannot be checked without waiting for them, so where the host-index form
+ * returns OVFCC_EINVAL this one goes on: an index outside [0, n_experts) selects nothing and its row Y[i, m, :] is
+ * written as zeros; every other row is what it would be without that pair.  Needs tiled 4-bit
  * experts with N % 256 == 0 and one scalar zero-point (what the grouped prefill kernel runs) and at most 64 experts;
  * otherwise OVFCC_EUNSUPPORTED.  ovfcc_gather_matmul_device takes this path itself wherever it fits, after copying
  * its indices to the device (OVFCC_MOE_HOST_ROUTING=1 in the environment keeps the bucketing on the host). */
@@ -323,8 +329,9 @@ int ovfcc_moe_device(ovfcc_request* req, const ovfcc_weights* const* gate_up, co
                      int top_k, void* y_dev);
 
 /* ovfcc_moe_device with indices_dev [M, top_k] int32 in device memory (see ovfcc_gather_matmul_routed_device): the
- * routing kernel runs once per projection, nothing in the call waits for the stream.  A pair whose index lies outside
- * [0, n_experts) contributes nothing to its row's sum. */
+ * routing kernel runs once per projection, nothing in the call waits for the stream.  Where ovfcc_moe_device returns
+ * OVFCC_EINVAL for an index outside [0, n_experts), this form cannot look: such a pair contributes nothing to its
+ * row's sum (a row whose pairs all name no expert is written as zeros), every other row is unaffected. */
 int ovfcc_moe_routed_device(ovfcc_request* req, const ovfcc_weights* const* gate_up, const ovfcc_weights* const* down,
                             int n_experts, const void* x_dev, const void* routing_dev, const int32_t* indices_dev,
                             int64_t M, int top_k, void* y_dev);
@@ -343,6 +350,9 @@ int ovfcc_last_kernel_info(const ovfcc_request* req, ovfcc_kernel_info* info);
 
 /* ---- device memory helpers (plain pointers; for hosts that do not link HIP themselves) ------ */
 int ovfcc_device_malloc(ovfcc_ctx* ctx, size_t bytes, void** out);
+/* Free and total memory of the context's device in bytes: the figures behind ov::intel_gpu::device_total_mem_size
+ * and ov::intel_gpu::memory_statistics (src/inference/include/openvino/runtime/intel_gpu/properties.hpp:33, :64). */
+int ovfcc_device_mem_info(ovfcc_ctx* ctx, size_t* free_bytes, size_t* total_bytes);
 int ovfcc_device_free(ovfcc_ctx* ctx, void* ptr);
 int ovfcc_memcpy_h2d(ovfcc_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
 int ovfcc_memcpy_d2h(ovfcc_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);

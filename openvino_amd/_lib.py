@@ -26,7 +26,7 @@ BENCH_SYMBOLS = ["ovfcc_bench_layers", "ovfcc_bench_grouped", "ovfcc_bench_copy"
 
 # every symbol include/ovfcc.h and include/ovfcc_graph.h declare (libovfcc.so)
 SYMBOLS = [
-    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_glu", "ovfcc_weights_mlp", "ovfcc_weights_export_size", "ovfcc_weights_export", "ovfcc_weights_import", "ovfcc_weights_destroy",
+    "ovfcc_init", "ovfcc_destroy", "ovfcc_device_count", "ovfcc_device_mem_info", "ovfcc_weights_create", "ovfcc_weights_clone", "ovfcc_weights_concat", "ovfcc_weights_glu", "ovfcc_weights_mlp", "ovfcc_weights_export_size", "ovfcc_weights_export", "ovfcc_weights_import", "ovfcc_weights_destroy",
     "ovfcc_weights_device_bytes", "ovfcc_weights_is_tiled", "ovfcc_request_create", "ovfcc_request_destroy",
     "ovfcc_fc_run", "ovfcc_fc_run_device", "ovfcc_fc_run_device_static", "ovfcc_fc_run_grouped_device", "ovfcc_grouped_matmul_device", "ovfcc_grouped_matmul_offsets_device", "ovfcc_gather_matmul_device", "ovfcc_gather_matmul_routed_device", "ovfcc_moe_device", "ovfcc_moe_routed_device", "ovfcc_request_sync", "ovfcc_request_force_kernel",
     "ovfcc_last_kernel_info", "ovfcc_device_malloc", "ovfcc_device_free",
@@ -168,6 +168,7 @@ def load() -> ctypes.CDLL:
         "ovfcc_last_kernel_info": (ci, [vp, ctypes.POINTER(KernelInfo)]),
         "ovfcc_bench_layers": (ci, [vp, pp, ci, vp, vp, i64, ci, ci, ci, ctypes.POINTER(ctypes.c_float)]),
         "ovfcc_device_malloc": (ci, [vp, sz, pp]),
+        "ovfcc_device_mem_info": (ci, [vp, ctypes.POINTER(sz), ctypes.POINTER(sz)]),
         "ovfcc_device_free": (ci, [vp, vp]),
         "ovfcc_memcpy_h2d": (ci, [vp, vp, vp, sz]),
         "ovfcc_memcpy_d2h": (ci, [vp, vp, vp, sz]),

@@ -67,6 +67,22 @@ int ensure_split_buffers(ovfcc_request* r, const ovfcc::LaunchPlan& plan) {
     return OVFCC_OK;
 }
 
+// The fixed scratch array of ovfcc_fc_run_device_static is one per device, shared by every context and request on
+// it: a launch that uses it waits, on its stream, for the event recorded behind the last such launch.  The event is
+// created by the first ovfcc_init on the device and lives as long as the array, so that the entry point itself
+// creates nothing.
+struct StaticGuard {
+    std::mutex mu;
+    hipEvent_t done = nullptr;
+    bool recorded = false;
+};
+constexpr int kGuardedDevices = 64;
+StaticGuard g_static_guard[kGuardedDevices];
+
+StaticGuard* static_guard(int device) {
+    return device >= 0 && device < kGuardedDevices ? &g_static_guard[device] : nullptr;
+}
+
 // Split-K workspace and arrival counters for one launch: the request's own buffers (grown on demand), or -- for
 // the entry point that allocates nothing -- the device's fixed scratch array, whose counters are cleared by a fill
 // kernel ahead of the launch (the array keeps whatever the last call left, on this or any other request).
@@ -93,9 +109,38 @@ int split_buffers(ovfcc_request* r, const ovfcc::LaunchPlan& plan, bool static_s
         return fail(OVFCC_EDEVICE, "the fixed scratch array was not set up on this device");
     a->counters = reinterpret_cast<unsigned*>(base);
     a->workspace = reinterpret_cast<float*>(base + ovfcc::kStaticCounterBytes);
+    // every request of the device shares the array: order this launch behind the last one that used it, whichever
+    // stream that ran on.  (A capturing stream cannot wait for an event from outside its capture; a caller that
+    // captures keeps such launches of different requests apart itself.)
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    HIP_TRY(hipStreamIsCapturing(r->stream, &cap));
+    StaticGuard* g = static_guard(r->ctx->device);
+    if (cap == hipStreamCaptureStatusNone && g && g->done) {
+        std::lock_guard<std::mutex> lock(g->mu);
+        if (g->recorded)
+            HIP_TRY(hipStreamWaitEvent(r->stream, g->done, 0));
+    }
     int e = ovfcc::launch_zero_u32(a->counters, plan.counter_count, r->stream);
     if (e)
         return hip_fail((hipError_t)e, "counter fill launch");
+    return OVFCC_OK;
+}
+
+// Behind a launch that used the fixed scratch array: the point the next such launch waits for.
+int static_scratch_released(ovfcc_request* r, const ovfcc::FcDeviceArgs& a) {
+    unsigned char* base = static_cast<unsigned char*>(ovfcc::static_scratch_ptr(r->ctx->device));
+    if (!base || reinterpret_cast<unsigned char*>(a.counters) != base)
+        return OVFCC_OK;  // the launch did not split K: nothing of the array was used
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    HIP_TRY(hipStreamIsCapturing(r->stream, &cap));
+    if (cap != hipStreamCaptureStatusNone)
+        return OVFCC_OK;
+    StaticGuard* g = static_guard(r->ctx->device);
+    if (!g || !g->done)
+        return OVFCC_OK;
+    std::lock_guard<std::mutex> lock(g->mu);
+    HIP_TRY(hipEventRecord(g->done, r->stream));
+    g->recorded = true;
     return OVFCC_OK;
 }
 
@@ -414,6 +459,8 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
             int e = ovfcc::launch_fc(a, p, r->stream);
             if (e)
                 return hip_fail((hipError_t)e, "kernel launch");
+            if (static_scratch && (rc = static_scratch_released(r, a)))
+                return rc;
             record(r, p);
         }
         return OVFCC_OK;
@@ -428,6 +475,8 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
     int e = ovfcc::launch_fc(a, p, r->stream);
     if (e)
         return hip_fail((hipError_t)e, "kernel launch");
+    if (static_scratch && (rc = static_scratch_released(r, a)))
+        return rc;
     record(r, p);
     return OVFCC_OK;
 }
@@ -483,7 +532,7 @@ bool plan_routed(ovfcc_request* r, const ovfcc_weights* w0, int64_t R, int n_exp
 int run_routed(ovfcc_request* r, const ovfcc_weights* const* experts, int n_experts, RoutedLaunch& L,
                const int* indices_dev, int64_t M, int top_k, int a_batches, int inverse, int x_mapped, const void* x_base,
                size_t x_row_bytes, void* y_base, size_t y_row_bytes, int* d_maps, ovfcc::RoutedHeader* d_header,
-               const ovfcc::SecondTable* second_table = nullptr) {
+               const ovfcc::SecondTable* second_table = nullptr, void* unrouted_y = nullptr) {
     auto* d_table = reinterpret_cast<ovfcc::BatchGroupItem*>(d_header + 1);
     ovfcc::ExpertPointers ptrs{};
     for (int e = 0; e < n_experts; ++e)
@@ -495,7 +544,7 @@ int run_routed(ovfcc_request* r, const ovfcc_weights* const* experts, int n_expe
     int e1 = ovfcc::launch_moe_route(indices_dev, M, top_k, n_experts, a_batches, inverse, L.cap, x_mapped, ptrs, x_base,
                                      x_row_bytes, y_base, y_row_bytes, d_maps, d_maps + R, d_table, L.n_slices, d_header,
                                      L.plan.tiles_x, (int)experts[0]->layout.k_blocks, L.plan.n_cus, r->stream,
-                                     second_table);
+                                     second_table, unrouted_y, y_row_bytes);
     if (e1)
         return hip_fail((hipError_t)e1, "routing kernel launch");
     return OVFCC_OK;
@@ -590,7 +639,7 @@ int gather_matmul_routed(ovfcc_request* r, const ovfcc_weights* const* experts, 
     }
     // (the grouped launch reads the rows of A through the map: no gathered copy)
     rc = run_routed(r, experts, n_experts, L, indices_dev, M, top_k, a_batches, 0, 1, a_dev, (size_t)K * 2, base + y_off,
-                    (size_t)N_out * out_bytes, d_maps, d_table);
+                    (size_t)N_out * out_bytes, d_maps, d_table, nullptr, y_dev);
     if (rc)
         return rc;
     rc = launch_routed(r, L, d_table);
@@ -790,6 +839,11 @@ int ovfcc_init(int device, ovfcc_ctx** out) {
     // the fixed scratch array of ovfcc_fc_run_device_static: its address on this device, looked up once
     if (int se = ovfcc::static_scratch_setup(device))
         return hip_fail((hipError_t)se, "hipGetSymbolAddress of the fixed scratch array");
+    if (StaticGuard* g = static_guard(device)) {
+        std::lock_guard<std::mutex> lock(g->mu);
+        if (!g->done)
+            HIP_TRY(hipEventCreateWithFlags(&g->done, hipEventDisableTiming));
+    }
     ovfcc_ctx* c = new ovfcc_ctx();
     c->device = device;
     c->n_cus = prop.multiProcessorCount;
@@ -802,6 +856,14 @@ void ovfcc_destroy(ovfcc_ctx* ctx) {
     if (ctx && ctx->coop_done)
         (void)hipEventDestroy(ctx->coop_done);
     delete ctx;
+}
+
+int ovfcc_device_mem_info(ovfcc_ctx* ctx, size_t* free_bytes, size_t* total_bytes) {
+    if (!ctx || !free_bytes || !total_bytes)
+        return fail(OVFCC_EINVAL, "null argument");
+    HIP_TRY(hipSetDevice(ctx->device));
+    HIP_TRY(hipMemGetInfo(free_bytes, total_bytes));
+    return OVFCC_OK;
 }
 
 int ovfcc_weights_create(ovfcc_ctx* ctx, const ovfcc_fc_desc* desc, const void* w, const void* scales, const void* zp,

@@ -154,7 +154,8 @@ __global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restric
                                                             int* __restrict__ first, int* __restrict__ second,
                                                             BatchGroupItem* __restrict__ table, int n_slices_max,
                                                             RoutedHeader* __restrict__ header, int tiles_x,
-                                                            int kb_total, int n_cus, SecondTable t2) {
+                                                            int kb_total, int n_cus, SecondTable t2,
+                                                            char* unrouted_y, size_t unrouted_row_bytes) {
     __shared__ int hist[kMaxGroupItems];
     __shared__ int wave_total[4];
     __shared__ int start_s, slice_s, total_slices_s, total_pairs_s;
@@ -165,10 +166,19 @@ __global__ __launch_bounds__(256) void fcc_moe_route_kernel(const int* __restric
     __syncthreads();
     for (int j = tid; j < R; j += 256) {
         const int v = indices[j];
-        if (v >= 0 && v < n_experts)
+        if (v >= 0 && v < n_experts) {
             atomicAdd(&hist[v], 1);
-        else if (e == 0 && inverse)
-            second[j] = -1;
+        } else if (e == 0) {
+            if (inverse)
+                second[j] = -1;
+            if (unrouted_y) {
+                // no expert computes this pair's row of the result [top_k, M, .]: it reads as zeros
+                const int m = j / top_k, i = j - m * top_k;
+                uint4_t* row = reinterpret_cast<uint4_t*>(unrouted_y + (size_t)(i * M + m) * unrouted_row_bytes);
+                for (size_t c = 0; c < unrouted_row_bytes / 16; ++c)
+                    row[c] = uint4_t{0u, 0u, 0u, 0u};
+            }
+        }
     }
     __syncthreads();
     if (tid == 0) {
@@ -254,8 +264,10 @@ int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts
                      int x_mapped, const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
                      size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
                      RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream,
-                     const SecondTable* second_table) {
+                     const SecondTable* second_table, void* unrouted_y, size_t unrouted_row_bytes) {
     const int64_t R = M * top_k;
+    if (unrouted_y && (unrouted_row_bytes == 0 || (unrouted_row_bytes & 15)))
+        return (int)hipErrorInvalidValue;
     SecondTable t2{};
     if (second_table) {
         t2 = *second_table;
@@ -269,7 +281,8 @@ int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts
     hipLaunchKernelGGL(fcc_moe_route_kernel, dim3((unsigned)n_experts), dim3(256), 0, static_cast<hipStream_t>(stream),
                        indices_dev, (int)R, (int)M, top_k, n_experts, a_batches, inverse, cap, x_mapped, experts,
                        static_cast<const char*>(x_base), x_row_bytes, static_cast<char*>(y_base), y_row_bytes, first,
-                       second, table, n_slices_max, header, tiles_x, kb_total, n_cus, t2);
+                       second, table, n_slices_max, header, tiles_x, kb_total, n_cus, t2, static_cast<char*>(unrouted_y),
+                       unrouted_row_bytes);
     return (int)hipGetLastError();
 }
 

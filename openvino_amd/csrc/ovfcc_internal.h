@@ -292,13 +292,15 @@ struct SecondTable {
     RoutedHeader* header;
     int tiles_x, kb_total;
 };
+// unrouted_y: the final result [top_k, M, row] of a GatherMatmul; the rows of pairs whose index names no expert are
+// zeroed there (no bucket owns them, so nothing else writes them).
 // x_mapped != 0: the slices leave the gather to the grouped launch -- every entry gets x = x_base and reserved = its
 // first bucket slot, and the launch reads its rows through `first`.
 int launch_moe_route(const int* indices_dev, int64_t M, int top_k, int n_experts, int a_batches, int inverse, int cap,
                      int x_mapped, const ExpertPointers& experts, const void* x_base, size_t x_row_bytes, void* y_base,
                      size_t y_row_bytes, int* first, int* second, BatchGroupItem* table, int n_slices_max,
                      RoutedHeader* header, int tiles_x, int kb_total, int n_cus, void* stream,
-                     const SecondTable* second_table = nullptr);
+                     const SecondTable* second_table = nullptr, void* unrouted_y = nullptr, size_t unrouted_row_bytes = 0);
 // GroupedMatMul with offsets in device memory: table[0 .. n_slices_max) and *header as for launch_moe_route, from
 // cumulative row ends over rows that are already contiguous per group; rows of y from the last offset on are
 // zeroed; tail: one int of scratch.

@@ -59,6 +59,12 @@ class Device:
             self.lib.ovfcc_destroy(self.handle)
             self.handle = None
 
+    def mem_info(self):
+        """(free, total) bytes of device memory"""
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        check(self.lib.ovfcc_device_mem_info(self.handle, ctypes.byref(free), ctypes.byref(total)))
+        return free.value, total.value
+
     # raw device buffers
     def malloc(self, nbytes: int) -> int:
         p = ctypes.c_void_p()

@@ -637,7 +637,7 @@ def test_gather_matmul(oracle, dev, req, monkeypatch, M, a_batches):
 def test_gather_matmul_routed_on_the_device(oracle, dev, req, monkeypatch, M, a_batches):
     """GatherMatmulCompressed with the indices in device memory: bucketed by the routing kernel.  Every output row
     against the oracle and, where the host-bucketed call runs the same grouped kernel, bit for bit against it; a
-    pair whose index names no expert leaves its row of Y as it was."""
+    pair whose index names no expert gets a row of zeros in Y."""
     say(f"gather matmul routed M={M} a_batches={a_batches}")
     E, top_k, K, N = 8, 2, 512, 256
     cases = [datagen.make_case(860 + e, 1, K, N, "u4", 128, "u4", with_bias=True) for e in range(E)]
@@ -654,7 +654,8 @@ def test_gather_matmul_routed_on_the_device(oracle, dev, req, monkeypatch, M, a_
         bad = indices.copy()
         bad[0, 0], bad[M - 1, 1] = E, -3
         got = req.gather_matmul(ws, A, bad, device_indices=True, y_fill=7.0)
-        assert np.all(got[0, 0] == 7.0) and np.all(got[1, M - 1] == 7.0)
+        # the two unrouted pairs' rows read as zeros (not as whatever Y held), every other row is unchanged
+        assert np.all(got[0, 0].view(np.uint16) == 0) and np.all(got[1, M - 1].view(np.uint16) == 0)
         got[0, 0], got[1, M - 1] = y[0, 0], y[1, M - 1]
         assert np.array_equal(got.view(np.uint16), y.view(np.uint16))
         monkeypatch.setenv("OVFCC_MOE_HOST_ROUTING", "1")

@@ -80,6 +80,48 @@ def test_static_entry_point_matches_on_split_k_launches(oracle, dev):
         other.close()
 
 
+def test_static_entry_point_allocates_nothing_and_orders_its_streams(dev):
+    """Free device memory reads the same before and after calls of the static entry point that split K (the
+    allocating entry point, on a fresh request, does take memory for its partial tiles: the check can see an
+    allocation).  And two requests -- two streams -- that call it back to back without waiting for each other share
+    the one scratch array safely: each launch waits for the one before it, so every result equals the allocating
+    entry point's."""
+    c = datagen.make_case(9103, 512, 4096, 1024, "i4", 128, "none")
+    w = fc.CompressedWeights.from_case(dev, c)
+    M = 512
+    n_bytes = M * c.N * 2
+    x_ptr = dev.malloc(c.x.nbytes)
+    ys = [dev.malloc(n_bytes) for _ in range(9)]
+    a, b = fc.InferRequest(dev), fc.InferRequest(dev)
+    try:
+        dev.upload(x_ptr, np.ascontiguousarray(c.x))
+        a.infer_device_static(w, x_ptr, ys[0], M)   # first use: whatever the runtime sets up lazily is in place
+        a.sync()
+        assert a.last_kernel()["split_k"] > 1
+        free0 = dev.mem_info()[0]
+        for i in range(4):
+            a.infer_device_static(w, x_ptr, ys[2 * i], M)
+            b.infer_device_static(w, x_ptr, ys[2 * i + 1], M)
+        a.sync()
+        b.sync()
+        assert dev.mem_info()[0] == free0, "the static entry point changed the free device memory"
+        fresh = fc.InferRequest(dev)
+        fresh.infer_device(w, x_ptr, ys[8], M)
+        fresh.sync()
+        assert dev.mem_info()[0] < free0, "an allocation of partial tiles should show in the free memory"
+        want = dev.download(ys[8], (M, c.N), np.uint16)
+        for i in range(8):
+            assert np.array_equal(dev.download(ys[i], (M, c.N), np.uint16), want), f"call {i}"
+        fresh.close()
+    finally:
+        a.close()
+        b.close()
+        w.close()
+        dev.free(x_ptr)
+        for p_ in ys:
+            dev.free(p_)
+
+
 def test_static_entry_point_refuses_what_does_not_fit(dev):
     """Partial tiles beyond 32 MiB: a clear error instead of an allocation; M = 0 is fine."""
     req = fc.InferRequest(dev)
