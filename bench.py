@@ -447,7 +447,7 @@ def main() -> int:
     ap.add_argument("--floors", action="store_true",
                     help="measure what bounds a decode node from below -- an empty graph node, a loads-only streaming "
                          "kernel over the node's weight bytes -- beside the node's own time, and print a markdown table")
-    ap.add_argument("--profile", choices=["decode", "batch", "prefill", "w8a8", "w4a8", "moe"], default=None,
+    ap.add_argument("--profile", choices=["decode", "decode-graph", "batch", "prefill", "w8a8", "w4a8", "moe"], default=None,
                     help="short run for rocprofv3: one copy-kernel launch of known size (the counter yardstick), "
                          "then a few eager passes of the chosen kernel family; prints no JSON")
     ap.add_argument("--profile-rows", type=int, default=32,
@@ -528,6 +528,10 @@ def main() -> int:
                     w.close()
                     dev.free(xq_dev)
                     dev.free(yq_dev)
+        elif args.profile == "decode-graph":
+            # the headline pass as the benchmark runs it: all nodes captured into one HIP graph, replayed four times
+            # (one capture and one instantiation in the whole process)
+            req.bench_layers([w for _, w in layers], x_dev, y_dev, 1, 1, 3, use_graph=True)
         elif args.profile in ("decode", "batch"):
             rows = 1 if args.profile == "decode" else min(32, max(2, args.profile_rows))
             for _ in range(3):

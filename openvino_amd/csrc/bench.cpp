@@ -28,11 +28,13 @@ int hip_fail(hipError_t e, const char* what) {
 // HIP objects of one benchmark call, released on every way out of it
 struct Held {
     hipStream_t stream = nullptr;
+    hipStream_t borrowed = nullptr;  // a stream of the caller's that may still run the graph: drained before the release
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     hipEvent_t t0 = nullptr, t1 = nullptr;
     void* mem = nullptr;
     ~Held() {
+        if (borrowed && (exec || graph)) (void)hipStreamSynchronize(borrowed);
         if (t0) (void)hipEventDestroy(t0);
         if (t1) (void)hipEventDestroy(t1);
         if (exec) (void)hipGraphExecDestroy(exec);
@@ -60,6 +62,7 @@ int ovfcc_bench_layers(ovfcc_request* r, const ovfcc_weights* const* layers, int
     HIP_TRY(hipStreamSynchronize(r->stream));
 
     Held h;  // graph, executable graph and events: released on every way out, error paths included
+    h.borrowed = r->stream;
     if (use_graph) {
         HIP_TRY(hipStreamBeginCapture(r->stream, hipStreamCaptureModeThreadLocal));
         int rc = OVFCC_OK;
