@@ -423,6 +423,21 @@ def floors_table(dev, req, args) -> int:
             tf = max(dev.mfma_ceiling(waves, valu, shape=shape) for _ in range(2))
             print(f"| {name}, {waves // 4} wave(s) per SIMD, {valu} packed-f16 multiplications per 16 x 16 x 32 of "
                   f"matrix work | {tf:.0f} | {100 * tf / 2500:.1f} % |")
+    # how one SIMD overlaps matrix-core and vector instructions, in shader cycles: one compute unit alone, then all
+    n_cus = 256
+    print("\n| matrix-core loop with vector instructions after every MFMA (v_mfma_f32_16x16x32_f16, two waves per SIMD) | "
+          "one compute unit: cycles, ns per MFMA and SIMD | all compute units: cycles, ns |")
+    print("|---|---|---|")
+    for mode, valu, what in ((0, 0, "no vector instruction"), (0, 2, "2 independent packed-f16 multiplications"),
+                             (0, 3, "3 independent"), (0, 4, "4 independent"), (0, 6, "6 independent"),
+                             (1, 3, "3 in one dependent chain"),
+                             (2, 3, "3, the first writes a register of the B operand just read"),
+                             (3, 3, "3 independent, MFMA destination is not its accumulator input")):
+        one = dev.issue_probe(1, 8, mode, valu)
+        all_ = dev.issue_probe(n_cus, 8, mode, valu)
+        print(f"| {what} | {one[0]:.1f}, {one[1]:.2f} | {all_[0]:.1f}, {all_[1]:.2f} |")
+    one = dev.issue_probe(1, 4, 0, 0)
+    print(f"| no vector instruction, one wave per SIMD | {one[0]:.1f}, {one[1]:.2f} | |")
     for ptr in (arena, x_dev, y_dev):
         dev.free(ptr)
     req.close()

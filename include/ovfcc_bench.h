@@ -47,6 +47,16 @@ int ovfcc_bench_floor(ovfcc_ctx* ctx, const void* arena_dev, size_t arena_bytes,
  * its clock) is the ceiling the prefill kernels are measured against beside the nominal peak. */
 int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int shape, int rounds, float* elapsed_ms, double* flops);
 
+/* How one SIMD overlaps matrix-core and vector instructions: `workgroups` workgroups (1: one compute unit alone, no
+ * power limit; the number of compute units: the whole chip) of `waves` waves (4 or 8) run the loop of
+ * ovfcc_bench_mfma with `valu` vector instructions after every v_mfma_f32_16x16x32_f16, arranged by `mode` -- 0:
+ * independent packed-f16 multiplications (valu 0, 2, 3, 4 or 6); 1: one dependent chain (valu 3); 2: the first one
+ * writes a register of the B operand the MFMA has just read (valu 3); 3: as 0 with MFMAs whose destination is not
+ * their accumulator input (valu 3).  Measured inside the kernel: *cycles_per_mfma = shader-clock ticks per MFMA and
+ * SIMD, *ns_per_mfma = the same from the 100 MHz wall clock (their ratio is the clock the loop ran at). */
+int ovfcc_bench_issue(ovfcc_ctx* ctx, int workgroups, int waves, int mode, int valu, int rounds, double* cycles_per_mfma,
+                      double* ns_per_mfma);
+
 #ifdef __cplusplus
 }
 #endif

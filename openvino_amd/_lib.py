@@ -22,7 +22,7 @@ W_INPUT_MAJOR = 16
 DYNQUANT_PER_GROUP = 32                                                # OVFCC_DYNQUANT_PER_GROUP                                                     # OVFCC_W_INPUT_MAJOR
 
 # every symbol include/ovfcc_bench.h declares (libovfcc_bench.so)
-BENCH_SYMBOLS = ["ovfcc_bench_layers", "ovfcc_bench_grouped", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_bench_mfma"]
+BENCH_SYMBOLS = ["ovfcc_bench_layers", "ovfcc_bench_grouped", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_bench_mfma", "ovfcc_bench_issue"]
 
 # every symbol include/ovfcc.h and include/ovfcc_graph.h declare (libovfcc.so)
 SYMBOLS = [
@@ -176,6 +176,7 @@ def load() -> ctypes.CDLL:
         "ovfcc_bench_copy": (ci, [vp, vp, vp, sz, ci, ctypes.POINTER(ctypes.c_float)]),
         "ovfcc_bench_floor": (ci, [vp, vp, sz, sz, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_float)]),
         "ovfcc_bench_mfma": (ci, [vp, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]),
+        "ovfcc_bench_issue": (ci, [vp, ci, ci, ci, ci, ci, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
         "ovfcc_desc_validate": (ci, [ctypes.POINTER(FcDesc)]),
         "ovfcc_env_reload": (None, []),
         "ovfcc_tiled_sizes": (ci, [ctypes.POINTER(FcDesc), ctypes.POINTER(sz), ctypes.POINTER(sz), ctypes.POINTER(sz)]),

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <string>
+#include <vector>
 
 #include "api_types.h"
 #include "bench_probe.h"
@@ -173,6 +174,35 @@ int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int shape, int rounds,
     if (e)
         return hip_fail((hipError_t)e, "matrix-core probe launch");
     *flops = 2.0 * 16 * 16 * 32 * 8.0 * rounds * waves * workgroups;  // either shape: 2^17 multiply-adds per round
+    return OVFCC_OK;
+}
+
+int ovfcc_bench_issue(ovfcc_ctx* ctx, int workgroups, int waves, int mode, int valu, int rounds, double* cycles_per_mfma,
+                      double* ns_per_mfma) {
+    if (!ctx || !cycles_per_mfma || !ns_per_mfma || rounds <= 0 || workgroups < 1 || workgroups > 4096 ||
+        (waves != 4 && waves != 8))
+        return fail(OVFCC_EINVAL, "bad issue benchmark arguments");
+    HIP_TRY(hipSetDevice(ctx->device));
+    Held h;
+    HIP_TRY(hipStreamCreateWithFlags(&h.stream, hipStreamNonBlocking));
+    const size_t sink_bytes = (size_t)workgroups * 64 * waves * sizeof(float);
+    HIP_TRY(hipMalloc(&h.mem, sink_bytes + (size_t)workgroups * 2 * sizeof(long long)));
+    float* sink = static_cast<float*>(h.mem);
+    long long* ticks = reinterpret_cast<long long*>(static_cast<char*>(h.mem) + sink_bytes);
+    int e = ovfcc::launch_issue_probe(sink, ticks, workgroups, waves, mode, valu, 64, h.stream);  // warm-up
+    if (!e)
+        e = ovfcc::launch_issue_probe(sink, ticks, workgroups, waves, mode, valu, rounds, h.stream);
+    if (e)
+        return hip_fail((hipError_t)e, "issue probe launch (mode and vector instruction count must be a built pair)");
+    HIP_TRY(hipStreamSynchronize(h.stream));
+    std::vector<long long> host((size_t)workgroups * 2);
+    HIP_TRY(hipMemcpy(host.data(), ticks, host.size() * sizeof(long long), hipMemcpyDeviceToHost));
+    double shader = 0.0, wall = 0.0;
+    for (int g = 0; g < workgroups; ++g)
+        shader += (double)host[2 * (size_t)g], wall += (double)host[2 * (size_t)g + 1];
+    const double mfmas_per_simd = 8.0 * rounds * (waves / 4);
+    *cycles_per_mfma = shader / workgroups / mfmas_per_simd;
+    *ns_per_mfma = wall / workgroups * 10.0 / mfmas_per_simd;  // the wall clock counts at 100 MHz
     return OVFCC_OK;
 }
 

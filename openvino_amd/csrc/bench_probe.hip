@@ -178,6 +178,80 @@ int launch_mfma_probe(float* sink, int workgroups, int waves, int valu, int shap
     return (int)hipGetLastError();
 }
 
+// How one SIMD overlaps matrix-core and vector instructions, in shader cycles: the loop of fcc_mfma_probe_kernel with
+// the vector instructions after each MFMA arranged by MODE -- 0: independent packed-f16 multiplications; 1: one
+// dependent chain of them; 2: the first one writes a register of the B operand that the MFMA has just read; 3: as 0,
+// with MFMAs whose destination is the next accumulator slot instead of their own input (what the compiler emits where
+// it is free to).  Lane 0 of every workgroup leaves its tick counts (shader clock, 100 MHz wall clock) in ticks[].
+template <int MODE, int VALU>
+__global__ __launch_bounds__(512) void fcc_issue_probe_kernel(float* __restrict__ sink, long long* __restrict__ ticks,
+                                                              int iters) {
+    half8_t a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        a[i] = probe_operand(threadIdx.x * 8u + i), b[i] = probe_operand(threadIdx.x * 8u + 4u + i);
+    float4_t acc[8];
+    uint32_t r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        acc[i] = float4_t{0.f, 0.f, 0.f, 0.f}, r[i] = 0x3c003c00u + (uint32_t)i;
+    const uint32_t c = 0x3c003c00u, m = 0x000f000fu;
+    __syncthreads();
+    const long long t0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if constexpr (MODE == 3)
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %2, %3, %1"
+                             : "=&v"(acc[(j + 1) & 7])
+                             : "v"(acc[j]), "v"(a[j & 3]), "v"(b[(j >> 1) & 3]));
+            else
+                asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a[j & 3]), "v"(b[(j >> 1) & 3]));
+#pragma unroll
+            for (int v = 0; v < VALU; ++v) {
+                if constexpr (MODE == 1)
+                    asm volatile("v_pk_mul_f16 %0, %0, %1" : "+v"(r[j & 7]) : "v"(c));
+                else if (MODE == 2 && v == 0)
+                    asm volatile("v_and_or_b32 %0, %0, %1, %2"
+                                 : "+v"(reinterpret_cast<uint32_t*>(&b[(j >> 1) & 3])[0])
+                                 : "v"(m), "v"(c));
+                else
+                    asm volatile("v_pk_mul_f16 %0, %0, %1" : "+v"(r[(j + v) & 7]) : "v"(c));
+            }
+        }
+    }
+    const long long t1 = clock64(), w1 = wall_clock64();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        s += acc[i].x + acc[i].y + acc[i].z + acc[i].w + (float)r[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        s += (float)b[i][0];
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
+    if (threadIdx.x == 0)
+        ticks[2 * blockIdx.x] = t1 - t0, ticks[2 * blockIdx.x + 1] = w1 - w0;
+}
+
+int launch_issue_probe(float* sink, long long* ticks, int workgroups, int waves, int mode, int valu, int iters, void* stream) {
+    if (!sink || !ticks || workgroups < 1 || (waves != 4 && waves != 8) || iters < 1)
+        return (int)hipErrorInvalidValue;
+    const dim3 g((unsigned)workgroups), b(64u * waves);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define OVFCC_ISSUE(MODE, VALU) hipLaunchKernelGGL((fcc_issue_probe_kernel<MODE, VALU>), g, b, 0, s, sink, ticks, iters)
+    if (mode == 0 && valu == 0) OVFCC_ISSUE(0, 0);
+    else if (mode == 0 && valu == 2) OVFCC_ISSUE(0, 2);
+    else if (mode == 0 && valu == 3) OVFCC_ISSUE(0, 3);
+    else if (mode == 0 && valu == 4) OVFCC_ISSUE(0, 4);
+    else if (mode == 0 && valu == 6) OVFCC_ISSUE(0, 6);
+    else if (mode == 1 && valu == 3) OVFCC_ISSUE(1, 3);
+    else if (mode == 2 && valu == 3) OVFCC_ISSUE(2, 3);
+    else if (mode == 3 && valu == 3) OVFCC_ISSUE(3, 3);
+    else return (int)hipErrorInvalidValue;
+#undef OVFCC_ISSUE
+    return (int)hipGetLastError();
+}
+
 int launch_empty(unsigned* out, void* stream) {
     hipLaunchKernelGGL(fcc_empty_kernel, dim3(256), dim3(256), 0, static_cast<hipStream_t>(stream), out);
     return (int)hipGetLastError();

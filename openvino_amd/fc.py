@@ -104,6 +104,13 @@ class Device:
         check(self.lib.ovfcc_bench_mfma(self.handle, waves, valu, shape, rounds, ctypes.byref(ms), ctypes.byref(flops)))
         return flops.value / (ms.value * 1e-3) / 1e12
 
+    def issue_probe(self, workgroups: int, waves: int, mode: int, valu: int, rounds: int = 20000):
+        """(shader cycles, ns) per MFMA and SIMD of the matrix-core loop with `valu` vector instructions after every
+        MFMA arranged by `mode` (ovfcc_bench_issue)."""
+        cyc, ns = ctypes.c_double(), ctypes.c_double()
+        check(self.lib.ovfcc_bench_issue(self.handle, workgroups, waves, mode, valu, rounds, ctypes.byref(cyc), ctypes.byref(ns)))
+        return cyc.value, ns.value
+
     def copy_bandwidth(self, nbytes: int = 1 << 30, iters: int = 10) -> float:
         """GB/s (read + write) of the plain copy kernel."""
         src, dst = self.malloc(nbytes), self.malloc(nbytes)
