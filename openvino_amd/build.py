@@ -11,7 +11,7 @@ ROOT = os.path.dirname(PKG)
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libovfcc.so")
 BENCH_LIB = os.path.join(PKG, "libovfcc_bench.so")
-SOURCES = ["api.cpp", "repack.cpp", "plan.cpp", "fold.cpp", "fold_data.cpp", "kernel_plain.hip", "scratch.hip", "kernel_decode.hip", "kernel_gemv.hip", "kernel_gemv16.hip", "kernel_mlp.hip", "kernel_batch.hip", "kernel_prefill.hip", "kernel_prefill_direct.hip", "kernel_prefill_async.hip", "kernel_prefill_big.hip",
+SOURCES = ["api.cpp", "repack.cpp", "plan.cpp", "fold.cpp", "fold_data.cpp", "kernel_plain.hip", "scratch.hip", "kernel_decode.hip", "kernel_gemv.hip", "kernel_gemv16.hip", "kernel_gemv16s.hip", "kernel_mlp.hip", "kernel_batch.hip", "kernel_prefill.hip", "kernel_prefill_direct.hip", "kernel_prefill_async.hip", "kernel_prefill_big.hip",
            "kernel_prefill_wide.hip", "kernel_prefill_i8.hip", "kernel_prefill_i8w4.hip"]
 BENCH_SOURCES = ["bench.cpp", "bench_probe.hip"]
 

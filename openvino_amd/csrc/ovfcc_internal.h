@@ -156,6 +156,7 @@ struct LaunchPlan {
     bool gemv = false;          // decode family: the matrix-vector kernel for M <= 4 (4-bit weights, G = 128)
     int gemv_c = 0;             // ... and its k-blocks per wave (2, 4 or 8)
     bool gemv16 = false;        // decode family: its 16-row sibling with stationary activations (5 <= M <= 48)
+    bool gemv16_stream = false; // decode family: the 16-row kernel that streams its activations (long K, 5 <= M <= 16)
     int tiles_x = 0, tiles_y = 0;  // async prefill kernel: the tile grid; its launch is 1-D
     int full_tiles = 0;         // ... of which this many run unsplit (the rest in split_k parts each)
     unsigned grid[3] = {1, 1, 1};
@@ -181,6 +182,9 @@ int launch_decode(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_batch(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_gemv(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+int launch_gemv16_stream(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
+// dynamic LDS of the 16-row kernel with streamed activations
+size_t gemv16s_lds_bytes(int waves);
 // dynamic LDS of the 16-row kernel: c k-blocks per wave, `waves` waves, one or two buffers of partial sums
 size_t gemv16_lds_bytes(int c, int waves, int red_bufs);
 // k-blocks per wave that the 16-row kernel runs a node with, given those of the node's channel-major tables and the

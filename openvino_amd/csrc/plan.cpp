@@ -21,6 +21,7 @@ namespace ovfcc {
 //            (small-batch kernel instead of the streaming kernel), OVFCC_GEMV = 0 | 1, OVFCC_GEMV_C = 2 | 4 | 8,
 //            OVFCC_GEMV16 = 0 | 1 (the 16-row kernel with stationary activations for 5-48 rows),
 //            OVFCC_GEMV16_GRID = n (its workgroups per row tile), OVFCC_GEMV16_SPLIT = 1 | 2 | 4 | 8 (parts it cuts K in),
+//            OVFCC_GEMV16_STREAM = 0 | 1 (the 16-row kernel that streams its activations, for long K at 5-16 rows),
 //            OVFCC_PREFILL_{DIRECT, ASYNC, WIDE, BIG, TAIL} = 0 | 1, OVFCC_PREFILL_ROWS = 64 | 128,
 //            OVFCC_MOE_HOST_ROUTING = 1, OVFCC_MLP_FUSED = 1 (an MLP node of up to four rows as one launch instead of two),
 //            OVFCC_MLP_GRID = n (its workgroups), OVFCC_MLP_SPIN_LIMIT = n (polls after which that launch's wait for its workgroups gives up; tests);
@@ -35,6 +36,7 @@ struct EnvEntry {
 EnvEntry g_env[] = {EnvEntry("OVFCC_DECODE_WAVES"),   EnvEntry("OVFCC_DECODE_RT"),      EnvEntry("OVFCC_DECODE_XLDS"),
                     EnvEntry("OVFCC_DECODE_BATCH"),   EnvEntry("OVFCC_GEMV"),           EnvEntry("OVFCC_GEMV_C"),
                     EnvEntry("OVFCC_GEMV16"),         EnvEntry("OVFCC_GEMV16_GRID"),    EnvEntry("OVFCC_GEMV16_SPLIT"),
+                    EnvEntry("OVFCC_GEMV16_STREAM"),
                     EnvEntry("OVFCC_PREFILL_DIRECT"), EnvEntry("OVFCC_PREFILL_ASYNC"),  EnvEntry("OVFCC_PREFILL_WIDE"),
                     EnvEntry("OVFCC_PREFILL_BIG"),    EnvEntry("OVFCC_PREFILL_TAIL"),   EnvEntry("OVFCC_PREFILL_ROWS"),
                     EnvEntry("OVFCC_MOE_HOST_ROUTING"), EnvEntry("OVFCC_MLP_FUSED"),      EnvEntry("OVFCC_MLP_SPIN_LIMIT"),
@@ -230,6 +232,41 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         }
         return false;
     };
+    // Five to sixteen rows where the kernel above has nothing to keep -- K too long for it (the down projection of
+    // an MLP), or no more channel tiles than compute units, so that every workgroup would visit one tile and wait
+    // for all of its activations first: the 16-row kernel that streams its activations k-block by k-block, one
+    // workgroup per channel tile over all of K -- no split along K, no second launch (4096 -> 4096 at 16 rows:
+    // 4.8 against 5.4 us; 14336 -> 4096 at 8 rows: 10.1 against 12.4 us for the small-batch kernel, at 16 rows 12.1
+    // against 12.7).  It needs about as many channel tiles as compute units to fill the chip (1024 channels: a tie),
+    // and from 17 rows on every tile's weights would be streamed twice.  OVFCC_GEMV16_STREAM = 0 switches it off, = 1 takes
+    // it wherever it can run (before the kernel above, and whatever the number of channel tiles).
+    const int stream_env = env_int("OVFCC_GEMV16_STREAM", -1);
+    auto plan_gemv16_stream = [&]() -> bool {
+        if (a.M <= 4 || a.M > 16 || !a.scale_cm || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 ||
+            force_split > 0 || L.gemv_c == 0 || L.glu || env_int("OVFCC_GEMV16", 1) == 0 ||
+            stream_env == 0 || env_int("OVFCC_GEMV16_SPLIT", 0) > 0 || env_int("OVFCC_GEMV16_GRID", 0) > 0 ||
+            env_int("OVFCC_DECODE_BATCH", -1) >= 0 || L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 31))
+            return false;
+        const int waves = (int)(L.k_blocks / L.gemv_c);
+        if (L.k_blocks % L.gemv_c != 0 || waves < 1 || waves > 16 || (stream_env != 1 && L.n_tiles * 2 < n_cus) ||
+            gemv16s_lds_bytes(waves) > 160 * 1024 - 64)
+            return false;
+        p.gemv16_stream = true;
+        p.gemv_c = L.gemv_c;
+        p.split_k = 1;
+        p.kblocks_per_split = (int)L.k_blocks;
+        p.tiles_per_group = 1;
+        p.grid[0] = (unsigned)L.n_tiles;
+        p.grid[1] = 1;
+        p.grid[2] = 1;
+        p.block = 64u * waves;
+        p.tile_m = 16;
+        p.tile_n = 16;
+        p.dynamic_lds = (unsigned)gemv16s_lds_bytes(waves);
+        p.workspace_bytes = 0;
+        p.name = "fcc_gemv16s_w4";
+        return true;
+    };
     if (kernel == OVFCC_KERNEL_PLAIN) {
         if (a.M > 65535)
             return fail(OVFCC_EUNSUPPORTED, "the plain kernel handles at most 65535 rows");
@@ -237,7 +274,7 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.grid[1] = (unsigned)a.M;
         p.block = 64;
         p.name = "fcc_plain";
-    } else if (kernel == OVFCC_KERNEL_DECODE && plan_gemv16()) {
+    } else if (kernel == OVFCC_KERNEL_DECODE && (((stream_env == 1 || L.n_tiles <= n_cus) && plan_gemv16_stream()) || plan_gemv16() || plan_gemv16_stream())) {
         // planned
     } else if (kernel == OVFCC_KERNEL_DECODE && want_batch) {
         if (int rc = plan_batch())
@@ -468,6 +505,7 @@ int launch_fc(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {
     case OVFCC_KERNEL_DECODE:
         return p.gemv     ? launch_gemv(a, p, stream)
                : p.gemv16 ? launch_gemv16(a, p, stream)
+               : p.gemv16_stream ? launch_gemv16_stream(a, p, stream)
                : p.batch  ? launch_batch(a, p, stream)
                           : launch_decode(a, p, stream);
     default:

@@ -2,7 +2,8 @@
 inputs) against the CPU oracle: every division of K over the waves of a workgroup (2, 4 or 8 k-blocks per wave),
 every row count class (part of a row tile, a whole one, part of the second, two, part of the third, three), workgroups that visit one, two
 and many channel tiles, zero-point table / constant / none, bias, both output types, the same bits on every
-repetition, the gated linear unit, and the node shapes of the benchmark."""
+repetition, the gated linear unit, and the node shapes of the benchmark; and of its sibling for five to 16 rows that
+streams the activations instead (K too long to keep them: the down projection)."""
 import sys
 
 import numpy as np
@@ -133,7 +134,9 @@ def test_gemv16_benchmark_nodes(oracle, dev, req, name, N, K):
             say(f"gemv16 {name} M={M}")
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
-            assert info["name"] == "fcc_gemv16_w4", info
+            # as many channel tiles as compute units and one row tile: nothing to keep, the activations are streamed
+            streamed = name == "q/o" and M <= 16
+            assert info["name"] == ("fcc_gemv16s_w4" if streamed else "fcc_gemv16_w4"), info
             check_parity(oracle, y[:, cols], ref[:M], K, f"{name} M={M} {info}")
     finally:
         w.close()
@@ -219,22 +222,92 @@ def test_gemv16_two_parts_by_policy(oracle, dev, req):
 
 
 def test_gemv16_down_projection(oracle, dev, req):
-    """The benchmark's down projection (14336 -> 4096) takes the kernel with K in four parts from 17 rows on."""
+    """The benchmark's down projection (14336 -> 4096): up to 16 rows the kernel that streams its activations (one
+    workgroup of 14 waves per channel tile, K whole), from 17 rows on stationary activations with K in four parts."""
     K, N = 14336, 4096
     c = datagen.make_case(7860, 48, K, N, "i4", 128, "none")
     w = fc.CompressedWeights.from_case(dev, c)
     cols = np.sort(np.random.default_rng(6).choice(N, size=256, replace=False))
     ref = oracle_y(oracle, c, n_index=cols)
     try:
-        for M in (8, 16, 17, 32, 48):
+        for M in (5, 8, 13, 16, 17, 32, 48):
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
             say(f"gemv16 down M={M} {info}")
-            if M <= 16:    # one row tile: the small-batch kernel is as fast and needs one launch
-                assert info["name"] == "fcc_batch_w4", info
+            if M <= 16:
+                assert info["name"] == "fcc_gemv16s_w4" and info["split_k"] == 1 and info["block"] == 64 * 14, info
+                assert info["grid"] == (N // 16, 1, 1), info
             else:
                 assert info["name"] == "fcc_gemv16_w4" and info["split_k"] == 4 and info["block"] == 64 * 14, info
             check_parity(oracle, y[:, cols], ref[:M], K, f"down M={M} {info}")
+            assert np.array_equal(req.infer(w, c.x[:M]).view(np.uint8), y.view(np.uint8))
+    finally:
+        w.close()
+
+
+# (w_type, zp_type, N, K, k-blocks per wave, bias, output)
+STREAM_SHAPES = [
+    ("u4", "u4", 64, 1024, 2, True, "f16"),      # 4 waves of 2 k-blocks: both activation buffers filled once, no refill
+    ("u4", "u4", 272, 1024, 8, False, "f32"),    # 1 wave walks all of K: six refills, adds its own four row groups
+    ("i4", "none", 48, 2048, 4, True, "f16"),    # 4 waves of 4; symmetric weights (zero-point 8 as a constant)
+    ("u4", "u8", 96, 4096, 8, True, "f16"),      # 8-bit zero-point table, two words per channel and wave
+    ("u4", "none", 32, 256, 2, True, "f32"),     # 1 wave, 2 k-blocks, no zero-point
+    ("u4", "u4", 80, 14336, 8, False, "f32"),    # the down projection's K: 14 waves, 126 KiB of LDS
+    ("i4", "none", 64, 14336, 8, True, "f16"),
+    ("u4", "u4", 64, 4096, 2, True, "f16"),      # 16 waves: the largest workgroup, 144 KiB of LDS
+]
+
+
+@pytest.mark.parametrize("wt,zt,N,K,C,bias,out", STREAM_SHAPES)
+def test_gemv16_streamed_activations(oracle, dev, req, monkeypatch, wt, zt, N, K, C, bias, out):
+    """The 16-row kernel that streams its activations through a double buffer per wave, taken wherever it can run
+    (OVFCC_GEMV16_STREAM = 1): every division of K over the waves, rows short of a tile (loaded out of range, so
+    that the count of loads in flight does not depend on M) and a whole tile, the same bits on every repetition."""
+    monkeypatch.setenv("OVFCC_GEMV_C", str(C))
+    monkeypatch.setenv("OVFCC_GEMV16_STREAM", "1")
+    c = datagen.make_case(7450 + N + K, 16, K, N, wt, 128, zt, with_bias=bias)
+    w = fc.CompressedWeights.from_case(dev, c, output_type=out)
+    ref = oracle_y(oracle, c)
+    try:
+        for M in (5, 8, 15, 16):
+            say(f"gemv16s {wt}/{zt} N={N} K={K} C={C} out={out} M={M}")
+            y = req.infer(w, c.x[:M])
+            info = req.last_kernel()
+            assert info["name"] == "fcc_gemv16s_w4" and info["block"] == 64 * (K // 128 // C), info
+            assert info["grid"] == (N // 16, 1, 1) and info["split_k"] == 1, info
+            assert y.dtype == (np.float32 if out == "f32" else np.float16)
+            check_parity(oracle, y, ref[:M], K, f"M={M} {info}", output_rounding_slack=True)
+            for _ in range(3):    # partial sums are added in wave order
+                assert np.array_equal(req.infer(w, c.x[:M]).view(np.uint8), y.view(np.uint8))
+        # 17 rows and the switch: other kernels
+        monkeypatch.setenv("OVFCC_GEMV16_STREAM", "0")
+        req.infer(w, c.x[:8])
+        assert req.last_kernel()["name"] != "fcc_gemv16s_w4"
+    finally:
+        w.close()
+
+
+def test_gemv16_streamed_tiny_and_huge_activations(oracle, dev, req, monkeypatch):
+    """Subnormal activations, activations near the top of the half range and a row of zeros through the streaming
+    kernel (same arithmetic as the stationary one: half of the activations are multiplied by 2^-4 in registers)."""
+    monkeypatch.setenv("OVFCC_GEMV16_STREAM", "1")
+    c = datagen.make_case(7701, 8, 2048, 64, "u4", 128, "u4")
+    x = c.x.astype(np.float32)
+    x[0] *= 2.0 ** -12
+    x[1] = np.where(np.arange(c.K) % 3 == 0, 6.0e-8, 0.0)
+    x[2] = np.where(np.arange(c.K) % 128 == 5, 60000.0, x[2])
+    x[3] = 0.0
+    xh = x.astype(np.float16)
+    w = fc.CompressedWeights.from_case(dev, c, output_type="f32")
+    try:
+        y = req.infer(w, xh)
+        assert req.last_kernel()["name"] == "fcc_gemv16s_w4"
+        ref = oracle_y(oracle, c, x=xh)
+        assert np.all(y[3] == 0.0)
+        for m in range(8):
+            scale = float(np.max(np.abs(ref[m]))) or 1.0
+            err = float(np.max(np.abs(y[m] - ref[m])))
+            assert err <= 1e-3 * scale + 2.0 ** -21 * (c.K / 2) * 15 * 0.02, (m, err, scale)
     finally:
         w.close()
 
