@@ -33,8 +33,9 @@
 // Waves: wn = wave & 3 picks 64 of the 256 channels, kg = wave >> 2 picks which two of the four 32-input
 // steps of every k-block the wave contracts.  A wave unpacks every weight it uses exactly once and multiplies
 // it with all 128 rows (eight 16-row operands read from LDS): 32 v_mfma_f32_16x16x32_f16 per step and 4
-// unpacked dwords.  After the last k-block k-group 1 hands its f32 accumulators to k-group 0 through LDS,
-// which adds, applies per-channel scale, bias and the gated linear unit and stores (prefill_epilogue.h).
+// unpacked dwords.  After the last k-block the k-groups exchange halves of their f32 accumulators through LDS
+// (each finishes half of the row tiles), add, apply per-channel scale, bias and the gated linear unit and store
+// whole 128-byte lines (prefill_epilogue.h).
 //
 // The inner loop is software-pipelined by hand and pinned with scheduling barriers: between every two MFMAs
 // of a step sit one or two vector-ALU operations of the *next* step's unpack, and every few MFMAs one memory
@@ -393,9 +394,11 @@ __device__ __forceinline__ void prefill_async_body(const uint4_t* __restrict__ w
         }
     }
 
-    // ---- epilogue (prefill_epilogue.h): k-group hand-over, scale / bias / gated linear unit, split-K fix-up ----
+    // ---- epilogue (prefill_epilogue.h): the k-groups exchange halves, scale / bias / gated linear unit, split-K fix-up ----
     __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(0));  // the out-of-range loads of the last trips still target LDS
-    tile_epilogue<PRESCALE, NT>(acc, lds_raw, st, bias, y, ws, counters, M, N, n0, m0, split_k, wk.z, tile_id, out_f32, glu);
+    static_assert(pa_lds_bytes(NT, GPB) >= 8u * 4u * ((NT + 1) / 2) * 1024u, "the epilogue's exchange buffer");
+    tile_epilogue_shared<PRESCALE, NT>(acc, lds_raw, st, bias, y, ws, counters, M, N, n0, m0, split_k, wk.z, tile_id,
+                                       out_f32, glu);
 }
 #undef PA_DESC_X
 #undef PA_DESC_W

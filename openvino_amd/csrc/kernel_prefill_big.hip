@@ -329,7 +329,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             *reinterpret_cast<float4_t*>(static_cast<float*>(y) + idx) = float4_t{o[0], o[1], o[2], o[3]};
         else
             *reinterpret_cast<half4_t*>(static_cast<half_t*>(y) + idx) =
-                half4_t{(half_t)o[0], (half_t)o[1], (half_t)o[2], (half_t)o[3]};
+                half4_t{to_half_rne(o[0]), to_half_rne(o[1]), to_half_rne(o[2]), to_half_rne(o[3])};
     };
     if (glu) {
         // channel tiles 2 j and 2 j + 1 of the wave are gate and up of output channels (n0 + 64 wave) / 2 + 16 j ..
@@ -372,8 +372,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float4_t v = acc[r][t];
-                const half4_t h = half4_t{(half_t)(v.x * sc[r][0] + bs[r][0]), (half_t)(v.y * sc[r][1] + bs[r][1]),
-                                          (half_t)(v.z * sc[r][2] + bs[r][2]), (half_t)(v.w * sc[r][3] + bs[r][3])};
+                const half4_t h = half4_t{to_half_rne(v.x * sc[r][0] + bs[r][0]), to_half_rne(v.y * sc[r][1] + bs[r][1]),
+                                          to_half_rne(v.z * sc[r][2] + bs[r][2]), to_half_rne(v.w * sc[r][3] + bs[r][3])};
                 const uint2_t u = __builtin_bit_cast(uint2_t, h);
                 p[r][0] = u.x, p[r][1] = u.y;
             }
