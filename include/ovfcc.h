@@ -57,7 +57,7 @@ typedef struct ovfcc_fc_desc {
     int32_t bias_type;  /* OVFCC_NONE | OVFCC_F16, [N] */
     int32_t act_type;   /* OVFCC_F16 */
     int32_t out_type;   /* OVFCC_F16 | OVFCC_F32 (FullyConnected's output_type; default = activation type) */
-    int32_t flags;      /* 0, or OVFCC_GLU_* [| OVFCC_GLU_GATE_SECOND] | OVFCC_DYNQUANT_I8 [| OVFCC_DYNQUANT_PER_GROUP] | OVFCC_W_INPUT_MAJOR */
+    int32_t flags;      /* 0, or OVFCC_GLU_* [| OVFCC_GLU_GATE_SECOND] | OVFCC_DYNQUANT_I8 [| OVFCC_DYNQUANT_PER_GROUP | OVFCC_DYNQUANT_ASYM] | OVFCC_W_INPUT_MAJOR */
 } ovfcc_fc_desc;
 
 /* Gated linear unit fused into the node (flags).  The reference fuses ov::op::internal::GLU
@@ -106,6 +106,22 @@ typedef struct ovfcc_fc_desc {
  *     y[m, n] = sum_g ( sum_{k in g} q[m, k] (W[n, k] - ZP[n, g]) ) * S[n, g] * inv_scale[m (, g)]  + bias[n],
  * q and inv_scale as above over a row or a group, the integer sums exact, the sum over groups in f32. */
 #define OVFCC_DYNQUANT_PER_GROUP 32
+
+/* With OVFCC_DYNQUANT_I8, per token only: the reference's asymmetric form of the same quantisation -- unsigned 8-bit
+ * activations with a zero-point per token (ov::op::internal::DynamicQuantize with QuantizationType::Asymmetric,
+ * quantization_dt = zp_dt = u8: src/common/transformations/include/ov_ops/dynamic_quantize.hpp:16-60, chosen by
+ * src/plugins/intel_gpu/src/plugin/transformations/dynamic_quantize_fully_connected.cpp:109-117; arithmetic of
+ * cl_kernels/dynamic_quantize_gpu_ref.cl:100-250 with ASYMMETRIC_QUANTIZATION and UNSIGNED_OUTPUT; consumed as the
+ * source zero-point of the matrix product, src/plugins/intel_gpu/src/graph/impls/onednn/fully_connected_onednn.cpp:
+ * 83-88,325-329).  Takes effect where OVFCC_DYNQUANT_I8 does for 8-bit weights with one scale per channel, and
+ * K < 65536:
+ *     d = max_k x - min_k x in half (0.003 if the two are equal), scale = half(255 / d), zp = half(-min * (255 / d)),
+ *     q[m, k] = sat_u8(rte(half(x[m, k] * scale) + zp)),  za[m] = sat_u8(rte(zp)),
+ *     y[m, n] = sum_k (q[m, k] - za[m]) (W[n, k] - ZP[n]) * (S[n] * half(1 / scale)) + bias[n],
+ * integers exact.  The conversions saturate where the reference's are undefined (a row whose values all lie on one
+ * side of zero has a zero-point outside 0..255; such a row is shifted by the clamped zero-point, as it would be on
+ * hardware whose conversion saturates). */
+#define OVFCC_DYNQUANT_ASYM 64
 
 /* Input-major constants (flags): W is given as [K, N] (grouped: [K/G, G, N]) and scales / zero-points as
  * [K/G, N], each packed over its own flattened index -- the form in which a MatMul with transpose_b = false holds

@@ -20,6 +20,7 @@ GLU_GATE_SECOND = 4
 DYNQUANT_I8 = 8                                                        # OVFCC_DYNQUANT_I8
 W_INPUT_MAJOR = 16
 DYNQUANT_PER_GROUP = 32                                                # OVFCC_DYNQUANT_PER_GROUP                                                     # OVFCC_W_INPUT_MAJOR
+DYNQUANT_ASYM = 64                                                      # OVFCC_DYNQUANT_ASYM
 
 # every symbol include/ovfcc_bench.h declares (libovfcc_bench.so)
 BENCH_SYMBOLS = ["ovfcc_bench_layers", "ovfcc_bench_grouped", "ovfcc_bench_copy", "ovfcc_bench_floor", "ovfcc_bench_mfma", "ovfcc_bench_issue"]

@@ -184,6 +184,17 @@ void fill_args(const ovfcc_weights* w, const void* x, void* y, int64_t M, ovfcc:
 int finish_weights(ovfcc_weights* W) {
     ovfcc::Layout& L = W->layout;
     L.gemv_c = 0;
+    // 8-bit nodes with one scale per channel whose activations may be quantised asymmetrically: the sums of their
+    // zero-point-corrected weights per channel, which the activations' zero-points multiply
+    if (L.dynquant_asym && L.tiled && L.bits == 8 && L.groups == 1 && W->desc.K <= ovfcc::kI8AsymMaxK && !W->d_colsum) {
+        HIP_TRY(hipMalloc(reinterpret_cast<void**>(&W->d_colsum), (size_t)W->desc.N * sizeof(int)));
+        W->bytes += (size_t)W->desc.N * sizeof(int);
+        int e = ovfcc::launch_i8_colsum(W->d_w, L.zp_table ? W->d_zp : nullptr, L.zp_const, W->d_colsum, L.n_tiles,
+                                        L.k_blocks, nullptr);
+        if (e)
+            return hip_fail((hipError_t)e, "column sum launch");
+        HIP_TRY(hipStreamSynchronize(nullptr));
+    }
     if (!L.tiled || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 || !W->d_scale)
         return OVFCC_OK;
     const int c = ovfcc::gemv_kblocks_per_wave(L, W->ctx->n_cus);
@@ -378,7 +389,7 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
         if (static_scratch)
             return fail(OVFCC_EUNSUPPORTED, "a node with int8 activations needs a quantisation buffer of the request");
         const size_t q_bytes = ((size_t)M * w->desc.K + 255) & ~(size_t)255;
-        const size_t need = q_bytes + (size_t)M * 8;
+        const size_t need = q_bytes + (size_t)M * 12;
         if (need > r->quant_cap)
             HIP_TRY(hipStreamSynchronize(r->stream));
         int rc = grow(&r->d_quant, &r->quant_cap, need);
@@ -387,16 +398,19 @@ int enqueue_rows(ovfcc_request* r, const ovfcc_weights* w, const void* x, void* 
         char* base = static_cast<char*>(r->d_quant);
         float* inv_scale = reinterpret_cast<float*>(base + q_bytes);
         int* qsum = reinterpret_cast<int*>(base + q_bytes + (size_t)M * 4);
-        int e = ovfcc::launch_dynquant(x, base, inv_scale, qsum, M, w->desc.K, r->stream);
+        // unsigned bytes with a zero-point per token where the node asks for them (and has its column sums)
+        int* za = w->d_colsum ? reinterpret_cast<int*>(base + q_bytes + (size_t)M * 8) : nullptr;
+        int e = za ? ovfcc::launch_dynquant_asym(x, base, inv_scale, qsum, za, M, w->desc.K, r->stream)
+                   : ovfcc::launch_dynquant(x, base, inv_scale, qsum, M, w->desc.K, r->stream);
         if (!e)
-            e = ovfcc::launch_prefill_i8(a, base, inv_scale, qsum, r->stream);
+            e = ovfcc::launch_prefill_i8(a, base, inv_scale, qsum, za, w->d_colsum, r->stream);
         if (e)
             return hip_fail((hipError_t)e, "integer kernel launch");
         ovfcc::LaunchPlan shown;
         shown.kernel = OVFCC_KERNEL_PREFILL;
         shown.tile_m = 128, shown.tile_n = 256, shown.block = 512;
         shown.grid[0] = (unsigned)(w->desc.N / 256), shown.grid[1] = (unsigned)((M + 127) / 128);
-        shown.name = "fcc_prefill_i8_w8";
+        shown.name = za ? "fcc_prefill_i8_w8_asym" : "fcc_prefill_i8_w8";
         record(r, shown);
         return OVFCC_OK;
     }
@@ -972,6 +986,7 @@ void ovfcc_weights_destroy(ovfcc_weights* w) {
     if (w->d_zp) (void)hipFree(w->d_zp);
     if (w->d_bias) (void)hipFree(w->d_bias);
     if (w->d_scale_cm) (void)hipFree(w->d_scale_cm);
+    if (w->d_colsum) (void)hipFree(w->d_colsum);
     if (w->d_zp_cm) (void)hipFree(w->d_zp_cm);
     delete w;
 }

@@ -31,6 +31,7 @@ struct ovfcc_weights {
     ovfcc_weights* mlp_down = nullptr;  // ovfcc_weights_mlp: this node is gate / up, that one (owned) the down projection
     void* d_scale_cm = nullptr;  // channel-major copies of the group parameters for the matrix-vector kernel
     void* d_zp_cm = nullptr;
+    int* d_colsum = nullptr;     // 8-bit per-channel node with OVFCC_DYNQUANT_ASYM: sum_k (w - zp) per channel, tiled order
     size_t bytes = 0;
     // Launch plans of recent calls, keyed by what a plan depends on besides the node itself.  Shared by every
     // request that runs the node, hence the lock; eight entries, replaced in turn.

@@ -57,6 +57,7 @@ struct Layout {
                             // parameter tables are written (0: the node has none)
     bool dynquant = false;  // the node allows int8 activations (OVFCC_DYNQUANT_I8) where a kernel exists
     bool dynquant_grouped = false;  // ... quantised per group of 128 inputs rather than per token (4-bit nodes)
+    bool dynquant_asym = false;     // ... as unsigned bytes with a zero-point per token (8-bit per-channel nodes)
     // element index of the scale / zero-point of channel r of tile nt for group g
     size_t param_index(int64_t nt, int64_t g, int r) const {
         if (groups_per_kblock == 1)
@@ -334,8 +335,18 @@ size_t dynquant_w4_scale_floats(int64_t M, int64_t K, bool grouped);
 int launch_dynquant_w4(const void* x, void* xq, float* inv, int64_t M, int64_t K, bool grouped, void* stream);
 bool prefill_i8w4_applies(const Layout& L, int64_t N, int zp_type);
 int launch_prefill_i8w4(const FcDeviceArgs& a, const void* xq, const float* inv, bool grouped, void* stream);
-// Integer prefill kernel over launch_dynquant's outputs: tiled 8-bit weights, one group per channel, N % 256 == 0.
-int launch_prefill_i8(const FcDeviceArgs& a, const void* xq, const float* inv_scale, const int* qsum, void* stream);
+// The asymmetric form: unsigned bytes with a zero-point per row, stored minus 128 (xq, za) for the integer kernel's
+// signed operands; and the per-channel sums cw[n] = sum_k (w[n, k] - zp[n]) that form needs, from a node's tiled
+// 8-bit weights (channels in tiled order).  sum_k (q - za)(w - zp) has to fit 32 bits: K <= kI8AsymMaxK.
+constexpr int64_t kI8AsymMaxK = 32768;
+int launch_dynquant_asym(const void* x, void* xq, float* inv_scale, int* qsum, int* za, int64_t M, int64_t K,
+                         void* stream);
+int launch_i8_colsum(const void* w_tiled, const void* zp_tiled, int zp_const, int* cw, int64_t n_tiles, int64_t k_blocks,
+                     void* stream);
+// Integer prefill kernel over launch_dynquant's outputs (za and cw null) or launch_dynquant_asym's: tiled 8-bit
+// weights, one group per channel, N % 256 == 0.
+int launch_prefill_i8(const FcDeviceArgs& a, const void* xq, const float* inv_scale, const int* qsum, const int* za,
+                      const int* cw, void* stream);
 // dst[r] = src[src_row[r]] (dst_row null) or dst[dst_row[r]] = src[r] (src_row null), rows of row_bytes % 16 == 0 bytes;
 // the caller guarantees that every index is a row of the buffer it addresses
 int launch_rows(void* dst, const void* src, const int* src_row, const int* dst_row, int rows, int row_bytes,

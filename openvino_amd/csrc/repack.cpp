@@ -63,10 +63,13 @@ int validate_desc(const ovfcc_fc_desc* d) {
         return fail(OVFCC_EUNSUPPORTED, "activations must be f16");
     if (d->out_type != OVFCC_F16 && d->out_type != OVFCC_F32)
         return fail(OVFCC_EUNSUPPORTED, "output must be f16 or f32");
-    if (d->flags & ~(OVFCC_GLU_TYPE_MASK | OVFCC_GLU_GATE_SECOND | OVFCC_DYNQUANT_I8 | OVFCC_DYNQUANT_PER_GROUP | OVFCC_W_INPUT_MAJOR))
+    if (d->flags & ~(OVFCC_GLU_TYPE_MASK | OVFCC_GLU_GATE_SECOND | OVFCC_DYNQUANT_I8 | OVFCC_DYNQUANT_PER_GROUP | OVFCC_DYNQUANT_ASYM |
+                     OVFCC_W_INPUT_MAJOR))
         return fail(OVFCC_EINVAL, "unknown bits in flags");
     if ((d->flags & OVFCC_DYNQUANT_PER_GROUP) && !(d->flags & OVFCC_DYNQUANT_I8))
         return fail(OVFCC_EINVAL, "OVFCC_DYNQUANT_PER_GROUP without OVFCC_DYNQUANT_I8");
+    if ((d->flags & OVFCC_DYNQUANT_ASYM) && (!(d->flags & OVFCC_DYNQUANT_I8) || (d->flags & OVFCC_DYNQUANT_PER_GROUP)))
+        return fail(OVFCC_EINVAL, "OVFCC_DYNQUANT_ASYM goes with OVFCC_DYNQUANT_I8 and per-token quantisation only");
     if ((d->flags & OVFCC_GLU_GATE_SECOND) && (d->flags & OVFCC_GLU_TYPE_MASK) == OVFCC_GLU_NONE)
         return fail(OVFCC_EINVAL, "OVFCC_GLU_GATE_SECOND without a gated-linear-unit type");
     if ((d->flags & OVFCC_GLU_TYPE_MASK) != OVFCC_GLU_NONE && (d->N % 2) != 0)
@@ -86,6 +89,7 @@ Layout make_layout(const ovfcc_fc_desc& d) {
     // K / 128 < 2^16 keeps the kernels' 32-bit offsets and reciprocal group index exact
     L.dynquant = (d.flags & OVFCC_DYNQUANT_I8) != 0;
     L.dynquant_grouped = L.dynquant && (d.flags & OVFCC_DYNQUANT_PER_GROUP) != 0;
+    L.dynquant_asym = L.dynquant && (d.flags & OVFCC_DYNQUANT_ASYM) != 0;
     L.glu = d.flags & OVFCC_GLU_TYPE_MASK;
     L.glu_gate_second = (d.flags & OVFCC_GLU_GATE_SECOND) != 0;
     const bool small_groups = L.bits == 4 && (d.group_size == 32 || d.group_size == 64);

@@ -35,7 +35,9 @@ def make_desc(N: int, K: int, group_size: int, w_type: str, zp_type: str = "none
     d.out_type = _lib.TYPE[out_type]
     d.flags = (_lib.GLU[glu] | (_lib.GLU_GATE_SECOND if glu_gate_second else 0) |
                (_lib.DYNQUANT_I8 if dynamic_quantization else 0) |
-               (_lib.DYNQUANT_PER_GROUP if dynamic_quantization == "per_group" else 0) | (_lib.W_INPUT_MAJOR if input_major else 0))
+               (_lib.DYNQUANT_PER_GROUP if dynamic_quantization == "per_group" else 0) |
+               (_lib.DYNQUANT_ASYM if dynamic_quantization == "asymmetric" else 0) |
+               (_lib.W_INPUT_MAJOR if input_major else 0))
     return d
 
 

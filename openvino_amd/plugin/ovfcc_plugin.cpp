@@ -977,18 +977,20 @@ public:
 
     std::shared_ptr<ov::ICompiledModel> compile_model(const std::shared_ptr<const ov::Model>& model,
                                                       const ov::AnyMap& properties) const override {
-        bool profiling = m_profiling;
+        bool profiling = m_profiling, dq_asym = m_dq_asym;
         uint64_t dq_group = m_dq_group;
         for (const auto& kv : properties) {
             if (kv.first == ov::enable_profiling.name())
                 profiling = kv.second.as<bool>();
             else if (kv.first == ov::hint::dynamic_quantization_group_size.name())
                 dq_group = kv.second.as<uint64_t>();
+            else if (kv.first == kAsymDynamicQuantization)
+                dq_asym = kv.second.as<bool>();
             else if (!known_hint(kv.first))
                 OPENVINO_THROW("MI355X: unsupported property ", kv.first);
         }
         return std::make_shared<CompiledModel>(model->clone(), shared_from_this(), context(), profiling,
-                                               dq_group != 0 ? OVFCC_DYNQUANT_I8 : 0);
+                                               dq_group == 0 ? 0 : OVFCC_DYNQUANT_I8 | (dq_asym ? OVFCC_DYNQUANT_ASYM : 0));
     }
     std::shared_ptr<ov::ICompiledModel> compile_model(const std::shared_ptr<const ov::Model>& model,
                                                       const ov::AnyMap& properties,
@@ -1002,6 +1004,8 @@ public:
                 m_profiling = kv.second.as<bool>();
             else if (kv.first == ov::hint::dynamic_quantization_group_size.name())
                 m_dq_group = kv.second.as<uint64_t>();  // non-zero: activations may be quantised per token
+            else if (kv.first == kAsymDynamicQuantization)
+                m_dq_asym = kv.second.as<bool>();  // ... as unsigned bytes with a zero-point per token
             else if (!known_hint(kv.first))
                 OPENVINO_THROW("MI355X: unsupported property ", kv.first);
         }
@@ -1020,6 +1024,7 @@ public:
                 {ov::execution_devices.name(), ov::PropertyMutability::RO},
                 {ov::enable_profiling.name(), ov::PropertyMutability::RW},
                 {ov::hint::dynamic_quantization_group_size.name(), ov::PropertyMutability::RW},
+                {kAsymDynamicQuantization, ov::PropertyMutability::RW},
                 {ov::hint::performance_mode.name(), ov::PropertyMutability::RW},
                 {ov::hint::inference_precision.name(), ov::PropertyMutability::RW},
                 {ov::hint::num_requests.name(), ov::PropertyMutability::RW},
@@ -1032,9 +1037,12 @@ public:
                 {ov::internal::caching_properties.name(), ov::PropertyMutability::RO}};
         if (name == ov::internal::caching_properties)
             return std::vector<ov::PropertyName>{ov::device::architecture.name(),
-                                                 ov::hint::dynamic_quantization_group_size.name()};
+                                                 ov::hint::dynamic_quantization_group_size.name(),
+                                                 kAsymDynamicQuantization};
         if (name == ov::hint::dynamic_quantization_group_size)
             return m_dq_group;
+        if (name == kAsymDynamicQuantization)
+            return m_dq_asym;
         if (name == ov::available_devices)
             return decltype(ov::available_devices)::value_type{"0"};
         if (name == ov::device::full_name)
@@ -1212,6 +1220,11 @@ private:
     mutable ovfcc_ctx* m_ctx = nullptr;
     bool m_profiling = false;
     uint64_t m_dq_group = 0;  // ov::hint::dynamic_quantization_group_size; 0 = off
+    // The Intel-GPU plugin's switch for the asymmetric form of that quantisation (ov::intel_gpu::
+    // asym_dynamic_quantization, src/plugins/intel_gpu/include/intel_gpu/runtime/internal_properties.hpp:177), by name:
+    // its header belongs to that plugin.
+    static constexpr const char* kAsymDynamicQuantization = "GPU_ASYM_DYNAMIC_QUANTIZATION";
+    bool m_dq_asym = false;
 };
 
 CompiledModel::CompiledModel(const std::shared_ptr<ov::Model>& model, const std::shared_ptr<const ov::IPlugin>& plugin,

@@ -55,6 +55,22 @@
  *                    sum and range of q; an independent numpy restatement; and, for the FC, equality with
  *                    ovo_fc_reference applied to the dequantised activations q * stored scale.
  *
+ *   dynquant_asym    the same with the reference's asymmetric form (unsigned 8-bit activations, a zero-point per
+ *                    token): dynamic_quantize_gpu_ref.cl:100-250 under ASYMMETRIC_QUANTIZATION and UNSIGNED_OUTPUT
+ *                    (d = max - min in half, 0.003 if equal; scale = half(255 / d); zp = half(-min * (255 / d));
+ *                    q = convert_uchar_rte(half(x * scale) + zp); stored scale 1 / scale; stored zero-point
+ *                    convert_uchar_rte(zp)), chosen by src/plugins/intel_gpu/src/plugin/transformations/
+ *                    dynamic_quantize_fully_connected.cpp:109-117 and consumed as the source zero-point of the
+ *                    product (graph/impls/onednn/fully_connected_onednn.cpp:83-88,325-329; oneDNN itself is a
+ *                    third-party dependency absent from the tree: its documented meaning, src = (q - zp) * scale,
+ *                    is what is restated).  The conversions saturate here where OpenCL leaves them undefined.
+ *                    The reference holds no numeric vector for it (its test compares two of its own kernels on
+ *                    inputs in [-16, 20]).  Pinned by: minimum -> 0 and maximum -> 255 on rows that straddle zero;
+ *                    |x - (q - za) * stored scale| bounded by half a step plus the half roundings; a constant row
+ *                    (d = 0.003); an independent numpy restatement in numpy's own half arithmetic; and, for the
+ *                    FC, equality with ovo_fc_reference applied to the dequantised activations (q - za) * stored
+ *                    scale (which fixes every cross term of the integer form).
+ *
  * Parity unpinned: the CPU plugin's numbers come from the oneDNN fork's decompression
  * inner-product kernel (openvinotoolkit/oneDNN, a submodule whose commit the tree does
  * not record and whose sources are absent).  Its summation order and intermediate
@@ -378,6 +394,97 @@ int ovo_fc_dynquant_reference(const int8_t* q, const float* inv_scale, const int
                 acc += (int32_t)q[m * K + k] * wv;
             }
             acc -= (int64_t)(zp ? (int32_t)zp[n] : 0) * qsum[m];
+            y[m * N + n] = (float)(int32_t)acc * (scale[n] * inv_scale[m]) + (bias ? bias[n] : 0.f);
+        }
+    return 0;
+}
+
+/* double -> f16 bits, round to nearest even (the exact sum of two halves fits a double; rounding it through float
+ * first could round twice). */
+static uint16_t ovo_f64_to_f16(double v) {
+    if (v != v)
+        return 0x7E00;
+    const uint16_t sign = signbit(v) ? 0x8000 : 0;
+    const double a = fabs(v);
+    if (a >= 65520.0)
+        return (uint16_t)(sign | 0x7C00);
+    if (a < 6.103515625e-05) /* below the smallest normal: a multiple of 2^-24 */
+        return (uint16_t)(sign | (uint16_t)nearbyint(a * 16777216.0));
+    int e;
+    (void)frexp(a, &e); /* a = f * 2^e, f in [0.5, 1): exponent of a is e - 1 */
+    int ex = e - 1;
+    double m = nearbyint(ldexp(a, 10 - ex)); /* 1024 .. 2048 */
+    if (m >= 2048.0) {
+        m = 1024.0;
+        ++ex;
+    }
+    if (ex > 15)
+        return (uint16_t)(sign | 0x7C00);
+    return (uint16_t)(sign | ((uint16_t)(ex + 15) << 10) | ((uint16_t)m - 1024));
+}
+
+static int32_t ovo_sat_u8_rte(float v) {
+    if (v != v)
+        return 0;
+    const float r = nearbyintf(v);
+    return (int32_t)(r > 255.f ? 255.f : (r < 0.f ? 0.f : r));
+}
+
+/* Per-token asymmetric quantisation of x [M, K] (f16 bit patterns) to unsigned bytes: q [M, K], inv_scale [M] (the
+ * f16 value the reference stores, as float), za [M] the stored zero-point, qsum [M] = sum_k q.  Half arithmetic as in
+ * the reference kernel: max, min exact; max - min one half subtraction; 255 / d and -min * (255 / d) in f32, each
+ * rounded to half; x * scale a half product (exact in f32, rounded once); + zp a half sum (exact in double, rounded
+ * once). */
+int ovo_dynquant_rows_asym(const uint16_t* x, int64_t M, int64_t K, uint8_t* q, float* inv_scale, int32_t* za,
+                           int32_t* qsum) {
+    if (!x || !q || !inv_scale || !za || !qsum || M < 0 || K <= 0)
+        return -1;
+    for (int64_t m = 0; m < M; ++m) {
+        float mx = -65504.f, mn = 65504.f;
+        for (int64_t k = 0; k < K; ++k) {
+            const float a = ovo_f16_to_f32(x[m * K + k]);
+            if (a > mx)
+                mx = a;
+            if (a < mn)
+                mn = a;
+        }
+        const float range = ovo_f16_to_f32(ovo_f64_to_f16((double)mx - (double)mn));
+        const float diff = mx == mn ? ovo_f16_to_f32(ovo_f32_to_f16(0.003f)) : range;
+        const float scale_f = 255.0f / diff;
+        const float scale = ovo_f16_to_f32(ovo_f32_to_f16(scale_f));
+        const float zp = ovo_f16_to_f32(ovo_f32_to_f16(-mn * scale_f));
+        int32_t sum = 0;
+        for (int64_t k = 0; k < K; ++k) {
+            const float p = ovo_f16_to_f32(ovo_f32_to_f16(ovo_f16_to_f32(x[m * K + k]) * scale));
+            const float v = ovo_f16_to_f32(ovo_f64_to_f16((double)p + (double)zp));
+            const int32_t i = ovo_sat_u8_rte(v);
+            q[m * K + k] = (uint8_t)i;
+            sum += i;
+        }
+        inv_scale[m] = ovo_f16_to_f32(ovo_f32_to_f16(1.0f / scale));
+        za[m] = ovo_sat_u8_rte(zp);
+        qsum[m] = sum;
+    }
+    return 0;
+}
+
+/* FullyConnected over asymmetrically quantised activations, 8-bit weights, one scale (and zero-point) per output
+ * channel: y[m, n] = sum_k (q[m, k] - za[m]) (w[n, k] - zp[n]) * (scale[n] * inv_scale[m]) (+ bias[n]), the sum
+ * exact, the rest in f32.  w_signed: weights are i8 instead of u8.  zp may be null (0), bias may be null. */
+int ovo_fc_dynquant_asym_reference(const uint8_t* q, const float* inv_scale, const int32_t* za, int64_t M, int64_t K,
+                                   int64_t N, const uint8_t* w, int32_t w_signed, const float* scale, const float* zp,
+                                   const float* bias, float* y) {
+    if (!q || !inv_scale || !za || !w || !scale || !y || M < 0 || K <= 0 || N <= 0)
+        return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; ++n)
+        for (int64_t m = 0; m < M; ++m) {
+            const int32_t zw = zp ? (int32_t)zp[n] : 0;
+            int64_t acc = 0;
+            for (int64_t k = 0; k < K; ++k) {
+                const int32_t wv = w_signed ? (int32_t)(int8_t)w[n * K + k] : (int32_t)w[n * K + k];
+                acc += (int64_t)((int32_t)q[m * K + k] - za[m]) * (wv - zw);
+            }
             y[m * N + n] = (float)(int32_t)acc * (scale[n] * inv_scale[m]) + (bias ? bias[n] : 0.f);
         }
     return 0;

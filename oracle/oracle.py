@@ -302,6 +302,43 @@ def fc_dynquant_reference(x, w, w_type, scale, zp=None, bias=None, *, N, K) -> n
     return y
 
 
+def dynquant_rows_asym(x):
+    """C oracle: per-token asymmetric quantisation of x [M, K] float16 to unsigned bytes -> (q uint8 [M, K],
+    inv_scale float32 [M], za int32 [M], qsum int32 [M])."""
+    x = np.ascontiguousarray(x, dtype=np.float16)
+    M, K = x.shape
+    q, inv = np.empty((M, K), np.uint8), np.empty(M, np.float32)
+    za, qs = np.empty(M, np.int32), np.empty(M, np.int32)
+    f = lib().ovo_dynquant_rows_asym
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                  ctypes.c_void_p]
+    if f(_ptr(x), M, K, _ptr(q), _ptr(inv), _ptr(za), _ptr(qs)) != 0:
+        raise ValueError("ovo_dynquant_rows_asym rejected its arguments")
+    return q, inv, za, qs
+
+
+def fc_dynquant_asym_reference(x, w, w_type, scale, zp=None, bias=None, *, N, K) -> np.ndarray:
+    """C oracle of the FullyConnected with per-token unsigned 8-bit activations and a zero-point per token: 8-bit
+    weights [N, K], one float scale (and zero-point) per channel.  Returns float32 [M, N]."""
+    if w_type not in (U8, I8):
+        raise ValueError("8-bit weights only")
+    q, inv, za, _ = dynquant_rows_asym(np.asarray(x).reshape(-1, K))
+    M = q.shape[0]
+    w = np.ascontiguousarray(w).view(np.uint8).reshape(N, K)
+    scale = np.ascontiguousarray(np.asarray(scale, dtype=np.float32).reshape(N))
+    zp = None if zp is None else np.ascontiguousarray(np.asarray(zp, dtype=np.float32).reshape(N))
+    bias = None if bias is None else np.ascontiguousarray(np.asarray(bias, dtype=np.float32).reshape(N))
+    y = np.empty((M, N), np.float32)
+    f = lib().ovo_fc_dynquant_asym_reference
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                  ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    if f(_ptr(q), _ptr(inv), _ptr(za), M, K, N, _ptr(w), int(w_type == I8), _ptr(scale), _ptr(zp), _ptr(bias), _ptr(y)) != 0:
+        raise ValueError("ovo_fc_dynquant_asym_reference rejected its arguments")
+    return y
+
+
 def dynquant_groups(x, G):
     """C oracle: symmetric int8 quantisation of x [M, K] float16 in groups of G inputs -> (q int8 [M, K],
     inv_scale float32 [M, K / G], qsum int32 [M, K / G])."""

@@ -59,6 +59,7 @@ def test_version_and_error_string():
     (dict(act_type=_lib.F32), _lib.EUNSUPPORTED), (dict(out_type=_lib.U8), _lib.EUNSUPPORTED),
     (dict(bias_type=_lib.F32), _lib.EUNSUPPORTED), (dict(flags=32), _lib.EINVAL), (dict(flags=64), _lib.EINVAL),
     (dict(flags=4), _lib.EINVAL), (dict(flags=1, N=63), _lib.EINVAL),
+    (dict(flags=8 | 32 | 64), _lib.EINVAL), (dict(flags=128), _lib.EINVAL),   # asymmetric: per token only; unknown bit
 ])
 def test_descriptor_gate(mutate, code):
     d = fc.make_desc(64, 256, 128, "u4", "u4")
@@ -67,6 +68,9 @@ def test_descriptor_gate(mutate, code):
         setattr(d, k, v)
     assert fc.validate(d) == code
     assert _lib.load().ovfcc_last_error() != b""
+    if "flags" in mutate and mutate["flags"] == 64:   # ... and only together with the permission itself
+        d.flags = _lib.DYNQUANT_I8 | _lib.DYNQUANT_ASYM
+        assert fc.validate(d) == _lib.OK
 
 
 def test_glu_descriptor_and_layout():

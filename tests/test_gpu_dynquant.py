@@ -216,3 +216,80 @@ def test_w4a8_llama8b_prefill_shape(oracle, dev, req, mode):
         assert r < (2e-2 if mode == "per_group" else 1e-1)
     finally:
         w.close()
+
+
+# ---- asymmetric form: unsigned 8-bit activations with a zero-point per token ----
+
+def dq_asym_reference(oracle, c, x=None):
+    zp = None if c.zp is None else c.zp.astype(np.float32)
+    return oracle.fc_dynquant_asym_reference(c.x if x is None else x, c.w, T[c.w_type], c.scale, zp, c.bias, N=c.N, K=c.K)
+
+
+@pytest.mark.parametrize("wt,zt,N,K,bias,out", [("u8", "u8", 256, 512, True, "f32"), ("u8", "none", 512, 384, False, "f16"),
+                                                ("i8", "none", 256, 1024, True, "f32"), ("u8", "u8", 768, 128, False, "f32"),
+                                                ("u8", "u8", 256, 4096, True, "f32")])
+def test_dynquant_asymmetric_matches_integer_oracle(oracle, dev, req, monkeypatch, wt, zt, N, K, bias, out):
+    """OVFCC_DYNQUANT_ASYM: the quantisation kernel's half arithmetic, the column sums of the node and the
+    zero-point terms of the epilogue against the oracle's sum_k (q - za)(w - zp) -- rows that straddle zero, rows
+    with an offset, a constant row, rows on one side of zero (clamped zero-point), the largest half."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    say(f"dynquant asym {wt}/{zt} N={N} K={K} bias={bias} out={out}")
+    c = datagen.make_case(1150, 300, K, N, wt, K, zt, with_bias=bias)
+    x = c.x.astype(np.float32)
+    x += np.linspace(-3, 3, 300, dtype=np.float32)[:, None]     # every row its own offset
+    x[5] = 0                                      # constant rows: d = 0.003
+    x[6] *= 40
+    x[7] = 0.125
+    x[8] = np.abs(x[8]) + 1                       # all positive: zero-point below 0, clamped
+    x[9] = -np.abs(x[9]) - 1                      # all negative: zero-point above 255, clamped
+    x[10, 3] = 65504
+    xh = x.astype(np.float16)
+    w = fc.CompressedWeights.from_case(dev, c, output_type=out, dynamic_quantization="asymmetric")
+    try:
+        for M in (49, 128, 129, 300):
+            y = req.infer(w, xh[:M])
+            info = req.last_kernel()
+            assert info["name"] == "fcc_prefill_i8_w8_asym", info
+            ref = dq_asym_reference(oracle, c, xh[:M])
+            # the row with 65504 overflows its half scale, and an f16 result its range: the same on both sides
+            with np.errstate(over="ignore"):
+                fin = np.isfinite(ref if out == "f32" else ref.astype(np.float16)).all(axis=1)
+            assert np.array_equal(np.isfinite(y).all(axis=1), fin)
+            if out == "f32":
+                assert oracle.rel_l2(y[fin], ref[fin]) < 1e-6, (M, oracle.rel_l2(y[fin], ref[fin]))
+                assert np.all(np.abs(y[fin] - ref[fin]) <= np.abs(ref[fin]) * 1e-6 + 1e-6)
+            else:
+                assert np.mean(y[fin].view(np.uint16) != ref[fin].astype(np.float16).view(np.uint16)) < 1e-3   # f32 ties
+                assert oracle.rel_l2(y[fin].astype(np.float32), ref[fin]) < 5e-4
+            # against the unquantised arithmetic on rows that straddle zero: the quantisation noise and nothing else
+            # (the zero-point enters q unrounded and is stored rounded, as in the reference: up to half a step of
+            # offset per row, which weights without a zero-point of their own add up coherently)
+            ok = fin.copy()
+            ok[[8, 9][:max(0, min(2, M - 8))]] = False
+            plain = oracle_y(oracle, c, x=xh[:M])
+            assert oracle.rel_l2(y[ok].astype(np.float32), plain[ok]) < 6e-2
+            assert np.array_equal(req.infer(w, xh[:M]).view(np.uint8), y.view(np.uint8))
+        y = req.infer(w, xh[:32])                 # decode row counts compute in f16: the flag is a permission
+        assert req.last_kernel()["kernel"] == _lib.KERNEL_DECODE
+    finally:
+        w.close()
+
+
+def test_dynquant_asymmetric_with_gated_linear_unit_and_copies(oracle, dev, req, monkeypatch):
+    """The zero-point terms in the gated epilogue (gate and up tiles interleaved: the column sums follow the tiled
+    channel order), and a clone of the node (its column sums are made anew)."""
+    monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
+    c = datagen.make_case(1160, 150, 512, 512, "u8", 512, "u8", with_bias=True)
+    xh = (c.x.astype(np.float32) + 1.5).astype(np.float16)
+    w = fc.CompressedWeights.from_case(dev, c, output_type="f32", glu="swish", dynamic_quantization="asymmetric")
+    w2 = w.clone()
+    try:
+        full = dq_asym_reference(oracle, c, xh)
+        ref = oracle.glu(full, oracle.GLU_SWISH, False)
+        for node in (w, w2):
+            y = req.infer(node, xh)
+            assert req.last_kernel()["name"] == "fcc_prefill_i8_w8_asym"
+            assert y.shape == (150, 256) and oracle.rel_l2(y, ref) < 2e-6
+    finally:
+        w2.close()
+        w.close()

@@ -150,3 +150,86 @@ def test_fc_dynquant_grouped_known_answer(oracle):
     inv1 = float(np.float16(1.0 / float(np.float16(63.5))))
     want = (127 * 2 - 127 * 0) * 0.5 * 1.0 + (127 * 0 + 64 * 3) * 2.0 * inv1
     assert abs(float(y[0, 0]) - want) < 1e-4
+
+
+# ---- asymmetric form: unsigned bytes with a zero-point per token ----
+
+def np_dynquant_asym(x):
+    """Independent restatement in numpy's float16 arithmetic (numpy rounds every half operation once)."""
+    x = np.asarray(x, dtype=np.float16)
+    mx, mn = x.max(axis=1), x.min(axis=1)
+    with np.errstate(over="ignore"):
+        rng_h = (mx - mn).astype(np.float16)                                  # half subtraction
+    diff = np.where(mx == mn, np.float32(np.float16(0.003)), rng_h.astype(np.float32))
+    with np.errstate(divide="ignore"):
+        scale_f = np.float32(255) / diff
+    with np.errstate(over="ignore", invalid="ignore"):
+        scale = scale_f.astype(np.float16)
+        zp = (-mn.astype(np.float32) * scale_f).astype(np.float16)
+    with np.errstate(over="ignore", invalid="ignore"):
+        v = ((x * scale[:, None]).astype(np.float16) + zp[:, None]).astype(np.float16)
+    q = np.nan_to_num(np.rint(v.astype(np.float32)), nan=0.0).clip(0, 255).astype(np.uint8)
+    with np.errstate(divide="ignore"):
+        inv = (np.float32(1) / scale.astype(np.float32)).astype(np.float16).astype(np.float32)
+    za = np.rint(zp.astype(np.float32)).clip(0, 255).astype(np.int32)
+    return q, inv, za, q.astype(np.int32).sum(axis=1).astype(np.int32)
+
+
+def test_dynquant_asym_matches_numpy_half_arithmetic(oracle):
+    rng = np.random.default_rng(21)
+    x = (rng.standard_normal((64, 384)) * rng.uniform(0.01, 30, (64, 1)) + rng.uniform(-3, 3, (64, 1))).astype(np.float16)
+    x[3] = 0                                  # constant rows: d = 0.003
+    x[4, :] = 1e-4
+    x[5, 7] = 65504                           # largest half against ordinary values
+    x[6] = np.abs(x[6]) + np.float16(1)       # all positive: the zero-point leaves 0..255 and is clamped
+    x[7] = -np.abs(x[7]) - np.float16(1)      # all negative
+    q, inv, za, qs = oracle.dynquant_rows_asym(x)
+    q2, inv2, za2, qs2 = np_dynquant_asym(x)
+    assert np.array_equal(q, q2) and np.array_equal(inv, inv2) and np.array_equal(za, za2) and np.array_equal(qs, qs2)
+    assert not q[3].any() and za[3] == 0 and za[6] == 0 and za[7] == 255
+
+
+def test_dynquant_asym_range_and_round_trip(oracle):
+    """Rows that straddle zero: the minimum maps to 0 and the maximum to 255 (within one step: scale and zero-point
+    are rounded to half), every value comes back within half a step plus the half roundings, and the stored scale is
+    the half of (max - min) / 255.  The inputs are those of the reference's own test (uniform in [-16, 20])."""
+    rng = np.random.default_rng(22)
+    x = rng.uniform(-16.0, 20.0, (48, 4096)).astype(np.float16)
+    q, inv, za, qs = oracle.dynquant_rows_asym(x)
+    xf = x.astype(np.float32)
+    lo, hi = xf.min(axis=1), xf.max(axis=1)
+    assert np.all(q[np.arange(48), xf.argmin(axis=1)] <= 1) and np.all(q[np.arange(48), xf.argmax(axis=1)] >= 254)
+    step = (hi - lo) / 255.0
+    assert np.all(np.abs(inv - step) <= step * 2.0 ** -9)
+    assert np.all(np.abs(za - (-lo / step)) <= 1.0)
+    back = (q.astype(np.float32) - za[:, None]) * inv[:, None]
+    # half a step from rounding q, half a step from rounding the zero-point, and 2^-10 of |x scale| and of |zp|
+    # from the two half roundings, in units of a step
+    slack = (1.0 + (np.abs(xf) / step[:, None] + (-lo / step)[:, None]) * 2.0 ** -10 + 0.25) * step[:, None]
+    assert np.all(np.abs(xf - back) <= slack)
+    assert np.array_equal(qs, q.astype(np.int64).sum(axis=1))
+    # exact case: a row of the integers -100 .. 155 has d = 255, scale 1, zero-point 100 and quantises to itself + 100
+    j = np.arange(-100, 156, dtype=np.float32)
+    q1, inv1, za1, qs1 = oracle.dynquant_rows_asym(j.astype(np.float16)[None, :])
+    assert inv1[0] == 1.0 and za1[0] == 100 and np.array_equal(q1[0], (j + 100).astype(np.uint8))
+    assert qs1[0] == int((j + 100).sum())
+
+
+@pytest.mark.parametrize("wt,zt", [("u8", "u8"), ("u8", "none"), ("i8", "none")])
+def test_fc_dynquant_asym_equals_float_oracle_on_dequantised_activations(oracle, wt, zt):
+    """sum (q - za)(w - zp) s inv == FC((q - za) inv): the integer form and the float oracle agree on the same
+    dequantised activations, which fixes every cross term; against the unquantised result the difference is the
+    quantisation noise (the zero-point enters q unrounded and is stored rounded, as in the reference: up to half
+    a step of offset per row on top of the rounding of q)."""
+    c = datagen.make_case(33, 24, 512, 96, wt, 512, zt, with_bias=True)
+    x = (c.x.astype(np.float32) + np.linspace(-2, 2, 24, dtype=np.float32)[:, None]).astype(np.float16)
+    T = {"u8": oracle.U8, "i8": oracle.I8}
+    zp = None if c.zp is None else c.zp.astype(np.float32)
+    y = oracle.fc_dynquant_asym_reference(x, c.w, T[wt], c.scale, zp, c.bias, N=c.N, K=c.K)
+    q, inv, za, _ = oracle.dynquant_rows_asym(x)
+    xd = ((q.astype(np.float32) - za[:, None].astype(np.float32)) * inv[:, None]).astype(np.float32)
+    zt_code = oracle.U8 if zt == "u8" else oracle.NONE
+    ref = oracle.fc_reference(xd, c.w, T[wt], c.scale, c.zp, zt_code, c.bias, N=c.N, K=c.K, group_size=c.K, acc_f64=True)
+    assert oracle.rel_l2(y, ref) < 2e-6
+    plain = oracle.fc_reference(x, c.w, T[wt], c.scale, c.zp, zt_code, c.bias, N=c.N, K=c.K, group_size=c.K)
+    assert 1e-4 < oracle.rel_l2(y, plain) < 3e-2
