@@ -287,6 +287,35 @@ def test_gemv16_streamed_activations(oracle, dev, req, monkeypatch, wt, zt, N, K
         w.close()
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_gemv16_streamed_random_nodes(oracle, dev, req, monkeypatch, seed):
+    """Seeded sweep of the streaming kernel: formats, K and its division over the waves, channel counts, row counts,
+    bias and output type that the table above does not pair up."""
+    rng = np.random.default_rng(7460 + seed)
+    monkeypatch.setenv("OVFCC_GEMV16_STREAM", "1")
+    for _ in range(4):
+        C = int(rng.choice([2, 4, 8]))
+        waves = int(rng.integers(1, 17))
+        K = 128 * C * waves
+        wt = str(rng.choice(["u4", "i4"]))
+        zt = str(rng.choice(["none", "u4", "u8"])) if wt == "u4" else "none"
+        N = 16 * int(rng.integers(1, 40))
+        M = int(rng.integers(5, 17))
+        bias, out = bool(rng.integers(0, 2)), str(rng.choice(["f16", "f32"]))
+        monkeypatch.setenv("OVFCC_GEMV_C", str(C))
+        what = f"seed {seed}: {wt}/{zt} N={N} K={K} C={C} waves={waves} M={M} bias={bias} out={out}"
+        say(what)
+        c = datagen.make_case(int(rng.integers(1, 1 << 30)), M, K, N, wt, 128, zt, with_bias=bias)
+        w = fc.CompressedWeights.from_case(dev, c, output_type=out)
+        try:
+            y = req.infer(w, c.x)
+            info = req.last_kernel()
+            assert info["name"] == "fcc_gemv16s_w4" and info["block"] == 64 * waves and info["grid"] == (N // 16, 1, 1), (what, info)
+            check_parity(oracle, y, oracle_y(oracle, c), K, f"{what} {info}", output_rounding_slack=True)
+        finally:
+            w.close()
+
+
 def test_gemv16_streamed_tiny_and_huge_activations(oracle, dev, req, monkeypatch):
     """Subnormal activations, activations near the top of the half range and a row of zeros through the streaming
     kernel (same arithmetic as the stationary one: half of the activations are multiplied by 2^-4 in registers)."""
