@@ -15,8 +15,9 @@
 // activations of k-blocks 0 and 1, then the weights of the first four k-blocks; after k-block s is multiplied, the
 // activations of k-block s + 2 go into the buffer it has freed and the weights of k-block s + 4 are requested.  The
 // wait before the LDS reads of k-block s counts the loads issued behind its activations (loads_after_x); scheduling
-// barriers keep the compiler from moving loads across those points, and rows beyond M are loaded out of range (zeros)
-// rather than skipped, so that the count never depends on M.  The compiler waits for the weight registers itself.
+// barriers keep the compiler from moving loads across those points.  The count must not depend on M at run time: the
+// kernel exists for 8, 12 and 16 rows of activations per k-block (two, three or four loads; a load costs its issue
+// cycles wherever its lanes point), and within those, rows beyond M are loaded out of range (zeros) rather than skipped.  The compiler waits for the weight registers itself.
 //
 // LDS buffer of a wave, in 16-byte units: row r, chunk c of the k-block's 16 sits at 16 r + (c ^ r): the sixteen rows
 // that one operand read touches lie in sixteen different bank groups.  Arithmetic as in the 16-row kernel: nibbles
@@ -52,16 +53,16 @@ constexpr int weights_ahead() {
     return C < 4 ? C : 4;
 }
 
-// vector-memory loads a wave has issued behind the four loads of k-block s's activations when it is about to read
+// vector-memory loads a wave has issued behind the XL loads of k-block s's activations when it is about to read
 // them: the order is X0, X1, W0 .. W(D-1), then after every k-block t: X(t+2), W(t+D)
-template <int C>
+template <int C, int XL>
 constexpr int loads_after_x(int s) {
     constexpr int D = weights_ahead<C>();
     int count = 0;
     bool seen = false;
     for (int i = 0; i < 2 && i < C; ++i) {
         if (seen)
-            count += 4;
+            count += XL;
         if (i == s)
             seen = true;
     }
@@ -71,7 +72,7 @@ constexpr int loads_after_x(int s) {
     for (int t = 0; t < s; ++t) {
         if (t + 2 < C) {
             if (seen)
-                count += 4;
+                count += XL;
             if (t + 2 == s)
                 seen = true;
         }
@@ -89,7 +90,10 @@ __device__ __forceinline__ void for_each_slot(F&& f, std::integer_sequence<int, 
 }
 }  // namespace
 
-template <int C, bool ZP_TABLE>
+// XL: direct-to-LDS loads per k-block of activations, four rows each (2, 3 or 4: rows beyond 4 XL are never loaded --
+// a load costs its 16 cycles of the address path wherever its lanes point -- and what is computed from them is
+// never stored)
+template <int C, bool ZP_TABLE, int XL>
 __global__ __launch_bounds__(1024) void fcc_gemv16s_kernel(const uint4_t* __restrict__ wt, const half_t* __restrict__ scale_cm,
                                                            const uint8_t* __restrict__ zp_cm, const half_t* __restrict__ x,
                                                            const half_t* __restrict__ bias, void* __restrict__ y, int M,
@@ -149,7 +153,7 @@ __global__ __launch_bounds__(1024) void fcc_gemv16s_kernel(const uint4_t* __rest
     auto load_x = [&](int s) {
         const int kb = wave + waves * s;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < XL; ++q) {
             const int row = 4 * q + kq;
             const int chunk = col ^ row;  // the chunk of the row that belongs in this lane's linear slot
             const unsigned ofs = ((unsigned)((m0 + row) * K + kb * 128 + chunk * 8) * 2u) |
@@ -183,7 +187,7 @@ __global__ __launch_bounds__(1024) void fcc_gemv16s_kernel(const uint4_t* __rest
     auto step = [&](auto slot) {
         constexpr int s = decltype(slot)::value;
         // the activations of this k-block have landed (and with them everything requested before them)
-        __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(loads_after_x<C>(s)));
+        __builtin_amdgcn_s_waitcnt(wait_vmcnt_imm(loads_after_x<C, XL>(s)));
         asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         const lds_byte_ptr xs_lane = lds3 + wave * (2 * kBufBytes) + (s & 1) * kBufBytes + col * 256;
@@ -274,10 +278,10 @@ size_t gemv16s_lds_bytes(int waves) {
     return (size_t)waves * (2 * 4096 + 1024);
 }
 
-template <int C, bool ZPT>
-static int launch_gemv16s_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+template <int C, bool ZPT, int XL>
+static int launch_gemv16s_rows(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
     const Layout& L = a.layout;
-    auto kern = fcc_gemv16s_kernel<C, ZPT>;
+    auto kern = fcc_gemv16s_kernel<C, ZPT, XL>;
     static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats it
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -290,6 +294,14 @@ static int launch_gemv16s_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipSt
                        (const half_t*)a.scale_cm, (const uint8_t*)a.zp_cm, (const half_t*)a.x, (const half_t*)a.bias, a.y,
                        (int)a.M, (int)a.N, (int)a.K, (int)L.k_blocks, (int)L.n_tiles, L.zp_const, a.out_f32);
     return (int)hipGetLastError();
+}
+
+template <int C, bool ZPT>
+static int launch_gemv16s_impl(const FcDeviceArgs& a, const LaunchPlan& p, hipStream_t s) {
+    // one row tile: as many four-row loads as M needs; several row tiles: all four
+    const int xl = a.M > 12 ? 4 : a.M > 8 ? 3 : 2;
+    return xl == 4 ? launch_gemv16s_rows<C, ZPT, 4>(a, p, s)
+                   : xl == 3 ? launch_gemv16s_rows<C, ZPT, 3>(a, p, s) : launch_gemv16s_rows<C, ZPT, 2>(a, p, s);
 }
 
 int launch_gemv16_stream(const FcDeviceArgs& a, const LaunchPlan& p, void* stream) {

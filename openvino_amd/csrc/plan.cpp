@@ -237,8 +237,8 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
     // for all of its activations first: the 16-row kernel that streams its activations k-block by k-block, one
     // workgroup per channel tile over all of K -- no split along K, no second launch (4096 -> 4096 at 16 rows:
     // 4.8 against 5.4 us; 14336 -> 4096 at 8 rows: 10.1 against 12.4 us for the small-batch kernel, at 16 rows 12.1
-    // against 12.7).  It needs about as many channel tiles as compute units to fill the chip (1024 channels: a tie),
-    // and from 17 rows on every tile's weights would be streamed twice.  OVFCC_GEMV16_STREAM = 0 switches it off, = 1 takes
+    // against 12.7; 4096 -> 1024, a quarter of the compute units: 3.75-4.7 against 3.9-4.8).  From 17 rows on every
+    // tile's weights would be streamed twice.  OVFCC_GEMV16_STREAM = 0 switches it off, = 1 takes
     // it wherever it can run (before the kernel above, and whatever the number of channel tiles).
     const int stream_env = env_int("OVFCC_GEMV16_STREAM", -1);
     auto plan_gemv16_stream = [&]() -> bool {
@@ -248,7 +248,7 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             env_int("OVFCC_DECODE_BATCH", -1) >= 0 || L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 31))
             return false;
         const int waves = (int)(L.k_blocks / L.gemv_c);
-        if (L.k_blocks % L.gemv_c != 0 || waves < 1 || waves > 16 || (stream_env != 1 && L.n_tiles * 2 < n_cus) ||
+        if (L.k_blocks % L.gemv_c != 0 || waves < 1 || waves > 16 || (stream_env != 1 && L.n_tiles * 4 < n_cus) ||
             gemv16s_lds_bytes(waves) > 160 * 1024 - 64)
             return false;
         p.gemv16_stream = true;

@@ -134,8 +134,8 @@ def test_gemv16_benchmark_nodes(oracle, dev, req, name, N, K):
             say(f"gemv16 {name} M={M}")
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
-            # as many channel tiles as compute units and one row tile: nothing to keep, the activations are streamed
-            streamed = name == "q/o" and M <= 16
+            # no more channel tiles than compute units and one row tile: nothing to keep, the activations are streamed
+            streamed = name in ("q/o", "k/v") and M <= 16
             assert info["name"] == ("fcc_gemv16s_w4" if streamed else "fcc_gemv16_w4"), info
             check_parity(oracle, y[:, cols], ref[:M], K, f"{name} M={M} {info}")
     finally:
