@@ -185,7 +185,7 @@ int launch_gemv(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_gemv16(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 int launch_gemv16_stream(const FcDeviceArgs& a, const LaunchPlan& plan, void* stream);
 // dynamic LDS of the 16-row kernel with streamed activations
-size_t gemv16s_lds_bytes(int waves);
+size_t gemv16s_lds_bytes(int waves, int tiles);
 // dynamic LDS of the 16-row kernel: c k-blocks per wave, `waves` waves, one or two buffers of partial sums
 size_t gemv16_lds_bytes(int c, int waves, int red_bufs);
 // k-blocks per wave that the 16-row kernel runs a node with, given those of the node's channel-major tables and the

@@ -36,7 +36,7 @@ struct EnvEntry {
 EnvEntry g_env[] = {EnvEntry("OVFCC_DECODE_WAVES"),   EnvEntry("OVFCC_DECODE_RT"),      EnvEntry("OVFCC_DECODE_XLDS"),
                     EnvEntry("OVFCC_DECODE_BATCH"),   EnvEntry("OVFCC_GEMV"),           EnvEntry("OVFCC_GEMV_C"),
                     EnvEntry("OVFCC_GEMV16"),         EnvEntry("OVFCC_GEMV16_GRID"),    EnvEntry("OVFCC_GEMV16_SPLIT"),
-                    EnvEntry("OVFCC_GEMV16_STREAM"),
+                    EnvEntry("OVFCC_GEMV16_STREAM"),  EnvEntry("OVFCC_GEMV16_STREAM_TILES"),
                     EnvEntry("OVFCC_PREFILL_DIRECT"), EnvEntry("OVFCC_PREFILL_ASYNC"),  EnvEntry("OVFCC_PREFILL_WIDE"),
                     EnvEntry("OVFCC_PREFILL_BIG"),    EnvEntry("OVFCC_PREFILL_TAIL"),   EnvEntry("OVFCC_PREFILL_ROWS"),
                     EnvEntry("OVFCC_MOE_HOST_ROUTING"), EnvEntry("OVFCC_MLP_FUSED"),      EnvEntry("OVFCC_MLP_SPIN_LIMIT"),
@@ -241,6 +241,16 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
     // tile's weights would be streamed twice.  OVFCC_GEMV16_STREAM = 0 switches it off, = 1 takes
     // it wherever it can run (before the kernel above, and whatever the number of channel tiles).
     const int stream_env = env_int("OVFCC_GEMV16_STREAM", -1);
+    // Channel tiles per workgroup (their activations travel once for all of them): two where the node has more
+    // tiles than the chip has compute units; OVFCC_GEMV16_STREAM_TILES = 1 | 2 | 4 overrides.  Measured against the
+    // kernel above (8 / 16 rows): 4096 -> 8192 5.96 / 6.55 against 6.92 / 7.71 us, 4096 -> 6144 5.51 / 6.02 against
+    // 6.53 / 7.22, 8192 -> 8192 9.08 / 10.29 against 11.90 / 12.45 (K in two parts and a summing launch) -- one round
+    // of workgroups, taken up to 16 rows; 4096 -> 14336 (448 workgroups) 8.60 / 9.90 against 9.19 / 9.96 -- taken up
+    // to 8 rows; 4096 -> 28672 (896 workgroups) 14.7 against 13.3 -- left to the kernel above.
+    const int stream_tiles =
+        env_int("OVFCC_GEMV16_STREAM_TILES", L.n_tiles > n_cus && L.n_tiles % 2 == 0 ? 2 : 1);
+    const int64_t stream_wgs = L.n_tiles / (stream_tiles == 2 || stream_tiles == 4 ? stream_tiles : 1);
+    const bool stream_first = stream_env == 1 || stream_wgs <= n_cus || (stream_wgs <= 2 * (int64_t)n_cus && a.M <= 8);
     auto plan_gemv16_stream = [&]() -> bool {
         if (a.M <= 4 || a.M > 16 || !a.scale_cm || L.bits != 4 || L.groups_per_kblock != 1 || L.kblocks_per_group != 1 ||
             force_split > 0 || L.gemv_c == 0 || L.glu || env_int("OVFCC_GEMV16", 1) == 0 ||
@@ -248,21 +258,27 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
             env_int("OVFCC_DECODE_BATCH", -1) >= 0 || L.n_tiles * L.k_blocks * kTileBytes >= ((int64_t)1 << 31))
             return false;
         const int waves = (int)(L.k_blocks / L.gemv_c);
-        if (L.k_blocks % L.gemv_c != 0 || waves < 1 || waves > 16 || (stream_env != 1 && L.n_tiles * 4 < n_cus) ||
-            gemv16s_lds_bytes(waves) > 160 * 1024 - 64)
+        if (L.k_blocks % L.gemv_c != 0 || waves < 1 || waves > 16 || (stream_env != 1 && L.n_tiles * 4 < n_cus))
+            return false;
+        int tiles = stream_tiles;
+        if ((tiles != 1 && tiles != 2 && tiles != 4) || L.n_tiles % tiles != 0)
+            tiles = 1;
+        while (tiles > 1 && gemv16s_lds_bytes(waves, tiles) > 160 * 1024 - 64)
+            tiles >>= 1;
+        if (gemv16s_lds_bytes(waves, tiles) > 160 * 1024 - 64)
             return false;
         p.gemv16_stream = true;
         p.gemv_c = L.gemv_c;
         p.split_k = 1;
         p.kblocks_per_split = (int)L.k_blocks;
-        p.tiles_per_group = 1;
-        p.grid[0] = (unsigned)L.n_tiles;
+        p.tiles_per_group = tiles;
+        p.grid[0] = (unsigned)(L.n_tiles / tiles);
         p.grid[1] = 1;
         p.grid[2] = 1;
         p.block = 64u * waves;
         p.tile_m = 16;
         p.tile_n = 16;
-        p.dynamic_lds = (unsigned)gemv16s_lds_bytes(waves);
+        p.dynamic_lds = (unsigned)gemv16s_lds_bytes(waves, tiles);
         p.workspace_bytes = 0;
         p.name = "fcc_gemv16s_w4";
         return true;
@@ -274,7 +290,7 @@ int plan_launch(const FcDeviceArgs& a, int force_kernel, int force_split, int n_
         p.grid[1] = (unsigned)a.M;
         p.block = 64;
         p.name = "fcc_plain";
-    } else if (kernel == OVFCC_KERNEL_DECODE && (((stream_env == 1 || L.n_tiles <= n_cus) && plan_gemv16_stream()) || plan_gemv16() || plan_gemv16_stream())) {
+    } else if (kernel == OVFCC_KERNEL_DECODE && ((stream_first && plan_gemv16_stream()) || plan_gemv16() || plan_gemv16_stream())) {
         // planned
     } else if (kernel == OVFCC_KERNEL_DECODE && want_batch) {
         if (int rc = plan_batch())

@@ -121,9 +121,10 @@ static void check_plan(const ovfcc_fc_desc& d, int64_t M, int force, int force_s
             CHECK(M > 4 && M <= 16 && L.bits == 4 && L.groups_per_kblock == 1 && L.kblocks_per_group == 1 && c == L.gemv_c && !L.glu,
                   "%s", what);
             CHECK((c == 2 || c == 4 || c == 8) && kb % c == 0 && nw == kb / c && nw <= 16, "%s c=%d nw=%d", what, c, nw);
-            CHECK((int64_t)p.grid[0] == L.n_tiles && p.grid[1] == 1 && p.grid[2] == 1 && p.split_k == 1 && p.workspace_bytes == 0,
-                  "%s grid=%u", what, p.grid[0]);
-            CHECK(p.dynamic_lds == ovfcc::gemv16s_lds_bytes(nw) && p.dynamic_lds <= 160 * 1024 - 64, "%s lds=%u", what, p.dynamic_lds);
+            CHECK((rt == 1 || rt == 2 || rt == 4) && (int64_t)p.grid[0] * rt == L.n_tiles && p.grid[1] == 1 && p.grid[2] == 1 &&
+                      p.split_k == 1 && p.workspace_bytes == 0,
+                  "%s grid=%u tiles=%d", what, p.grid[0], rt);
+            CHECK(p.dynamic_lds == ovfcc::gemv16s_lds_bytes(nw, rt) && p.dynamic_lds <= 160 * 1024 - 64, "%s lds=%u", what, p.dynamic_lds);
         } else if (p.batch) {
             const int mt = (int)(M + 15) / 16;
             CHECK(p.tile_m == 16 * mt && (rt == 1 || rt == 2), "%s", what);

@@ -134,8 +134,8 @@ def test_gemv16_benchmark_nodes(oracle, dev, req, name, N, K):
             say(f"gemv16 {name} M={M}")
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
-            # no more channel tiles than compute units and one row tile: nothing to keep, the activations are streamed
-            streamed = name in ("q/o", "k/v") and M <= 16
+            # one round of workgroups (two for up to 8 rows) and one row tile: the activations are streamed
+            streamed = (name in ("q/o", "k/v") and M <= 16) or (name == "gate/up" and M <= 8)
             assert info["name"] == ("fcc_gemv16s_w4" if streamed else "fcc_gemv16_w4"), info
             check_parity(oracle, y[:, cols], ref[:M], K, f"{name} M={M} {info}")
     finally:
@@ -252,19 +252,23 @@ STREAM_SHAPES = [
     ("i4", "none", 48, 2048, 4, True, "f16"),    # 4 waves of 4; symmetric weights (zero-point 8 as a constant)
     ("u4", "u8", 96, 4096, 8, True, "f16"),      # 8-bit zero-point table, two words per channel and wave
     ("u4", "none", 32, 256, 2, True, "f32"),     # 1 wave, 2 k-blocks, no zero-point
-    ("u4", "u4", 80, 14336, 8, False, "f32"),    # the down projection's K: 14 waves, 126 KiB of LDS
+    ("u4", "u4", 80, 14336, 8, False, "f32"),    # the down projection's K: 14 waves, 112 KiB of LDS
     ("i4", "none", 64, 14336, 8, True, "f16"),
-    ("u4", "u4", 64, 4096, 2, True, "f16"),      # 16 waves: the largest workgroup, 144 KiB of LDS
+    ("u4", "u4", 64, 4096, 2, True, "f16"),      # 16 waves: the largest workgroup, 128 KiB of LDS
 ]
 
 
+@pytest.mark.parametrize("tiles", [1, 2, 4])
 @pytest.mark.parametrize("wt,zt,N,K,C,bias,out", STREAM_SHAPES)
-def test_gemv16_streamed_activations(oracle, dev, req, monkeypatch, wt, zt, N, K, C, bias, out):
+def test_gemv16_streamed_activations(oracle, dev, req, monkeypatch, wt, zt, N, K, C, bias, out, tiles):
     """The 16-row kernel that streams its activations through a double buffer per wave, taken wherever it can run
     (OVFCC_GEMV16_STREAM = 1): every division of K over the waves, rows short of a tile (loaded out of range, so
     that the count of loads in flight does not depend on M) and a whole tile, the same bits on every repetition."""
     monkeypatch.setenv("OVFCC_GEMV_C", str(C))
     monkeypatch.setenv("OVFCC_GEMV16_STREAM", "1")
+    monkeypatch.setenv("OVFCC_GEMV16_STREAM_TILES", str(tiles))   # channel tiles per workgroup, where N divides
+    if (N // 16) % tiles:
+        tiles = 1
     c = datagen.make_case(7450 + N + K, 16, K, N, wt, 128, zt, with_bias=bias)
     w = fc.CompressedWeights.from_case(dev, c, output_type=out)
     ref = oracle_y(oracle, c)
@@ -274,7 +278,7 @@ def test_gemv16_streamed_activations(oracle, dev, req, monkeypatch, wt, zt, N, K
             y = req.infer(w, c.x[:M])
             info = req.last_kernel()
             assert info["name"] == "fcc_gemv16s_w4" and info["block"] == 64 * (K // 128 // C), info
-            assert info["grid"] == (N // 16, 1, 1) and info["split_k"] == 1, info
+            assert info["grid"] == (N // 16 // tiles, 1, 1) and info["split_k"] == 1, info
             assert y.dtype == (np.float32 if out == "f32" else np.float16)
             check_parity(oracle, y, ref[:M], K, f"M={M} {info}", output_rounding_slack=True)
             for _ in range(3):    # partial sums are added in wave order
@@ -302,16 +306,45 @@ def test_gemv16_streamed_random_nodes(oracle, dev, req, monkeypatch, seed):
         N = 16 * int(rng.integers(1, 40))
         M = int(rng.integers(5, 17))
         bias, out = bool(rng.integers(0, 2)), str(rng.choice(["f16", "f32"]))
+        tiles = int(rng.choice([1, 2, 4]))
         monkeypatch.setenv("OVFCC_GEMV_C", str(C))
-        what = f"seed {seed}: {wt}/{zt} N={N} K={K} C={C} waves={waves} M={M} bias={bias} out={out}"
+        monkeypatch.setenv("OVFCC_GEMV16_STREAM_TILES", str(tiles))
+        if (N // 16) % tiles:
+            tiles = 1
+        what = f"seed {seed}: {wt}/{zt} N={N} K={K} C={C} waves={waves} tiles={tiles} M={M} bias={bias} out={out}"
         say(what)
         c = datagen.make_case(int(rng.integers(1, 1 << 30)), M, K, N, wt, 128, zt, with_bias=bias)
         w = fc.CompressedWeights.from_case(dev, c, output_type=out)
         try:
             y = req.infer(w, c.x)
             info = req.last_kernel()
-            assert info["name"] == "fcc_gemv16s_w4" and info["block"] == 64 * waves and info["grid"] == (N // 16, 1, 1), (what, info)
+            assert info["name"] == "fcc_gemv16s_w4" and info["block"] == 64 * waves, (what, info)
+            assert info["grid"] == (N // 16 // tiles, 1, 1), (what, info)
             check_parity(oracle, y, oracle_y(oracle, c), K, f"{what} {info}", output_rounding_slack=True)
+        finally:
+            w.close()
+
+
+def test_gemv16_streamed_two_tiles_by_policy(oracle, dev, req):
+    """More channel tiles than compute units: two tiles per workgroup share a k-block of activations.  One round of
+    workgroups (4096 -> 8192: 512 tiles, 256 workgroups) is taken up to 16 rows, more than one (4096 -> 14336: 448
+    workgroups) up to 8."""
+    for N, rows in ((8192, (5, 8, 16)), (14336, (8,))):
+        K = 4096
+        c = datagen.make_case(7880 + N, 16, K, N, "u4", 128, "u4", with_bias=True)
+        w = fc.CompressedWeights.from_case(dev, c)
+        cols = np.sort(np.random.default_rng(8).choice(N, size=256, replace=False))
+        ref = oracle_y(oracle, c, n_index=cols)
+        try:
+            for M in rows:
+                y = req.infer(w, c.x[:M])
+                info = req.last_kernel()
+                say(f"gemv16s two tiles N={N} M={M} {info}")
+                assert info["name"] == "fcc_gemv16s_w4" and info["grid"] == (N // 32, 1, 1), info
+                check_parity(oracle, y[:, cols], ref[:M], K, f"N={N} M={M} {info}")
+            y = req.infer(w, c.x[:16])
+            if N == 14336:
+                assert req.last_kernel()["name"] == "fcc_gemv16_w4", req.last_kernel()
         finally:
             w.close()
 
