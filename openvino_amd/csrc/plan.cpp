@@ -21,7 +21,8 @@ namespace ovfcc {
 //            (small-batch kernel instead of the streaming kernel), OVFCC_GEMV = 0 | 1, OVFCC_GEMV_C = 2 | 4 | 8,
 //            OVFCC_GEMV16 = 0 | 1 (the 16-row kernel with stationary activations for 5-48 rows),
 //            OVFCC_GEMV16_GRID = n (its workgroups per row tile), OVFCC_GEMV16_SPLIT = 1 | 2 | 4 | 8 (parts it cuts K in),
-//            OVFCC_GEMV16_STREAM = 0 | 1 (the 16-row kernel that streams its activations, for long K at 5-16 rows),
+//            OVFCC_GEMV16_STREAM = 0 | 1 (the 16-row kernel that streams its activations, 5-16 rows),
+//            OVFCC_GEMV16_STREAM_TILES = 1 | 2 | 4 (its channel tiles per workgroup),
 //            OVFCC_PREFILL_{DIRECT, ASYNC, WIDE, BIG, TAIL} = 0 | 1, OVFCC_PREFILL_ROWS = 64 | 128,
 //            OVFCC_MOE_HOST_ROUTING = 1, OVFCC_MLP_FUSED = 1 (an MLP node of up to four rows as one launch instead of two),
 //            OVFCC_MLP_GRID = n (its workgroups), OVFCC_MLP_SPIN_LIMIT = n (polls after which that launch's wait for its workgroups gives up; tests);
