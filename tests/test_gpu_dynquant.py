@@ -277,19 +277,24 @@ def test_dynquant_asymmetric_matches_integer_oracle(oracle, dev, req, monkeypatc
 
 def test_dynquant_asymmetric_with_gated_linear_unit_and_copies(oracle, dev, req, monkeypatch):
     """The zero-point terms in the gated epilogue (gate and up tiles interleaved: the column sums follow the tiled
-    channel order), and a clone of the node (its column sums are made anew)."""
+    channel order), a clone of the node and a node imported from its blob (their column sums are made anew)."""
     monkeypatch.setenv("OVFCC_PREFILL_WIDE", "1")
     c = datagen.make_case(1160, 150, 512, 512, "u8", 512, "u8", with_bias=True)
     xh = (c.x.astype(np.float32) + 1.5).astype(np.float16)
     w = fc.CompressedWeights.from_case(dev, c, output_type="f32", glu="swish", dynamic_quantization="asymmetric")
     w2 = w.clone()
+    w3 = fc.CompressedWeights.import_blob(dev, w.export_blob())   # ... and so does a node that comes back from its blob
     try:
         full = dq_asym_reference(oracle, c, xh)
         ref = oracle.glu(full, oracle.GLU_SWISH, False)
-        for node in (w, w2):
+        first = None
+        for node in (w, w2, w3):
             y = req.infer(node, xh)
             assert req.last_kernel()["name"] == "fcc_prefill_i8_w8_asym"
             assert y.shape == (150, 256) and oracle.rel_l2(y, ref) < 2e-6
+            first = y if first is None else first
+            assert np.array_equal(y.view(np.uint8), first.view(np.uint8))
     finally:
+        w3.close()
         w2.close()
         w.close()
