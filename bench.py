@@ -423,6 +423,14 @@ def floors_table(dev, req, args) -> int:
             tf = max(dev.mfma_ceiling(waves, valu, shape=shape) for _ in range(2))
             print(f"| {name}, {waves // 4} wave(s) per SIMD, {valu} packed-f16 multiplications per 16 x 16 x 32 of "
                   f"matrix work | {tf:.0f} | {100 * tf / 2500:.1f} % |")
+    # ... and how that depends on what the weight operand looks like (activation operand random halves)
+    print("\n| v_mfma_f32_16x16x32_f16 on registers, two waves per SIMD, all compute units; one operand random halves, "
+          "the other: | TFLOP/s | of 2.5 PFLOP/s |")
+    print("|---|---|---|")
+    for shape, name in ((0, "random halves too"), (4, "integers -8 .. 7 times a scale, rounded to half (what the prefill kernels feed)"),
+                        (2, "integers -8 .. 7 as halves"), (3, "integers 0 .. 15 as subnormal halves (what the decode kernels feed)")):
+        tf = max(dev.mfma_ceiling(8, 0, shape=shape) for _ in range(3))
+        print(f"| {name} | {tf:.0f} | {100 * tf / 2500:.1f} % |")
     # how one SIMD overlaps matrix-core and vector instructions, in shader cycles: one compute unit alone, then all
     n_cus = 256
     print("\n| matrix-core loop with vector instructions after every MFMA (v_mfma_f32_16x16x32_f16, two waves per SIMD) | "

@@ -44,7 +44,10 @@ int ovfcc_bench_floor(ovfcc_ctx* ctx, const void* arena_dev, size_t arena_bytes,
  * v_mfma_f32_32x32x16_f16 (shape 1; the same matrix-core work) on registers, each followed by `valu` (0..4; twice
  * that for shape 1) packed-f16 vector multiplications on other registers; no memory traffic.  Timed with HIP
  * events; *flops is the matrix-core work of the timed launch.  What the chip sustains under that load (it lowers
- * its clock) is the ceiling the prefill kernels are measured against beside the nominal peak. */
+ * its clock) is the ceiling the prefill kernels are measured against beside the nominal peak.  Both operands are
+ * random halves; shapes 2, 3 and 4 (valu = 0) are shape 0 with the second operand looking like weights instead:
+ * integers -8 .. 7 as halves, the integers 0 .. 15 as subnormal halves, integers -8 .. 7 times a scale rounded to
+ * half -- the sustained rate depends on how many operand bits toggle. */
 int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int shape, int rounds, float* elapsed_ms, double* flops);
 
 /* How one SIMD overlaps matrix-core and vector instructions: `workgroups` workgroups (1: one compute unit alone, no

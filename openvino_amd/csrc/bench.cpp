@@ -153,7 +153,7 @@ int ovfcc_bench_copy(ovfcc_ctx* ctx, void* dst_dev, const void* src_dev, size_t 
 
 int ovfcc_bench_mfma(ovfcc_ctx* ctx, int waves, int valu, int shape, int rounds, float* elapsed_ms, double* flops) {
     if (!ctx || !elapsed_ms || !flops || rounds <= 0 || (waves != 4 && waves != 8) || valu < 0 || valu > 4 ||
-        shape < 0 || shape > 1)
+        shape < 0 || shape > 4 || (shape >= 2 && valu != 0))
         return fail(OVFCC_EINVAL, "bad matrix-core benchmark arguments");
     HIP_TRY(hipSetDevice(ctx->device));
     Held h;

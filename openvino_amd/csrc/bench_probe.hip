@@ -151,13 +151,63 @@ __global__ __launch_bounds__(512) void fcc_mfma32_probe_kernel(float* __restrict
     sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// What the weight operand looks like to the matrix cores, with the activation operand random as above: PATTERN 1
+// small integers -8 .. 7 as halves (a 4-bit weight minus its zero-point, unscaled), 2 the integers 0 .. 15 in the low
+// mantissa bits of subnormal halves (what the decode kernels feed), 3 integers -8 .. 7 times a scale between 0.002 and
+// 0.02 rounded to half (what the prefill kernels feed).  The chip's clock under this load depends on how many operand
+// bits toggle.
+__device__ __forceinline__ half8_t probe_weight_operand(unsigned seed, int pattern) {
+    half8_t v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        unsigned h = (seed * 8u + e) * 2654435761u;
+        h ^= h >> 15, h *= 2246822519u, h ^= h >> 13;
+        const int w = (int)(h & 15u);
+        if (pattern == 1)
+            v[e] = (half_t)(float)(w - 8);
+        else if (pattern == 2)
+            v[e] = __builtin_bit_cast(half_t, (uint16_t)w);
+        else
+            v[e] = (half_t)((float)(w - 8) * (0.002f + 0.018f * (float)((seed >> 3) & 63u) / 63.f));
+    }
+    return v;
+}
+
+__global__ __launch_bounds__(512) void fcc_mfma_pattern_probe_kernel(float* __restrict__ sink, int iters, int pattern) {
+    half8_t a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a[i] = probe_operand(threadIdx.x * 8u + i);
+        b[i] = probe_weight_operand(threadIdx.x * 8u + 4u + i, pattern);
+    }
+    float4_t acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        acc[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[j]) : "v"(a[j & 3]), "v"(b[(j >> 1) & 3]));
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        s += acc[i].x + acc[i].y + acc[i].z + acc[i].w;
+    sink[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 // sink: 4 * workgroups * 64 * waves bytes.  valu: 0 to 4 multiplications after every MFMA.  shape 0: 16 x 16 x 32
-// instructions, shape 1: 32 x 32 x 16.
+// instructions, shape 1: 32 x 32 x 16; shapes 2, 3, 4: 16 x 16 x 32 with weight-operand pattern 1, 2, 3 (valu = 0).
 int launch_mfma_probe(float* sink, int workgroups, int waves, int valu, int shape, int iters, void* stream) {
-    if (!sink || workgroups < 1 || (waves != 4 && waves != 8) || valu < 0 || valu > 4 || iters < 1 || shape < 0 || shape > 1)
+    if (!sink || workgroups < 1 || (waves != 4 && waves != 8) || valu < 0 || valu > 4 || iters < 1 || shape < 0 || shape > 4 ||
+        (shape >= 2 && valu != 0))
         return (int)hipErrorInvalidValue;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 g((unsigned)workgroups), b(64u * waves);
+    if (shape >= 2) {
+        hipLaunchKernelGGL(fcc_mfma_pattern_probe_kernel, g, b, 0, s, sink, iters, shape - 1);
+        return (int)hipGetLastError();
+    }
     if (shape == 1) {
         switch (valu) {
         case 0: hipLaunchKernelGGL(fcc_mfma32_probe_kernel<0>, g, b, 0, s, sink, iters); break;
