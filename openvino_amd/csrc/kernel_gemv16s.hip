@@ -20,7 +20,8 @@
 // wait before the LDS reads of k-block s counts the loads issued behind its activations (loads_after_x); scheduling
 // barriers keep the compiler from moving loads across those points.  The count must not depend on M at run time: the
 // kernel exists for 8, 12 and 16 rows of activations per k-block (two, three or four loads; a load costs its issue
-// cycles wherever its lanes point), and within those, rows beyond M are loaded out of range (zeros) rather than skipped.  The compiler waits for the weight registers itself.
+// cycles wherever its lanes point), and within those, rows beyond M are loaded out of range (zeros) rather than
+// skipped.  The compiler waits for the weight registers itself.
 //
 // LDS buffer of a wave, in 16-byte units: row r, chunk c of the k-block's 16 sits at 16 r + (c ^ r): the sixteen rows
 // that one operand read touches lie in sixteen different bank groups.  Arithmetic as in the 16-row kernel: nibbles
