@@ -114,7 +114,7 @@ typedef struct ovfcc_fc_desc {
  * cl_kernels/dynamic_quantize_gpu_ref.cl:100-250 with ASYMMETRIC_QUANTIZATION and UNSIGNED_OUTPUT; consumed as the
  * source zero-point of the matrix product, src/plugins/intel_gpu/src/graph/impls/onednn/fully_connected_onednn.cpp:
  * 83-88,325-329).  Takes effect where OVFCC_DYNQUANT_I8 does for 8-bit weights with one scale per channel, and
- * K < 65536:
+ * K <= 32768 (the sums below must fit 32 bits; a longer K keeps the symmetric form):
  *     d = max_k x - min_k x in half (0.003 if the two are equal), scale = half(255 / d), zp = half(-min * (255 / d)),
  *     q[m, k] = sat_u8(rte(half(x[m, k] * scale) + zp)),  za[m] = sat_u8(rte(zp)),
  *     y[m, n] = sum_k (q[m, k] - za[m]) (W[n, k] - ZP[n]) * (S[n] * half(1 / scale)) + bias[n],
